@@ -1,0 +1,313 @@
+// Chunked reduced-precision-accumulation matmuls (int8 -> int32 and e4m3/f16/bf16/f32 -> fp32).
+//
+// D[M,N] = sum over K-chunks of round_trunc( A_chunk . B_chunk^T ) (+ C).  Every chunk is
+// multiplied into a FRESH MFMA accumulator (the C operand is the inline constant 0 for the
+// first MFMA of the chunk), the chunk result is range-clamped / LSB-rounded on the vector ALU,
+// and only then added to the running accumulator -- the same order of operations as the
+// reference's Triton kernels, whose BLOCK_SIZE_K equals the chunk size.
+//
+// Tiling: 128x128 block, 4 waves of 64x64 (2x2 MFMA 32x32 blocks each); K advances in 64-byte
+// stages through two LDS buffers filled with bounds-checked 16-byte loads (zero fill past M, N
+// and K, which is what "the K tail is masked to 0" means).  One MFMA k-step is 32 bytes of K
+// for every operand type, so chunk boundaries (multiples of 32 bytes) always fall between
+// k-steps.
+#include "common.hpp"
+
+namespace fmsmo {
+
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+
+struct ChunkArgs {
+  const uint8_t* a;
+  const uint8_t* b;
+  int64_t lda, ldb;  // bytes
+  int M, N, Kb;      // Kb = K in bytes
+  int chunk_bytes;
+  int trun_bits, max_acc_bits, dl16, tta;
+  const void* c_in;
+  void* d;
+  int64_t ldd;
+};
+
+template <int OP>
+struct ChunkMma;
+template <>
+struct ChunkMma<FMSMO_OP_I8> {
+  typedef int Elem;
+  typedef v16i Acc;
+  __device__ static __forceinline__ Acc mma(const v4i& a, const v4i& b, const Acc& c) {
+    return __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c, 0, 0, 0);
+  }
+};
+template <>
+struct ChunkMma<FMSMO_OP_E4M3> {
+  typedef float Elem;
+  typedef v16f Acc;
+  __device__ static __forceinline__ Acc mma(const v4i& a, const v4i& b, const Acc& c) {
+    // two K=16 MFMAs on the low / high 8 bytes of the lane's 16-byte operand chunk
+    const long a0 = ((long)(unsigned)a[1] << 32) | (unsigned)a[0];
+    const long a1 = ((long)(unsigned)a[3] << 32) | (unsigned)a[2];
+    const long b0 = ((long)(unsigned)b[1] << 32) | (unsigned)b[0];
+    const long b1 = ((long)(unsigned)b[3] << 32) | (unsigned)b[2];
+    Acc t = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(a0, b0, c, 0, 0, 0);
+    return __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(a1, b1, t, 0, 0, 0);
+  }
+};
+template <>
+struct ChunkMma<FMSMO_OP_F16> {
+  typedef float Elem;
+  typedef v16f Acc;
+  __device__ static __forceinline__ Acc mma(const v4i& a, const v4i& b, const Acc& c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, a),
+                                                  __builtin_bit_cast(v8h, b), c, 0, 0, 0);
+  }
+};
+template <>
+struct ChunkMma<FMSMO_OP_BF16> {
+  typedef float Elem;
+  typedef v16f Acc;
+  __device__ static __forceinline__ Acc mma(const v4i& a, const v4i& b, const Acc& c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, a),
+                                                   __builtin_bit_cast(v8bf, b), c, 0, 0, 0);
+  }
+};
+
+template <>
+struct ChunkMma<FMSMO_OP_F32> {
+  typedef float Elem;
+  typedef v16f Acc;
+  __device__ static __forceinline__ Acc mma(const v4i& a, const v4i& b, const Acc& c) {
+    // four K=2 fp32 MFMAs, one per float of the lane's 16-byte operand chunk
+    Acc t = c;
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      t = __builtin_amdgcn_mfma_f32_32x32x2f32(__int_as_float(a[e]), __int_as_float(b[e]), t, 0, 0, 0);
+    return t;
+  }
+};
+
+// Chunk post-processing on one accumulator value.
+__device__ __forceinline__ int trunc_i32(int p, int lo, int hi, int round_bit, int t) {
+  p = max(min(p, hi), lo);
+  // (p + 2^(t-1)) >> t << t with two's-complement wrap on the add, arithmetic right shift
+  p = (int)((unsigned)p + (unsigned)round_bit);
+  return (int)((unsigned)(p >> t) << t);
+}
+__device__ __forceinline__ float trunc_f32(float p, unsigned round_bit, unsigned mask, int dl16) {
+  float x = __uint_as_float((__float_as_uint(p) + round_bit) & mask);
+  if (dl16) {
+    x = x >= 8581545984.0f ? __builtin_inff() : x;
+    x = x <= -8581545984.0f ? -__builtin_inff() : x;
+    x = fabsf(x) < 4.665707820095122e-10f ? 0.0f : x;
+  }
+  return x;
+}
+
+template <int OP>
+__global__ __launch_bounds__(256) void chunk_matmul_kernel(ChunkArgs g) {
+  typedef ChunkMma<OP> MM;
+  typedef typename MM::Acc Acc;
+  typedef typename MM::Elem Elem;
+  constexpr int BM = 128, BN = 128, BK = 64, CPR = 4;
+  __shared__ __attribute__((aligned(16))) uint8_t lds[2][(BM + BN) * BK];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int row0 = blockIdx.y * BM, col0 = blockIdx.x * BN;
+
+  // loader: thread -> (row = tid / 4 + 64 j, 16-byte chunk = tid % 4), swizzled position in LDS
+  const int lr = tid >> 2, lc = tid & 3;
+  auto sw = [](int r) { return ((r >> 1) & 3) ^ ((r >> 3) & 1); };
+  v4i stage_reg[4];
+  auto gload = [&](int k0) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int ra = row0 + lr + 64 * j, rb = col0 + lr + 64 * j;
+      const int kb = k0 + lc * 16;
+      const bool kin = kb + 16 <= g.Kb;
+      stage_reg[j] = (ra < g.M && kin) ? *(const v4i*)(g.a + (int64_t)ra * g.lda + kb) : v4i{0, 0, 0, 0};
+      stage_reg[2 + j] = (rb < g.N && kin) ? *(const v4i*)(g.b + (int64_t)rb * g.ldb + kb) : v4i{0, 0, 0, 0};
+    }
+  };
+  auto lstore = [&](int buf) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int r = lr + 64 * j;
+      const int pos = lc ^ sw(r);
+      *(v4i*)(&lds[buf][r * BK + pos * 16]) = stage_reg[j];
+      *(v4i*)(&lds[buf][BM * BK + r * BK + pos * 16]) = stage_reg[2 + j];
+    }
+  };
+
+  const int fr = lane & 31, fg = lane >> 5, fsw = sw(fr);
+
+  Acc acc[2][2], tmp[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        tmp[i][j][v] = 0;
+        Elem init = 0;
+        if (g.c_in) {
+          const int m = row0 + wm * 64 + i * 32 + (v >> 2) * 8 + fg * 4 + (v & 3);
+          const int n = col0 + wn * 64 + j * 32 + fr;
+          if (m < g.M && n < g.N) init = ((const Elem*)g.c_in)[(int64_t)m * g.ldd + n];
+        }
+        acc[i][j][v] = init;
+      }
+
+  const int t = g.dl16 ? 14 : g.trun_bits;
+  const unsigned round_bit = t > 0 ? 1u << (t - 1) : 0u;
+  const unsigned mask = ~((1u << t) - 1u);
+  const int lo = g.max_acc_bits < 32 ? -(1 << (g.max_acc_bits - 1)) : (int)0x80000000;
+  const int hi = g.max_acc_bits < 32 ? (1 << (g.max_acc_bits - 1)) - 1 : 0x7fffffff;
+  const bool post = g.dl16 || t > 0 || g.max_acc_bits < 32;
+
+  auto finish_chunk = [&]() {
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          Elem p = tmp[i][j][v];
+          if (post) {
+            if constexpr (OP == FMSMO_OP_I8) p = trunc_i32(p, lo, hi, (int)round_bit, t);
+            else p = trunc_f32(p, round_bit, mask, g.dl16);
+          }
+          if (g.tta) {
+            if constexpr (OP == FMSMO_OP_I8) acc[i][j][v] = (int)((unsigned)acc[i][j][v] + (unsigned)p);
+            else acc[i][j][v] += p;
+            tmp[i][j][v] = 0;
+          } else {
+            acc[i][j][v] = p;   // the running accumulator itself was rounded
+            tmp[i][j][v] = p;
+          }
+        }
+  };
+  if (!g.tta) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) tmp[i][j] = acc[i][j];
+  }
+
+  const int nstage = (g.Kb + BK - 1) / BK;
+  gload(0);
+  lstore(0);
+  __syncthreads();
+  int in_chunk = 0;  // bytes of the current chunk already multiplied
+  for (int st = 0; st < nstage; ++st) {
+    const int cur = st & 1;
+    if (st + 1 < nstage) gload((st + 1) * BK);
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      const int c = (2 * s + fg) ^ fsw;
+      v4i af[2], bf[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) af[i] = *(const v4i*)(&lds[cur][(wm * 64 + i * 32 + fr) * BK + c * 16]);
+#pragma unroll
+      for (int j = 0; j < 2; ++j) bf[j] = *(const v4i*)(&lds[cur][BM * BK + (wn * 64 + j * 32 + fr) * BK + c * 16]);
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) tmp[i][j] = MM::mma(af[i], bf[j], tmp[i][j]);
+      in_chunk += 32;
+      if (in_chunk == g.chunk_bytes) {
+        finish_chunk();
+        in_chunk = 0;
+      }
+    }
+    if (st + 1 < nstage) {
+      lstore(cur ^ 1);
+      __syncthreads();
+    }
+  }
+  if (in_chunk != 0) finish_chunk();  // zero-padded K tail
+
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int m = row0 + wm * 64 + i * 32 + (v >> 2) * 8 + fg * 4 + (v & 3);
+      if (m < g.M) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          const int n = col0 + wn * 64 + j * 32 + fr;
+          if (n < g.N) ((Elem*)g.d)[(int64_t)m * g.ldd + n] = acc[i][j][v];
+        }
+      }
+    }
+}
+
+}  // namespace fmsmo
+
+using namespace fmsmo;
+int fmsmo_check_launch();
+
+static int check_chunk(const void* a, int64_t lda, const void* b, int64_t ldb, const void* d,
+                       int64_t ldd, int64_t M, int64_t N, int64_t K, int64_t esz, int chunk_size,
+                       int min_chunk) {
+  if (!a || !b || !d) return FMSMO_ERR_NULL;
+  if (M < 0 || N <= 0 || K <= 0 || lda < K || ldb < K || ldd < N) return FMSMO_ERR_SHAPE;
+  if (M >= (1 << 30) || N >= (1 << 30) || K * esz >= (1ll << 31)) return FMSMO_ERR_UNSUPPORTED;
+  if (chunk_size < min_chunk || (chunk_size & (chunk_size - 1))) return FMSMO_ERR_UNSUPPORTED;
+  if ((K * esz) % 16 || (lda * esz) % 16 || (ldb * esz) % 16 || (((uintptr_t)a) & 15) ||
+      (((uintptr_t)b) & 15))
+    return FMSMO_ERR_ALIGN;
+  return FMSMO_OK;
+}
+
+extern "C" int fmsmo_matmul_chunk_i8(const int8_t* a, int64_t lda, const int8_t* b, int64_t ldb,
+                                     const int32_t* c_in, int32_t* d, int64_t ldd, int64_t M,
+                                     int64_t N, int64_t K, int chunk_size, int chunk_trun_bits,
+                                     int max_acc_bits, int truncate_then_accumulate,
+                                     fmsmo_stream_t stream) {
+  int rc = check_chunk(a, lda, b, ldb, d, ldd, M, N, K, 1, chunk_size, 32);
+  if (rc) return rc;
+  if (chunk_trun_bits < 0 || chunk_trun_bits > 31 || max_acc_bits < 2 || max_acc_bits > 32)
+    return FMSMO_ERR_UNSUPPORTED;
+  if (M == 0) return FMSMO_OK;
+  ChunkArgs g{};
+  g.a = (const uint8_t*)a; g.b = (const uint8_t*)b; g.lda = lda; g.ldb = ldb;
+  g.M = (int)M; g.N = (int)N; g.Kb = (int)K; g.chunk_bytes = chunk_size;
+  g.trun_bits = chunk_trun_bits; g.max_acc_bits = max_acc_bits; g.dl16 = 0;
+  g.tta = truncate_then_accumulate != 0; g.c_in = c_in; g.d = d; g.ldd = ldd;
+  dim3 grid(div_up(N, 128), div_up(M, 128));
+  hipLaunchKernelGGL((chunk_matmul_kernel<FMSMO_OP_I8>), grid, dim3(256), 0, (hipStream_t)stream, g);
+  return fmsmo_check_launch();
+}
+
+extern "C" int fmsmo_matmul_chunk_fp(const void* a, int64_t lda, const void* b, int64_t ldb,
+                                     int op_dtype, const float* c_in, float* d, int64_t ldd,
+                                     int64_t M, int64_t N, int64_t K, int chunk_size,
+                                     int chunk_trun_bits, int clamp_dl16,
+                                     int truncate_then_accumulate, fmsmo_stream_t stream) {
+  if (op_dtype != FMSMO_OP_E4M3 && op_dtype != FMSMO_OP_F16 && op_dtype != FMSMO_OP_BF16 &&
+      op_dtype != FMSMO_OP_F32)
+    return FMSMO_ERR_UNSUPPORTED;
+  const int esz = op_dtype == FMSMO_OP_E4M3 ? 1 : op_dtype == FMSMO_OP_F32 ? 4 : 2;
+  int rc = check_chunk(a, lda, b, ldb, d, ldd, M, N, K, esz, chunk_size, esz == 1 ? 32 : 16);
+  if (rc) return rc;
+  if (chunk_trun_bits < 0 || chunk_trun_bits > 22) return FMSMO_ERR_UNSUPPORTED;
+  if (M == 0) return FMSMO_OK;
+  ChunkArgs g{};
+  g.a = (const uint8_t*)a; g.b = (const uint8_t*)b; g.lda = lda * esz; g.ldb = ldb * esz;
+  g.M = (int)M; g.N = (int)N; g.Kb = (int)(K * esz); g.chunk_bytes = chunk_size * esz;
+  g.trun_bits = chunk_trun_bits; g.max_acc_bits = 32; g.dl16 = clamp_dl16 != 0;
+  g.tta = truncate_then_accumulate != 0; g.c_in = c_in; g.d = d; g.ldd = ldd;
+  dim3 grid(div_up(N, 128), div_up(M, 128));
+  hipStream_t st = (hipStream_t)stream;
+  if (op_dtype == FMSMO_OP_E4M3)
+    hipLaunchKernelGGL((chunk_matmul_kernel<FMSMO_OP_E4M3>), grid, dim3(256), 0, st, g);
+  else if (op_dtype == FMSMO_OP_F16)
+    hipLaunchKernelGGL((chunk_matmul_kernel<FMSMO_OP_F16>), grid, dim3(256), 0, st, g);
+  else if (op_dtype == FMSMO_OP_F32)
+    hipLaunchKernelGGL((chunk_matmul_kernel<FMSMO_OP_F32>), grid, dim3(256), 0, st, g);
+  else
+    hipLaunchKernelGGL((chunk_matmul_kernel<FMSMO_OP_BF16>), grid, dim3(256), 0, st, g);
+  return fmsmo_check_launch();
+}

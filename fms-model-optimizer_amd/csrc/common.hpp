@@ -1,0 +1,94 @@
+// Shared device/host helpers for the gfx950 quantized-linear kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/fmsmo_hip.h"
+
+namespace fmsmo {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef short s8v __attribute__((ext_vector_type(8)));
+typedef unsigned short u16;
+
+#define FMSMO_GPTR(p) ((const __attribute__((address_space(1))) void*)(p))
+#define FMSMO_LPTR(p) ((__attribute__((address_space(3))) void*)(p))
+
+// ---------------------------------------------------------------- 16-bit float conversions
+// All conversions are round-to-nearest-even and keep subnormals, matching torch's casts.
+__device__ __forceinline__ float f16_to_f32(u16 h) {
+  _Float16 v;
+  __builtin_memcpy(&v, &h, 2);
+  return (float)v;
+}
+__device__ __forceinline__ u16 f32_to_f16(float f) {
+  // Keep the conversion a separate instruction: without this the compiler folds
+  // "round_to_f16(a * b)" / "(a + b)" into v_fma_mixlo_f16, which rounds the exact product or
+  // sum once to fp16 instead of fp32-then-fp16 as torch does (differs at fp16 ties).
+  asm volatile("" : "+v"(f));
+  _Float16 v = (_Float16)f;  // v_cvt_f16_f32: RNE, overflow -> inf
+  u16 h;
+  __builtin_memcpy(&h, &v, 2);
+  return h;
+}
+__device__ __forceinline__ float bf16_to_f32(u16 h) { return __uint_as_float(((uint32_t)h) << 16); }
+__device__ __forceinline__ u16 f32_to_bf16(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (u16)((u >> 16) | 0x40);  // quiet NaN
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (u16)(u >> 16);
+}
+
+// Round a float to the value grid of dtype T (T in FMSMO_F16/BF16/F32) and come back to f32.
+template <int T>
+__device__ __forceinline__ float round_to(float f) {
+  if constexpr (T == FMSMO_F16) return f16_to_f32(f32_to_f16(f));
+  else if constexpr (T == FMSMO_BF16) return bf16_to_f32(f32_to_bf16(f));
+  else return f;
+}
+template <int T>
+__device__ __forceinline__ float load_as_f32(const void* p, size_t i) {
+  if constexpr (T == FMSMO_F16) return f16_to_f32(((const u16*)p)[i]);
+  else if constexpr (T == FMSMO_BF16) return bf16_to_f32(((const u16*)p)[i]);
+  else return ((const float*)p)[i];
+}
+template <int T>
+__device__ __forceinline__ void store_from_f32(void* p, size_t i, float v) {
+  if constexpr (T == FMSMO_F16) ((u16*)p)[i] = f32_to_f16(v);
+  else if constexpr (T == FMSMO_BF16) ((u16*)p)[i] = f32_to_bf16(v);
+  else ((float*)p)[i] = v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+
+// OCP e4m3fn encode of one float, RNE, the way torch's float->float8_e4m3fn cast does it:
+// |x| <= 464 rounds into the finite range (max 448), anything above and NaN give 0x7f|sign.
+__device__ __forceinline__ uint8_t f32_to_e4m3_sw(float f) {
+  uint32_t u = __float_as_uint(f);
+  uint8_t sign = (u >> 24) & 0x80;
+  uint32_t a = u & 0x7fffffffu;
+  if (a > 0x43e80000u) return sign | 0x7f;       // > 464 (incl. inf / NaN) -> NaN
+  if (a < 0x3c800000u) {                          // subnormal target: < 2^-6, quantum 2^-9
+    float q = __uint_as_float(a) * 512.0f;        // exact scaling
+    float r = __builtin_rintf(q);                 // RNE
+    return sign | (uint8_t)(int)r;                // r in [0,8]; 8 == smallest normal 0x08
+  }
+  // normal: keep 3 mantissa bits
+  uint32_t r = a + 0x7ffffu + ((a >> 20) & 1u);
+  r >>= 20;                                       // exponent(8) | mant(3)
+  int e = (int)(r >> 3) - 127 + 7;
+  return sign | (uint8_t)((e << 3) | (r & 7));
+}
+
+inline int div_up(int64_t a, int64_t b) { return (int)((a + b - 1) / b); }
+
+}  // namespace fmsmo

@@ -1,0 +1,428 @@
+// LDS-tiled MFMA GEMM core for gfx950:  C[M,N] = A[M,K] . B[N,K]^T with 1-byte operands.
+//
+// Data movement: both operands are K-contiguous, so a tile is a set of rows of BK bytes.  Tiles
+// go HBM/L2 -> LDS with global_load_lds_dwordx4 (no VGPR staging); each wave instruction moves
+// 64 x 16 B = 1 KiB that lands contiguously in LDS, i.e. 1024/BK whole rows, so every row is
+// fetched as one BK-byte run (full 128-byte lines for BK = 128).  The 16-byte chunks of a row
+// are XOR-permuted on the way in (the lane picks which global chunk it fetches) so that the
+// ds_read_b128 operand fetches of the MFMA phase are bank-conflict free.
+//
+// Math: each wave owns a (BM/WGM) x (BN/WGN) sub-tile built from 32x32 MFMA blocks
+// (v_mfma_i32_32x32x32_i8, or v_mfma_f32_32x32x64_f8f6f4 with both operands e4m3).  The MFMA
+// sums over k, so any assignment of k-bytes to (lane group, register byte) is valid as long as
+// A and B use the same one; the loaders exploit that and never transpose anything.
+//
+// Pipeline: NSTAGE LDS buffers.  The DMA of stage kt+NSTAGE is issued during the last MFMA k-step
+// of stage kt, so every stage has NSTAGE-1 full iterations (> 1 us) to arrive from L2/HBM.
+// One barrier per stage; the barrier, the DMA issue and the first operand reads of the next
+// stage are hidden under MFMAs whose operands were read earlier (register double buffering).
+#pragma once
+#include "common.hpp"
+#include <type_traits>
+#include <utility>
+
+namespace fmsmo {
+
+enum { MMA_I8 = 0, MMA_FP8 = 1 };
+
+struct GemmArgs {
+  const uint8_t* a;
+  const uint8_t* b;
+  int64_t lda, ldb;  // bytes
+  int M, N, K;
+  int grid_m, grid_n;  // tiles along M and N (grid_m is an upper bound in grouped mode)
+  int group_m;         // tile-order grouping along M
+  // grouped (mixture-of-experts) mode
+  const int32_t* offsets;
+  int num_experts;
+  int64_t ldb_e;  // bytes between experts in B
+#ifdef FMSMO_CLK
+  unsigned long long* clk;  // harness only: {core clock, 100 MHz wall clock} at start / end
+#endif
+};
+
+// 16-byte chunk c of row r is stored at chunk position c ^ swz(r).  Depends on r & 15 only.
+template <int CPR, int SWZ>
+__device__ __forceinline__ int swz(int r) {
+  if constexpr (SWZ == 0) return 0;
+  if constexpr (CPR == 8) {
+    if constexpr (SWZ == 1) return (r & 7) ^ ((r >> 3) & 1);
+    if constexpr (SWZ == 2) return (r & 7);
+    return (r >> 1) & 7;
+  } else {  // CPR == 4
+    if constexpr (SWZ == 1) return ((r >> 1) & 3) ^ ((r >> 3) & 1);
+    if constexpr (SWZ == 2) return (r >> 1) & 3;
+    return (r >> 2) & 3;
+  }
+}
+
+template <int OP>
+struct Mma;
+template <>
+struct Mma<MMA_I8> {
+  typedef v4i Frag;
+  typedef v16i Acc;
+  typedef int Elem;
+  static constexpr int KSTEP = 32;  // bytes of K per MFMA
+  __device__ static __forceinline__ Acc mma(const Frag& a, const Frag& b, const Acc& c) {
+    return __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c, 0, 0, 0);
+  }
+};
+template <>
+struct Mma<MMA_FP8> {
+  typedef v8i Frag;
+  typedef v16f Acc;
+  typedef float Elem;
+  static constexpr int KSTEP = 64;
+  __device__ static __forceinline__ Acc mma(const Frag& a, const Frag& b, const Acc& c) {
+    // cbsz = blgp = 0: both operands OCP e4m3; zero scale operands select the unscaled form.
+    return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0);
+  }
+};
+
+// Map the hardware block id to a tile.  Work-groups are dealt round-robin to the 8 XCDs (each
+// with a private L2), so block b runs on XCD b % 8; give every XCD one contiguous span of the
+// tile sequence, and order that sequence in column-major groups of `group_m` tile rows so the
+// tiles resident on an XCD at the same time share A rows and B rows.
+__device__ __forceinline__ void tile_of_block(int bid, int nblk, int grid_m, int grid_n,
+                                              int group_m, int& tm, int& tn) {
+  const int per = nblk >> 3, rem = nblk & 7;
+  const int xcd = bid & 7, idx = bid >> 3;
+  const int pid = (xcd < rem ? xcd * (per + 1) : rem * (per + 1) + (xcd - rem) * per) + idx;
+  const int in_group = group_m * grid_n;
+  const int gid = pid / in_group;
+  const int first_m = gid * group_m;
+  const int gsz = min(grid_m - first_m, group_m);
+  const int r = pid - gid * in_group;
+  tm = first_m + r % gsz;
+  tn = r / gsz;
+}
+
+template <int BM, int BN, int BK, int NSTAGE, int WGM, int WGN, int OP, int SWZ, bool GROUPED,
+          class Epi>
+__global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(GemmArgs g, Epi epi) {
+#if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stub
+  typedef Mma<OP> MM;
+  typedef typename MM::Frag Frag;
+  typedef typename MM::Acc Acc;
+  constexpr int THREADS = WGM * WGN * 64;
+  constexpr int CPR = BK / 16;              // 16-byte chunks per tile row
+  constexpr int RPI = THREADS / CPR;        // tile rows moved by one block-wide load instruction
+  constexpr int NIA = BM / RPI, NIB = BN / RPI;
+  constexpr int TM = BM / WGM, TN = BN / WGN;  // wave sub-tile
+  constexpr int FM = TM / 32, FN = TN / 32;    // 32x32 MFMA blocks per wave
+  constexpr int NKS = BK / MM::KSTEP;          // MFMA k-steps per stage
+  constexpr int CL = MM::KSTEP / 32;           // 16-byte chunks per lane per k-step
+  static_assert(RPI % 16 == 0 && BM % RPI == 0 && BN % RPI == 0, "loader shape");
+  static_assert(TM % 32 == 0 && TN % 32 == 0, "wave tile");
+
+  constexpr int STAGE_BYTES = (BM + BN) * BK;
+  __shared__ __attribute__((aligned(16))) uint8_t lds[NSTAGE][STAGE_BYTES];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / WGN, wn = wave % WGN;
+
+#ifdef FMSMO_CLK
+  if (blockIdx.x == 0 && tid == 0 && g.clk) { g.clk[0] = clock64(); g.clk[1] = wall_clock64(); }
+#endif
+  int tile_m, tile_n;
+  tile_of_block(blockIdx.x, gridDim.x, g.grid_m, g.grid_n, g.group_m, tile_m, tile_n);
+
+#ifdef FMSMO_ABLATE_SAME_TILE
+  tile_m = FMSMO_ABLATE_SAME_TILE == 1 ? 0 : (blockIdx.x & 7) / 4 + 2 * ((blockIdx.x >> 3) & 1);
+  tile_n = FMSMO_ABLATE_SAME_TILE == 1 ? 0 : (blockIdx.x & 7) % 4 + 4 * ((blockIdx.x >> 4) & 1);
+#endif
+  // Row range of A (and of the output) this tile may touch.
+  int row_lo = 0, row_hi = g.M, expert = 0;
+  if constexpr (GROUPED) {
+    int t = tile_m;
+    bool found = false;
+    for (int e = 0; e < g.num_experts; ++e) {
+      const int lo = g.offsets[e], hi = g.offsets[e + 1];
+      const int nt = (hi - lo + BM - 1) / BM;
+      if (t < nt) {
+        row_lo = lo + t * BM;
+        row_hi = hi;
+        expert = e;
+        found = true;
+        break;
+      }
+      t -= nt;
+    }
+    if (!found) return;  // uniform for the whole block
+  } else {
+    row_lo = tile_m * BM;
+  }
+  const int col_lo = tile_n * BN;
+
+  const uint8_t* __restrict__ A = g.a;
+  const uint8_t* __restrict__ B = g.b + (GROUPED ? (int64_t)expert * g.ldb_e : 0);
+
+  // ---- global -> LDS loader addressing (per thread, constant over the K loop)
+  const int ld_row = tid / CPR;
+  const int ld_pos = tid % CPR;
+  const int ld_chunk = ld_pos ^ swz<CPR, SWZ>(ld_row);
+  uint32_t a_off[NIA], b_off[NIB];
+#pragma unroll
+  for (int j = 0; j < NIA; ++j) {
+    const int r = min(row_lo + ld_row + j * RPI, row_hi - 1);  // clamp: rows past the end re-read
+    a_off[j] = (uint32_t)r * (uint32_t)g.lda + ld_chunk * 16;  // the last valid row, never stored
+  }
+#pragma unroll
+  for (int j = 0; j < NIB; ++j) {
+    const int r = min(col_lo + ld_row + j * RPI, g.N - 1);
+    b_off[j] = (uint32_t)r * (uint32_t)g.ldb + ld_chunk * 16;
+  }
+
+  // DMA instructions j in [j0, j1) of a stage (A rows first, then B rows).  Buffer addressing:
+  // per-lane 32-bit row/chunk offset (constant over K) + scalar K offset, so the loop needs no
+  // vector address arithmetic.
+  const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc((void*)A, 0, -1, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc((void*)B, 0, -1, 0x00020000);
+  auto issue_part = [&](int stage, int k0, auto j0_c, auto j1_c) {
+    constexpr int J0 = decltype(j0_c)::value, J1 = decltype(j1_c)::value;
+    uint8_t* la = &lds[0][0] + stage * STAGE_BYTES + wave * 1024;
+#pragma unroll
+    for (int j = J0; j < J1; ++j) {
+      if (j < NIA)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, FMSMO_LPTR(la + j * THREADS * 16), 16,
+                                                 a_off[j], k0, 0, 0);
+      else
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, FMSMO_LPTR(la + j * THREADS * 16), 16,
+                                                 b_off[j - NIA], k0, 0, 0);
+    }
+  };
+
+  // ---- LDS -> MFMA operand addressing
+  const int fr = lane & 31, fg = lane >> 5;
+  const int fsw = swz<CPR, SWZ>(fr);
+  int a_rd[NKS][CL], b_rd[NKS][CL];
+#pragma unroll
+  for (int s = 0; s < NKS; ++s)
+#pragma unroll
+    for (int e = 0; e < CL; ++e) {
+      const int c = s * 2 * CL + fg * CL + e;
+      a_rd[s][e] = (wm * TM + fr) * BK + ((c ^ fsw) * 16);
+      b_rd[s][e] = BM * BK + (wn * TN + fr) * BK + ((c ^ fsw) * 16);
+    }
+
+  Acc acc[FM][FN];
+#pragma unroll
+  for (int i = 0; i < FM; ++i)
+#pragma unroll
+    for (int j = 0; j < FN; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
+
+  auto read_frags = [&](const uint8_t* ls, int s, Frag* af, Frag* bf) {
+#ifdef FMSMO_ABLATE_NO_LDSREAD
+    if (g.K > 0) return;
+#endif
+#pragma unroll
+    for (int i = 0; i < FM; ++i) {
+      if constexpr (CL == 1) {
+        af[i] = *(const v4i*)(ls + a_rd[s][0] + i * 32 * BK);
+      } else {
+        const v4i lo = *(const v4i*)(ls + a_rd[s][0] + i * 32 * BK);
+        const v4i hi = *(const v4i*)(ls + a_rd[s][1] + i * 32 * BK);
+        af[i] = Frag{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < FN; ++j) {
+      if constexpr (CL == 1) {
+        bf[j] = *(const v4i*)(ls + b_rd[s][0] + j * 32 * BK);
+      } else {
+        const v4i lo = *(const v4i*)(ls + b_rd[s][0] + j * 32 * BK);
+        const v4i hi = *(const v4i*)(ls + b_rd[s][1] + j * 32 * BK);
+        bf[j] = Frag{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      }
+    }
+  };
+  auto mma_step = [&](const Frag* af, const Frag* bf) {
+#ifdef FMSMO_ABLATE_NO_MMA
+    if (g.K > 0) return;
+#endif
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+      for (int j = 0; j < FN; ++j) acc[i][j] = MM::mma(af[i], bf[j], acc[i][j]);
+  };
+  // Instruction-order hints (DS read = 0x100, MFMA = 0x008, VMEM = 0x020): the operand reads of
+  // the next k-step go between the first MFMAs of the current one, so their latency is covered
+  // by the remaining MFMAs; the DMA instructions are spread evenly behind them (the texture
+  // path takes ~16 cycles per 1 KiB wave instruction and is shared by the whole CU, so bursts
+  // of DMA issue would stall the in-order wave and starve the MFMA pipe).
+  constexpr int NRD = (FM + FN) * CL, NMMA = FM * FN, NLD = NIA + NIB;
+  constexpr int LDP = NLD / NKS;  // DMA instructions issued per k-step
+  static_assert(NLD % NKS == 0, "DMA instructions must split evenly over the k-steps");
+  static_assert(NSTAGE >= 3, "pipeline needs at least three LDS stages");
+  auto interleave = [&]() {
+    constexpr int PER = (NMMA / 2) / NRD > 0 ? (NMMA / 2) / NRD : 1;
+#pragma unroll
+    for (int r = 0; r < NRD; ++r) {
+      __builtin_amdgcn_sched_group_barrier(0x008, PER, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+    constexpr int REST = NMMA - PER * NRD > 0 ? NMMA - PER * NRD : 0;
+    if constexpr (REST >= LDP && LDP > 0) {
+      constexpr int MPL = REST / LDP;  // MFMAs per DMA instruction
+#pragma unroll
+      for (int r = 0; r < LDP; ++r) {
+        __builtin_amdgcn_sched_group_barrier(0x008, MPL, 0);
+        __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+      }
+      if constexpr (REST - MPL * LDP > 0) __builtin_amdgcn_sched_group_barrier(0x008, REST - MPL * LDP, 0);
+    } else if constexpr (REST > 0) {
+      __builtin_amdgcn_sched_group_barrier(0x008, REST, 0);
+    }
+  };
+
+  Frag fa[2][FM], fb[2][FN];
+  const int nk = g.K / BK;
+
+  // One K-stage.  PAR = parity of kt * NKS, so that operand-register buffer indices are static.
+  // While stage kt is multiplied, the DMA of stage kt+NSTAGE-1 refills the buffer that stage
+  // kt-1 occupied (free since the barrier at the end of stage kt-1).  Stages past the end of K
+  // are "phantom": their DMA re-reads the last real stage into a buffer nobody consumes, which
+  // keeps the loop body and the vmcnt bookkeeping uniform.
+  auto stage = [&](int kt, auto par_c) {
+    constexpr int PAR = decltype(par_c)::value;
+    const int cur = kt % NSTAGE;
+    const int fill = (kt + NSTAGE - 1) % NSTAGE;
+    const int fill_k0 = min(kt + NSTAGE - 1, nk - 1) * BK;
+    const uint8_t* ls = &lds[0][0] + cur * STAGE_BYTES;
+    auto dma = [&](auto s_c) {
+      constexpr int S = decltype(s_c)::value;
+#ifdef FMSMO_ABLATE_NO_DMA
+      if (g.K < 0)
+#endif
+      issue_part(fill, fill_k0, std::integral_constant<int, S * LDP>{},
+                 std::integral_constant<int, (S + 1) * LDP>{});
+    };
+    [&]<int... S>(std::integer_sequence<int, S...>) {
+      (
+          [&] {
+            read_frags(ls, S + 1, fa[(PAR + S + 1) & 1], fb[(PAR + S + 1) & 1]);
+            dma(std::integral_constant<int, S>{});
+            mma_step(fa[(PAR + S) & 1], fb[(PAR + S) & 1]);
+            interleave();
+          }(),
+          ...);
+    }(std::make_integer_sequence<int, NKS - 1>{});
+    // Last k-step: its operands are already in registers.  Wait until this wave's share of
+    // stage kt+1 has landed (younger DMA may stay in flight) and until its own LDS reads of
+    // stage kt have returned, then barrier: stage kt+1 is now complete for all waves and buffer
+    // `cur` may be refilled during the next stage.
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"((NSTAGE - 3) * NLD + (NKS - 1) * LDP)
+                 : "memory");
+    const int nxt = (kt + 1) % NSTAGE;
+    read_frags(&lds[0][0] + nxt * STAGE_BYTES, 0, fa[(PAR + NKS) & 1], fb[(PAR + NKS) & 1]);
+    dma(std::integral_constant<int, NKS - 1>{});
+    mma_step(fa[(PAR + NKS - 1) & 1], fb[(PAR + NKS - 1) & 1]);
+    interleave();
+  };
+
+#pragma unroll
+  for (int st = 0; st < NSTAGE - 1; ++st)
+    issue_part(st, min(st, nk - 1) * BK, std::integral_constant<int, 0>{},
+               std::integral_constant<int, NLD>{});
+  asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"((NSTAGE - 2) * NLD) : "memory");
+  read_frags(&lds[0][0], 0, fa[0], fb[0]);
+  {
+    int kt = 0;
+    if constexpr (NKS % 2 == 0) {
+      for (; kt < nk; ++kt) stage(kt, std::integral_constant<int, 0>{});
+    } else {
+      for (; kt + 1 < nk; kt += 2) {
+        stage(kt, std::integral_constant<int, 0>{});
+        stage(kt + 1, std::integral_constant<int, 1>{});
+      }
+      if (kt < nk) stage(kt, std::integral_constant<int, 0>{});
+    }
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no DMA may be in flight when LDS is released
+
+#ifdef FMSMO_CLK
+  if (blockIdx.x == 0 && tid == 0 && g.clk) { g.clk[2] = clock64(); g.clk[3] = wall_clock64(); }
+#endif
+  // ---- epilogue: acc[i][j][v] is C(row, col) with
+  //      row = 32 i + 8 (v / 4) + 4 (lane / 32) + v % 4,   col = 32 j + lane % 32
+  const int m_base = row_lo + wm * TM + fg * 4;
+  const int n_base = col_lo + wn * TN + fr;
+  typename Epi::Col colctx[FN];
+#pragma unroll
+  for (int j = 0; j < FN; ++j) colctx[j] = epi.col(min(n_base + j * 32, g.N - 1), expert, g.N);
+#pragma unroll
+  for (int i = 0; i < FM; ++i)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int m = m_base + i * 32 + (v >> 2) * 8 + (v & 3);
+      if (m < row_hi) {
+        const typename Epi::Row rowctx = epi.row(m);
+#pragma unroll
+        for (int j = 0; j < FN; ++j) {
+          const int n = n_base + j * 32;
+          if (n < g.N) epi.store(m, n, acc[i][j][v], rowctx, colctx[j]);
+        }
+      }
+    }
+#ifdef FMSMO_CLK
+  if (blockIdx.x == 0 && tid == 0 && g.clk) { g.clk[4] = clock64(); g.clk[5] = wall_clock64(); }
+#endif
+#endif  // __HIP_DEVICE_COMPILE__
+}
+
+// ------------------------------------------------------------------------------ epilogues
+struct EpiStoreI32 {
+  int32_t* c;
+  int64_t ldc;
+  struct Col {};
+  struct Row {};
+  __device__ __forceinline__ Col col(int, int, int) const { return Col{}; }
+  __device__ __forceinline__ Row row(int) const { return Row{}; }
+  __device__ __forceinline__ void store(int m, int n, int v, Row, Col) const {
+    c[(int64_t)m * ldc + n] = v;
+  }
+};
+
+// y = acc * (a_scale[m] x w_scale[n]) + bias[n], see FMSMO_EPI_* in fmsmo_hip.h.
+template <int OUT, int BIAS, bool REF_F16, class AccT>
+struct EpiDequant {
+  void* y;
+  int64_t ldy;
+  const float* a_scale;
+  const float* w_scale;
+  const void* bias;
+  int a_stride, w_stride;  // 0 = one value for all rows / columns, 1 = per row / column
+  struct Col {
+    float ws, b;
+  };
+  struct Row {
+    float as;
+  };
+  __device__ __forceinline__ Col col(int n, int expert, int N) const {
+    Col c;
+    const int64_t o = (int64_t)expert * N + n;
+    c.ws = w_scale[w_stride ? o : 0];
+    c.b = bias ? load_as_f32<BIAS>(bias, o) : 0.0f;
+    return c;
+  }
+  __device__ __forceinline__ Row row(int m) const { return Row{a_scale[a_stride ? m : 0]}; }
+  __device__ __forceinline__ void store(int m, int n, AccT v, Row r, Col c) const {
+    float out;
+    if constexpr (REF_F16) {
+      // separate fp32 multiply and add (no fma), scale product rounded to fp16 first,
+      // result rounded to fp16 before the cast to the output dtype
+      const float sc = round_to<FMSMO_F16>(__fmul_rn(r.as, c.ws));
+      out = round_to<FMSMO_F16>(__fadd_rn(__fmul_rn((float)v, sc), c.b));
+    } else {
+      out = __fmaf_rn((float)v, __fmul_rn(r.as, c.ws), c.b);
+    }
+    store_from_f32<OUT>(y, (int64_t)m * ldy + n, out);
+  }
+};
+
+}  // namespace fmsmo

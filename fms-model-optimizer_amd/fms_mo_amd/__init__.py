@@ -1,0 +1,11 @@
+"""MI355X-native (gfx950) implementation of fms-model-optimizer's quantized-linear inference path.
+
+Layout mirrors the reference package for the modules on that path:
+  fms_mo_amd.modules.linear            QLinear, QLinearINT8Deploy, LinearFPxAcc, QLinearINT8Train
+  fms_mo_amd.modules.fp8_linear        FP8Linear
+  fms_mo_amd.quant.quantizers          the quantizer subset those modules need
+  fms_mo_amd.custom_ext_kernels.utils  torch.ops.fms_mo.* registration, lowering helpers
+  fms_mo_amd.custom_ext_kernels.hip_kernels  matmul_chunk_truncate (the tl_matmul_chunk_truncate API)
+  fms_mo_amd.kernels / fms_mo_amd._lib tensor-level and ctypes bindings of libfmsmo_hip.so
+"""
+__version__ = "0.1.0"

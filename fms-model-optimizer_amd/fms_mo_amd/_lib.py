@@ -1,0 +1,87 @@
+"""ctypes binding of libfmsmo_hip.so, the C-ABI library of hand-written gfx950 kernels.
+
+There is no CPU fallback: every operator of this package ends in one of these entry points, and
+loading fails loudly when the library has not been built
+(``make -C fms-model-optimizer_amd/csrc`` or ``python -c 'import __graft_entry__ as g; g.build()'``).
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from ctypes import c_char_p, c_float, c_int, c_int64, c_void_p
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.normpath(os.path.join(_HERE, "..", "lib", "libfmsmo_hip.so"))
+
+# dtype / enum codes of include/fmsmo_hip.h
+F16, BF16, F32 = 0, 1, 2
+OP_I8, OP_E4M3, OP_F16, OP_BF16, OP_F32 = 0, 1, 2, 3, 4
+EPI_REF_F16, EPI_F32 = 0, 1
+FP8_LINEAR, FP8_FPXACC, FP8_FPXACC_DL8 = 0, 1, 2
+ABI_VERSION = 1
+
+_P, _I, _L, _F = c_void_p, c_int, c_int64, c_float
+
+# name -> argument types (all functions return int except the three below)
+SIGNATURES = {
+    "fmsmo_quant_act_i8_pertoken": [_P, _I, _L, _P, _I, _I, _I, _P, _L, _P, _L, _L, _P],
+    "fmsmo_quant_act_i8_static": [_P, _I, _L, _F, _I, _I, _P, _L, _L, _L, _P],
+    "fmsmo_quant_act_fp8_pertoken": [_P, _I, _L, _I, _I, _P, _L, _P, _L, _L, _P],
+    "fmsmo_gemm_i8_i32": [_P, _L, _P, _L, _P, _L, _L, _L, _L, _P],
+    "fmsmo_gemm_i8_dq": [_P, _L, _P, _L, _P, _L, _P, _L, _P, _I, _I, _P, _I, _L, _L, _L, _L, _P],
+    "fmsmo_gemm_fp8_dq": [_P, _L, _P, _L, _P, _L, _P, _L, _P, _I, _P, _I, _L, _L, _L, _L, _P],
+    "fmsmo_gemv_i8_dq": [_P, _L, _P, _L, _P, _L, _P, _L, _P, _I, _I, _P, _I, _L, _L, _L, _L, _P],
+    "fmsmo_gemv_fp8_dq": [_P, _L, _P, _L, _P, _L, _P, _L, _P, _I, _P, _I, _L, _L, _L, _L, _P],
+    "fmsmo_matmul_chunk_i8": [_P, _L, _P, _L, _P, _P, _L, _L, _L, _L, _I, _I, _I, _I, _P],
+    "fmsmo_matmul_chunk_fp": [_P, _L, _P, _L, _I, _P, _P, _L, _L, _L, _L, _I, _I, _I, _I, _P],
+    "fmsmo_grouped_gemm_i8_dq": [_P, _L, _P, _L, _L, _P, _I, _L, _P, _P, _P, _I, _I, _P, _I, _L,
+                                 _L, _L, _P],
+}
+OTHER = {
+    "fmsmo_abi_version": ([], c_int),
+    "fmsmo_status_str": ([c_int], c_char_p),
+    "fmsmo_last_error": ([], c_char_p),
+}
+
+_lib = None
+
+
+class FmsMoHipError(RuntimeError):
+    """A C-ABI entry point returned a non-zero status (the reference raises RuntimeError from
+    TORCH_CHECK in the same situations, fms_mo/custom_ext_kernels/cutlass_i8i32gemm.cu:118)."""
+
+
+def load() -> ctypes.CDLL:
+    """Load the shared library once and attach argument / return types."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise FmsMoHipError(
+            f"{LIB_PATH} is missing: build the HIP kernels first "
+            "(make -C fms-model-optimizer_amd/csrc). There is no fallback path."
+        )
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, argtypes in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.argtypes = argtypes
+        fn.restype = c_int
+    for name, (argtypes, restype) in OTHER.items():
+        fn = getattr(lib, name)
+        fn.argtypes = argtypes
+        fn.restype = restype
+    if lib.fmsmo_abi_version() != ABI_VERSION:
+        raise FmsMoHipError("libfmsmo_hip.so ABI version mismatch; rebuild the library")
+    _lib = lib
+    return lib
+
+
+def call(name: str, *args) -> None:
+    """Invoke an entry point and raise on a non-zero status."""
+    lib = load()
+    rc = getattr(lib, name)(*args)
+    if rc != 0:
+        msg = lib.fmsmo_status_str(rc).decode()
+        if rc == 5:
+            msg += ": " + lib.fmsmo_last_error().decode()
+        raise FmsMoHipError(f"{name} failed with status {rc} ({msg})")

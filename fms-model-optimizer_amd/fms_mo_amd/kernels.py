@@ -1,0 +1,240 @@
+"""Tensor-level wrappers over the C-ABI kernels: argument checks, output allocation through
+torch's caching allocator, the current HIP stream of the tensors' device.  No arithmetic happens
+here; torch is only the owner of device memory and streams."""
+from __future__ import annotations
+
+import torch
+
+from . import _lib as L
+
+_DT = {torch.float16: L.F16, torch.bfloat16: L.BF16, torch.float32: L.F32}
+_OPDT = {torch.int8: L.OP_I8, torch.float8_e4m3fn: L.OP_E4M3, torch.float16: L.OP_F16,
+         torch.bfloat16: L.OP_BF16, torch.float32: L.OP_F32}
+_BITS = {1: torch.uint8, 2: torch.int16, 4: torch.int32}
+
+
+def _need_gpu(*ts):
+    for t in ts:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError(
+                "fms_mo_amd kernels run on an AMD GPU only (tensor is on %s); there is no CPU path"
+                % t.device
+            )
+
+
+def _stream(t: torch.Tensor):
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def _dt(t: torch.Tensor) -> int:
+    try:
+        return _DT[t.dtype]
+    except KeyError:
+        raise TypeError(f"unsupported floating dtype {t.dtype}") from None
+
+
+def _rows(t: torch.Tensor) -> torch.Tensor:
+    """2-D, unit inner stride (row stride may be larger than the row)."""
+    if t.dim() != 2:
+        raise ValueError("expected a 2-D tensor")
+    if t.stride(1) != 1 or (t.shape[0] > 1 and t.stride(0) < t.shape[1]):
+        t = t.contiguous()
+    return t
+
+
+def _ld(t: torch.Tensor) -> int:
+    return t.stride(0) if t.shape[0] > 1 else max(t.shape[1], t.stride(0))
+
+
+def _scale_vec(s, n, device, name):
+    if not torch.is_tensor(s):
+        s = torch.tensor([float(s)], dtype=torch.float32, device=device)
+    s = s.detach().to(device=device, dtype=torch.float32).reshape(-1).contiguous()
+    if s.numel() not in (1, n):
+        raise ValueError(f"{name} must have 1 or {n} elements, got {s.numel()}")
+    return s
+
+
+# ------------------------------------------------------------------------------- quantizers
+def quant_act_i8_pertoken(x, smooth=None, compute_dtype=None, saturate=False):
+    """(q int8 [M,K], scale fp32 [M]) -- see fmsmo_quant_act_i8_pertoken."""
+    _need_gpu(x, smooth)
+    x = _rows(x)
+    M, K = x.shape
+    if smooth is not None:
+        smooth = smooth.detach().reshape(-1).contiguous()
+        if smooth.numel() != K:
+            raise ValueError("smooth scale must have K elements")
+    if compute_dtype is None:
+        compute_dtype = x.dtype if smooth is None else torch.promote_types(x.dtype, smooth.dtype)
+    q = torch.empty((M, K), dtype=torch.int8, device=x.device)
+    scale = torch.empty((M,), dtype=torch.float32, device=x.device)
+    with torch.cuda.device(x.device):
+        L.call("fmsmo_quant_act_i8_pertoken", x.data_ptr(), _dt(x), _ld(x), _ptr(smooth),
+               _dt(smooth) if smooth is not None else 0, _DT[compute_dtype], int(bool(saturate)),
+               q.data_ptr(), K, scale.data_ptr(), M, K, _stream(x))
+    return q, scale
+
+
+def quant_act_i8_static(x, scale: float, zp: int, sym: int):
+    _need_gpu(x)
+    x = _rows(x)
+    M, K = x.shape
+    q = torch.empty((M, K), dtype=torch.int8, device=x.device)
+    with torch.cuda.device(x.device):
+        L.call("fmsmo_quant_act_i8_static", x.data_ptr(), _dt(x), _ld(x), float(scale), int(zp),
+               int(sym), q.data_ptr(), K, M, K, _stream(x))
+    return q
+
+
+def quant_act_fp8_pertoken(x, variant=L.FP8_LINEAR, static_scale=None):
+    """(q e4m3 [M,K], scale fp32 [M] or the [1] static scale)."""
+    _need_gpu(x)
+    x = _rows(x)
+    M, K = x.shape
+    q = torch.empty((M, K), dtype=torch.float8_e4m3fn, device=x.device)
+    if static_scale is not None:
+        scale = _scale_vec(static_scale, 1, x.device, "static_scale")[:1].contiguous()
+    else:
+        scale = torch.empty((M,), dtype=torch.float32, device=x.device)
+    with torch.cuda.device(x.device):
+        L.call("fmsmo_quant_act_fp8_pertoken", x.data_ptr(), _dt(x), _ld(x), int(variant),
+               int(static_scale is not None), q.data_ptr(), K, scale.data_ptr(), M, K, _stream(x))
+    return q, scale
+
+
+# ------------------------------------------------------------------------------------ GEMMs
+def _check_ab(a, w, dtype):
+    _need_gpu(a, w)
+    if a.dtype != dtype or w.dtype != dtype:
+        raise TypeError(f"operands must be {dtype}, got {a.dtype} and {w.dtype}")
+    a, w = _rows(a), _rows(w)
+    if a.shape[1] != w.shape[1]:
+        raise ValueError(f"K mismatch: a is {tuple(a.shape)}, w is {tuple(w.shape)} ([N,K] layout)")
+    return a, w
+
+
+def gemm_i8_i32(a, w):
+    """int32 [M,N] = a int8 [M,K] . w int8 [N,K]^T."""
+    a, w = _check_ab(a, w, torch.int8)
+    M, K = a.shape
+    N = w.shape[0]
+    c = torch.empty((M, N), dtype=torch.int32, device=a.device)
+    with torch.cuda.device(a.device):
+        L.call("fmsmo_gemm_i8_i32", a.data_ptr(), _ld(a), w.data_ptr(), _ld(w), c.data_ptr(), N,
+               M, N, K, _stream(a))
+    return c
+
+
+def gemm_i8_dq(a, w, a_scale, w_scale, bias=None, out_dtype=torch.float16, exact_ref=True,
+               force_gemv=False):
+    a, w = _check_ab(a, w, torch.int8)
+    M, K = a.shape
+    N = w.shape[0]
+    a_scale = _scale_vec(a_scale, M, a.device, "a_scale")
+    w_scale = _scale_vec(w_scale, N, a.device, "w_scale")
+    if bias is not None:
+        _need_gpu(bias)
+        bias = bias.detach().reshape(-1).contiguous()
+        if bias.numel() != N:
+            raise ValueError("bias must have N elements")
+    y = torch.empty((M, N), dtype=out_dtype, device=a.device)
+    fn = "fmsmo_gemv_i8_dq" if force_gemv else "fmsmo_gemm_i8_dq"
+    with torch.cuda.device(a.device):
+        L.call(fn, a.data_ptr(), _ld(a), w.data_ptr(), _ld(w), a_scale.data_ptr(),
+               a_scale.numel(), w_scale.data_ptr(), w_scale.numel(), _ptr(bias),
+               _dt(bias) if bias is not None else 0, L.EPI_REF_F16 if exact_ref else L.EPI_F32,
+               y.data_ptr(), _DT[out_dtype], N, M, N, K, _stream(a))
+    return y
+
+
+def gemm_fp8_dq(a, w, a_scale, w_scale, bias=None, out_dtype=torch.bfloat16, force_gemv=False):
+    a, w = _check_ab(a, w, torch.float8_e4m3fn)
+    M, K = a.shape
+    N = w.shape[0]
+    a_scale = _scale_vec(a_scale, M, a.device, "a_scale")
+    w_scale = _scale_vec(w_scale, N, a.device, "w_scale")
+    if bias is not None:
+        _need_gpu(bias)
+        bias = bias.detach().reshape(-1).contiguous()
+    y = torch.empty((M, N), dtype=out_dtype, device=a.device)
+    fn = "fmsmo_gemv_fp8_dq" if force_gemv else "fmsmo_gemm_fp8_dq"
+    with torch.cuda.device(a.device):
+        L.call(fn, a.data_ptr(), _ld(a), w.data_ptr(), _ld(w), a_scale.data_ptr(),
+               a_scale.numel(), w_scale.data_ptr(), w_scale.numel(), _ptr(bias),
+               _dt(bias) if bias is not None else 0, y.data_ptr(), _DT[out_dtype], N, M, N, K,
+               _stream(a))
+    return y
+
+
+def grouped_gemm_i8_dq(a, w, offsets, a_scale, w_scale, bias=None, out_dtype=torch.float16,
+                       exact_ref=True):
+    """a int8 [T,K] rows sorted by expert, w int8 [E,N,K], offsets int32 [E+1] (device),
+    a_scale fp32 [T], w_scale fp32 [E,N], bias [E,N] or None -> [T,N]."""
+    _need_gpu(a, w, offsets)
+    if a.dtype != torch.int8 or w.dtype != torch.int8 or w.dim() != 3:
+        raise TypeError("a must be int8 [T,K], w int8 [E,N,K]")
+    a = _rows(a)
+    w = w.contiguous()
+    T, K = a.shape
+    E, N, K2 = w.shape
+    if K2 != K or offsets.numel() != E + 1 or offsets.dtype != torch.int32:
+        raise ValueError("shape mismatch (w [E,N,K], offsets int32 [E+1])")
+    a_scale = _scale_vec(a_scale, T, a.device, "a_scale")
+    w_scale = w_scale.detach().to(torch.float32).reshape(-1).contiguous()
+    if a_scale.numel() != T or w_scale.numel() != E * N:
+        raise ValueError("a_scale must be [T], w_scale [E,N]")
+    if bias is not None:
+        bias = bias.detach().reshape(-1).contiguous()
+        if bias.numel() != E * N:
+            raise ValueError("bias must be [E,N]")
+    y = torch.empty((T, N), dtype=out_dtype, device=a.device)
+    with torch.cuda.device(a.device):
+        L.call("fmsmo_grouped_gemm_i8_dq", a.data_ptr(), _ld(a), w.data_ptr(), K, N * K,
+               offsets.contiguous().data_ptr(), E, T, a_scale.data_ptr(), w_scale.data_ptr(),
+               _ptr(bias), _dt(bias) if bias is not None else 0,
+               L.EPI_REF_F16 if exact_ref else L.EPI_F32, y.data_ptr(), _DT[out_dtype], N, N, K,
+               _stream(a))
+    return y
+
+
+# ----------------------------------------------------------------------- chunked accumulation
+def matmul_chunk(a, w, c=None, chunk_size=64, chunk_trun_bits=0, max_acc_bits=32,
+                 truncate_then_accumulate=True, clamp_acc_to_dl16=False):
+    """a [M,K], w [N,K] (int8 | float8_e4m3fn | float16 | bfloat16 | float32) -> int32 / fp32 [M,N]."""
+    _need_gpu(a, w, c)
+    if a.dtype != w.dtype or a.dtype not in _OPDT:
+        raise TypeError(f"unsupported operand dtypes {a.dtype}, {w.dtype}")
+    a, w = _rows(a), _rows(w)
+    M, K = a.shape
+    N = w.shape[0]
+    if w.shape[1] != K:
+        raise ValueError("K mismatch")
+    esz = a.element_size()
+    per16 = 16 // esz
+    if K % per16 or _ld(a) % per16 or _ld(w) % per16:  # zero-pad K: contributes nothing to any chunk
+        Kp = (K + 63) // 64 * 64
+        a = torch.nn.functional.pad(a.view(_BITS[esz]), (0, Kp - K)).view(a.dtype)
+        w = torch.nn.functional.pad(w.view(_BITS[esz]), (0, Kp - K)).view(w.dtype)
+        K = Kp
+    acc_dtype = torch.int32 if a.dtype == torch.int8 else torch.float32
+    d = torch.empty((M, N), dtype=acc_dtype, device=a.device)
+    if c is not None:
+        if c.shape != (M, N):
+            raise ValueError("C shape is inconsistent with A B.")
+        c = c.to(acc_dtype).contiguous()
+    with torch.cuda.device(a.device):
+        if a.dtype == torch.int8:
+            L.call("fmsmo_matmul_chunk_i8", a.data_ptr(), _ld(a), w.data_ptr(), _ld(w), _ptr(c),
+                   d.data_ptr(), N, M, N, K, int(chunk_size), int(chunk_trun_bits),
+                   int(max_acc_bits), int(bool(truncate_then_accumulate)), _stream(a))
+        else:
+            L.call("fmsmo_matmul_chunk_fp", a.data_ptr(), _ld(a), w.data_ptr(), _ld(w),
+                   _OPDT[a.dtype], _ptr(c), d.data_ptr(), N, M, N, K, int(chunk_size),
+                   int(chunk_trun_bits), int(bool(clamp_acc_to_dl16)),
+                   int(bool(truncate_then_accumulate)), _stream(a))
+    return d

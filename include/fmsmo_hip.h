@@ -1,0 +1,225 @@
+/*
+ * fmsmo_hip.h -- C ABI of the gfx950 (MI355X) quantized-linear kernels.
+ *
+ * Every entry point takes raw device pointers, element counts / leading dimensions in ELEMENTS,
+ * small enums and a HIP stream handle (passed as void*; NULL = the default stream).  Nothing is
+ * allocated, freed or synchronised inside the library: the caller owns inputs, outputs and
+ * lifetimes, and kernels are enqueued asynchronously on the given stream.  Every function
+ * returns FMSMO_OK (0) or a negative-free small error code; fmsmo_status_str() names it.
+ *
+ * Matrix convention (the one the reference's int8 GEMM extensions use): activations A are
+ * [M,K] row-major, weights B are stored [N,K] row-major (nn.Linear layout, i.e. the memory the
+ * reference's `W.t()` view points at), outputs are [M,N] row-major.
+ *
+ * Each declaration cites the interface of the reference (paths relative to the root of
+ * foundation-model-stack/fms-model-optimizer) whose arithmetic it reproduces.
+ */
+#ifndef FMSMO_HIP_H_
+#define FMSMO_HIP_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FMSMO_ABI_VERSION 1
+
+typedef void* fmsmo_stream_t; /* hipStream_t */
+
+/* 16/32-bit floating types of activations, scales, biases and outputs. */
+enum { FMSMO_F16 = 0, FMSMO_BF16 = 1, FMSMO_F32 = 2 };
+
+/* Element type of the 8-bit (or 16-bit) GEMM operands of the chunked matmul. */
+enum { FMSMO_OP_I8 = 0, FMSMO_OP_E4M3 = 1, FMSMO_OP_F16 = 2, FMSMO_OP_BF16 = 3, FMSMO_OP_F32 = 4 };
+
+/* Status codes. */
+enum {
+  FMSMO_OK = 0,
+  FMSMO_ERR_NULL = 1,        /* a required pointer is NULL                          */
+  FMSMO_ERR_SHAPE = 2,       /* negative size, leading dimension too small, ...     */
+  FMSMO_ERR_ALIGN = 3,       /* pointer / leading dimension not 16-byte aligned     */
+  FMSMO_ERR_UNSUPPORTED = 4, /* enum value or size outside what the kernels handle  */
+  FMSMO_ERR_LAUNCH = 5       /* hipLaunchKernel / hipGetLastError reported an error */
+};
+
+/* Epilogue arithmetic of the fused int8 GEMM. */
+enum {
+  /* y = f16( f32(acc) * f32( f16(a_scale[m]*w_scale[n]) ) + f32(bias[n]) ): the exact operation
+     order of iaddmm_int's plain branch (fms_mo/modules/linear.py:1185-1188), then a cast to the
+     output dtype (linear.py:1338). */
+  FMSMO_EPI_REF_F16 = 0,
+  /* y = out( f32(acc) * (a_scale[m]*w_scale[n]) + f32(bias[n]) ) with the scale product kept in
+     fp32 (no fp16 rounding of the scale, single rounding to the output dtype). */
+  FMSMO_EPI_F32 = 1
+};
+
+int fmsmo_abi_version(void);
+const char* fmsmo_status_str(int status);
+/* hipGetLastError text of the most recent FMSMO_ERR_LAUNCH on this thread ("" if none). */
+const char* fmsmo_last_error(void);
+
+/* ------------------------------------------------------------------------------------------
+ * 1. Activation quantizers (one pass over x: read 2-4 B, write 1 B per element).
+ * ------------------------------------------------------------------------------------------ */
+
+/*
+ * Dynamic symmetric per-token int8 quantizer, optionally preceded by the SmoothQuant divide.
+ *   x'      = smooth ? rnd_T(x / smooth[k]) : x
+ *   amax_m  = max_k |x'_mk| ; s_m = rnd_T( max(amax_m, rnd_T(1e-5)) / 127 )
+ *   q_mk    = int8( rint( rnd_T(x'_mk / s_m) ) )          (half-to-even)
+ * T = compute_dtype (FMSMO_F16/BF16/F32) is the dtype in which torch would evaluate the
+ * expression (x's dtype, or fp32 when an fp32 SmoothQuant scale promotes it).
+ * saturate = 0 reproduces the reference: no clamp, 128 wraps to -128 on the int8 cast (reachable
+ * only for T = bf16); saturate = 1 clamps to [-127,127].
+ * scale[m] receives s_m as fp32 (exactly representable).
+ * Reference: QLinearINT8Deploy.qa_dynamic_max_qfunc (fms_mo/modules/linear.py:1085-1100), the
+ * divide in QLinearINT8Deploy.forward (:1331-1334), QMaxDynamic.forward
+ * (fms_mo/quant/quantizers.py:3531-3534).
+ */
+int fmsmo_quant_act_i8_pertoken(const void* x, int x_dtype, int64_t ldx, const void* smooth,
+                                int smooth_dtype, int compute_dtype, int saturate, int8_t* q,
+                                int64_t ldq, float* scale, int64_t M, int64_t K,
+                                fmsmo_stream_t stream);
+
+/*
+ * Static per-tensor int8 quantizer:  q = clamp( rint( x/scale + zp - 128 + sym ), -128, 127 )
+ * evaluated in fp32 in exactly that order.  Reference: QLinearINT8Deploy.qa_raw_qfunc
+ * (fms_mo/modules/linear.py:1061-1071); also the quantize step of fms_mo::q_iaddmm_dq
+ * (fms_mo/custom_ext_kernels/utils.py:770) with sym = 0.
+ */
+int fmsmo_quant_act_i8_static(const void* x, int x_dtype, int64_t ldx, float scale, int zp,
+                              int sym, int8_t* q, int64_t ldq, int64_t M, int64_t K,
+                              fmsmo_stream_t stream);
+
+/* Variants of the per-token FP8 (OCP e4m3fn) activation quantizer. */
+enum {
+  /* s_m = max(amax_m/448, 1e-12) in fp32; q = e4m3( clamp(f32(x)/s_m, -448, 448) ).
+     Cast and clamp: _quantize_affine_float8_custom (fms_mo/aiu_addons/fp8/fp8_linear.py:54-72);
+     scale: tests/aiu_addons/test_fp8_addon.py:65-79 (the dynamic-scale rule itself lives in
+     torchao, outside the reference tree). */
+  FMSMO_FP8_LINEAR = 0,
+  /* s_m = max( rnd_T(amax_m/448), 1e-5 ) in x's dtype T; q = e4m3( rnd_T(x/s_m) ), no clamp.
+     LinearFuncFPxFwdBwd.forward (fms_mo/modules/linear.py:1939-1948). */
+  FMSMO_FP8_FPXACC = 1,
+  /* as FMSMO_FP8_FPXACC, then |q| < 0.0087890625 flushed to zero (linear.py:1949-1953). */
+  FMSMO_FP8_FPXACC_DL8 = 2
+};
+/* scale != NULL on input with static_scale != 0: use scale[0] for every row (per-tensor static
+   activation scale, fp8_linear.py:150-161) instead of the dynamic per-token one. */
+int fmsmo_quant_act_fp8_pertoken(const void* x, int x_dtype, int64_t ldx, int variant,
+                                 int static_scale, uint8_t* q, int64_t ldq, float* scale,
+                                 int64_t M, int64_t K, fmsmo_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * 2. W8A8 GEMMs on MFMA.   C[M,N] = A[M,K] . B[N,K]^T
+ *    Requirements: K % 16 == 0, lda/ldb % 16 == 0, A and B 16-byte aligned.
+ * ------------------------------------------------------------------------------------------ */
+
+/*
+ * int8 x int8 -> int32, exact (no saturation can occur for K < 2^17).
+ * Reference: cutlass_mm.run (fms_mo/custom_ext_kernels/cutlass_i8i32gemm.cu:100-120, .cpp:34),
+ * torch.ops.cutlass_gemm.i8i32nt (custom_ext_kernels/utils.py:336-364),
+ * gemm_i8<int32_t,NT> / torch.ops.mygemm.gemm_nt_i8i32 (ext_kernel_cublas.cpp:103-195,
+ * utils.py:186-206), torch.ops.fms_mo.imatmul (utils.py:690-720).
+ */
+int fmsmo_gemm_i8_i32(const int8_t* a, int64_t lda, const int8_t* b, int64_t ldb, int32_t* c,
+                      int64_t ldc, int64_t M, int64_t N, int64_t K, fmsmo_stream_t stream);
+
+/*
+ * int8 GEMM with the dequantizing epilogue fused:  y = acc * (a_scale x w_scale) + bias.
+ * a_scale: fp32 [M] (a_scale_n == M) or one value (a_scale_n == 1); w_scale likewise [N] or 1;
+ * bias: [N] of bias_dtype or NULL.  epilogue: FMSMO_EPI_REF_F16 | FMSMO_EPI_F32.
+ * M <= 16 is routed to the weight-streaming (HBM-bound) kernel.
+ * Reference: QLinearINT8Deploy.iaddmm_int, plain branch (fms_mo/modules/linear.py:1177-1188),
+ * torch.ops.fms_mo.iaddmm (custom_ext_kernels/utils.py:729-737).
+ */
+int fmsmo_gemm_i8_dq(const int8_t* a, int64_t lda, const int8_t* b, int64_t ldb,
+                     const float* a_scale, int64_t a_scale_n, const float* w_scale,
+                     int64_t w_scale_n, const void* bias, int bias_dtype, int epilogue, void* y,
+                     int y_dtype, int64_t ldy, int64_t M, int64_t N, int64_t K,
+                     fmsmo_stream_t stream);
+
+/*
+ * e4m3 x e4m3 -> fp32 accumulate, y = out( acc * a_scale[m] * w_scale[n] + bias[n] ).
+ * Reference: the torch._scaled_mm call made through addmm_float8_unwrapped_inference in
+ * FP8Linear.forward (fms_mo/aiu_addons/fp8/fp8_linear.py:275-283); CPU semantics
+ * _scaled_mm_cpu_out (fms_mo/aiu_addons/fp8/fp8_spyre_op.py:35-60).
+ */
+int fmsmo_gemm_fp8_dq(const uint8_t* a, int64_t lda, const uint8_t* b, int64_t ldb,
+                      const float* a_scale, int64_t a_scale_n, const float* w_scale,
+                      int64_t w_scale_n, const void* bias, int bias_dtype, void* y, int y_dtype,
+                      int64_t ldy, int64_t M, int64_t N, int64_t K, fmsmo_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * 3. Skinny-M (decode) variants, M <= 16: stream the weights once from HBM.
+ *    Same arithmetic and arguments as the two *_dq GEMMs above.
+ * ------------------------------------------------------------------------------------------ */
+int fmsmo_gemv_i8_dq(const int8_t* a, int64_t lda, const int8_t* b, int64_t ldb,
+                     const float* a_scale, int64_t a_scale_n, const float* w_scale,
+                     int64_t w_scale_n, const void* bias, int bias_dtype, int epilogue, void* y,
+                     int y_dtype, int64_t ldy, int64_t M, int64_t N, int64_t K,
+                     fmsmo_stream_t stream);
+int fmsmo_gemv_fp8_dq(const uint8_t* a, int64_t lda, const uint8_t* b, int64_t ldb,
+                      const float* a_scale, int64_t a_scale_n, const float* w_scale,
+                      int64_t w_scale_n, const void* bias, int bias_dtype, void* y, int y_dtype,
+                      int64_t ldy, int64_t M, int64_t N, int64_t K, fmsmo_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * 4. Chunked reduced-precision accumulation ("chunk-truncate") matmuls.
+ *    Per K-chunk of chunk_size: p = dot(a_chunk, b_chunk) in a fresh accumulator; p is
+ *    range-clamped / LSB-rounded; acc += p (truncate_then_accumulate != 0) or the running
+ *    accumulator itself is rounded after each chunk (== 0).  A K tail is zero-padded.
+ * ------------------------------------------------------------------------------------------ */
+
+/*
+ * int8 -> int32.  p = clamp(p, -2^(b-1), 2^(b-1)-1) if b = max_acc_bits < 32;
+ * p = ((p + 2^(t-1)) >> t) << t if t = chunk_trun_bits > 0 (arithmetic shift).
+ * c_in (int32 [M,N], may be NULL, may alias d) is the initial accumulator.
+ * chunk_size: a power of two >= 32.
+ * Reference: imatmul_kernel (fms_mo/custom_ext_kernels/triton_kernels.py:211-302) as launched
+ * by tl_matmul_chunk_truncate (:468-621); the PyTorch chunk loop of iaddmm_int
+ * (fms_mo/modules/linear.py:1142-1175) gives the same values after its final 2^t scaling.
+ */
+int fmsmo_matmul_chunk_i8(const int8_t* a, int64_t lda, const int8_t* b, int64_t ldb,
+                          const int32_t* c_in, int32_t* d, int64_t ldd, int64_t M, int64_t N,
+                          int64_t K, int chunk_size, int chunk_trun_bits, int max_acc_bits,
+                          int truncate_then_accumulate, fmsmo_stream_t stream);
+
+/*
+ * Floating point -> fp32.  op_dtype: FMSMO_OP_E4M3 (1-byte operands), FMSMO_OP_F16 or
+ * FMSMO_OP_BF16 (2-byte operands), FMSMO_OP_F32 (4-byte operands).  lda / ldb / K count
+ * ELEMENTS.  On the IEEE-754 word u of p:
+ *   u = (u + (t ? 1<<(t-1) : 0)) & ~((1<<t)-1),  t = chunk_trun_bits in [0,22];
+ * clamp_dl16 != 0 forces t = 14 and then p >= 8581545984 -> +inf, p <= -8581545984 -> -inf,
+ * |p| < 4.665707820095122e-10 -> 0.   The order of the fp32 additions inside one chunk is the
+ * MFMA unit's (the reference leaves it to tl.dot).  chunk_size: power of two >= 32 (e4m3) or
+ * >= 16 (f16/bf16/f32).  c_in: optional fp32 initial accumulator (D = A.B + C).
+ * Reference: matmul_kernel / matmul_kernel_DABC / round_and_trun
+ * (fms_mo/custom_ext_kernels/triton_kernels.py:96-205,305-423,432-465).
+ */
+int fmsmo_matmul_chunk_fp(const void* a, int64_t lda, const void* b, int64_t ldb, int op_dtype,
+                          const float* c_in, float* d, int64_t ldd, int64_t M, int64_t N,
+                          int64_t K, int chunk_size, int chunk_trun_bits, int clamp_dl16,
+                          int truncate_then_accumulate, fmsmo_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * 5. Grouped int8 GEMM for mixture-of-experts FFNs (uneven rows per expert, one launch).
+ *    Rows of A are sorted by expert; expert e owns rows [offsets[e], offsets[e+1]).
+ *    B is [E][N][K] (expert stride ldb_e elements), w_scale [E][N], bias [E][N] or NULL.
+ *    offsets is a DEVICE array of E+1 int32.  total_rows = offsets[E] must be given on the
+ *    host (it sizes the grid).  Arithmetic per expert == fmsmo_gemm_i8_dq.
+ *    The reference has no grouped type: every expert w1/w2/w3 is its own QLinearINT8Deploy
+ *    (fms_mo/utils/dq_utils.py:86-106), so each expert's rows must equal that module's output.
+ * ------------------------------------------------------------------------------------------ */
+int fmsmo_grouped_gemm_i8_dq(const int8_t* a, int64_t lda, const int8_t* b, int64_t ldb,
+                             int64_t ldb_e, const int32_t* offsets, int num_experts,
+                             int64_t total_rows, const float* a_scale, const float* w_scale,
+                             const void* bias, int bias_dtype, int epilogue, void* y,
+                             int y_dtype, int64_t ldy, int64_t N, int64_t K,
+                             fmsmo_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FMSMO_HIP_H_ */

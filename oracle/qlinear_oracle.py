@@ -1,0 +1,400 @@
+"""CPU restatement of the reference's quantized-linear arithmetic.  TEST INFRASTRUCTURE ONLY.
+
+This module is the checker for the HIP kernels: only ``tests/``, ``__graft_entry__.smoke()`` and
+the ``cpu_baseline`` leg of ``bench.py`` may import it.  Nothing in the product package imports
+it, and it is never the thing that is measured or shipped.
+
+Every function follows one piece of foundation-model-stack/fms-model-optimizer (paths relative to
+that repository) and keeps its operation order, dtypes and rounding, using plain torch CPU ops
+(torch is the library the reference itself computes with).  Integer products are exact
+(``torch._int_mm`` / int64 accumulation), never ``torch.matmul`` on int8 (which wraps to int8).
+
+How each function is pinned (see tests/test_oracle_*.py):
+  * act quantizers      -- closed form re-evaluated with exact rational arithmetic (fractions)
+                           and explicit IEEE roundings; special rows (all-zero, single +-amax,
+                           exact .5 ties); the C restatement in oracle/qlinear_ref.c
+  * weight quantizer    -- invariants (|w| <= 127, row arg-max hits +-127) and
+                           torch.fake_quantize_per_channel_affine away from ties
+  * int GEMM            -- brute-force int64 loops; the C restatement
+  * epilogue            -- exact rational re-evaluation
+  * chunked int / fp    -- brute force per chunk; bit-level closed form of the truncation
+                           (C restatement, all exponent classes, NaN/Inf)
+  * fp8 cast            -- all 256 codes and all midpoints against torch's own cast
+  * i8i8_aiu            -- the six stored vectors of the reference's own test-suite
+                           (tests/golden/ref_w-*_a-*_sq-N.pt)
+  * FP8Linear dynamic scale (computed inside torchao 0.11, not in the reference tree):
+                           PARITY UNPINNED -- the rule used is the one of the reference's test
+                           helper (tests/aiu_addons/test_fp8_addon.py:65-79).
+"""
+from __future__ import annotations
+
+import torch
+
+E4M3_MAX = 448.0
+DL8_MIN = 0.0087890625
+DL16_MAX = 8581545984.0
+DL16_MIN = 4.665707820095122e-10
+
+
+# ------------------------------------------------------------------------------------------
+# SmoothQuant scale
+# ------------------------------------------------------------------------------------------
+def smoothq_scale_qlinear(weight: torch.Tensor, act_scale: torch.Tensor, alpha: float, x_dtype):
+    """QLinear.get_smoothq_scale (fms_mo/modules/linear.py:345-368): ``[1.0]`` when the stored
+    activation scale sums to zero, else clamp(a^alpha / wmax^(1-alpha), 1e-5) cast to x's dtype."""
+    if act_scale.sum().item() == 0.0:
+        return torch.tensor([1.0]).to(x_dtype)
+    wmax = weight.abs().max(dim=0, keepdim=True)[0].clamp(min=1e-5)
+    return (act_scale.pow(alpha) / wmax.pow(1.0 - alpha)).clamp(min=1e-5).to(x_dtype)
+
+
+def smoothq_scale_deploy(weight: torch.Tensor, act_scale: torch.Tensor, alpha):
+    """QLinearINT8Deploy.from_fms_mo (linear.py:800-817): computed only if every a_k != 0, kept in
+    the dtype of the stored activation scale; otherwise ``[1.0]`` in the weight dtype."""
+    if not torch.all(act_scale != 0).item():
+        return torch.tensor([1.0], dtype=weight.dtype)
+    wmax = weight.abs().max(dim=0, keepdim=True)[0].clamp(min=1e-5)
+    return (act_scale**alpha / wmax ** (1.0 - alpha)).clamp(min=1e-5).to(act_scale.dtype)
+
+
+# ------------------------------------------------------------------------------------------
+# Activation quantizers
+# ------------------------------------------------------------------------------------------
+def quant_act_pertoken_i8(x: torch.Tensor, smooth: torch.Tensor | None = None, saturate=False):
+    """qa_dynamic_max_qfunc with reduce dim -1 (linear.py:1085-1100) after the optional
+    ``x / smoothq_scale`` of QLinearINT8Deploy.forward (:1331-1334).
+
+    Returns (q int8 [M,K], scale [M,1] in the dtype torch promotion gives, x' the divided input).
+    ``saturate`` is NOT reference behaviour: it clamps to +-127 before the int8 cast."""
+    if smooth is not None:
+        x = x / smooth  # fp16 / fp32 tensor -> fp32 (torch type promotion)
+    amax = x.abs().max(dim=-1, keepdim=True)[0]
+    scale = amax.clamp(min=1e-5).div(127)
+    r = torch.round(x / scale)
+    if saturate:
+        r = r.clamp(-127, 127)
+    else:
+        # the reference's float -> int8 cast wraps 128 to -128 (only reachable in bfloat16);
+        # make the wrap explicit instead of relying on an out-of-range cast
+        r = torch.where(r > 127, r - 256, r)
+    return r.to(torch.int8), scale, x
+
+
+def fake_quant_act_pertoken(x: torch.Tensor):
+    """QMaxDynamic.forward, dim=-1 (fms_mo/quant/quantizers.py:3531-3534): Q/dQ in x's dtype."""
+    amax = x.abs().max(dim=-1, keepdim=True)[0]
+    scales = amax.clamp(min=1e-5).div(127)
+    return x.div(scales).round().mul(scales)
+
+
+def quant_act_static_raw(x: torch.Tensor, scale: torch.Tensor, zp: int, sym: int):
+    """qa_raw_qfunc (linear.py:1061-1071)."""
+    return torch.clamp((x / scale + zp - 128 + sym).round(), -128, 127).to(torch.int8)
+
+
+# ------------------------------------------------------------------------------------------
+# Weight quantizers
+# ------------------------------------------------------------------------------------------
+def qmax_perch_clipval(weight: torch.Tensor):
+    """Qmax.forward, perCh symmetric branch (quantizers.py:3058-3063): cv_n = max_k |W_nk|."""
+    return torch.max(weight.abs().reshape([weight.shape[0], -1]), dim=1).values
+
+
+def fake_quant_weight_perch(weight: torch.Tensor, cv: torch.Tensor):
+    """QmaxPerChSTE.forward (quantizers.py:3190-3224), 8 bits: scale = cv*2/254."""
+    scale = cv * 2 / 254
+    return torch.fake_quantize_per_channel_affine(
+        weight.float(), scale.float(), torch.zeros_like(scale).float(), axis=0,
+        quant_min=-127, quant_max=127,
+    ).to(weight.dtype)
+
+
+def quant_weight_deploy(weight: torch.Tensor, w_cv: torch.Tensor, smoothq_scale: torch.Tensor):
+    """from_fms_mo weight path (linear.py:821,863-871).  Returns (int8 [N,K], w_scale)."""
+    w_scale = w_cv * 2 / 254
+    w = torch.round((weight * smoothq_scale).t() / w_scale).clamp(-127, 127).t()
+    return w.to(torch.int).to(torch.int8), w_scale
+
+
+# ------------------------------------------------------------------------------------------
+# Integer GEMM and epilogue
+# ------------------------------------------------------------------------------------------
+def int_gemm(a_i8: torch.Tensor, w_i8: torch.Tensor) -> torch.Tensor:
+    """Exact int32 C = A[M,K] . W[N,K]^T (cutlass_i8i32gemm.cu:29-62; utils.py:690-714)."""
+    M, K = a_i8.shape
+    if M > 16 and K % 8 == 0 and w_i8.shape[0] % 8 == 0:
+        return torch._int_mm(a_i8.contiguous(), w_i8.t())
+    return (a_i8.to(torch.int64) @ w_i8.to(torch.int64).t()).to(torch.int32)
+
+
+def epilogue_ref(acc: torch.Tensor, input_scale: torch.Tensor, w_scale: torch.Tensor,
+                 bias: torch.Tensor | None, org_dtype=torch.float16):
+    """iaddmm_int plain branch (linear.py:1185-1188) then ``.to(org_dtype)`` (:1338)."""
+    y = acc.float() * (input_scale * w_scale).to(torch.float16)
+    if bias is not None:
+        y = y + bias
+    return y.to(torch.float16).to(org_dtype)
+
+
+def epilogue_f32(acc, input_scale, w_scale, bias, out_dtype):
+    """Not reference arithmetic: the fp32-scale epilogue of FMSMO_EPI_F32 (fused multiply-add in
+    fp64 is exact enough to give the correctly rounded fp32 fma for these magnitudes)."""
+    sc = input_scale.float() * w_scale.float()
+    y = acc.double() * sc.double()
+    if bias is not None:
+        y = y + bias.double()
+    return y.float().to(out_dtype)
+
+
+# ------------------------------------------------------------------------------------------
+# Whole modules
+# ------------------------------------------------------------------------------------------
+def qlinear_forward(x, weight, bias, act_scale=None, alpha=0.5, w_clip_val=None):
+    """QLinear.forward, qa_mode='pertokenmax', qw_mode='maxperCh', 8/8 bits (linear.py:248-305).
+
+    ``w_clip_val=None`` behaves like a training-mode first call (clip values = fresh abs-max)."""
+    if act_scale is not None:
+        s = smoothq_scale_qlinear(weight, act_scale, alpha, x.dtype)
+    else:
+        s = torch.tensor([1.0]).to(x.dtype)
+    qinput = fake_quant_act_pertoken(x / s).to(x.dtype)
+    ws = weight * s
+    cv = qmax_perch_clipval(ws) if w_clip_val is None else w_clip_val
+    qweight = fake_quant_weight_perch(ws, cv).to(weight.dtype)
+    return torch.nn.functional.linear(qinput, qweight, bias)
+
+
+def deploy_prepare(weight, bias, w_clip_val, act_scale=None, alpha=0.5):
+    """from_fms_mo with use_dynamic_max_act_Qfunc=-1, symmetric activations (linear.py:717-920):
+    returns the module buffers {weight int8, w_scale, smoothq_scale, bias}."""
+    if act_scale is not None:
+        sq = smoothq_scale_deploy(weight, act_scale, torch.tensor([alpha], dtype=torch.float32))
+    else:
+        sq = torch.tensor([1.0], dtype=weight.dtype)
+    w_i8, w_scale = quant_weight_deploy(weight, w_clip_val, sq)
+    # symmetric activations: corr_term = 0, bias <- bias.float() - 0, cast back to W dtype
+    new_bias = None if bias is None else (bias.float() - 0.0).to(weight.dtype)
+    return {"weight": w_i8, "w_scale": w_scale, "smoothq_scale": sq, "bias": new_bias}
+
+
+def deploy_forward(x, bufs):
+    """QLinearINT8Deploy.forward + iaddmm_int plain branch (linear.py:1309-1338,1115-1188).
+    Returns every intermediate: q_x, input_scale, acc, y."""
+    org_dtype = x.dtype
+    x2 = x.reshape(-1, x.shape[-1])
+    sq = bufs["smoothq_scale"]
+    use_sq = torch.all(sq != 1).item()
+    q_x, input_scale, _ = quant_act_pertoken_i8(x2, sq if use_sq else None)
+    acc = int_gemm(q_x, bufs["weight"])
+    bias = bufs["bias"]
+    y = acc.float() * (input_scale * bufs["w_scale"]).to(torch.float16)
+    y = (y + bias) if bias is not None else y
+    y = y.to(torch.float16).reshape(tuple(x.shape[:-1]) + (bufs["weight"].shape[0],))
+    return {"q_x": q_x, "input_scale": input_scale, "acc": acc, "y": y.to(org_dtype)}
+
+
+def deploy_forward_fp(x, bufs):
+    """iaddmm_FP (linear.py:1190-1211): the reference's fallback without an int kernel; needs
+    every buffer in x's dtype."""
+    x2 = x.reshape(-1, x.shape[-1])
+    sq = bufs["smoothq_scale"]
+    q_x, input_scale, _ = quant_act_pertoken_i8(x2, sq if torch.all(sq != 1).item() else None)
+    y = torch.matmul(q_x * input_scale, bufs["weight"].t() * bufs["w_scale"]) + bufs["bias"]
+    return y.reshape(tuple(x.shape[:-1]) + (bufs["weight"].shape[0],)).to(x.dtype)
+
+
+# ------------------------------------------------------------------------------------------
+# Chunked accumulation
+# ------------------------------------------------------------------------------------------
+def chunk_matmul_i8(a_i8, w_i8, c=None, chunk_size=64, trun_bits=0, max_acc_bits=32,
+                    truncate_then_accumulate=True):
+    """imatmul_kernel (fms_mo/custom_ext_kernels/triton_kernels.py:262-302).  a [M,K], w [N,K]."""
+    M, K = a_i8.shape
+    N = w_i8.shape[0]
+    acc = torch.zeros(M, N, dtype=torch.int64) if c is None else c.to(torch.int64).clone()
+    rb = (1 << (trun_bits - 1)) if trun_bits > 0 else 0
+    lo, hi = -(1 << (max_acc_bits - 1)), (1 << (max_acc_bits - 1)) - 1
+
+    def wrap32(t):
+        return ((t + (1 << 31)) % (1 << 32)) - (1 << 31)
+
+    for k0 in range(0, K, chunk_size):
+        p = a_i8[:, k0:k0 + chunk_size].to(torch.int64) @ w_i8[:, k0:k0 + chunk_size].to(torch.int64).t()
+        if not truncate_then_accumulate:
+            p = wrap32(p + acc)
+        if max_acc_bits < 32:
+            p = p.clamp(lo, hi)
+        if trun_bits != 0:
+            p = wrap32(wrap32(p + rb) >> trun_bits << trun_bits)
+        acc = wrap32(acc + p) if truncate_then_accumulate else p
+    return acc.to(torch.int32)
+
+
+def round_and_trun(p: torch.Tensor, trun_bits: int, clamp_dl16: bool = False) -> torch.Tensor:
+    """round_and_trun_mask + round_and_trun (triton_kernels.py:432-465) on an fp32 tensor."""
+    if clamp_dl16:
+        trun_bits = 14
+    u = p.contiguous().view(torch.int32).to(torch.int64) & 0xFFFFFFFF
+    rb = (1 << (trun_bits - 1)) if trun_bits > 0 else 0
+    mask = (~((1 << trun_bits) - 1)) & 0xFFFFFFFF
+    u = ((u + rb) & 0xFFFFFFFF) & mask
+    u = torch.where(u >= (1 << 31), u - (1 << 32), u).to(torch.int32)
+    x = u.view(torch.float32)
+    if clamp_dl16:
+        x = torch.where(x >= DL16_MAX, torch.full_like(x, float("inf")), x)
+        x = torch.where(x <= -DL16_MAX, torch.full_like(x, float("-inf")), x)
+        x = torch.where(x.abs() < DL16_MIN, torch.zeros_like(x), x)
+    return x
+
+
+def chunk_matmul_fp(a, w, c=None, chunk_size=64, trun_bits=0, clamp_dl16=False,
+                    truncate_then_accumulate=True):
+    """matmul_kernel / matmul_kernel_DABC (triton_kernels.py:162-187,379-409).  a [M,K] and
+    w [N,K] hold the operand values (any float dtype); the per-chunk dot is formed in fp64 and
+    rounded once to fp32 -- the reference leaves the fp32 summation order to tl.dot."""
+    M, K = a.shape
+    acc = torch.zeros(M, w.shape[0], dtype=torch.float32) if c is None else c.float().clone()
+    for k0 in range(0, K, chunk_size):
+        p = a[:, k0:k0 + chunk_size].double() @ w[:, k0:k0 + chunk_size].double().t()
+        if not truncate_then_accumulate:
+            p = p + acc.double()
+        p = p.float()
+        if clamp_dl16 or trun_bits > 0:
+            p = round_and_trun(p, trun_bits, clamp_dl16)
+        acc = (acc + p) if truncate_then_accumulate else p
+    return acc
+
+
+# ------------------------------------------------------------------------------------------
+# FP8
+# ------------------------------------------------------------------------------------------
+def fp8_quant_fpxacc(t: torch.Tensor, per_tensor=False, dl8=False):
+    """Dynamic FP8 Q of LinearFuncFPxFwdBwd.forward (linear.py:1939-1953): returns
+    (e4m3 tensor, scale in t's dtype).  Reduction over dim 1 (per token / per out-channel)."""
+    reduce_dim = None if per_tensor else 1
+    scale = (t.abs().amax(dim=reduce_dim, keepdim=True) / E4M3_MAX).clamp(min=1e-5)
+    q = (t / scale).to(torch.float8_e4m3fn)
+    if dl8:
+        f = q.to(torch.float32)
+        f.masked_fill_(f.abs() < DL8_MIN, 0)
+        q = f.to(torch.float8_e4m3fn)
+    return q, scale
+
+
+def fpxacc_forward(x, weight, bias=None, trun_bits=0, chunk_size=16, fp8_dyn=False,
+                   clamp_acc_to_dl16=False):
+    """LinearFuncFPxFwdBwd.forward (linear.py:1902-1975)."""
+    org_dtype = x.dtype
+    out_shape = x.shape[:-1] + (weight.shape[0],)
+    x = x.reshape(-1, x.shape[-1])
+    x_scale = torch.tensor(1.0, dtype=org_dtype)
+    w_scale = x_scale.clone()
+    if fp8_dyn:
+        xq, x_scale = fp8_quant_fpxacc(x, fp8_dyn == "per_tensor", clamp_acc_to_dl16)
+        wq, w_scale = fp8_quant_fpxacc(weight, fp8_dyn == "per_tensor", clamp_acc_to_dl16)
+        x, weight = xq.to(torch.float32), wq.to(torch.float32)
+    min_chunk = 16  # fp32 / 16-bit operands; the fp8-valued operands are fp32 tensors here
+    cs = max(chunk_size, min_chunk) if (chunk_size & (chunk_size - 1)) == 0 else min_chunk
+    acc = chunk_matmul_fp(x, weight, None, cs, trun_bits, clamp_acc_to_dl16)
+    out = (acc.to(x.dtype) * x_scale * w_scale.t()).to(org_dtype).reshape(out_shape)
+    if bias is not None:
+        out = out + bias.to(org_dtype)
+    return out
+
+
+def int8train_forward(x, weight, bias=None, lsb_trun_bits=0, chunk_size=64, max_acc_bits=32):
+    """LinearFuncINT8FwdFP32Bwd.forward (linear.py:2141-2189)."""
+    org_dtype = x.dtype
+    out_shape = x.shape[:-1] + (weight.shape[0],)
+    x = x.reshape(-1, x.shape[-1])
+    x_scale = x.abs().amax(dim=-1, keepdim=True) / 127
+    w_scale = weight.abs().amax(dim=-1, keepdim=True) / 127
+    x_i8 = torch.round(x / x_scale).to(torch.int8)
+    w_i8 = torch.round(weight / w_scale).to(torch.int8)
+    cs = max(chunk_size, 32) if (chunk_size & (chunk_size - 1)) == 0 else 32
+    acc = chunk_matmul_i8(x_i8, w_i8, None, cs, lsb_trun_bits, max_acc_bits)
+    out = (acc.to(torch.float) * x_scale * w_scale.t()).reshape(out_shape).to(org_dtype)
+    if bias is not None:
+        out = out + bias.to(org_dtype)
+    return out, x_i8, w_i8, acc
+
+
+def fp8_quant_static(x: torch.Tensor, scale: torch.Tensor):
+    """_quantize_affine_float8_custom (fms_mo/aiu_addons/fp8/fp8_linear.py:54-72)."""
+    t = x.to(torch.float32) / scale
+    return t.clamp(min=-E4M3_MAX, max=E4M3_MAX).to(torch.float8_e4m3fn)
+
+
+def fp8_dynamic_scale(x: torch.Tensor):
+    """Per-row dynamic scale, rule of the reference's test helper
+    (tests/aiu_addons/test_fp8_addon.py:65-79).  PARITY UNPINNED w.r.t. torchao 0.11."""
+    return (x.abs().amax(dim=-1, keepdim=True).to(torch.float32) / E4M3_MAX).clamp(min=1e-12)
+
+
+def scaled_mm_cpu(mat1, mat2, scale1, scale2, bias=None, out_dtype=torch.float32):
+    """_scaled_mm_cpu_out (fms_mo/aiu_addons/fp8/fp8_spyre_op.py:35-60).  mat2 is [K,N]."""
+    m1 = (mat1.to(dtype=out_dtype) * scale1).to(dtype=out_dtype)
+    m2 = (mat2.to(dtype=out_dtype) * scale2).to(dtype=out_dtype)
+    if bias is not None:
+        return torch.addmm(bias.to(dtype=out_dtype), m1, m2)
+    return torch.mm(m1, m2)
+
+
+def fp8_linear_forward(x, w_e4m3, weight_scale, bias=None, input_scale=None):
+    """FP8Linear.forward with quantized activations (fp8_linear.py:217-283) evaluated with the
+    CPU _scaled_mm.  weight_scale: (1,) per tensor or (N,1) per row; input_scale None = dynamic
+    per token."""
+    x2 = x.reshape(-1, x.shape[-1])
+    s_x = fp8_dynamic_scale(x2) if input_scale is None else input_scale.to(torch.float32)
+    qx = fp8_quant_static(x2, s_x)
+    s_w = weight_scale.to(torch.float32)
+    s_w = s_w.reshape(1, -1) if s_w.numel() > 1 else s_w.reshape(())
+    s_xx = s_x if s_x.numel() > 1 else s_x.reshape(())
+    y = scaled_mm_cpu(qx, w_e4m3.t(), s_xx, s_w, bias, out_dtype=x.dtype)
+    return y.reshape(tuple(x.shape[:-1]) + (w_e4m3.shape[0],)), qx, s_x
+
+
+# ------------------------------------------------------------------------------------------
+# fms_mo::i8i8_aiu (the op the reference's stored vectors exercise)
+# ------------------------------------------------------------------------------------------
+def i8i8_aiu(x, weight, bias, qdata, weight_quant_type, activ_quant_type, smoothquant):
+    """fms_mo/aiu_addons/i8i8/i8i8_aiu_op.py:86-231."""
+    dtype = x.dtype
+    out_feat, in_feat = weight.size()
+    if weight_quant_type == "per_tensor":
+        i1 = 1
+    elif weight_quant_type == "per_channel":
+        i1 = out_feat
+    else:
+        raise NotImplementedError(weight_quant_type)
+    i2 = i1 + i1
+    i3, i4 = i2 + 1, i2 + 2
+    i5 = i4 + (out_feat if activ_quant_type == "per_tensor_asymm" else 1)
+    i6 = i5 + (in_feat if smoothquant else 1)
+    if len(qdata) != i6:
+        raise ValueError(f"qdata length ({len(qdata)}) does not match {i6}")
+    w_cv, _, a_cv, a_cvn, _, sq = torch.tensor_split(qdata, (i1, i2, i3, i4, i5))
+
+    if activ_quant_type == "per_tensor_symm":
+        scale_x = 127 / a_cv
+        x_int = torch.round(x / sq * scale_x).clamp(-127, 127).to(torch.int8)
+        x_dq = x_int.div(scale_x).mul(sq)
+    elif activ_quant_type == "per_tensor_asymm":
+        scale_x = 255 / (a_cv - a_cvn)
+        zp_x = a_cvn * scale_x
+        x_int = torch.round(x / sq * scale_x - zp_x).clamp(0, 255)
+        x_dq = x_int.add(zp_x).div(scale_x).mul(sq)
+    elif activ_quant_type == "per_token":
+        x_sq = x / sq
+        a_cv_tok = x_sq.abs().max(dim=-1, keepdim=True)[0]
+        scale_x = 127 / a_cv_tok
+        x_int = torch.round(x_sq * scale_x).clamp(-127, 127)
+        x_dq = x_int.div(scale_x).mul(sq)
+    else:
+        raise NotImplementedError(activ_quant_type)
+
+    if weight_quant_type == "per_tensor":
+        w_dq = (weight * w_cv / 127) / sq
+    else:
+        w_dq = (weight * w_cv.unsqueeze(dim=1) / 127) / sq
+    return torch.nn.functional.linear(x_dq.to(dtype), w_dq.to(dtype), bias.to(dtype))
