@@ -1,0 +1,216 @@
+#!/usr/bin/env python3
+"""Benchmark of the W8A8 quantized-linear hot path on one MI355X.
+
+A step = one pass of the path over one batch of synthetic activations already resident in HBM:
+for each of the four Llama-3-8B decoder-layer linears at M = 4096 tokens (q/k/v fused 4096->6144,
+o 4096->4096, gate+up 4096->28672, down 14336->4096) run the fused SmoothQuant-divide + per-token
+int8 activation quantizer, then the int8 MFMA GEMM with the dequantizing epilogue (fp16 out).
+Weights are quantized once, before the timed region (they are constants of the deployed module).
+
+Prints ONE JSON line (see the keys below).  `value` is 2*M*N*K summed over the four linears
+divided by the wall time of a step; `roofline` prices the GEMM kernel alone (HIP-event time of
+its launches inside the timed region) against the published dense INT8 MFMA peak; `cpu_baseline`
+is the CPU restatement of the reference's QLinear forward timed on the host cores on a bounded
+sample of the same workload.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "fms-model-optimizer_amd"))
+
+PEAK_INT8_TOPS = 5000.0   # MI355X dense INT8 MFMA, published
+PEAK_FP8_TFLOPS = 5000.0  # MI355X dense FP8 MFMA, published
+PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, published
+
+LLAMA3_8B = [("qkv", 4096, 6144), ("o", 4096, 4096), ("gate_up", 4096, 28672), ("down", 14336, 4096)]
+M_TOKENS = 4096
+
+
+def make_layer(torch, dev, K, N, seed):
+    """BASELINE config 2 inputs: x ~ N(0,1) with 1 % of the input channels scaled x50, W ~ N(0,0.02),
+    SmoothQuant alpha = 0.5 with a_k = max_m |x_mk|.  Generated on the CPU from a seeded generator
+    (so the CPU baseline sees the same bits), quantized offline with the deploy-module recipe."""
+    from fms_mo_amd.modules.linear import prepare_deploy_weights
+
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(M_TOKENS, K, generator=g)
+    idx = torch.randperm(K, generator=g)[: round(0.01 * K)]
+    x[:, idx] *= 50
+    W = 0.02 * torch.randn(N, K, generator=g)
+    b = 0.01 * torch.randn(N, generator=g)
+    x, W, b = x.half(), W.half(), b.half()
+    act_scale = x.float().abs().amax(dim=0)
+    xd, Wd = x.to(dev), W.to(dev)
+    w_i8, w_scale, smooth = prepare_deploy_weights(Wd, act_scale.to(dev), 0.5)
+    return {"x": xd, "w": w_i8, "w_scale": w_scale.float(), "smooth": smooth.reshape(-1).float(),
+            "bias": b.to(dev), "x_cpu": x, "W_cpu": W, "b_cpu": b, "act_scale_cpu": act_scale}
+
+
+def cpu_baseline(torch, layer, budget_s=20.0):
+    """The reference's CPU QLinear path (fake-quant forward with per-call weight re-quantization,
+    fms_mo/modules/linear.py:248-305) restated in oracle/, on the first rows of the `o` linear."""
+    from oracle import qlinear_oracle as O
+
+    torch.set_num_threads(os.cpu_count() or 1)
+    rows = 512
+    x, W, b = layer["x_cpu"][:rows], layer["W_cpu"], layer["b_cpu"]
+    a = layer["act_scale_cpu"]
+    O.qlinear_forward(x, W, b, a, 0.5)  # warm-up
+    times = []
+    t_all = time.perf_counter()
+    while len(times) < 5 and time.perf_counter() - t_all < budget_s:
+        t0 = time.perf_counter()
+        O.qlinear_forward(x, W, b, a, 0.5)
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    med = times[len(times) // 2]
+    ops = 2.0 * rows * W.shape[0] * W.shape[1]
+    return {"value": ops / med / 1e12, "unit": "TOPS", "cores": torch.get_num_threads(),
+            "kind": "port",
+            "sample": f"QLinear fake-quant forward (act Q/dQ, per-call weight Q/dQ, fp16 F.linear), "
+                      f"o-proj K=N=4096, first {rows} of 4096 tokens, median of {len(times)} runs, "
+                      f"{med * 1e3:.1f} ms each"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--extras", action="store_true", help="also time FP8 GEMMs and decode shapes")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (no collectives are part of it); "
+              "run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    from fms_mo_amd import kernels as K
+
+    dev = torch.device("cuda:0")
+    layers = [make_layer(torch, dev, k, n, seed=1 + i) for i, (_, k, n) in enumerate(LLAMA3_8B)]
+    total_ops = sum(2.0 * M_TOKENS * k * n for _, k, n in LLAMA3_8B)
+
+    def step(events=None):
+        for i, L in enumerate(layers):
+            q, s = K.quant_act_i8_pertoken(L["x"], L["smooth"])
+            if events is not None:
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+            y = K.gemm_i8_dq(q, L["w"], s, L["w_scale"], L["bias"], out_dtype=torch.float16,
+                             exact_ref=True)
+            if events is not None:
+                e1.record()
+                events[i].append((e0, e1))
+        return y
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    events = [[] for _ in layers]
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step(events)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms_per_step = dt / args.steps * 1e3
+    value = total_ops / (dt / args.steps) / 1e12
+
+    gemm_ms = [sum(a.elapsed_time(b) for a, b in ev) / len(ev) for ev in events]
+    gemm_ops = [2.0 * M_TOKENS * k * n for _, k, n in LLAMA3_8B]
+    per_shape = {name: round(o / (ms * 1e-3) / 1e12, 1) for (name, _, _), o, ms in zip(LLAMA3_8B, gemm_ops, gemm_ms)}
+    achieved = sum(gemm_ops) / (sum(gemm_ms) * 1e-3) / 1e12
+    traffic = None
+    tfile = os.path.join(ROOT, "profiles", "gemm_i8_traffic.json")
+    if os.path.exists(tfile):
+        with open(tfile) as f:
+            traffic = json.load(f).get("hbm_bytes_per_launch_avg")
+
+    out = {
+        "metric": "W8A8 INT8 linear (SmoothQuant act-quant + int8 MFMA GEMM + dequant) throughput, "
+                  "Llama-3-8B decoder-layer linears, M=4096",
+        "value": round(value, 2), "unit": "TOPS", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "int8", "data": "synthetic",
+        "config": {"workload": "Llama-3-8B decoder-layer linears W8A8 INT8 + SmoothQuant(alpha=0.5), "
+                               "M=4096 tokens: qkv 4096->6144, o 4096->4096, gate+up 4096->28672, "
+                               "down 14336->4096; fp16 in/out, per-token act / per-channel weight scales",
+                   "tokens": M_TOKENS},
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_INT8_TOPS,
+                     "unit": "TFLOP/s", "frac": round(achieved / PEAK_INT8_TOPS, 4),
+                     "traffic": traffic, "kernel": "gemm_tile_kernel<int8> (4 launches per step)",
+                     "per_shape_tops": per_shape,
+                     "avg_launch_ms": {n: round(ms, 4) for (n, _, _), ms in zip(LLAMA3_8B, gemm_ms)}},
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(torch, layers[1])
+    if args.extras:
+        out["extras"] = extras(torch, K, dev)
+    print(json.dumps(out))
+
+
+def extras(torch, K, dev):
+    """FP8 GEMMs (Granite-3-8B-like shapes, M=2048) and decode shapes (M in 1,4,16); reported in
+    addition to the headline value."""
+    from fms_mo_amd import _lib as L
+
+    res = {}
+
+    def timeit(fn, iters=30, warm=5):
+        for _ in range(warm):
+            fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(iters):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / iters
+
+    g = torch.Generator().manual_seed(3)
+    M = 2048
+    for name, k, n in [("qkv", 4096, 6144), ("o", 4096, 4096), ("gate_up", 4096, 25600), ("down", 12800, 4096)]:
+        x = torch.randn(M, k, generator=g).bfloat16().to(dev)
+        w = (0.02 * torch.randn(n, k, generator=g)).to(dev)
+        ws = (w.abs().amax() / 448).reshape(1).float()
+        w8 = (w / ws).clamp(-448, 448).to(torch.float8_e4m3fn)
+        q, s = K.quant_act_fp8_pertoken(x, L.FP8_LINEAR)
+        ms = timeit(lambda: K.gemm_fp8_dq(q, w8, s, ws, None, out_dtype=torch.bfloat16))
+        tf = 2.0 * M * k * n / (ms * 1e-3) / 1e12
+        res[f"fp8_M2048_{name}"] = {"ms": round(ms, 4), "tflops": round(tf, 1), "frac_peak": round(tf / PEAK_FP8_TFLOPS, 4)}
+    # decode: rotate weight copies totalling > 256 MiB so the Infinity Cache cannot hold them
+    for name, k, n in LLAMA3_8B:
+        wbytes = k * n
+        copies = max(3, (300 * 1024 * 1024 + wbytes - 1) // wbytes)
+        ws_i8 = [torch.randint(-127, 128, (n, k), dtype=torch.int8, device=dev) for _ in range(copies)]
+        wsc = torch.rand(n, device=dev) * 1e-3
+        for M in (1, 4, 16):
+            x = torch.randn(M, k, device=dev).bfloat16()
+            q, s = K.quant_act_i8_pertoken(x)
+            it = [0]
+
+            def run():
+                it[0] += 1
+                K.gemm_i8_dq(q, ws_i8[it[0] % copies], s, wsc, None, out_dtype=torch.bfloat16, exact_ref=True)
+
+            ms = timeit(run, iters=60, warm=copies)
+            byts = wbytes + M * k + M * n * 2 + 4 * n
+            gbs = byts / (ms * 1e-3) / 1e9
+            res[f"decode_i8_M{M}_{name}"] = {"us": round(ms * 1e3, 2), "GBps": round(gbs, 1), "frac_hbm": round(gbs / PEAK_HBM_GBS, 4)}
+        del ws_i8
+    return res
+
+
+if __name__ == "__main__":
+    main()

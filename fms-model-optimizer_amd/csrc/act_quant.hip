@@ -129,10 +129,11 @@ __global__ __launch_bounds__(AQ_THREADS) void quant_i8_pertoken_kernel(
 // ------------------------------------------------------------------ int8, static per tensor
 template <int XT>
 __global__ __launch_bounds__(AQ_THREADS) void quant_i8_static_kernel(
-    const void* __restrict__ x, int64_t ldx, float scale, float zp, float sym,
+    const void* __restrict__ x, int64_t ldx, float scale, float zp, float sym, int pt_native,
     int8_t* __restrict__ q, int64_t ldq, int K) {
   const int row = blockIdx.x;
   const int nchunk = K / AQ_VEC;
+  const float inv_scale = 1.0f / scale;
   for (int c = threadIdx.x; c < nchunk; c += AQ_THREADS) {
     float e[8];
     load8<XT>(x, (size_t)row * ldx + (size_t)c * AQ_VEC, e);
@@ -140,8 +141,12 @@ __global__ __launch_bounds__(AQ_THREADS) void quant_i8_static_kernel(
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       // ((x/s + zp) - 128) + sym, each step rounded to fp32, then round-half-even and clamp
-      float t = __fadd_rn(__fadd_rn(__fadd_rn(e[j] / scale, zp), -128.0f), sym);
-      t = fminf(fmaxf(__builtin_rintf(t), -128.0f), 127.0f);
+      float t;
+      if (pt_native)  // torch.quantize_per_tensor: rint(x * (1/scale)) + zero_point
+        t = __builtin_rintf(__fmul_rn(e[j], inv_scale)) + (zp - 128.0f + sym);
+      else
+        t = __builtin_rintf(__fadd_rn(__fadd_rn(__fadd_rn(e[j] / scale, zp), -128.0f), sym));
+      t = fminf(fmaxf(t, -128.0f), 127.0f);
       b[j] = (uint8_t)(int)t;
     }
     store8((uint8_t*)q, (size_t)row * ldq + (size_t)c * AQ_VEC, b);
@@ -270,7 +275,7 @@ extern "C" int fmsmo_quant_act_i8_static(const void* x, int x_dtype, int64_t ldx
   dim3 grid((unsigned)M), block(AQ_THREADS);
 #define LAUNCH(XT)                                                                           \
   hipLaunchKernelGGL((quant_i8_static_kernel<XT>), grid, block, 0, st, x, ldx, scale,        \
-                     (float)zp, (float)sym, q, ldq, (int)K)
+                     (float)zp, (float)(sym & 1), (sym >> 1) & 1, q, ldq, (int)K)
   switch (x_dtype) {
     case FMSMO_F16: LAUNCH(FMSMO_F16); break;
     case FMSMO_BF16: LAUNCH(FMSMO_BF16); break;

@@ -1,0 +1,637 @@
+"""Quantized-linear modules of the inference path, running on hand-written gfx950 kernels.
+
+Class names, constructor / classmethod signatures, keyword arguments, buffer names and
+``_get_name`` strings follow fms_mo/modules/linear.py so that model-surgery code
+(``qcfg["mapping"]``, lowering loops, checkpoint code reading ``clip_val`` / ``w_scale`` ...)
+keeps working when this package is imported in place of the reference:
+
+  QLinear                 linear.py:51-393     fake-quant training/calibration wrapper; its eval
+                                               forward runs as act-quant -> int8 GEMM -> dequant
+  QLinearINT8Deploy       linear.py:708-1338   Q -> int8 matmul -> dQ deploy module
+  LinearFPxAcc            linear.py:2048-2124  chunked reduced-precision FP accumulation
+  QLinearINT8Train        linear.py:2227-2285  chunked int8 forward (forward only here)
+
+There is no CPU path: a forward on CPU tensors raises.
+"""
+from __future__ import annotations
+
+import json
+import logging
+
+import torch
+import torch.nn.functional as F
+from torch import nn
+
+from .. import _lib as L
+from .. import kernels
+from ..custom_ext_kernels.hip_kernels import matmul_chunk_truncate as tl_matmul
+from ..quant.quantizers import (
+    Qbypass,
+    QMaxDynamic,
+    Qmax,
+    get_activation_quantizer,
+    get_weight_quantizer,
+)
+
+logger = logging.getLogger(__name__)
+
+
+def prepare_deploy_weights(weight, smoothq_act_scale=None, smoothq_alpha=0.5, w_clip_val=None):
+    """Offline weight preparation of the deploy module (from_fms_mo, linear.py:800-871):
+
+    smoothq_scale = clamp(a^alpha / clamp(max_n |W|, 1e-5)^(1-alpha), 1e-5)   if every a_k != 0
+    w_scale       = clip_val * 2 / 254          (clip_val defaults to the per-channel abs-max of W*s)
+    w_int8        = clamp(round((W * s).t() / w_scale), -127, 127).t()
+
+    Returns (w_int8 [N,K], w_scale [N], smoothq_scale [1,K] or [1])."""
+    with torch.no_grad():
+        sq = torch.tensor([1.0], device=weight.device, dtype=weight.dtype)
+        if smoothq_act_scale is not None and torch.all(smoothq_act_scale != 0).item():
+            a = smoothq_act_scale.to(weight.device)
+            wmax = weight.abs().max(dim=0, keepdim=True)[0].clamp(min=1e-5)
+            alpha = torch.as_tensor(smoothq_alpha, dtype=torch.float32, device=weight.device)
+            sq = (a**alpha / wmax ** (1.0 - alpha)).clamp(min=1e-5).to(a.dtype)
+        ws = weight * sq
+        if w_clip_val is None:
+            w_clip_val = ws.abs().amax(dim=1).float()
+        # divide by a tensor, not a Python scalar: on the GPU torch turns "/ scalar" into a multiply
+        # by the reciprocal, which is one ulp off the IEEE quotient the CPU evaluation gives
+        w_scale = w_clip_val * 2 / torch.tensor(254.0, device=w_clip_val.device, dtype=w_clip_val.dtype)
+        w_int8 = torch.round(ws.t() / w_scale).clamp(-127, 127).t().to(torch.int).to(torch.int8)
+    return w_int8.contiguous(), w_scale, sq
+
+
+def _compute_dtype(x_dtype, smooth):
+    return x_dtype if smooth is None else torch.promote_types(x_dtype, smooth.dtype)
+
+
+class QLinear(nn.Linear):
+    """Quantized linear wrapper (weights and activations to int8 / fp8 levels, bias untouched).
+
+    Training-mode and calibration forwards evaluate the quantizers with torch ops exactly like
+    the reference (they also update ``clip_val`` buffers).  The eval-mode forward of the W8A8
+    configuration (``qa_mode`` per-token max, ``qw_mode`` max / maxperCh, 8 bits) computes the same
+    fake-quant result as integer arithmetic on the GPU: fused SmoothQuant divide + per-token
+    quantizer, int8 MFMA GEMM against the (cached) integer weights, dequantizing epilogue."""
+
+    def __init__(self, in_features, out_features, bias=True, num_bits_feature=32, qa_mode=None,
+                 num_bits_weight=32, qw_mode=None, **kwargs):
+        super().__init__(in_features, out_features, bias, device=kwargs.get("device", "cuda"))
+        qcfg = kwargs.pop("qcfg")
+        self.num_bits_feature = num_bits_feature
+        self.num_bits_weight = num_bits_weight
+        self.qa_mode = qa_mode
+        self.qw_mode = qw_mode
+        default_calib = "max" if num_bits_feature == 8 else "percentile"
+        self.qa_mode_calib = kwargs.get("qa_mode_calib", qcfg.get("qa_mode_calib", default_calib))
+        self.qw_mode_calib = kwargs.get("qw_mode_calib", qcfg.get("qw_mode_calib", default_calib))
+        self.act_clip_init_val = kwargs.get("act_clip_init_val", qcfg.get("act_clip_init_val", 8.0))
+        self.act_clip_init_valn = kwargs.get("act_clip_init_valn", qcfg.get("act_clip_init_valn", -8.0))
+        self.w_clip_init_val = kwargs.get("w_clip_init_val", qcfg.get("w_clip_init_val", 1.0))
+        self.w_clip_init_valn = kwargs.get("w_clip_init_valn", qcfg.get("w_clip_init_valn", -1.0))
+        self.non_neg = kwargs.get("non_neg", qcfg.get("non_neg", False))
+        self.align_zero = kwargs.get("align_zero", qcfg.get("align_zero", True))
+        self.extend_act_range = kwargs.get("extend_act_range", qcfg.get("extend_act_range", False))
+        self.fp8_use_subnormal = kwargs.get("fp8_use_subnormal", qcfg.get("fp8_use_subnormal", False))
+        self.register_buffer("calib_counter", torch.tensor(qcfg.get("qmodel_calibration_new", 0)))
+        self.register_buffer("num_module_called", torch.tensor(0))
+        self.ptqmode = "qout"
+        self.W_fp = None
+        self.use_PT_native_Qfunc = kwargs.get("use_PT_native_Qfunc", qcfg.get("use_PT_native_Qfunc", False))
+        self.perGp = kwargs.get("qgroup", qcfg.get("qgroup", None))
+        self.qcfg = qcfg
+        self.calib_iterator = []
+        self.quantize_feature = Qbypass()
+        self.quantize_calib_feature = Qbypass()
+        if self.num_bits_feature not in [32, 16]:
+            self.quantize_feature = get_activation_quantizer(
+                self.qa_mode, nbits=self.num_bits_feature, clip_val=self.act_clip_init_val,
+                clip_valn=self.act_clip_init_valn, non_neg=self.non_neg, align_zero=self.align_zero,
+                extend_act_range=bool(self.extend_act_range),
+                use_PT_native_Qfunc=self.use_PT_native_Qfunc, use_subnormal=self.fp8_use_subnormal)
+            if self.calib_counter > 0:
+                self.quantize_calib_feature = self.quantize_feature
+        self.quantize_weight = Qbypass()
+        self.quantize_calib_weight = Qbypass()
+        if self.num_bits_weight not in [32, 16]:
+            self.quantize_weight = get_weight_quantizer(
+                self.qw_mode, nbits=self.num_bits_weight, clip_val=self.w_clip_init_val,
+                clip_valn=self.w_clip_init_valn, align_zero=self.align_zero,
+                w_shape=self.weight.shape, perGp=self.perGp, use_subnormal=self.fp8_use_subnormal)
+            if self.calib_counter > 0:
+                self.quantize_calib_weight = self.quantize_weight
+        self.mask = None
+        self.smoothq = qcfg.get("smoothq", False)
+        if self.smoothq:
+            self.register_buffer("smoothq_act_scale", torch.zeros(self.weight.shape[1]))
+            self.register_buffer("smoothq_alpha",
+                                 torch.tensor([qcfg.get("smoothq_alpha", 0.5)], dtype=torch.float32))
+        self._wcache = None  # (key, w_int8, w_scale) of the eval-mode integer path
+
+    # -- SmoothQuant ------------------------------------------------------------------------
+    def set_act_scale(self, act_scale):
+        assert act_scale.shape[0] == self.weight.shape[1], "scale applies to per-channel"
+        self.smoothq_act_scale.copy_(act_scale)
+
+    def get_smoothq_scale(self, x):
+        if self.smoothq_act_scale.sum().item() == 0.0:
+            return torch.tensor([1.0]).to(x.dtype).to(x.device)
+        wmax = self.weight.abs().max(dim=0, keepdim=True)[0].clamp(min=1e-5)
+        alpha = self.smoothq_alpha.item() if isinstance(self.smoothq_alpha, torch.Tensor) else self.smoothq_alpha
+        return (self.smoothq_act_scale.pow(alpha) / wmax.pow(1.0 - alpha)).clamp(min=1e-5).to(x.dtype)
+
+    # -- forward ----------------------------------------------------------------------------
+    def _int_path_ok(self, x):
+        return (not self.training and self.calib_counter <= 0 and self.ptqmode != "fp32_out"
+                and self.mask is None and x.is_cuda
+                and self.num_bits_feature == 8 and self.num_bits_weight == 8
+                and isinstance(self.quantize_feature, QMaxDynamic)
+                and self.quantize_feature.reduce_dim == -1
+                and isinstance(self.quantize_weight, Qmax))
+
+    def _int_weights(self, scale):
+        """Integer weights of the fake-quantized W*scale, cached until W, the clip values or the
+        SmoothQuant scale change.  Levels: fake_quantize_per_channel_affine / QmaxSTE, i.e. the
+        stored ``clip_val`` of the weight quantizer defines the grid (eval-mode semantics)."""
+        qw = self.quantize_weight
+        key = (self.weight._version, self.weight.data_ptr(), qw.clip_val._version,
+               None if scale is None else (scale.data_ptr(), scale._version))
+        if self._wcache is not None and self._wcache[0] == key:
+            return self._wcache[1], self._wcache[2]
+        with torch.no_grad():
+            ws = self.weight if scale is None else self.weight * scale
+            cv = qw.clip_val.to(ws.device).float()
+            w_scale = cv * 2 / 254
+            if qw.perCh:
+                # torch.fake_quantize_per_channel_affine rounds x * (1/scale)
+                inv = 1.0 / w_scale
+                w_int = torch.clamp(torch.round(ws.float() * inv[:, None]), -127, 127)
+            else:
+                u = ws.mul(1 / cv.to(ws.dtype)).clamp(-1, 1).mul(0.5).add(0.5)
+                w_int = torch.round(254 * u) - 127
+            w_int8 = w_int.to(torch.int8).contiguous()
+        self._wcache = (key, w_int8, w_scale.float().reshape(-1))
+        return w_int8, self._wcache[2]
+
+    def forward(self, x):
+        if self.smoothq:
+            scale = self.get_smoothq_scale(x)
+        else:
+            scale = torch.tensor([1.0]).to(x.dtype).to(x.device)
+        if self._int_path_ok(x):
+            x2 = x.reshape(-1, x.shape[-1])
+            smooth = scale.reshape(-1) if scale.numel() > 1 else None
+            q, s = kernels.quant_act_i8_pertoken(x2, smooth, compute_dtype=x.dtype)
+            w_int8, w_scale = self._int_weights(scale if scale.numel() > 1 else None)
+            y = kernels.gemm_i8_dq(q, w_int8, s, w_scale, self.bias, out_dtype=x.dtype, exact_ref=False)
+            self.num_module_called += 1
+            return y.reshape(tuple(x.shape[:-1]) + (self.out_features,))
+        if not x.is_cuda:
+            raise RuntimeError("fms_mo_amd.QLinear runs on an AMD GPU only; there is no CPU path")
+        # training / calibration / other quantizer modes: quantizer modules evaluated with torch ops
+        if self.calib_counter > 0:
+            with torch.no_grad():
+                qinput = self.quantize_calib_feature(x / scale)
+                qweight = self.quantize_calib_weight(self.weight * scale)
+            self.calib_counter -= 1
+            if self.calib_counter == 0:
+                self.quantize_calib_feature = None
+                self.quantize_calib_weight = None
+        elif self.ptqmode == "fp32_out":
+            if self.W_fp is None:
+                self.W_fp = self.weight.detach().clone()
+                self.weight.requires_grad = True
+            return F.linear(x, self.W_fp, self.bias)
+        else:
+            qinput = self.quantize_feature(x / scale).to(x.dtype)
+            qweight = self.quantize_weight(self.weight * scale).to(self.weight.dtype)
+        output = F.linear(qinput, qweight, self.bias)
+        self.num_module_called += 1
+        return output
+
+    def __repr__(self):
+        s = ",QntzerW,A="
+        s += "" if self.num_bits_weight == 32 else f"{self.quantize_weight.__repr__().split('(')[0]},"
+        s += "" if self.num_bits_feature == 32 else f"{self.quantize_feature.__repr__().split('(')[0]}"
+        return (f"{self.__class__.__name__}({self.in_features},{self.out_features}, "
+                f"Nbits_W,A={self.num_bits_weight},{self.num_bits_feature}{s})")
+
+
+class QLinearINT8Deploy(nn.Linear):
+    """Deploy-time W8A8 linear: quantize -> int8 matmul (int32 accumulate) -> dequantize.
+
+    Buffers: ``weight`` (int8 [N,K]), ``input_scale``, ``input_zp``, ``w_scale``, ``w_zp``,
+    ``smoothq_scale``, ``corr_term``, ``bias`` -- the names the reference registers
+    (linear.py:843-911)."""
+
+    @classmethod
+    def from_fms_mo(cls, fms_mo_qlinear, **kwargs):
+        """Convert a QLinear.  Keyword arguments as in the reference: use_int_kernel
+        ('cutlass' | 'triton' | True all select the HIP kernels, False the FP emulation),
+        use_PT_native_Qfunc, use_dynamic_max_act_Qfunc (-1 | -2 | 1..64 | False), max_acc_bits,
+        truncate_lsb, chunk_size, recalc_clipvals, target_device."""
+        assert all(getattr(fms_mo_qlinear, a) in [4, 8] for a in ["num_bits_feature", "num_bits_weight"]), \
+            "Please check nbits setting!"
+        tar_dev = kwargs.get("target_device", kwargs.get("device", next(fms_mo_qlinear.parameters()).device))
+        w_dtype = fms_mo_qlinear.weight.dtype
+        # All offline arithmetic runs where the source module lives (the reference requires source
+        # and target on one device; converting a CPU module for a GPU target also works here and
+        # gives the CPU roundings of pow / division for the offline scales).
+        src_dev = fms_mo_qlinear.weight.device
+        m = cls(fms_mo_qlinear.in_features, fms_mo_qlinear.out_features,
+                bias=fms_mo_qlinear.bias is not None, device="meta")
+        qcfg = getattr(fms_mo_qlinear, "qcfg", {})
+        m.use_int_kernel = kwargs.get("use_int_kernel", qcfg.get("use_int_kernel", "cutlass"))
+        m.usePTnativeQfunc = kwargs.get("use_PT_native_Qfunc", False)
+        m.useDynMaxQfunc = kwargs.get("use_dynamic_max_act_Qfunc", False)
+        m.useSymAct = "sym" in fms_mo_qlinear.qa_mode or fms_mo_qlinear.qa_mode in ["pertokenmax", "max"]
+        m.max_acc_bits = kwargs.get("max_acc_bits", 32)
+        m.accminmax = (-(1 << (m.max_acc_bits - 1)), (1 << (m.max_acc_bits - 1)) - 1)
+        m.truncate_lsb = kwargs.get("truncate_lsb", 0)
+        m.chunk_size = kwargs.get("chunk_size", 100000)
+        m.acc_dtype = torch.float16
+        m.nbits_a = fms_mo_qlinear.num_bits_feature
+        m.nbits_w = fms_mo_qlinear.num_bits_weight
+        w_levels = 2**m.nbits_w - 2
+        a_levels = 2**m.nbits_a - 1 - m.useSymAct
+        with torch.no_grad():
+            Qa, Qw = fms_mo_qlinear.quantize_feature, fms_mo_qlinear.quantize_weight
+            if kwargs.get("recalc_clipvals", True):
+                Qw(fms_mo_qlinear.weight)
+            w_cv = Qw.clip_val
+            a_cv = getattr(Qa, "clip_val", torch.tensor(8.0, device=src_dev))
+            a_cvn = getattr(Qa, "clip_valn", torch.tensor(-8.0, device=src_dev))
+            m.cvs = [a_cv, a_cvn, w_cv]
+            smoothq_scale = torch.tensor([1.0], device=src_dev, dtype=w_dtype)
+            if getattr(fms_mo_qlinear, "smoothq", False):
+                a_s = fms_mo_qlinear.smoothq_act_scale
+                w_s = fms_mo_qlinear.weight.abs().max(dim=0, keepdim=True)[0].clamp(min=1e-5)
+                alpha = fms_mo_qlinear.smoothq_alpha
+                if torch.all(a_s != 0).item():
+                    smoothq_scale = (a_s**alpha / w_s ** (1.0 - alpha)).clamp(min=1e-5).to(a_s.dtype)
+            input_scale = torch.tensor(1.0, device=src_dev)
+            # tensor divisor: keeps the IEEE quotient on the GPU as well (see prepare_deploy_weights)
+            w_scale = w_cv * 2 / torch.tensor(float(w_levels), device=w_cv.device, dtype=w_cv.dtype)
+            m.use_fake_zero_shift = False
+            if m.useDynMaxQfunc in [-1, -2]:
+                input_zero_point = torch.tensor(128 - m.useSymAct, device=src_dev)
+            elif 0 < m.useDynMaxQfunc < 65:
+                m.use_fake_zero_shift = True
+                input_zero_point = torch.tensor(m.useDynMaxQfunc, device=src_dev)
+            elif m.usePTnativeQfunc:
+                input_scale = torch.tensor([(a_cv - a_cvn) / a_levels], device=src_dev)
+                input_zero_point = torch.round(-a_cvn / input_scale)
+            else:
+                quant_scale = a_levels / torch.tensor([a_cv - a_cvn], device=src_dev)
+                quant_stepsize = 1.0 / quant_scale
+                quant_zero_point = torch.round(a_cvn * quant_scale)
+                input_scale = quant_stepsize
+                input_zero_point = -quant_zero_point
+                w_scale = 1.0 / (w_levels / (w_cv * 2))
+                m.register_buffer("quant_scale", quant_scale)
+                m.register_buffer("quant_stepsize", quant_stepsize)
+                m.register_buffer("quant_zero_point", quant_zero_point)
+            w_zp = torch.zeros_like(w_scale, dtype=torch.int)
+            input_zero_point = input_zero_point.to(torch.int)
+            m.register_buffer("input_scale", input_scale)
+            m.register_buffer("input_zp", input_zero_point)
+            m.register_buffer("w_scale", w_scale)
+            m.register_buffer("w_zp", w_zp)
+            m.register_buffer("smoothq_scale", smoothq_scale)
+            w_int8 = (torch.round((fms_mo_qlinear.weight * smoothq_scale).t() / w_scale)
+                      .clamp(-w_levels / 2, w_levels / 2).t())
+            w_int8 = w_int8.to(torch.int)
+            m.weight = nn.Parameter(w_int8.to(torch.int8), requires_grad=False)
+            if m.useSymAct:
+                corr_term_int = 0
+                if m.use_fake_zero_shift:
+                    corr_term_int = input_zero_point * (w_int8.sum(dim=1))
+            else:
+                corr_term_int = (input_zero_point - 128) * (w_int8.sum(dim=1))
+            m.register_buffer("corr_term", corr_term_int * w_scale.float() * input_scale.float())
+            m.org_model_has_bias = fms_mo_qlinear.bias is not None
+            new_bias = (fms_mo_qlinear.bias.float() - m.corr_term) if m.org_model_has_bias else -m.corr_term
+            if m.use_fake_zero_shift:
+                new_bias += m.corr_term
+            delattr(m, "bias")
+            m.register_buffer("bias", new_bias.to(w_dtype))
+        m.set_matmul_op()
+        return m.to(tar_dev)
+
+    @classmethod
+    def from_torch_iW(cls, nnlin_iW, prec, a_cv, a_cvn, w_cv, zero_shift, **kwargs):
+        """Build the module from an nn.Linear that already holds integer weights (linear.py:923-1023)."""
+        assert prec == "int8", "Only support INT8 for now."
+        target_device = kwargs.get("target_device", kwargs.get("device", next(nnlin_iW.parameters()).device))
+        m = cls(nnlin_iW.in_features, nnlin_iW.out_features, bias=nnlin_iW.bias is not None, device=target_device)
+        m.nbits_a = m.nbits_w = 8
+        m.acc_dtype = kwargs.get("acc_dtype", torch.float)
+        m.usePTnativeQfunc = kwargs.get("use_PT_native_Qfunc", True)
+        m.use_int_kernel = kwargs.get("use_int_kernel", "triton")
+        m.useDynMaxQfunc = False
+        m.useSymAct = False
+        m.use_fake_zero_shift = False
+        m.weight = nn.Parameter(nnlin_iW.weight.to(torch.int8), requires_grad=False)
+        m.max_acc_bits = kwargs.get("max_acc_bits", 32)
+        m.accminmax = (-(1 << (m.max_acc_bits - 1)), (1 << (m.max_acc_bits - 1)) - 1)
+        m.truncate_lsb = kwargs.get("truncate_lsb", False)
+        m.chunk_size = kwargs.get("chunk_size", 100000)
+        with torch.no_grad():
+            if m.usePTnativeQfunc:
+                input_scale = torch.Tensor([(a_cv - a_cvn) / (2**m.nbits_a - 1)])
+                input_zero_point = torch.round(-a_cvn / input_scale).to(torch.int)
+                w_scale = torch.Tensor([w_cv * 2 / (2**m.nbits_w - 2)])
+            else:
+                quant_scale = (2**m.nbits_a - 1) / torch.Tensor([a_cv - a_cvn])
+                quant_stepsize = 1.0 / quant_scale
+                quant_zero_point = torch.round(a_cvn * quant_scale)
+                input_scale = quant_stepsize
+                input_zero_point = -quant_zero_point
+                w_scale = 1.0 / ((2**m.nbits_a - 2) / torch.Tensor([w_cv * 2]))
+                m.register_buffer("quant_scale", quant_scale)
+                m.register_buffer("quant_stepsize", quant_stepsize)
+                m.register_buffer("quant_zero_point", quant_zero_point)
+            m.register_buffer("input_scale", input_scale)
+            m.register_buffer("input_zp", input_zero_point)
+            m.register_buffer("w_scale", w_scale)
+            m.register_buffer("w_zp", torch.zeros_like(w_scale, dtype=torch.int))
+            m.register_buffer("smoothq_scale", torch.tensor([1.0]))
+            m.cvs = [a_cv, a_cvn, w_cv]
+            zero_s = torch.Tensor(json.loads(zero_shift)) if isinstance(zero_shift, str) else torch.Tensor([zero_shift])
+            corr_term = (input_zero_point - 128) * zero_s * w_scale * input_scale
+            m.register_buffer("corr_term", corr_term)
+            m.register_buffer("zero_shift", zero_s)
+            if nnlin_iW.bias is not None:
+                m.bias = nn.Parameter((nnlin_iW.bias - corr_term.to(target_device)).to(m.acc_dtype),
+                                      requires_grad=False)
+                m.org_mod_has_bias = True
+            else:
+                delattr(m, "bias")
+                m.register_buffer("bias", -corr_term.to(m.acc_dtype))
+                m.org_mod_has_bias = False
+        m.set_matmul_op()
+        return m.to(target_device)
+
+    # -- activation quantizers (device kernels) ----------------------------------------------
+    def qa_raw_qfunc(self, x):
+        return kernels.quant_act_i8_static(x, float(self.input_scale.reshape(-1)[0]),
+                                           int(self.input_zp.reshape(-1)[0]), int(self.useSymAct))
+
+    def qa_pt_quant_func(self, x):
+        """torch.quantize_per_tensor(x.float(), scale, zp - 128 + sym) arithmetic (linear.py:1043-1059)."""
+        return kernels.quant_act_i8_static(x, float(self.input_scale.reshape(-1)[0]),
+                                           int(self.input_zp.reshape(-1)[0]), int(self.useSymAct) | 2)
+
+    qa_pt_qfunc_wrapped = qa_pt_quant_func
+
+    def qa_fmo_mo_qfunc(self, x):
+        """round(clamp(x, cvn, cv) / stepsize - zero_point) - (128 - sym): clamp-then-round with the
+        fms_mo formula (linear.py:1073-1083).  Offline-calibrated static path; torch ops."""
+        xq = torch.round(x.clamp(self.cvs[1], self.cvs[0]) / self.quant_stepsize - self.quant_zero_point) \
+            - (128 - self.useSymAct)
+        return xq.to(torch.int8)
+
+    def qa_dynamic_max_qfunc(self, x):
+        """Per-token (dim -1) dynamic abs-max quantizer; stores ``input_scale`` [M,1] and
+        ``cvs[0:2]`` like the reference."""
+        if self.useDynMaxQfunc == -2:
+            amax = x.abs().max(dim=-2, keepdim=True)[0]
+            self.cvs[0], self.cvs[1] = amax, -amax
+            self.input_scale = amax.clamp(min=1e-5).div(127)
+            return torch.round(x / self.input_scale).to(torch.int8)
+        smooth = None
+        q, s = kernels.quant_act_i8_pertoken(x, smooth, compute_dtype=x.dtype)
+        self.input_scale = s.reshape(-1, 1)
+        self.cvs[0], self.cvs[1] = s.reshape(-1, 1) * 127, -(s.reshape(-1, 1) * 127)
+        return q
+
+    def qa_dyn_max_fake_zero_shift(self, x):
+        amax = x.abs().max()
+        levels = 2 ** (self.nbits_a - 1) - 1 - self.input_zp
+        self.cvs[0], self.cvs[1] = amax, -amax
+        self.input_scale = amax.clamp(min=1e-5) / levels
+        return (torch.round(x / self.input_scale) + self.input_zp).to(torch.int8)
+
+    # -- matmul + dequant ----------------------------------------------------------------------
+    def _quantize(self, m1):
+        if self.useDynMaxQfunc in [-1, -2]:
+            return self.qa_dynamic_max_qfunc(m1)
+        if self.use_fake_zero_shift:
+            return self.qa_dyn_max_fake_zero_shift(m1)
+        if self.usePTnativeQfunc:
+            return self.qa_raw_qfunc(m1)
+        return self.qa_fmo_mo_qfunc(m1)
+
+    def iaddmm_int(self, bias, m1, m2):
+        """Q(m1) -> int matmul -> dQ (+bias).  m2 is ``W.t()`` ([K,N] view of the [N,K] weight).
+
+        Three cases, as in the reference (linear.py:1115-1188):
+          * K > chunk_size and kernel != 'triton': its serial PyTorch chunk loop (clamp to
+            max_acc_bits, (p + 2^(t-1)) >> t, int32 accumulate, fp32 scales) -- one launch of
+            the chunked int8 kernel here;
+          * kernel == 'triton' with LSB truncation: imatmul is the chunked kernel (chunk_size /
+            truncate_lsb only, max_acc_bits is not forwarded there either), then the fp16-scale
+            epilogue;
+          * otherwise the int8 MFMA GEMM with the fused fp16-scale epilogue."""
+        w = m2.t()
+        m1 = self._quantize(m1)
+        K = m1.shape[1]
+        if K > self.chunk_size and self.use_int_kernel != "triton":
+            cs = int(self.chunk_size)
+            if cs < 32 or cs & (cs - 1):
+                raise NotImplementedError("chunk_size must be a power of two >= 32 on this backend")
+            acc = kernels.matmul_chunk(m1, w, None, chunk_size=cs, chunk_trun_bits=int(self.truncate_lsb),
+                                       max_acc_bits=self.max_acc_bits)
+            # acc == 2^t * (the reference's shifted accumulator); (2^t a) * s == a * (2^t s) exactly
+            return (acc * (self.input_scale * self.w_scale) + bias).to(self.acc_dtype)
+        updated_bias = bias
+        if self.use_fake_zero_shift:
+            updated_bias = bias - self.input_scale * self.corr_term
+        if self.use_int_kernel == "triton" and self.truncate_lsb > 0:
+            imm_out = tl_matmul(m1, m2, chunk_trun_bits=int(self.truncate_lsb), chunk_size=int(self.chunk_size))
+            return (imm_out.float() * (self.input_scale * self.w_scale).to(torch.float16)
+                    + updated_bias).to(self.acc_dtype)
+        ref16 = self.acc_dtype == torch.float16
+        y = kernels.gemm_i8_dq(m1, w, self.input_scale.float().reshape(-1), self.w_scale.float().reshape(-1),
+                               updated_bias, out_dtype=torch.float16 if ref16 else torch.float32,
+                               exact_ref=True)
+        return y if ref16 else y.to(self.acc_dtype)
+
+    def iaddmm_FP(self, bias, m1, m2):
+        """The reference's non-integer emulation (torch.matmul on dequantized operands)."""
+        m1 = self._quantize(m1)
+        return torch.matmul(m1 * self.input_scale, m2 * self.w_scale) + bias
+
+    def set_matmul_op(self):
+        from ..custom_ext_kernels.utils import imatmul_ops_reg
+
+        imatmul_ops_reg(self.use_int_kernel)
+        self.imatmul = torch.ops.fms_mo.imatmul
+        self.iaddmm = self.iaddmm_int if self.use_int_kernel else self.iaddmm_FP
+
+    def _get_name(self):
+        return "QLinear_INT8"
+
+    def extra_repr(self) -> str:
+        s = (f"in={self.in_features}, out={self.out_features}, bias={self.bias is not None}, "
+             f"int_kernel={self.use_int_kernel}")
+        if self.truncate_lsb > 0 or self.max_acc_bits < 32:
+            s += f", acc_bits={self.max_acc_bits}, trun_lsb={self.truncate_lsb}"
+        return s
+
+    def __getstate__(self):
+        state = self.__dict__.copy()
+        state.pop("imatmul", None)
+        state.pop("iaddmm", None)
+        return state
+
+    def __setstate__(self, state):
+        self.__dict__.update(state)
+        self.set_matmul_op()
+
+    def _smoothq_active(self):
+        """The reference divides by ``smoothq_scale`` only if EVERY element differs from 1
+        (linear.py:1331); the answer is cached until the buffer changes (it costs a host sync)."""
+        sq = self.smoothq_scale
+        key = (sq.data_ptr(), sq._version)
+        if getattr(self, "_sq_key", None) != key:
+            self._sq_key = key
+            self._sq_on = bool(torch.all(sq != 1).item())
+        return self._sq_on
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        with torch.no_grad():
+            org_dtype = x.dtype
+            tar_shape = tuple(x.shape[:-1]) + (self.weight.shape[0],)
+            x2 = x.reshape(-1, x.shape[-1])
+            if not x2.is_cuda:
+                raise RuntimeError("fms_mo_amd.QLinearINT8Deploy runs on an AMD GPU only; there is no CPU path")
+            use_sq = self._smoothq_active()
+            if (use_sq and self.useDynMaxQfunc == -1 and self.use_int_kernel
+                    and self.smoothq_scale.numel() == x2.shape[1]
+                    and not (x2.shape[1] > self.chunk_size or self.truncate_lsb > 0)):
+                # fused path: SmoothQuant divide inside the quantizer kernel
+                sq = self.smoothq_scale.reshape(-1)
+                q, s = kernels.quant_act_i8_pertoken(x2, sq, compute_dtype=_compute_dtype(x2.dtype, sq))
+                self.input_scale = s.reshape(-1, 1)
+                y = kernels.gemm_i8_dq(q, self.weight, s, self.w_scale.float().reshape(-1), self.bias,
+                                       out_dtype=torch.float16, exact_ref=True).to(self.acc_dtype)
+            else:
+                if use_sq:
+                    x2 = x2 / self.smoothq_scale
+                y = self.iaddmm(self.bias, x2, self.weight.t())
+            return y.reshape(tar_shape).to(org_dtype)
+
+
+class LinearFPxAcc(torch.nn.Linear):
+    """Linear layer whose FP32 accumulator is LSB-rounded after every K-chunk (forward only)."""
+
+    @classmethod
+    def from_nn(cls, nnlin, trun_bits=0, **kwargs):
+        target_device = kwargs.get("target_device", kwargs.get("device", next(nnlin.parameters()).device))
+        m = cls(nnlin.in_features, nnlin.out_features, bias=nnlin.bias is not None, device="meta")
+        m.weight = nnlin.weight
+        m.trun_bits = trun_bits
+        m.chunk_size = kwargs.get("chunk_size", False)
+        m.fp8_dyn = kwargs.get("dynamic_fp8", False)
+        m.clamp_acc_to_dl16 = kwargs.get("clamp_acc_to_dl16", False)
+        if nnlin.bias is not None:
+            m.bias = nnlin.bias
+        return m.to(target_device)
+
+    def forward(self, inputs):
+        x = inputs
+        assert x.dtype in [torch.float, torch.bfloat16, torch.float16]
+        org_dtype = x.dtype
+        out_shape = x.shape[:-1] + (self.weight.shape[0],)
+        x = x.reshape(-1, x.shape[-1])
+        weight = self.weight.detach()
+        with torch.no_grad():
+            if self.fp8_dyn:
+                variant = L.FP8_FPXACC_DL8 if self.clamp_acc_to_dl16 else L.FP8_FPXACC
+                if self.fp8_dyn == "per_tensor":
+                    # one scale per tensor, formed in the original dtype like the reference
+                    xs = (x.abs().amax() / 448.0).clamp(min=1e-5)
+                    wsc = (weight.abs().amax() / 448.0).clamp(min=1e-5)
+                    xq, _ = kernels.quant_act_fp8_pertoken(x, variant, static_scale=xs.float())
+                    wq, _ = kernels.quant_act_fp8_pertoken(weight, variant, static_scale=wsc.float())
+                    x_scale, w_scale = xs.reshape(1, 1), wsc.reshape(1, 1)
+                else:
+                    xq, xs = kernels.quant_act_fp8_pertoken(x, variant)
+                    wq, wsc = kernels.quant_act_fp8_pertoken(weight, variant)
+                    x_scale, w_scale = xs.reshape(-1, 1).to(org_dtype), wsc.reshape(-1, 1).to(weight.dtype)
+                acc = tl_matmul(xq, wq.t(), chunk_trun_bits=self.trun_bits, chunk_size=int(self.chunk_size),
+                                clamp_acc_to_dl16=self.clamp_acc_to_dl16)
+            else:
+                x_scale = torch.tensor(1.0, device=x.device, dtype=org_dtype)
+                w_scale = x_scale.clone().reshape(1, 1)
+                acc = tl_matmul(x.contiguous(), weight.to(x.dtype).t(), chunk_trun_bits=self.trun_bits,
+                                chunk_size=int(self.chunk_size), clamp_acc_to_dl16=self.clamp_acc_to_dl16)
+            out = (acc * x_scale * w_scale.t()).to(org_dtype).reshape(out_shape)
+            if self.bias is not None:
+                out = out + self.bias.to(org_dtype)
+        return out
+
+    def extra_repr(self) -> str:
+        s = f"{self.in_features},{self.out_features}"
+        if self.bias is not None:
+            s += f",bias={self.bias is not None}"
+        if self.trun_bits > 0:
+            s += f",trun_bits={self.trun_bits}"
+        if self.fp8_dyn:
+            s += f",fp8_dyn={self.fp8_dyn}"
+        if self.clamp_acc_to_dl16:
+            s += ",use_DL16_acc"
+        return s + f",chunk_size={self.chunk_size}"
+
+
+class QLinearINT8Train(torch.nn.Linear):
+    """INT8 forward with chunked accumulation (MSB clamp / LSB rounding), dynamic per-token
+    activation and per-channel weight scales (linear.py:2141-2189).  Forward only."""
+
+    @classmethod
+    def from_fms_mo(cls, nnlin, lsb_trun_bits=0, **kwargs):
+        target_device = kwargs.get("target_device", kwargs.get("device", next(nnlin.parameters()).device))
+        m = cls(nnlin.in_features, nnlin.out_features, bias=nnlin.bias is not None, device="meta")
+        m.weight = nnlin.weight
+        m.lsb_trun_bits = lsb_trun_bits
+        m.chunk_size = kwargs.get("chunk_size", 64)
+        m.max_acc_bits = kwargs.get("max_acc_bits", 32)
+        if nnlin.bias is not None:
+            m.bias = nnlin.bias
+        return m.to(target_device)
+
+    def forward(self, inputs):
+        x = inputs
+        assert x.dtype in [torch.float, torch.bfloat16, torch.float16]
+        org_dtype = x.dtype
+        out_shape = x.shape[:-1] + (self.weight.shape[0],)
+        x = x.reshape(-1, x.shape[-1])
+        with torch.no_grad():
+            # amax/127 scales; all-zero rows give scale 1e-5/127 here where the reference divides
+            # 0/0 (its int8 result is undefined there)
+            x_i8, x_scale = kernels.quant_act_i8_pertoken(x, None, compute_dtype=x.dtype)
+            w = self.weight.detach()
+            w_i8, w_scale = kernels.quant_act_i8_pertoken(w, None, compute_dtype=w.dtype)
+            acc = tl_matmul(x_i8, w_i8.t(), chunk_trun_bits=self.lsb_trun_bits, chunk_size=self.chunk_size,
+                            max_acc_bits=self.max_acc_bits)
+            out = (acc.to(torch.float) * x_scale.reshape(-1, 1).to(org_dtype)
+                   * w_scale.reshape(1, -1).to(w.dtype)).reshape(out_shape).to(org_dtype)
+            if self.bias is not None:
+                out = out + self.bias.to(org_dtype)
+        return out
+
+    def extra_repr(self) -> str:
+        s = f"{self.in_features},{self.out_features},bias={self.bias is not None},chunk_size={self.chunk_size}"
+        if self.lsb_trun_bits > 0:
+            s += f",lsb_trun={self.lsb_trun_bits}"
+        if self.max_acc_bits < 32:
+            s += f",max_acc_bits={self.max_acc_bits}"
+        return s
+
+
+QLinear_modules = (QLinear, QLinearINT8Deploy, LinearFPxAcc, QLinearINT8Train)
+
+
+def isinstance_qlinear(module):
+    return isinstance(module, QLinear_modules)

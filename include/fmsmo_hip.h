@@ -84,9 +84,13 @@ int fmsmo_quant_act_i8_pertoken(const void* x, int x_dtype, int64_t ldx, const v
 
 /*
  * Static per-tensor int8 quantizer:  q = clamp( rint( x/scale + zp - 128 + sym ), -128, 127 )
- * evaluated in fp32 in exactly that order.  Reference: QLinearINT8Deploy.qa_raw_qfunc
+ * evaluated in fp32 in exactly that order (sym in {0,1}).  Reference: QLinearINT8Deploy.qa_raw_qfunc
  * (fms_mo/modules/linear.py:1061-1071); also the quantize step of fms_mo::q_iaddmm_dq
  * (fms_mo/custom_ext_kernels/utils.py:770) with sym = 0.
+ * sym | 2 selects torch.quantize_per_tensor's arithmetic instead,
+ *   q = clamp( rint( x * (1/scale) ) + (zp - 128 + (sym & 1)), -128, 127 ),
+ * used by fms_mo::q_per_t_sym (custom_ext_kernels/utils.py:792-794) and qa_pt_quant_func
+ * (linear.py:1043-1059).
  */
 int fmsmo_quant_act_i8_static(const void* x, int x_dtype, int64_t ldx, float scale, int zp,
                               int sym, int8_t* q, int64_t ldq, int64_t M, int64_t K,

@@ -1,0 +1,226 @@
+"""The drop-in modules and custom ops on the GPU against the CPU oracle."""
+import pytest
+import torch
+
+from oracle import qlinear_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def gen(seed):
+    return torch.Generator().manual_seed(seed)
+
+
+def make_qlinear(dev, K, N, smoothq=False, bias=True, seed=0, dtype=torch.float16):
+    from fms_mo_amd.modules.linear import QLinear
+
+    m = QLinear(K, N, bias=bias, num_bits_feature=8, qa_mode="pertokenmax", num_bits_weight=8,
+                qw_mode="maxperCh", qcfg={"smoothq": smoothq, "smoothq_alpha": 0.5}, device="cpu")
+    g = gen(seed)
+    with torch.no_grad():
+        m.weight.copy_(0.02 * torch.randn(N, K, generator=g))
+        if bias:
+            m.bias.copy_(0.01 * torch.randn(N, generator=g))
+    m.to(dtype)
+    m.quantize_weight.float()
+    if smoothq:
+        m.smoothq_act_scale = m.smoothq_act_scale.float()
+        m.smoothq_alpha = m.smoothq_alpha.float()
+    with torch.no_grad():
+        m.quantize_weight.train()
+        m.quantize_weight(m.weight)       # one training-mode pass initialises the weight clip values
+    m.eval()
+    return m if dev is None else m.to(dev)
+
+
+def outlier_x(M, K, seed, dtype=torch.float16):
+    g = gen(seed)
+    x = torch.randn(M, K, generator=g)
+    idx = torch.randperm(K, generator=g)[: max(1, round(0.01 * K))]
+    x[:, idx] *= 50
+    return x.to(dtype)
+
+
+@pytest.mark.parametrize("smoothq", [False, True])
+@pytest.mark.parametrize("shape", [(3, 40, 256, 384), (1, 512, 1024, 512)])
+def test_deploy_module_bit_exact_vs_oracle(dev, smoothq, shape):
+    """Conversion (offline weight / scale preparation) runs on the CPU like the reference's
+    lower_qmodel_cutlass (custom_ext_kernels/utils.py:830); the forward runs on the GPU."""
+    from fms_mo_amd.modules.linear import QLinearINT8Deploy
+
+    B, S, K, N = shape
+    m = make_qlinear(None, K, N, smoothq=smoothq)
+    x = outlier_x(B * S, K, 5).reshape(B, S, K)
+    act_scale = None
+    if smoothq:
+        act_scale = x.reshape(-1, K).float().abs().amax(dim=0)
+        m.set_act_scale(act_scale)
+    dep = QLinearINT8Deploy.from_fms_mo(m, use_int_kernel="cutlass", use_dynamic_max_act_Qfunc=-1,
+                                        recalc_clipvals=False, target_device=dev)
+    y = dep(x.to(dev))
+    bufs = O.deploy_prepare(m.weight.detach(), m.bias.detach(), m.quantize_weight.clip_val, act_scale, 0.5)
+    ref = O.deploy_forward(x, bufs)
+    assert torch.equal(dep.weight.cpu(), bufs["weight"]) and torch.equal(dep.w_scale.cpu(), bufs["w_scale"])
+    assert y.shape == (B, S, N) and y.dtype == torch.float16
+    assert torch.equal(dep.input_scale.cpu().reshape(-1), ref["input_scale"].float().reshape(-1))
+    assert torch.equal(y.cpu().view(torch.int16), ref["y"].view(torch.int16))
+
+
+def test_deploy_module_converted_on_gpu_matches_within_tolerance(dev):
+    """Converting on the GPU uses the GPU's pow / division roundings for the offline scales, so it
+    is only tolerance-equal to the CPU-converted module."""
+    from fms_mo_amd.modules.linear import QLinearINT8Deploy
+
+    K, N = 512, 256
+    m = make_qlinear(None, K, N, smoothq=True)
+    x = outlier_x(64, K, 5)
+    m.set_act_scale(x.float().abs().amax(dim=0))
+    dep_cpu = QLinearINT8Deploy.from_fms_mo(m, use_dynamic_max_act_Qfunc=-1, recalc_clipvals=False, target_device=dev)
+    dep_gpu = QLinearINT8Deploy.from_fms_mo(m.to(dev), use_dynamic_max_act_Qfunc=-1, recalc_clipvals=False)
+    assert (dep_cpu.weight != dep_gpu.weight).float().mean() < 1e-3
+    torch.testing.assert_close(dep_gpu(x.to(dev)).float(), dep_cpu(x.to(dev)).float(), rtol=1e-2, atol=1e-2)
+
+
+def test_qlinear_eval_forward_within_tolerance_of_fake_quant(dev):
+    K, N = 1024, 768
+    m = make_qlinear(dev, K, N, smoothq=True)
+    x = outlier_x(300, K, 6)
+    a = x.float().abs().amax(dim=0)
+    m.set_act_scale(a.to(dev))
+    m.train()
+    with torch.no_grad():
+        y_train = m(x.to(dev))            # torch-op fake-quant path (also sets clip_val)
+    m.eval()
+    with torch.no_grad():
+        y = m(x.to(dev))                  # integer path on the HIP kernels
+    assert m.num_module_called.item() == 2 and y.dtype == torch.float16
+    ref = O.qlinear_forward(x, m.weight.detach().cpu(), m.bias.detach().cpu(), a, 0.5,
+                            w_clip_val=m.quantize_weight.clip_val.cpu())
+    d = (y.cpu().float() - ref.float()).abs()
+    assert (d > 1e-2 + 1e-2 * ref.float().abs()).float().mean() < 1e-3 and d.max() < 5e-2
+    # the training-mode forward quantizes the weights on the grid of the CURRENT abs-max
+    ref_train = O.qlinear_forward(x, m.weight.detach().cpu(), m.bias.detach().cpu(), a, 0.5)
+    d2 = (y_train.cpu().float() - ref_train.float()).abs()
+    assert (d2 > 1e-2 + 1e-2 * ref_train.float().abs()).float().mean() < 1e-2
+
+
+def test_deploy_chunked_branches(dev):
+    from fms_mo_amd.modules.linear import QLinearINT8Deploy
+
+    K, N = 512, 256
+    x = outlier_x(64, K, 7)
+    m = make_qlinear(None, K, N)
+    bufs = O.deploy_prepare(m.weight.detach(), m.bias.detach(), m.quantize_weight.clip_val)
+    q_x, s_x, _ = O.quant_act_pertoken_i8(x)
+    # cutlass + chunk loop: clamp to 24 bits, drop 4 LSBs per 64-chunk, fp32 scales
+    dep = QLinearINT8Deploy.from_fms_mo(m, use_int_kernel="cutlass", use_dynamic_max_act_Qfunc=-1,
+                                        recalc_clipvals=False, chunk_size=64, truncate_lsb=4, max_acc_bits=24,
+                                        target_device=dev)
+    y = dep(x.to(dev)).cpu()
+    acc = O.chunk_matmul_i8(q_x, bufs["weight"], None, 64, 4, 24)
+    ref = (acc * (s_x * bufs["w_scale"]) + bufs["bias"]).to(torch.float16)
+    assert torch.equal(y.view(torch.int16), ref.view(torch.int16))
+    # triton flavour: chunked kernel + fp16-scale epilogue
+    dep2 = QLinearINT8Deploy.from_fms_mo(m, use_int_kernel="triton", use_dynamic_max_act_Qfunc=-1,
+                                         recalc_clipvals=False, chunk_size=64, truncate_lsb=8, target_device=dev)
+    y2 = dep2(x.to(dev)).cpu()
+    acc2 = O.chunk_matmul_i8(q_x, bufs["weight"], None, 64, 8, 32)
+    ref2 = O.epilogue_ref(acc2, s_x, bufs["w_scale"], bufs["bias"])
+    assert torch.equal(y2.view(torch.int16), ref2.view(torch.int16))
+
+
+def test_custom_ops(dev):
+    from fms_mo_amd.custom_ext_kernels.utils import imatmul_ops_reg, native_gemm_ops_reg
+
+    imatmul_ops_reg()
+    native_gemm_ops_reg()
+    a = torch.randint(-128, 128, (2, 9, 256), generator=gen(8), dtype=torch.int8)
+    w = torch.randint(-128, 128, (96, 256), generator=gen(9), dtype=torch.int8)
+    ref = O.int_gemm(a.reshape(-1, 256), w).reshape(2, 9, 96)
+    ad, wd = a.to(dev), w.to(dev)
+    assert torch.equal(torch.ops.fms_mo.imatmul(ad, wd.t()).cpu(), ref)                 # W.t() view
+    assert torch.equal(torch.ops.fms_mo.imatmul(ad, wd.t().contiguous()).cpu(), ref)    # row-major [K,N]
+    assert torch.equal(torch.ops.cutlass_gemm.i8i32nt(ad[0], wd.t()).cpu(), ref[0])
+    assert torch.equal(torch.ops.mygemm.gemm_nt_i8i32(ad[0], wd).cpu(), ref[0])
+    s_i, s_w = torch.tensor([0.02]), torch.rand(96, generator=gen(10)) * 1e-2
+    bias = torch.randn(96, generator=gen(11))
+    y = torch.ops.fms_mo.iaddmm(bias.to(dev), ad[0], wd.t(), s_i.to(dev), s_w.to(dev)).cpu()
+    torch.testing.assert_close(y, s_i.float() * ref[0] * s_w + bias, rtol=1e-5, atol=1e-5)
+    x = (torch.randn(9, 256, generator=gen(12)) * 2).half()
+    zp = torch.tensor([131])
+    y2 = torch.ops.fms_mo.q_iaddmm_dq(bias.to(dev), x.to(dev), wd.t(), s_i.to(dev), zp.to(dev), s_w.to(dev)).cpu()
+    q = torch.clamp((x / s_i + zp - 128).round(), -128, 127).to(torch.int8)
+    exp = (s_i.float() * O.int_gemm(q, w) * s_w + bias).to(torch.float16)
+    torch.testing.assert_close(y2.float(), exp.float(), rtol=2e-3, atol=2e-3)
+    q3 = torch.ops.fms_mo.q_per_t_sym(x.float().to(dev), s_i.to(dev), torch.tensor([3]).to(dev)).cpu()
+    exp3 = torch.quantize_per_tensor(x.float(), 0.02, 3, torch.qint8).int_repr()
+    assert torch.equal(q3, exp3)
+
+
+def test_linear_fpx_acc_like_reference_test(dev):
+    """fms-model-optimizer tests/triton_kernels/test_triton_mm.py:125-149 (fp32 Linear, 512 tokens)."""
+    from fms_mo_amd.modules.linear import LinearFPxAcc
+
+    torch.manual_seed(23)
+    for fin, fout in [(64, 128), (256, 1024)]:
+        lin = torch.nn.Linear(fin, fout).to(dev)
+        inputs = torch.randn((512, fin)).to(dev)
+        for t in [0, 8, 12, 16]:
+            fpx = LinearFPxAcc.from_nn(lin, trun_bits=t)
+            with torch.no_grad():
+                base = lin(inputs)
+                rel = (torch.norm(fpx(inputs) - base) / torch.norm(base)).item()
+            assert rel < (1e-2 if t > 10 else 1e-4), (fin, t, rel)
+
+
+@pytest.mark.parametrize("dl16", [False, True])
+def test_linear_fpx_acc_dynamic_fp8_vs_oracle(dev, dl16):
+    from fms_mo_amd.modules.linear import LinearFPxAcc
+
+    lin = torch.nn.Linear(256, 192).to(torch.bfloat16)
+    x = (torch.randn(40, 256, generator=gen(13)) * 2).bfloat16()
+    fpx = LinearFPxAcc.from_nn(lin.to(dev), trun_bits=8, chunk_size=64, dynamic_fp8="per_token",
+                               clamp_acc_to_dl16=dl16)
+    y = fpx(x.to(dev)).cpu()
+    ref = O.fpxacc_forward(x, lin.weight.detach().cpu(), lin.bias.detach().cpu(), 8, 64, "per_token", dl16)
+    torch.testing.assert_close(y.float(), ref.float(), rtol=2e-2, atol=2e-2)
+
+
+def test_qlinear_int8_train_forward_vs_oracle(dev):
+    from fms_mo_amd.modules.linear import QLinearINT8Train
+
+    lin = torch.nn.Linear(512, 128).half()
+    x = (torch.randn(64, 512, generator=gen(14))).half()
+    m = QLinearINT8Train.from_fms_mo(lin.to(dev), lsb_trun_bits=8, chunk_size=64, max_acc_bits=24)
+    y = m(x.to(dev)).cpu()
+    ref, _, _, _ = O.int8train_forward(x, lin.weight.detach().cpu(), lin.bias.detach().cpu(), 8, 64, 24)
+    assert torch.equal(y.view(torch.int16), ref.view(torch.int16))
+
+
+@pytest.mark.parametrize("cfg", [("tensor", "token", True), ("channel", "token", True),
+                                 ("tensor", "tensor", True), ("tensor", "tensor", False)])
+def test_fp8_linear_vs_oracle(dev, cfg):
+    from fms_mo_amd.modules.fp8_linear import FP8Linear
+
+    wstrat, astrat, dynamic = cfg
+    g = gen(15)
+    W = 0.02 * torch.randn(384, 512, generator=g)
+    b = 0.1 * torch.randn(384, generator=g)
+    x = torch.randn(2, 50, 512, generator=g).bfloat16()
+    m = FP8Linear.from_float(W, b, per_channel=wstrat == "channel", act=astrat)
+    if not dynamic:
+        m.linear_config["input_activations"]["dynamic"] = False
+        m.input_scale = torch.nn.Parameter(torch.tensor([0.0123]), requires_grad=False)
+    y = m.to(dev)(x.to(dev)).cpu()
+    assert y.shape == (2, 50, 384) and y.dtype == torch.bfloat16 and torch.isfinite(y).all()
+    x2 = x.reshape(-1, 512)
+    if not dynamic:
+        in_scale = torch.tensor([0.0123])
+    elif astrat == "tensor":
+        in_scale = (x2.abs().amax().float() / 448).clamp(min=1e-12).reshape(1)
+    else:
+        in_scale = None
+    ref, qx, s_x = O.fp8_linear_forward(x, m.weight.data.cpu(), m.weight_scale.data.cpu(), b.bfloat16(), in_scale)
+    exact = (qx.double() * s_x.double()) @ (m.weight.data.cpu().double() * m.weight_scale.data.cpu().double()).t() + b.double()
+    torch.testing.assert_close(y.reshape(-1, 384).double(), exact, rtol=1e-2, atol=1e-2)
+    torch.testing.assert_close(y.float(), ref.float(), rtol=3e-2, atol=3e-2)

@@ -1,0 +1,228 @@
+"""Host-side logic that needs no GPU: quantizer state machines, module construction and
+conversion (offline weight preparation) against the oracle, op registration, chunk-size rules."""
+import pickle
+
+import pytest
+import torch
+
+from oracle import qlinear_oracle as O
+
+
+def gen(seed):
+    return torch.Generator().manual_seed(seed)
+
+
+def make_qlinear(K=128, N=96, smoothq=False, bias=True, qw_mode="maxperCh", dtype=torch.float16):
+    from fms_mo_amd.modules.linear import QLinear
+
+    qcfg = {"smoothq": smoothq, "smoothq_alpha": 0.5}
+    m = QLinear(K, N, bias=bias, num_bits_feature=8, qa_mode="pertokenmax", num_bits_weight=8,
+                qw_mode=qw_mode, qcfg=qcfg, device="cpu")
+    g = gen(0)
+    with torch.no_grad():
+        m.weight.copy_(0.02 * torch.randn(N, K, generator=g))
+        if bias:
+            m.bias.copy_(0.01 * torch.randn(N, generator=g))
+    m.to(dtype)
+    m.quantize_weight.float()       # quantizer buffers stay fp32, as when they are created after .half()
+    if smoothq:
+        m.smoothq_act_scale = m.smoothq_act_scale.float()
+        m.smoothq_alpha = m.smoothq_alpha.float()
+    return m
+
+
+def test_quantizer_factories_and_scope():
+    from fms_mo_amd.quant import quantizers as Q
+
+    assert isinstance(Q.get_activation_quantizer("pertokenmax", 8), Q.QMaxDynamic)
+    assert Q.get_activation_quantizer("max_perCh", 8).reduce_dim == -2
+    assert isinstance(Q.get_activation_quantizer("maxsym", 8), Q.Qmax)
+    assert Q.get_weight_quantizer("maxperCh", 8, w_shape=(16, 32)).perCh == 16
+    assert not Q.get_weight_quantizer("max", 8, w_shape=(16, 32)).perCh
+    assert isinstance(Q.get_weight_quantizer("fp8_e4m3_scale_perCh", 8, w_shape=(16, 32)), Q.to_fp8)
+    for mode in ["pact+", "lsq+", "sawb+", "brecq"]:
+        with pytest.raises(NotImplementedError):
+            Q.get_activation_quantizer(mode, 8)
+    with pytest.raises(ValueError):
+        Q.get_weight_quantizer("nonsense", 8)
+
+
+def test_qmaxdynamic_matches_oracle():
+    from fms_mo_amd.quant.quantizers import QMaxDynamic
+
+    x = (torch.randn(8, 64, generator=gen(1)) * 2).half()
+    assert torch.equal(QMaxDynamic(8, dim=-1)(x), O.fake_quant_act_pertoken(x))
+    with pytest.raises(ValueError):
+        QMaxDynamic(8, dim=0)
+
+
+def test_qmax_state_machine_and_per_channel_levels():
+    from fms_mo_amd.quant.quantizers import Qmax
+
+    W = (0.02 * torch.randn(16, 64, generator=gen(2)))
+    q = Qmax(8, align_zero=True, perCh=16)
+    assert torch.all(q.clip_val == 0)
+    q.train()
+    out = q(W)
+    cv = W.abs().amax(dim=1)
+    assert torch.allclose(q.clip_val, cv)                              # first call copies, EMA of equal values
+    assert torch.equal(out, O.fake_quant_weight_perch(W, cv))
+    q.eval()
+    out2 = q(W * 0.5)                                                  # eval: stored clip values define the grid
+    assert torch.equal(out2, O.fake_quant_weight_perch(W * 0.5, q.clip_val))
+    q.train()
+    q(W * 2)
+    assert torch.allclose(q.clip_val, 0.9 * cv + 0.1 * 2 * cv, rtol=1e-6)   # moving average, factor 0.1
+    # per-tensor variant: 254 levels, symmetric
+    qt = Qmax(8, align_zero=True)
+    qt.train()
+    o = qt(W)
+    step = W.abs().max() * 2 / 254
+    assert torch.allclose(o / step, torch.round(o / step), atol=1e-3)
+    assert torch.allclose(o, W, atol=step.item() / 2 + 1e-7)
+
+
+def test_fp8_emulation_quantizer_closed_form():
+    from fms_mo_amd.quant.quantizers import to_fp8
+
+    x = (torch.randn(4, 64, generator=gen(3)) * 5).bfloat16()
+    q = to_fp8(8, "fp8_e4m3_scale", perToken=True)
+    s = 448 / x.abs().amax(dim=-1, keepdim=True).clamp(min=1e-12)     # multiplicative scale, in bf16
+    expect = ((x * s).clamp(-448, 448).to(torch.float8_e4m3fn).to(torch.bfloat16) / s).to(torch.bfloat16)
+    assert torch.equal(q(x), expect)
+    sat = to_fp8(8, "fp8_e4m3_sat")
+    assert sat(torch.tensor([1000.0, -1000.0, 0.3])).tolist() == [448.0, -448.0, 0.3125]
+    with pytest.raises(ValueError):
+        to_fp8(8, "fp8_e5m2_sat")
+
+
+def test_qlinear_constructor_surface():
+    m = make_qlinear(smoothq=True)
+    for attr in ["quantize_feature", "quantize_weight", "num_bits_feature", "num_bits_weight", "qa_mode",
+                 "qw_mode", "smoothq", "smoothq_act_scale", "smoothq_alpha", "qcfg", "calib_counter",
+                 "num_module_called"]:
+        assert hasattr(m, attr)
+    assert m.smoothq_act_scale.shape == (128,) and m.smoothq_alpha.item() == 0.5
+    assert "QLinear(128,96" in repr(m)
+    with pytest.raises(KeyError):
+        from fms_mo_amd.modules.linear import QLinear
+
+        QLinear(8, 8, device="cpu")      # qcfg is required, like the reference
+    m.set_act_scale(torch.ones(128))
+    s = m.get_smoothq_scale(torch.zeros(1, 128, dtype=torch.float16))
+    assert s.dtype == torch.float16 and s.shape == (1, 128)
+    assert torch.equal(s, O.smoothq_scale_qlinear(m.weight, m.smoothq_act_scale, 0.5, torch.float16))
+
+
+@pytest.mark.parametrize("smoothq", [False, True])
+def test_from_fms_mo_offline_preparation_matches_oracle(smoothq):
+    from fms_mo_amd.modules.linear import QLinearINT8Deploy, prepare_deploy_weights
+
+    m = make_qlinear(smoothq=smoothq)
+    act_scale = None
+    if smoothq:
+        act_scale = torch.rand(128, generator=gen(4)) * 8 + 0.5
+        m.set_act_scale(act_scale)
+    with torch.no_grad():
+        m.quantize_weight.train()
+        m.quantize_weight(m.weight)            # one training-mode pass initialises clip_val
+    m.eval()
+    dep = QLinearINT8Deploy.from_fms_mo(m, use_int_kernel="cutlass", use_dynamic_max_act_Qfunc=-1,
+                                        recalc_clipvals=False, target_device="cpu")
+    bufs = O.deploy_prepare(m.weight.detach(), m.bias.detach(), m.quantize_weight.clip_val, act_scale, 0.5)
+    assert dep.weight.dtype == torch.int8 and torch.equal(dep.weight, bufs["weight"])
+    assert torch.equal(dep.w_scale, bufs["w_scale"])
+    assert torch.equal(dep.smoothq_scale, bufs["smoothq_scale"])
+    assert torch.equal(dep.bias, bufs["bias"])
+    assert dep.input_zp.item() == 127 and torch.all(dep.corr_term == 0) and torch.all(dep.w_zp == 0)
+    assert dep._get_name() == "QLinear_INT8" and "int_kernel=cutlass" in dep.extra_repr()
+    for name in ["input_scale", "input_zp", "w_scale", "w_zp", "smoothq_scale", "corr_term", "bias"]:
+        assert name in dict(dep.named_buffers())
+    # the standalone helper used by the benchmark performs the same recipe
+    if not smoothq:
+        w8, ws, sq = prepare_deploy_weights(m.weight.detach(), None, 0.5, m.quantize_weight.clip_val)
+        assert torch.equal(w8, bufs["weight"]) and torch.equal(ws, bufs["w_scale"])
+    # forward on CPU raises instead of taking some other path
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        dep(torch.zeros(2, 128, dtype=torch.float16))
+    # pickling drops and rebinds the op handles
+    dep2 = pickle.loads(pickle.dumps(dep))
+    assert torch.equal(dep2.weight, dep.weight) and callable(dep2.iaddmm)
+
+
+def test_static_activation_variants_of_from_fms_mo():
+    from fms_mo_amd.modules.linear import QLinearINT8Deploy
+
+    m = make_qlinear()
+    m.qa_mode = "maxsym"
+    m.quantize_feature.clip_val = torch.tensor([4.0])
+    m.quantize_feature.clip_valn = torch.tensor([-4.0])
+    dep = QLinearINT8Deploy.from_fms_mo(m, use_PT_native_Qfunc=True, target_device="cpu")
+    assert dep.useSymAct and dep.input_scale.item() == pytest.approx(8.0 / 254)
+    assert dep.input_zp.item() == 127
+    dep2 = QLinearINT8Deploy.from_fms_mo(m, target_device="cpu")          # fms_mo formula
+    assert "quant_stepsize" in dict(dep2.named_buffers())
+    assert dep2.input_scale.item() == pytest.approx(8.0 / 254)
+    dep3 = QLinearINT8Deploy.from_fms_mo(m, use_dynamic_max_act_Qfunc=5, target_device="cpu")
+    assert dep3.use_fake_zero_shift and dep3.input_zp.item() == 5
+    w_sum = dep3.weight.to(torch.int).sum(dim=1)
+    assert torch.allclose(dep3.corr_term, 5 * w_sum * dep3.w_scale.float() * 1.0)
+
+
+def test_from_torch_iw():
+    from fms_mo_amd.modules.linear import QLinearINT8Deploy
+
+    lin = torch.nn.Linear(64, 32)
+    with torch.no_grad():
+        lin.weight.copy_(torch.randint(-127, 128, (32, 64), generator=gen(5)).float())
+    dep = QLinearINT8Deploy.from_torch_iW(lin, "int8", 6.0, -2.0, 0.3, 0.0, target_device="cpu")
+    assert dep.weight.dtype == torch.int8 and torch.equal(dep.weight.float(), lin.weight)
+    assert dep.input_scale.item() == pytest.approx(8.0 / 255) and dep.input_zp.item() == round(2.0 / (8.0 / 255))
+    assert dep.w_scale.item() == pytest.approx(0.6 / 254)
+
+
+def test_custom_ops_are_registered_with_fake_impls():
+    from fms_mo_amd.custom_ext_kernels.utils import imatmul_ops_reg, native_gemm_ops_reg
+
+    imatmul_ops_reg()
+    native_gemm_ops_reg()
+    for ns, op in [("fms_mo", "imatmul"), ("fms_mo", "iaddmm"), ("fms_mo", "q_iaddmm_dq"),
+                   ("fms_mo", "q_per_t_sym"), ("cutlass_gemm", "i8i32nt"), ("mygemm", "gemm_nt_i8i32")]:
+        assert hasattr(getattr(torch.ops, ns), op)
+    m1 = torch.empty(2, 3, 64, dtype=torch.int8, device="meta")
+    m2 = torch.empty(64, 48, dtype=torch.int8, device="meta")
+    out = torch.ops.fms_mo.imatmul(m1, m2)
+    assert out.shape == (2, 3, 48) and out.dtype == torch.int32
+    with pytest.raises((NotImplementedError, RuntimeError)):
+        torch.ops.fms_mo.imatmul(torch.zeros(2, 64, dtype=torch.int8), torch.zeros(64, 8, dtype=torch.int8))
+
+
+def test_chunk_wrapper_argument_rules():
+    from fms_mo_amd.custom_ext_kernels.hip_kernels import matmul_chunk_truncate
+
+    a = torch.zeros(4, 64)
+    with pytest.raises(AssertionError, match="Incompatible dimensions"):
+        matmul_chunk_truncate(a, torch.zeros(32, 8))
+    with pytest.raises(AssertionError, match="dtypes inconsistent"):
+        matmul_chunk_truncate(a, torch.zeros(64, 8, dtype=torch.float16))
+    with pytest.raises(AssertionError, match="23 mantissa bits"):
+        matmul_chunk_truncate(a, torch.zeros(64, 8), chunk_trun_bits=23)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        matmul_chunk_truncate(a, torch.zeros(64, 8))
+
+
+def test_fp8_linear_construction_and_offline_quantization():
+    from fms_mo_amd.modules.fp8_linear import FP8Linear, get_fp8_linear
+
+    cfg = {"weights": {"strategy": "channel", "symmetric": True, "dynamic": False},
+           "input_activations": {"strategy": "token", "symmetric": True, "dynamic": True}}
+    m = get_fp8_linear(64, 32, True, cfg)
+    assert m.weight.dtype == torch.float8_e4m3fn and m.weight_scale.shape == (32, 1) and m.bias.shape == (32,)
+    W = 0.02 * torch.randn(32, 64, generator=gen(6))
+    f = FP8Linear.from_float(W, None, per_channel=True)
+    scale = (W.abs().amax(dim=1, keepdim=True) / 448).clamp(min=1e-12)
+    assert torch.equal(f.weight_scale.data, scale)
+    assert torch.equal(f.weight.data.view(torch.uint8), (W / scale).clamp(-448, 448).to(torch.float8_e4m3fn).view(torch.uint8))
+    assert "FP8Linear(in=64, out=32" in repr(f)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        f(torch.zeros(2, 64, dtype=torch.bfloat16))

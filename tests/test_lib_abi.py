@@ -1,0 +1,89 @@
+"""The C-ABI library: it loads, exports every symbol the header declares, validates arguments
+(no compute is launched here -- every call below is rejected before any kernel launch)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "fmsmo_hip.h")
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(fmsmo_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_the_expected_entry_points():
+    syms = declared_symbols()
+    for s in ["fmsmo_quant_act_i8_pertoken", "fmsmo_quant_act_i8_static", "fmsmo_quant_act_fp8_pertoken",
+              "fmsmo_gemm_i8_i32", "fmsmo_gemm_i8_dq", "fmsmo_gemm_fp8_dq", "fmsmo_gemv_i8_dq",
+              "fmsmo_gemv_fp8_dq", "fmsmo_matmul_chunk_i8", "fmsmo_matmul_chunk_fp",
+              "fmsmo_grouped_gemm_i8_dq", "fmsmo_abi_version", "fmsmo_status_str", "fmsmo_last_error"]:
+        assert s in syms
+
+
+def test_library_exports_every_declared_symbol():
+    from fms_mo_amd import _lib
+
+    lib = _lib.load()
+    for s in declared_symbols():
+        assert hasattr(lib, s), f"{s} declared in include/fmsmo_hip.h but not exported"
+    assert set(_lib.SIGNATURES) | set(_lib.OTHER) == set(declared_symbols())
+    assert lib.fmsmo_abi_version() == 1
+    assert lib.fmsmo_status_str(0) == b"ok"
+
+
+def test_every_declaration_cites_the_reference():
+    text = open(HEADER).read()
+    for name in ["fms_mo/modules/linear.py:1085-1100", "cutlass_i8i32gemm.cu:100-120",
+                 "ext_kernel_cublas.cpp:103-195", "triton_kernels.py:211-302", "fp8_linear.py:275-283"]:
+        assert name in text
+
+
+def test_argument_validation_without_a_gpu():
+    from fms_mo_amd import _lib
+
+    lib = _lib.load()
+    buf = (ctypes.c_char * 4096)()
+    p = ctypes.addressof(buf)
+    p = (p + 15) // 16 * 16
+    # NULL pointers
+    assert lib.fmsmo_gemm_i8_i32(None, 64, p, 64, p, 64, 1, 1, 64, None) == 1
+    assert lib.fmsmo_quant_act_i8_pertoken(None, 0, 64, None, 0, 0, 0, p, 64, p, 1, 64, None) == 1
+    # bad shapes: leading dimension smaller than K, negative M
+    assert lib.fmsmo_gemm_i8_i32(p, 32, p, 64, p, 64, 1, 1, 64, None) == 2
+    assert lib.fmsmo_gemm_i8_i32(p, 64, p, 64, p, 64, -1, 1, 64, None) == 2
+    # alignment: K not a multiple of 16, misaligned pointer
+    assert lib.fmsmo_gemm_i8_i32(p, 24, p, 24, p, 64, 1, 1, 24, None) == 3
+    assert lib.fmsmo_gemm_i8_i32(p + 1, 64, p, 64, p, 64, 1, 1, 64, None) == 3
+    # unsupported enum values
+    assert lib.fmsmo_quant_act_i8_pertoken(p, 7, 64, None, 0, 0, 0, p, 64, p, 1, 64, None) == 4
+    assert lib.fmsmo_gemv_i8_dq(p, 128, p, 128, p, 1, p, 1, None, 0, 0, p, 0, 64, 17, 64, 128, None) == 4  # M > 16
+    assert lib.fmsmo_matmul_chunk_i8(p, 64, p, 64, None, p, 64, 1, 1, 64, 48, 0, 32, 1, None) == 4  # chunk not 2^n
+    assert lib.fmsmo_matmul_chunk_fp(p, 64, p, 64, 1, None, p, 64, 1, 1, 64, 64, 23, 0, 1, None) == 4  # t > 22
+    # empty problems are accepted without a launch
+    assert lib.fmsmo_gemm_i8_i32(p, 64, p, 64, p, 64, 0, 1, 64, None) == 0
+
+
+def test_python_wrapper_raises_on_cpu_tensors():
+    import torch
+
+    from fms_mo_amd import kernels
+
+    a = torch.zeros(4, 64, dtype=torch.int8)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        kernels.gemm_i8_i32(a, a)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        kernels.quant_act_i8_pertoken(torch.zeros(4, 64, dtype=torch.float16))
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    from fms_mo_amd import _lib
+
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libfmsmo_hip.so")
+    with pytest.raises(_lib.FmsMoHipError, match="no fallback"):
+        _lib.load()
