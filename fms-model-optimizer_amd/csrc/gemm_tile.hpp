@@ -355,20 +355,36 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(GemmArgs g, Ep
   typename Epi::Col colctx[FN];
 #pragma unroll
   for (int j = 0; j < FN; ++j) colctx[j] = epi.col(min(n_base + j * 32, g.N - 1), expert, g.N);
+  // Interior tiles (the common case) take a branch-free path; per-row epilogue data is fetched
+  // 16 rows at a time with clamped indices so that the loads are issued back to back.
+  const bool interior = (row_lo + BM <= row_hi) && (col_lo + BN <= g.N);
 #pragma unroll
-  for (int i = 0; i < FM; ++i)
+  for (int i = 0; i < FM; ++i) {
+    typename Epi::Row rowctx[16];
 #pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      const int m = m_base + i * 32 + (v >> 2) * 8 + (v & 3);
-      if (m < row_hi) {
-        const typename Epi::Row rowctx = epi.row(m);
+    for (int v = 0; v < 16; ++v)
+      rowctx[v] = epi.row(min(m_base + i * 32 + (v >> 2) * 8 + (v & 3), row_hi - 1));
+    if (interior) {
 #pragma unroll
-        for (int j = 0; j < FN; ++j) {
-          const int n = n_base + j * 32;
-          if (n < g.N) epi.store(m, n, acc[i][j][v], rowctx, colctx[j]);
+      for (int v = 0; v < 16; ++v) {
+        const int m = m_base + i * 32 + (v >> 2) * 8 + (v & 3);
+#pragma unroll
+        for (int j = 0; j < FN; ++j) epi.store(m, n_base + j * 32, acc[i][j][v], rowctx[v], colctx[j]);
+      }
+    } else {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int m = m_base + i * 32 + (v >> 2) * 8 + (v & 3);
+        if (m < row_hi) {
+#pragma unroll
+          for (int j = 0; j < FN; ++j) {
+            const int n = n_base + j * 32;
+            if (n < g.N) epi.store(m, n, acc[i][j][v], rowctx[v], colctx[j]);
+          }
         }
       }
     }
+  }
 #ifdef FMSMO_CLK
   if (blockIdx.x == 0 && tid == 0 && g.clk) { g.clk[4] = clock64(); g.clk[5] = wall_clock64(); }
 #endif
@@ -412,16 +428,17 @@ struct EpiDequant {
   }
   __device__ __forceinline__ Row row(int m) const { return Row{a_scale[a_stride ? m : 0]}; }
   __device__ __forceinline__ void store(int m, int n, AccT v, Row r, Col c) const {
-    float out;
+    const int64_t idx = (int64_t)m * ldy + n;
     if constexpr (REF_F16) {
       // separate fp32 multiply and add (no fma), scale product rounded to fp16 first,
       // result rounded to fp16 before the cast to the output dtype
       const float sc = round_to<FMSMO_F16>(__fmul_rn(r.as, c.ws));
-      out = round_to<FMSMO_F16>(__fadd_rn(__fmul_rn((float)v, sc), c.b));
+      const u16 h = f32_to_f16(__fadd_rn(__fmul_rn((float)v, sc), c.b));
+      if constexpr (OUT == FMSMO_F16) ((u16*)y)[idx] = h;
+      else store_from_f32<OUT>(y, idx, f16_to_f32(h));
     } else {
-      out = __fmaf_rn((float)v, __fmul_rn(r.as, c.ws), c.b);
+      store_from_f32<OUT>(y, idx, __fmaf_rn((float)v, __fmul_rn(r.as, c.ws), c.b));
     }
-    store_from_f32<OUT>(y, (int64_t)m * ldy + n, out);
   }
 };
 
