@@ -1,6 +1,8 @@
 // Host launchers of the tiled MFMA GEMMs (int8 -> int32, int8 / e4m3 with fused dequantizing
 // epilogue, grouped mixture-of-experts variant).
 #include "gemm_tile.hpp"
+#include <cmath>
+#include <cstdlib>
 
 using namespace fmsmo;
 
@@ -53,7 +55,33 @@ int check_gemm(const void* a, int64_t lda, const void* b, int64_t ldb, const voi
 // by the caller-visible rule "K % 64 == 0" for the MFMA path (all transformer shapes), anything
 // else goes to the slow generic kernel.
 struct TileBig { static constexpr int BM = 256, BN = 256, BK = 64, NST = 4, WGM = 2, WGN = 2; };
+struct TileWide { static constexpr int BM = 128, BN = 256, BK = 64, NST = 4, WGM = 2, WGN = 2; };
 struct TileMid { static constexpr int BM = 128, BN = 128, BK = 64, NST = 4, WGM = 2, WGN = 2; };
+
+// Pick the tile shape by (relative kernel efficiency) x (fill of the last round of tiles over
+// the 256 compute units).  The efficiencies are measured loop efficiencies of the three shapes
+// (bigger tiles move fewer bytes per MFMA); 128x128 tiles fit two blocks per CU.
+int pick_tile(int M, int N) {
+  static const char* force = getenv("FMSMO_TILE");  // tuning aid: 0 = 256x256, 1 = 128x256, 2 = 128x128
+  if (force && force[0] >= '0' && force[0] <= '2') return force[0] - '0';
+  // Fitted to measurements on the Llama / Granite shapes: relative loop efficiency of the three
+  // tile shapes, and a sub-linear penalty for a partially filled last round (idle CUs leave
+  // power, hence clock, to the busy ones).
+  const double eff[3] = {1.0, 0.76, 0.70};
+  const int bm[3] = {256, 128, 128}, bn[3] = {256, 256, 128};
+  int best = 0;
+  double best_score = -1;
+  for (int t = 0; t < 3; ++t) {
+    const long tiles = (long)div_up(M, bm[t]) * div_up(N, bn[t]);
+    const long slots = (t == 2 && tiles > 256) ? 512 : 256;  // two 128x128 blocks fit per CU
+    const long rounds = (tiles + slots - 1) / slots;
+    const double fill = (double)tiles / (double)(rounds * slots);
+    const double pad = ((double)M * N) / ((double)div_up(M, bm[t]) * bm[t] * (double)div_up(N, bn[t]) * bn[t]);
+    const double score = eff[t] * pow(fill, 0.6) * pad;
+    if (score > best_score) { best_score = score; best = t; }
+  }
+  return best;
+}
 
 template <class Tile, int OP, bool GROUPED, class Epi>
 void launch_tile(const GemmArgs& g0, const Epi& epi, hipStream_t st) {
@@ -99,11 +127,11 @@ __global__ void gemm_simple_kernel(GemmArgs g, Epi epi) {
 template <int OP, class Epi>
 void launch_any(const GemmArgs& g, const Epi& epi, hipStream_t st) {
   if (g.K % 64 == 0) {
-    const long tiles_big = (long)div_up(g.M, 256) * div_up(g.N, 256);
-    if (tiles_big >= 200 || (g.M >= 2048 && g.N >= 2048))
-      launch_tile<TileBig, OP, false>(g, epi, st);
-    else
-      launch_tile<TileMid, OP, false>(g, epi, st);
+    switch (pick_tile(g.M, g.N)) {
+      case 0: launch_tile<TileBig, OP, false>(g, epi, st); break;
+      case 1: launch_tile<TileWide, OP, false>(g, epi, st); break;
+      default: launch_tile<TileMid, OP, false>(g, epi, st); break;
+    }
   } else {
     dim3 grid(div_up(g.N, 64), (unsigned)g.M), block(64);
     hipLaunchKernelGGL((gemm_simple_kernel<OP, Epi>), grid, block, 0, st, g, epi);

@@ -116,6 +116,139 @@ __global__ __launch_bounds__(NW * 64) void gemv_kernel(GemvArgs g) {
   }
 }
 
+
+// Streaming variant (K = 128 * STEPS * NW).  Weight rows must be fetched as whole 128-byte
+// lines: a wave load that touches 16 rows x 64 B tops out near 4.4 TB/s on this part, 8 rows x
+// 128 B per instruction reaches 6.3 TB/s (a fully contiguous stream: 6.7).  MFMA operands want
+// 16 rows x 16 B per lane group instead, so every K step of 16 rows (2 KiB: two 8-row loads)
+// is transposed through a tiny wave-private LDS buffer (ds_write_b128 with an XOR swizzle,
+// ds_read_b128 of the operand fragments).  D steps of loads stay in flight in registers; nothing
+// is shared between waves except the final 16x16 partial sums, so the only barrier is one per
+// group of 16 rows.  The activation fragments of the wave's K slice stay in registers.
+template <int OP, int STEPS, int NW, int D>
+__global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(GemvArgs g, int G) {
+  static_assert(STEPS % D == 0, "pipeline depth must divide the steps per group");
+  typedef typename std::conditional<OP == FMSMO_OP_I8, int, float>::type AccT;
+  typedef AccT Acc4 __attribute__((ext_vector_type(4)));
+  __shared__ __attribute__((aligned(16))) uint8_t stage[NW][2][2048];
+  __shared__ AccT red[2][NW][256];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int r = lane & 15, kg = lane >> 4;
+  const int group0 = blockIdx.x * G;
+  const int ngroups = (g.N + 15) >> 4;
+  const int gcount = min(G, ngroups - group0);
+  const int kwave = wave * (STEPS * 128);
+
+  // activation fragments: lane (m = r, kg) holds x[m][kwave + s*128 + (h*4 + kg)*16 ...]
+  v4i xf[STEPS][2];
+  {
+    const uint8_t* xp = g.a + (int64_t)min(r, g.M - 1) * g.lda + kwave + kg * 16;
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) {
+      xf[s][0] = *(const v4i*)(xp + s * 128);
+      xf[s][1] = *(const v4i*)(xp + s * 128 + 64);
+    }
+  }
+  // weight loads: lane -> (row = lane / 8 [+8], 16-byte chunk = lane % 8): 8 rows x 128 B each
+  const int drow = lane >> 3, dpos = lane & 7;
+  // per-group row pointers, clamped (branch-free) for prefetch past the end and a ragged last group
+  const int64_t kcol = kwave + dpos * 16;
+  auto rowptr = [&](int gi, int half) {
+    const int row0 = min(group0 + min(gi, gcount - 1), ngroups - 1) * 16;
+    return g.b + (int64_t)min(row0 + half * 8 + drow, g.N - 1) * g.ldb + kcol;
+  };
+  const uint8_t* pc[2] = {rowptr(0, 0), rowptr(0, 1)};  // current group
+  const uint8_t* pn[2] = {rowptr(1, 0), rowptr(1, 1)};  // next group
+  auto load_item = [&](bool next, int s, v4i (&w)[2]) {
+    w[0] = __builtin_nontemporal_load((const v4i*)((next ? pn[0] : pc[0]) + s * 128));
+    w[1] = __builtin_nontemporal_load((const v4i*)((next ? pn[1] : pc[1]) + s * 128));
+  };
+  // staging: row-major [16 rows][128 B], chunk c of row q stored at position c ^ (q % 8)
+  const int wr0 = drow * 128 + ((dpos ^ drow) * 16);
+  const int wr1 = (8 + drow) * 128 + ((dpos ^ drow) * 16);
+  const int rr = r & 7;
+  const int rd0 = r * 128 + ((kg ^ rr) * 16), rd1 = r * 128 + (((4 + kg) ^ rr) * 16);
+
+  v4i wb[D][2];
+#pragma unroll
+  for (int j = 0; j < D; ++j) load_item(false, j, wb[j]);
+
+  // epilogue operands of output element e = threadIdx.x (n = e / 16, m = e % 16 of the group) are
+  // fetched at the top of each group so that their latency hides behind the weight stream
+  const int em = min((int)(threadIdx.x & 15), g.M - 1);
+  const float as = g.a_scale[g.a_stride ? em : 0];
+
+  // The last group of a block refills nothing (its prefetches would fall into the next block's
+  // rows), so the group body exists twice: streaming (LAST = false) and draining (LAST = true).
+  auto do_group = [&](auto last_tag, int gi) {
+    constexpr bool LAST = decltype(last_tag)::value;
+    const int en = min((group0 + gi) * 16 + (int)((threadIdx.x >> 4) & 15), g.N - 1);
+    const float ws = g.w_scale[g.w_stride ? en : 0];
+    float bv = 0.f;
+    if (g.bias) {
+      bv = g.bias_dtype == FMSMO_F16 ? f16_to_f32(((const u16*)g.bias)[en])
+           : g.bias_dtype == FMSMO_BF16 ? bf16_to_f32(((const u16*)g.bias)[en])
+                                        : ((const float*)g.bias)[en];
+    }
+    Acc4 acc = {0, 0, 0, 0};
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) {
+      uint8_t* st = &stage[wave][s & 1][0];
+      *(v4i*)(st + wr0) = wb[s % D][0];
+      *(v4i*)(st + wr1) = wb[s % D][1];
+      __builtin_amdgcn_sched_barrier(0);  // keep the refill right behind the registers it frees
+      if (!LAST || s + D < STEPS) load_item(s + D >= STEPS, (s + D) % STEPS, wb[s % D]);
+      __builtin_amdgcn_sched_barrier(0);
+      const v4i w0 = *(const v4i*)(st + rd0);
+      const v4i w1 = *(const v4i*)(st + rd1);
+      if constexpr (OP == FMSMO_OP_I8) {
+        acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(w0, xf[s][0], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(w1, xf[s][1], acc, 0, 0, 0);
+      } else {
+        const v8i wv = {w0[0], w0[1], w0[2], w0[3], w1[0], w1[1], w1[2], w1[3]};
+        const v8i xv = {xf[s][0][0], xf[s][0][1], xf[s][0][2], xf[s][0][3],
+                        xf[s][1][0], xf[s][1][1], xf[s][1][2], xf[s][1][3]};
+        acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wv, xv, acc, 0, 0, 0, 0, 0, 0);
+      }
+    }
+    // acc[v] = partial C(n = 16 (group0+gi) + 4 kg + v, m = r) of this wave's K slice.  The NW
+    // partials are summed by the first 256 threads; two exchange buffers alternate so that one
+    // barrier per group is enough.
+    if (!LAST) {
+      pc[0] = pn[0], pc[1] = pn[1];
+      pn[0] = rowptr(gi + 2, 0), pn[1] = rowptr(gi + 2, 1);
+    }
+    AccT* mine = &red[gi & 1][wave][0];
+#pragma unroll
+    for (int v = 0; v < 4; ++v) mine[(kg * 4 + v) * 16 + r] = acc[v];
+    __syncthreads();
+    if (threadIdx.x < 256) {
+      const int e = threadIdx.x;
+      AccT sum = red[gi & 1][0][e];
+#pragma unroll
+      for (int w = 1; w < NW; ++w) sum += red[gi & 1][w][e];
+      const int n = (group0 + gi) * 16 + (e >> 4), m = e & 15;
+      if (n < g.N && m < g.M) {
+        float out;
+        if (g.ref_f16) {
+          const float sc = round_to<FMSMO_F16>(__fmul_rn(as, ws));
+          out = round_to<FMSMO_F16>(__fadd_rn(__fmul_rn((float)sum, sc), bv));
+        } else {
+          out = __fmaf_rn((float)sum, __fmul_rn(as, ws), bv);
+        }
+        const int64_t idx = (int64_t)m * g.ldy + n;
+        if (g.y_dtype == FMSMO_F16) ((u16*)g.y)[idx] = f32_to_f16(out);
+        else if (g.y_dtype == FMSMO_BF16) ((u16*)g.y)[idx] = f32_to_bf16(out);
+        else ((float*)g.y)[idx] = out;
+      }
+    }
+  };
+  for (int gi = 0; gi + 1 < gcount; ++gi) do_group(std::false_type{}, gi);
+  do_group(std::true_type{}, gcount - 1);
+}
+
 }  // namespace fmsmo
 
 using namespace fmsmo;
@@ -145,6 +278,42 @@ int fmsmo_gemv_dispatch(int op, const void* a, int64_t lda, const void* b, int64
   g.a_stride = a_scale_n == 1 ? 0 : 1; g.w_stride = w_scale_n == 1 ? 0 : 1;
   g.bias = bias; g.bias_dtype = bias_dtype; g.ref_f16 = epilogue == FMSMO_EPI_REF_F16;
   g.y = y; g.y_dtype = y_dtype; g.ldy = ldy;
+  // Streaming variant when the K steps of 128 split evenly over the waves of a block in one of
+  // the instantiated (waves, steps per wave, loads in flight) shapes; other K use the generic
+  // kernel below.  One block per compute unit, each walking G consecutive groups: every block
+  // re-reads the activations and pays one memory latency before its stream starts, so fewer,
+  // longer-lived blocks win (measured: N = 28672, K = 4096 runs 26.5 us at G = 1, 21.0 us at
+  // G = 7).  FMSMO_GEMV_G overrides G for tuning.
+  {
+    static const int env_g = getenv("FMSMO_GEMV_G") ? atoi(getenv("FMSMO_GEMV_G")) : 0;
+    const int steps_total = (int)(K / 128);
+    const int64_t groups = (N + 15) / 16;
+    int NW = 0;
+    if (steps_total % 8 == 0) NW = 8;
+    else if (steps_total % 10 == 0) NW = 10;
+    const int STEPS = NW ? steps_total / NW : 0;
+    int G = env_g > 0 ? env_g : (int)((groups + 255) / 256);
+    if (G > 64) G = 64;
+    dim3 grid((unsigned)((groups + G - 1) / G)), block(NW * 64);
+    bool handled = true;
+#define GEMV_STREAM(OPV, NWV, ST, DV) \
+  hipLaunchKernelGGL((gemv_stream_kernel<OPV, ST, NWV, DV>), grid, block, 0, st, g, G)
+#define GEMV_SHAPES(OPV)                                            \
+  switch (NW * 100 + STEPS) {                                       \
+    case 801: GEMV_STREAM(OPV, 8, 1, 1); break;                     \
+    case 802: GEMV_STREAM(OPV, 8, 2, 2); break;                     \
+    case 804: GEMV_STREAM(OPV, 8, 4, 4); break;                     \
+    case 808: GEMV_STREAM(OPV, 8, 8, 4); break;                     \
+    case 814: GEMV_STREAM(OPV, 8, 14, 7); break;                    \
+    case 816: GEMV_STREAM(OPV, 8, 16, 4); break;                    \
+    case 1010: GEMV_STREAM(OPV, 10, 10, 5); break;                  \
+    default: handled = false; break;                                \
+  }
+    if (op == FMSMO_OP_I8) { GEMV_SHAPES(FMSMO_OP_I8) } else { GEMV_SHAPES(FMSMO_OP_E4M3) }
+#undef GEMV_SHAPES
+#undef GEMV_STREAM
+    if (handled) return fmsmo_check_launch();
+  }
   int nw = 8;
   while (nw > 1 && K % (128 * nw)) nw >>= 1;
   // enough row groups per block to amortise the activation re-reads, while keeping >= 2 blocks
