@@ -47,7 +47,9 @@ def make_layer(torch, dev, K, N, seed):
     act_scale = x.float().abs().amax(dim=0)
     xd, Wd = x.to(dev), W.to(dev)
     w_i8, w_scale, smooth = prepare_deploy_weights(Wd, act_scale.to(dev), 0.5)
-    return {"x": xd, "w": w_i8, "w_scale": w_scale.float(), "smooth": smooth.reshape(-1).float(),
+    # buffers as in a module cast with .half() for deployment: SmoothQuant scale in fp16, so
+    # x / smoothq_scale is an fp16 division (fms_mo/modules/linear.py:1331-1332)
+    return {"x": xd, "w": w_i8, "w_scale": w_scale.float(), "smooth": smooth.reshape(-1).half(),
             "bias": b.to(dev), "x_cpu": x, "W_cpu": W, "b_cpu": b, "act_scale_cpu": act_scale}
 
 

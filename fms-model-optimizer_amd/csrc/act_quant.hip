@@ -9,6 +9,8 @@
 // and then rounded to T, which equals the correctly rounded T division torch performs.
 #include "common.hpp"
 
+#include <type_traits>
+
 namespace fmsmo {
 
 constexpr int AQ_THREADS = 256;
@@ -35,12 +37,6 @@ __device__ __forceinline__ void load8(const void* x, size_t elem, float (&v)[8])
       }
     }
   }
-}
-
-__device__ __forceinline__ float load_any(const void* p, int dtype, size_t i) {
-  if (dtype == FMSMO_F16) return f16_to_f32(((const u16*)p)[i]);
-  if (dtype == FMSMO_BF16) return bf16_to_f32(((const u16*)p)[i]);
-  return ((const float*)p)[i];
 }
 
 __device__ __forceinline__ float block_max(float v, float* red) {
@@ -77,9 +73,12 @@ __global__ __launch_bounds__(AQ_THREADS) void quant_i8_pertoken_kernel(
   auto fetch = [&](int c, float (&e)[8]) {
     load8<XT>(x, xrow + (size_t)c * AQ_VEC, e);
     if (smooth) {
+      float d[8];
+      if (smooth_dtype == FMSMO_F16) load8<FMSMO_F16>(smooth, (size_t)c * AQ_VEC, d);
+      else if (smooth_dtype == FMSMO_BF16) load8<FMSMO_BF16>(smooth, (size_t)c * AQ_VEC, d);
+      else load8<FMSMO_F32>(smooth, (size_t)c * AQ_VEC, d);
 #pragma unroll
-      for (int i = 0; i < 8; ++i)
-        e[i] = round_to<T>(e[i] / load_any(smooth, smooth_dtype, (size_t)c * AQ_VEC + i));
+      for (int i = 0; i < 8; ++i) e[i] = round_to<T>(e[i] / d[i]);
     }
   };
 
@@ -123,6 +122,217 @@ __global__ __launch_bounds__(AQ_THREADS) void quant_i8_pertoken_kernel(
     float e[8];
     fetch(c, e);
     emit(c, e);
+  }
+}
+
+// ------------------------------------------------------------------ int8, dynamic per token,
+// 16-bit compute dtype (x, the SmoothQuant scale and every intermediate in fp16 or bf16).
+//
+// Blocks walk rows with a stride of gridDim.x and fetch the next row while they work on the
+// current one, so the bytes in flight per compute unit stay constant for the life of the kernel.
+// The SmoothQuant scale (or its reciprocal) of the thread's columns lives in registers for all
+// rows of the block, and the divided row is kept as packed 16-bit values.
+//
+// fp16 divisions do not use the IEEE fp32 sequence.  For fp16 operands e, s the quotient is never
+// closer than 2^-23 (relative) to a rounding boundary of the fp16 grid without lying exactly on
+// it (e - m s is a non-zero multiple of the product's last bit, m has 12 significant bits, s 11),
+// so any faithfully rounded fp32 quotient that is exact when e / s is representable rounds to
+// the same fp16 value as the correctly rounded one.  q1 = fma(fma(-q0, s, e), r, q0) with
+// q0 = e r, r = rcp(s) (1 ulp) is such a quotient: the inner fma is exact, the correction
+// carries a relative error of 2^-23 on a term of 2 ulp.  div_fixup restores the IEEE results
+// for zero and non-finite operands.
+template <int T, bool FIXUP>
+__device__ __forceinline__ float div16(float e, float s, float r) {
+  if constexpr (T == FMSMO_F16) {
+    const float q0 = __fmul_rn(e, r);
+    const float q1 = __builtin_fmaf(__builtin_fmaf(-q0, s, e), r, q0);
+    return FIXUP ? __builtin_amdgcn_div_fixupf(q1, s, e) : q1;
+  } else {
+    return e / s;
+  }
+}
+template <int T>
+__device__ __forceinline__ float cvt16(u16 h) {
+  if constexpr (T == FMSMO_F16) return f16_to_f32(h);
+  else return bf16_to_f32(h);
+}
+template <int T>
+__device__ __forceinline__ u16 to16(float f) {
+  if constexpr (T == FMSMO_F16) return f32_to_f16(f);
+  else return f32_to_bf16(f);
+}
+
+typedef unsigned short us2 __attribute__((ext_vector_type(2)));
+typedef _Float16 hf2 __attribute__((ext_vector_type(2)));
+
+// int8 code of rint(h) for a 16-bit value h with |h| <= 511, in the low byte of each half:
+// h + 1536 lands in [1024, 2048), where the fp16 grid is the integers, so the addition itself
+// rounds to nearest-even and the low mantissa bits are the two's-complement integer.
+template <int T>
+__device__ __forceinline__ uint32_t rint_codes(u16 lo, u16 hi) {
+  if constexpr (T == FMSMO_F16) {
+    hf2 h;
+    const uint32_t packed = (uint32_t)lo | ((uint32_t)hi << 16);
+    __builtin_memcpy(&h, &packed, 4);
+    const hf2 magic = {(_Float16)1536.0f, (_Float16)1536.0f};
+    h = h + magic;
+    uint32_t r;
+    __builtin_memcpy(&r, &h, 4);
+    return r;
+  } else {
+    const uint32_t a = (uint32_t)(int)__builtin_rintf(bf16_to_f32(lo)) & 0xffu;
+    const uint32_t c = (uint32_t)(int)__builtin_rintf(bf16_to_f32(hi)) & 0xffu;
+    return a | (c << 16);
+  }
+}
+
+template <int T, int NCH, bool SMOOTH>
+__global__ __launch_bounds__(AQ_THREADS) void quant_i8_pertoken16_kernel(
+    const u16* __restrict__ x, int64_t ldx, const u16* __restrict__ smooth, int saturate,
+    int8_t* __restrict__ q, int64_t ldq, float* __restrict__ scale, int M, int K) {
+  constexpr bool FAST = T == FMSMO_F16;
+  // reciprocals of the divisors stay in registers across rows while the row is short enough
+  constexpr bool KEEP_RCP = SMOOTH && FAST && NCH <= 4;
+  __shared__ float red[2][AQ_THREADS / 64];
+  const int nchunk = K / AQ_VEC;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+
+  // divisors of this thread's columns, packed as loaded
+  v4i sm[SMOOTH ? NCH : 1];
+  float sr[KEEP_RCP ? NCH : 1][8];
+  if constexpr (SMOOTH) {
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      const int c = threadIdx.x + i * AQ_THREADS;
+      if (c < nchunk) {
+        sm[i] = *(const v4i*)(smooth + (size_t)c * AQ_VEC);
+        if constexpr (KEEP_RCP) {
+#pragma unroll
+          for (int j = 0; j < 8; ++j)
+            sr[i][j] = __builtin_amdgcn_rcpf(cvt16<T>((u16)((uint32_t)sm[i][j >> 1] >> ((j & 1) * 16))));
+        }
+      }
+    }
+  }
+
+  v4i cur[NCH], nxt[NCH];
+  auto load_row = [&](int row, v4i (&dst)[NCH]) {
+    const u16* xr = x + (size_t)row * ldx;
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      const int c = threadIdx.x + i * AQ_THREADS;
+      if (c < nchunk) dst[i] = __builtin_nontemporal_load((const v4i*)(xr + (size_t)c * AQ_VEC));
+    }
+  };
+  // cur <- rnd_T(cur / smooth), packed.  Without FIX the fp16 quotient of a zero / non-finite
+  // operand comes out NaN instead of its IEEE value; the caller detects that from the row maximum.
+  auto divide_row = [&](auto fix_tag) {
+    constexpr bool FIX = decltype(fix_tag)::value;
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      const int c = threadIdx.x + i * AQ_THREADS;
+      if (c < nchunk) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const uint32_t w = (uint32_t)cur[i][j], d = (uint32_t)sm[i][j];
+          const float lo = cvt16<T>((u16)(w & 0xffff)), hi = cvt16<T>((u16)(w >> 16));
+          const float dl = cvt16<T>((u16)(d & 0xffff)), dh = cvt16<T>((u16)(d >> 16));
+          float rl = 0.f, rh = 0.f;
+          if constexpr (KEEP_RCP) {
+            rl = sr[i][2 * j], rh = sr[i][2 * j + 1];
+          } else if constexpr (FAST) {
+            rl = __builtin_amdgcn_rcpf(dl), rh = __builtin_amdgcn_rcpf(dh);
+          }
+          const u16 el = to16<T>(div16<T, FIX>(lo, dl, rl));
+          const u16 eh = to16<T>(div16<T, FIX>(hi, dh, rh));
+          cur[i][j] = (int)((uint32_t)el | ((uint32_t)eh << 16));
+        }
+      }
+    }
+  };
+  // max |cur| over the row.  |e| is monotone in its bit pattern, so the maximum is taken on the
+  // packed 15-bit magnitudes, two per instruction (a NaN outranks inf).
+  int parity = 0;
+  auto row_amax_bits = [&]() -> uint32_t {
+    us2 amax2 = {0, 0};
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      const int c = threadIdx.x + i * AQ_THREADS;
+      if (c < nchunk) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const uint32_t mag = (uint32_t)cur[i][j] & 0x7fff7fffu;
+          us2 m2;
+          __builtin_memcpy(&m2, &mag, 4);
+          amax2 = __builtin_elementwise_max(amax2, m2);
+        }
+      }
+    }
+    // non-negative floats order like their bit patterns: reduce as floats of the raw bits
+    float v = wave_max(__uint_as_float((uint32_t)(amax2[0] > amax2[1] ? amax2[0] : amax2[1])));
+    float* rb = red[parity];
+    parity ^= 1;
+    if (lane == 0) rb[wave] = v;
+    __syncthreads();
+    v = fmaxf(fmaxf(rb[0], rb[1]), fmaxf(rb[2], rb[3]));
+    return __float_as_uint(v);
+  };
+  constexpr uint32_t INF_BITS = T == FMSMO_F16 ? 0x7c00u : 0x7f80u;
+
+  int row = blockIdx.x;
+  if (row < M) load_row(row, cur);
+  const float floor_T = cvt16<T>(to16<T>(1e-5f));
+  const float sat_hi = saturate ? 127.0f : 3.0e38f;
+  for (; row < M; row += gridDim.x) {
+    const int nrow = row + gridDim.x;
+    if (nrow < M) load_row(nrow, nxt);
+
+    if constexpr (SMOOTH) divide_row(std::false_type{});
+    uint32_t abits = row_amax_bits();
+    if constexpr (SMOOTH && FAST) {
+      if (abits >= INF_BITS) {  // zero / non-finite operands somewhere in the row: IEEE results
+        load_row(row, cur);
+        divide_row(std::true_type{});
+        abits = row_amax_bits();
+      }
+    }
+    const float amax = cvt16<T>((u16)abits);
+
+    // s = rnd_T( max(amax, rnd_T(1e-5)) / 127 ): finite and non-zero, so the quotients below
+    // need no special-case fix-up unless the row overflowed the 16-bit range (amax = inf)
+    const float s = cvt16<T>(to16<T>(div16<T, true>(fmaxf(amax, floor_T), 127.0f, 1.0f / 127.0f)));
+    const float rs = FAST ? __builtin_amdgcn_rcpf(s) : 0.0f;
+    if (threadIdx.x == 0) scale[row] = s;
+    int8_t* qr = q + (size_t)row * ldq;
+    auto emit = [&](auto fix_tag) {
+      constexpr bool FIX = decltype(fix_tag)::value;
+#pragma unroll
+      for (int i = 0; i < NCH; ++i) {
+        const int c = threadIdx.x + i * AQ_THREADS;
+        if (c < nchunk) {
+          uint32_t code[4];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const uint32_t w = (uint32_t)cur[i][j];
+            float ql = div16<T, FIX>(cvt16<T>((u16)(w & 0xffff)), s, rs);
+            float qh = div16<T, FIX>(cvt16<T>((u16)(w >> 16)), s, rs);
+            if (saturate) {  // clamp before rounding: the bounds are integers
+              ql = fminf(fmaxf(ql, -sat_hi), sat_hi);
+              qh = fminf(fmaxf(qh, -sat_hi), sat_hi);
+            }
+            code[j] = rint_codes<T>(to16<T>(ql), to16<T>(qh));
+          }
+          // bytes 0 and 2 of each code word -> 8 consecutive int8
+          const uint32_t o0 = __builtin_amdgcn_perm(code[1], code[0], 0x06040200u);
+          const uint32_t o1 = __builtin_amdgcn_perm(code[3], code[2], 0x06040200u);
+          *(uint2*)(qr + (size_t)c * AQ_VEC) = make_uint2(o0, o1);
+        }
+      }
+    };
+    if (abits < INF_BITS) emit(std::false_type{});
+    else emit(std::true_type{});
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) cur[i] = nxt[i];
   }
 }
 
@@ -231,6 +441,26 @@ int fmsmo_check_launch();
 
 static bool aligned16(const void* p) { return (((uintptr_t)p) & 15) == 0; }
 
+// Blocks of AQ_THREADS threads the current device keeps resident for a row-walking kernel (its
+// grid size); asked of the runtime once per kernel and device.
+static int64_t resident_blocks(const void* kernel) {
+  struct Entry { const void* k; int dev; int64_t n; };
+  static thread_local Entry cache[64];
+  static thread_local int used = 0;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) dev = 0;
+  for (int i = 0; i < used; ++i)
+    if (cache[i].k == kernel && cache[i].dev == dev) return cache[i].n;
+  int per_cu = 0, cus = 0;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, AQ_THREADS, 0) != hipSuccess || per_cu < 1)
+    per_cu = 2;
+  if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1)
+    cus = 256;
+  const int64_t n = (int64_t)per_cu * cus;
+  if (used < 64) cache[used++] = Entry{kernel, dev, n};
+  return n;
+}
+
 extern "C" int fmsmo_quant_act_i8_pertoken(const void* x, int x_dtype, int64_t ldx,
                                            const void* smooth, int smooth_dtype,
                                            int compute_dtype, int saturate, int8_t* q, int64_t ldq,
@@ -241,8 +471,36 @@ extern "C" int fmsmo_quant_act_i8_pertoken(const void* x, int x_dtype, int64_t l
   if (x_dtype < 0 || x_dtype > 2 || compute_dtype < 0 || compute_dtype > 2) return FMSMO_ERR_UNSUPPORTED;
   if (smooth && (smooth_dtype < 0 || smooth_dtype > 2)) return FMSMO_ERR_UNSUPPORTED;
   if (K % 8 || ldx % 8 || ldq % 8 || !aligned16(x) || (((uintptr_t)q) & 7)) return FMSMO_ERR_ALIGN;
+  if (smooth && !aligned16(smooth)) return FMSMO_ERR_ALIGN;
   if (M == 0) return FMSMO_OK;
   hipStream_t st = (hipStream_t)stream;
+  // 16-bit fast path: x, the divisor and the compute dtype all fp16 (or all bf16), row cached in
+  // registers (K <= 16384)
+  if (x_dtype != FMSMO_F32 && compute_dtype == x_dtype && (!smooth || smooth_dtype == x_dtype) &&
+      K <= AQ_MAXCHUNK * AQ_THREADS * AQ_VEC) {
+    const int64_t per_thread = div_up(K, AQ_THREADS * AQ_VEC);
+    const int nch = per_thread <= 1 ? 1 : per_thread <= 2 ? 2 : per_thread <= 4 ? 4 : 8;
+    dim3 block16(AQ_THREADS);
+#define LAUNCH16(T, NCH, SM)                                                                     \
+  {                                                                                              \
+    const int64_t resident = resident_blocks((const void*)quant_i8_pertoken16_kernel<T, NCH, SM>); \
+    dim3 grid16((unsigned)(M < resident ? M : resident));                                        \
+    hipLaunchKernelGGL((quant_i8_pertoken16_kernel<T, NCH, SM>), grid16, block16, 0, st,         \
+                       (const u16*)x, ldx, (const u16*)smooth, saturate, q, ldq, scale, (int)M,  \
+                       (int)K);                                                                  \
+  }
+#define PICK16(T)                                                                     \
+  switch (nch * 2 + (smooth ? 1 : 0)) {                                               \
+    case 2: LAUNCH16(T, 1, false); break;  case 3: LAUNCH16(T, 1, true); break;      \
+    case 4: LAUNCH16(T, 2, false); break;  case 5: LAUNCH16(T, 2, true); break;      \
+    case 8: LAUNCH16(T, 4, false); break;  case 9: LAUNCH16(T, 4, true); break;      \
+    case 16: LAUNCH16(T, 8, false); break; default: LAUNCH16(T, 8, true); break;     \
+  }
+    if (x_dtype == FMSMO_F16) { PICK16(FMSMO_F16) } else { PICK16(FMSMO_BF16) }
+#undef PICK16
+#undef LAUNCH16
+    return fmsmo_check_launch();
+  }
   dim3 grid((unsigned)M), block(AQ_THREADS);
 #define LAUNCH(XT, T)                                                                          \
   hipLaunchKernelGGL((quant_i8_pertoken_kernel<XT, T>), grid, block, 0, st, x, ldx, smooth,    \

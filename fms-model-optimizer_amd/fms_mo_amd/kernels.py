@@ -69,6 +69,8 @@ def quant_act_i8_pertoken(x, smooth=None, compute_dtype=None, saturate=False):
         smooth = smooth.detach().reshape(-1).contiguous()
         if smooth.numel() != K:
             raise ValueError("smooth scale must have K elements")
+        if smooth.data_ptr() % 16:
+            smooth = smooth.clone()
     if compute_dtype is None:
         compute_dtype = x.dtype if smooth is None else torch.promote_types(x.dtype, smooth.dtype)
     q = torch.empty((M, K), dtype=torch.int8, device=x.device)

@@ -73,6 +73,8 @@ const char* fmsmo_last_error(void);
  * saturate = 0 reproduces the reference: no clamp, 128 wraps to -128 on the int8 cast (reachable
  * only for T = bf16); saturate = 1 clamps to [-127,127].
  * scale[m] receives s_m as fp32 (exactly representable).
+ * x and smooth 16-byte aligned, K and ldx multiples of 8 elements.  Rows holding NaN are not
+ * specified (the reference's int8 cast of NaN is platform-defined).
  * Reference: QLinearINT8Deploy.qa_dynamic_max_qfunc (fms_mo/modules/linear.py:1085-1100), the
  * divide in QLinearINT8Deploy.forward (:1331-1334), QMaxDynamic.forward
  * (fms_mo/quant/quantizers.py:3531-3534).

@@ -67,6 +67,42 @@ def test_quant_act_i8_smoothquant(dev, sdtype):
     assert torch.equal(q.cpu(), q_ref)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(4133, 64), (2500, 4096), (530, 14336)])
+def test_quant_act_i8_rows_walked_by_one_block(dev, dtype, shape):
+    """More rows than resident blocks (each block quantizes several rows, prefetching the next),
+    16-bit SmoothQuant divisors with a narrow range so that every x / smooth rounding shows in q."""
+    M, Kd = shape
+    g = gen(11)
+    x = ((torch.rand(M, Kd, generator=g) + 0.5) * torch.sign(torch.randn(M, Kd, generator=g))).to(dtype)
+    x = _special_rows(x)
+    smooth = (torch.rand(Kd, generator=g) * 1.5 + 0.5).to(dtype)
+    for sm in (None, smooth):
+        q_ref, s_ref, _ = O.quant_act_pertoken_i8(x, None if sm is None else sm.reshape(1, -1))
+        q, s = K().quant_act_i8_pertoken(x.to(dev), None if sm is None else sm.to(dev))
+        assert torch.equal(s.cpu(), s_ref.float().reshape(-1))
+        assert torch.equal(q.cpu(), q_ref)
+
+
+def test_quant_act_i8_fp16_division_ties_and_subnormals(dev):
+    """Every finite fp16 bit pattern as x against divisors that make exact ties (powers of two on
+    subnormal quotients), tiny and huge quotients: x / smooth must round like torch's fp16
+    division.  One column per row group keeps the per-row scale from hiding the quotient."""
+    bits = torch.arange(0, 1 << 16, dtype=torch.int32)
+    vals = bits.to(torch.int16).view(torch.float16)
+    vals = vals[torch.isfinite(vals)]                       # 63488 values
+    Kd = 64
+    vals = vals[: vals.numel() // Kd * Kd].reshape(-1, Kd)  # [992, 64], similar magnitudes per row
+    for sval in (2.0, 4.0, 0.5, 3.0, 0.3330078125, 1.0009765625, 1.9990234375, 6.103515625e-05, 1024.0):
+        smooth = torch.full((Kd,), sval, dtype=torch.float16)
+        q_ref, s_ref, _ = O.quant_act_pertoken_i8(vals, smooth.reshape(1, -1))
+        q, s = K().quant_act_i8_pertoken(vals.to(dev), smooth.to(dev))
+        assert torch.equal(s.cpu(), s_ref.float().reshape(-1)), sval
+        ok = torch.isfinite(s_ref.float().reshape(-1))   # rows that overflowed hold inf / inf = nan
+        assert torch.equal(q.cpu()[ok], q_ref[ok]), sval
+        assert torch.equal(q.cpu()[~ok] == 0, q_ref[~ok] == 0), sval   # finite / inf = 0 there
+
+
 def test_quant_act_i8_static(dev):
     x = (torch.randn(37, 1024, generator=gen(5)) * 4).half()
     for scale, zp, sym in [(0.0627, 128, 1), (0.031, 117, 0), (0.05, 128, 0)]:

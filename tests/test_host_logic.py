@@ -226,3 +226,33 @@ def test_fp8_linear_construction_and_offline_quantization():
     assert "FP8Linear(in=64, out=32" in repr(f)
     with pytest.raises(RuntimeError, match="no CPU path"):
         f(torch.zeros(2, 64, dtype=torch.bfloat16))
+
+
+def test_fp16_quotient_from_reciprocal_rounds_like_ieee_division():
+    """The act-quant kernel forms fp16 quotients as q1 = fma(fma(-q0, s, e), r, q0), q0 = e r, with
+    r a 1-ulp reciprocal, and rounds q1 to fp16.  Check against correctly rounded division over
+    every pair of fp16 significands (normal results) and over subnormal results, with the
+    reciprocal perturbed by -1, 0, +1 ulp."""
+    import numpy as np
+
+    def f32(a):
+        return a.astype(np.float32)
+
+    def fma32(a, b, c):  # products of a 24-bit and an 11/24-bit number are exact in float64
+        return f32(a.astype(np.float64) * b.astype(np.float64) + c.astype(np.float64))
+
+    sig = (1024 + np.arange(1024)).astype(np.float32)
+    e, s = np.meshgrid(sig, sig, indexing="ij")
+    e, s = e.ravel(), s.ravel()
+    cases = [(e, s), (e * np.float32(2.0 ** -24), s * np.float32(2.0 ** -9)),   # quotients ~2^-15: subnormal
+             (e * np.float32(2.0 ** -20), s * np.float32(2.0 ** -6)),           # ~2^-14 boundary
+             (e * np.float32(2.0 ** -10), s)]                                   # ~2^-10..2^-9
+    for e, s in cases:
+        exact = (e.astype(np.float64) / s.astype(np.float64)).astype(np.float16)
+        r0 = f32(np.float64(1.0) / s.astype(np.float64))
+        for ulps in (-1, 0, 1):
+            r = (r0.view(np.int32) + ulps).view(np.float32)
+            q0 = f32(e.astype(np.float64) * r.astype(np.float64))
+            q1 = fma32(fma32(-q0, s, e), r, q0)
+            got = q1.astype(np.float16)
+            assert np.array_equal(got.view(np.uint16), exact.view(np.uint16)), ulps
