@@ -57,13 +57,14 @@ int check_gemm(const void* a, int64_t lda, const void* b, int64_t ldb, const voi
 struct TileBig { static constexpr int BM = 256, BN = 256, BK = 64, NST = 4, WGM = 2, WGN = 2; };
 struct TileWide { static constexpr int BM = 128, BN = 256, BK = 64, NST = 4, WGM = 2, WGN = 2; };
 struct TileMid { static constexpr int BM = 128, BN = 128, BK = 64, NST = 4, WGM = 2, WGN = 2; };
+struct TileBig192 { static constexpr int BM = 256, BN = 192, BK = 64, NST = 4, WGM = 2, WGN = 2; };
 
 // Pick the tile shape by (relative kernel efficiency) x (fill of the last round of tiles over
 // the 256 compute units).  The efficiencies are measured loop efficiencies of the three shapes
 // (bigger tiles move fewer bytes per MFMA); 128x128 tiles fit two blocks per CU.
 int pick_tile(int M, int N) {
   static const char* force = getenv("FMSMO_TILE");  // tuning aid: 0 = 256x256, 1 = 128x256, 2 = 128x128
-  if (force && force[0] >= '0' && force[0] <= '2') return force[0] - '0';
+  if (force && force[0] >= '0' && force[0] <= '3') return force[0] - '0';
   // Fitted to measurements on the Llama / Granite shapes: relative loop efficiency of the three
   // tile shapes, and a sub-linear penalty for a partially filled last round (idle CUs leave
   // power, hence clock, to the busy ones).
@@ -130,6 +131,7 @@ void launch_any(const GemmArgs& g, const Epi& epi, hipStream_t st) {
     switch (pick_tile(g.M, g.N)) {
       case 0: launch_tile<TileBig, OP, false>(g, epi, st); break;
       case 1: launch_tile<TileWide, OP, false>(g, epi, st); break;
+      case 3: launch_tile<TileBig192, OP, false>(g, epi, st); break;
       default: launch_tile<TileMid, OP, false>(g, epi, st); break;
     }
   } else {

@@ -128,7 +128,18 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(GemmArgs g, Ep
   if (blockIdx.x == 0 && tid == 0 && g.clk) { g.clk[0] = clock64(); g.clk[1] = wall_clock64(); }
 #endif
   int tile_m, tile_n;
-  tile_of_block(blockIdx.x, gridDim.x, g.grid_m, g.grid_n, g.group_m, tile_m, tile_n);
+  if constexpr (GROUPED) {
+    // The launch grid is an upper bound (the host cannot see the expert sizes).  Count the real
+    // row tiles and map only the first real_tiles block ids, so that every XCD gets an equal
+    // share of real work; the surplus blocks are the last to be dispatched and exit at once.
+    int real_m = 0;
+    for (int e = 0; e < g.num_experts; ++e) real_m += (g.offsets[e + 1] - g.offsets[e] + BM - 1) / BM;
+    const int real_tiles = real_m * g.grid_n;
+    if ((int)blockIdx.x >= real_tiles) return;  // uniform for the whole block
+    tile_of_block(blockIdx.x, real_tiles, real_m, g.grid_n, g.group_m, tile_m, tile_n);
+  } else {
+    tile_of_block(blockIdx.x, gridDim.x, g.grid_m, g.grid_n, g.group_m, tile_m, tile_n);
+  }
 
 #ifdef FMSMO_ABLATE_SAME_TILE
   tile_m = FMSMO_ABLATE_SAME_TILE == 1 ? 0 : (blockIdx.x & 7) / 4 + 2 * ((blockIdx.x >> 3) & 1);
@@ -138,7 +149,6 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(GemmArgs g, Ep
   int row_lo = 0, row_hi = g.M, expert = 0;
   if constexpr (GROUPED) {
     int t = tile_m;
-    bool found = false;
     for (int e = 0; e < g.num_experts; ++e) {
       const int lo = g.offsets[e], hi = g.offsets[e + 1];
       const int nt = (hi - lo + BM - 1) / BM;
@@ -146,12 +156,10 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(GemmArgs g, Ep
         row_lo = lo + t * BM;
         row_hi = hi;
         expert = e;
-        found = true;
         break;
       }
       t -= nt;
     }
-    if (!found) return;  // uniform for the whole block
   } else {
     row_lo = tile_m * BM;
   }
@@ -256,10 +264,10 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(GemmArgs g, Ep
   // path takes ~16 cycles per 1 KiB wave instruction and is shared by the whole CU, so bursts
   // of DMA issue would stall the in-order wave and starve the MFMA pipe).
   constexpr int NRD = (FM + FN) * CL, NMMA = FM * FN, NLD = NIA + NIB;
-  constexpr int LDP = NLD / NKS;  // DMA instructions issued per k-step
-  static_assert(NLD % NKS == 0, "DMA instructions must split evenly over the k-steps");
+  // DMA instructions [NLD * S / NKS, NLD * (S + 1) / NKS) are issued during k-step S
   static_assert(NSTAGE >= 3, "pipeline needs at least three LDS stages");
-  auto interleave = [&]() {
+  auto interleave = [&](auto ldp_c) {
+    constexpr int LDP = decltype(ldp_c)::value;  // DMA instructions issued in this k-step
     constexpr int PER = (NMMA / 2) / NRD > 0 ? (NMMA / 2) / NRD : 1;
 #pragma unroll
     for (int r = 0; r < NRD; ++r) {
@@ -299,8 +307,8 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(GemmArgs g, Ep
 #ifdef FMSMO_ABLATE_NO_DMA
       if (g.K < 0)
 #endif
-      issue_part(fill, fill_k0, std::integral_constant<int, S * LDP>{},
-                 std::integral_constant<int, (S + 1) * LDP>{});
+      issue_part(fill, fill_k0, std::integral_constant<int, NLD * S / NKS>{},
+                 std::integral_constant<int, NLD * (S + 1) / NKS>{});
     };
     [&]<int... S>(std::integer_sequence<int, S...>) {
       (
@@ -308,7 +316,7 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(GemmArgs g, Ep
             read_frags(ls, S + 1, fa[(PAR + S + 1) & 1], fb[(PAR + S + 1) & 1]);
             dma(std::integral_constant<int, S>{});
             mma_step(fa[(PAR + S) & 1], fb[(PAR + S) & 1]);
-            interleave();
+            interleave(std::integral_constant<int, NLD * (S + 1) / NKS - NLD * S / NKS>{});
           }(),
           ...);
     }(std::make_integer_sequence<int, NKS - 1>{});
@@ -316,13 +324,13 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(GemmArgs g, Ep
     // stage kt+1 has landed (younger DMA may stay in flight) and until its own LDS reads of
     // stage kt have returned, then barrier: stage kt+1 is now complete for all waves and buffer
     // `cur` may be refilled during the next stage.
-    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"((NSTAGE - 3) * NLD + (NKS - 1) * LDP)
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"((NSTAGE - 3) * NLD + NLD * (NKS - 1) / NKS)
                  : "memory");
     const int nxt = (kt + 1) % NSTAGE;
     read_frags(&lds[0][0] + nxt * STAGE_BYTES, 0, fa[(PAR + NKS) & 1], fb[(PAR + NKS) & 1]);
     dma(std::integral_constant<int, NKS - 1>{});
     mma_step(fa[(PAR + NKS - 1) & 1], fb[(PAR + NKS - 1) & 1]);
-    interleave();
+    interleave(std::integral_constant<int, NLD - NLD * (NKS - 1) / NKS>{});
   };
 
 #pragma unroll
