@@ -6,12 +6,15 @@
 // and only then added to the running accumulator -- the same order of operations as the
 // reference's Triton kernels, whose BLOCK_SIZE_K equals the chunk size.
 //
-// Tiling: 128x128 block, 4 waves of 64x64 (2x2 MFMA 32x32 blocks each); K advances in 64-byte
+// Two kernels.  K (in bytes) a multiple of 64: the pipelined tile kernel of gemm_tile.hpp
+// (128x128 block, 4-stage DMA ring) with its chunk hook.  Any other K: the simple kernel below.
+//
+// Simple kernel tiling: 128x128 block, 4 waves of 64x64 (2x2 MFMA 32x32 blocks each); K advances in 64-byte
 // stages through two LDS buffers filled with bounds-checked 16-byte loads (zero fill past M, N
 // and K, which is what "the K tail is masked to 0" means).  One MFMA k-step is 32 bytes of K
 // for every operand type, so chunk boundaries (multiples of 32 bytes) always fall between
 // k-steps.
-#include "common.hpp"
+#include "gemm_tile.hpp"
 
 namespace fmsmo {
 
@@ -86,23 +89,6 @@ struct ChunkMma<FMSMO_OP_F32> {
     return t;
   }
 };
-
-// Chunk post-processing on one accumulator value.
-__device__ __forceinline__ int trunc_i32(int p, int lo, int hi, int round_bit, int t) {
-  p = max(min(p, hi), lo);
-  // (p + 2^(t-1)) >> t << t with two's-complement wrap on the add, arithmetic right shift
-  p = (int)((unsigned)p + (unsigned)round_bit);
-  return (int)((unsigned)(p >> t) << t);
-}
-__device__ __forceinline__ float trunc_f32(float p, unsigned round_bit, unsigned mask, int dl16) {
-  float x = __uint_as_float((__float_as_uint(p) + round_bit) & mask);
-  if (dl16) {
-    x = x >= 8581545984.0f ? __builtin_inff() : x;
-    x = x <= -8581545984.0f ? -__builtin_inff() : x;
-    x = fabsf(x) < 4.665707820095122e-10f ? 0.0f : x;
-  }
-  return x;
-}
 
 template <int OP>
 __global__ __launch_bounds__(256) void chunk_matmul_kernel(ChunkArgs g) {
@@ -248,6 +234,43 @@ __global__ __launch_bounds__(256) void chunk_matmul_kernel(ChunkArgs g) {
 using namespace fmsmo;
 int fmsmo_check_launch();
 
+// Pipelined path: the tile GEMM kernel with the chunk hook.  Needs whole 64-byte K stages and
+// 32-bit row offsets; the K tail inside the last chunk (K not a multiple of the chunk) is
+// finished after the loop like any chunk.
+template <int MMA, class Epi>
+static bool launch_chunk_tile(const ChunkArgs& c, const Epi& epi, hipStream_t st) {
+  if (c.Kb % 64 || c.chunk_bytes % 32 || (int64_t)c.M * c.lda >= (1ll << 31) ||
+      (int64_t)c.N * c.ldb >= (1ll << 31))
+    return false;
+  GemmArgs g{};
+  g.a = c.a; g.b = c.b; g.lda = c.lda; g.ldb = c.ldb;
+  g.M = c.M; g.N = c.N; g.K = c.Kb;
+  g.grid_m = div_up(c.M, 128); g.grid_n = div_up(c.N, 128); g.group_m = 8;
+  const bool fast = c.tta && !c.dl16 && c.max_acc_bits >= 32;
+  ChunkTrunc<false> k{};
+  k.chunk_ks = c.chunk_bytes / 32;
+  k.t = c.dl16 ? 14 : c.trun_bits;
+  k.round_bit = k.t > 0 ? 1u << (k.t - 1) : 0u;
+  k.mask = ~((1u << k.t) - 1u);
+  k.lo = c.max_acc_bits < 32 ? -(1 << (c.max_acc_bits - 1)) : (int)0x80000000;
+  k.hi = c.max_acc_bits < 32 ? (1 << (c.max_acc_bits - 1)) - 1 : 0x7fffffff;
+  k.post = c.dl16 || k.t > 0 || c.max_acc_bits < 32;
+  k.dl16 = c.dl16; k.tta = c.tta; k.c_in = c.c_in; k.ldc = c.ldd;
+  dim3 grid((unsigned)(g.grid_m * g.grid_n)), block(256);
+  if (fast) {
+    ChunkTrunc<true> kf{};
+    kf.chunk_ks = k.chunk_ks; kf.t = k.t; kf.round_bit = k.round_bit; kf.mask = k.mask;
+    kf.lo = k.lo; kf.hi = k.hi; kf.post = k.post; kf.dl16 = 0; kf.tta = 1;
+    kf.c_in = k.c_in; kf.ldc = k.ldc;
+    hipLaunchKernelGGL((gemm_tile_kernel<128, 128, 64, 4, 2, 2, MMA, 1, false, Epi, ChunkTrunc<true>>),
+                       grid, block, 0, st, g, epi, kf);
+  } else {
+    hipLaunchKernelGGL((gemm_tile_kernel<128, 128, 64, 4, 2, 2, MMA, 1, false, Epi, ChunkTrunc<false>>),
+                       grid, block, 0, st, g, epi, k);
+  }
+  return true;
+}
+
 static int check_chunk(const void* a, int64_t lda, const void* b, int64_t ldb, const void* d,
                        int64_t ldd, int64_t M, int64_t N, int64_t K, int64_t esz, int chunk_size,
                        int min_chunk) {
@@ -271,11 +294,16 @@ extern "C" int fmsmo_matmul_chunk_i8(const int8_t* a, int64_t lda, const int8_t*
   if (chunk_trun_bits < 0 || chunk_trun_bits > 31 || max_acc_bits < 2 || max_acc_bits > 32)
     return FMSMO_ERR_UNSUPPORTED;
   if (M == 0) return FMSMO_OK;
+  // Nothing to round or clamp: int32 addition wraps and is associative, so the chunked sum is
+  // the plain int32 GEMM.
+  if (chunk_trun_bits == 0 && max_acc_bits == 32 && !c_in)
+    return fmsmo_gemm_i8_i32(a, lda, b, ldb, d, ldd, M, N, K, stream);
   ChunkArgs g{};
   g.a = (const uint8_t*)a; g.b = (const uint8_t*)b; g.lda = lda; g.ldb = ldb;
   g.M = (int)M; g.N = (int)N; g.Kb = (int)K; g.chunk_bytes = chunk_size;
   g.trun_bits = chunk_trun_bits; g.max_acc_bits = max_acc_bits; g.dl16 = 0;
   g.tta = truncate_then_accumulate != 0; g.c_in = c_in; g.d = d; g.ldd = ldd;
+  if (launch_chunk_tile<MMA_I8>(g, EpiStoreI32{d, ldd}, (hipStream_t)stream)) return fmsmo_check_launch();
   dim3 grid(div_up(N, 128), div_up(M, 128));
   hipLaunchKernelGGL((chunk_matmul_kernel<FMSMO_OP_I8>), grid, dim3(256), 0, (hipStream_t)stream, g);
   return fmsmo_check_launch();
@@ -299,8 +327,16 @@ extern "C" int fmsmo_matmul_chunk_fp(const void* a, int64_t lda, const void* b, 
   g.M = (int)M; g.N = (int)N; g.Kb = (int)(K * esz); g.chunk_bytes = chunk_size * esz;
   g.trun_bits = chunk_trun_bits; g.max_acc_bits = 32; g.dl16 = clamp_dl16 != 0;
   g.tta = truncate_then_accumulate != 0; g.c_in = c_in; g.d = d; g.ldd = ldd;
-  dim3 grid(div_up(N, 128), div_up(M, 128));
   hipStream_t st = (hipStream_t)stream;
+  {
+    const EpiStoreF32 epi{d, ldd};
+    const bool done = op_dtype == FMSMO_OP_E4M3 ? launch_chunk_tile<MMA_FP8_K32>(g, epi, st)
+                      : op_dtype == FMSMO_OP_F16 ? launch_chunk_tile<MMA_F16>(g, epi, st)
+                      : op_dtype == FMSMO_OP_BF16 ? launch_chunk_tile<MMA_BF16>(g, epi, st)
+                                                  : launch_chunk_tile<MMA_F32>(g, epi, st);
+    if (done) return fmsmo_check_launch();
+  }
+  dim3 grid(div_up(N, 128), div_up(M, 128));
   if (op_dtype == FMSMO_OP_E4M3)
     hipLaunchKernelGGL((chunk_matmul_kernel<FMSMO_OP_E4M3>), grid, dim3(256), 0, st, g);
   else if (op_dtype == FMSMO_OP_F16)

@@ -94,7 +94,7 @@ void launch_tile(const GemmArgs& g0, const Epi& epi, hipStream_t st) {
   hipLaunchKernelGGL(
       (gemm_tile_kernel<Tile::BM, Tile::BN, Tile::BK, Tile::NST, Tile::WGM, Tile::WGN, OP, 1,
                         GROUPED, Epi>),
-      grid, block, 0, st, g, epi);
+      grid, block, 0, st, g, epi, NoChunk{});
 }
 
 // Generic fallback (any K % 16 == 0): one thread per output element, 4-byte dot products.

@@ -23,7 +23,7 @@
 
 namespace fmsmo {
 
-enum { MMA_I8 = 0, MMA_FP8 = 1 };
+enum { MMA_I8 = 0, MMA_FP8 = 1, MMA_FP8_K32 = 2, MMA_F16 = 3, MMA_BF16 = 4, MMA_F32 = 5 };
 
 struct GemmArgs {
   const uint8_t* a;
@@ -80,6 +80,99 @@ struct Mma<MMA_FP8> {
   }
 };
 
+// 32-byte k-steps for the chunked-accumulation kernels (chunk boundaries are multiples of 32
+// bytes of K for every operand type): two legacy K=16 e4m3 MFMAs, one K=16 f16 / bf16 MFMA, four
+// K=2 fp32 MFMAs per 16-byte lane operand.
+template <>
+struct Mma<MMA_FP8_K32> {
+  typedef v4i Frag;
+  typedef v16f Acc;
+  typedef float Elem;
+  static constexpr int KSTEP = 32;
+  __device__ static __forceinline__ Acc mma(const Frag& a, const Frag& b, const Acc& c) {
+    const long a0 = ((long)(unsigned)a[1] << 32) | (unsigned)a[0];
+    const long a1 = ((long)(unsigned)a[3] << 32) | (unsigned)a[2];
+    const long b0 = ((long)(unsigned)b[1] << 32) | (unsigned)b[0];
+    const long b1 = ((long)(unsigned)b[3] << 32) | (unsigned)b[2];
+    Acc t = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(a0, b0, c, 0, 0, 0);
+    return __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(a1, b1, t, 0, 0, 0);
+  }
+};
+template <>
+struct Mma<MMA_F16> {
+  typedef v4i Frag;
+  typedef v16f Acc;
+  typedef float Elem;
+  static constexpr int KSTEP = 32;
+  typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+  __device__ static __forceinline__ Acc mma(const Frag& a, const Frag& b, const Acc& c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, a),
+                                                  __builtin_bit_cast(v8h, b), c, 0, 0, 0);
+  }
+};
+template <>
+struct Mma<MMA_BF16> {
+  typedef v4i Frag;
+  typedef v16f Acc;
+  typedef float Elem;
+  static constexpr int KSTEP = 32;
+  typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+  __device__ static __forceinline__ Acc mma(const Frag& a, const Frag& b, const Acc& c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, a),
+                                                   __builtin_bit_cast(v8bf, b), c, 0, 0, 0);
+  }
+};
+template <>
+struct Mma<MMA_F32> {
+  typedef v4i Frag;
+  typedef v16f Acc;
+  typedef float Elem;
+  static constexpr int KSTEP = 32;
+  __device__ static __forceinline__ Acc mma(const Frag& a, const Frag& b, const Acc& c) {
+    Acc t = c;
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      t = __builtin_amdgcn_mfma_f32_32x32x2f32(__int_as_float(a[e]), __int_as_float(b[e]), t, 0, 0, 0);
+    return t;
+  }
+};
+
+// ---- chunked accumulation: every `chunk_ks` MFMA k-steps the partial product is range-clamped /
+// LSB-rounded and folded into the running accumulator (or the running accumulator itself is
+// rounded when tta == 0).
+struct NoChunk {
+  static constexpr bool enabled = false;
+  static constexpr bool fast = false;
+};
+// FAST = the common configuration (truncate-then-accumulate, no integer clamp, no DL16 clamp):
+// three vector ALU operations per accumulator element and chunk.
+template <bool FAST>
+struct ChunkTrunc {
+  static constexpr bool enabled = true;
+  static constexpr bool fast = FAST;
+  int chunk_ks;           // MFMA k-steps (32 bytes of K) per chunk
+  int t, lo, hi;          // LSBs to round away; integer clamp range
+  unsigned round_bit, mask;
+  int post, dl16, tta;
+  const void* c_in;       // optional initial accumulator [M, N], same element type as the output
+  int64_t ldc;
+};
+__device__ __forceinline__ int trunc_i32(int p, int lo, int hi, int round_bit, int t) {
+  p = max(min(p, hi), lo);
+  // (p + 2^(t-1)) >> t << t with two's-complement wrap on the add, arithmetic right shift
+  p = (int)((unsigned)p + (unsigned)round_bit);
+  return (int)((unsigned)(p >> t) << t);
+}
+__device__ __forceinline__ float trunc_f32(float p, unsigned round_bit, unsigned mask, int dl16) {
+  float x = __uint_as_float((__float_as_uint(p) + round_bit) & mask);
+  if (dl16) {
+    x = x >= 8581545984.0f ? __builtin_inff() : x;
+    x = x <= -8581545984.0f ? -__builtin_inff() : x;
+    x = fabsf(x) < 4.665707820095122e-10f ? 0.0f : x;
+  }
+  return x;
+}
+
 // Map the hardware block id to a tile.  Work-groups are dealt round-robin to the 8 XCDs (each
 // with a private L2), so block b runs on XCD b % 8; give every XCD one contiguous span of the
 // tile sequence, and order that sequence in column-major groups of `group_m` tile rows so the
@@ -99,8 +192,8 @@ __device__ __forceinline__ void tile_of_block(int bid, int nblk, int grid_m, int
 }
 
 template <int BM, int BN, int BK, int NSTAGE, int WGM, int WGN, int OP, int SWZ, bool GROUPED,
-          class Epi>
-__global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(GemmArgs g, Epi epi) {
+          class Epi, class Chk = NoChunk>
+__global__ __launch_bounds__(WGM* WGN * 64, (Chk::enabled && (OP == MMA_I8 || Chk::fast)) ? 2 : 1) void gemm_tile_kernel(GemmArgs g, Epi epi, Chk chk) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stub
   typedef Mma<OP> MM;
   typedef typename MM::Frag Frag;
@@ -224,6 +317,85 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(GemmArgs g, Ep
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
 
+  // chunked accumulation: MFMAs run into `work`, finished chunks are folded into `acc`
+  typedef typename MM::Elem Elem;
+  Acc work[Chk::enabled ? FM : 1][Chk::enabled ? FN : 1];
+  int ks_cnt = 0;
+  if constexpr (Chk::enabled) {
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+      for (int j = 0; j < FN; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          Elem init = 0;
+          if (chk.c_in) {
+            const int m = row_lo + wm * TM + i * 32 + (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3);
+            const int n = col_lo + wn * TN + j * 32 + (lane & 31);
+            if (m < row_hi && n < g.N) init = ((const Elem*)chk.c_in)[(int64_t)m * chk.ldc + n];
+          }
+          acc[i][j][v] = chk.tta ? init : (Elem)0;
+          work[i][j][v] = chk.tta ? (Elem)0 : init;
+        }
+  }
+  auto finish_chunk = [&](auto post_c, auto tta_c) __attribute__((always_inline)) {
+    constexpr bool POST = decltype(post_c)::value, TTA = decltype(tta_c)::value;
+    if constexpr (Chk::enabled) {
+#pragma unroll
+      for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) {
+            Elem p = work[i][j][v];
+            if constexpr (POST) {
+              if constexpr (std::is_same<Elem, int>::value) p = trunc_i32(p, chk.lo, chk.hi, (int)chk.round_bit, chk.t);
+              else p = trunc_f32(p, chk.round_bit, chk.mask, chk.dl16);
+            }
+            if constexpr (TTA) {
+              if constexpr (std::is_same<Elem, int>::value) acc[i][j][v] = (int)((unsigned)acc[i][j][v] + (unsigned)p);
+              else acc[i][j][v] += p;
+              work[i][j][v] = 0;
+            } else {
+              work[i][j][v] = p;  // the running accumulator itself is rounded
+            }
+          }
+    }
+  };
+  auto finish_any = [&]() __attribute__((always_inline)) {
+    if constexpr (Chk::fast) {
+#pragma unroll
+      for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) {
+            // (p + 2^(t-1)) with the low t bits cleared: same bits for two's-complement integers
+            // ((p + r) >> t << t) and for fp32 patterns; work is overwritten by the next chunk
+            if constexpr (std::is_same<Elem, int>::value) {
+              acc[i][j][v] = (int)((unsigned)acc[i][j][v] + (((unsigned)work[i][j][v] + chk.round_bit) & chk.mask));
+            } else {
+              acc[i][j][v] += __uint_as_float((__float_as_uint(work[i][j][v]) + chk.round_bit) & chk.mask);
+            }
+          }
+    } else if constexpr (Chk::enabled) {
+      if (chk.tta) {
+        if (chk.post) finish_chunk(std::true_type{}, std::true_type{});
+        else finish_chunk(std::false_type{}, std::true_type{});
+      } else if (chk.post) {
+        finish_chunk(std::true_type{}, std::false_type{});
+      }
+    }
+  };
+  auto chunk_tick = [&]() __attribute__((always_inline)) {
+    if constexpr (Chk::enabled) {
+      if (++ks_cnt == chk.chunk_ks) {
+        finish_any();
+        ks_cnt = 0;
+      }
+    }
+  };
+
   auto read_frags = [&](const uint8_t* ls, int s, Frag* af, Frag* bf) {
 #ifdef FMSMO_ABLATE_NO_LDSREAD
     if (g.K > 0) return;
@@ -256,7 +428,29 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(GemmArgs g, Ep
 #pragma unroll
     for (int i = 0; i < FM; ++i)
 #pragma unroll
-      for (int j = 0; j < FN; ++j) acc[i][j] = MM::mma(af[i], bf[j], acc[i][j]);
+      for (int j = 0; j < FN; ++j) {
+        if constexpr (Chk::enabled) work[i][j] = MM::mma(af[i], bf[j], work[i][j]);
+        else acc[i][j] = MM::mma(af[i], bf[j], acc[i][j]);
+      }
+  };
+  // first k-step of a chunk in FAST mode: the MFMA's C operand is the constant 0, so `work` needs
+  // no clearing between chunks
+  auto mma_step_fresh = [&](const Frag* af, const Frag* bf) {
+    Acc zero;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) zero[v] = 0;
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+      for (int j = 0; j < FN; ++j) work[i][j] = MM::mma(af[i], bf[j], zero);
+  };
+  auto mma_any = [&](const Frag* af, const Frag* bf) __attribute__((always_inline)) {
+    if constexpr (Chk::fast) {
+      if (ks_cnt == 0) mma_step_fresh(af, bf);
+      else mma_step(af, bf);
+    } else {
+      mma_step(af, bf);
+    }
   };
   // Instruction-order hints (DS read = 0x100, MFMA = 0x008, VMEM = 0x020): the operand reads of
   // the next k-step go between the first MFMAs of the current one, so their latency is covered
@@ -315,8 +509,9 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(GemmArgs g, Ep
           [&] {
             read_frags(ls, S + 1, fa[(PAR + S + 1) & 1], fb[(PAR + S + 1) & 1]);
             dma(std::integral_constant<int, S>{});
-            mma_step(fa[(PAR + S) & 1], fb[(PAR + S) & 1]);
+            mma_any(fa[(PAR + S) & 1], fb[(PAR + S) & 1]);
             interleave(std::integral_constant<int, NLD * (S + 1) / NKS - NLD * S / NKS>{});
+            chunk_tick();
           }(),
           ...);
     }(std::make_integer_sequence<int, NKS - 1>{});
@@ -329,8 +524,9 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(GemmArgs g, Ep
     const int nxt = (kt + 1) % NSTAGE;
     read_frags(&lds[0][0] + nxt * STAGE_BYTES, 0, fa[(PAR + NKS) & 1], fb[(PAR + NKS) & 1]);
     dma(std::integral_constant<int, NKS - 1>{});
-    mma_step(fa[(PAR + NKS - 1) & 1], fb[(PAR + NKS - 1) & 1]);
+    mma_any(fa[(PAR + NKS - 1) & 1], fb[(PAR + NKS - 1) & 1]);
     interleave(std::integral_constant<int, NLD - NLD * (NKS - 1) / NKS>{});
+    chunk_tick();
   };
 
 #pragma unroll
@@ -352,6 +548,15 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_tile_kernel(GemmArgs g, Ep
     }
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no DMA may be in flight when LDS is released
+  if constexpr (Chk::enabled) {
+    if (ks_cnt != 0) finish_any();  // K ended inside a chunk
+    if (!chk.tta) {
+#pragma unroll
+      for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j) acc[i][j] = work[i][j];
+    }
+  }
 
 #ifdef FMSMO_CLK
   if (blockIdx.x == 0 && tid == 0 && g.clk) { g.clk[2] = clock64(); g.clk[3] = wall_clock64(); }
@@ -408,6 +613,18 @@ struct EpiStoreI32 {
   __device__ __forceinline__ Col col(int, int, int) const { return Col{}; }
   __device__ __forceinline__ Row row(int) const { return Row{}; }
   __device__ __forceinline__ void store(int m, int n, int v, Row, Col) const {
+    c[(int64_t)m * ldc + n] = v;
+  }
+};
+
+struct EpiStoreF32 {
+  float* c;
+  int64_t ldc;
+  struct Col {};
+  struct Row {};
+  __device__ __forceinline__ Col col(int, int, int) const { return Col{}; }
+  __device__ __forceinline__ Row row(int) const { return Row{}; }
+  __device__ __forceinline__ void store(int m, int n, float v, Row, Col) const {
     c[(int64_t)m * ldc + n] = v;
   }
 };
