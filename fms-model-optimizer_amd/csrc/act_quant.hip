@@ -336,6 +336,153 @@ __global__ __launch_bounds__(AQ_THREADS) void quant_i8_pertoken16_kernel(
   }
 }
 
+// ------------------------------------------------------------------ int8, dynamic per token,
+// fp16 x with an fp32 SmoothQuant scale: torch promotes x / smooth to fp32 and the whole
+// quantizer then runs in fp32.
+//
+// Same row-walking structure as the 16-bit kernel.  Divisions use the correctly rounded fp32
+// sequence without its range-scaling steps: r1 = rcp(s) refined once, q0 = x r1, two residual
+// corrections q <- fma(fma(-s, q, x), r1, q).  That is the IEEE result whenever no intermediate
+// leaves the normal range, which holds for fp16 x (6e-8 .. 65504) and 2^-60 <= |s| <= 2^60;
+// a block that sees a divisor outside that range, or a row whose maximum is not finite, takes
+// the plain IEEE division instead.  Quotients by the row scale only feed rint(); where they
+// underflow they are far below 0.5.
+__device__ __forceinline__ float rcp_refined(float s) {
+  const float r0 = __builtin_amdgcn_rcpf(s);
+  return __builtin_fmaf(__builtin_fmaf(-s, r0, 1.0f), r0, r0);
+}
+__device__ __forceinline__ float div32_fast(float x, float s, float r1) {
+  float q = __fmul_rn(x, r1);
+  q = __builtin_fmaf(__builtin_fmaf(-s, q, x), r1, q);
+  q = __builtin_fmaf(__builtin_fmaf(-s, q, x), r1, q);
+  return q;
+}
+
+template <int NCH, bool KEEP>
+__global__ __launch_bounds__(AQ_THREADS) void quant_i8_pertoken_f16x_f32s_kernel(
+    const u16* __restrict__ x, int64_t ldx, const float* __restrict__ smooth, int saturate,
+    int8_t* __restrict__ q, int64_t ldq, float* __restrict__ scale, int M, int K) {
+  __shared__ float red[2][AQ_THREADS / 64];
+  const int nchunk = K / AQ_VEC;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+
+  // divisors (and refined reciprocals) of this thread's columns; kept across rows for short rows,
+  // re-read from L2 per row otherwise
+  float sv[KEEP ? NCH : 1][8], sr[KEEP ? NCH : 1][8];
+  int bad = 0;
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) {
+    const int c = threadIdx.x + i * AQ_THREADS;
+    if (c < nchunk) {
+      const float4 a = *(const float4*)(smooth + (size_t)c * AQ_VEC);
+      const float4 b = *(const float4*)(smooth + (size_t)c * AQ_VEC + 4);
+      const float d[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float m = fabsf(d[j]);
+        bad |= !(m >= 8.6736174e-19f && m <= 1.1529215e18f);  // outside 2^-60 .. 2^60, or NaN
+        if constexpr (KEEP) {
+          sv[i][j] = d[j];
+          sr[i][j] = rcp_refined(d[j]);
+        }
+      }
+    }
+  }
+  const bool ieee_block = __syncthreads_or(bad) != 0;
+
+  v4i cur[NCH], nxt[NCH];
+  float e[NCH][8];
+  auto load_row = [&](int row, v4i (&dst)[NCH]) {
+    const u16* xr = x + (size_t)row * ldx;
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      const int c = threadIdx.x + i * AQ_THREADS;
+      if (c < nchunk) dst[i] = __builtin_nontemporal_load((const v4i*)(xr + (size_t)c * AQ_VEC));
+    }
+  };
+  // e <- x / smooth (fp32); returns the thread's max |e|
+  auto divide_row = [&](auto ieee_tag) -> float {
+    constexpr bool IEEE = decltype(ieee_tag)::value;
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      const int c = threadIdx.x + i * AQ_THREADS;
+      if (c < nchunk) {
+        float d[8];
+        if constexpr (!KEEP || IEEE) {
+          const float4 a = *(const float4*)(smooth + (size_t)c * AQ_VEC);
+          const float4 b = *(const float4*)(smooth + (size_t)c * AQ_VEC + 4);
+          d[0] = a.x; d[1] = a.y; d[2] = a.z; d[3] = a.w; d[4] = b.x; d[5] = b.y; d[6] = b.z; d[7] = b.w;
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const float xv = f16_to_f32((u16)((uint32_t)cur[i][j >> 1] >> ((j & 1) * 16)));
+          if constexpr (IEEE) e[i][j] = xv / d[j];
+          else if constexpr (KEEP) e[i][j] = div32_fast(xv, sv[i][j], sr[i][j]);
+          else e[i][j] = div32_fast(xv, d[j], rcp_refined(d[j]));
+          amax = fmaxf(amax, fabsf(e[i][j]));
+        }
+      }
+    }
+    return amax;
+  };
+  int parity = 0;
+  auto block_amax = [&](float v) -> float {
+    // NaN must survive the reduction (it selects the IEEE path): compare bit patterns of |v|
+    uint32_t b = __float_as_uint(v) & 0x7fffffffu;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) b = max(b, (uint32_t)__shfl_xor((int)b, o, 64));
+    float* rb = red[parity];
+    parity ^= 1;
+    if (lane == 0) rb[wave] = __uint_as_float(b);
+    __syncthreads();
+    const uint32_t r = max(max(__float_as_uint(rb[0]), __float_as_uint(rb[1])),
+                           max(__float_as_uint(rb[2]), __float_as_uint(rb[3])));
+    return __uint_as_float(r);
+  };
+
+  int row = blockIdx.x;
+  if (row < M) load_row(row, cur);
+  for (; row < M; row += gridDim.x) {
+    const int nrow = row + gridDim.x;
+    if (nrow < M) load_row(nrow, nxt);
+
+    float amax;
+    bool ieee = ieee_block;
+    if (!ieee) {
+      amax = block_amax(divide_row(std::false_type{}));
+      ieee = !(amax < __builtin_inff());  // inf or NaN somewhere in the row
+    }
+    if (ieee) {
+      // fmaxf drops NaN like the generic kernel does
+      float v = divide_row(std::true_type{});
+      amax = block_amax(v);
+    }
+    const float s = fmaxf(amax, 1e-5f) / 127.0f;
+    const float rs = rcp_refined(s);
+    if (threadIdx.x == 0) scale[row] = s;
+    int8_t* qr = q + (size_t)row * ldq;
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      const int c = threadIdx.x + i * AQ_THREADS;
+      if (c < nchunk) {
+        uint32_t o[2] = {0, 0};
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          float r = __builtin_rintf(ieee ? e[i][j] / s : div32_fast(e[i][j], s, rs));
+          if (saturate) r = fminf(fmaxf(r, -127.0f), 127.0f);
+          // |r| <= 128 in every finite row: r + 1.5 * 2^23 holds the two's-complement integer in
+          // its low mantissa bits
+          o[j >> 2] |= (__float_as_uint(r + 12582912.0f) & 0xffu) << ((j & 3) * 8);
+        }
+        *(uint2*)(qr + (size_t)c * AQ_VEC) = make_uint2(o[0], o[1]);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) cur[i] = nxt[i];
+  }
+}
+
 // ------------------------------------------------------------------ int8, static per tensor
 template <int XT>
 __global__ __launch_bounds__(AQ_THREADS) void quant_i8_static_kernel(
@@ -499,6 +646,26 @@ extern "C" int fmsmo_quant_act_i8_pertoken(const void* x, int x_dtype, int64_t l
     if (x_dtype == FMSMO_F16) { PICK16(FMSMO_F16) } else { PICK16(FMSMO_BF16) }
 #undef PICK16
 #undef LAUNCH16
+    return fmsmo_check_launch();
+  }
+  // fp16 x promoted to fp32 by an fp32 SmoothQuant scale
+  if (x_dtype == FMSMO_F16 && smooth && smooth_dtype == FMSMO_F32 && compute_dtype == FMSMO_F32 &&
+      K <= AQ_MAXCHUNK * AQ_THREADS * AQ_VEC) {
+    const int64_t per_thread = div_up(K, AQ_THREADS * AQ_VEC);
+    dim3 block32(AQ_THREADS);
+#define LAUNCH32(NCH, KEEP)                                                                       \
+  {                                                                                               \
+    const int64_t resident = resident_blocks((const void*)quant_i8_pertoken_f16x_f32s_kernel<NCH, KEEP>); \
+    dim3 grid32((unsigned)(M < resident ? M : resident));                                         \
+    hipLaunchKernelGGL((quant_i8_pertoken_f16x_f32s_kernel<NCH, KEEP>), grid32, block32, 0, st,   \
+                       (const u16*)x, ldx, (const float*)smooth, saturate, q, ldq, scale, (int)M, \
+                       (int)K);                                                                   \
+  }
+    if (per_thread <= 1) LAUNCH32(1, true)
+    else if (per_thread <= 2) LAUNCH32(2, true)
+    else if (per_thread <= 4) LAUNCH32(4, false)
+    else LAUNCH32(8, false)
+#undef LAUNCH32
     return fmsmo_check_launch();
   }
   dim3 grid((unsigned)M), block(AQ_THREADS);

@@ -84,6 +84,30 @@ def test_quant_act_i8_rows_walked_by_one_block(dev, dtype, shape):
         assert torch.equal(q.cpu(), q_ref)
 
 
+@pytest.mark.parametrize("shape", [(4133, 64), (2500, 4096), (300, 6144), (530, 14336)])
+def test_quant_act_i8_fp16_x_fp32_smooth_rows(dev, shape):
+    """fp16 x with an fp32 SmoothQuant scale: torch promotes to fp32, the quantizer runs in fp32
+    (the reference's example flow keeps quantizer buffers fp32).  Includes divisors outside the
+    fast path's range (block-wide IEEE fallback) and rows that overflow to inf."""
+    M, Kd = shape
+    g = gen(12)
+    x = ((torch.rand(M, Kd, generator=g) * 3 + 0.01) * torch.sign(torch.randn(M, Kd, generator=g))).half()
+    x = _special_rows(x)
+    x[5, 3] = 65504.0
+    base = torch.rand(Kd, generator=g) * 1.5 + 0.5
+    for variant in ("plain", "tiny_divisor", "huge_divisor"):
+        smooth = base.clone()
+        if variant == "tiny_divisor":
+            smooth[7] = 1e-30      # x / 1e-30 stays finite in fp32 only for small x; outside 2^-60
+        if variant == "huge_divisor":
+            smooth[9] = 3e30
+        q_ref, s_ref, _ = O.quant_act_pertoken_i8(x, smooth.reshape(1, -1))
+        q, s = K().quant_act_i8_pertoken(x.to(dev), smooth.to(dev))
+        ok = torch.isfinite(s_ref.float().reshape(-1))
+        assert torch.equal(s.cpu()[ok], s_ref.float().reshape(-1)[ok]), variant
+        assert torch.equal(q.cpu()[ok], q_ref[ok]), variant
+
+
 def test_quant_act_i8_fp16_division_ties_and_subnormals(dev):
     """Every finite fp16 bit pattern as x against divisors that make exact ties (powers of two on
     subnormal quotients), tiny and huge quotients: x / smooth must round like torch's fp16

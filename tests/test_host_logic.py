@@ -256,3 +256,46 @@ def test_fp16_quotient_from_reciprocal_rounds_like_ieee_division():
             q1 = fma32(fma32(-q0, s, e), r, q0)
             got = q1.astype(np.float16)
             assert np.array_equal(got.view(np.uint16), exact.view(np.uint16)), ulps
+
+
+def test_fp32_quotient_by_two_residual_corrections_is_correctly_rounded():
+    """The fp32-compute act-quant kernel divides as q0 = x r1, q <- fma(fma(-s, q, x), r1, q) twice,
+    r1 = one Newton step on a 1-ulp reciprocal.  Emulated with exact rational arithmetic (every
+    fma rounded once) and compared with the correctly rounded quotient, for fp16-valued x and
+    random fp32 divisors, the hardware reciprocal modelled as the exact one moved by -1/0/+1 ulp."""
+    import random
+    from fractions import Fraction
+
+    import numpy as np
+
+    def rn32(fr):  # round a Fraction to the nearest fp32, ties to even (normal range only)
+        if fr == 0:
+            return Fraction(0)
+        sign = -1 if fr < 0 else 1
+        a = abs(fr)
+        e = a.numerator.bit_length() - a.denominator.bit_length()
+        if Fraction(2) ** e > a:
+            e -= 1
+        ulp = Fraction(2) ** (e - 23)
+        n = a / ulp
+        f = n.numerator // n.denominator
+        rem = n - f
+        if rem > Fraction(1, 2) or (rem == Fraction(1, 2) and f % 2 == 1):
+            f += 1
+        return sign * f * ulp
+
+    def fma(a, b, c):
+        return rn32(a * b + c)
+
+    rnd = random.Random(7)
+    for trial in range(4000):
+        xv = Fraction(float(np.float16(rnd.choice([-1, 1]) * rnd.uniform(0.001, 60000.0))))
+        sv = Fraction(float(np.float32(rnd.uniform(0.3, 3.0) * 2.0 ** rnd.randint(-20, 20))))
+        for ulps in (-1, 0, 1):
+            r0 = rn32(1 / sv)
+            r0 = r0 + ulps * Fraction(2) ** (int(np.floor(np.log2(float(r0)))) - 23)
+            r1 = fma(fma(-sv, r0, Fraction(1)), r0, r0)
+            q = rn32(xv * r1)
+            q = fma(fma(-sv, q, xv), r1, q)
+            q = fma(fma(-sv, q, xv), r1, q)
+            assert q == rn32(xv / sv), (float(xv), float(sv), ulps)
