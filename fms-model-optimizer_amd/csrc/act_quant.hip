@@ -139,16 +139,18 @@ __global__ __launch_bounds__(AQ_THREADS) void quant_i8_pertoken_kernel(
 // so any faithfully rounded fp32 quotient that is exact when e / s is representable rounds to
 // the same fp16 value as the correctly rounded one.  q1 = fma(fma(-q0, s, e), r, q0) with
 // q0 = e r, r = rcp(s) (1 ulp) is such a quotient: the inner fma is exact, the correction
-// carries a relative error of 2^-23 on a term of 2 ulp.  div_fixup restores the IEEE results
-// for zero and non-finite operands.
-template <int T, bool FIXUP>
+// carries a relative error of 2^-23 on a term of 2 ulp.  The same holds for bf16 (boundaries at
+// least 2^-17 apart from any inexact quotient) as long as nothing leaves the fp32 normal range:
+// a block whose bf16 divisors fall outside 2^-60 .. 2^60, and any row whose maximum comes out
+// inf / NaN (zero or non-finite operands, overflow), is computed with plain IEEE divisions.
+// Quotients below 2^-66 may round differently, which can change neither q nor the scale.
+template <int T, bool IEEE>
 __device__ __forceinline__ float div16(float e, float s, float r) {
-  if constexpr (T == FMSMO_F16) {
-    const float q0 = __fmul_rn(e, r);
-    const float q1 = __builtin_fmaf(__builtin_fmaf(-q0, s, e), r, q0);
-    return FIXUP ? __builtin_amdgcn_div_fixupf(q1, s, e) : q1;
-  } else {
+  if constexpr (IEEE) {
     return e / s;
+  } else {
+    const float q0 = __fmul_rn(e, r);
+    return __builtin_fmaf(__builtin_fmaf(-q0, s, e), r, q0);
   }
 }
 template <int T>
@@ -180,8 +182,9 @@ __device__ __forceinline__ uint32_t rint_codes(u16 lo, u16 hi) {
     __builtin_memcpy(&r, &h, 4);
     return r;
   } else {
-    const uint32_t a = (uint32_t)(int)__builtin_rintf(bf16_to_f32(lo)) & 0xffu;
-    const uint32_t c = (uint32_t)(int)__builtin_rintf(bf16_to_f32(hi)) & 0xffu;
+    // same trick in fp32: r + 1.5 * 2^23 (|r| <= 511 is far inside its range)
+    const uint32_t a = __float_as_uint(bf16_to_f32(lo) + 12582912.0f) & 0xffu;
+    const uint32_t c = __float_as_uint(bf16_to_f32(hi) + 12582912.0f) & 0xffu;
     return a | (c << 16);
   }
 }
@@ -190,9 +193,8 @@ template <int T, int NCH, bool SMOOTH>
 __global__ __launch_bounds__(AQ_THREADS) void quant_i8_pertoken16_kernel(
     const u16* __restrict__ x, int64_t ldx, const u16* __restrict__ smooth, int saturate,
     int8_t* __restrict__ q, int64_t ldq, float* __restrict__ scale, int M, int K) {
-  constexpr bool FAST = T == FMSMO_F16;
   // reciprocals of the divisors stay in registers across rows while the row is short enough
-  constexpr bool KEEP_RCP = SMOOTH && FAST && NCH <= 4;
+  constexpr bool KEEP_RCP = SMOOTH && NCH <= 4;
   __shared__ float red[2][AQ_THREADS / 64];
   const int nchunk = K / AQ_VEC;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -200,19 +202,23 @@ __global__ __launch_bounds__(AQ_THREADS) void quant_i8_pertoken16_kernel(
   // divisors of this thread's columns, packed as loaded
   v4i sm[SMOOTH ? NCH : 1];
   float sr[KEEP_RCP ? NCH : 1][8];
+  bool ieee_block = false;
   if constexpr (SMOOTH) {
+    int bad = 0;
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
       const int c = threadIdx.x + i * AQ_THREADS;
       if (c < nchunk) {
         sm[i] = *(const v4i*)(smooth + (size_t)c * AQ_VEC);
-        if constexpr (KEEP_RCP) {
 #pragma unroll
-          for (int j = 0; j < 8; ++j)
-            sr[i][j] = __builtin_amdgcn_rcpf(cvt16<T>((u16)((uint32_t)sm[i][j >> 1] >> ((j & 1) * 16))));
+        for (int j = 0; j < 8; ++j) {
+          const float d = cvt16<T>((u16)((uint32_t)sm[i][j >> 1] >> ((j & 1) * 16)));
+          if constexpr (T == FMSMO_BF16) bad |= !(fabsf(d) >= 8.6736174e-19f && fabsf(d) <= 1.1529215e18f);
+          if constexpr (KEEP_RCP) sr[i][j] = __builtin_amdgcn_rcpf(d);
         }
       }
     }
+    if constexpr (T == FMSMO_BF16) ieee_block = __syncthreads_or(bad) != 0;
   }
 
   v4i cur[NCH], nxt[NCH];
@@ -224,8 +230,9 @@ __global__ __launch_bounds__(AQ_THREADS) void quant_i8_pertoken16_kernel(
       if (c < nchunk) dst[i] = __builtin_nontemporal_load((const v4i*)(xr + (size_t)c * AQ_VEC));
     }
   };
-  // cur <- rnd_T(cur / smooth), packed.  Without FIX the fp16 quotient of a zero / non-finite
-  // operand comes out NaN instead of its IEEE value; the caller detects that from the row maximum.
+  // cur <- rnd_T(cur / smooth), packed.  FIX = plain IEEE divisions.  Without it the quotient of a
+  // zero / non-finite operand comes out NaN instead of its IEEE value; the caller detects that
+  // from the row maximum.
   auto divide_row = [&](auto fix_tag) {
     constexpr bool FIX = decltype(fix_tag)::value;
 #pragma unroll
@@ -238,9 +245,10 @@ __global__ __launch_bounds__(AQ_THREADS) void quant_i8_pertoken16_kernel(
           const float lo = cvt16<T>((u16)(w & 0xffff)), hi = cvt16<T>((u16)(w >> 16));
           const float dl = cvt16<T>((u16)(d & 0xffff)), dh = cvt16<T>((u16)(d >> 16));
           float rl = 0.f, rh = 0.f;
-          if constexpr (KEEP_RCP) {
+          if constexpr (FIX) {
+          } else if constexpr (KEEP_RCP) {
             rl = sr[i][2 * j], rh = sr[i][2 * j + 1];
-          } else if constexpr (FAST) {
+          } else {
             rl = __builtin_amdgcn_rcpf(dl), rh = __builtin_amdgcn_rcpf(dh);
           }
           const u16 el = to16<T>(div16<T, FIX>(lo, dl, rl));
@@ -287,10 +295,13 @@ __global__ __launch_bounds__(AQ_THREADS) void quant_i8_pertoken16_kernel(
     const int nrow = row + gridDim.x;
     if (nrow < M) load_row(nrow, nxt);
 
-    if constexpr (SMOOTH) divide_row(std::false_type{});
+    if constexpr (SMOOTH) {
+      if (ieee_block) divide_row(std::true_type{});
+      else divide_row(std::false_type{});
+    }
     uint32_t abits = row_amax_bits();
-    if constexpr (SMOOTH && FAST) {
-      if (abits >= INF_BITS) {  // zero / non-finite operands somewhere in the row: IEEE results
+    if constexpr (SMOOTH) {
+      if (abits >= INF_BITS && !ieee_block) {  // zero / non-finite operands or overflow in the row
         load_row(row, cur);
         divide_row(std::true_type{});
         abits = row_amax_bits();
@@ -300,8 +311,8 @@ __global__ __launch_bounds__(AQ_THREADS) void quant_i8_pertoken16_kernel(
 
     // s = rnd_T( max(amax, rnd_T(1e-5)) / 127 ): finite and non-zero, so the quotients below
     // need no special-case fix-up unless the row overflowed the 16-bit range (amax = inf)
-    const float s = cvt16<T>(to16<T>(div16<T, true>(fmaxf(amax, floor_T), 127.0f, 1.0f / 127.0f)));
-    const float rs = FAST ? __builtin_amdgcn_rcpf(s) : 0.0f;
+    const float s = cvt16<T>(to16<T>(fmaxf(amax, floor_T) / 127.0f));
+    const float rs = __builtin_amdgcn_rcpf(s);
     if (threadIdx.x == 0) scale[row] = s;
     int8_t* qr = q + (size_t)row * ldq;
     auto emit = [&](auto fix_tag) {

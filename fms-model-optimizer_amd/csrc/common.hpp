@@ -38,10 +38,10 @@ __device__ __forceinline__ u16 f32_to_f16(float f) {
 }
 __device__ __forceinline__ float bf16_to_f32(u16 h) { return __uint_as_float(((uint32_t)h) << 16); }
 __device__ __forceinline__ u16 f32_to_bf16(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (u16)((u >> 16) | 0x40);  // quiet NaN
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return (u16)(u >> 16);
+  __bf16 v = (__bf16)f;  // v_cvt_pk_bf16_f32: RNE, NaN stays NaN
+  u16 h;
+  __builtin_memcpy(&h, &v, 2);
+  return h;
 }
 
 // Round a float to the value grid of dtype T (T in FMSMO_F16/BF16/F32) and come back to f32.

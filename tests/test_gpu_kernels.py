@@ -84,6 +84,24 @@ def test_quant_act_i8_rows_walked_by_one_block(dev, dtype, shape):
         assert torch.equal(q.cpu(), q_ref)
 
 
+def test_quant_act_i8_bf16_division_all_patterns(dev):
+    """Every finite bf16 bit pattern of moderate magnitude as x against bf16 divisors that make
+    exact ties and inexact neighbours; plus divisors outside the fast path's range."""
+    bits = torch.arange(0, 1 << 16, dtype=torch.int32)
+    vals = bits.to(torch.int16).view(torch.bfloat16)
+    keep = torch.isfinite(vals) & (vals.float().abs() < 1e30) & ((vals.float().abs() > 1e-30) | (vals == 0))
+    vals = vals[keep]
+    Kd = 64
+    vals = vals[: vals.numel() // Kd * Kd].reshape(-1, Kd)
+    for sval in (2.0, 0.5, 3.0, 0.33203125, 1.0078125, 1.9921875, 1e-25, 1e25):
+        smooth = torch.full((Kd,), sval, dtype=torch.bfloat16)
+        q_ref, s_ref, _ = O.quant_act_pertoken_i8(vals, smooth.reshape(1, -1))
+        q, s = K().quant_act_i8_pertoken(vals.to(dev), smooth.to(dev))
+        ok = torch.isfinite(s_ref.float().reshape(-1))
+        assert torch.equal(s.cpu()[ok], s_ref.float().reshape(-1)[ok]), sval
+        assert torch.equal(q.cpu()[ok], q_ref[ok]), sval
+
+
 @pytest.mark.parametrize("shape", [(4133, 64), (2500, 4096), (300, 6144), (530, 14336)])
 def test_quant_act_i8_fp16_x_fp32_smooth_rows(dev, shape):
     """fp16 x with an fp32 SmoothQuant scale: torch promotes to fp32, the quantizer runs in fp32

@@ -299,3 +299,26 @@ def test_fp32_quotient_by_two_residual_corrections_is_correctly_rounded():
             q = fma(fma(-sv, q, xv), r1, q)
             q = fma(fma(-sv, q, xv), r1, q)
             assert q == rn32(xv / sv), (float(xv), float(sv), ulps)
+
+
+def test_bf16_quotient_from_reciprocal_rounds_like_ieee_division():
+    """Same construction for bf16 operands (8-bit significands): all 128 x 128 pairs, reciprocal
+    off by -1/0/+1 ulp, result rounded to bf16 (RNE on the upper 16 bits of the fp32 pattern)."""
+    import numpy as np
+
+    def to_bf16_bits(a32):
+        u = a32.view(np.uint32).astype(np.uint64)
+        return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+
+    sig = (128 + np.arange(128)).astype(np.float32)
+    e, s = np.meshgrid(sig, sig, indexing="ij")
+    e, s = e.ravel(), s.ravel()
+    for e_, s_ in [(e, s), (e * np.float32(2.0 ** -7), s), (e, s * np.float32(2.0 ** 5))]:
+        exact = to_bf16_bits((e_.astype(np.float64) / s_.astype(np.float64)).astype(np.float32))
+        r0 = (np.float64(1.0) / s_.astype(np.float64)).astype(np.float32)
+        for ulps in (-1, 0, 1):
+            r = (r0.view(np.int32) + ulps).view(np.float32)
+            q0 = (e_.astype(np.float64) * r.astype(np.float64)).astype(np.float32)
+            t = (-q0.astype(np.float64) * s_.astype(np.float64) + e_.astype(np.float64)).astype(np.float32)
+            q1 = (t.astype(np.float64) * r.astype(np.float64) + q0.astype(np.float64)).astype(np.float32)
+            assert np.array_equal(to_bf16_bits(q1), exact), ulps
