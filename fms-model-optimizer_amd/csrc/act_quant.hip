@@ -590,6 +590,118 @@ __global__ __launch_bounds__(AQ_THREADS) void quant_fp8_pertoken_kernel(
   }
 }
 
+// ------------------------------------------------------------------ e4m3, per token, 16-bit x
+// Row-walking variant of the kernel above (dynamic scale, fp16 / bf16 x, K <= 16384): next row
+// prefetched, packed abs-max, divisions from a refined reciprocal (fp32 quotients for the
+// FP8Linear recipe, 16-bit-rounded quotients for the FPx recipe, see div32_fast / div16), and the
+// hardware OCP e4m3 conversion on values clamped to +-448 (torch maps (448, 464] to 448 and
+// finite rows cannot exceed that).  Rows whose maximum is inf / NaN take the IEEE + software
+// encoder route of the generic kernel.
+template <int XT, int NCH>
+__global__ __launch_bounds__(AQ_THREADS) void quant_fp8_pertoken16_kernel(
+    const u16* __restrict__ x, int64_t ldx, int variant, uint8_t* __restrict__ q, int64_t ldq,
+    float* __restrict__ scale, int M, int K) {
+  __shared__ float red[2][AQ_THREADS / 64];
+  const int nchunk = K / AQ_VEC;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  constexpr uint32_t INF_BITS = XT == FMSMO_F16 ? 0x7c00u : 0x7f80u;
+
+  v4i cur[NCH], nxt[NCH];
+  auto load_row = [&](int row, v4i (&dst)[NCH]) {
+    const u16* xr = x + (size_t)row * ldx;
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      const int c = threadIdx.x + i * AQ_THREADS;
+      if (c < nchunk) dst[i] = __builtin_nontemporal_load((const v4i*)(xr + (size_t)c * AQ_VEC));
+    }
+  };
+  int parity = 0;
+  int row = blockIdx.x;
+  if (row < M) load_row(row, cur);
+  const float floor_X = cvt16<XT>(to16<XT>(1e-5f));
+  for (; row < M; row += gridDim.x) {
+    const int nrow = row + gridDim.x;
+    if (nrow < M) load_row(nrow, nxt);
+
+    us2 amax2 = {0, 0};
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      const int c = threadIdx.x + i * AQ_THREADS;
+      if (c < nchunk) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const uint32_t mag = (uint32_t)cur[i][j] & 0x7fff7fffu;
+          us2 m2;
+          __builtin_memcpy(&m2, &mag, 4);
+          amax2 = __builtin_elementwise_max(amax2, m2);
+        }
+      }
+    }
+    float v = wave_max(__uint_as_float((uint32_t)(amax2[0] > amax2[1] ? amax2[0] : amax2[1])));
+    float* rb = red[parity];
+    parity ^= 1;
+    if (lane == 0) rb[wave] = v;
+    __syncthreads();
+    const uint32_t abits = __float_as_uint(fmaxf(fmaxf(rb[0], rb[1]), fmaxf(rb[2], rb[3])));
+    const float amax = cvt16<XT>((u16)abits);
+
+    float s;
+    if (variant == FMSMO_FP8_LINEAR) s = fmaxf(amax / 448.0f, 1e-12f);
+    else s = fmaxf(cvt16<XT>(to16<XT>(amax / 448.0f)), floor_X);
+    if (threadIdx.x == 0) scale[row] = s;
+    uint8_t* qr = q + (size_t)row * ldq;
+
+    if (abits < INF_BITS) {
+      const float r1 = rcp_refined(s);
+      const bool dl8 = variant == FMSMO_FP8_FPXACC_DL8;
+#pragma unroll
+      for (int i = 0; i < NCH; ++i) {
+        const int c = threadIdx.x + i * AQ_THREADS;
+        if (c < nchunk) {
+          float t[8];
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            const float xv = cvt16<XT>((u16)((uint32_t)cur[i][j >> 1] >> ((j & 1) * 16)));
+            if (variant == FMSMO_FP8_LINEAR) t[j] = div32_fast(xv, s, r1);
+            else t[j] = cvt16<XT>(to16<XT>(div16<XT, false>(xv, s, r1)));
+            // the residual corrections lose the sign of a zero quotient; s > 0
+            t[j] = __builtin_copysignf(fminf(fmaxf(t[j], -448.0f), 448.0f), xv);
+            // DL8: the codes 1..4 (|t| up to the tie 4.5 * 2^-9, which rounds to code 4) flush to +0
+            if (dl8) t[j] = fabsf(t[j]) <= 0.0087890625f ? 0.0f : t[j];
+          }
+          int o0 = 0, o1 = 0;
+          o0 = __builtin_amdgcn_cvt_pk_fp8_f32(t[0], t[1], o0, false);
+          o0 = __builtin_amdgcn_cvt_pk_fp8_f32(t[2], t[3], o0, true);
+          o1 = __builtin_amdgcn_cvt_pk_fp8_f32(t[4], t[5], o1, false);
+          o1 = __builtin_amdgcn_cvt_pk_fp8_f32(t[6], t[7], o1, true);
+          *(uint2*)(qr + (size_t)c * AQ_VEC) = make_uint2((uint32_t)o0, (uint32_t)o1);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < NCH; ++i) {
+        const int c = threadIdx.x + i * AQ_THREADS;
+        if (c < nchunk) {
+          uint8_t b[8];
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            const float xv = cvt16<XT>((u16)((uint32_t)cur[i][j >> 1] >> ((j & 1) * 16)));
+            float t;
+            if (variant == FMSMO_FP8_LINEAR) t = fminf(fmaxf(xv / s, -448.0f), 448.0f);
+            else t = round_to<XT>(xv / s);
+            uint8_t code = f32_to_e4m3_sw(t);
+            if (variant == FMSMO_FP8_FPXACC_DL8 && (code & 0x7f) <= 0x04) code = 0x00;
+            b[j] = code;
+          }
+          store8(qr, (size_t)c * AQ_VEC, b);
+        }
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) cur[i] = nxt[i];
+  }
+}
+
 }  // namespace fmsmo
 
 using namespace fmsmo;
@@ -731,6 +843,26 @@ extern "C" int fmsmo_quant_act_fp8_pertoken(const void* x, int x_dtype, int64_t 
   if (K % 8 || ldx % 8 || ldq % 8 || !aligned16(x) || (((uintptr_t)q) & 7)) return FMSMO_ERR_ALIGN;
   if (M == 0) return FMSMO_OK;
   hipStream_t st = (hipStream_t)stream;
+  if (x_dtype != FMSMO_F32 && !static_scale && K <= AQ_MAXCHUNK * AQ_THREADS * AQ_VEC) {
+    const int64_t per_thread = div_up(K, AQ_THREADS * AQ_VEC);
+    dim3 block16(AQ_THREADS);
+#define LAUNCH8(XT, NCH)                                                                          \
+  {                                                                                               \
+    const int64_t resident = resident_blocks((const void*)quant_fp8_pertoken16_kernel<XT, NCH>);  \
+    dim3 grid16((unsigned)(M < resident ? M : resident));                                         \
+    hipLaunchKernelGGL((quant_fp8_pertoken16_kernel<XT, NCH>), grid16, block16, 0, st,            \
+                       (const u16*)x, ldx, variant, q, ldq, scale, (int)M, (int)K);               \
+  }
+#define PICK8(XT)                                  \
+  if (per_thread <= 1) LAUNCH8(XT, 1)              \
+  else if (per_thread <= 2) LAUNCH8(XT, 2)         \
+  else if (per_thread <= 4) LAUNCH8(XT, 4)         \
+  else LAUNCH8(XT, 8)
+    if (x_dtype == FMSMO_F16) { PICK8(FMSMO_F16) } else { PICK8(FMSMO_BF16) }
+#undef PICK8
+#undef LAUNCH8
+    return fmsmo_check_launch();
+  }
   dim3 grid((unsigned)M), block(AQ_THREADS);
 #define LAUNCH(XT)                                                                             \
   hipLaunchKernelGGL((quant_fp8_pertoken_kernel<XT>), grid, block, 0, st, x, ldx, variant,     \

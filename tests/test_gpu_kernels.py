@@ -173,6 +173,44 @@ def test_fp8_cast_all_codes_and_midpoints(dev):
     assert torch.equal(q.cpu().view(torch.uint8), ref.view(torch.uint8))
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_quant_act_fp8_dynamic_all_codes_midpoints_and_many_rows(dev, dtype):
+    """Dynamic per-token path on 16-bit inputs: a row whose maximum is 448 (scale exactly 1) holding
+    every e4m3 value, every midpoint and the 16-bit neighbours of the midpoints; more rows than
+    resident blocks; rows with inf."""
+    from fms_mo_amd import _lib as L
+
+    codes = torch.arange(256, dtype=torch.uint8).view(torch.float8_e4m3fn).float()
+    vals = torch.unique(codes[~codes.isnan()])
+    mids = ((vals[:-1] + vals[1:]) / 2).to(dtype)
+    up = torch.nextafter(mids, torch.full_like(mids, 1e4)).float()
+    dn = torch.nextafter(mids, torch.full_like(mids, -1e4)).float()
+    t = torch.cat([vals, mids.float(), up, dn, torch.tensor([0.0, -0.0, 2.0**-10, 2.0**-9, 1e-7])])
+    t = t[t.abs() <= 448.0]
+    n = (t.numel() + 7) // 8 * 8
+    row = torch.zeros(n)
+    row[: t.numel()] = t
+    g = gen(31)
+    x = (torch.randn(2600, n, generator=g) * 3)
+    x[0] = row
+    x[1] = row * 0.5
+    x[2] = row * 3.0
+    x[7, 5] = float("inf")
+    x = x.to(dtype)
+    s_ref = O.fp8_dynamic_scale(x)
+    q_ref = O.fp8_quant_static(x, s_ref)
+    q, s = K().quant_act_fp8_pertoken(x.to(dev), L.FP8_LINEAR)
+    ok = torch.isfinite(s_ref.reshape(-1))
+    assert torch.equal(s.cpu()[ok], s_ref.reshape(-1)[ok])
+    assert torch.equal(q.cpu().view(torch.uint8)[ok], q_ref.view(torch.uint8)[ok])
+    for dl8 in (False, True):
+        q_ref, s_ref = O.fp8_quant_fpxacc(x, per_tensor=False, dl8=dl8)
+        q, s = K().quant_act_fp8_pertoken(x.to(dev), L.FP8_FPXACC_DL8 if dl8 else L.FP8_FPXACC)
+        ok = torch.isfinite(s_ref.float().reshape(-1))
+        assert torch.equal(s.cpu()[ok], s_ref.float().reshape(-1)[ok])
+        assert torch.equal(q.cpu().view(torch.uint8)[ok], q_ref.view(torch.uint8)[ok])
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 def test_quant_act_fp8_linear(dev, dtype):
     from fms_mo_amd import _lib as L
