@@ -249,6 +249,125 @@ __global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(GemvArgs g, int G)
   do_group(std::true_type{}, gcount - 1);
 }
 
+// Row-streaming variant for M <= 2: no MFMA, no LDS.  A wave owns whole weight rows and reads
+// each as one contiguous run (lane l takes the 16-byte chunks l, l + 64, ...: every wave load is
+// 1 KiB of consecutive bytes, the access pattern HBM serves best), multiplies with the
+// activation chunks it keeps in registers (v_dot4_i32_i8, exact; e4m3 is widened to fp32 and
+// accumulated with FMAs), and reduces the 64 partial sums with a butterfly.  U rows are in
+// flight per wave; rows are dealt to waves so that neighbouring waves read neighbouring rows.
+// KCH = ceil(K / 1024) chunks per lane; chunks past K are zero.
+template <int OP, int MR, int KCH, int U>
+__global__ __launch_bounds__(256) void gemv_rows_kernel(GemvArgs g) {
+  typedef typename std::conditional<OP == FMSMO_OP_I8, int, float>::type AccT;
+  const int lane = threadIdx.x & 63;
+  const int wave_g = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int nwaves = gridDim.x * 4;
+  const int kchunks = g.K >> 4;
+
+  v4i xr[MR][KCH];
+#pragma unroll
+  for (int m = 0; m < MR; ++m) {
+    const uint8_t* xp = g.a + (int64_t)min(m, g.M - 1) * g.lda;
+#pragma unroll
+    for (int c = 0; c < KCH; ++c) {
+      const int ch = c * 64 + lane;
+      xr[m][c] = ch < kchunks ? *(const v4i*)(xp + (int64_t)ch * 16) : v4i{0, 0, 0, 0};
+    }
+  }
+
+  for (int n0 = wave_g * U; n0 < g.N; n0 += nwaves * U) {
+    v4i w[U][KCH];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const uint8_t* wp = g.b + (int64_t)min(n0 + u, g.N - 1) * g.ldb;
+#pragma unroll
+      for (int c = 0; c < KCH; ++c) {
+        const int ch = c * 64 + lane;
+        // chunks past K: re-read the row's first chunk; the zero activation chunk cancels it
+        w[u][c] = __builtin_nontemporal_load((const v4i*)(wp + (int64_t)(ch < kchunks ? ch : lane % kchunks) * 16));
+      }
+    }
+    AccT acc[U][MR];
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int m = 0; m < MR; ++m) {
+        AccT a = 0;
+#pragma unroll
+        for (int c = 0; c < KCH; ++c) {
+#pragma unroll
+          for (int d = 0; d < 4; ++d) {
+            if constexpr (OP == FMSMO_OP_I8) {
+              a = __builtin_amdgcn_sdot4(w[u][c][d], xr[m][c][d], a, false);
+            } else {
+              const auto w0 = __builtin_amdgcn_cvt_pk_f32_fp8(w[u][c][d], false);
+              const auto w1 = __builtin_amdgcn_cvt_pk_f32_fp8(w[u][c][d], true);
+              const auto x0 = __builtin_amdgcn_cvt_pk_f32_fp8(xr[m][c][d], false);
+              const auto x1 = __builtin_amdgcn_cvt_pk_f32_fp8(xr[m][c][d], true);
+              a = __builtin_fmaf(w0[0], x0[0], a);
+              a = __builtin_fmaf(w0[1], x0[1], a);
+              a = __builtin_fmaf(w1[0], x1[0], a);
+              a = __builtin_fmaf(w1[1], x1[1], a);
+            }
+          }
+        }
+        acc[u][m] = a;
+      }
+    // Transposing butterfly over the V = U * MR partial sums of a lane: each exchange halves the
+    // number of values a lane still carries (the upper half of the lanes keeps the upper half of
+    // the values), so V - 1 + log2(64 / V) exchanges replace 6 V.  Lane l ends with the total of
+    // value index idx(l) (same in the 64 / V lanes that share its upper bits).
+    constexpr int V = U * MR;
+    AccT vals[V];
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int m = 0; m < MR; ++m) vals[u * MR + m] = acc[u][m];
+    int idx = 0;
+    {
+      int width = 32;
+#pragma unroll
+      for (int nv = V; nv > 1; nv >>= 1, width >>= 1) {
+        const int half = nv >> 1;
+        const bool upper = (lane & width) != 0;
+#pragma unroll
+        for (int i = 0; i < half; ++i) {
+          const AccT send = upper ? vals[i] : vals[i + half];
+          const AccT keep = upper ? vals[i + half] : vals[i];
+          vals[i] = keep + __shfl_xor(send, width, 64);
+        }
+        idx += upper ? half : 0;
+      }
+#pragma unroll
+      for (; width > 0; width >>= 1) vals[0] += __shfl_xor(vals[0], width, 64);
+    }
+    const AccT sum = vals[0];
+    const int eu = idx / MR, em = idx % MR;
+    constexpr int SHARE = 64 / V;  // lanes holding the same total; the first of them writes it
+    const int n = n0 + eu;
+    if ((lane & (SHARE - 1)) == 0 && n < g.N && em < g.M) {
+      const float as = g.a_scale[g.a_stride ? em : 0], ws = g.w_scale[g.w_stride ? n : 0];
+      float bv = 0.f;
+      if (g.bias) {
+        bv = g.bias_dtype == FMSMO_F16 ? f16_to_f32(((const u16*)g.bias)[n])
+             : g.bias_dtype == FMSMO_BF16 ? bf16_to_f32(((const u16*)g.bias)[n])
+                                          : ((const float*)g.bias)[n];
+      }
+      float out;
+      if (g.ref_f16) {
+        const float sc = round_to<FMSMO_F16>(__fmul_rn(as, ws));
+        out = round_to<FMSMO_F16>(__fadd_rn(__fmul_rn((float)sum, sc), bv));
+      } else {
+        out = __fmaf_rn((float)sum, __fmul_rn(as, ws), bv);
+      }
+      const int64_t idx = (int64_t)em * g.ldy + n;
+      if (g.y_dtype == FMSMO_F16) ((u16*)g.y)[idx] = f32_to_f16(out);
+      else if (g.y_dtype == FMSMO_BF16) ((u16*)g.y)[idx] = f32_to_bf16(out);
+      else ((float*)g.y)[idx] = out;
+    }
+  }
+}
+
 }  // namespace fmsmo
 
 using namespace fmsmo;
@@ -278,6 +397,44 @@ int fmsmo_gemv_dispatch(int op, const void* a, int64_t lda, const void* b, int64
   g.a_stride = a_scale_n == 1 ? 0 : 1; g.w_stride = w_scale_n == 1 ? 0 : 1;
   g.bias = bias; g.bias_dtype = bias_dtype; g.ref_f16 = epilogue == FMSMO_EPI_REF_F16;
   g.y = y; g.y_dtype = y_dtype; g.ldy = ldy;
+  // M <= 2: whole-row streaming on the vector ALUs (at M = 4 its register use halves the
+  // occupancy and the MFMA streaming kernel below is faster) (FMSMO_GEMV_KIND=1 disables it for tuning)
+  {
+    static const int env_kind = getenv("FMSMO_GEMV_KIND") ? atoi(getenv("FMSMO_GEMV_KIND")) : 0;
+    const int kch = (int)((K + 1023) / 1024);
+    const int mr = M <= 1 ? 1 : 2;
+    bool handled = env_kind != 1 && M <= 2 && K >= 1024;
+    if (handled) {
+      // 16 waves per CU resident (register use allows it), rows dealt round-robin to waves
+      const int64_t waves_needed = N;  // at U = 1
+      dim3 block(256);
+#define GEMV_ROWS(OPV, MRV, KCHV, UV)                                                        \
+  {                                                                                          \
+    const int64_t blocks = (waves_needed + 4 * UV - 1) / (4 * UV);                           \
+    dim3 grid((unsigned)(blocks < 1024 ? blocks : 1024));                                    \
+    hipLaunchKernelGGL((gemv_rows_kernel<OPV, MRV, KCHV, UV>), grid, block, 0, st, g);       \
+  }
+#define GEMV_ROWS_M(OPV, KCHV, UV)                                   \
+  if (mr == 1) GEMV_ROWS(OPV, 1, KCHV, UV)                           \
+  else GEMV_ROWS(OPV, 2, KCHV, UV)
+#define GEMV_ROWS_K(OPV)                                        \
+  switch (kch) {                                                \
+    case 1: GEMV_ROWS_M(OPV, 1, 8) break;                       \
+    case 2: GEMV_ROWS_M(OPV, 2, 8) break;                       \
+    case 4: GEMV_ROWS_M(OPV, 4, 4) break;                       \
+    case 8: GEMV_ROWS_M(OPV, 8, 2) break;                       \
+    case 13: GEMV_ROWS_M(OPV, 13, 1) break;                     \
+    case 14: GEMV_ROWS_M(OPV, 14, 1) break;                     \
+    case 16: GEMV_ROWS_M(OPV, 16, 1) break;                     \
+    default: handled = false; break;                            \
+  }
+      if (op == FMSMO_OP_I8) { GEMV_ROWS_K(FMSMO_OP_I8) } else { GEMV_ROWS_K(FMSMO_OP_E4M3) }
+#undef GEMV_ROWS_K
+#undef GEMV_ROWS_M
+#undef GEMV_ROWS
+      if (handled) return fmsmo_check_launch();
+    }
+  }
   // Streaming variant when the K steps of 128 split evenly over the waves of a block in one of
   // the instantiated (waves, steps per wave, loads in flight) shapes; other K use the generic
   // kernel below.  One block per compute unit, each walking G consecutive groups: every block
