@@ -1,0 +1,171 @@
+// Offline weight path: fp16 / bf16 / fp32 weights -> int8 rows (+ per-row integer sums).
+//
+//   t_nk = rnd_T1( W_nk * smooth_k )                      (SmoothQuant folding, optional)
+//   mode FMSMO_WQ_MUL:  q_nk = rint( clamp( rnd_T2( coef_n * t_nk ), -127, 127 ) )
+//   mode FMSMO_WQ_DIV:  q_nk = clamp( rint( rnd_T2( t_nk / coef_n ) ), -127, 127 )
+//   row_sum_n = sum_k q_nk                                 (the "zero shift" of asymmetric activations)
+//
+// T1 = promote(weight dtype, smooth dtype), T2 = promote(T1, coef dtype): the dtypes in which torch
+// evaluates the two expressions.  One 256-thread block per weight row, 16-byte loads, 8-byte
+// stores; read 2-4 B and write 1 B per element (HBM bound, offline).
+#include "common.hpp"
+
+namespace fmsmo {
+
+__device__ __forceinline__ float round_dyn(float v, int t) {
+  return t == FMSMO_F16 ? round_to<FMSMO_F16>(v) : t == FMSMO_BF16 ? round_to<FMSMO_BF16>(v) : v;
+}
+__device__ __forceinline__ float load_dyn(const void* p, int t, size_t i) {
+  return t == FMSMO_F16 ? f16_to_f32(((const u16*)p)[i])
+         : t == FMSMO_BF16 ? bf16_to_f32(((const u16*)p)[i])
+                           : ((const float*)p)[i];
+}
+
+template <int WT>
+__global__ __launch_bounds__(256) void quant_weight_i8_kernel(
+    const void* __restrict__ w, int64_t ldw, const void* __restrict__ smooth, int smooth_dtype,
+    const void* __restrict__ coef, int coef_dtype, int coef_stride, int t1, int t2, int mode,
+    int8_t* __restrict__ q, int64_t ldq, int32_t* __restrict__ row_sum, int K) {
+  __shared__ int red[4];
+  const int row = blockIdx.x;
+  const float c = load_dyn(coef, coef_dtype, coef_stride ? row : 0);
+  int sum = 0;
+  for (int k0 = threadIdx.x * 8; k0 < K; k0 += 256 * 8) {
+    float v[8];
+    if constexpr (WT == FMSMO_F32) {
+      const float4 a = *(const float4*)((const float*)w + (size_t)row * ldw + k0);
+      const float4 b = *(const float4*)((const float*)w + (size_t)row * ldw + k0 + 4);
+      v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+    } else {
+      const uint4 r = *(const uint4*)((const u16*)w + (size_t)row * ldw + k0);
+      const uint32_t ww[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const u16 h = (u16)(ww[i >> 1] >> ((i & 1) * 16));
+        v[i] = WT == FMSMO_F16 ? f16_to_f32(h) : bf16_to_f32(h);
+      }
+    }
+    uint32_t o[2] = {0, 0};
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      float t = v[i];
+      if (smooth) t = round_dyn(__fmul_rn(t, load_dyn(smooth, smooth_dtype, (size_t)k0 + i)), t1);
+      float r;
+      if (mode == FMSMO_WQ_MUL) {
+        r = __builtin_rintf(fminf(fmaxf(round_dyn(__fmul_rn(c, t), t2), -127.0f), 127.0f));
+      } else {
+        r = fminf(fmaxf(__builtin_rintf(round_dyn(t / c, t2)), -127.0f), 127.0f);
+      }
+      const int qi = (int)r;
+      sum += qi;
+      o[i >> 2] |= ((uint32_t)qi & 0xffu) << ((i & 3) * 8);
+    }
+    *(uint2*)(q + (size_t)row * ldq + k0) = make_uint2(o[0], o[1]);
+  }
+  if (row_sum) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = sum;
+    __syncthreads();
+    if (threadIdx.x == 0) row_sum[row] = red[0] + red[1] + red[2] + red[3];
+  }
+}
+
+// Per-column running abs-max:  out_k = max( out_k, max_m |x_mk| ).  A block covers 2048 columns
+// (256 threads x 8) and a slab of rows; |x| >= 0 orders like its bit pattern, so the slabs merge
+// with an unsigned atomic max on the fp32 bits.
+template <int XT>
+__global__ __launch_bounds__(256) void absmax_cols_kernel(const void* __restrict__ x, int64_t ldx,
+                                                          int M, int K, int rows_per_block,
+                                                          uint32_t* __restrict__ out) {
+  const int k0 = (blockIdx.x * 256 + threadIdx.x) * 8;
+  if (k0 >= K) return;
+  const int m0 = blockIdx.y * rows_per_block, m1 = min(M, m0 + rows_per_block);
+  float best[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  for (int m = m0; m < m1; ++m) {
+    float v[8];
+    if constexpr (XT == FMSMO_F32) {
+      const float4 a = *(const float4*)((const float*)x + (size_t)m * ldx + k0);
+      const float4 b = *(const float4*)((const float*)x + (size_t)m * ldx + k0 + 4);
+      v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+    } else {
+      const uint4 r = *(const uint4*)((const u16*)x + (size_t)m * ldx + k0);
+      const uint32_t ww[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const u16 h = (u16)(ww[i >> 1] >> ((i & 1) * 16));
+        v[i] = XT == FMSMO_F16 ? f16_to_f32(h) : bf16_to_f32(h);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) best[i] = fmaxf(best[i], fabsf(v[i]));
+  }
+#pragma unroll
+  for (int i = 0; i < 8; ++i) atomicMax(out + k0 + i, __float_as_uint(best[i]));
+}
+
+}  // namespace fmsmo
+
+using namespace fmsmo;
+int fmsmo_check_launch();
+
+static int promote(int a, int b) {
+  if (a == b) return a;
+  return FMSMO_F32;  // fp16 with bf16, or anything with fp32
+}
+
+extern "C" int fmsmo_quant_weight_i8(const void* w, int w_dtype, int64_t ldw, const void* smooth,
+                                     int smooth_dtype, const void* coef, int coef_dtype,
+                                     int64_t coef_n, int mode, int8_t* q, int64_t ldq,
+                                     int32_t* row_sum, int64_t N, int64_t K,
+                                     fmsmo_stream_t stream) {
+  if (!w || !coef || !q) return FMSMO_ERR_NULL;
+  if (N <= 0 || K <= 0 || ldw < K || ldq < K || N > 0x7fffffff || K > 0x7fffffff) return FMSMO_ERR_SHAPE;
+  if (coef_n != 1 && coef_n != N) return FMSMO_ERR_SHAPE;
+  if (w_dtype < 0 || w_dtype > 2 || coef_dtype < 0 || coef_dtype > 2 ||
+      (smooth && (smooth_dtype < 0 || smooth_dtype > 2)) || (mode != FMSMO_WQ_MUL && mode != FMSMO_WQ_DIV))
+    return FMSMO_ERR_UNSUPPORTED;
+  if (K % 8 || ldw % 8 || ldq % 8 || (((uintptr_t)w) & 15) || (((uintptr_t)q) & 7)) return FMSMO_ERR_ALIGN;
+  const int t1 = smooth ? promote(w_dtype, smooth_dtype) : w_dtype;
+  const int t2 = promote(t1, coef_dtype);
+  dim3 grid((unsigned)N), block(256);
+  hipStream_t st = (hipStream_t)stream;
+#define LAUNCH(WT)                                                                              \
+  hipLaunchKernelGGL((quant_weight_i8_kernel<WT>), grid, block, 0, st, w, ldw, smooth,          \
+                     smooth_dtype, coef, coef_dtype, coef_n == 1 ? 0 : 1, t1, t2, mode, q, ldq, \
+                     row_sum, (int)K)
+  switch (w_dtype) {
+    case FMSMO_F16: LAUNCH(FMSMO_F16); break;
+    case FMSMO_BF16: LAUNCH(FMSMO_BF16); break;
+    default: LAUNCH(FMSMO_F32); break;
+  }
+#undef LAUNCH
+  return fmsmo_check_launch();
+}
+
+extern "C" int fmsmo_absmax_cols(const void* x, int x_dtype, int64_t ldx, int64_t M, int64_t K,
+                                 float* out, fmsmo_stream_t stream) {
+  if (!x || !out) return FMSMO_ERR_NULL;
+  if (M < 0 || K <= 0 || ldx < K || M > 0x7fffffff || K > 0x7fffffff) return FMSMO_ERR_SHAPE;
+  if (x_dtype < 0 || x_dtype > 2) return FMSMO_ERR_UNSUPPORTED;
+  if (K % 8 || ldx % 8 || (((uintptr_t)x) & 15)) return FMSMO_ERR_ALIGN;
+  if (M == 0) return FMSMO_OK;
+  // enough row slabs to occupy the chip, at least 32 rows each
+  const int col_blocks = div_up(K, 2048);
+  int slabs = (int)((M + 31) / 32);
+  const int want = (2048 + col_blocks - 1) / col_blocks;
+  if (slabs > want) slabs = want;
+  const int rows_per_block = div_up(M, slabs);
+  dim3 grid(col_blocks, div_up(M, rows_per_block)), block(256);
+  hipStream_t st = (hipStream_t)stream;
+#define LAUNCH(XT)                                                                             \
+  hipLaunchKernelGGL((absmax_cols_kernel<XT>), grid, block, 0, st, x, ldx, (int)M, (int)K,     \
+                     rows_per_block, (uint32_t*)out)
+  switch (x_dtype) {
+    case FMSMO_F16: LAUNCH(FMSMO_F16); break;
+    case FMSMO_BF16: LAUNCH(FMSMO_BF16); break;
+    default: LAUNCH(FMSMO_F32); break;
+  }
+#undef LAUNCH
+  return fmsmo_check_launch();
+}

@@ -18,6 +18,7 @@ F16, BF16, F32 = 0, 1, 2
 OP_I8, OP_E4M3, OP_F16, OP_BF16, OP_F32 = 0, 1, 2, 3, 4
 EPI_REF_F16, EPI_F32 = 0, 1
 FP8_LINEAR, FP8_FPXACC, FP8_FPXACC_DL8 = 0, 1, 2
+WQ_MUL, WQ_DIV = 0, 1
 ABI_VERSION = 1
 
 _P, _I, _L, _F = c_void_p, c_int, c_int64, c_float
@@ -36,6 +37,8 @@ SIGNATURES = {
     "fmsmo_matmul_chunk_fp": [_P, _L, _P, _L, _I, _P, _P, _L, _L, _L, _L, _I, _I, _I, _I, _P],
     "fmsmo_grouped_gemm_i8_dq": [_P, _L, _P, _L, _L, _P, _I, _L, _P, _P, _P, _I, _I, _P, _I, _L,
                                  _L, _L, _P],
+    "fmsmo_quant_weight_i8": [_P, _I, _L, _P, _I, _P, _I, _L, _I, _P, _L, _P, _L, _L, _P],
+    "fmsmo_absmax_cols": [_P, _I, _L, _L, _L, _P, _P],
 }
 OTHER = {
     "fmsmo_abi_version": ([], c_int),

@@ -240,3 +240,44 @@ def matmul_chunk(a, w, c=None, chunk_size=64, chunk_trun_bits=0, max_acc_bits=32
                    int(chunk_trun_bits), int(bool(clamp_acc_to_dl16)),
                    int(bool(truncate_then_accumulate)), _stream(a))
     return d
+
+
+def quant_weight_i8(w, coef, smooth=None, mode="mul", want_row_sum=False):
+    """Offline weight quantizer (see fmsmo_quant_weight_i8): w [N,K] fp16/bf16/fp32, coef [N] or [1]
+    (``127 / clip_val`` for mode "mul", ``w_scale`` for mode "div"), smooth [K] or None.
+    Returns int8 [N,K] (and the int32 row sums [N] when asked)."""
+    _need_gpu(w, coef, smooth)
+    if w.dim() != 2:
+        raise ValueError("w must be [N, K]")
+    if w.stride(1) != 1:
+        w = w.contiguous()
+    N, K = w.shape
+    coef = coef.detach().reshape(-1).contiguous()
+    if coef.numel() not in (1, N):
+        raise ValueError("coef must have 1 or N elements")
+    if smooth is not None:
+        smooth = smooth.detach().reshape(-1).contiguous()
+        if smooth.numel() != K:
+            raise ValueError("smooth must have K elements")
+    q = torch.empty((N, K), dtype=torch.int8, device=w.device)
+    rs = torch.empty((N,), dtype=torch.int32, device=w.device) if want_row_sum else None
+    with torch.cuda.device(w.device):
+        L.call("fmsmo_quant_weight_i8", w.data_ptr(), _dt(w), _ld(w), _ptr(smooth),
+               _dt(smooth) if smooth is not None else 0, coef.data_ptr(), _dt(coef), coef.numel(),
+               L.WQ_MUL if mode == "mul" else L.WQ_DIV, q.data_ptr(), K, _ptr(rs), N, K, _stream(w))
+    return (q, rs) if want_row_sum else q
+
+
+def absmax_cols(x, running=None):
+    """Per-column abs-max of x [*, K] as fp32 [K]; with ``running`` (fp32 [K], >= 0) the result is
+    the element-wise maximum of both, updated in place and returned."""
+    _need_gpu(x, running)
+    x = _rows(x.reshape(-1, x.shape[-1]))
+    M, K = x.shape
+    if running is None:
+        running = torch.zeros((K,), dtype=torch.float32, device=x.device)
+    elif running.dtype != torch.float32 or running.numel() != K or not running.is_contiguous():
+        raise ValueError("running must be a contiguous fp32 tensor with K elements")
+    with torch.cuda.device(x.device):
+        L.call("fmsmo_absmax_cols", x.data_ptr(), _dt(x), _ld(x), M, K, running.data_ptr(), _stream(x))
+    return running

@@ -57,8 +57,24 @@ def prepare_deploy_weights(weight, smoothq_act_scale=None, smoothq_alpha=0.5, w_
         # divide by a tensor, not a Python scalar: on the GPU torch turns "/ scalar" into a multiply
         # by the reciprocal, which is one ulp off the IEEE quotient the CPU evaluation gives
         w_scale = w_clip_val * 2 / torch.tensor(254.0, device=w_clip_val.device, dtype=w_clip_val.dtype)
-        w_int8 = torch.round(ws.t() / w_scale).clamp(-127, 127).t().to(torch.int).to(torch.int8)
+        w_int8 = _quantize_weight_rows(weight, sq, w_scale)
     return w_int8.contiguous(), w_scale, sq
+
+
+def _quantize_weight_rows(weight, smoothq_scale, w_scale):
+    """clamp(round((W * s).t() / w_scale), -127, 127).t() as int8 (from_fms_mo, linear.py:861-866).
+    On the GPU this is one pass of the HIP weight quantizer (bit-identical to the torch expression
+    for the same operands); weights still on the CPU are converted with the torch expression."""
+    N, Kd = weight.shape
+    if weight.is_cuda and Kd % 8 == 0 and weight.dtype in (torch.float16, torch.bfloat16, torch.float32):
+        sq = smoothq_scale.to(weight.device).reshape(-1)
+        smooth = None if sq.numel() == 1 and float(sq[0]) == 1.0 else sq.expand(Kd).contiguous()
+        ws = torch.as_tensor(w_scale, device=weight.device).reshape(-1)
+        if not ws.is_floating_point():
+            ws = ws.float()
+        return kernels.quant_weight_i8(weight.detach(), ws, smooth, mode="div")
+    w = torch.round((weight * smoothq_scale).t() / w_scale).clamp(-127, 127).t()
+    return w.to(torch.int).to(torch.int8)
 
 
 def _compute_dtype(x_dtype, smooth):
@@ -298,9 +314,7 @@ class QLinearINT8Deploy(nn.Linear):
             m.register_buffer("w_scale", w_scale)
             m.register_buffer("w_zp", w_zp)
             m.register_buffer("smoothq_scale", smoothq_scale)
-            w_int8 = (torch.round((fms_mo_qlinear.weight * smoothq_scale).t() / w_scale)
-                      .clamp(-w_levels / 2, w_levels / 2).t())
-            w_int8 = w_int8.to(torch.int)
+            w_int8 = _quantize_weight_rows(fms_mo_qlinear.weight, smoothq_scale, w_scale).to(torch.int)
             m.weight = nn.Parameter(w_int8.to(torch.int8), requires_grad=False)
             if m.useSymAct:
                 corr_term_int = 0

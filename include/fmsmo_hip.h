@@ -225,6 +225,37 @@ int fmsmo_grouped_gemm_i8_dq(const int8_t* a, int64_t lda, const int8_t* b, int6
                              int y_dtype, int64_t ldy, int64_t N, int64_t K,
                              fmsmo_stream_t stream);
 
+/* ------------------------------------------------------------------------------------------
+ * 6. Offline weight path: float weights -> int8 rows (+ integer row sums), one pass over W.
+ *      t_nk = rnd_T1( W_nk * smooth_k )                              (smooth may be NULL)
+ *      FMSMO_WQ_MUL:  q_nk = rint( clamp( rnd_T2( coef_n * t_nk ), -127, 127 ) )
+ *      FMSMO_WQ_DIV:  q_nk = clamp( rint( rnd_T2( t_nk / coef_n ) ), -127, 127 )
+ *      row_sum_n = sum_k q_nk                                         (row_sum may be NULL)
+ *    T1 = promote(w_dtype, smooth_dtype), T2 = promote(T1, coef_dtype), the dtypes torch uses.
+ *    coef has N elements or 1.  W 16-byte aligned, K and ldw multiples of 8 elements.
+ *    MUL with coef = 127 / clip_val: the AIU checkpoint writer, process_weight
+ *    (fms_mo/utils/aiu_utils.py:237-279) after process_smoothquant (:87-122); row_sum is
+ *    process_zero_shift (:282-333).  DIV with coef = w_scale: QLinearINT8Deploy.from_fms_mo
+ *    (fms_mo/modules/linear.py:861-866).
+ * ------------------------------------------------------------------------------------------ */
+enum { FMSMO_WQ_MUL = 0, FMSMO_WQ_DIV = 1 };
+int fmsmo_quant_weight_i8(const void* w, int w_dtype, int64_t ldw, const void* smooth,
+                          int smooth_dtype, const void* coef, int coef_dtype, int64_t coef_n,
+                          int mode, int8_t* q, int64_t ldq, int32_t* row_sum, int64_t N, int64_t K,
+                          fmsmo_stream_t stream);
+
+/*
+ * Per-column running abs-max over the rows of x:  out[k] = max( out[k], max_m |x[m][k]| ), fp32.
+ * The caller initialises out (zeros for a fresh statistic, the running value otherwise; values
+ * must be >= 0).  Serves the SmoothQuant statistics: the activation scale collected by forward
+ * hooks (fms_mo/quant/ptq.py:2586-2595: comming_max = x.view(-1, K).abs().max(dim=0), running
+ * max) and the weight column maximum of get_smoothq_scale (fms_mo/modules/linear.py:345-368) and
+ * process_smoothquant (fms_mo/utils/aiu_utils.py:105-107).  x 16-byte aligned, K and ldx
+ * multiples of 8 elements.
+ */
+int fmsmo_absmax_cols(const void* x, int x_dtype, int64_t ldx, int64_t M, int64_t K, float* out,
+                      fmsmo_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -398,3 +398,31 @@ def i8i8_aiu(x, weight, bias, qdata, weight_quant_type, activ_quant_type, smooth
     else:
         w_dq = (weight * w_cv.unsqueeze(dim=1) / 127) / sq
     return torch.nn.functional.linear(x_dq.to(dtype), w_dq.to(dtype), bias.to(dtype))
+
+
+# ------------------------------------------------------------------------------------------
+# AIU checkpoint conversion (offline weight path)
+# ------------------------------------------------------------------------------------------
+def aiu_convert_layer(weight, w_cv, sq_a_scale=None, sq_alpha=None, a_cv=None, a_cvn=None):
+    """One layer of convert_sd_for_aiu: process_smoothquant (fms_mo/utils/aiu_utils.py:87-122),
+    process_weight without SAWB recomputation (:237-279), process_zero_shift (:282-333).
+    Returns a dict with ``weight`` (int8) and, when they apply, ``smoothq_scale`` (fp16) and
+    ``zero_shift`` (fp32)."""
+    out = {}
+    pre = weight
+    if sq_a_scale is not None and sum(sq_a_scale) != 0:
+        sq_w_scale = weight.abs().max(dim=0, keepdim=True).values.clamp(min=1e-5)
+        sq_scale = sq_a_scale.pow(sq_alpha) / sq_w_scale.pow(1 - sq_alpha)
+        pre = weight * sq_scale
+        out["smoothq_scale"] = sq_scale.squeeze().to(torch.float16)
+    cv = w_cv.unsqueeze(dim=1) if w_cv.numel() > 1 else w_cv
+    w_int = torch.clamp(127 / cv * pre, -127, 127).round()
+    out["weight"] = w_int.to(torch.int8)
+    if a_cv is not None and a_cvn is not None and not torch.equal(a_cv, -a_cvn):
+        out["zero_shift"] = torch.sum(w_int, dim=1).to(torch.float32)
+    return out
+
+
+def absmax_cols(x):
+    """comming_max of the SmoothQuant statistics hook (fms_mo/quant/ptq.py:2586-2595)."""
+    return x.reshape(-1, x.shape[-1]).abs().max(dim=0).values.float()

@@ -1,0 +1,168 @@
+"""Offline weight path and SmoothQuant statistics on the GPU against the CPU oracle: the weight
+quantizer (both recipes, all dtype regimes), the column abs-max, the AIU-style checkpoint writer
+and its reader."""
+import os
+import types
+
+import pytest
+import torch
+from torch import nn
+
+from oracle import qlinear_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def K():
+    from fms_mo_amd import kernels
+
+    return kernels
+
+
+def gen(seed):
+    return torch.Generator().manual_seed(seed)
+
+
+@pytest.mark.parametrize("wdt,cdt", [(torch.float16, torch.float32), (torch.float16, torch.float16),
+                                     (torch.bfloat16, torch.bfloat16), (torch.float32, torch.float32)])
+@pytest.mark.parametrize("perch", [False, True])
+@pytest.mark.parametrize("shape", [(96, 256), (4096, 4096), (513, 14336)])
+def test_weight_quantizer_aiu_recipe_bit_exact(dev, wdt, cdt, perch, shape):
+    N, Kd = shape
+    g = gen(81)
+    w = (0.02 * torch.randn(N, Kd, generator=g)).to(wdt)
+    w[3, 5] = 0.0
+    w_cv = (w.float().abs().amax(dim=1) if perch else w.float().abs().amax().reshape(1)).to(cdt)
+    a_scale = (torch.rand(Kd, generator=g) * 4 + 0.1).to(cdt)
+    alpha = torch.tensor([0.5], dtype=cdt)
+    a_cv, a_cvn = torch.tensor(3.0), torch.tensor(-1.0)
+    for sq in (None, a_scale):
+        ref = O.aiu_convert_layer(w, w_cv, sq, alpha, a_cv, a_cvn)
+        smooth = None
+        if sq is not None:
+            wmax = w.abs().max(dim=0, keepdim=True).values.clamp(min=1e-5)
+            smooth = (sq.pow(alpha) / wmax.pow(1 - alpha)).reshape(-1)
+        q, rs = K().quant_weight_i8(w.to(dev), (127 / w_cv).to(dev), None if smooth is None else smooth.to(dev),
+                                    mode="mul", want_row_sum=True)
+        assert torch.equal(q.cpu(), ref["weight"])
+        # exact integer sums; the reference rounds them to the dtype the weights were computed in
+        t2 = torch.promote_types(wdt, cdt)
+        assert torch.equal(rs.cpu().to(t2).float(), ref["zero_shift"])
+        assert torch.equal(rs.cpu().long(), ref["weight"].long().sum(dim=1))
+        assert q.abs().max().item() <= 127
+
+
+@pytest.mark.parametrize("wdt,cdt", [(torch.float16, torch.float32), (torch.float16, torch.float16)])
+def test_weight_quantizer_deploy_recipe_bit_exact(dev, wdt, cdt):
+    g = gen(82)
+    w = (0.02 * torch.randn(1000, 2048, generator=g)).to(wdt)
+    w_cv = w.float().abs().amax(dim=1).to(cdt)
+    smooth = (torch.rand(2048, generator=g) * 2 + 0.2).to(cdt)
+    for sm in (torch.ones(1, dtype=cdt), smooth):
+        q_ref, w_scale = O.quant_weight_deploy(w, w_cv.reshape(1, -1), sm.reshape(1, -1) if sm.numel() > 1 else sm)
+        q = K().quant_weight_i8(w.to(dev), w_scale.reshape(-1).to(dev), sm.expand(2048).contiguous().to(dev), mode="div")
+        assert torch.equal(q.cpu(), q_ref)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("shape", [(1, 64), (37, 4096), (5000, 14336), (4096, 2056)])
+def test_absmax_cols_and_running_update(dev, dtype, shape):
+    M, Kd = shape
+    x1 = (torch.randn(M, Kd, generator=gen(83)) * 3).to(dtype)
+    x2 = (torch.randn(M, Kd, generator=gen(84)) * 2).to(dtype)
+    x1[0, 3] = -77.0
+    r = K().absmax_cols(x1.to(dev))
+    assert torch.equal(r.cpu(), O.absmax_cols(x1))
+    K().absmax_cols(x2.reshape(1, M, Kd).to(dev), r)      # leading dims are flattened, running max
+    assert torch.equal(r.cpu(), torch.max(O.absmax_cols(x1), O.absmax_cols(x2)))
+
+
+def test_act_scale_hooks_collect_running_maximum(dev):
+    from fms_mo_amd.quant.ptq import get_act_scales
+
+    torch.manual_seed(0)
+    model = nn.Sequential(nn.Linear(256, 512), nn.ReLU(), nn.Linear(512, 128)).half().to(dev)
+    batches = [torch.randn(2, 33, 256, generator=gen(90 + i)).half() for i in range(3)]
+    scales = get_act_scales(model, batches, {"sample_id": 0})
+    assert set(scales) == {"0", "2"}
+    ref0 = torch.stack([O.absmax_cols(b) for b in batches]).amax(dim=0)
+    assert torch.equal(scales["0"], ref0) and scales["0"].device.type == "cpu"
+    assert scales["2"].shape == (512,) and scales["2"].min() >= 0
+
+
+class _Toy(nn.Module):
+    """Two decoder-style linears named like a llama layer, carrying the buffers fms_mo registers."""
+
+    def __init__(self, smoothq):
+        super().__init__()
+        self.config = types.SimpleNamespace(model_type="llama")
+        blk = nn.Module()
+        blk.self_attn = nn.Module()
+        blk.mlp = nn.Module()
+        self.layers = nn.ModuleList([blk])
+        g = gen(85)
+        for parent, name, k, n in [(blk.self_attn, "q_proj", 256, 384), (blk.mlp, "down_proj", 512, 256)]:
+            lin = nn.Linear(k, n, bias=True)
+            with torch.no_grad():
+                lin.weight.copy_(0.05 * torch.randn(n, k, generator=g))
+                lin.bias.copy_(0.01 * torch.randn(n, generator=g))
+            lin.quantize_weight = nn.Module()
+            # with SmoothQuant the weight quantizer sees W * s (s up to ~5 here)
+            lin.quantize_weight.register_buffer(
+                "clip_val", lin.weight.detach().abs().max().reshape(1).clone() * (5.0 if smoothq else 1.0))
+            lin.quantize_weight.register_buffer("clip_valn", -lin.quantize_weight.clip_val.clone())
+            lin.quantize_feature = nn.Module()
+            lin.quantize_feature.register_buffer("clip_val", torch.tensor(4.0))
+            lin.quantize_feature.register_buffer("clip_valn", torch.tensor(-2.5))
+            lin.register_buffer("calib_counter", torch.tensor(0))
+            if smoothq:
+                lin.register_buffer("smoothq_act_scale", torch.rand(k, generator=g) * 3 + 0.2)
+                lin.register_buffer("smoothq_alpha", torch.tensor([0.5]))
+            setattr(parent, name, lin)
+        self.norm = nn.LayerNorm(256)
+
+
+@pytest.mark.parametrize("smoothq", [False, True])
+def test_checkpoint_writer_matches_oracle_and_reader_runs(dev, smoothq, tmp_path):
+    from fms_mo_amd.utils import aiu_utils as A
+
+    model = _Toy(smoothq)
+    A.save_sd_for_aiu(model, {"nbits_w": 8, "qw_mode": "max"}, output_dir=tmp_path, device=dev)
+    sd = torch.load(os.path.join(tmp_path, "qmodel_for_aiu.pt"), weights_only=True)
+    msd = model.state_dict()
+    for layer in ("layers.0.self_attn.q_proj", "layers.0.mlp.down_proj"):
+        ref = O.aiu_convert_layer(msd[layer + ".weight"], msd[layer + ".quantize_weight.clip_val"],
+                                  msd.get(layer + ".smoothq_act_scale"), msd.get(layer + ".smoothq_alpha"),
+                                  msd[layer + ".quantize_feature.clip_val"], msd[layer + ".quantize_feature.clip_valn"])
+        assert sd[layer + ".weight"].dtype == torch.int8 and torch.equal(sd[layer + ".weight"], ref["weight"])
+        assert sd[layer + ".zero_shift"].dtype == torch.float32
+        assert torch.equal(sd[layer + ".zero_shift"], ref["zero_shift"])
+        assert (layer + ".smoothq_scale" in sd) == smoothq
+        if smoothq:
+            assert torch.equal(sd[layer + ".smoothq_scale"], ref["smoothq_scale"])
+        assert sd[layer + ".quantize_weight.clip_val"].dtype == torch.float16
+        assert layer + ".calib_counter" not in sd and layer + ".smoothq_act_scale" not in sd
+    assert sd["norm.weight"].dtype == torch.float16
+
+    # reader: the deployed int8 module reproduces the float layer within quantization error
+    layer = "layers.0.self_attn.q_proj"
+    m = A.deploy_linear_from_aiu_sd(sd, layer, device=dev, use_int_kernel="cutlass")
+    x = (torch.randn(40, 256, generator=gen(86)) * 0.5).clamp(-2.4, 3.9).half()
+    y = m(x.to(dev)).float().cpu()
+    lin = model.layers[0].self_attn.q_proj
+    ref = torch.nn.functional.linear(x.float(), lin.weight, lin.bias)
+    err = (y - ref).abs().max().item()
+    assert err < 0.05 * ref.abs().max().item() + 0.02, err
+
+
+def test_writer_rejects_what_it_cannot_do(dev):
+    from fms_mo_amd.utils import aiu_utils as A
+
+    model = _Toy(False)
+    with pytest.raises(NotImplementedError):
+        A.convert_sd_for_aiu(model, recompute_narrow_weights=True, device=dev)
+    with pytest.raises(ValueError):
+        A.save_sd_for_aiu(model, {"nbits_w": 4}, device=dev)
+    model.config.model_type = "mamba"
+    with pytest.raises(NotImplementedError):
+        A.convert_sd_for_aiu(model, device=dev)

@@ -329,3 +329,38 @@ def test_qlinear_forward_with_smoothquant_close_to_fp():
     ref = x @ W.t()
     e = lambda t: ((t - ref).norm() / ref.norm()).item()
     assert e(y) < 0.02 and e(y) < e(y0)          # SmoothQuant helps with outlier channels
+
+
+# ------------------------------------------------------------------------------------------
+# AIU checkpoint conversion
+# ------------------------------------------------------------------------------------------
+def test_aiu_convert_layer_closed_forms_and_invariants():
+    g = torch.Generator().manual_seed(5)
+    w = 0.03 * torch.randn(64, 128, generator=g)
+    w_cv = w.abs().amax(dim=1)
+    a = torch.rand(128, generator=g) * 4 + 0.1
+    out = O.aiu_convert_layer(w, w_cv, a, torch.tensor([0.5]), torch.tensor(2.0), torch.tensor(-1.0))
+    q = out["weight"]
+    assert q.dtype == torch.int8 and q.abs().max() <= 127
+    # alpha = 0.5: s_k = sqrt(a_k) / sqrt(max_n |W_nk|)
+    s = (a.double().sqrt() / w.abs().amax(dim=0).double().sqrt())
+    assert torch.allclose(out["smoothq_scale"].double(), s, rtol=1e-3)
+    # q = rint(127 W s / cv) away from ties, clamped
+    t = (127.0 * w.double() * s / w_cv.double()[:, None]).clamp(-127, 127)
+    away = (t - t.round()).abs() < 0.49
+    assert torch.equal(q.double()[away], t.round()[away])
+    # zero shift = integer row sums, fp32, only for asymmetric activations
+    assert torch.equal(out["zero_shift"], q.sum(dim=1).float())
+    sym = O.aiu_convert_layer(w, w_cv, None, None, torch.tensor(2.0), torch.tensor(-2.0))
+    assert "zero_shift" not in sym and "smoothq_scale" not in sym
+    # every row reaches +-127 at its arg-max when the clip value is the row maximum
+    assert torch.equal(sym["weight"].abs().amax(dim=1), torch.full((64,), 127, dtype=torch.int8))
+    # all-zero activation scale switches SmoothQuant off
+    off = O.aiu_convert_layer(w, w_cv, torch.zeros(128), torch.tensor([0.5]))
+    assert "smoothq_scale" not in off and torch.equal(off["weight"], sym["weight"])
+
+
+def test_absmax_cols_is_a_running_maximum():
+    x = torch.tensor([[1.0, -5.0], [-3.0, 2.0]])
+    assert torch.equal(O.absmax_cols(x), torch.tensor([3.0, 5.0]))
+    assert torch.equal(O.absmax_cols(x.reshape(1, 2, 2).half()), torch.tensor([3.0, 5.0]))
