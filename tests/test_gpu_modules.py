@@ -224,3 +224,44 @@ def test_fp8_linear_vs_oracle(dev, cfg):
     exact = (qx.double() * s_x.double()) @ (m.weight.data.cpu().double() * m.weight_scale.data.cpu().double()).t() + b.double()
     torch.testing.assert_close(y.reshape(-1, 384).double(), exact, rtol=1e-2, atol=1e-2)
     torch.testing.assert_close(y.float(), ref.float(), rtol=3e-2, atol=3e-2)
+
+
+def test_swapped_mlp_replays_from_a_hip_graph(dev):
+    """The reference's route to a speed-up is capturing the lowered model (torch.compile /
+    CUDA graphs, examples/QAT_INT8/README.md:116-122).  A gated MLP of three deploy modules is
+    captured once and replayed with new inputs, with eager work and synchronisations between the
+    replays; every replay must equal the eager result bit for bit.  No entry point allocates,
+    synchronises or clears memory, so the capture holds only kernel launches."""
+    from fms_mo_amd.modules.linear import QLinearINT8Deploy
+
+    H, I, T = 512, 1536, 48
+    mods = {}
+    for name, k, n, seed in [("gate", H, I, 1), ("up", H, I, 2), ("down", I, H, 3)]:
+        q = make_qlinear(None, k, n, smoothq=True, seed=seed)
+        q.set_act_scale(torch.rand(k, generator=gen(10 + seed)) * 3 + 0.2)
+        mods[name] = QLinearINT8Deploy.from_fms_mo(q, use_int_kernel="cutlass", use_dynamic_max_act_Qfunc=-1,
+                                                   recalc_clipvals=False, target_device=dev)
+
+    def mlp(x):
+        return mods["down"](torch.nn.functional.silu(mods["gate"](x)) * mods["up"](x))
+
+    xs = [outlier_x(T, H, 20 + i).to(dev) for i in range(4)]
+    eager = [mlp(x).clone() for x in xs]            # also warms the cached host-side checks
+    static_x = xs[0].clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        mlp(static_x)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static_y = mlp(static_x)
+    for rnd in range(2):
+        for x, ref in zip(xs, eager):
+            static_x.copy_(x)
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(static_y.view(torch.int16), ref.view(torch.int16))
+            _ = mlp(x)                               # eager work between replays
+            torch.cuda.synchronize()
