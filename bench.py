@@ -171,8 +171,9 @@ def main():
 
 
 def extras(torch, K, dev):
-    """FP8 GEMMs (Granite-3-8B-like shapes, M=2048) and decode shapes (M in 1,4,16); reported in
-    addition to the headline value."""
+    """FP8 GEMMs (Granite-3-8B-like shapes, M=2048), decode shapes (M in 1,4,16), the Mixtral-style
+    grouped expert GEMMs and the chunk-truncate emulation; reported in addition to the headline
+    value."""
     from fms_mo_amd import _lib as L
 
     res = {}
@@ -235,6 +236,33 @@ def extras(torch, K, dev):
             res[f"decode_i8_M{M}_{name}"] = {"us": round(ms * 1e3, 2), "GBps": round(gbs, 1), "frac_hbm": round(gbs / PEAK_HBM_GBS, 4)}
             del graph
         del ws_i8
+    # Mixtral-style MoE (8 experts, 4096 tokens routed top-2 with uniform-random logits) in one
+    # grouped launch per projection, and the chunk-truncate emulation on one expert's w2
+    E, T, H, I = 8, 4096, 4096, 14336
+    g = torch.Generator().manual_seed(4)
+    flat = torch.rand(T, E, generator=g).topk(2, dim=-1).indices.reshape(-1)
+    counts = torch.bincount(flat, minlength=E)
+    offsets = torch.zeros(E + 1, dtype=torch.int32)
+    offsets[1:] = counts.cumsum(0)
+    rows = int(offsets[-1])
+    off_d = offsets.to(dev)
+    for name, k, n in (("w1_w3", H, I), ("w2", I, H)):
+        a = torch.randint(-127, 128, (rows, k), dtype=torch.int8, device=dev)
+        w = torch.randint(-127, 128, (E, n, k), dtype=torch.int8, device=dev)
+        a_s = torch.rand(rows, device=dev) * 1e-2
+        w_s = torch.rand(E, n, device=dev) * 1e-3
+        ms = timeit(lambda: K.grouped_gemm_i8_dq(a, w, off_d, a_s, w_s, None, out_dtype=torch.float16), iters=10, warm=3)
+        tops = 2.0 * rows * k * n / (ms * 1e-3) / 1e12
+        res[f"moe_grouped_i8_{name}"] = {"ms": round(ms, 4), "tops": round(tops, 1), "frac_peak": round(tops / PEAK_INT8_TOPS, 4),
+                                         "rows_per_expert": counts.tolist()}
+        del a, w
+    m_e = int(counts[0])
+    a = torch.randint(-127, 128, (m_e, I), dtype=torch.int8, device=dev)
+    w = torch.randint(-127, 128, (H, I), dtype=torch.int8, device=dev)
+    for t in (7, 16):
+        ms = timeit(lambda: K.matmul_chunk(a, w, chunk_size=64, chunk_trun_bits=t), iters=10, warm=3)
+        tops = 2.0 * m_e * I * H / (ms * 1e-3) / 1e12
+        res[f"chunk64_trunc{t}_i8_w2_M{m_e}"] = {"ms": round(ms, 4), "tops": round(tops, 1), "frac_peak": round(tops / PEAK_INT8_TOPS, 4)}
     return res
 
 
