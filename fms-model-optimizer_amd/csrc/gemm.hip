@@ -1,6 +1,6 @@
 // Host launchers of the tiled MFMA GEMMs (int8 -> int32, int8 / e4m3 with fused dequantizing
 // epilogue, grouped mixture-of-experts variant).
-#include "gemm_tile.hpp"
+#include "gemm_rs.hpp"
 #include <cmath>
 #include <cstdlib>
 
@@ -57,14 +57,13 @@ int check_gemm(const void* a, int64_t lda, const void* b, int64_t ldb, const voi
 struct TileBig { static constexpr int BM = 256, BN = 256, BK = 64, NST = 4, WGM = 2, WGN = 2; };
 struct TileWide { static constexpr int BM = 128, BN = 256, BK = 64, NST = 4, WGM = 2, WGN = 2; };
 struct TileMid { static constexpr int BM = 128, BN = 128, BK = 64, NST = 4, WGM = 2, WGN = 2; };
-struct TileBig192 { static constexpr int BM = 256, BN = 192, BK = 64, NST = 4, WGM = 2, WGN = 2; };
 
 // Pick the tile shape by (relative kernel efficiency) x (fill of the last round of tiles over
 // the 256 compute units).  The efficiencies are measured loop efficiencies of the three shapes
 // (bigger tiles move fewer bytes per MFMA); 128x128 tiles fit two blocks per CU.
 int pick_tile(int M, int N) {
   static const char* force = getenv("FMSMO_TILE");  // tuning aid: 0 = 256x256, 1 = 128x256, 2 = 128x128
-  if (force && force[0] >= '0' && force[0] <= '3') return force[0] - '0';
+  if (force && force[0] >= '0' && force[0] <= '2') return force[0] - '0';
   // Fitted to measurements on the Llama / Granite shapes: relative loop efficiency of the three
   // tile shapes, and a sub-linear penalty for a partially filled last round (idle CUs leave
   // power, hence clock, to the busy ones).
@@ -95,6 +94,24 @@ void launch_tile(const GemmArgs& g0, const Epi& epi, hipStream_t st) {
       (gemm_tile_kernel<Tile::BM, Tile::BN, Tile::BK, Tile::NST, Tile::WGM, Tile::WGN, OP, 1,
                         GROUPED, Epi>),
       grid, block, 0, st, g, epi, NoChunk{});
+}
+
+// 256x256 tiles with K a multiple of 128 run the register-staged pipeline (gemm_rs.hpp: whole
+// 128-byte lines, half the L2 -> L1 traffic).  FMSMO_RS=0 / 1 forces the choice for tuning.
+static bool use_register_staged(int op) {
+  static const char* force = getenv("FMSMO_RS");
+  if (force && (force[0] == '0' || force[0] == '1')) return force[0] == '1';
+  (void)op;
+  return true;
+}
+template <int OP, class Epi>
+void launch_rs(const GemmArgs& g0, const Epi& epi, hipStream_t st) {
+  GemmArgs g = g0;
+  g.grid_n = div_up(g.N, 256);
+  g.grid_m = div_up(g.M, 256);
+  g.group_m = 4;
+  dim3 grid((unsigned)(g.grid_m * g.grid_n)), block(256);
+  hipLaunchKernelGGL((gemm_rs_kernel<OP, Epi>), grid, block, 0, st, g, epi);
 }
 
 // Generic fallback (any K % 16 == 0): one thread per output element, 4-byte dot products.
@@ -129,9 +146,11 @@ template <int OP, class Epi>
 void launch_any(const GemmArgs& g, const Epi& epi, hipStream_t st) {
   if (g.K % 64 == 0) {
     switch (pick_tile(g.M, g.N)) {
-      case 0: launch_tile<TileBig, OP, false>(g, epi, st); break;
+      case 0:
+        if (g.K % 128 == 0 && use_register_staged(OP)) launch_rs<OP>(g, epi, st);
+        else launch_tile<TileBig, OP, false>(g, epi, st);
+        break;
       case 1: launch_tile<TileWide, OP, false>(g, epi, st); break;
-      case 3: launch_tile<TileBig192, OP, false>(g, epi, st); break;
       default: launch_tile<TileMid, OP, false>(g, epi, st); break;
     }
   } else {

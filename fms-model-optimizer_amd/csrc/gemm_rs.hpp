@@ -1,0 +1,259 @@
+// Register-staged MFMA GEMM for gfx950: C[M,N] = A[M,K] . B[N,K]^T, 1-byte operands, 256x256 tile.
+//
+// Why a second pipeline: with 64-byte K stages (gemm_tile.hpp) every 128-byte L2 line is requested
+// twice, one stage apart, and the 64 KiB of lines a stage touches do not survive in the vector L1;
+// the L2 -> L1 traffic is therefore twice the operand bytes and, with all 256 CUs active, that is
+// what bounds the loop.  Here K advances in slabs of 128 bytes (whole lines, fetched once).  A
+// 256x256 slab is 64 KiB, so only two fit in LDS; the third pipeline level is the register file:
+// the slab after next is fetched with plain buffer loads (8 rows x 128 B per wave instruction)
+// into 64 VGPRs per lane and written to LDS (ds_write_b128, XOR-swizzled) as soon as the buffer it
+// replaces has been read for the last time.
+//
+// Per slab: NKS MFMA k-steps with register double-buffered operand fragments.  At the start of
+// the last k-step every wave holds its last fragments of the current buffer, so after one
+// barrier the buffer is refilled (from the staging registers) and the staging registers are
+// re-loaded (slab + 3), all interleaved with the MFMAs of that k-step.  One barrier per slab.
+// Rows past M / N read as zero through the buffer descriptor's range check.
+#pragma once
+#include "gemm_tile.hpp"
+
+namespace fmsmo {
+
+template <int OP, class Epi>
+__global__ __launch_bounds__(256) void gemm_rs_kernel(GemmArgs g, Epi epi) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  typedef Mma<OP> MM;
+  typedef typename MM::Frag Frag;
+  typedef typename MM::Acc Acc;
+  constexpr int BM = 256, BN = 256, BK = 128, CPR = 8;
+  constexpr int TM = 128, TN = 128, FM = 4, FN = 4;
+  constexpr int NKS = BK / MM::KSTEP;   // MFMA k-steps per slab (int8 4, e4m3 2)
+  constexpr int CL = MM::KSTEP / 32;    // 16-byte chunks per lane per k-step
+  constexpr int SLAB = (BM + BN) * BK;  // 64 KiB
+  constexpr int NJ = 8;                 // row groups of 32 per operand and thread
+  static_assert(NKS % 2 == 0, "fragment buffers alternate per k-step");
+  __shared__ __attribute__((aligned(16))) uint8_t lds[2 * SLAB];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+  int tile_m, tile_n;
+  tile_of_block(blockIdx.x, gridDim.x, g.grid_m, g.grid_n, g.group_m, tile_m, tile_n);
+  const int row_lo = tile_m * BM, row_hi = g.M, col_lo = tile_n * BN;
+
+  // ---- global -> register staging: thread -> (row = tid / 8 + 32 j, 16-byte chunk = tid % 8)
+  const int ld_row = tid >> 3, ld_chunk = tid & 7;
+  const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)g.a, 0, (int)((int64_t)(g.M - 1) * g.lda + g.K), 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)g.b, 0, (int)((int64_t)(g.N - 1) * g.ldb + g.K), 0x00020000);
+  const int va = (row_lo + ld_row) * (int)g.lda + ld_chunk * 16;
+  const int vb = (col_lo + ld_row) * (int)g.ldb + ld_chunk * 16;
+  const int sa32 = 32 * (int)g.lda, sb32 = 32 * (int)g.ldb;
+  const int nslab = g.K / BK;
+  v4i sta[NJ], stb[NJ];
+  // The loads keep their program order (a scheduling barrier that only memory instructions may
+  // not cross follows each one): the compiler's vmcnt bookkeeping is exact only if the order in
+  // the prologue and in the loop is the same.
+  constexpr int NOT_VMEM = 0x7ff & ~(0x010 | 0x020 | 0x040);
+  auto load_a = [&](int j, int k0) {
+    sta[j] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, va, j * sa32 + k0, 0));
+    __builtin_amdgcn_sched_barrier(NOT_VMEM);
+  };
+  auto load_b = [&](int j, int k0) {
+    stb[j] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, vb, j * sb32 + k0, 0));
+    __builtin_amdgcn_sched_barrier(NOT_VMEM);
+  };
+  auto load_slab = [&](int s) {
+    const int k0 = min(s, nslab - 1) * BK;  // slabs past the end re-read the last one (never used)
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+      load_a(j, k0);
+      load_b(j, k0);
+    }
+  };
+  // LDS position of the thread's chunk: row-major [row][128 B], chunk c of row r at c ^ swz(r);
+  // swz depends on r % 16 only, so it is the same for all 8 row groups
+  const int wr = ld_row * BK + ((ld_chunk ^ swz<CPR, 1>(ld_row)) * 16);
+  auto store_slab = [&](uint8_t* buf) {
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+      *(v4i*)(buf + wr + j * 32 * BK) = sta[j];
+      *(v4i*)(buf + BM * BK + wr + j * 32 * BK) = stb[j];
+    }
+  };
+
+  // ---- LDS -> MFMA operand addressing
+  const int fr = lane & 31, fg = lane >> 5;
+  const int fsw = swz<CPR, 1>(fr);
+  int a_rd[NKS][CL], b_rd[NKS][CL];
+#pragma unroll
+  for (int s = 0; s < NKS; ++s)
+#pragma unroll
+    for (int e = 0; e < CL; ++e) {
+      const int c = s * 2 * CL + fg * CL + e;
+      a_rd[s][e] = (wm * TM + fr) * BK + ((c ^ fsw) * 16);
+      b_rd[s][e] = BM * BK + (wn * TN + fr) * BK + ((c ^ fsw) * 16);
+    }
+  // operand fragments are kept as their 16-byte halves so that single reads can be placed
+  // between MFMAs; index r enumerates the reads of one k-step: A (i, e) first, then B (j, e)
+  v4i ha[2][FM][CL], hb[2][FN][CL];
+  constexpr int NRD = (FM + FN) * CL, NMMA = FM * FN;
+  auto read_one = [&](const uint8_t* ls, int s, int buf, auto r_c) {
+    constexpr int R = decltype(r_c)::value;
+    if constexpr (R < FM * CL) {
+      ha[buf][R / CL][R % CL] = *(const v4i*)(ls + a_rd[s][R % CL] + (R / CL) * 32 * BK);
+    } else {
+      constexpr int Q = R - FM * CL;
+      hb[buf][Q / CL][Q % CL] = *(const v4i*)(ls + b_rd[s][Q % CL] + (Q / CL) * 32 * BK);
+    }
+  };
+  auto read_all = [&](const uint8_t* ls, int s, int buf) {
+    [&]<int... R>(std::integer_sequence<int, R...>) {
+      (read_one(ls, s, buf, std::integral_constant<int, R>{}), ...);
+    }(std::make_integer_sequence<int, NRD>{});
+  };
+  auto frag_a = [&](int buf, int i) -> Frag {
+    if constexpr (CL == 1) return ha[buf][i][0];
+    else return Frag{ha[buf][i][0][0], ha[buf][i][0][1], ha[buf][i][0][2], ha[buf][i][0][3],
+                     ha[buf][i][1][0], ha[buf][i][1][1], ha[buf][i][1][2], ha[buf][i][1][3]};
+  };
+  auto frag_b = [&](int buf, int j) -> Frag {
+    if constexpr (CL == 1) return hb[buf][j][0];
+    else return Frag{hb[buf][j][0][0], hb[buf][j][0][1], hb[buf][j][0][2], hb[buf][j][0][3],
+                     hb[buf][j][1][0], hb[buf][j][1][1], hb[buf][j][1][2], hb[buf][j][1][3]};
+  };
+
+  Acc acc[FM][FN];
+#pragma unroll
+  for (int i = 0; i < FM; ++i)
+#pragma unroll
+    for (int j = 0; j < FN; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
+  auto mma_step = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+      for (int j = 0; j < FN; ++j) acc[i][j] = MM::mma(frag_a(buf, i), frag_b(buf, j), acc[i][j]);
+  };
+
+  // One k-step in explicit order.  Behind MFMA r (a full scheduling barrier closes every group):
+  // read r of the fragments for the following k-step (from `rd_ls`, k-step `RS`, into buffer RB)
+  // and the staging pairs [P0, P1) spread evenly over the 16 MFMAs.  A pair = write one staged
+  // 16-byte chunk into `wr_buf`, then re-load its registers from slab `k0`.  Pair p < NJ is
+  // operand A row group p, pair p >= NJ operand B row group p - NJ.
+  auto pair = [&](uint8_t* wr_buf, int k0, auto p_c) {
+    constexpr int P = decltype(p_c)::value;
+    if constexpr (P < NJ) {
+      *(v4i*)(wr_buf + wr + P * 32 * BK) = sta[P];
+      sta[P] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, va, P * sa32 + k0, 0));
+    } else {
+      *(v4i*)(wr_buf + BM * BK + wr + (P - NJ) * 32 * BK) = stb[P - NJ];
+      stb[P - NJ] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, vb, (P - NJ) * sb32 + k0, 0));
+    }
+  };
+  auto kstep = [&](auto mb_c, const uint8_t* rd_ls, auto rs_c, auto rb_c, uint8_t* wr_buf, int k0,
+                   auto p0_c, auto p1_c) {
+    constexpr int MB = decltype(mb_c)::value, RS = decltype(rs_c)::value, RB = decltype(rb_c)::value;
+    constexpr int P0 = decltype(p0_c)::value, P1 = decltype(p1_c)::value, NP = P1 - P0;
+    [&]<int... R>(std::integer_sequence<int, R...>) {
+      (
+          [&] {
+            constexpr int I = R / FN, J = R % FN;
+            acc[I][J] = MM::mma(frag_a(MB, I), frag_b(MB, J), acc[I][J]);
+            if constexpr (R < NRD) read_one(rd_ls, RS, RB, std::integral_constant<int, R>{});
+            if constexpr (NP > 0) {
+              constexpr int PA = P0 + R * NP / NMMA, PB = P0 + (R + 1) * NP / NMMA;
+              if constexpr (PB > PA) pair(wr_buf, k0, std::integral_constant<int, PA>{});
+              if constexpr (PB > PA + 1) pair(wr_buf, k0, std::integral_constant<int, PA + 1>{});
+            }
+            __builtin_amdgcn_sched_barrier(0);
+          }(),
+          ...);
+    }(std::make_integer_sequence<int, NMMA>{});
+  };
+  // Staging pairs [0, NP0) are handled in the last k-step of a slab, [NP0, 16) in the first
+  // k-step of the next one (int8 MFMAs are half as long as e4m3 ones: 16 of them cannot hide 16
+  // buffer loads and 16 LDS writes).
+  constexpr int NPAIR = 2 * NJ;
+  constexpr int NP0 = OP == MMA_I8 ? NPAIR / 2 : NPAIR;
+  auto pairs_now = [&](uint8_t* wr_buf, int k0, auto p0_c, auto p1_c) {  // no MFMAs to hide behind
+    [&]<int... P>(std::integer_sequence<int, P...>) {
+      (pair(wr_buf, k0, std::integral_constant<int, decltype(p0_c)::value + P>{}), ...);
+    }(std::make_integer_sequence<int, decltype(p1_c)::value - decltype(p0_c)::value>{});
+  };
+  typedef std::integral_constant<int, 0> C0;
+  typedef std::integral_constant<int, 1> C1;
+  typedef std::integral_constant<int, NP0> CNP0;
+  typedef std::integral_constant<int, NPAIR> CNP;
+  auto slab_k0 = [&](int s) { return min(s, nslab - 1) * BK; };  // slabs past the end: never used
+
+  // ---- prologue: slab 0 into LDS; slab 1: pairs [0, NP0) into LDS and their registers re-loaded
+  // with slab 2, pairs [NP0, 16) still staged (the first k-step of the loop writes them)
+  load_slab(0);
+  pairs_now(lds, slab_k0(1), C0{}, CNP{});
+  pairs_now(lds + SLAB, slab_k0(2), C0{}, CNP0{});
+  __syncthreads();
+  read_all(lds, 0, 0);
+
+  for (int s = 0; s < nslab; ++s) {
+    uint8_t* cur = lds + (s & 1) * SLAB;
+    uint8_t* nxt = lds + ((s + 1) & 1) * SLAB;
+    // first k-step: the rest of the staged slab s + 1 goes into `nxt`, re-loaded with slab s + 2
+    kstep(C0{}, cur, C1{}, C1{}, nxt, slab_k0(s + 2), CNP0{}, CNP{});
+    // middle k-steps
+    [&]<int... KS>(std::integer_sequence<int, KS...>) {
+      (kstep(std::integral_constant<int, (KS + 1) & 1>{}, cur, std::integral_constant<int, KS + 2>{},
+             std::integral_constant<int, KS & 1>{}, nxt, 0, C0{}, C0{}),
+       ...);
+    }(std::make_integer_sequence<int, NKS - 2>{});
+    // Last k-step.  Its fragments are in registers once the LDS counter drains; after the
+    // barrier nobody reads `cur` any more: the staged slab s + 2 starts to go into it, and the
+    // first fragments of slab s + 1 are read from `nxt`.
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+    kstep(std::integral_constant<int, (NKS - 1) & 1>{}, nxt, C0{}, C0{}, cur, slab_k0(s + 3), C0{}, CNP0{});
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+
+  // ---- epilogue: acc[i][j][v] is C(row, col) with
+  //      row = 32 i + 8 (v / 4) + 4 (lane / 32) + v % 4,   col = 32 j + lane % 32
+  const int m_base = row_lo + wm * TM + fg * 4;
+  const int n_base = col_lo + wn * TN + fr;
+  typename Epi::Col colctx[FN];
+#pragma unroll
+  for (int j = 0; j < FN; ++j) colctx[j] = epi.col(min(n_base + j * 32, g.N - 1), 0, g.N);
+  const bool interior = (row_lo + BM <= row_hi) && (col_lo + BN <= g.N);
+#pragma unroll
+  for (int i = 0; i < FM; ++i) {
+    typename Epi::Row rowctx[16];
+#pragma unroll
+    for (int v = 0; v < 16; ++v)
+      rowctx[v] = epi.row(min(m_base + i * 32 + (v >> 2) * 8 + (v & 3), row_hi - 1));
+    if (interior) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int m = m_base + i * 32 + (v >> 2) * 8 + (v & 3);
+#pragma unroll
+        for (int j = 0; j < FN; ++j) epi.store(m, n_base + j * 32, acc[i][j][v], rowctx[v], colctx[j]);
+      }
+    } else {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int m = m_base + i * 32 + (v >> 2) * 8 + (v & 3);
+        if (m < row_hi) {
+#pragma unroll
+          for (int j = 0; j < FN; ++j) {
+            const int n = n_base + j * 32;
+            if (n < g.N) epi.store(m, n, acc[i][j][v], rowctx[v], colctx[j]);
+          }
+        }
+      }
+    }
+  }
+#endif  // __HIP_DEVICE_COMPILE__
+}
+
+}  // namespace fmsmo
