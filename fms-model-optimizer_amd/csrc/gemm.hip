@@ -104,14 +104,14 @@ static bool use_register_staged(int op) {
   (void)op;
   return true;
 }
-template <int OP, class Epi>
+template <int OP, bool GROUPED = false, class Epi>
 void launch_rs(const GemmArgs& g0, const Epi& epi, hipStream_t st) {
   GemmArgs g = g0;
   g.grid_n = div_up(g.N, 256);
-  g.grid_m = div_up(g.M, 256);
+  if (!GROUPED) g.grid_m = div_up(g.M, 256);
   g.group_m = 4;
   dim3 grid((unsigned)(g.grid_m * g.grid_n)), block(256);
-  hipLaunchKernelGGL((gemm_rs_kernel<OP, Epi>), grid, block, 0, st, g, epi);
+  hipLaunchKernelGGL((gemm_rs_kernel<OP, Epi, GROUPED>), grid, block, 0, st, g, epi);
 }
 
 // Generic fallback (any K % 16 == 0): one thread per output element, 4-byte dot products.
@@ -167,9 +167,10 @@ int launch_dq(const GemmArgs& g, const float* a_scale, int a_stride, const float
 #define GO(OUT, BIAS)                                                                         \
   {                                                                                           \
     EpiDequant<OUT, BIAS, REF, AccT> epi{y, ldy, a_scale, w_scale, bias, a_stride, w_stride}; \
-    if constexpr (GROUPED)                                                                    \
-      launch_tile<TileBig, OP, true>(g, epi, st);                                             \
-    else                                                                                      \
+    if constexpr (GROUPED) {                                                                  \
+      if (g.K % 128 == 0 && use_register_staged(OP)) launch_rs<OP, true>(g, epi, st);         \
+      else launch_tile<TileBig, OP, true>(g, epi, st);                                        \
+    } else                                                                                    \
       launch_any<OP>(g, epi, st);                                                             \
   }
 #define GO_BIAS(OUT)                            \

@@ -19,7 +19,7 @@
 
 namespace fmsmo {
 
-template <int OP, class Epi>
+template <int OP, class Epi, bool GROUPED = false>
 __global__ __launch_bounds__(256) void gemm_rs_kernel(GemmArgs g, Epi epi) {
 #if defined(__HIP_DEVICE_COMPILE__)
   typedef Mma<OP> MM;
@@ -39,15 +39,41 @@ __global__ __launch_bounds__(256) void gemm_rs_kernel(GemmArgs g, Epi epi) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
   int tile_m, tile_n;
-  tile_of_block(blockIdx.x, gridDim.x, g.grid_m, g.grid_n, g.group_m, tile_m, tile_n);
-  const int row_lo = tile_m * BM, row_hi = g.M, col_lo = tile_n * BN;
+  int row_lo, row_hi = g.M, expert = 0;
+  if constexpr (GROUPED) {
+    // grouped (mixture-of-experts) mode, as in gemm_tile.hpp: the grid is an upper bound, only
+    // the first real_tiles block ids are mapped; a tile covers rows of one expert
+    int real_m = 0;
+    for (int e = 0; e < g.num_experts; ++e) real_m += (g.offsets[e + 1] - g.offsets[e] + BM - 1) / BM;
+    const int real_tiles = real_m * g.grid_n;
+    if ((int)blockIdx.x >= real_tiles) return;  // uniform for the whole block
+    tile_of_block(blockIdx.x, real_tiles, real_m, g.grid_n, g.group_m, tile_m, tile_n);
+    int t = tile_m;
+    row_lo = 0;
+    for (int e = 0; e < g.num_experts; ++e) {
+      const int lo = g.offsets[e], hi = g.offsets[e + 1];
+      const int nt = (hi - lo + BM - 1) / BM;
+      if (t < nt) {
+        row_lo = lo + t * BM;
+        row_hi = hi;
+        expert = e;
+        break;
+      }
+      t -= nt;
+    }
+  } else {
+    tile_of_block(blockIdx.x, gridDim.x, g.grid_m, g.grid_n, g.group_m, tile_m, tile_n);
+    row_lo = tile_m * BM;
+  }
+  const int col_lo = tile_n * BN;
 
   // ---- global -> register staging: thread -> (row = tid / 8 + 32 j, 16-byte chunk = tid % 8)
   const int ld_row = tid >> 3, ld_chunk = tid & 7;
   const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
       (void*)g.a, 0, (int)((int64_t)(g.M - 1) * g.lda + g.K), 0x00020000);
   const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(
-      (void*)g.b, 0, (int)((int64_t)(g.N - 1) * g.ldb + g.K), 0x00020000);
+      (void*)(g.b + (GROUPED ? (int64_t)expert * g.ldb_e : 0)), 0,
+      (int)((int64_t)(g.N - 1) * g.ldb + g.K), 0x00020000);
   const int va = (row_lo + ld_row) * (int)g.lda + ld_chunk * 16;
   const int vb = (col_lo + ld_row) * (int)g.ldb + ld_chunk * 16;
   const int sa32 = 32 * (int)g.lda, sb32 = 32 * (int)g.ldb;
@@ -224,7 +250,7 @@ __global__ __launch_bounds__(256) void gemm_rs_kernel(GemmArgs g, Epi epi) {
   const int n_base = col_lo + wn * TN + fr;
   typename Epi::Col colctx[FN];
 #pragma unroll
-  for (int j = 0; j < FN; ++j) colctx[j] = epi.col(min(n_base + j * 32, g.N - 1), 0, g.N);
+  for (int j = 0; j < FN; ++j) colctx[j] = epi.col(min(n_base + j * 32, g.N - 1), expert, g.N);
   const bool interior = (row_lo + BM <= row_hi) && (col_lo + BN <= g.N);
 #pragma unroll
   for (int i = 0; i < FM; ++i) {
