@@ -159,7 +159,7 @@ def main():
                    "tokens": M_TOKENS},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_INT8_TOPS,
                      "unit": "TFLOP/s", "frac": round(achieved / PEAK_INT8_TOPS, 4),
-                     "traffic": traffic, "kernel": "gemm_tile_kernel<int8> (4 launches per step)",
+                     "traffic": traffic, "kernel": "gemm_rs_kernel<int8, dequant epilogue> (4 launches per step)",
                      "per_shape_tops": per_shape,
                      "avg_launch_ms": {n: round(ms, 4) for (n, _, _), ms in zip(LLAMA3_8B, gemm_ms)}},
     }

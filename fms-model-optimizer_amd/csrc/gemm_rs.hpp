@@ -67,6 +67,9 @@ __global__ __launch_bounds__(256) void gemm_rs_kernel(GemmArgs g, Epi epi) {
   }
   const int col_lo = tile_n * BN;
 
+#ifdef FMSMO_CLK
+  if (blockIdx.x == 0 && tid == 0 && g.clk) { g.clk[0] = clock64(); g.clk[1] = wall_clock64(); }
+#endif
   // ---- global -> register staging: thread -> (row = tid / 8 + 32 j, 16-byte chunk = tid % 8)
   const int ld_row = tid >> 3, ld_chunk = tid & 7;
   const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
@@ -189,7 +192,10 @@ __global__ __launch_bounds__(256) void gemm_rs_kernel(GemmArgs g, Epi epi) {
           [&] {
             constexpr int I = R / FN, J = R % FN;
             acc[I][J] = MM::mma(frag_a(MB, I), frag_b(MB, J), acc[I][J]);
-            if constexpr (R < NRD) read_one(rd_ls, RS, RB, std::integral_constant<int, R>{});
+            // two fragment reads behind each of the first MFMAs: the last one must be back
+            // well before the k-step ends (its consumers are the first MFMAs of the next one)
+            if constexpr (2 * R < NRD) read_one(rd_ls, RS, RB, std::integral_constant<int, 2 * R>{});
+            if constexpr (2 * R + 1 < NRD) read_one(rd_ls, RS, RB, std::integral_constant<int, 2 * R + 1>{});
             if constexpr (NP > 0) {
               constexpr int PA = P0 + R * NP / NMMA, PB = P0 + (R + 1) * NP / NMMA;
               if constexpr (PB > PA) pair(wr_buf, k0, std::integral_constant<int, PA>{});
@@ -218,9 +224,43 @@ __global__ __launch_bounds__(256) void gemm_rs_kernel(GemmArgs g, Epi epi) {
 
   // ---- prologue: slab 0 into LDS; slab 1: pairs [0, NP0) into LDS and their registers re-loaded
   // with slab 2, pairs [NP0, 16) still staged (the first k-step of the loop writes them)
-  load_slab(0);
-  pairs_now(lds, slab_k0(1), C0{}, CNP{});
-  pairs_now(lds + SLAB, slab_k0(2), C0{}, CNP0{});
+  // (slabs 0 and 1 are fetched together: the accumulators and fragments are not live yet, so
+  // there are registers for a second staging set)
+  {
+    load_slab(0);
+    v4i ta[NJ], tb[NJ];
+    const int k1 = slab_k0(1);
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+      ta[j] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, va, j * sa32 + k1, 0));
+      tb[j] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, vb, j * sb32 + k1, 0));
+    }
+    store_slab(lds);
+    // slab 1: pairs [0, NP0) go to LDS, the rest stay staged
+    [&]<int... P>(std::integer_sequence<int, P...>) {
+      (
+          [&] {
+            if constexpr (P < NP0) {
+              if constexpr (P < NJ) *(v4i*)(lds + SLAB + wr + P * 32 * BK) = ta[P];
+              else *(v4i*)(lds + SLAB + BM * BK + wr + (P - NJ) * 32 * BK) = tb[P - NJ];
+            } else {
+              if constexpr (P < NJ) sta[P] = ta[P];
+              else stb[P - NJ] = tb[P - NJ];
+            }
+          }(),
+          ...);
+    }(std::make_integer_sequence<int, NPAIR>{});
+    const int k2 = slab_k0(2);
+    [&]<int... P>(std::integer_sequence<int, P...>) {
+      (
+          [&] {
+            if constexpr (P < NJ) sta[P] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, va, P * sa32 + k2, 0));
+            else stb[P - NJ] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, vb, (P - NJ) * sb32 + k2, 0));
+            __builtin_amdgcn_sched_barrier(NOT_VMEM);
+          }(),
+          ...);
+    }(std::make_integer_sequence<int, NP0>{});
+  }
   __syncthreads();
   read_all(lds, 0, 0);
 
@@ -243,6 +283,9 @@ __global__ __launch_bounds__(256) void gemm_rs_kernel(GemmArgs g, Epi epi) {
     kstep(std::integral_constant<int, (NKS - 1) & 1>{}, nxt, C0{}, C0{}, cur, slab_k0(s + 3), C0{}, CNP0{});
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#ifdef FMSMO_CLK
+  if (blockIdx.x == 0 && tid == 0 && g.clk) { g.clk[2] = clock64(); g.clk[3] = wall_clock64(); }
+#endif
 
   // ---- epilogue: acc[i][j][v] is C(row, col) with
   //      row = 32 i + 8 (v / 4) + 4 (lane / 32) + v % 4,   col = 32 j + lane % 32
@@ -279,6 +322,9 @@ __global__ __launch_bounds__(256) void gemm_rs_kernel(GemmArgs g, Epi epi) {
       }
     }
   }
+#ifdef FMSMO_CLK
+  if (blockIdx.x == 0 && tid == 0 && g.clk) { g.clk[4] = clock64(); g.clk[5] = wall_clock64(); }
+#endif
 #endif  // __HIP_DEVICE_COMPILE__
 }
 
