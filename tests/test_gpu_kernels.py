@@ -243,7 +243,9 @@ def _rand_i8(shape, seed):
 
 @pytest.mark.parametrize("shape", [(512, 4096, 4096), (300, 520, 1024), (256, 256, 64),
                                    (17, 4096, 4096), (1000, 1200, 256), (129, 130, 80),
-                                   (64, 72, 4112), (2048, 2304, 512)])
+                                   (64, 72, 4112), (2048, 2304, 512),
+                                   # large ragged shapes: 256x256 tiles, K in whole 128-byte slabs
+                                   (4000, 4100, 384), (4097, 4095, 128), (3900, 4352, 256)])
 def test_gemm_i8_i32_exact(dev, shape):
     M, N, Kd = shape
     a, w = _rand_i8((M, Kd), 11), _rand_i8((N, Kd), 12)
@@ -355,10 +357,12 @@ def test_gemm_fp8_dq(dev, M):
     torch.testing.assert_close(y.cpu().float(), ref.float(), rtol=2e-2, atol=2e-2)
 
 
-def test_gemm_fp8_integer_valued_is_exact(dev):
+@pytest.mark.parametrize("shape", [(256, 512, 1024), (4000, 4100, 384), (4097, 4095, 128)])
+def test_gemm_fp8_integer_valued_is_exact(dev, shape):
     # small-integer operands: every product and partial sum is exact in fp32, so any MFMA
-    # summation order must give the exact integer result
-    M, N, Kd = 256, 512, 1024
+    # summation order must give the exact integer result (the large ragged shapes run 256x256
+    # tiles with K in whole 128-byte slabs)
+    M, N, Kd = shape
     a = torch.randint(-4, 5, (M, Kd), generator=gen(46)).float().to(torch.float8_e4m3fn)
     w = torch.randint(-4, 5, (N, Kd), generator=gen(47)).float().to(torch.float8_e4m3fn)
     exact = a.float() @ w.float().t()
