@@ -22,6 +22,9 @@ How each function is pinned (see tests/test_oracle_*.py):
   * fp8 cast            -- all 256 codes and all midpoints against torch's own cast
   * i8i8_aiu            -- the six stored vectors of the reference's own test-suite
                            (tests/golden/ref_w-*_a-*_sq-N.pt)
+  * AIU checkpoint conversion, column abs-max
+                        -- closed forms (sqrt(a)/sqrt(wmax) at alpha = 0.5, rint(127 W s / cv) away
+                           from ties), invariants (|q| <= 127, zero shift = integer row sums)
   * FP8Linear dynamic scale (computed inside torchao 0.11, not in the reference tree):
                            PARITY UNPINNED -- the rule used is the one of the reference's test
                            helper (tests/aiu_addons/test_fp8_addon.py:65-79).
