@@ -189,12 +189,63 @@ __device__ __forceinline__ uint32_t rint_codes(u16 lo, u16 hi) {
   }
 }
 
-template <int T, int NCH, bool SMOOTH, int TH = AQ_THREADS>
+// One row with plain IEEE divisions, chunk by chunk from memory (no register cache, so that this
+// rarely taken path does not raise the register allocation of the kernels that call it).  Same
+// arithmetic as the generic kernel for a 16-bit compute dtype.  `red` holds TH / 64 floats.
+template <int T, int TH>
+__device__ __forceinline__ void quant_i8_row_ieee16(const u16* __restrict__ xr, const u16* __restrict__ smooth,
+                                                 int saturate, int8_t* __restrict__ qr, float* __restrict__ scale_out,
+                                                 int K, float* red) {
+  const int nchunk = K / AQ_VEC;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  auto chunk = [&](int c, float (&e)[8]) {
+    load8<T>(xr, (size_t)c * AQ_VEC, e);
+    if (smooth) {
+      float d[8];
+      load8<T>(smooth, (size_t)c * AQ_VEC, d);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) e[i] = round_to<T>(e[i] / d[i]);
+    }
+  };
+  float amax = 0.0f;
+#pragma unroll 1
+  for (int c = threadIdx.x; c < nchunk; c += TH) {
+    float e[8];
+    chunk(c, e);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(e[j]));
+  }
+  amax = wave_max(amax);
+  __syncthreads();
+  if (lane == 0) red[wave] = amax;
+  __syncthreads();
+  amax = red[0];
+#pragma unroll
+  for (int w = 1; w < TH / 64; ++w) amax = fmaxf(amax, red[w]);
+  __syncthreads();
+  const float s = round_to<T>(fmaxf(amax, round_to<T>(1e-5f)) / 127.0f);
+  if (threadIdx.x == 0) *scale_out = s;
+#pragma unroll 1
+  for (int c = threadIdx.x; c < nchunk; c += TH) {
+    float e[8];
+    chunk(c, e);
+    uint8_t b[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      float r = __builtin_rintf(round_to<T>(e[j] / s));
+      if (saturate) r = fminf(fmaxf(r, -127.0f), 127.0f);
+      b[j] = (uint8_t)(int)r;
+    }
+    store8((uint8_t*)qr, (size_t)c * AQ_VEC, b);
+  }
+}
+
+template <int T, int NCH, bool SMOOTH, int TH = AQ_THREADS, bool KEEP = true>
 __global__ __launch_bounds__(TH) void quant_i8_pertoken16_kernel(
     const u16* __restrict__ x, int64_t ldx, const u16* __restrict__ smooth, int saturate,
     int8_t* __restrict__ q, int64_t ldq, float* __restrict__ scale, int M, int K) {
   // reciprocals of the divisors stay in registers across rows while the row is short enough
-  constexpr bool KEEP_RCP = SMOOTH && NCH <= 4;
+  constexpr bool KEEP_RCP = SMOOTH && KEEP;
   __shared__ float red[2][TH / 64];
   const int nchunk = K / AQ_VEC;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -230,32 +281,34 @@ __global__ __launch_bounds__(TH) void quant_i8_pertoken16_kernel(
       if (c < nchunk) dst[i] = __builtin_nontemporal_load((const v4i*)(xr + (size_t)c * AQ_VEC));
     }
   };
-  // cur <- rnd_T(cur / smooth), packed.  FIX = plain IEEE divisions.  Without it the quotient of a
-  // zero / non-finite operand comes out NaN instead of its IEEE value; the caller detects that
-  // from the row maximum.
-  auto divide_row = [&](auto fix_tag) {
-    constexpr bool FIX = decltype(fix_tag)::value;
+  // cur <- rnd_T(cur / smooth), packed.  The quotient of a zero / non-finite operand comes out NaN
+  // instead of its IEEE value; the caller detects that from the row maximum.
+  auto divide_row = [&]() {
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
       const int c = threadIdx.x + i * TH;
       if (c < nchunk) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          const uint32_t w = (uint32_t)cur[i][j], d = (uint32_t)sm[i][j];
+          uint32_t d = (uint32_t)sm[i][j];
+          // long rows: keep the compiler from hoisting the 2 x NCH x 8 widened divisors and
+          // reciprocals out of the row loop (that costs 128 registers and halves the occupancy)
+          if constexpr (!KEEP_RCP) asm volatile("" : "+v"(d));
+          const uint32_t w = (uint32_t)cur[i][j];
           const float lo = cvt16<T>((u16)(w & 0xffff)), hi = cvt16<T>((u16)(w >> 16));
           const float dl = cvt16<T>((u16)(d & 0xffff)), dh = cvt16<T>((u16)(d >> 16));
-          float rl = 0.f, rh = 0.f;
-          if constexpr (FIX) {
-          } else if constexpr (KEEP_RCP) {
+          float rl, rh;
+          if constexpr (KEEP_RCP) {
             rl = sr[i][2 * j], rh = sr[i][2 * j + 1];
           } else {
             rl = __builtin_amdgcn_rcpf(dl), rh = __builtin_amdgcn_rcpf(dh);
           }
-          const u16 el = to16<T>(div16<T, FIX>(lo, dl, rl));
-          const u16 eh = to16<T>(div16<T, FIX>(hi, dh, rh));
+          const u16 el = to16<T>(div16<T, false>(lo, dl, rl));
+          const u16 eh = to16<T>(div16<T, false>(hi, dh, rh));
           cur[i][j] = (int)((uint32_t)el | ((uint32_t)eh << 16));
         }
       }
+      __builtin_amdgcn_sched_barrier(0);  // one chunk at a time: keeps the live ranges short
     }
   };
   // max |cur| over the row.  |e| is monotone in its bit pattern, so the maximum is taken on the
@@ -297,17 +350,19 @@ __global__ __launch_bounds__(TH) void quant_i8_pertoken16_kernel(
     const int nrow = row + gridDim.x;
     if (nrow < M) load_row(nrow, nxt);
 
-    if constexpr (SMOOTH) {
-      if (ieee_block) divide_row(std::true_type{});
-      else divide_row(std::false_type{});
+    uint32_t abits = INF_BITS;
+    if (!ieee_block) {
+      if constexpr (SMOOTH) divide_row();
+      abits = row_amax_bits();
     }
-    uint32_t abits = row_amax_bits();
-    if constexpr (SMOOTH) {
-      if (abits >= INF_BITS && !ieee_block) {  // zero / non-finite operands or overflow in the row
-        load_row(row, cur);
-        divide_row(std::true_type{});
-        abits = row_amax_bits();
-      }
+    if (abits >= INF_BITS) {
+      // divisors outside the fast path's range, zero / non-finite operands or overflow in the
+      // row: IEEE divisions, straight from memory (block-uniform branch)
+      quant_i8_row_ieee16<T, TH>(x + (size_t)row * ldx, SMOOTH ? smooth : nullptr, saturate,
+                                 q + (size_t)row * ldq, scale + row, K, red[0]);
+#pragma unroll
+      for (int i = 0; i < NCH; ++i) cur[i] = nxt[i];
+      continue;
     }
     const float amax = cvt16<T>((u16)abits);
 
@@ -317,8 +372,7 @@ __global__ __launch_bounds__(TH) void quant_i8_pertoken16_kernel(
     const float rs = __builtin_amdgcn_rcpf(s);
     if (threadIdx.x == 0) scale[row] = s;
     int8_t* qr = q + (size_t)row * ldq;
-    auto emit = [&](auto fix_tag) {
-      constexpr bool FIX = decltype(fix_tag)::value;
+    {
 #pragma unroll
       for (int i = 0; i < NCH; ++i) {
         const int c = threadIdx.x + i * TH;
@@ -327,8 +381,8 @@ __global__ __launch_bounds__(TH) void quant_i8_pertoken16_kernel(
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
             const uint32_t w = (uint32_t)cur[i][j];
-            float ql = div16<T, FIX>(cvt16<T>((u16)(w & 0xffff)), s, rs);
-            float qh = div16<T, FIX>(cvt16<T>((u16)(w >> 16)), s, rs);
+            float ql = div16<T, false>(cvt16<T>((u16)(w & 0xffff)), s, rs);
+            float qh = div16<T, false>(cvt16<T>((u16)(w >> 16)), s, rs);
             if (saturate) {  // clamp before rounding: the bounds are integers
               ql = fminf(fmaxf(ql, -sat_hi), sat_hi);
               qh = fminf(fmaxf(qh, -sat_hi), sat_hi);
@@ -340,10 +394,9 @@ __global__ __launch_bounds__(TH) void quant_i8_pertoken16_kernel(
           const uint32_t o1 = __builtin_amdgcn_perm(code[3], code[2], 0x06040200u);
           *(uint2*)(qr + (size_t)c * AQ_VEC) = make_uint2(o0, o1);
         }
+        __builtin_amdgcn_sched_barrier(0);
       }
-    };
-    if (abits < INF_BITS) emit(std::false_type{});
-    else emit(std::true_type{});
+    }
 #pragma unroll
     for (int i = 0; i < NCH; ++i) cur[i] = nxt[i];
   }
@@ -371,11 +424,11 @@ __device__ __forceinline__ float div32_fast(float x, float s, float r1) {
   return q;
 }
 
-template <int NCH, bool KEEP>
-__global__ __launch_bounds__(AQ_THREADS) void quant_i8_pertoken_f16x_f32s_kernel(
+template <int NCH, bool KEEP, int TH = AQ_THREADS>
+__global__ __launch_bounds__(TH) void quant_i8_pertoken_f16x_f32s_kernel(
     const u16* __restrict__ x, int64_t ldx, const float* __restrict__ smooth, int saturate,
     int8_t* __restrict__ q, int64_t ldq, float* __restrict__ scale, int M, int K) {
-  __shared__ float red[2][AQ_THREADS / 64];
+  __shared__ float red[2][TH / 64];
   const int nchunk = K / AQ_VEC;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 
@@ -385,7 +438,7 @@ __global__ __launch_bounds__(AQ_THREADS) void quant_i8_pertoken_f16x_f32s_kernel
   int bad = 0;
 #pragma unroll
   for (int i = 0; i < NCH; ++i) {
-    const int c = threadIdx.x + i * AQ_THREADS;
+    const int c = threadIdx.x + i * TH;
     if (c < nchunk) {
       const float4 a = *(const float4*)(smooth + (size_t)c * AQ_VEC);
       const float4 b = *(const float4*)(smooth + (size_t)c * AQ_VEC + 4);
@@ -409,7 +462,7 @@ __global__ __launch_bounds__(AQ_THREADS) void quant_i8_pertoken_f16x_f32s_kernel
     const u16* xr = x + (size_t)row * ldx;
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
-      const int c = threadIdx.x + i * AQ_THREADS;
+      const int c = threadIdx.x + i * TH;
       if (c < nchunk) dst[i] = __builtin_nontemporal_load((const v4i*)(xr + (size_t)c * AQ_VEC));
     }
   };
@@ -419,7 +472,7 @@ __global__ __launch_bounds__(AQ_THREADS) void quant_i8_pertoken_f16x_f32s_kernel
     float amax = 0.0f;
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
-      const int c = threadIdx.x + i * AQ_THREADS;
+      const int c = threadIdx.x + i * TH;
       if (c < nchunk) {
         float d[8];
         if constexpr (!KEEP || IEEE) {
@@ -449,8 +502,9 @@ __global__ __launch_bounds__(AQ_THREADS) void quant_i8_pertoken_f16x_f32s_kernel
     parity ^= 1;
     if (lane == 0) rb[wave] = __uint_as_float(b);
     __syncthreads();
-    const uint32_t r = max(max(__float_as_uint(rb[0]), __float_as_uint(rb[1])),
-                           max(__float_as_uint(rb[2]), __float_as_uint(rb[3])));
+    uint32_t r = __float_as_uint(rb[0]);
+#pragma unroll
+    for (int w = 1; w < TH / 64; ++w) r = max(r, __float_as_uint(rb[w]));
     return __uint_as_float(r);
   };
 
@@ -477,7 +531,7 @@ __global__ __launch_bounds__(AQ_THREADS) void quant_i8_pertoken_f16x_f32s_kernel
     int8_t* qr = q + (size_t)row * ldq;
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
-      const int c = threadIdx.x + i * AQ_THREADS;
+      const int c = threadIdx.x + i * TH;
       if (c < nchunk) {
         uint32_t o[2] = {0, 0};
 #pragma unroll
@@ -752,24 +806,24 @@ extern "C" int fmsmo_quant_act_i8_pertoken(const void* x, int x_dtype, int64_t l
       K <= AQ_MAXCHUNK * AQ_THREADS * AQ_VEC) {
     const int64_t per_thread = div_up(K, AQ_THREADS * AQ_VEC);
     const int nch = per_thread <= 1 ? 1 : per_thread <= 2 ? 2 : per_thread <= 4 ? 4 : 8;
-    // rows longer than 8192 elements without a SmoothQuant divide: 512-thread blocks with 4
-    // chunks per thread (measured 34 vs 38 us at K = 14336; with the divide the 256-thread
-    // shape is faster, 47 vs 69 us)
-#define LAUNCH16(T, NCH, SM, TH)                                                                 \
+    // rows longer than 8192 elements: 512-thread blocks with 4 chunks per thread (more, shorter
+    // lanes: 45 vs 49 us at K = 14336 with the SmoothQuant divide, 34 vs 38 us without)
+#define LAUNCH16(T, NCH, SM, TH, KEEP)                                                           \
   {                                                                                              \
     const int64_t resident =                                                                     \
-        resident_blocks((const void*)quant_i8_pertoken16_kernel<T, NCH, SM, TH>, TH);            \
+        resident_blocks((const void*)quant_i8_pertoken16_kernel<T, NCH, SM, TH, KEEP>, TH);      \
     dim3 grid16((unsigned)(M < resident ? M : resident)), block16(TH);                           \
-    hipLaunchKernelGGL((quant_i8_pertoken16_kernel<T, NCH, SM, TH>), grid16, block16, 0, st,     \
-                       (const u16*)x, ldx, (const u16*)smooth, saturate, q, ldq, scale, (int)M,  \
-                       (int)K);                                                                  \
+    hipLaunchKernelGGL((quant_i8_pertoken16_kernel<T, NCH, SM, TH, KEEP>), grid16, block16, 0,   \
+                       st, (const u16*)x, ldx, (const u16*)smooth, saturate, q, ldq, scale,      \
+                       (int)M, (int)K);                                                          \
   }
-#define PICK16(T)                                                                               \
-  switch (nch * 2 + (smooth ? 1 : 0)) {                                                         \
-    case 2: LAUNCH16(T, 1, false, 256); break;  case 3: LAUNCH16(T, 1, true, 256); break;      \
-    case 4: LAUNCH16(T, 2, false, 256); break;  case 5: LAUNCH16(T, 2, true, 256); break;      \
-    case 8: LAUNCH16(T, 4, false, 256); break;  case 9: LAUNCH16(T, 4, true, 256); break;      \
-    case 16: LAUNCH16(T, 4, false, 512); break; default: LAUNCH16(T, 8, true, 256); break;     \
+#define PICK16(T)                                                                                        \
+  switch (nch * 2 + (smooth ? 1 : 0)) {                                                                  \
+    case 2: LAUNCH16(T, 1, false, 256, true); break;  case 3: LAUNCH16(T, 1, true, 256, true); break;   \
+    case 4: LAUNCH16(T, 2, false, 256, true); break;  case 5: LAUNCH16(T, 2, true, 256, true); break;   \
+    case 8: LAUNCH16(T, 4, false, 256, true); break;  case 9: LAUNCH16(T, 4, true, 256, true); break;   \
+    case 16: LAUNCH16(T, 4, false, 512, true); break;                                                   \
+    default: LAUNCH16(T, 4, true, 512, false); break;                                                   \
   }
     if (x_dtype == FMSMO_F16) { PICK16(FMSMO_F16) } else { PICK16(FMSMO_BF16) }
 #undef PICK16
@@ -780,19 +834,19 @@ extern "C" int fmsmo_quant_act_i8_pertoken(const void* x, int x_dtype, int64_t l
   if (x_dtype == FMSMO_F16 && smooth && smooth_dtype == FMSMO_F32 && compute_dtype == FMSMO_F32 &&
       K <= AQ_MAXCHUNK * AQ_THREADS * AQ_VEC) {
     const int64_t per_thread = div_up(K, AQ_THREADS * AQ_VEC);
-    dim3 block32(AQ_THREADS);
-#define LAUNCH32(NCH, KEEP)                                                                       \
+#define LAUNCH32(NCH, KEEP, TH)                                                                   \
   {                                                                                               \
-    const int64_t resident = resident_blocks((const void*)quant_i8_pertoken_f16x_f32s_kernel<NCH, KEEP>); \
-    dim3 grid32((unsigned)(M < resident ? M : resident));                                         \
-    hipLaunchKernelGGL((quant_i8_pertoken_f16x_f32s_kernel<NCH, KEEP>), grid32, block32, 0, st,   \
-                       (const u16*)x, ldx, (const float*)smooth, saturate, q, ldq, scale, (int)M, \
-                       (int)K);                                                                   \
+    const int64_t resident =                                                                      \
+        resident_blocks((const void*)quant_i8_pertoken_f16x_f32s_kernel<NCH, KEEP, TH>, TH);      \
+    dim3 grid32((unsigned)(M < resident ? M : resident)), block32(TH);                            \
+    hipLaunchKernelGGL((quant_i8_pertoken_f16x_f32s_kernel<NCH, KEEP, TH>), grid32, block32, 0,   \
+                       st, (const u16*)x, ldx, (const float*)smooth, saturate, q, ldq, scale,     \
+                       (int)M, (int)K);                                                           \
   }
-    if (per_thread <= 1) LAUNCH32(1, true)
-    else if (per_thread <= 2) LAUNCH32(2, true)
-    else if (per_thread <= 4) LAUNCH32(4, false)
-    else LAUNCH32(8, false)
+    if (per_thread <= 1) LAUNCH32(1, true, 256)
+    else if (per_thread <= 2) LAUNCH32(2, true, 256)
+    else if (per_thread <= 4) LAUNCH32(4, false, 256)
+    else LAUNCH32(4, false, 512)
 #undef LAUNCH32
     return fmsmo_check_launch();
   }
