@@ -577,6 +577,113 @@ __global__ __launch_bounds__(AQ_THREADS) void quant_i8_static_kernel(
   }
 }
 
+// ------------------------------------------------------------------ int8, multiplicative scale
+// The quantize half of the W8A8 accelerator op: the scale is  levels / clip  as torch evaluates
+// "number / tensor", i.e. rnd_T( rnd_T(1 / clip) * levels )  (the reflected division of a Python
+// scalar by a tensor is reciprocal-then-multiply), and the codes are  rint( rnd_T( rnd_T(x / sq) * scale ) [- zp] ),  every
+// intermediate rounded to T as torch's elementwise kernels do.  Products of two 16-bit floats are
+// exact in fp32, so rounding the fp32 product to T is the correctly rounded T product.
+//   mode 0: per token, scale_m = 127 / max_k |x/sq|, codes clamped to +-127
+//   mode 1: per tensor symmetric, scale = 127 / clip[0], codes clamped to +-127
+//   mode 2: per tensor asymmetric, scale = 255 / (clip[0] - clip[1]), zp = clip[1] * scale, codes
+//           clamped to [0, 255] and stored minus 128
+// a_scale receives 1 / scale_m per row (mode 0) or { 1 / scale, zp } (modes 1 and 2).
+template <int T>
+__device__ __forceinline__ float levels_over(float levels, float clip) {
+  return round_to<T>(__fmul_rn(round_to<T>(1.0f / clip), levels));
+}
+
+template <int XT, int T>
+__global__ __launch_bounds__(AQ_THREADS) void quant_i8_mulscale_kernel(
+    const void* __restrict__ x, int64_t ldx, const void* __restrict__ smooth,
+    const void* __restrict__ clip, int meta_dtype, int mode, int8_t* __restrict__ q, int64_t ldq,
+    float* __restrict__ a_scale, int K) {
+  __shared__ float red[AQ_THREADS / 64];
+  const int row = blockIdx.x;
+  const size_t xrow = (size_t)row * ldx;
+  const int nchunk = K / AQ_VEC;
+  float v[AQ_MAXCHUNK][8];
+
+  auto meta = [&](const void* p, size_t i) {
+    return meta_dtype == FMSMO_F16 ? load_as_f32<FMSMO_F16>(p, i)
+           : meta_dtype == FMSMO_BF16 ? load_as_f32<FMSMO_BF16>(p, i)
+                                      : load_as_f32<FMSMO_F32>(p, i);
+  };
+  auto fetch = [&](int c, float (&e)[8]) {
+    load8<XT>(x, xrow + (size_t)c * AQ_VEC, e);
+    if (smooth) {
+      float d[8];
+      if (meta_dtype == FMSMO_F16) load8<FMSMO_F16>(smooth, (size_t)c * AQ_VEC, d);
+      else if (meta_dtype == FMSMO_BF16) load8<FMSMO_BF16>(smooth, (size_t)c * AQ_VEC, d);
+      else load8<FMSMO_F32>(smooth, (size_t)c * AQ_VEC, d);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) e[i] = round_to<T>(e[i] / d[i]);
+    }
+  };
+
+  float sx, zp = 0.0f, lo = -127.0f, hi = 127.0f, shift = 0.0f;
+  if (mode == 0) {
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < AQ_MAXCHUNK; ++i) {
+      const int c = threadIdx.x + i * AQ_THREADS;
+      if (c < nchunk) {
+        fetch(c, v[i]);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(v[i][j]));
+      }
+    }
+    for (int c = threadIdx.x + AQ_MAXCHUNK * AQ_THREADS; c < nchunk; c += AQ_THREADS) {
+      float e[8];
+      fetch(c, e);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(e[j]));
+    }
+    amax = block_max(amax, red);
+    // a row of zeros has no scale (127 / 0): it is quantized to zeros with a zero output scale
+    sx = amax > 0.0f ? levels_over<T>(127.0f, amax) : 0.0f;
+    if (threadIdx.x == 0) a_scale[row] = (sx > 0.0f) ? 1.0f / sx : 0.0f;
+  } else {
+#pragma unroll
+    for (int i = 0; i < AQ_MAXCHUNK; ++i) {
+      const int c = threadIdx.x + i * AQ_THREADS;
+      if (c < nchunk) fetch(c, v[i]);
+    }
+    const float cv = meta(clip, 0);
+    if (mode == 1) {
+      sx = levels_over<T>(127.0f, cv);
+    } else {
+      const float cvn = meta(clip, 1);
+      sx = levels_over<T>(255.0f, round_to<T>(__fsub_rn(cv, cvn)));
+      zp = round_to<T>(__fmul_rn(cvn, sx));
+      lo = 0.0f; hi = 255.0f; shift = 128.0f;
+    }
+    if (row == 0 && threadIdx.x == 0) { a_scale[0] = 1.0f / sx; a_scale[1] = zp; }
+  }
+
+  auto emit = [&](int c, const float (&e)[8]) {
+    uint8_t b[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      float t = round_to<T>(__fmul_rn(e[j], sx));
+      if (mode == 2) t = round_to<T>(__fsub_rn(t, zp));
+      t = fminf(fmaxf(__builtin_rintf(t), lo), hi) - shift;
+      b[j] = (uint8_t)(int)t;
+    }
+    store8((uint8_t*)q, (size_t)row * ldq + (size_t)c * AQ_VEC, b);
+  };
+#pragma unroll
+  for (int i = 0; i < AQ_MAXCHUNK; ++i) {
+    const int c = threadIdx.x + i * AQ_THREADS;
+    if (c < nchunk) emit(c, v[i]);
+  }
+  for (int c = threadIdx.x + AQ_MAXCHUNK * AQ_THREADS; c < nchunk; c += AQ_THREADS) {
+    float e[8];
+    fetch(c, e);
+    emit(c, e);
+  }
+}
+
 // ------------------------------------------------------------------ e4m3, per token
 template <int XT>
 __global__ __launch_bounds__(AQ_THREADS) void quant_fp8_pertoken_kernel(
@@ -887,6 +994,44 @@ extern "C" int fmsmo_quant_act_i8_static(const void* x, int x_dtype, int64_t ldx
     case FMSMO_F16: LAUNCH(FMSMO_F16); break;
     case FMSMO_BF16: LAUNCH(FMSMO_BF16); break;
     default: LAUNCH(FMSMO_F32); break;
+  }
+#undef LAUNCH
+  return fmsmo_check_launch();
+}
+
+extern "C" int fmsmo_quant_act_i8_mulscale(const void* x, int x_dtype, int64_t ldx,
+                                           const void* smooth, const void* clip, int meta_dtype,
+                                           int compute_dtype, int mode, int8_t* q, int64_t ldq,
+                                           float* a_scale, int64_t M, int64_t K,
+                                           fmsmo_stream_t stream) {
+  if (!x || !q || !a_scale) return FMSMO_ERR_NULL;
+  if (mode < 0 || mode > 2) return FMSMO_ERR_UNSUPPORTED;
+  if (mode != 0 && !clip) return FMSMO_ERR_NULL;
+  if (M < 0 || K <= 0 || ldx < K || ldq < K || M > 0x7fffffff || K > 0x7fffffff) return FMSMO_ERR_SHAPE;
+  if (x_dtype < 0 || x_dtype > 2 || meta_dtype < 0 || meta_dtype > 2 || compute_dtype < 0 ||
+      compute_dtype > 2)
+    return FMSMO_ERR_UNSUPPORTED;
+  // the compute dtype is the promotion of x's and the metadata's dtype, as torch would choose it
+  if (compute_dtype != FMSMO_F32 && compute_dtype != x_dtype) return FMSMO_ERR_UNSUPPORTED;
+  if (K % 8 || ldx % 8 || ldq % 8 || !aligned16(x) || (((uintptr_t)q) & 7) ||
+      (smooth && !aligned16(smooth)))
+    return FMSMO_ERR_ALIGN;
+  if (M == 0) return FMSMO_OK;
+  hipStream_t st = (hipStream_t)stream;
+  dim3 grid((unsigned)M), block(AQ_THREADS);
+#define LAUNCH(XT, T)                                                                        \
+  hipLaunchKernelGGL((quant_i8_mulscale_kernel<XT, T>), grid, block, 0, st, x, ldx, smooth,  \
+                     clip, meta_dtype, mode, q, ldq, a_scale, (int)K)
+  if (compute_dtype == FMSMO_F32) {
+    switch (x_dtype) {
+      case FMSMO_F16: LAUNCH(FMSMO_F16, FMSMO_F32); break;
+      case FMSMO_BF16: LAUNCH(FMSMO_BF16, FMSMO_F32); break;
+      default: LAUNCH(FMSMO_F32, FMSMO_F32); break;
+    }
+  } else if (x_dtype == FMSMO_F16) {
+    LAUNCH(FMSMO_F16, FMSMO_F16);
+  } else {
+    LAUNCH(FMSMO_BF16, FMSMO_BF16);
   }
 #undef LAUNCH
   return fmsmo_check_launch();

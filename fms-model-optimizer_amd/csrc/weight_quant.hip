@@ -104,6 +104,34 @@ __global__ __launch_bounds__(256) void absmax_cols_kernel(const void* __restrict
   for (int i = 0; i < 8; ++i) atomicMax(out + k0 + i, __float_as_uint(best[i]));
 }
 
+// Bias with the zero-point correction of asymmetric activations folded in:
+//   out_n = bias_n + (offset + a_meta[1]) * (sum_k w_nk) * a_meta[0] * w_scale_n
+// a_meta = { 1 / activation scale, activation zero point } as left on the device by the
+// activation quantizer; one wavefront per weight row, 16-byte loads, integer row sums.
+__global__ __launch_bounds__(256) void zero_shift_bias_kernel(
+    const int8_t* __restrict__ w, int64_t ldw, const float* __restrict__ w_scale, int w_scale_n,
+    const float* __restrict__ a_meta, float offset, const void* __restrict__ bias, int bias_dtype,
+    float* __restrict__ out, int N, int K) {
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= N) return;
+  int sum = 0;
+  for (int k0 = lane * 16; k0 < K; k0 += 64 * 16) {
+    const uint4 r = *(const uint4*)(w + (size_t)row * ldw + k0);
+    sum = __builtin_amdgcn_sdot4((int)r.x, 0x01010101, sum, false);
+    sum = __builtin_amdgcn_sdot4((int)r.y, 0x01010101, sum, false);
+    sum = __builtin_amdgcn_sdot4((int)r.z, 0x01010101, sum, false);
+    sum = __builtin_amdgcn_sdot4((int)r.w, 0x01010101, sum, false);
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o, 64);
+  if (lane == 0) {
+    const float b = bias ? load_dyn(bias, bias_dtype, row) : 0.0f;
+    const float ws = w_scale[w_scale_n > 1 ? row : 0];
+    out[row] = b + (offset + a_meta[1]) * (float)sum * a_meta[0] * ws;
+  }
+}
+
 }  // namespace fmsmo
 
 using namespace fmsmo;
@@ -140,6 +168,21 @@ extern "C" int fmsmo_quant_weight_i8(const void* w, int w_dtype, int64_t ldw, co
     default: LAUNCH(FMSMO_F32); break;
   }
 #undef LAUNCH
+  return fmsmo_check_launch();
+}
+
+extern "C" int fmsmo_zero_shift_bias(const int8_t* w, int64_t ldw, const float* w_scale,
+                                     int64_t w_scale_n, const float* a_meta, float offset,
+                                     const void* bias, int bias_dtype, float* out, int64_t N,
+                                     int64_t K, fmsmo_stream_t stream) {
+  if (!w || !w_scale || !a_meta || !out) return FMSMO_ERR_NULL;
+  if (N <= 0 || K <= 0 || ldw < K || N > 0x7fffffff || K > 0x7fffffff) return FMSMO_ERR_SHAPE;
+  if (w_scale_n != 1 && w_scale_n != N) return FMSMO_ERR_SHAPE;
+  if (bias && (bias_dtype < 0 || bias_dtype > 2)) return FMSMO_ERR_UNSUPPORTED;
+  if (K % 16 || ldw % 16 || (((uintptr_t)w) & 15)) return FMSMO_ERR_ALIGN;
+  hipLaunchKernelGGL(zero_shift_bias_kernel, dim3((unsigned)div_up(N, 4)), dim3(256), 0,
+                     (hipStream_t)stream, w, ldw, w_scale, (int)w_scale_n, a_meta, offset, bias,
+                     bias_dtype, out, (int)N, (int)K);
   return fmsmo_check_launch();
 }
 

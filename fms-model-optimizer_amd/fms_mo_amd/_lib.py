@@ -19,6 +19,7 @@ OP_I8, OP_E4M3, OP_F16, OP_BF16, OP_F32 = 0, 1, 2, 3, 4
 EPI_REF_F16, EPI_F32 = 0, 1
 FP8_LINEAR, FP8_FPXACC, FP8_FPXACC_DL8 = 0, 1, 2
 WQ_MUL, WQ_DIV = 0, 1
+MS_PER_TOKEN, MS_SYMM, MS_ASYMM = 0, 1, 2
 ABI_VERSION = 1
 
 _P, _I, _L, _F = c_void_p, c_int, c_int64, c_float
@@ -27,6 +28,7 @@ _P, _I, _L, _F = c_void_p, c_int, c_int64, c_float
 SIGNATURES = {
     "fmsmo_quant_act_i8_pertoken": [_P, _I, _L, _P, _I, _I, _I, _P, _L, _P, _L, _L, _P],
     "fmsmo_quant_act_i8_static": [_P, _I, _L, _F, _I, _I, _P, _L, _L, _L, _P],
+    "fmsmo_quant_act_i8_mulscale": [_P, _I, _L, _P, _P, _I, _I, _I, _P, _L, _P, _L, _L, _P],
     "fmsmo_quant_act_fp8_pertoken": [_P, _I, _L, _I, _I, _P, _L, _P, _L, _L, _P],
     "fmsmo_gemm_i8_i32": [_P, _L, _P, _L, _P, _L, _L, _L, _L, _P],
     "fmsmo_gemm_i8_dq": [_P, _L, _P, _L, _P, _L, _P, _L, _P, _I, _I, _P, _I, _L, _L, _L, _L, _P],
@@ -39,6 +41,7 @@ SIGNATURES = {
                                  _L, _L, _P],
     "fmsmo_quant_weight_i8": [_P, _I, _L, _P, _I, _P, _I, _L, _I, _P, _L, _P, _L, _L, _P],
     "fmsmo_absmax_cols": [_P, _I, _L, _L, _L, _P, _P],
+    "fmsmo_zero_shift_bias": [_P, _L, _P, _L, _P, _F, _P, _I, _P, _L, _L, _P],
 }
 OTHER = {
     "fmsmo_abi_version": ([], c_int),

@@ -93,6 +93,39 @@ def quant_act_i8_static(x, scale: float, zp: int, sym: int):
     return q
 
 
+def quant_act_i8_mulscale(x, mode, clip=None, smooth=None, meta_dtype=None):
+    """(q int8 [M,K], a_scale fp32 [M] or [2]) -- see fmsmo_quant_act_i8_mulscale.  clip: device
+    tensor {a_clip_val, a_clip_valn}; smooth: device tensor [K]; both of one dtype.  meta_dtype:
+    dtype of the metadata vector when neither is passed (it still decides the compute dtype)."""
+    _need_gpu(x, clip, smooth)
+    x = _rows(x)
+    M, K = x.shape
+    meta = smooth if smooth is not None else clip
+    if clip is not None and smooth is not None and clip.dtype != smooth.dtype:
+        raise TypeError("clip and smooth must share one dtype")
+    if mode != L.MS_PER_TOKEN:
+        if clip is None or clip.numel() != 2:
+            raise ValueError("clip must hold {a_clip_val, a_clip_valn}")
+        clip = clip.detach().reshape(-1).contiguous()
+    if smooth is not None:
+        smooth = smooth.detach().reshape(-1).contiguous()
+        if smooth.numel() != K:
+            raise ValueError("smooth scale must have K elements")
+        if smooth.data_ptr() % 16:
+            smooth = smooth.clone()
+    if meta is not None:
+        meta_dtype = meta.dtype
+    compute_dtype = x.dtype if meta_dtype is None else torch.promote_types(x.dtype, meta_dtype)
+    q = torch.empty((M, K), dtype=torch.int8, device=x.device)
+    a_scale = torch.empty((M if mode == L.MS_PER_TOKEN else 2,), dtype=torch.float32,
+                          device=x.device)
+    with torch.cuda.device(x.device):
+        L.call("fmsmo_quant_act_i8_mulscale", x.data_ptr(), _dt(x), _ld(x), _ptr(smooth),
+               _ptr(clip), _DT[meta_dtype] if meta_dtype is not None else _dt(x), _DT[compute_dtype],
+               int(mode), q.data_ptr(), K, a_scale.data_ptr(), M, K, _stream(x))
+    return q, a_scale
+
+
 def quant_act_fp8_pertoken(x, variant=L.FP8_LINEAR, static_scale=None):
     """(q e4m3 [M,K], scale fp32 [M] or the [1] static scale)."""
     _need_gpu(x)
@@ -281,3 +314,26 @@ def absmax_cols(x, running=None):
     with torch.cuda.device(x.device):
         L.call("fmsmo_absmax_cols", x.data_ptr(), _dt(x), _ld(x), M, K, running.data_ptr(), _stream(x))
     return running
+
+
+def zero_shift_bias(w, w_scale, a_meta, bias=None, offset=128.0):
+    """fp32 [N] bias with the zero-point correction of asymmetric activations folded in
+    (see fmsmo_zero_shift_bias).  w int8 [N,K]; w_scale fp32 [N] or [1]; a_meta fp32 [2]."""
+    _need_gpu(w, w_scale, a_meta, bias)
+    if w.dtype != torch.int8:
+        raise TypeError("w must be int8")
+    w = _rows(w)
+    N, K = w.shape
+    w_scale = _scale_vec(w_scale, N, w.device, "w_scale")
+    if a_meta.dtype != torch.float32 or a_meta.numel() != 2:
+        raise ValueError("a_meta must be fp32 {1/scale, zero point}")
+    if bias is not None:
+        bias = bias.detach().reshape(-1).contiguous()
+        if bias.numel() != N:
+            raise ValueError("bias must have N elements")
+    out = torch.empty((N,), dtype=torch.float32, device=w.device)
+    with torch.cuda.device(w.device):
+        L.call("fmsmo_zero_shift_bias", w.data_ptr(), _ld(w), w_scale.data_ptr(), w_scale.numel(),
+               a_meta.contiguous().data_ptr(), float(offset), _ptr(bias),
+               _dt(bias) if bias is not None else 0, out.data_ptr(), N, K, _stream(w))
+    return out

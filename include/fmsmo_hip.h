@@ -98,6 +98,30 @@ int fmsmo_quant_act_i8_static(const void* x, int x_dtype, int64_t ldx, float sca
                               int sym, int8_t* q, int64_t ldq, int64_t M, int64_t K,
                               fmsmo_stream_t stream);
 
+/*
+ * int8 quantizers with a multiplicative scale (the quantize half of the accelerator op
+ * fms_mo::i8i8_aiu).  T = compute_dtype is torch's promotion of x's dtype and the metadata's
+ * (meta_dtype: dtype of smooth and clip); every intermediate is rounded to T.
+ *   x' = smooth ? rnd_T(x / smooth[k]) : x
+ *   L / c below is torch's "number / tensor" = rnd_T( rnd_T(1 / c) * L ) (reciprocal, then multiply)
+ *   FMSMO_MS_PER_TOKEN : s_m = 127 / max_k|x'_mk|;   q = clamp(rint(rnd_T(x' s_m)), -127, 127)
+ *   FMSMO_MS_SYMM      : s = 127 / clip[0];          q = clamp(rint(rnd_T(x' s)), -127, 127)
+ *   FMSMO_MS_ASYMM     : s = 255 / rnd_T(clip[0] - clip[1]);  zp = rnd_T(clip[1] s);
+ *                        u = clamp(rint(rnd_T(rnd_T(x' s) - zp)), 0, 255);  q = u - 128
+ * clip: device pointer to { a_clip_val, a_clip_valn } (unused for per-token; nothing is read on
+ * the host, so the call can be captured in a HIP graph).
+ * a_scale (fp32, device): per token [M] <- 1 / s_m;  otherwise [2] <- { 1 / s, zp }.
+ * The dequantized activation of the reference is then (q [+ 128 + zp]) * a_scale * smooth[k].
+ * A row of zeros (s_m = 127/0) is quantized to zeros with a_scale 0; the reference produces NaN.
+ * x and smooth 16-byte aligned, K and ldx multiples of 8 elements.
+ * Reference: quant_dequant_activ (fms_mo/aiu_addons/i8i8/i8i8_aiu_op.py:203-231).
+ */
+enum { FMSMO_MS_PER_TOKEN = 0, FMSMO_MS_SYMM = 1, FMSMO_MS_ASYMM = 2 };
+int fmsmo_quant_act_i8_mulscale(const void* x, int x_dtype, int64_t ldx, const void* smooth,
+                                const void* clip, int meta_dtype, int compute_dtype, int mode,
+                                int8_t* q, int64_t ldq, float* a_scale, int64_t M, int64_t K,
+                                fmsmo_stream_t stream);
+
 /* Variants of the per-token FP8 (OCP e4m3fn) activation quantizer. */
 enum {
   /* s_m = max(amax_m/448, 1e-12) in fp32; q = e4m3( clamp(f32(x)/s_m, -448, 448) ).
@@ -255,6 +279,21 @@ int fmsmo_quant_weight_i8(const void* w, int w_dtype, int64_t ldw, const void* s
  */
 int fmsmo_absmax_cols(const void* x, int x_dtype, int64_t ldx, int64_t M, int64_t K, float* out,
                       fmsmo_stream_t stream);
+
+/*
+ * Bias with the zero-point correction of asymmetric per-tensor activations folded in, for use
+ * as the bias of fmsmo_gemm_i8_dq when the activation codes are stored minus `offset`:
+ *   out[n] = bias[n] + (offset + a_meta[1]) * (sum_k w[n,k]) * a_meta[0] * w_scale[n]
+ * a_meta: device fp32 { 1 / activation scale, zero point }, as written by
+ * fmsmo_quant_act_i8_mulscale(FMSMO_MS_ASYMM); bias may be NULL; out: fp32 [N].
+ * w 16-byte aligned, K and ldw multiples of 16.
+ * Reference: the (x_int + zp_x) / scale_x dequantization of quant_dequant_activ
+ * (fms_mo/aiu_addons/i8i8/i8i8_aiu_op.py:219-223) multiplied out over the integer GEMM; the
+ * integer row sums are the zero_shift of process_zero_shift (fms_mo/utils/aiu_utils.py:282-333).
+ */
+int fmsmo_zero_shift_bias(const int8_t* w, int64_t ldw, const float* w_scale, int64_t w_scale_n,
+                          const float* a_meta, float offset, const void* bias, int bias_dtype,
+                          float* out, int64_t N, int64_t K, fmsmo_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -21,7 +21,8 @@ How each function is pinned (see tests/test_oracle_*.py):
                            (C restatement, all exponent classes, NaN/Inf)
   * fp8 cast            -- all 256 codes and all midpoints against torch's own cast
   * i8i8_aiu            -- the six stored vectors of the reference's own test-suite
-                           (tests/golden/ref_w-*_a-*_sq-N.pt)
+                           (tests/golden/ref_w-*_a-*_sq-N.pt); its SmoothQuant branch, which no
+                           stored vector exercises, by exactness under power-of-two scales
   * AIU checkpoint conversion, column abs-max
                         -- closed forms (sqrt(a)/sqrt(wmax) at alpha = 0.5, rint(127 W s / cv) away
                            from ties), invariants (|q| <= 127, zero shift = integer row sums)
@@ -360,6 +361,25 @@ def fp8_linear_forward(x, w_e4m3, weight_scale, bias=None, input_scale=None):
 # ------------------------------------------------------------------------------------------
 # fms_mo::i8i8_aiu (the op the reference's stored vectors exercise)
 # ------------------------------------------------------------------------------------------
+def i8i8_aiu_quant_act(x, a_cv, a_cvn, sq, activ_quant_type):
+    """Quantize step of quant_dequant_activ (fms_mo/aiu_addons/i8i8/i8i8_aiu_op.py:203-231):
+    returns (x_int, scale_x, zp_x) in the promoted dtype; x_int holds integers in [-127,127]
+    or, for per_tensor_asymm, [0,255]."""
+    if activ_quant_type == "per_tensor_symm":
+        scale_x = 127 / a_cv
+        return torch.round(x / sq * scale_x).clamp(-127, 127), scale_x, None
+    if activ_quant_type == "per_tensor_asymm":
+        scale_x = 255 / (a_cv - a_cvn)
+        zp_x = a_cvn * scale_x
+        return torch.round(x / sq * scale_x - zp_x).clamp(0, 255), scale_x, zp_x
+    if activ_quant_type == "per_token":
+        x_sq = x / sq
+        a_cv_tok = x_sq.abs().max(dim=-1, keepdim=True)[0]
+        scale_x = 127 / a_cv_tok
+        return torch.round(x_sq * scale_x).clamp(-127, 127), scale_x, None
+    raise NotImplementedError(activ_quant_type)
+
+
 def i8i8_aiu(x, weight, bias, qdata, weight_quant_type, activ_quant_type, smoothquant):
     """fms_mo/aiu_addons/i8i8/i8i8_aiu_op.py:86-231."""
     dtype = x.dtype
@@ -378,23 +398,11 @@ def i8i8_aiu(x, weight, bias, qdata, weight_quant_type, activ_quant_type, smooth
         raise ValueError(f"qdata length ({len(qdata)}) does not match {i6}")
     w_cv, _, a_cv, a_cvn, _, sq = torch.tensor_split(qdata, (i1, i2, i3, i4, i5))
 
-    if activ_quant_type == "per_tensor_symm":
-        scale_x = 127 / a_cv
-        x_int = torch.round(x / sq * scale_x).clamp(-127, 127).to(torch.int8)
-        x_dq = x_int.div(scale_x).mul(sq)
-    elif activ_quant_type == "per_tensor_asymm":
-        scale_x = 255 / (a_cv - a_cvn)
-        zp_x = a_cvn * scale_x
-        x_int = torch.round(x / sq * scale_x - zp_x).clamp(0, 255)
+    x_int, scale_x, zp_x = i8i8_aiu_quant_act(x, a_cv, a_cvn, sq, activ_quant_type)
+    if activ_quant_type == "per_tensor_asymm":
         x_dq = x_int.add(zp_x).div(scale_x).mul(sq)
-    elif activ_quant_type == "per_token":
-        x_sq = x / sq
-        a_cv_tok = x_sq.abs().max(dim=-1, keepdim=True)[0]
-        scale_x = 127 / a_cv_tok
-        x_int = torch.round(x_sq * scale_x).clamp(-127, 127)
-        x_dq = x_int.div(scale_x).mul(sq)
     else:
-        raise NotImplementedError(activ_quant_type)
+        x_dq = x_int.div(scale_x).mul(sq)
 
     if weight_quant_type == "per_tensor":
         w_dq = (weight * w_cv / 127) / sq

@@ -48,3 +48,26 @@ def test_per_token_vectors_also_pin_the_integer_path(path):
     ref = d["reference_out"].reshape(-1, n).float()
     # the stored outputs went through fp16 operands and an fp16 F.linear (ulp 0.008 at |y| = 8)
     assert torch.all((y - ref).abs() < 5e-3 + 2e-3 * ref.abs())
+
+
+@pytest.mark.parametrize("path", GOLDEN, ids=[os.path.basename(p) for p in GOLDEN])
+def test_smoothquant_branch_by_power_of_two_invariance(path):
+    """The stored vectors all have SmoothQuant off.  With a power-of-two scale per input channel
+    every division and multiplication by it is exact, so feeding x * sq together with sq must give
+    the stored outputs again, bit for bit at the quantize step and to the same tolerance at the
+    output: a dropped, transposed or doubly applied scale fails this."""
+    d = torch.load(path, weights_only=True)
+    x = d["x"].to(torch.float16)
+    k = x.shape[-1]
+    sq = torch.tensor([2.0 ** e for e in [-2, 1, 0, 3, -1, 2, -3, 1, 0, 2][:k]], dtype=torch.float16)
+    qdata = torch.cat((d["qdata"].to(torch.float16)[:-1], sq))
+    out = O.i8i8_aiu(x * sq, d["w_int"], d["bias"], qdata, d["weight_quant_type"],
+                     d["activ_quant_type"], True)
+    assert torch.all((out - d["reference_out"]).abs() < 1e-4)
+    n = d["w_int"].shape[0]
+    i1 = n if d["weight_quant_type"] == "per_channel" else 1
+    a_cv, a_cvn = qdata[2 * i1: 2 * i1 + 1], qdata[2 * i1 + 1: 2 * i1 + 2]
+    q_plain, _, _ = O.i8i8_aiu_quant_act(x, a_cv, a_cvn, torch.ones(1, dtype=torch.float16),
+                                         d["activ_quant_type"])
+    q_sq, _, _ = O.i8i8_aiu_quant_act(x * sq, a_cv, a_cvn, sq, d["activ_quant_type"])
+    assert torch.equal(q_plain, q_sq)
