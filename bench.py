@@ -263,6 +263,40 @@ def extras(torch, K, dev):
         ms = timeit(lambda: K.matmul_chunk(a, w, chunk_size=64, chunk_trun_bits=t), iters=10, warm=3)
         tops = 2.0 * m_e * I * H / (ms * 1e-3) / 1e12
         res[f"chunk64_trunc{t}_i8_w2_M{m_e}"] = {"ms": round(ms, 4), "tops": round(tops, 1), "frac_peak": round(tops / PEAK_INT8_TOPS, 4)}
+    # the steps either side of the hot path: offline weight quantizer, SmoothQuant statistics, the
+    # accelerator op's quantizer (HBM bound; inputs rotated so the Infinity Cache cannot hold them)
+    # and the accelerator op end to end
+    n, k = 28672, 4096
+    ws = [(0.02 * torch.randn(n, k, device=dev)).half() for _ in range(2)]
+    coef = (127.0 / ws[0].float().abs().amax(dim=1)).float()
+    smooth = (torch.rand(k, device=dev) + 0.5).half()
+    it = iter(range(10 ** 9))
+    ms = timeit(lambda: K.quant_weight_i8(ws[next(it) % 2], coef, smooth=smooth, mode="mul", want_row_sum=True), iters=10, warm=2)
+    gbs = n * k * 3 / (ms * 1e-3) / 1e9
+    res["offline_weight_quant_fp16_gate_up"] = {"ms": round(ms, 4), "GBps": round(gbs, 1), "frac_hbm": round(gbs / PEAK_HBM_GBS, 4)}
+    del ws
+    M, k = 4096, 14336
+    xs = [torch.randn(M, k, device=dev).half() for _ in range(3)]
+    run = torch.zeros(k, device=dev)
+    ms = timeit(lambda: K.absmax_cols(xs[next(it) % 3], run), iters=12, warm=3)
+    gbs = M * k * 2 / (ms * 1e-3) / 1e9
+    res["smoothquant_stats_absmax_cols_M4096_K14336"] = {"us": round(ms * 1e3, 1), "GBps": round(gbs, 1), "frac_hbm": round(gbs / PEAK_HBM_GBS, 4)}
+    sm = (torch.rand(k, device=dev) + 0.5).half()
+    clip = torch.tensor([3.0, -2.0], device=dev).half()
+    for mode, label in ((L.MS_PER_TOKEN, "per_token"), (L.MS_ASYMM, "per_tensor_asymm")):
+        ms = timeit(lambda: K.quant_act_i8_mulscale(xs[next(it) % 3], mode, clip=None if mode == L.MS_PER_TOKEN else clip, smooth=sm), iters=12, warm=3)
+        gbs = M * k * 3 / (ms * 1e-3) / 1e9
+        res[f"aiu_act_quant_{label}_smooth_M4096_K14336"] = {"us": round(ms * 1e3, 1), "GBps": round(gbs, 1), "frac_hbm": round(gbs / PEAK_HBM_GBS, 4)}
+    from fms_mo_amd.aiu_addons.i8i8.i8i8_aiu_op import i8i8_aiu
+    n = 4096
+    w = torch.randint(-127, 128, (n, k), dtype=torch.int8, device=dev)
+    bias = torch.zeros(n, device=dev).half()
+    for act in ("per_token", "per_tensor_asymm"):
+        zs = torch.zeros(n if act == "per_tensor_asymm" else 1, device=dev).half()
+        qdata = torch.cat((torch.full((n,), 0.3, device=dev).half(), torch.full((n,), -0.3, device=dev).half(), clip, zs, sm))
+        ms = timeit(lambda: i8i8_aiu(xs[0], w, bias, qdata, "per_channel", act, True), iters=10, warm=3)
+        tops = 2.0 * M * k * n / (ms * 1e-3) / 1e12
+        res[f"i8i8_aiu_op_{act}_down_M4096"] = {"ms": round(ms, 4), "tops": round(tops, 1), "frac_peak": round(tops / PEAK_INT8_TOPS, 4)}
     return res
 
 

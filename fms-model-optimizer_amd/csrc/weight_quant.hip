@@ -10,6 +10,8 @@
 // stores; read 2-4 B and write 1 B per element (HBM bound, offline).
 #include "common.hpp"
 
+#include <type_traits>
+
 namespace fmsmo {
 
 __device__ __forceinline__ float round_dyn(float v, int t) {
@@ -21,6 +23,23 @@ __device__ __forceinline__ float load_dyn(const void* p, int t, size_t i) {
                            : ((const float*)p)[i];
 }
 
+// 8 consecutive elements of a dtype known at run time, widened to fp32
+__device__ __forceinline__ void load8_dyn(const void* p, int t, size_t i, float (&v)[8]) {
+  if (t == FMSMO_F32) {
+    const float4 a = *(const float4*)((const float*)p + i);
+    const float4 b = *(const float4*)((const float*)p + i + 4);
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+  } else {
+    const uint4 r = *(const uint4*)((const u16*)p + i);
+    const uint32_t ww[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const u16 h = (u16)(ww[j >> 1] >> ((j & 1) * 16));
+      v[j] = t == FMSMO_F16 ? f16_to_f32(h) : bf16_to_f32(h);
+    }
+  }
+}
+
 template <int WT>
 __global__ __launch_bounds__(256) void quant_weight_i8_kernel(
     const void* __restrict__ w, int64_t ldw, const void* __restrict__ smooth, int smooth_dtype,
@@ -30,37 +49,57 @@ __global__ __launch_bounds__(256) void quant_weight_i8_kernel(
   const int row = blockIdx.x;
   const float c = load_dyn(coef, coef_dtype, coef_stride ? row : 0);
   int sum = 0;
-  for (int k0 = threadIdx.x * 8; k0 < K; k0 += 256 * 8) {
-    float v[8];
-    if constexpr (WT == FMSMO_F32) {
-      const float4 a = *(const float4*)((const float*)w + (size_t)row * ldw + k0);
-      const float4 b = *(const float4*)((const float*)w + (size_t)row * ldw + k0 + 4);
-      v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
-    } else {
-      const uint4 r = *(const uint4*)((const u16*)w + (size_t)row * ldw + k0);
-      const uint32_t ww[4] = {r.x, r.y, r.z, r.w};
+  constexpr int U = 4;  // 16-byte groups in flight per thread
+  typedef typename std::conditional<WT == FMSMO_F32, float4, uint4>::type Raw;
+  for (int kb = threadIdx.x * 8; kb < K; kb += U * 256 * 8) {
+    Raw ra[U], rb[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int k0 = kb + u * 256 * 8;
+      if (k0 < K) {
+        if constexpr (WT == FMSMO_F32) {
+          ra[u] = *(const float4*)((const float*)w + (size_t)row * ldw + k0);
+          rb[u] = *(const float4*)((const float*)w + (size_t)row * ldw + k0 + 4);
+        } else {
+          ra[u] = *(const uint4*)((const u16*)w + (size_t)row * ldw + k0);
+        }
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int k0 = kb + u * 256 * 8;
+      if (k0 >= K) break;
+      float v[8];
+      if constexpr (WT == FMSMO_F32) {
+        v[0] = ra[u].x; v[1] = ra[u].y; v[2] = ra[u].z; v[3] = ra[u].w;
+        v[4] = rb[u].x; v[5] = rb[u].y; v[6] = rb[u].z; v[7] = rb[u].w;
+      } else {
+        const uint32_t ww[4] = {ra[u].x, ra[u].y, ra[u].z, ra[u].w};
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const u16 h = (u16)(ww[i >> 1] >> ((i & 1) * 16));
+          v[i] = WT == FMSMO_F16 ? f16_to_f32(h) : bf16_to_f32(h);
+        }
+      }
+      float sm[8];
+      if (smooth) load8_dyn(smooth, smooth_dtype, (size_t)k0, sm);
+      uint32_t o[2] = {0, 0};
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
-        const u16 h = (u16)(ww[i >> 1] >> ((i & 1) * 16));
-        v[i] = WT == FMSMO_F16 ? f16_to_f32(h) : bf16_to_f32(h);
+        float t = v[i];
+        if (smooth) t = round_dyn(__fmul_rn(t, sm[i]), t1);
+        float r;
+        if (mode == FMSMO_WQ_MUL) {
+          r = __builtin_rintf(fminf(fmaxf(round_dyn(__fmul_rn(c, t), t2), -127.0f), 127.0f));
+        } else {
+          r = fminf(fmaxf(__builtin_rintf(round_dyn(t / c, t2)), -127.0f), 127.0f);
+        }
+        const int qi = (int)r;
+        sum += qi;
+        o[i >> 2] |= ((uint32_t)qi & 0xffu) << ((i & 3) * 8);
       }
+      *(uint2*)(q + (size_t)row * ldq + k0) = make_uint2(o[0], o[1]);
     }
-    uint32_t o[2] = {0, 0};
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      float t = v[i];
-      if (smooth) t = round_dyn(__fmul_rn(t, load_dyn(smooth, smooth_dtype, (size_t)k0 + i)), t1);
-      float r;
-      if (mode == FMSMO_WQ_MUL) {
-        r = __builtin_rintf(fminf(fmaxf(round_dyn(__fmul_rn(c, t), t2), -127.0f), 127.0f));
-      } else {
-        r = fminf(fmaxf(__builtin_rintf(round_dyn(t / c, t2)), -127.0f), 127.0f);
-      }
-      const int qi = (int)r;
-      sum += qi;
-      o[i >> 2] |= ((uint32_t)qi & 0xffu) << ((i & 3) * 8);
-    }
-    *(uint2*)(q + (size_t)row * ldq + k0) = make_uint2(o[0], o[1]);
   }
   if (row_sum) {
 #pragma unroll
@@ -71,37 +110,85 @@ __global__ __launch_bounds__(256) void quant_weight_i8_kernel(
   }
 }
 
-// Per-column running abs-max:  out_k = max( out_k, max_m |x_mk| ).  A block covers 2048 columns
-// (256 threads x 8) and a slab of rows; |x| >= 0 orders like its bit pattern, so the slabs merge
-// with an unsigned atomic max on the fp32 bits.
+// Per-column running abs-max:  out_k = max( out_k, max_m |x_mk| ).  A block covers 512 columns
+// (64 lanes x 8) and a slab of rows shared out over its four waves, merged through LDS; |x| >= 0 orders like its bit pattern, so the slabs merge
+// with an unsigned atomic max on the fp32 bits (a NaN, whose pattern is above infinity's, wins).
 template <int XT>
 __global__ __launch_bounds__(256) void absmax_cols_kernel(const void* __restrict__ x, int64_t ldx,
                                                           int M, int K, int rows_per_block,
                                                           uint32_t* __restrict__ out) {
-  const int k0 = (blockIdx.x * 256 + threadIdx.x) * 8;
-  if (k0 >= K) return;
-  const int m0 = blockIdx.y * rows_per_block, m1 = min(M, m0 + rows_per_block);
-  float best[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-  for (int m = m0; m < m1; ++m) {
-    float v[8];
-    if constexpr (XT == FMSMO_F32) {
-      const float4 a = *(const float4*)((const float*)x + (size_t)m * ldx + k0);
-      const float4 b = *(const float4*)((const float*)x + (size_t)m * ldx + k0 + 4);
-      v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
-    } else {
-      const uint4 r = *(const uint4*)((const u16*)x + (size_t)m * ldx + k0);
-      const uint32_t ww[4] = {r.x, r.y, r.z, r.w};
+  __shared__ uint32_t part[3][64][8];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int k0 = (blockIdx.x * 64 + lane) * 8;
+  const bool live = k0 < K;
+  // the four waves of a block take interleaved groups of U rows of the block's slab
+  constexpr int U = 8;  // rows in flight per thread
+  const int mb = blockIdx.y * rows_per_block, m1 = min(M, mb + rows_per_block);
+  const int m0 = mb + wave * U;
+  uint32_t bits[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  if (!live) {
+  } else if constexpr (XT == FMSMO_F32) {
+    float best[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (int m = m0; m < m1; m += 4 * U) {
+      float4 a[U], b[U];
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const u16 h = (u16)(ww[i >> 1] >> ((i & 1) * 16));
-        v[i] = XT == FMSMO_F16 ? f16_to_f32(h) : bf16_to_f32(h);
+      for (int u = 0; u < U; ++u) {
+        const int r = min(m + u, m1 - 1);  // the tail re-reads the last row
+        a[u] = *(const float4*)((const float*)x + (size_t)r * ldx + k0);
+        b[u] = *(const float4*)((const float*)x + (size_t)r * ldx + k0 + 4);
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const float v[8] = {a[u].x, a[u].y, a[u].z, a[u].w, b[u].x, b[u].y, b[u].z, b[u].w};
+#pragma unroll
+        for (int i = 0; i < 8; ++i) best[i] = fmaxf(best[i], fabsf(v[i]));
       }
     }
 #pragma unroll
-    for (int i = 0; i < 8; ++i) best[i] = fmaxf(best[i], fabsf(v[i]));
-  }
+    for (int i = 0; i < 8; ++i) bits[i] = __float_as_uint(best[i]);
+  } else {
+    // 15-bit magnitudes of non-NaN 16-bit floats order like unsigned integers: packed maxima
+    typedef unsigned short us2 __attribute__((ext_vector_type(2)));
+    us2 best[4] = {{0, 0}, {0, 0}, {0, 0}, {0, 0}};
+    for (int m = m0; m < m1; m += 4 * U) {
+      uint4 r[U];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) atomicMax(out + k0 + i, __float_as_uint(best[i]));
+      for (int u = 0; u < U; ++u)
+        r[u] = *(const uint4*)((const u16*)x + (size_t)min(m + u, m1 - 1) * ldx + k0);
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const uint32_t w[4] = {r[u].x, r[u].y, r[u].z, r[u].w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const uint32_t mag = w[i] & 0x7fff7fffu;
+          us2 m2;
+          __builtin_memcpy(&m2, &mag, 4);
+          best[i] = __builtin_elementwise_max(best[i], m2);
+        }
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const u16 h = best[i >> 1][i & 1];
+      const float v = XT == FMSMO_F16 ? f16_to_f32(h) : bf16_to_f32(h);
+      bits[i] = __float_as_uint(v);
+    }
+  }
+  // merge the four waves, then one atomic per column and block
+  if (wave > 0) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) part[wave - 1][lane][i] = bits[i];
+  }
+  __syncthreads();
+  if (wave == 0 && live) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      uint32_t b = bits[i];
+#pragma unroll
+      for (int w = 0; w < 3; ++w) b = max(b, part[w][lane][i]);
+      atomicMax(out + k0 + i, b);
+    }
+  }
 }
 
 // Bias with the zero-point correction of asymmetric activations folded in:
@@ -153,7 +240,9 @@ extern "C" int fmsmo_quant_weight_i8(const void* w, int w_dtype, int64_t ldw, co
   if (w_dtype < 0 || w_dtype > 2 || coef_dtype < 0 || coef_dtype > 2 ||
       (smooth && (smooth_dtype < 0 || smooth_dtype > 2)) || (mode != FMSMO_WQ_MUL && mode != FMSMO_WQ_DIV))
     return FMSMO_ERR_UNSUPPORTED;
-  if (K % 8 || ldw % 8 || ldq % 8 || (((uintptr_t)w) & 15) || (((uintptr_t)q) & 7)) return FMSMO_ERR_ALIGN;
+  if (K % 8 || ldw % 8 || ldq % 8 || (((uintptr_t)w) & 15) || (((uintptr_t)q) & 7) ||
+      (smooth && (((uintptr_t)smooth) & 15)))
+    return FMSMO_ERR_ALIGN;
   const int t1 = smooth ? promote(w_dtype, smooth_dtype) : w_dtype;
   const int t2 = promote(t1, coef_dtype);
   dim3 grid((unsigned)N), block(256);
@@ -193,10 +282,10 @@ extern "C" int fmsmo_absmax_cols(const void* x, int x_dtype, int64_t ldx, int64_
   if (x_dtype < 0 || x_dtype > 2) return FMSMO_ERR_UNSUPPORTED;
   if (K % 8 || ldx % 8 || (((uintptr_t)x) & 15)) return FMSMO_ERR_ALIGN;
   if (M == 0) return FMSMO_OK;
-  // enough row slabs to occupy the chip, at least 32 rows each
-  const int col_blocks = div_up(K, 2048);
-  int slabs = (int)((M + 31) / 32);
-  const int want = (2048 + col_blocks - 1) / col_blocks;
+  // enough row slabs to occupy the chip, at least 128 rows each (32 per wave)
+  const int col_blocks = div_up(K, 512);
+  int slabs = (int)((M + 127) / 128);
+  const int want = (1024 + col_blocks - 1) / col_blocks;
   if (slabs > want) slabs = want;
   const int rows_per_block = div_up(M, slabs);
   dim3 grid(col_blocks, div_up(M, rows_per_block)), block(256);

@@ -292,6 +292,8 @@ def quant_weight_i8(w, coef, smooth=None, mode="mul", want_row_sum=False):
         smooth = smooth.detach().reshape(-1).contiguous()
         if smooth.numel() != K:
             raise ValueError("smooth must have K elements")
+        if smooth.data_ptr() % 16:
+            smooth = smooth.clone()
     q = torch.empty((N, K), dtype=torch.int8, device=w.device)
     rs = torch.empty((N,), dtype=torch.int32, device=w.device) if want_row_sum else None
     with torch.cuda.device(w.device):

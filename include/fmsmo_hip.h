@@ -256,7 +256,7 @@ int fmsmo_grouped_gemm_i8_dq(const int8_t* a, int64_t lda, const int8_t* b, int6
  *      FMSMO_WQ_DIV:  q_nk = clamp( rint( rnd_T2( t_nk / coef_n ) ), -127, 127 )
  *      row_sum_n = sum_k q_nk                                         (row_sum may be NULL)
  *    T1 = promote(w_dtype, smooth_dtype), T2 = promote(T1, coef_dtype), the dtypes torch uses.
- *    coef has N elements or 1.  W 16-byte aligned, K and ldw multiples of 8 elements.
+ *    coef has N elements or 1.  W and smooth 16-byte aligned, K and ldw multiples of 8 elements.
  *    MUL with coef = 127 / clip_val: the AIU checkpoint writer, process_weight
  *    (fms_mo/utils/aiu_utils.py:237-279) after process_smoothquant (:87-122); row_sum is
  *    process_zero_shift (:282-333).  DIV with coef = w_scale: QLinearINT8Deploy.from_fms_mo
