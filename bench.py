@@ -297,6 +297,31 @@ def extras(torch, K, dev):
         ms = timeit(lambda: i8i8_aiu(xs[0], w, bias, qdata, "per_channel", act, True), iters=10, warm=3)
         tops = 2.0 * M * k * n / (ms * 1e-3) / 1e12
         res[f"i8i8_aiu_op_{act}_down_M4096"] = {"ms": round(ms, 4), "tops": round(tops, 1), "frac_peak": round(tops / PEAK_INT8_TOPS, 4)}
+    # attention matmuls of one Llama-3-8B sequence (32 heads, head dimension 128, 4096 tokens):
+    # with K or N of 128 these are HBM bound (the score matrix dominates the bytes)
+    h, sq, d = 32, 4096, 128
+    qi = torch.randint(-128, 128, (h, sq, d), dtype=torch.int8, device=dev)
+    ki = torch.randint(-128, 128, (h, sq, d), dtype=torch.int8, device=dev)
+    one = torch.full((1,), 1e-3, device=dev)
+    ms = timeit(lambda: K.bmm_i8_dq(qi, ki, one, one, out_dtype=torch.float16), iters=10, warm=3)
+    byts = 2 * h * sq * d + h * sq * sq * 2
+    res["attn_bmm_i8_qk_S4096"] = {"ms": round(ms, 4), "tops": round(2.0 * h * sq * sq * d / ms / 1e9, 1),
+                                   "GBps": round(byts / ms / 1e6, 1), "frac_hbm": round(byts / ms / 1e6 / PEAK_HBM_GBS, 4)}
+    pi = torch.randint(0, 128, (h, sq, sq), dtype=torch.int8, device=dev)
+    vt = torch.randint(-128, 128, (h, d, sq), dtype=torch.int8, device=dev)
+    ms = timeit(lambda: K.bmm_i8_dq(pi, vt, one, one, out_dtype=torch.float16), iters=10, warm=3)
+    byts = h * sq * sq + h * sq * d + h * sq * d * 2
+    res["attn_bmm_i8_pv_S4096"] = {"ms": round(ms, 4), "tops": round(2.0 * h * sq * sq * d / ms / 1e9, 1),
+                                   "GBps": round(byts / ms / 1e6, 1), "frac_hbm": round(byts / ms / 1e6 / PEAK_HBM_GBS, 4)}
+    del pi
+    pf = torch.rand(h, sq, sq, device=dev).half()
+    ms = timeit(lambda: K.quant_i8_affine(pf, 1.0 / 127, -64.0, torch.float16), iters=5, warm=2)
+    byts = h * sq * sq * 3
+    res["attn_quant_scores_fp16_S4096"] = {"ms": round(ms, 4), "GBps": round(byts / ms / 1e6, 1), "frac_hbm": round(byts / ms / 1e6 / PEAK_HBM_GBS, 4)}
+    vf = torch.randn(h, sq, d, device=dev).half()
+    ms = timeit(lambda: K.quant_i8_affine(vf, 0.03, 0.0, torch.float16, transpose=True), iters=10, warm=3)
+    byts = h * sq * d * 3
+    res["attn_quant_v_transposed_fp16_S4096"] = {"us": round(ms * 1e3, 1), "GBps": round(byts / ms / 1e6, 1), "frac_hbm": round(byts / ms / 1e6 / PEAK_HBM_GBS, 4)}
     return res
 
 

@@ -684,6 +684,76 @@ __global__ __launch_bounds__(AQ_THREADS) void quant_i8_mulscale_kernel(
   }
 }
 
+// ------------------------------------------------------------------ int8, static per tensor,
+// evaluated in the compute dtype T, for the operands of a batched matmul:
+//   q = clamp( rint( rnd_T( rnd_T(x / scale) + offset ) ), -128, 127 )
+// x is [batch][R][C].  The plain kernel writes q [batch][R][ldq]; the transposing kernel writes
+// q [batch][C][ldq] (q[c][r] = code of x[r][c]) so that an operand stored with its reduction
+// dimension outermost becomes reduction-contiguous for the MFMA kernels.  Columns of q past the
+// data are filled with zeros (they pad the reduction dimension of the matmul).
+template <int T>
+__device__ __forceinline__ float affine_code(float e, float scale, float offset) {
+  const float t = round_to<T>(__fadd_rn(round_to<T>(e / scale), offset));
+  return fminf(fmaxf(__builtin_rintf(t), -128.0f), 127.0f);
+}
+
+// 8 consecutive elements starting at column c of a row; vec: the 16-byte load is legal
+template <int XT>
+__device__ __forceinline__ void load8_guard(const void* x, size_t row_elem, int c, int C, bool vec,
+                                            float (&e)[8]) {
+  if (vec && c + 8 <= C) {
+    load8<XT>(x, row_elem + c, e);
+  } else {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) e[j] = (c + j < C) ? load_as_f32<XT>(x, row_elem + c + j) : 0.0f;
+  }
+}
+
+template <int XT, int T>
+__global__ __launch_bounds__(AQ_THREADS) void quant_i8_affine_kernel(
+    const void* __restrict__ x, int64_t ldx, int64_t stride_x, float scale, float offset, bool vec,
+    int8_t* __restrict__ q, int64_t ldq, int64_t stride_q, int C) {
+  const size_t xrow = (size_t)blockIdx.y * stride_x + (size_t)blockIdx.x * ldx;
+  uint8_t* qrow = (uint8_t*)q + (size_t)blockIdx.y * stride_q + (size_t)blockIdx.x * ldq;
+  for (int c = threadIdx.x * 8; c < (int)ldq; c += AQ_THREADS * 8) {
+    uint8_t b[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (c < C) {
+      float e[8];
+      load8_guard<XT>(x, xrow, c, C, vec, e);
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        b[j] = (c + j < C) ? (uint8_t)(int)affine_code<T>(e[j], scale, offset) : (uint8_t)0;
+    }
+    store8(qrow, (size_t)c, b);
+  }
+}
+
+template <int XT, int T>
+__global__ __launch_bounds__(256) void quant_i8_affine_t_kernel(
+    const void* __restrict__ x, int64_t ldx, int64_t stride_x, float scale, float offset, bool vec,
+    int8_t* __restrict__ q, int64_t ldq, int64_t stride_q, int R, int C) {
+  __shared__ __attribute__((aligned(16))) uint8_t tile[64][80];  // [c][r], rows 16-byte aligned
+  const int r0 = blockIdx.x * 64, c0 = blockIdx.y * 64;
+  const size_t xb = (size_t)blockIdx.z * stride_x;
+  const int cl = (threadIdx.x & 7) * 8;
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int rl = (threadIdx.x >> 3) + 32 * i;
+    const int r = r0 + rl, c = c0 + cl;
+    float e[8];
+    if (r < R && c < C) load8_guard<XT>(x, xb + (size_t)r * ldx, c, C, vec, e);
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      tile[cl + j][rl] =
+          (r < R && c + j < C) ? (uint8_t)(int)affine_code<T>(e[j], scale, offset) : (uint8_t)0;
+  }
+  __syncthreads();
+  const int oc = threadIdx.x >> 2, chunk = threadIdx.x & 3;
+  if (c0 + oc < C)
+    *(uint4*)((uint8_t*)q + (size_t)blockIdx.z * stride_q + (size_t)(c0 + oc) * ldq + r0 + chunk * 16) =
+        *(const uint4*)&tile[oc][chunk * 16];
+}
+
 // ------------------------------------------------------------------ e4m3, per token
 template <int XT>
 __global__ __launch_bounds__(AQ_THREADS) void quant_fp8_pertoken_kernel(
@@ -1022,6 +1092,51 @@ extern "C" int fmsmo_quant_act_i8_mulscale(const void* x, int x_dtype, int64_t l
 #define LAUNCH(XT, T)                                                                        \
   hipLaunchKernelGGL((quant_i8_mulscale_kernel<XT, T>), grid, block, 0, st, x, ldx, smooth,  \
                      clip, meta_dtype, mode, q, ldq, a_scale, (int)K)
+  if (compute_dtype == FMSMO_F32) {
+    switch (x_dtype) {
+      case FMSMO_F16: LAUNCH(FMSMO_F16, FMSMO_F32); break;
+      case FMSMO_BF16: LAUNCH(FMSMO_BF16, FMSMO_F32); break;
+      default: LAUNCH(FMSMO_F32, FMSMO_F32); break;
+    }
+  } else if (x_dtype == FMSMO_F16) {
+    LAUNCH(FMSMO_F16, FMSMO_F16);
+  } else {
+    LAUNCH(FMSMO_BF16, FMSMO_BF16);
+  }
+#undef LAUNCH
+  return fmsmo_check_launch();
+}
+
+extern "C" int fmsmo_quant_i8_affine(const void* x, int x_dtype, int64_t ldx, int64_t stride_x,
+                                     float scale, float offset, int compute_dtype, int transpose,
+                                     int8_t* q, int64_t ldq, int64_t stride_q, int64_t batch,
+                                     int64_t R, int64_t C, fmsmo_stream_t stream) {
+  if (!x || !q) return FMSMO_ERR_NULL;
+  if (batch <= 0 || R <= 0 || C <= 0 || ldx < C || batch > 65535 || R > 0x7fffffff ||
+      C > 0x7fffffff || stride_x < 0 || stride_q < 0)
+    return FMSMO_ERR_SHAPE;
+  if (x_dtype < 0 || x_dtype > 2 || compute_dtype < 0 || compute_dtype > 2) return FMSMO_ERR_UNSUPPORTED;
+  if (compute_dtype != FMSMO_F32 && compute_dtype != x_dtype) return FMSMO_ERR_UNSUPPORTED;
+  if (transpose) {
+    if (ldq < R || ldq % 64 || stride_q % 16 || !aligned16(q)) return FMSMO_ERR_ALIGN;
+    if (C > 65535 * 64ll) return FMSMO_ERR_SHAPE;
+  } else {
+    if (ldq < C || ldq % 8 || stride_q % 8 || (((uintptr_t)q) & 7)) return FMSMO_ERR_ALIGN;
+    if (ldq > 0x7fffffff) return FMSMO_ERR_SHAPE;
+  }
+  const int esz = x_dtype == FMSMO_F32 ? 4 : 2;
+  const bool vec = aligned16(x) && (ldx * esz) % 16 == 0 && (stride_x * esz) % 16 == 0;
+  hipStream_t st = (hipStream_t)stream;
+#define LAUNCH(XT, T)                                                                          \
+  if (transpose)                                                                               \
+    hipLaunchKernelGGL((quant_i8_affine_t_kernel<XT, T>),                                      \
+                       dim3((unsigned)(ldq / 64), (unsigned)div_up(C, 64), (unsigned)batch),   \
+                       dim3(256), 0, st, x, ldx, stride_x, scale, offset, vec, q, ldq,         \
+                       stride_q, (int)R, (int)C);                                              \
+  else                                                                                         \
+    hipLaunchKernelGGL((quant_i8_affine_kernel<XT, T>), dim3((unsigned)R, (unsigned)batch),    \
+                       dim3(AQ_THREADS), 0, st, x, ldx, stride_x, scale, offset, vec, q, ldq,  \
+                       stride_q, (int)C)
   if (compute_dtype == FMSMO_F32) {
     switch (x_dtype) {
       case FMSMO_F16: LAUNCH(FMSMO_F16, FMSMO_F32); break;

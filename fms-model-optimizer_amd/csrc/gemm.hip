@@ -288,3 +288,64 @@ extern "C" int fmsmo_grouped_gemm_i8_dq(const int8_t* a, int64_t lda, const int8
   return launch_dq<MMA_I8, false, int, true>(g, a_scale, 1, w_scale, 1, bias, bias_dtype, y,
                                              y_dtype, ldy, (hipStream_t)stream);
 }
+
+// ------------------------------------------------------------------------------ batched matmul
+namespace {
+
+// Batches are the "groups" of the grouped kernels with a uniform row count: the rows of A (and of
+// y) of all batches are stacked, B advances by stride_b per batch, the bias by N.
+template <int OP, class AccT>
+int launch_bmm(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t stride_b,
+               const float* a_scale, const float* b_scale, const float* bias, void* y, int y_dtype,
+               int64_t ldy, int64_t batch, int64_t M, int64_t N, int64_t K, hipStream_t st) {
+  int rc = check_gemm(a, lda, b, ldb, y, ldy, batch * M, N, K);
+  if (rc) return rc;
+  if (!a_scale || !b_scale) return FMSMO_ERR_NULL;
+  if (batch <= 0 || M <= 0 || stride_b < N * ldb) return FMSMO_ERR_SHAPE;
+  if (batch * stride_b >= (1ll << 40) || batch >= (1 << 20)) return FMSMO_ERR_UNSUPPORTED;
+  if (K % 64 || stride_b % 16) return FMSMO_ERR_ALIGN;
+  if (y_dtype < 0 || y_dtype > 2) return FMSMO_ERR_UNSUPPORTED;
+  GemmArgs g{};
+  g.a = (const uint8_t*)a; g.b = (const uint8_t*)b; g.lda = lda; g.ldb = ldb;
+  g.M = (int)(batch * M); g.N = (int)N; g.K = (int)K;
+  g.num_experts = (int)batch; g.ldb_e = stride_b; g.rows_per_group = (int)M;
+  // small per-batch outputs (attention heads: N or M of 128) take the 128x128 tile
+  const bool mid = N <= 128 || M <= 128;
+#define GO(OUT)                                                                             \
+  {                                                                                         \
+    EpiDequant<OUT, FMSMO_F32, false, AccT> epi{y, ldy, a_scale, b_scale, bias, 0, 0};      \
+    if (mid) {                                                                              \
+      g.grid_m = (int)batch * div_up(M, TileMid::BM);                                       \
+      launch_tile<TileMid, OP, true>(g, epi, st);                                           \
+    } else {                                                                                \
+      g.grid_m = (int)batch * div_up(M, 256);                                               \
+      if (K % 128 == 0 && use_register_staged(OP)) launch_rs<OP, true>(g, epi, st);         \
+      else launch_tile<TileBig, OP, true>(g, epi, st);                                      \
+    }                                                                                       \
+  }
+  switch (y_dtype) {
+    case FMSMO_F16: GO(FMSMO_F16) break;
+    case FMSMO_BF16: GO(FMSMO_BF16) break;
+    default: GO(FMSMO_F32) break;
+  }
+#undef GO
+  return fmsmo_check_launch();
+}
+
+}  // namespace
+
+extern "C" int fmsmo_bmm_i8_dq(const int8_t* a, int64_t lda, const int8_t* b, int64_t ldb,
+                               int64_t stride_b, const float* a_scale, const float* b_scale,
+                               const float* bias, void* y, int y_dtype, int64_t ldy, int64_t batch,
+                               int64_t M, int64_t N, int64_t K, fmsmo_stream_t stream) {
+  return launch_bmm<MMA_I8, int>(a, lda, b, ldb, stride_b, a_scale, b_scale, bias, y, y_dtype, ldy,
+                                 batch, M, N, K, (hipStream_t)stream);
+}
+
+extern "C" int fmsmo_bmm_fp8_dq(const uint8_t* a, int64_t lda, const uint8_t* b, int64_t ldb,
+                                int64_t stride_b, const float* a_scale, const float* b_scale,
+                                const float* bias, void* y, int y_dtype, int64_t ldy, int64_t batch,
+                                int64_t M, int64_t N, int64_t K, fmsmo_stream_t stream) {
+  return launch_bmm<MMA_FP8, float>(a, lda, b, ldb, stride_b, a_scale, b_scale, bias, y, y_dtype,
+                                    ldy, batch, M, N, K, (hipStream_t)stream);
+}

@@ -41,25 +41,34 @@ __global__ __launch_bounds__(256) void gemm_rs_kernel(GemmArgs g, Epi epi) {
   int tile_m, tile_n;
   int row_lo, row_hi = g.M, expert = 0;
   if constexpr (GROUPED) {
-    // grouped (mixture-of-experts) mode, as in gemm_tile.hpp: the grid is an upper bound, only
-    // the first real_tiles block ids are mapped; a tile covers rows of one expert
-    int real_m = 0;
-    for (int e = 0; e < g.num_experts; ++e) real_m += (g.offsets[e + 1] - g.offsets[e] + BM - 1) / BM;
-    const int real_tiles = real_m * g.grid_n;
-    if ((int)blockIdx.x >= real_tiles) return;  // uniform for the whole block
-    tile_of_block(blockIdx.x, real_tiles, real_m, g.grid_n, g.group_m, tile_m, tile_n);
-    int t = tile_m;
-    row_lo = 0;
-    for (int e = 0; e < g.num_experts; ++e) {
-      const int lo = g.offsets[e], hi = g.offsets[e + 1];
-      const int nt = (hi - lo + BM - 1) / BM;
-      if (t < nt) {
-        row_lo = lo + t * BM;
-        row_hi = hi;
-        expert = e;
-        break;
+    if (g.rows_per_group > 0) {
+      // batched matmul: every group has the same number of rows, the grid is exact
+      const int nt = (g.rows_per_group + BM - 1) / BM;
+      tile_of_block(blockIdx.x, gridDim.x, g.num_experts * nt, g.grid_n, g.group_m, tile_m, tile_n);
+      expert = tile_m / nt;
+      row_lo = expert * g.rows_per_group + (tile_m - expert * nt) * BM;
+      row_hi = (expert + 1) * g.rows_per_group;
+    } else {
+      // grouped (mixture-of-experts) mode, as in gemm_tile.hpp: the grid is an upper bound, only
+      // the first real_tiles block ids are mapped; a tile covers rows of one expert
+      int real_m = 0;
+      for (int e = 0; e < g.num_experts; ++e) real_m += (g.offsets[e + 1] - g.offsets[e] + BM - 1) / BM;
+      const int real_tiles = real_m * g.grid_n;
+      if ((int)blockIdx.x >= real_tiles) return;  // uniform for the whole block
+      tile_of_block(blockIdx.x, real_tiles, real_m, g.grid_n, g.group_m, tile_m, tile_n);
+      int t = tile_m;
+      row_lo = 0;
+      for (int e = 0; e < g.num_experts; ++e) {
+        const int lo = g.offsets[e], hi = g.offsets[e + 1];
+        const int nt = (hi - lo + BM - 1) / BM;
+        if (t < nt) {
+          row_lo = lo + t * BM;
+          row_hi = hi;
+          expert = e;
+          break;
+        }
+        t -= nt;
       }
-      t -= nt;
     }
   } else {
     tile_of_block(blockIdx.x, gridDim.x, g.grid_m, g.grid_n, g.group_m, tile_m, tile_n);

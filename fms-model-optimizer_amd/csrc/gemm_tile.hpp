@@ -36,6 +36,7 @@ struct GemmArgs {
   const int32_t* offsets;
   int num_experts;
   int64_t ldb_e;  // bytes between experts in B
+  int rows_per_group;  // > 0: every group owns this many rows (batched matmul), offsets unused
 #ifdef FMSMO_CLK
   unsigned long long* clk;  // harness only: {core clock, 100 MHz wall clock} at start / end
 #endif
@@ -221,39 +222,40 @@ __global__ __launch_bounds__(WGM* WGN * 64, (Chk::enabled && (OP == MMA_I8 || Ch
   if (blockIdx.x == 0 && tid == 0 && g.clk) { g.clk[0] = clock64(); g.clk[1] = wall_clock64(); }
 #endif
   int tile_m, tile_n;
-  if constexpr (GROUPED) {
-    // The launch grid is an upper bound (the host cannot see the expert sizes).  Count the real
-    // row tiles and map only the first real_tiles block ids, so that every XCD gets an equal
-    // share of real work; the surplus blocks are the last to be dispatched and exit at once.
-    int real_m = 0;
-    for (int e = 0; e < g.num_experts; ++e) real_m += (g.offsets[e + 1] - g.offsets[e] + BM - 1) / BM;
-    const int real_tiles = real_m * g.grid_n;
-    if ((int)blockIdx.x >= real_tiles) return;  // uniform for the whole block
-    tile_of_block(blockIdx.x, real_tiles, real_m, g.grid_n, g.group_m, tile_m, tile_n);
-  } else {
-    tile_of_block(blockIdx.x, gridDim.x, g.grid_m, g.grid_n, g.group_m, tile_m, tile_n);
-  }
-
-#ifdef FMSMO_ABLATE_SAME_TILE
-  tile_m = FMSMO_ABLATE_SAME_TILE == 1 ? 0 : (blockIdx.x & 7) / 4 + 2 * ((blockIdx.x >> 3) & 1);
-  tile_n = FMSMO_ABLATE_SAME_TILE == 1 ? 0 : (blockIdx.x & 7) % 4 + 4 * ((blockIdx.x >> 4) & 1);
-#endif
-  // Row range of A (and of the output) this tile may touch.
   int row_lo = 0, row_hi = g.M, expert = 0;
   if constexpr (GROUPED) {
-    int t = tile_m;
-    for (int e = 0; e < g.num_experts; ++e) {
-      const int lo = g.offsets[e], hi = g.offsets[e + 1];
-      const int nt = (hi - lo + BM - 1) / BM;
-      if (t < nt) {
-        row_lo = lo + t * BM;
-        row_hi = hi;
-        expert = e;
-        break;
+    if (g.rows_per_group > 0) {
+      // batched matmul: every group has the same number of rows, the grid is exact
+      const int nt = (g.rows_per_group + BM - 1) / BM;
+      tile_of_block(blockIdx.x, gridDim.x, g.num_experts * nt, g.grid_n, g.group_m, tile_m, tile_n);
+      expert = tile_m / nt;
+      row_lo = expert * g.rows_per_group + (tile_m - expert * nt) * BM;
+      row_hi = (expert + 1) * g.rows_per_group;
+    } else {
+      // The launch grid is an upper bound (the host cannot see the expert sizes).  Count the
+      // real row tiles and map only the first real_tiles block ids, so that every XCD gets an
+      // equal share of real work; the surplus blocks are the last to be dispatched and exit at
+      // once.
+      int real_m = 0;
+      for (int e = 0; e < g.num_experts; ++e) real_m += (g.offsets[e + 1] - g.offsets[e] + BM - 1) / BM;
+      const int real_tiles = real_m * g.grid_n;
+      if ((int)blockIdx.x >= real_tiles) return;  // uniform for the whole block
+      tile_of_block(blockIdx.x, real_tiles, real_m, g.grid_n, g.group_m, tile_m, tile_n);
+      int t = tile_m;
+      for (int e = 0; e < g.num_experts; ++e) {
+        const int lo = g.offsets[e], hi = g.offsets[e + 1];
+        const int nt = (hi - lo + BM - 1) / BM;
+        if (t < nt) {
+          row_lo = lo + t * BM;
+          row_hi = hi;
+          expert = e;
+          break;
+        }
+        t -= nt;
       }
-      t -= nt;
     }
   } else {
+    tile_of_block(blockIdx.x, gridDim.x, g.grid_m, g.grid_n, g.group_m, tile_m, tile_n);
     row_lo = tile_m * BM;
   }
   const int col_lo = tile_n * BN;

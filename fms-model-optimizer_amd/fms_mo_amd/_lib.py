@@ -41,6 +41,9 @@ SIGNATURES = {
                                  _L, _L, _P],
     "fmsmo_quant_weight_i8": [_P, _I, _L, _P, _I, _P, _I, _L, _I, _P, _L, _P, _L, _L, _P],
     "fmsmo_absmax_cols": [_P, _I, _L, _L, _L, _P, _P],
+    "fmsmo_quant_i8_affine": [_P, _I, _L, _L, _F, _F, _I, _I, _P, _L, _L, _L, _L, _L, _P],
+    "fmsmo_bmm_i8_dq": [_P, _L, _P, _L, _L, _P, _P, _P, _P, _I, _L, _L, _L, _L, _L, _P],
+    "fmsmo_bmm_fp8_dq": [_P, _L, _P, _L, _L, _P, _P, _P, _P, _I, _L, _L, _L, _L, _L, _P],
     "fmsmo_zero_shift_bias": [_P, _L, _P, _L, _P, _F, _P, _I, _P, _L, _L, _P],
 }
 OTHER = {

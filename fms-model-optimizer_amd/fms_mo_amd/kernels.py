@@ -339,3 +339,64 @@ def zero_shift_bias(w, w_scale, a_meta, bias=None, offset=128.0):
                a_meta.contiguous().data_ptr(), float(offset), _ptr(bias),
                _dt(bias) if bias is not None else 0, out.data_ptr(), N, K, _stream(w))
     return out
+
+
+# ---------------------------------------------------------------------------- batched matmul
+def _batched3(t: torch.Tensor) -> torch.Tensor:
+    """[..., R, C] -> [batch, R, C] with unit inner stride and one batch stride (a view when the
+    leading dimensions collapse, a copy otherwise)."""
+    t3 = t.reshape(-1, t.shape[-2], t.shape[-1])
+    if t3.stride(2) != 1 or (t3.shape[1] > 1 and t3.stride(1) < t3.shape[2]):
+        t3 = t3.contiguous()
+    return t3
+
+
+def quant_i8_affine(x, scale: float, offset: float, compute_dtype=None, transpose=False, pad_to=64):
+    """int8 codes of x [..., R, C] (see fmsmo_quant_i8_affine) as [batch, R, Cp] or, transposed,
+    [batch, C, Rp]; the last dimension is zero-padded to a multiple of ``pad_to``."""
+    _need_gpu(x)
+    x3 = _batched3(x)
+    B, R, C = x3.shape
+    compute_dtype = compute_dtype or x.dtype
+    inner = R if transpose else C
+    ldq = (inner + pad_to - 1) // pad_to * pad_to
+    q = torch.empty((B, C if transpose else R, ldq), dtype=torch.int8, device=x.device)
+    with torch.cuda.device(x.device):
+        L.call("fmsmo_quant_i8_affine", x3.data_ptr(), _dt(x3), x3.stride(1) if R > 1 else C,
+               x3.stride(0) if B > 1 else R * C, float(scale), float(offset), _DT[compute_dtype],
+               int(bool(transpose)), q.data_ptr(), ldq, q.stride(0), B, R, C, _stream(x))
+    return q
+
+
+def _bmm(fn, dtype, a, b, a_scale, b_scale, bias, out_dtype):
+    _need_gpu(a, b, bias)
+    if a.dtype != dtype or b.dtype != dtype or a.dim() != 3 or b.dim() != 3:
+        raise TypeError(f"operands must be 3-D {dtype} tensors: a [batch,M,K], b [batch,N,K]")
+    a = a.contiguous()
+    if b.stride(2) != 1 or b.stride(1) < b.shape[2]:
+        b = b.contiguous()
+    B, M, K = a.shape
+    if b.shape[0] != B or b.shape[2] != K:
+        raise ValueError(f"shape mismatch: a {tuple(a.shape)}, b {tuple(b.shape)} ([batch,N,K] layout)")
+    N = b.shape[1]
+    a_scale = _scale_vec(a_scale, 1, a.device, "a_scale")
+    b_scale = _scale_vec(b_scale, 1, a.device, "b_scale")
+    if bias is not None:
+        bias = bias.detach().to(torch.float32).reshape(-1).contiguous()
+        if bias.numel() != B * N:
+            raise ValueError("bias must be [batch, N]")
+    y = torch.empty((B, M, N), dtype=out_dtype, device=a.device)
+    with torch.cuda.device(a.device):
+        L.call(fn, a.data_ptr(), K, b.data_ptr(), b.stride(1) if N > 1 else K,
+               b.stride(0) if B > 1 else N * K, a_scale.data_ptr(), b_scale.data_ptr(), _ptr(bias),
+               y.data_ptr(), _DT[out_dtype], N, B, M, N, K, _stream(a))
+    return y
+
+
+def bmm_i8_dq(a, b, a_scale, b_scale, bias=None, out_dtype=torch.float16):
+    """y [batch,M,N] = (a [batch,M,K] . b [batch,N,K]^T) * a_scale * b_scale + bias [batch,N]."""
+    return _bmm("fmsmo_bmm_i8_dq", torch.int8, a, b, a_scale, b_scale, bias, out_dtype)
+
+
+def bmm_fp8_dq(a, b, a_scale, b_scale, bias=None, out_dtype=torch.bfloat16):
+    return _bmm("fmsmo_bmm_fp8_dq", torch.float8_e4m3fn, a, b, a_scale, b_scale, bias, out_dtype)

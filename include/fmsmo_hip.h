@@ -295,6 +295,48 @@ int fmsmo_zero_shift_bias(const int8_t* w, int64_t ldw, const float* w_scale, in
                           const float* a_meta, float offset, const void* bias, int bias_dtype,
                           float* out, int64_t N, int64_t K, fmsmo_stream_t stream);
 
+/* ------------------------------------------------------------------------------------------
+ * 7. Batched matmuls of attention (quantized m1 . m2 per batch entry).
+ * ------------------------------------------------------------------------------------------ */
+
+/*
+ * Static per-tensor int8 quantizer in the compute dtype T (torch's promotion of x's dtype and the
+ * scale's), for both operands of a batched matmul:
+ *   q = clamp( rint( rnd_T( rnd_T(x / scale) + offset ) ), -128, 127 )
+ * x: [batch][R][C] (row stride ldx, batch stride stride_x, in elements).
+ * transpose == 0: q [batch][R][ldq];  transpose != 0: q [batch][C][ldq] with q[c][r] = code of
+ * x[r][c], which turns an operand stored as [k][n] into the [n][k] layout the MFMA kernels read.
+ * Columns of q past the data are zero-filled (ldq pads the reduction dimension: a multiple of 8,
+ * of 64 when transposing; use a multiple of 64 for fmsmo_bmm_i8_dq).  batch <= 65535.
+ * Reference: QBmmINT8Deploy.qfunc_raw as called by its forward with offset = zero point - 128 for
+ * m1 and 0 for m2 (fms_mo/modules/bmm.py:699-711, 735-737).
+ */
+int fmsmo_quant_i8_affine(const void* x, int x_dtype, int64_t ldx, int64_t stride_x, float scale,
+                          float offset, int compute_dtype, int transpose, int8_t* q, int64_t ldq,
+                          int64_t stride_q, int64_t batch, int64_t R, int64_t C,
+                          fmsmo_stream_t stream);
+
+/*
+ * y[b] = ( a[b] . b[b]^T ) * (a_scale[0] * b_scale[0]) + bias[b][n]      for b in [0, batch)
+ * a: [batch * M][K] (the batches stacked, row stride lda), b: [batch][N][K] (row stride ldb, batch
+ * stride stride_b), y: [batch * M][N] (row stride ldy); a_scale, b_scale: device fp32 scalars;
+ * bias: device fp32 [batch][N] or NULL (the zero-point correction of an asymmetric m1, see
+ * fmsmo_zero_shift_bias, which accepts the stacked [batch * N][K] operand).  int32 (int8) or fp32
+ * (e4m3) accumulation on MFMA, fp32 epilogue.  K % 64 == 0 (zero-pad the operands),
+ * lda/ldb/stride_b % 16 == 0, 16-byte aligned operands, batch * M * lda < 2^31.
+ * Reference: QBmmINT8Deploy.forward (fms_mo/modules/bmm.py:719-748; the reference still
+ * simulates this product with an fp16 matmul) and spyre::scaled_bmm
+ * (fms_mo/aiu_addons/fp8/fp8_spyre_op.py:102-140).
+ */
+int fmsmo_bmm_i8_dq(const int8_t* a, int64_t lda, const int8_t* b, int64_t ldb, int64_t stride_b,
+                    const float* a_scale, const float* b_scale, const float* bias, void* y,
+                    int y_dtype, int64_t ldy, int64_t batch, int64_t M, int64_t N, int64_t K,
+                    fmsmo_stream_t stream);
+int fmsmo_bmm_fp8_dq(const uint8_t* a, int64_t lda, const uint8_t* b, int64_t ldb,
+                     int64_t stride_b, const float* a_scale, const float* b_scale,
+                     const float* bias, void* y, int y_dtype, int64_t ldy, int64_t batch,
+                     int64_t M, int64_t N, int64_t K, fmsmo_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -23,6 +23,10 @@ How each function is pinned (see tests/test_oracle_*.py):
   * i8i8_aiu            -- the six stored vectors of the reference's own test-suite
                            (tests/golden/ref_w-*_a-*_sq-N.pt); its SmoothQuant branch, which no
                            stored vector exercises, by exactness under power-of-two scales
+  * attention matmuls   -- scaled_bmm reduces to scaled_mm per batch entry; qbmm_int8_deploy:
+                           the exact form equals the product of the dequantized operands
+                           ((q1 - zp) s1) . (q2 s2) (closed form), the literal form equals it to
+                           fp16 rounding where the fp16 matmul does not overflow (2-D operands)
   * AIU checkpoint conversion, column abs-max
                         -- closed forms (sqrt(a)/sqrt(wmax) at alpha = 0.5, rint(127 W s / cv) away
                            from ties), invariants (|q| <= 127, zero shift = integer row sums)
@@ -356,6 +360,49 @@ def fp8_linear_forward(x, w_e4m3, weight_scale, bias=None, input_scale=None):
     s_xx = s_x if s_x.numel() > 1 else s_x.reshape(())
     y = scaled_mm_cpu(qx, w_e4m3.t(), s_xx, s_w, bias, out_dtype=x.dtype)
     return y.reshape(tuple(x.shape[:-1]) + (w_e4m3.shape[0],)), qx, s_x
+
+
+# ------------------------------------------------------------------------------------------
+# Attention matmuls
+# ------------------------------------------------------------------------------------------
+def scaled_bmm(mat1, mat2, scale1, scale2, out_dtype=None):
+    """spyre::scaled_bmm (fms_mo/aiu_addons/fp8/fp8_spyre_op.py:102-140): _scaled_mm per batch
+    entry with per-tensor scales.  mat1 [..., M, K], mat2 [..., K, N]."""
+    assert mat1.shape[:-2] == mat2.shape[:-2]
+    assert scale1.numel() == 1 and scale2.numel() == 1
+    od = torch.float32 if out_dtype is None else out_dtype
+    m1 = mat1.reshape(-1, *mat1.shape[-2:])
+    m2 = mat2.reshape(-1, *mat2.shape[-2:])
+    out = torch.empty((m1.shape[0], m1.shape[1], m2.shape[2]), dtype=od)
+    for b in range(m1.shape[0]):
+        out[b] = scaled_mm_cpu(m1[b], m2[b], scale1, scale2, out_dtype=od)
+    return out.reshape(*mat1.shape[:-2], m1.shape[1], m2.shape[2])
+
+
+def qbmm_quant(x, scale, zp):
+    """QBmmINT8Deploy.qfunc_raw (fms_mo/modules/bmm.py:699-711)."""
+    return torch.clamp((x / scale + zp).round(), -128, 127).to(torch.int8)
+
+
+def qbmm_int8_deploy(m1, m2, m1_scale, m1_zp, m2_scale, m2_zp, literal=False):
+    """QBmmINT8Deploy.forward (fms_mo/modules/bmm.py:719-748).  Returns (y, m1_i8, m2_i8).
+
+    literal=True follows the reference line by line: the integer operands are multiplied by an
+    fp16 matmul (whose fp16 result overflows beyond 65504 and is rounded to 11 bits) and the
+    correction sums m2_i8 over dim 0, which is the reduction dimension only for a 2-D m2.
+    literal=False is the product that line stands for: exact integer accumulation and the
+    correction summed over the reduction dimension (dim -2) of every batch entry."""
+    m1_i8 = qbmm_quant(m1, m1_scale, m1_zp - 128)
+    m2_i8 = qbmm_quant(m2, m2_scale, m2_zp)
+    if literal:
+        corr = m1_scale.float() * (m1_zp - 128) * m2_i8.sum(dim=0) * m2_scale.float()
+        x = torch.matmul(m1_i8.half(), m2_i8.half()) * m1_scale * m2_scale - corr
+        return x.to(m1.dtype), m1_i8, m2_i8
+    acc = torch.matmul(m1_i8.to(torch.int64), m2_i8.to(torch.int64))
+    colsum = m2_i8.to(torch.int64).sum(dim=-2, keepdim=True)
+    s = m1_scale.double() * m2_scale.double()
+    x = acc.double() * s - (m1_zp - 128).double() * colsum.double() * s
+    return x.to(m1.dtype), m1_i8, m2_i8
 
 
 # ------------------------------------------------------------------------------------------

@@ -364,3 +364,46 @@ def test_absmax_cols_is_a_running_maximum():
     x = torch.tensor([[1.0, -5.0], [-3.0, 2.0]])
     assert torch.equal(O.absmax_cols(x), torch.tensor([3.0, 5.0]))
     assert torch.equal(O.absmax_cols(x.reshape(1, 2, 2).half()), torch.tensor([3.0, 5.0]))
+
+
+# ------------------------------------------------------------------ attention matmuls
+def test_qbmm_exact_form_is_the_product_of_the_dequantized_operands():
+    """(q1 - zp) s1 and q2 s2 are the dequantized operands; their float64 product is what the
+    quantize -> integer matmul -> dequantize-with-correction chain must return.  A wrong sign, a
+    correction summed over the wrong dimension or applied to the wrong operand fails this."""
+    g = torch.Generator().manual_seed(3)
+    m1 = torch.randn(2, 3, 17, 29, generator=g, dtype=torch.float64)
+    m2 = torch.randn(2, 3, 29, 11, generator=g, dtype=torch.float64)
+    s1, z1 = torch.tensor([0.031], dtype=torch.float64), torch.tensor([113], dtype=torch.int)
+    s2, z2 = torch.tensor([0.027], dtype=torch.float64), torch.tensor([0], dtype=torch.int)
+    y, q1, q2 = O.qbmm_int8_deploy(m1, m2, s1, z1, s2, z2)
+    dq1 = (q1.double() - (z1 - 128).double()) * s1
+    dq2 = q2.double() * s2
+    torch.testing.assert_close(y, dq1 @ dq2, rtol=1e-12, atol=1e-12)
+    # the codes are a faithful quantization: dequantized operands within half a step (unclipped)
+    inside = (m1 / s1 + (z1 - 128)).abs() < 127
+    assert torch.all(((dq1 - m1).abs() <= 0.5 * s1 + 1e-12)[inside])
+
+
+def test_qbmm_literal_form_agrees_where_the_reference_forward_is_well_defined():
+    g = torch.Generator().manual_seed(4)
+    m1 = (0.2 * torch.randn(12, 8, generator=g)).half()
+    m2 = (0.2 * torch.randn(8, 9, generator=g)).half()
+    s1, z1 = torch.tensor([0.02]), torch.tensor([128], dtype=torch.int)
+    s2, z2 = torch.tensor([0.02]), torch.tensor([0], dtype=torch.int)
+    lit, q1, q2 = O.qbmm_int8_deploy(m1, m2, s1, z1, s2, z2, literal=True)
+    ex, q1e, q2e = O.qbmm_int8_deploy(m1, m2, s1, z1, s2, z2)
+    assert torch.equal(q1, q1e) and torch.equal(q2, q2e)
+    assert (q1.int() @ q2.int()).abs().max() < 2048  # exactly representable in the fp16 matmul
+    torch.testing.assert_close(lit.float(), ex.float(), rtol=2e-3, atol=1e-4)
+
+
+def test_scaled_bmm_is_scaled_mm_per_batch_entry():
+    g = torch.Generator().manual_seed(5)
+    a = torch.randn(2, 3, 5, 16, generator=g).to(torch.float8_e4m3fn)
+    b = torch.randn(2, 3, 16, 7, generator=g).to(torch.float8_e4m3fn)
+    s1, s2 = torch.tensor([0.5]), torch.tensor([0.25])
+    y = O.scaled_bmm(a, b, s1, s2, torch.float32)
+    ref = torch.matmul(a.float() * 0.5, b.float() * 0.25)
+    torch.testing.assert_close(y, ref, rtol=1e-6, atol=1e-6)
+    assert O.scaled_bmm(a, b, s1, s2).dtype == torch.float32
