@@ -211,3 +211,52 @@ def test_op_schema_and_shape_only_twin(dev):
     op()  # make sure it is registered
     torch.library.opcheck(torch.ops.fms_mo.i8i8_aiu.default, args,
                           test_utils=("test_schema", "test_faketensor"))
+
+
+def _replay_equals_eager(fn, inputs, static_in):
+    """Capture fn(static_in) once, replay it for every input with eager work and synchronisations
+    in between; every replay must equal the eager result bit for bit."""
+    eager = [fn(x).clone() for x in inputs]
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        fn(static_in)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static_out = fn(static_in)
+    for _ in range(2):
+        for x, ref in zip(inputs, eager):
+            static_in.copy_(x)
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(static_out.view(torch.int16), ref.view(torch.int16))
+            fn(x)
+            torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("act", MODES)
+def test_node_replays_from_a_hip_graph(dev, act):
+    """Nothing in the node reads a value back to the host (clip values, zero point and scales stay
+    on the device), so it can be captured; asymmetric activations add the zero-shift bias kernel."""
+    M, K, N = 40, 1024, 768
+    x, w_int, bias, qdata, *_ = make_case(71, M, K, N, torch.float16, torch.float16, True, act, True)
+    w, b, qd = w_int.to(dev), bias.to(dev), qdata.to(dev)
+    f = op()
+    xs = [(x * (0.5 + 0.25 * i)).to(dev) for i in range(3)]
+    _replay_equals_eager(lambda t: f(t, w, b, qd, "per_channel", act, True), xs, xs[0].clone())
+
+
+@pytest.mark.parametrize("act", MODES)
+def test_node_at_llama3_8b_down_projection(dev, act):
+    """M = 4096 tokens through the 14336 -> 4096 projection: codes against the oracle on a sample of
+    rows, outputs against the float64 evaluation of the oracle's integers on those rows."""
+    M, K, N = 4096, 14336, 4096
+    x, w_int, bias, qdata, w_cv, a_cv, a_cvn, sq = make_case(81, M, K, N, torch.float16, torch.float16,
+                                                             True, act, True)
+    y = op()(x.to(dev), w_int.to(dev), bias.to(dev), qdata.to(dev), "per_channel", act, True).cpu()
+    rows = torch.tensor([0, 1, 777, 2048, 4095])
+    exact = exact_from_oracle_codes(x[rows], w_int, bias, w_cv, a_cv, a_cvn, sq, act)
+    err = (y[rows].double() - exact).abs()
+    assert torch.all(err <= 1.1 * 2.0 ** -11 * exact.abs() + 4e-6 * exact.abs().max() + 1e-6)

@@ -206,3 +206,34 @@ def test_attention_shapes_of_llama3_8b(dev):
     y = K().bmm_i8_dq(p, vt, one, one, out_dtype=torch.float32)
     ref = torch.matmul(p.double(), vt.double().transpose(1, 2))
     torch.testing.assert_close(y.double(), ref, rtol=1e-7, atol=0)
+
+
+def test_qbmm_replays_from_a_hip_graph(dev):
+    """Scales and zero points are cached on the host at conversion, the correction is computed on
+    the device: forward holds only kernel launches and can be captured."""
+    from fms_mo_amd.modules.bmm import QBmmINT8Deploy
+
+    g = gen(15)
+    mod = QBmmINT8Deploy.from_fms_mo(stub_qbmm(3.0, -3.5, 3.2), target_device=dev)
+    k = torch.randn(2, 4, 80, 128, generator=g).half().to(dev)
+    qs = [torch.randn(2, 4, 96, 128, generator=g).half().to(dev) for _ in range(3)]
+    fn = lambda q: mod(q, k.transpose(-1, -2))
+    eager = [fn(q).clone() for q in qs]
+    static_q = qs[0].clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        fn(static_q)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = fn(static_q)
+    for _ in range(2):
+        for q, ref in zip(qs, eager):
+            static_q.copy_(q)
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(out.view(torch.int16), ref.view(torch.int16))
+            fn(q)
+            torch.cuda.synchronize()
