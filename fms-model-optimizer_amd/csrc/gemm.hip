@@ -1,10 +1,6 @@
 // Host launchers of the tiled MFMA GEMMs (int8 -> int32, int8 / e4m3 with fused dequantizing
 // epilogue, grouped mixture-of-experts variant).
-#include "gemm_rs.hpp"
-#include <cmath>
-#include <cstdlib>
-
-using namespace fmsmo;
+#include "gemm_launch.hpp"
 
 thread_local char g_fmsmo_last_error[256] = {0};
 
@@ -29,176 +25,6 @@ extern "C" const char* fmsmo_status_str(int s) {
   }
 }
 
-int fmsmo_gemv_dispatch(int op, const void* a, int64_t lda, const void* b, int64_t ldb,
-                        const float* a_scale, int64_t a_scale_n, const float* w_scale,
-                        int64_t w_scale_n, const void* bias, int bias_dtype, int epilogue,
-                        void* y, int y_dtype, int64_t ldy, int64_t M, int64_t N, int64_t K,
-                        hipStream_t st);
-
-namespace {
-
-bool aligned16(const void* p) { return (((uintptr_t)p) & 15) == 0; }
-
-int check_gemm(const void* a, int64_t lda, const void* b, int64_t ldb, const void* c,
-               int64_t ldc, int64_t M, int64_t N, int64_t K) {
-  if (!a || !b || !c) return FMSMO_ERR_NULL;
-  if (M < 0 || N <= 0 || K <= 0 || lda < K || ldb < K || ldc < N) return FMSMO_ERR_SHAPE;
-  // 32-bit byte offsets inside the kernels
-  if ((M > 0 && (M * lda) >= (1ll << 31)) || N * ldb >= (1ll << 31) || M >= (1 << 30) ||
-      N >= (1 << 30))
-    return FMSMO_ERR_UNSUPPORTED;
-  if (K % 16 || lda % 16 || ldb % 16 || !aligned16(a) || !aligned16(b)) return FMSMO_ERR_ALIGN;
-  return FMSMO_OK;
-}
-
-// Tile shapes.  K is consumed in stages of BK bytes; a K that is not a multiple of BK is handled
-// by the caller-visible rule "K % 64 == 0" for the MFMA path (all transformer shapes), anything
-// else goes to the slow generic kernel.
-struct TileBig { static constexpr int BM = 256, BN = 256, BK = 64, NST = 4, WGM = 2, WGN = 2; };
-struct TileWide { static constexpr int BM = 128, BN = 256, BK = 64, NST = 4, WGM = 2, WGN = 2; };
-struct TileMid { static constexpr int BM = 128, BN = 128, BK = 64, NST = 4, WGM = 2, WGN = 2; };
-
-// Pick the tile shape by (relative kernel efficiency) x (fill of the last round of tiles over
-// the 256 compute units).  The efficiencies are measured loop efficiencies of the three shapes
-// (bigger tiles move fewer bytes per MFMA); 128x128 tiles fit two blocks per CU.
-int pick_tile(int M, int N) {
-  static const char* force = getenv("FMSMO_TILE");  // tuning aid: 0 = 256x256, 1 = 128x256, 2 = 128x128
-  if (force && force[0] >= '0' && force[0] <= '2') return force[0] - '0';
-  // Fitted to measurements on the Llama / Granite shapes: relative loop efficiency of the three
-  // tile shapes, and a sub-linear penalty for a partially filled last round (idle CUs leave
-  // power, hence clock, to the busy ones).
-  const double eff[3] = {1.0, 0.76, 0.70};
-  const int bm[3] = {256, 128, 128}, bn[3] = {256, 256, 128};
-  int best = 0;
-  double best_score = -1;
-  for (int t = 0; t < 3; ++t) {
-    const long tiles = (long)div_up(M, bm[t]) * div_up(N, bn[t]);
-    const long slots = (t == 2 && tiles > 256) ? 512 : 256;  // two 128x128 blocks fit per CU
-    const long rounds = (tiles + slots - 1) / slots;
-    const double fill = (double)tiles / (double)(rounds * slots);
-    const double pad = ((double)M * N) / ((double)div_up(M, bm[t]) * bm[t] * (double)div_up(N, bn[t]) * bn[t]);
-    const double score = eff[t] * pow(fill, 0.6) * pad;
-    if (score > best_score) { best_score = score; best = t; }
-  }
-  return best;
-}
-
-template <class Tile, int OP, bool GROUPED, class Epi>
-void launch_tile(const GemmArgs& g0, const Epi& epi, hipStream_t st) {
-  GemmArgs g = g0;
-  g.grid_n = div_up(g.N, Tile::BN);
-  if (!GROUPED) g.grid_m = div_up(g.M, Tile::BM);
-  g.group_m = 4;
-  dim3 grid((unsigned)(g.grid_m * g.grid_n)), block(Tile::WGM * Tile::WGN * 64);
-  hipLaunchKernelGGL(
-      (gemm_tile_kernel<Tile::BM, Tile::BN, Tile::BK, Tile::NST, Tile::WGM, Tile::WGN, OP, 1,
-                        GROUPED, Epi>),
-      grid, block, 0, st, g, epi, NoChunk{});
-}
-
-// 256x256 tiles with K a multiple of 128 run the register-staged pipeline (gemm_rs.hpp: whole
-// 128-byte lines, half the L2 -> L1 traffic).  FMSMO_RS=0 / 1 forces the choice for tuning.
-static bool use_register_staged(int op) {
-  static const char* force = getenv("FMSMO_RS");
-  if (force && (force[0] == '0' || force[0] == '1')) return force[0] == '1';
-  (void)op;
-  return true;
-}
-template <int OP, bool GROUPED = false, class Epi>
-void launch_rs(const GemmArgs& g0, const Epi& epi, hipStream_t st) {
-  GemmArgs g = g0;
-  g.grid_n = div_up(g.N, 256);
-  if (!GROUPED) g.grid_m = div_up(g.M, 256);
-  g.group_m = 4;
-  dim3 grid((unsigned)(g.grid_m * g.grid_n)), block(256);
-  hipLaunchKernelGGL((gemm_rs_kernel<OP, Epi, GROUPED>), grid, block, 0, st, g, epi);
-}
-
-// Generic fallback (any K % 16 == 0): one thread per output element, 4-byte dot products.
-template <int OP, class Epi>
-__global__ void gemm_simple_kernel(GemmArgs g, Epi epi) {
-  const int n = blockIdx.x * blockDim.x + threadIdx.x;
-  const int m = blockIdx.y;
-  if (n >= g.N) return;
-  const uint8_t* ar = g.a + (int64_t)m * g.lda;
-  const uint8_t* br = g.b + (int64_t)n * g.ldb;
-  typename Epi::Col c = epi.col(n, 0, g.N);
-  typename Epi::Row r = epi.row(m);
-  if constexpr (OP == MMA_I8) {
-    int acc = 0;
-    for (int k = 0; k < g.K; k += 4)
-      acc = __builtin_amdgcn_sdot4(*(const int*)(ar + k), *(const int*)(br + k), acc, false);
-    epi.store(m, n, acc, r, c);
-  } else {
-    float acc = 0.f;
-    for (int k = 0; k < g.K; k += 4) {
-      const uint32_t av = *(const uint32_t*)(ar + k), bv = *(const uint32_t*)(br + k);
-      acc = __fmaf_rn(__builtin_amdgcn_cvt_f32_fp8(av, 0), __builtin_amdgcn_cvt_f32_fp8(bv, 0), acc);
-      acc = __fmaf_rn(__builtin_amdgcn_cvt_f32_fp8(av, 1), __builtin_amdgcn_cvt_f32_fp8(bv, 1), acc);
-      acc = __fmaf_rn(__builtin_amdgcn_cvt_f32_fp8(av, 2), __builtin_amdgcn_cvt_f32_fp8(bv, 2), acc);
-      acc = __fmaf_rn(__builtin_amdgcn_cvt_f32_fp8(av, 3), __builtin_amdgcn_cvt_f32_fp8(bv, 3), acc);
-    }
-    epi.store(m, n, acc, r, c);
-  }
-}
-
-template <int OP, class Epi>
-void launch_any(const GemmArgs& g, const Epi& epi, hipStream_t st) {
-  if (g.K % 64 == 0) {
-    switch (pick_tile(g.M, g.N)) {
-      case 0:
-        if (g.K % 128 == 0 && use_register_staged(OP)) launch_rs<OP>(g, epi, st);
-        else launch_tile<TileBig, OP, false>(g, epi, st);
-        break;
-      case 1: launch_tile<TileWide, OP, false>(g, epi, st); break;
-      default: launch_tile<TileMid, OP, false>(g, epi, st); break;
-    }
-  } else {
-    dim3 grid(div_up(g.N, 64), (unsigned)g.M), block(64);
-    hipLaunchKernelGGL((gemm_simple_kernel<OP, Epi>), grid, block, 0, st, g, epi);
-  }
-}
-
-template <int OP, bool REF, class AccT, bool GROUPED>
-int launch_dq(const GemmArgs& g, const float* a_scale, int a_stride, const float* w_scale,
-              int w_stride, const void* bias, int bias_dtype, void* y, int y_dtype, int64_t ldy,
-              hipStream_t st) {
-  if (!bias) bias_dtype = FMSMO_F32;
-#define GO(OUT, BIAS)                                                                         \
-  {                                                                                           \
-    EpiDequant<OUT, BIAS, REF, AccT> epi{y, ldy, a_scale, w_scale, bias, a_stride, w_stride}; \
-    if constexpr (GROUPED) {                                                                  \
-      if (g.K % 128 == 0 && use_register_staged(OP)) launch_rs<OP, true>(g, epi, st);         \
-      else launch_tile<TileBig, OP, true>(g, epi, st);                                        \
-    } else                                                                                    \
-      launch_any<OP>(g, epi, st);                                                             \
-  }
-#define GO_BIAS(OUT)                            \
-  switch (bias_dtype) {                         \
-    case FMSMO_F16: GO(OUT, FMSMO_F16) break;   \
-    case FMSMO_BF16: GO(OUT, FMSMO_BF16) break; \
-    default: GO(OUT, FMSMO_F32) break;          \
-  }
-  switch (y_dtype) {
-    case FMSMO_F16: GO_BIAS(FMSMO_F16) break;
-    case FMSMO_BF16: GO_BIAS(FMSMO_BF16) break;
-    case FMSMO_F32: GO_BIAS(FMSMO_F32) break;
-    default: return FMSMO_ERR_UNSUPPORTED;
-  }
-#undef GO
-#undef GO_BIAS
-  return fmsmo_check_launch();
-}
-
-int check_dq(const float* a_scale, int64_t a_scale_n, const float* w_scale, int64_t w_scale_n,
-             const void* bias, int bias_dtype, int y_dtype, int64_t M, int64_t N) {
-  if (!a_scale || !w_scale) return FMSMO_ERR_NULL;
-  if ((a_scale_n != 1 && a_scale_n != M) || (w_scale_n != 1 && w_scale_n != N)) return FMSMO_ERR_SHAPE;
-  if (y_dtype < 0 || y_dtype > 2 || (bias && (bias_dtype < 0 || bias_dtype > 2))) return FMSMO_ERR_UNSUPPORTED;
-  return FMSMO_OK;
-}
-
-}  // namespace
 
 extern "C" int fmsmo_gemm_i8_i32(const int8_t* a, int64_t lda, const int8_t* b, int64_t ldb,
                                  int32_t* c, int64_t ldc, int64_t M, int64_t N, int64_t K,
@@ -240,28 +66,6 @@ extern "C" int fmsmo_gemm_i8_dq(const int8_t* a, int64_t lda, const int8_t* b, i
                                               y_dtype, ldy, (hipStream_t)stream);
 }
 
-extern "C" int fmsmo_gemm_fp8_dq(const uint8_t* a, int64_t lda, const uint8_t* b, int64_t ldb,
-                                 const float* a_scale, int64_t a_scale_n, const float* w_scale,
-                                 int64_t w_scale_n, const void* bias, int bias_dtype, void* y,
-                                 int y_dtype, int64_t ldy, int64_t M, int64_t N, int64_t K,
-                                 fmsmo_stream_t stream) {
-  int rc = check_gemm(a, lda, b, ldb, y, ldy, M, N, K);
-  if (rc) return rc;
-  rc = check_dq(a_scale, a_scale_n, w_scale, w_scale_n, bias, bias_dtype, y_dtype, M, N);
-  if (rc) return rc;
-  if (M == 0) return FMSMO_OK;
-  if (M <= 16 && K % 128 == 0)
-    return fmsmo_gemv_dispatch(FMSMO_OP_E4M3, a, lda, b, ldb, a_scale, a_scale_n, w_scale,
-                               w_scale_n, bias, bias_dtype, FMSMO_EPI_F32, y, y_dtype, ldy, M, N, K,
-                               (hipStream_t)stream);
-  GemmArgs g{};
-  g.a = a; g.b = b; g.lda = lda; g.ldb = ldb;
-  g.M = (int)M; g.N = (int)N; g.K = (int)K;
-  const int as = a_scale_n == 1 ? 0 : 1, ws = w_scale_n == 1 ? 0 : 1;
-  return launch_dq<MMA_FP8, false, float, false>(g, a_scale, as, w_scale, ws, bias, bias_dtype, y,
-                                                 y_dtype, ldy, (hipStream_t)stream);
-}
-
 extern "C" int fmsmo_grouped_gemm_i8_dq(const int8_t* a, int64_t lda, const int8_t* b,
                                         int64_t ldb, int64_t ldb_e, const int32_t* offsets,
                                         int num_experts, int64_t total_rows, const float* a_scale,
@@ -289,50 +93,6 @@ extern "C" int fmsmo_grouped_gemm_i8_dq(const int8_t* a, int64_t lda, const int8
                                              y_dtype, ldy, (hipStream_t)stream);
 }
 
-// ------------------------------------------------------------------------------ batched matmul
-namespace {
-
-// Batches are the "groups" of the grouped kernels with a uniform row count: the rows of A (and of
-// y) of all batches are stacked, B advances by stride_b per batch, the bias by N.
-template <int OP, class AccT>
-int launch_bmm(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t stride_b,
-               const float* a_scale, const float* b_scale, const float* bias, void* y, int y_dtype,
-               int64_t ldy, int64_t batch, int64_t M, int64_t N, int64_t K, hipStream_t st) {
-  int rc = check_gemm(a, lda, b, ldb, y, ldy, batch * M, N, K);
-  if (rc) return rc;
-  if (!a_scale || !b_scale) return FMSMO_ERR_NULL;
-  if (batch <= 0 || M <= 0 || stride_b < N * ldb) return FMSMO_ERR_SHAPE;
-  if (batch * stride_b >= (1ll << 40) || batch >= (1 << 20)) return FMSMO_ERR_UNSUPPORTED;
-  if (K % 64 || stride_b % 16) return FMSMO_ERR_ALIGN;
-  if (y_dtype < 0 || y_dtype > 2) return FMSMO_ERR_UNSUPPORTED;
-  GemmArgs g{};
-  g.a = (const uint8_t*)a; g.b = (const uint8_t*)b; g.lda = lda; g.ldb = ldb;
-  g.M = (int)(batch * M); g.N = (int)N; g.K = (int)K;
-  g.num_experts = (int)batch; g.ldb_e = stride_b; g.rows_per_group = (int)M;
-  // small per-batch outputs (attention heads: N or M of 128) take the 128x128 tile
-  const bool mid = N <= 128 || M <= 128;
-#define GO(OUT)                                                                             \
-  {                                                                                         \
-    EpiDequant<OUT, FMSMO_F32, false, AccT> epi{y, ldy, a_scale, b_scale, bias, 0, 0};      \
-    if (mid) {                                                                              \
-      g.grid_m = (int)batch * div_up(M, TileMid::BM);                                       \
-      launch_tile<TileMid, OP, true>(g, epi, st);                                           \
-    } else {                                                                                \
-      g.grid_m = (int)batch * div_up(M, 256);                                               \
-      if (K % 128 == 0 && use_register_staged(OP)) launch_rs<OP, true>(g, epi, st);         \
-      else launch_tile<TileBig, OP, true>(g, epi, st);                                      \
-    }                                                                                       \
-  }
-  switch (y_dtype) {
-    case FMSMO_F16: GO(FMSMO_F16) break;
-    case FMSMO_BF16: GO(FMSMO_BF16) break;
-    default: GO(FMSMO_F32) break;
-  }
-#undef GO
-  return fmsmo_check_launch();
-}
-
-}  // namespace
 
 extern "C" int fmsmo_bmm_i8_dq(const int8_t* a, int64_t lda, const int8_t* b, int64_t ldb,
                                int64_t stride_b, const float* a_scale, const float* b_scale,
@@ -342,10 +102,3 @@ extern "C" int fmsmo_bmm_i8_dq(const int8_t* a, int64_t lda, const int8_t* b, in
                                  batch, M, N, K, (hipStream_t)stream);
 }
 
-extern "C" int fmsmo_bmm_fp8_dq(const uint8_t* a, int64_t lda, const uint8_t* b, int64_t ldb,
-                                int64_t stride_b, const float* a_scale, const float* b_scale,
-                                const float* bias, void* y, int y_dtype, int64_t ldy, int64_t batch,
-                                int64_t M, int64_t N, int64_t K, fmsmo_stream_t stream) {
-  return launch_bmm<MMA_FP8, float>(a, lda, b, ldb, stride_b, a_scale, b_scale, bias, y, y_dtype,
-                                    ldy, batch, M, N, K, (hipStream_t)stream);
-}
