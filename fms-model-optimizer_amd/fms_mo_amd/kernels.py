@@ -400,3 +400,114 @@ def bmm_i8_dq(a, b, a_scale, b_scale, bias=None, out_dtype=torch.float16):
 
 def bmm_fp8_dq(a, b, a_scale, b_scale, bias=None, out_dtype=torch.bfloat16):
     return _bmm("fmsmo_bmm_fp8_dq", torch.float8_e4m3fn, a, b, a_scale, b_scale, bias, out_dtype)
+
+
+# ------------------------------------------------------- the hot-path wrappers as torch operators
+# The five wrappers every module forward ends in are registered under ``torch.ops.fms_mo_amd`` with
+# shape-only twins, so that ``torch.compile`` traces a swapped model without graph breaks (the
+# reference gets the same from registering its integer matmuls as ``torch.ops.fms_mo.*``,
+# fms_mo/custom_ext_kernels/utils.py:642-802).  Only GPU kernels are registered: a CPU tensor that
+# gets this far fails in the dispatcher.
+_OPS = torch.library.Library("fms_mo_amd", "FRAGMENT")
+_quant_act_i8_pertoken_impl = quant_act_i8_pertoken
+_quant_act_i8_static_impl = quant_act_i8_static
+_quant_act_fp8_pertoken_impl = quant_act_fp8_pertoken
+_gemm_i8_dq_impl = gemm_i8_dq
+_gemm_fp8_dq_impl = gemm_fp8_dq
+
+
+def _register(name, schema, impl, fake):
+    _OPS.define(name + schema)
+    _OPS.impl(name, impl, "CUDA")
+    torch.library.register_fake("fms_mo_amd::" + name)(fake)
+
+
+def _rows_shape(x):
+    return (x.shape[0], x.shape[1])
+
+
+_register(
+    "quant_act_i8_pertoken",
+    "(Tensor x, Tensor? smooth, ScalarType? compute_dtype, bool saturate) -> (Tensor, Tensor)",
+    lambda x, smooth, compute_dtype, saturate: _quant_act_i8_pertoken_impl(x, smooth, compute_dtype, saturate),
+    lambda x, smooth, compute_dtype, saturate: (
+        torch.empty(_rows_shape(x), dtype=torch.int8, device=x.device),
+        torch.empty((x.shape[0],), dtype=torch.float32, device=x.device)),
+)
+_register(
+    "quant_act_i8_static",
+    "(Tensor x, float scale, int zp, int sym) -> Tensor",
+    lambda x, scale, zp, sym: _quant_act_i8_static_impl(x, scale, zp, sym),
+    lambda x, scale, zp, sym: torch.empty(_rows_shape(x), dtype=torch.int8, device=x.device),
+)
+_register(
+    "quant_act_fp8_pertoken",
+    "(Tensor x, int variant, Tensor? static_scale) -> (Tensor, Tensor)",
+    lambda x, variant, static_scale: _quant_act_fp8_pertoken_impl(x, variant, static_scale),
+    lambda x, variant, static_scale: (
+        torch.empty(_rows_shape(x), dtype=torch.float8_e4m3fn, device=x.device),
+        torch.empty((1 if static_scale is not None else x.shape[0],), dtype=torch.float32,
+                    device=x.device)),
+)
+_register(
+    "gemm_i8_dq",
+    "(Tensor a, Tensor w, Tensor a_scale, Tensor w_scale, Tensor? bias, ScalarType out_dtype, "
+    "bool exact_ref, bool force_gemv) -> Tensor",
+    lambda a, w, a_scale, w_scale, bias, out_dtype, exact_ref, force_gemv: _gemm_i8_dq_impl(
+        a, w, a_scale, w_scale, bias, out_dtype, exact_ref, force_gemv),
+    lambda a, w, a_scale, w_scale, bias, out_dtype, exact_ref, force_gemv: torch.empty(
+        (a.shape[0], w.shape[0]), dtype=out_dtype, device=a.device),
+)
+_register(
+    "gemm_fp8_dq",
+    "(Tensor a, Tensor w, Tensor a_scale, Tensor w_scale, Tensor? bias, ScalarType out_dtype, "
+    "bool force_gemv) -> Tensor",
+    lambda a, w, a_scale, w_scale, bias, out_dtype, force_gemv: _gemm_fp8_dq_impl(
+        a, w, a_scale, w_scale, bias, out_dtype, force_gemv),
+    lambda a, w, a_scale, w_scale, bias, out_dtype, force_gemv: torch.empty(
+        (a.shape[0], w.shape[0]), dtype=out_dtype, device=a.device),
+)
+
+
+def _as_scale(s, device):
+    if torch.is_tensor(s):
+        return s
+    return torch.tensor([float(s)], dtype=torch.float32, device=device)
+
+
+def quant_act_i8_pertoken(x, smooth=None, compute_dtype=None, saturate=False):  # noqa: F811
+    """(q int8 [M,K], scale fp32 [M]) -- see fmsmo_quant_act_i8_pertoken."""
+    _need_gpu(x, smooth)
+    if x.dim() != 2:
+        raise ValueError("expected a 2-D tensor")
+    return torch.ops.fms_mo_amd.quant_act_i8_pertoken(x, smooth, compute_dtype, bool(saturate))
+
+
+def quant_act_i8_static(x, scale: float, zp: int, sym: int):  # noqa: F811
+    _need_gpu(x)
+    if x.dim() != 2:
+        raise ValueError("expected a 2-D tensor")
+    return torch.ops.fms_mo_amd.quant_act_i8_static(x, float(scale), int(zp), int(sym))
+
+
+def quant_act_fp8_pertoken(x, variant=L.FP8_LINEAR, static_scale=None):  # noqa: F811
+    """(q e4m3 [M,K], scale fp32 [M] or the [1] static scale)."""
+    _need_gpu(x)
+    if x.dim() != 2:
+        raise ValueError("expected a 2-D tensor")
+    if static_scale is not None:
+        static_scale = _as_scale(static_scale, x.device)
+    return torch.ops.fms_mo_amd.quant_act_fp8_pertoken(x, int(variant), static_scale)
+
+
+def gemm_i8_dq(a, w, a_scale, w_scale, bias=None, out_dtype=torch.float16, exact_ref=True,  # noqa: F811
+               force_gemv=False):
+    _need_gpu(a, w, bias)
+    return torch.ops.fms_mo_amd.gemm_i8_dq(a, w, _as_scale(a_scale, a.device), _as_scale(w_scale, a.device),
+                                           bias, out_dtype, bool(exact_ref), bool(force_gemv))
+
+
+def gemm_fp8_dq(a, w, a_scale, w_scale, bias=None, out_dtype=torch.bfloat16, force_gemv=False):  # noqa: F811
+    _need_gpu(a, w, bias)
+    return torch.ops.fms_mo_amd.gemm_fp8_dq(a, w, _as_scale(a_scale, a.device), _as_scale(w_scale, a.device),
+                                            bias, out_dtype, bool(force_gemv))

@@ -507,6 +507,10 @@ class QLinearINT8Deploy(nn.Linear):
         """The reference divides by ``smoothq_scale`` only if EVERY element differs from 1
         (linear.py:1331); the answer is cached until the buffer changes (it costs a host sync)."""
         sq = self.smoothq_scale
+        if torch.compiler.is_compiling():
+            # the answer of the last eager call (the module has to run eagerly once before it is
+            # compiled, as it has to before it is captured in a graph)
+            return self._sq_on
         key = (sq.data_ptr(), sq._version)
         if getattr(self, "_sq_key", None) != key:
             self._sq_key = key

@@ -265,3 +265,54 @@ def test_swapped_mlp_replays_from_a_hip_graph(dev):
             assert torch.equal(static_y.view(torch.int16), ref.view(torch.int16))
             _ = mlp(x)                               # eager work between replays
             torch.cuda.synchronize()
+
+
+def test_swapped_mlp_traces_without_graph_breaks(dev):
+    """torch.compile must see the lowered modules as operator calls (the reference registers its
+    integer matmuls as torch.ops.fms_mo.* for this, custom_ext_kernels/utils.py:642-802): the
+    kernel wrappers are torch.ops.fms_mo_amd.* with shape-only twins.  ``fullgraph=True`` turns
+    any graph break into an error; the backend replays the traced graph with the real kernels."""
+    from fms_mo_amd.modules.linear import QLinearINT8Deploy
+
+    H, I, T = 512, 1536, 48
+    mods = {}
+    for name, k, n, seed in [("gate", H, I, 1), ("up", H, I, 2), ("down", I, H, 3)]:
+        q = make_qlinear(None, k, n, smoothq=True, seed=seed)
+        q.set_act_scale(torch.rand(k, generator=gen(10 + seed)) * 3 + 0.2)
+        mods[name] = QLinearINT8Deploy.from_fms_mo(q, use_int_kernel="cutlass", use_dynamic_max_act_Qfunc=-1,
+                                                   recalc_clipvals=False, target_device=dev)
+
+    class MLP(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.gate, self.up, self.down = mods["gate"], mods["up"], mods["down"]
+
+        def forward(self, x):
+            return self.down(torch.nn.functional.silu(self.gate(x)) * self.up(x))
+
+    mlp = MLP()
+    xs = [outlier_x(T, H, 30 + i).to(dev) for i in range(3)]
+    eager = [mlp(x).clone() for x in xs]
+    compiled = torch.compile(mlp, backend="aot_eager", fullgraph=True)
+    for x, ref in zip(xs, eager):
+        y = compiled(x)
+        assert torch.equal(y.view(torch.int16), ref.view(torch.int16))
+    ops = [n for n in dir(torch.ops.fms_mo_amd) if not n.startswith("_")]
+    assert {"quant_act_i8_pertoken", "gemm_i8_dq"} <= set(ops)
+
+
+def test_operator_twins_agree_with_the_kernels_on_shapes(dev):
+    from fms_mo_amd import kernels
+
+    x = torch.randn(24, 256, device=dev).half()
+    sm = (torch.rand(256, device=dev) + 0.5).half()
+    w = torch.randint(-127, 128, (96, 256), dtype=torch.int8, device=dev)
+    ws = torch.rand(96, device=dev)
+    q, s = kernels.quant_act_i8_pertoken(x, sm)
+    torch.library.opcheck(torch.ops.fms_mo_amd.quant_act_i8_pertoken.default, (x, sm, torch.float16, False),
+                          test_utils=("test_schema", "test_faketensor"))
+    torch.library.opcheck(torch.ops.fms_mo_amd.gemm_i8_dq.default,
+                          (q, w, s, ws, None, torch.float16, True, False),
+                          test_utils=("test_schema", "test_faketensor"))
+    torch.library.opcheck(torch.ops.fms_mo_amd.quant_act_i8_static.default, (x, 0.05, 128, 0),
+                          test_utils=("test_schema", "test_faketensor"))
