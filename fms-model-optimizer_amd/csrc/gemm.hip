@@ -40,11 +40,11 @@ extern "C" int fmsmo_gemm_i8_i32(const int8_t* a, int64_t lda, const int8_t* b, 
   return fmsmo_check_launch();
 }
 
-extern "C" int fmsmo_gemm_i8_dq(const int8_t* a, int64_t lda, const int8_t* b, int64_t ldb,
-                                const float* a_scale, int64_t a_scale_n, const float* w_scale,
-                                int64_t w_scale_n, const void* bias, int bias_dtype, int epilogue,
-                                void* y, int y_dtype, int64_t ldy, int64_t M, int64_t N,
-                                int64_t K, fmsmo_stream_t stream) {
+static int gemm_i8_dq_impl(const int8_t* a, int64_t lda, const int8_t* b, int64_t ldb,
+                           const float* a_scale, int64_t a_scale_n, const float* w_scale,
+                           int64_t w_scale_n, const void* bias, int bias_dtype, int epilogue,
+                           void* y, int y_dtype, int64_t ldy, int64_t M, int64_t N, int64_t K,
+                           void* workspace, int64_t workspace_bytes, fmsmo_stream_t stream) {
   int rc = check_gemm(a, lda, b, ldb, y, ldy, M, N, K);
   if (rc) return rc;
   rc = check_dq(a_scale, a_scale_n, w_scale, w_scale_n, bias, bias_dtype, y_dtype, M, N);
@@ -59,11 +59,43 @@ extern "C" int fmsmo_gemm_i8_dq(const int8_t* a, int64_t lda, const int8_t* b, i
   g.a = (const uint8_t*)a; g.b = (const uint8_t*)b; g.lda = lda; g.ldb = ldb;
   g.M = (int)M; g.N = (int)N; g.K = (int)K;
   const int as = a_scale_n == 1 ? 0 : 1, ws = w_scale_n == 1 ? 0 : 1;
+  const SplitPlan plan = plan_split_k(M, N, K);
+  if (plan.splits > 1 && workspace && workspace_bytes >= plan.ws_bytes && aligned16(workspace) &&
+      plan.splits * M * lda < (1ll << 31)) {
+    if (epilogue == FMSMO_EPI_REF_F16)
+      return launch_split_k<MMA_I8, true, int>(plan, g, workspace, a_scale, as, w_scale, ws, bias,
+                                               bias_dtype, y, y_dtype, ldy, (hipStream_t)stream);
+    return launch_split_k<MMA_I8, false, int>(plan, g, workspace, a_scale, as, w_scale, ws, bias,
+                                              bias_dtype, y, y_dtype, ldy, (hipStream_t)stream);
+  }
   if (epilogue == FMSMO_EPI_REF_F16)
     return launch_dq<MMA_I8, true, int, false>(g, a_scale, as, w_scale, ws, bias, bias_dtype, y,
                                                y_dtype, ldy, (hipStream_t)stream);
   return launch_dq<MMA_I8, false, int, false>(g, a_scale, as, w_scale, ws, bias, bias_dtype, y,
                                               y_dtype, ldy, (hipStream_t)stream);
+}
+
+extern "C" int fmsmo_gemm_i8_dq(const int8_t* a, int64_t lda, const int8_t* b, int64_t ldb,
+                                const float* a_scale, int64_t a_scale_n, const float* w_scale,
+                                int64_t w_scale_n, const void* bias, int bias_dtype, int epilogue,
+                                void* y, int y_dtype, int64_t ldy, int64_t M, int64_t N,
+                                int64_t K, fmsmo_stream_t stream) {
+  return gemm_i8_dq_impl(a, lda, b, ldb, a_scale, a_scale_n, w_scale, w_scale_n, bias, bias_dtype,
+                         epilogue, y, y_dtype, ldy, M, N, K, nullptr, 0, stream);
+}
+
+extern "C" int fmsmo_gemm_i8_dq_ws(const int8_t* a, int64_t lda, const int8_t* b, int64_t ldb,
+                                   const float* a_scale, int64_t a_scale_n, const float* w_scale,
+                                   int64_t w_scale_n, const void* bias, int bias_dtype,
+                                   int epilogue, void* y, int y_dtype, int64_t ldy, int64_t M,
+                                   int64_t N, int64_t K, void* workspace, int64_t workspace_bytes,
+                                   fmsmo_stream_t stream) {
+  return gemm_i8_dq_impl(a, lda, b, ldb, a_scale, a_scale_n, w_scale, w_scale_n, bias, bias_dtype,
+                         epilogue, y, y_dtype, ldy, M, N, K, workspace, workspace_bytes, stream);
+}
+
+extern "C" int64_t fmsmo_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+  return plan_split_k(M, N, K).ws_bytes;
 }
 
 extern "C" int fmsmo_grouped_gemm_i8_dq(const int8_t* a, int64_t lda, const int8_t* b,

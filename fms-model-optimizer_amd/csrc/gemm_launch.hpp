@@ -179,6 +179,89 @@ int check_dq(const float* a_scale, int64_t a_scale_n, const float* w_scale, int6
 
 }  // namespace
 
+// ---------------------------------------------------------------------------------- split K
+// Few output tiles and a long reduction (a batch of tens to hundreds of tokens through a
+// projection with few output columns) leave most compute units idle: 17 x 4096 x 14336 is 32 tiles
+// of 128 x 128.  With a caller-provided workspace the reduction is cut into slices that run as
+// the uniform "groups" of the grouped kernels (A and B advance along K per group, the partial
+// sums of group s land in rows [s M, (s + 1) M) of the workspace) and a second kernel adds the
+// slices in a fixed order and applies the dequantizing epilogue.  int32 partial sums are exact, so
+// the int8 result is bit-identical to the single-pass one.
+namespace {
+
+struct SplitPlan {
+  int splits;
+  int64_t k_len, ws_bytes;
+};
+
+inline SplitPlan plan_split_k(int64_t M, int64_t N, int64_t K) {
+  SplitPlan p{1, K, 0};
+  static const char* off = getenv("FMSMO_SPLIT_K");  // FMSMO_SPLIT_K=0 disables (tuning aid)
+  if (off && off[0] == '0') return p;
+  if (M <= 16 || M > 1024 || K % 128) return p;
+  const int64_t tiles = (int64_t)div_up(M, TileMid::BM) * div_up(N, TileMid::BN);
+  if (tiles > 128) return p;
+  int s = (int)(256 / tiles);  // one block per compute unit; 512 and 1024 blocks measured slower
+  while (s > 1 && (K % (s * 128) != 0 || K / s < 512)) --s;
+  if (s < 2) return p;
+  p.splits = s;
+  p.k_len = K / s;
+  p.ws_bytes = (int64_t)s * M * N * 4;
+  return p;
+}
+
+template <class AccT, class Epi>
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const AccT* __restrict__ ws, int S, int M,
+                                                            int N, Epi epi) {
+  const int n = blockIdx.x * 256 + threadIdx.x, m = blockIdx.y;
+  if (n >= N) return;
+  AccT sum = ws[(int64_t)m * N + n];
+  for (int s = 1; s < S; ++s) sum += ws[((int64_t)s * M + m) * N + n];
+  epi.store(m, n, sum, epi.row(m), epi.col(n, 0, N));
+}
+
+// y = epilogue( sum over K slices ), see above.  The caller has checked the operands.
+template <int OP, bool REF, class AccT>
+int launch_split_k(const SplitPlan& p, const GemmArgs& g0, void* workspace, const float* a_scale,
+                   int a_stride, const float* w_scale, int w_stride, const void* bias,
+                   int bias_dtype, void* y, int y_dtype, int64_t ldy, hipStream_t st) {
+  GemmArgs g = g0;
+  g.K = (int)p.k_len;
+  g.num_experts = p.splits;
+  g.rows_per_group = g0.M;
+  g.M = p.splits * g0.M;
+  g.lda_e = p.k_len;
+  g.ldb_e = p.k_len;
+  g.grid_m = p.splits * div_up(g0.M, TileMid::BM);
+  if constexpr (OP == MMA_I8) launch_tile<TileMid, OP, true>(g, EpiStoreI32{(int32_t*)workspace, g0.N}, st);
+  else launch_tile<TileMid, OP, true>(g, EpiStoreF32{(float*)workspace, g0.N}, st);
+  if (!bias) bias_dtype = FMSMO_F32;
+  dim3 grid(div_up(g0.N, 256), (unsigned)g0.M), block(256);
+#define GO(OUT, BIAS)                                                                         \
+  {                                                                                           \
+    EpiDequant<OUT, BIAS, REF, AccT> epi{y, ldy, a_scale, w_scale, bias, a_stride, w_stride}; \
+    hipLaunchKernelGGL((splitk_reduce_kernel<AccT, decltype(epi)>), grid, block, 0, st,       \
+                       (const AccT*)workspace, p.splits, g0.M, g0.N, epi);                    \
+  }
+#define GO_BIAS(OUT)                            \
+  switch (bias_dtype) {                         \
+    case FMSMO_F16: GO(OUT, FMSMO_F16) break;   \
+    case FMSMO_BF16: GO(OUT, FMSMO_BF16) break; \
+    default: GO(OUT, FMSMO_F32) break;          \
+  }
+  switch (y_dtype) {
+    case FMSMO_F16: GO_BIAS(FMSMO_F16) break;
+    case FMSMO_BF16: GO_BIAS(FMSMO_BF16) break;
+    case FMSMO_F32: GO_BIAS(FMSMO_F32) break;
+    default: return FMSMO_ERR_UNSUPPORTED;
+  }
+#undef GO
+#undef GO_BIAS
+  return fmsmo_check_launch();
+}
+
+}  // namespace
+
 // ------------------------------------------------------------------------------ batched matmul
 namespace {
 
@@ -199,6 +282,7 @@ int launch_bmm(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t s
   g.a = (const uint8_t*)a; g.b = (const uint8_t*)b; g.lda = lda; g.ldb = ldb;
   g.M = (int)(batch * M); g.N = (int)N; g.K = (int)K;
   g.num_experts = (int)batch; g.ldb_e = stride_b; g.rows_per_group = (int)M;
+  g.lda_e = M * lda;
   // small per-batch outputs (attention heads: N or M of 128) take the 128x128 tile
   const bool mid = N <= 128 || M <= 128;
 #define GO(OUT)                                                                             \

@@ -40,6 +40,8 @@ __global__ __launch_bounds__(256) void gemm_rs_kernel(GemmArgs g, Epi epi) {
   const int wm = wave >> 1, wn = wave & 1;
   int tile_m, tile_n;
   int row_lo, row_hi = g.M, expert = 0;
+  int64_t a_adj = 0;
+  int a_rows = g.M;  // rows addressable through the A descriptor (numbered like row_lo)
   if constexpr (GROUPED) {
     if (g.rows_per_group > 0) {
       // batched matmul: every group has the same number of rows, the grid is exact
@@ -48,6 +50,10 @@ __global__ __launch_bounds__(256) void gemm_rs_kernel(GemmArgs g, Epi epi) {
       expert = tile_m / nt;
       row_lo = expert * g.rows_per_group + (tile_m - expert * nt) * BM;
       row_hi = (expert + 1) * g.rows_per_group;
+      // rows are numbered as stacked groups (the layout of the output); A may be laid out
+      // differently: shift its base so that stacked row numbers address the group's rows
+      a_adj = (int64_t)expert * (g.lda_e - (int64_t)g.rows_per_group * g.lda);
+      a_rows = row_hi;
     } else {
       // grouped (mixture-of-experts) mode, as in gemm_tile.hpp: the grid is an upper bound, only
       // the first real_tiles block ids are mapped; a tile covers rows of one expert
@@ -82,7 +88,7 @@ __global__ __launch_bounds__(256) void gemm_rs_kernel(GemmArgs g, Epi epi) {
   // ---- global -> register staging: thread -> (row = tid / 8 + 32 j, 16-byte chunk = tid % 8)
   const int ld_row = tid >> 3, ld_chunk = tid & 7;
   const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
-      (void*)g.a, 0, (int)((int64_t)(g.M - 1) * g.lda + g.K), 0x00020000);
+      (void*)(g.a + a_adj), 0, (int)((int64_t)(a_rows - 1) * g.lda + g.K), 0x00020000);
   const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(
       (void*)(g.b + (GROUPED ? (int64_t)expert * g.ldb_e : 0)), 0,
       (int)((int64_t)(g.N - 1) * g.ldb + g.K), 0x00020000);

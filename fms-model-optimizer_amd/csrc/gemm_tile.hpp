@@ -36,7 +36,9 @@ struct GemmArgs {
   const int32_t* offsets;
   int num_experts;
   int64_t ldb_e;  // bytes between experts in B
-  int rows_per_group;  // > 0: every group owns this many rows (batched matmul), offsets unused
+  int rows_per_group;  // > 0: every group owns this many rows (batched matmul, split K), offsets unused
+  int64_t lda_e;       // uniform groups: bytes between groups in A (rows * lda for stacked batches,
+                       // the K slice length when the groups are slices of one reduction)
 #ifdef FMSMO_CLK
   unsigned long long* clk;  // harness only: {core clock, 100 MHz wall clock} at start / end
 #endif
@@ -223,6 +225,7 @@ __global__ __launch_bounds__(WGM* WGN * 64, (Chk::enabled && (OP == MMA_I8 || Ch
 #endif
   int tile_m, tile_n;
   int row_lo = 0, row_hi = g.M, expert = 0;
+  int64_t a_adj = 0;
   if constexpr (GROUPED) {
     if (g.rows_per_group > 0) {
       // batched matmul: every group has the same number of rows, the grid is exact
@@ -231,6 +234,9 @@ __global__ __launch_bounds__(WGM* WGN * 64, (Chk::enabled && (OP == MMA_I8 || Ch
       expert = tile_m / nt;
       row_lo = expert * g.rows_per_group + (tile_m - expert * nt) * BM;
       row_hi = (expert + 1) * g.rows_per_group;
+      // rows are numbered as stacked groups (that is how the output is laid out); A may be laid
+      // out differently
+      a_adj = (int64_t)expert * (g.lda_e - (int64_t)g.rows_per_group * g.lda);
     } else {
       // The launch grid is an upper bound (the host cannot see the expert sizes).  Count the
       // real row tiles and map only the first real_tiles block ids, so that every XCD gets an
@@ -260,7 +266,7 @@ __global__ __launch_bounds__(WGM* WGN * 64, (Chk::enabled && (OP == MMA_I8 || Ch
   }
   const int col_lo = tile_n * BN;
 
-  const uint8_t* __restrict__ A = g.a;
+  const uint8_t* __restrict__ A = g.a + a_adj;
   const uint8_t* __restrict__ B = g.b + (GROUPED ? (int64_t)expert * g.ldb_e : 0);
 
   // ---- global -> LDS loader addressing (per thread, constant over the K loop)

@@ -33,6 +33,8 @@ SIGNATURES = {
     "fmsmo_gemm_i8_i32": [_P, _L, _P, _L, _P, _L, _L, _L, _L, _P],
     "fmsmo_gemm_i8_dq": [_P, _L, _P, _L, _P, _L, _P, _L, _P, _I, _I, _P, _I, _L, _L, _L, _L, _P],
     "fmsmo_gemm_fp8_dq": [_P, _L, _P, _L, _P, _L, _P, _L, _P, _I, _P, _I, _L, _L, _L, _L, _P],
+    "fmsmo_gemm_i8_dq_ws": [_P, _L, _P, _L, _P, _L, _P, _L, _P, _I, _I, _P, _I, _L, _L, _L, _L, _P, _L, _P],
+    "fmsmo_gemm_fp8_dq_ws": [_P, _L, _P, _L, _P, _L, _P, _L, _P, _I, _P, _I, _L, _L, _L, _L, _P, _L, _P],
     "fmsmo_gemv_i8_dq": [_P, _L, _P, _L, _P, _L, _P, _L, _P, _I, _I, _P, _I, _L, _L, _L, _L, _P],
     "fmsmo_gemv_fp8_dq": [_P, _L, _P, _L, _P, _L, _P, _L, _P, _I, _P, _I, _L, _L, _L, _L, _P],
     "fmsmo_matmul_chunk_i8": [_P, _L, _P, _L, _P, _P, _L, _L, _L, _L, _I, _I, _I, _I, _P],
@@ -50,6 +52,7 @@ OTHER = {
     "fmsmo_abi_version": ([], c_int),
     "fmsmo_status_str": ([c_int], c_char_p),
     "fmsmo_last_error": ([], c_char_p),
+    "fmsmo_gemm_workspace_bytes": ([c_int64, c_int64, c_int64], c_int64),
 }
 
 _lib = None

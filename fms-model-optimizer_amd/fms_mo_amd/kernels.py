@@ -143,6 +143,14 @@ def quant_act_fp8_pertoken(x, variant=L.FP8_LINEAR, static_scale=None):
 
 
 # ------------------------------------------------------------------------------------ GEMMs
+def _workspace(M, N, K, device):
+    """Scratch for the split-K form of the *_dq GEMMs (None when the shape does not use one).  It
+    comes from torch's caching allocator like every output, so it is also valid under graph
+    capture; the library itself never allocates."""
+    nbytes = L.load().fmsmo_gemm_workspace_bytes(M, N, K)
+    return torch.empty((nbytes,), dtype=torch.uint8, device=device) if nbytes > 0 else None
+
+
 def _check_ab(a, w, dtype):
     _need_gpu(a, w)
     if a.dtype != dtype or w.dtype != dtype:
@@ -178,12 +186,16 @@ def gemm_i8_dq(a, w, a_scale, w_scale, bias=None, out_dtype=torch.float16, exact
         if bias.numel() != N:
             raise ValueError("bias must have N elements")
     y = torch.empty((M, N), dtype=out_dtype, device=a.device)
-    fn = "fmsmo_gemv_i8_dq" if force_gemv else "fmsmo_gemm_i8_dq"
+    args = (a.data_ptr(), _ld(a), w.data_ptr(), _ld(w), a_scale.data_ptr(),
+            a_scale.numel(), w_scale.data_ptr(), w_scale.numel(), _ptr(bias),
+            _dt(bias) if bias is not None else 0, L.EPI_REF_F16 if exact_ref else L.EPI_F32,
+            y.data_ptr(), _DT[out_dtype], N, M, N, K)
+    ws = None if force_gemv else _workspace(M, N, K, a.device)
     with torch.cuda.device(a.device):
-        L.call(fn, a.data_ptr(), _ld(a), w.data_ptr(), _ld(w), a_scale.data_ptr(),
-               a_scale.numel(), w_scale.data_ptr(), w_scale.numel(), _ptr(bias),
-               _dt(bias) if bias is not None else 0, L.EPI_REF_F16 if exact_ref else L.EPI_F32,
-               y.data_ptr(), _DT[out_dtype], N, M, N, K, _stream(a))
+        if ws is not None:
+            L.call("fmsmo_gemm_i8_dq_ws", *args, ws.data_ptr(), ws.numel(), _stream(a))
+        else:
+            L.call("fmsmo_gemv_i8_dq" if force_gemv else "fmsmo_gemm_i8_dq", *args, _stream(a))
     return y
 
 
@@ -197,12 +209,15 @@ def gemm_fp8_dq(a, w, a_scale, w_scale, bias=None, out_dtype=torch.bfloat16, for
         _need_gpu(bias)
         bias = bias.detach().reshape(-1).contiguous()
     y = torch.empty((M, N), dtype=out_dtype, device=a.device)
-    fn = "fmsmo_gemv_fp8_dq" if force_gemv else "fmsmo_gemm_fp8_dq"
+    args = (a.data_ptr(), _ld(a), w.data_ptr(), _ld(w), a_scale.data_ptr(),
+            a_scale.numel(), w_scale.data_ptr(), w_scale.numel(), _ptr(bias),
+            _dt(bias) if bias is not None else 0, y.data_ptr(), _DT[out_dtype], N, M, N, K)
+    ws = None if force_gemv else _workspace(M, N, K, a.device)
     with torch.cuda.device(a.device):
-        L.call(fn, a.data_ptr(), _ld(a), w.data_ptr(), _ld(w), a_scale.data_ptr(),
-               a_scale.numel(), w_scale.data_ptr(), w_scale.numel(), _ptr(bias),
-               _dt(bias) if bias is not None else 0, y.data_ptr(), _DT[out_dtype], N, M, N, K,
-               _stream(a))
+        if ws is not None:
+            L.call("fmsmo_gemm_fp8_dq_ws", *args, ws.data_ptr(), ws.numel(), _stream(a))
+        else:
+            L.call("fmsmo_gemv_fp8_dq" if force_gemv else "fmsmo_gemm_fp8_dq", *args, _stream(a))
     return y
 
 

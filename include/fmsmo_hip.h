@@ -181,6 +181,31 @@ int fmsmo_gemm_fp8_dq(const uint8_t* a, int64_t lda, const uint8_t* b, int64_t l
                       int64_t w_scale_n, const void* bias, int bias_dtype, void* y, int y_dtype,
                       int64_t ldy, int64_t M, int64_t N, int64_t K, fmsmo_stream_t stream);
 
+/*
+ * The two *_dq GEMMs with a caller-provided workspace (the library allocates nothing).  When the
+ * output has few tiles and the reduction is long (16 < M <= 1024, at most 128 tiles of 128 x 128,
+ * K % 128 == 0: a batch of tens to hundreds of tokens through a projection with few output
+ * columns) the reduction is split into slices that run side by side and a second kernel adds the
+ * slices in a fixed order and applies the epilogue: 17 x 4096 x 14336 runs on 256 compute units
+ * instead of 32.  int32 partial sums are exact, so the int8 result is bit-identical to
+ * fmsmo_gemm_i8_dq's; the e4m3 result differs from fmsmo_gemm_fp8_dq's only by the order of the
+ * fp32 additions.  fmsmo_gemm_workspace_bytes returns the bytes a shape can use (0: no split);
+ * with workspace == NULL or fewer bytes the call is fmsmo_gemm_*_dq.  workspace: 16-byte aligned
+ * device memory, contents undefined before and after, private to the call while it runs.
+ * No counterpart in the reference (its GEMMs are single launches of CUTLASS / cuBLASLt kernels).
+ */
+int64_t fmsmo_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
+int fmsmo_gemm_i8_dq_ws(const int8_t* a, int64_t lda, const int8_t* b, int64_t ldb,
+                        const float* a_scale, int64_t a_scale_n, const float* w_scale,
+                        int64_t w_scale_n, const void* bias, int bias_dtype, int epilogue, void* y,
+                        int y_dtype, int64_t ldy, int64_t M, int64_t N, int64_t K, void* workspace,
+                        int64_t workspace_bytes, fmsmo_stream_t stream);
+int fmsmo_gemm_fp8_dq_ws(const uint8_t* a, int64_t lda, const uint8_t* b, int64_t ldb,
+                         const float* a_scale, int64_t a_scale_n, const float* w_scale,
+                         int64_t w_scale_n, const void* bias, int bias_dtype, void* y, int y_dtype,
+                         int64_t ldy, int64_t M, int64_t N, int64_t K, void* workspace,
+                         int64_t workspace_bytes, fmsmo_stream_t stream);
+
 /* ------------------------------------------------------------------------------------------
  * 3. Skinny-M (decode) variants, M <= 16: stream the weights once from HBM.
  *    Same arithmetic and arguments as the two *_dq GEMMs above.

@@ -485,3 +485,69 @@ def test_errors_are_raised_not_swallowed(dev):
         K().gemm_i8_i32(a.float(), w)
     with pytest.raises(RuntimeError):
         K().gemm_i8_i32(a.cpu(), w.cpu())
+
+
+# ------------------------------------------------------------------ split-K (workspace) GEMMs
+def _plain_i8_dq(a, w, a_s, w_s, bias, out_dtype, exact_ref):
+    """fmsmo_gemm_i8_dq without a workspace: the single-pass kernels."""
+    from fms_mo_amd import _lib as L
+    from fms_mo_amd import kernels as Kn
+
+    M, K = a.shape
+    N = w.shape[0]
+    y = torch.empty((M, N), dtype=out_dtype, device=a.device)
+    L.call("fmsmo_gemm_i8_dq", a.data_ptr(), K, w.data_ptr(), K, a_s.data_ptr(), a_s.numel(),
+           w_s.data_ptr(), w_s.numel(), None if bias is None else bias.data_ptr(),
+           Kn._DT[bias.dtype] if bias is not None else 0, L.EPI_REF_F16 if exact_ref else L.EPI_F32,
+           y.data_ptr(), Kn._DT[out_dtype], N, M, N, K, torch.cuda.current_stream().cuda_stream)
+    return y
+
+
+@pytest.mark.parametrize("shape", [(17, 4096, 14336), (64, 4096, 4096), (200, 1024, 1536), (512, 4096, 4096),
+                                   (100, 520, 2048), (128, 6144, 4096), (1000, 1024, 14336)])
+@pytest.mark.parametrize("exact_ref,out_dtype", [(True, torch.float16), (False, torch.bfloat16), (False, torch.float32)])
+def test_split_k_int8_is_bit_identical_to_single_pass(dev, shape, exact_ref, out_dtype):
+    from fms_mo_amd import _lib as L
+    from fms_mo_amd import kernels as Kn
+
+    M, N, Kd = shape
+    assert L.load().fmsmo_gemm_workspace_bytes(M, N, Kd) > 0
+    g = torch.Generator().manual_seed(91)
+    a = torch.randint(-128, 128, (M, Kd), generator=g, dtype=torch.int32).to(torch.int8).to(dev)
+    w = torch.randint(-128, 128, (N, Kd), generator=g, dtype=torch.int32).to(torch.int8).to(dev)
+    a_s = (torch.rand(M, generator=g) * 1e-2).to(dev)
+    w_s = (torch.rand(N, generator=g) * 1e-2).to(dev)
+    bias = torch.randn(N, generator=g).half().to(dev)
+    for b in (None, bias):
+        y = Kn.gemm_i8_dq(a, w, a_s, w_s, b, out_dtype=out_dtype, exact_ref=exact_ref)
+        ref = _plain_i8_dq(a, w, a_s, w_s, b, out_dtype, exact_ref)
+        assert torch.equal(y.view(torch.int16 if out_dtype != torch.float32 else torch.int32),
+                           ref.view(torch.int16 if out_dtype != torch.float32 else torch.int32))
+    # and against exact integer arithmetic on a sample of rows
+    acc = O.int_gemm(a[:5].cpu(), w.cpu())
+    exact = acc.double() * a_s[:5].cpu().double()[:, None] * w_s.cpu().double()[None, :]
+    y = Kn.gemm_i8_dq(a, w, a_s, w_s, None, out_dtype=torch.float32, exact_ref=False)
+    torch.testing.assert_close(y[:5].cpu().double(), exact, rtol=1e-6, atol=1e-6)
+
+
+@pytest.mark.parametrize("shape", [(17, 4096, 14336), (64, 4096, 4096), (200, 1024, 1536), (100, 520, 2048)])
+def test_split_k_fp8(dev, shape):
+    from fms_mo_amd import kernels as Kn
+
+    M, N, Kd = shape
+    g = torch.Generator().manual_seed(92)
+    # integer-valued operands: every partial sum is exact, so the split result is the exact product
+    a = torch.randint(-8, 9, (M, Kd), generator=g).float().to(torch.float8_e4m3fn).to(dev)
+    w = torch.randint(-8, 9, (N, Kd), generator=g).float().to(torch.float8_e4m3fn).to(dev)
+    one = torch.ones(1, device=dev)
+    y = Kn.gemm_fp8_dq(a, w, one, one, None, out_dtype=torch.float32)
+    ref = a.cpu().double() @ w.cpu().double().t()
+    assert torch.equal(y.cpu().double(), ref)
+    # general operands: within the tolerance of the fp8 path
+    a = torch.randn(M, Kd, generator=g).to(torch.float8_e4m3fn).to(dev)
+    w = torch.randn(N, Kd, generator=g).to(torch.float8_e4m3fn).to(dev)
+    a_s = (torch.rand(M, generator=g) + 0.5).to(dev)
+    w_s = (torch.rand(N, generator=g) + 0.5).to(dev)
+    y = Kn.gemm_fp8_dq(a, w, a_s, w_s, None, out_dtype=torch.bfloat16)
+    ref = (a.cpu().double() @ w.cpu().double().t()) * a_s.cpu().double()[:, None] * w_s.cpu().double()[None, :]
+    torch.testing.assert_close(y.cpu().double(), ref, rtol=1e-2, atol=1e-2 * ref.abs().max().item())

@@ -23,7 +23,8 @@ def test_header_declares_the_expected_entry_points():
               "fmsmo_gemv_fp8_dq", "fmsmo_matmul_chunk_i8", "fmsmo_matmul_chunk_fp",
               "fmsmo_grouped_gemm_i8_dq", "fmsmo_quant_weight_i8", "fmsmo_absmax_cols",
               "fmsmo_quant_act_i8_mulscale", "fmsmo_zero_shift_bias", "fmsmo_quant_i8_affine",
-              "fmsmo_bmm_i8_dq", "fmsmo_bmm_fp8_dq", "fmsmo_abi_version", "fmsmo_status_str", "fmsmo_last_error"]:
+              "fmsmo_bmm_i8_dq", "fmsmo_bmm_fp8_dq", "fmsmo_gemm_i8_dq_ws", "fmsmo_gemm_fp8_dq_ws",
+              "fmsmo_gemm_workspace_bytes", "fmsmo_abi_version", "fmsmo_status_str", "fmsmo_last_error"]:
         assert s in syms
 
 
@@ -89,3 +90,21 @@ def test_missing_library_fails_loudly(monkeypatch):
     monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libfmsmo_hip.so")
     with pytest.raises(_lib.FmsMoHipError, match="no fallback"):
         _lib.load()
+
+
+def test_workspace_plan_is_host_logic():
+    """Which shapes split their reduction is decided on the host: decode and large problems do
+    not, a batch of tokens through a projection with few output columns does, and the slices
+    divide K into multiples of 128 of at least 512."""
+    from fms_mo_amd import _lib
+
+    lib = _lib.load()
+    assert lib.fmsmo_gemm_workspace_bytes(1, 4096, 14336) == 0
+    assert lib.fmsmo_gemm_workspace_bytes(16, 4096, 14336) == 0
+    assert lib.fmsmo_gemm_workspace_bytes(4096, 4096, 14336) == 0
+    assert lib.fmsmo_gemm_workspace_bytes(64, 28672, 4096) == 0      # 224 tiles already
+    assert lib.fmsmo_gemm_workspace_bytes(64, 4096, 4000) == 0       # K not a multiple of 128
+    b = lib.fmsmo_gemm_workspace_bytes(64, 4096, 14336)
+    assert b > 0 and b % (64 * 4096 * 4) == 0
+    s = b // (64 * 4096 * 4)
+    assert 2 <= s <= 8 and 14336 % (s * 128) == 0 and 14336 // s >= 512
