@@ -51,7 +51,7 @@ static int gemm_i8_dq_impl(const int8_t* a, int64_t lda, const int8_t* b, int64_
   if (rc) return rc;
   if (epilogue != FMSMO_EPI_REF_F16 && epilogue != FMSMO_EPI_F32) return FMSMO_ERR_UNSUPPORTED;
   if (M == 0) return FMSMO_OK;
-  if (M <= 16 && K % 128 == 0)
+  if ((M <= 16 && K % 128 == 0) || fmsmo_gemv_batch_ok(M, K))
     return fmsmo_gemv_dispatch(FMSMO_OP_I8, a, lda, b, ldb, a_scale, a_scale_n, w_scale, w_scale_n,
                                bias, bias_dtype, epilogue, y, y_dtype, ldy, M, N, K,
                                (hipStream_t)stream);

@@ -11,7 +11,7 @@ static int gemm_fp8_dq_impl(const uint8_t* a, int64_t lda, const uint8_t* b, int
   rc = check_dq(a_scale, a_scale_n, w_scale, w_scale_n, bias, bias_dtype, y_dtype, M, N);
   if (rc) return rc;
   if (M == 0) return FMSMO_OK;
-  if (M <= 16 && K % 128 == 0)
+  if ((M <= 16 && K % 128 == 0) || fmsmo_gemv_batch_ok(M, K))
     return fmsmo_gemv_dispatch(FMSMO_OP_E4M3, a, lda, b, ldb, a_scale, a_scale_n, w_scale,
                                w_scale_n, bias, bias_dtype, FMSMO_EPI_F32, y, y_dtype, ldy, M, N, K,
                                (hipStream_t)stream);

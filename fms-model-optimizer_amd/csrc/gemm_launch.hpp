@@ -8,6 +8,7 @@
 using namespace fmsmo;
 
 int fmsmo_check_launch();
+bool fmsmo_gemv_batch_ok(int64_t M, int64_t K);
 int fmsmo_gemv_dispatch(int op, const void* a, int64_t lda, const void* b, int64_t ldb,
                         const float* a_scale, int64_t a_scale_n, const float* w_scale,
                         int64_t w_scale_n, const void* bias, int bias_dtype, int epilogue,

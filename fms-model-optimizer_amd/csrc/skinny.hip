@@ -125,13 +125,16 @@ __global__ __launch_bounds__(NW * 64) void gemv_kernel(GemvArgs g) {
 // ds_read_b128 of the operand fragments).  D steps of loads stay in flight in registers; nothing
 // is shared between waves except the final 16x16 partial sums, so the only barrier is one per
 // group of 16 rows.  The activation fragments of the wave's K slice stay in registers.
-template <int OP, int STEPS, int NW, int D>
+// MT > 1: batches of up to 16 MT tokens.  The weight stream is the same; every step feeds MT
+// MFMAs (one per tile of 16 tokens) from the same weight fragment, so up to 64 tokens cost little
+// more than 16 as long as their activation fragments fit in registers (MT * STEPS * 8 VGPRs).
+template <int OP, int STEPS, int NW, int D, int MT = 1>
 __global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(GemvArgs g, int G) {
   static_assert(STEPS % D == 0, "pipeline depth must divide the steps per group");
   typedef typename std::conditional<OP == FMSMO_OP_I8, int, float>::type AccT;
   typedef AccT Acc4 __attribute__((ext_vector_type(4)));
   __shared__ __attribute__((aligned(16))) uint8_t stage[NW][2][2048];
-  __shared__ AccT red[2][NW][256];
+  __shared__ AccT red[2][NW][256 * MT];
 
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -142,13 +145,14 @@ __global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(GemvArgs g, int G)
   const int kwave = wave * (STEPS * 128);
 
   // activation fragments: lane (m = r, kg) holds x[m][kwave + s*128 + (h*4 + kg)*16 ...]
-  v4i xf[STEPS][2];
-  {
-    const uint8_t* xp = g.a + (int64_t)min(r, g.M - 1) * g.lda + kwave + kg * 16;
+  v4i xf[MT][STEPS][2];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    const uint8_t* xp = g.a + (int64_t)min(t * 16 + r, g.M - 1) * g.lda + kwave + kg * 16;
 #pragma unroll
     for (int s = 0; s < STEPS; ++s) {
-      xf[s][0] = *(const v4i*)(xp + s * 128);
-      xf[s][1] = *(const v4i*)(xp + s * 128 + 64);
+      xf[t][s][0] = *(const v4i*)(xp + s * 128);
+      xf[t][s][1] = *(const v4i*)(xp + s * 128 + 64);
     }
   }
   // weight loads: lane -> (row = lane / 8 [+8], 16-byte chunk = lane % 8): 8 rows x 128 B each
@@ -192,7 +196,9 @@ __global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(GemvArgs g, int G)
            : g.bias_dtype == FMSMO_BF16 ? bf16_to_f32(((const u16*)g.bias)[en])
                                         : ((const float*)g.bias)[en];
     }
-    Acc4 acc = {0, 0, 0, 0};
+    Acc4 acc[MT];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) acc[t] = Acc4{0, 0, 0, 0};
 #pragma unroll
     for (int s = 0; s < STEPS; ++s) {
       uint8_t* st = &stage[wave][s & 1][0];
@@ -203,14 +209,17 @@ __global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(GemvArgs g, int G)
       __builtin_amdgcn_sched_barrier(0);
       const v4i w0 = *(const v4i*)(st + rd0);
       const v4i w1 = *(const v4i*)(st + rd1);
-      if constexpr (OP == FMSMO_OP_I8) {
-        acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(w0, xf[s][0], acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(w1, xf[s][1], acc, 0, 0, 0);
-      } else {
-        const v8i wv = {w0[0], w0[1], w0[2], w0[3], w1[0], w1[1], w1[2], w1[3]};
-        const v8i xv = {xf[s][0][0], xf[s][0][1], xf[s][0][2], xf[s][0][3],
-                        xf[s][1][0], xf[s][1][1], xf[s][1][2], xf[s][1][3]};
-        acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wv, xv, acc, 0, 0, 0, 0, 0, 0);
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        if constexpr (OP == FMSMO_OP_I8) {
+          acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w0, xf[t][s][0], acc[t], 0, 0, 0);
+          acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w1, xf[t][s][1], acc[t], 0, 0, 0);
+        } else {
+          const v8i wv = {w0[0], w0[1], w0[2], w0[3], w1[0], w1[1], w1[2], w1[3]};
+          const v8i xv = {xf[t][s][0][0], xf[t][s][0][1], xf[t][s][0][2], xf[t][s][0][3],
+                          xf[t][s][1][0], xf[t][s][1][1], xf[t][s][1][2], xf[t][s][1][3]};
+          acc[t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wv, xv, acc[t], 0, 0, 0, 0, 0, 0);
+        }
       }
     }
     // acc[v] = partial C(n = 16 (group0+gi) + 4 kg + v, m = r) of this wave's K slice.  The NW
@@ -222,26 +231,38 @@ __global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(GemvArgs g, int G)
     }
     AccT* mine = &red[gi & 1][wave][0];
 #pragma unroll
-    for (int v = 0; v < 4; ++v) mine[(kg * 4 + v) * 16 + r] = acc[v];
+    for (int t = 0; t < MT; ++t)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) mine[t * 256 + (kg * 4 + v) * 16 + r] = acc[t][v];
     __syncthreads();
-    if (threadIdx.x < 256) {
-      const int e = threadIdx.x;
+    auto finish = [&](int e, float as_e, float ws_e, float bv_e) {
       AccT sum = red[gi & 1][0][e];
 #pragma unroll
       for (int w = 1; w < NW; ++w) sum += red[gi & 1][w][e];
-      const int n = (group0 + gi) * 16 + (e >> 4), m = e & 15;
+      const int n = (group0 + gi) * 16 + ((e >> 4) & 15), m = (e >> 8) * 16 + (e & 15);
       if (n < g.N && m < g.M) {
         float out;
         if (g.ref_f16) {
-          const float sc = round_to<FMSMO_F16>(__fmul_rn(as, ws));
-          out = round_to<FMSMO_F16>(__fadd_rn(__fmul_rn((float)sum, sc), bv));
+          const float sc = round_to<FMSMO_F16>(__fmul_rn(as_e, ws_e));
+          out = round_to<FMSMO_F16>(__fadd_rn(__fmul_rn((float)sum, sc), bv_e));
         } else {
-          out = __fmaf_rn((float)sum, __fmul_rn(as, ws), bv);
+          out = __fmaf_rn((float)sum, __fmul_rn(as_e, ws_e), bv_e);
         }
         const int64_t idx = (int64_t)m * g.ldy + n;
         if (g.y_dtype == FMSMO_F16) ((u16*)g.y)[idx] = f32_to_f16(out);
         else if (g.y_dtype == FMSMO_BF16) ((u16*)g.y)[idx] = f32_to_bf16(out);
         else ((float*)g.y)[idx] = out;
+      }
+    };
+    if constexpr (MT == 1) {
+      if (threadIdx.x < 256) finish(threadIdx.x, as, ws, bv);
+    } else {
+      // the column of output e is that of thread e % 256 (already fetched: ws, bv); its token row
+      // differs per tile, so the token scale is fetched here
+      static_assert(MT == 1 || (NW * 64) % 256 == 0, "outputs of a thread must share its column");
+      for (int e = threadIdx.x; e < 256 * MT; e += NW * 64) {
+        const int m = min((e >> 8) * 16 + (e & 15), g.M - 1);
+        finish(e, g.a_scale[g.a_stride ? m : 0], ws, bv);
       }
     }
   };
@@ -385,6 +406,16 @@ static void launch_gemv(const GemvArgs& g, int nw, hipStream_t st) {
   }
 }
 
+// Batches of 17 .. 64 tokens that the weight-streaming kernel takes in one pass (their
+// activation fragments must fit in registers): K = 1024 * {1, 2, 4, 8} up to 32 tokens,
+// K = 1024 * {1, 2, 4} up to 64.
+bool fmsmo_gemv_batch_ok(int64_t M, int64_t K) {
+  if (M <= 16 || M > 64 || K % 1024) return false;
+  const int64_t steps = K / 1024;
+  if (steps != 1 && steps != 2 && steps != 4 && steps != 8) return false;
+  return M <= 32 || steps <= 4;
+}
+
 int fmsmo_gemv_dispatch(int op, const void* a, int64_t lda, const void* b, int64_t ldb,
                         const float* a_scale, int64_t a_scale_n, const float* w_scale,
                         int64_t w_scale_n, const void* bias, int bias_dtype, int epilogue,
@@ -453,8 +484,13 @@ int fmsmo_gemv_dispatch(int op, const void* a, int64_t lda, const void* b, int64
     if (G > 64) G = 64;
     dim3 grid((unsigned)((groups + G - 1) / G)), block(NW * 64);
     bool handled = true;
-#define GEMV_STREAM(OPV, NWV, ST, DV) \
-  hipLaunchKernelGGL((gemv_stream_kernel<OPV, ST, NWV, DV>), grid, block, 0, st, g, G)
+#define GEMV_STREAM(OPV, NWV, ST, DV)                                                             \
+  if (M <= 16) hipLaunchKernelGGL((gemv_stream_kernel<OPV, ST, NWV, DV>), grid, block, 0, st, g, G); \
+  else if constexpr (NWV == 8 && ST <= 8) {                                                        \
+    if (M <= 32) hipLaunchKernelGGL((gemv_stream_kernel<OPV, ST, NWV, DV, 2>), grid, block, 0, st, g, G); \
+    else if constexpr (ST <= 4) hipLaunchKernelGGL((gemv_stream_kernel<OPV, ST, NWV, DV, 4>), grid, block, 0, st, g, G); \
+    else handled = false;                                                                          \
+  } else handled = false
 #define GEMV_SHAPES(OPV)                                            \
   switch (NW * 100 + STEPS) {                                       \
     case 801: GEMV_STREAM(OPV, 8, 1, 1); break;                     \
@@ -471,6 +507,7 @@ int fmsmo_gemv_dispatch(int op, const void* a, int64_t lda, const void* b, int64
 #undef GEMV_STREAM
     if (handled) return fmsmo_check_launch();
   }
+  if (M > 16) return FMSMO_ERR_UNSUPPORTED;  // callers ask fmsmo_gemv_batch_ok first
   int nw = 8;
   while (nw > 1 && K % (128 * nw)) nw >>= 1;
   // enough row groups per block to amortise the activation re-reads, while keeping >= 2 blocks

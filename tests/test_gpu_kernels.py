@@ -551,3 +551,47 @@ def test_split_k_fp8(dev, shape):
     y = Kn.gemm_fp8_dq(a, w, a_s, w_s, None, out_dtype=torch.bfloat16)
     ref = (a.cpu().double() @ w.cpu().double().t()) * a_s.cpu().double()[:, None] * w_s.cpu().double()[None, :]
     torch.testing.assert_close(y.cpu().double(), ref, rtol=1e-2, atol=1e-2 * ref.abs().max().item())
+
+
+# ------------------------------------------------------------------ 17 .. 64 tokens, one weight pass
+@pytest.mark.parametrize("M", [17, 24, 32, 33, 48, 64])
+@pytest.mark.parametrize("NK", [(4096, 4096), (520, 1024), (1000, 2048), (256, 8192), (6144, 4096)])
+def test_batched_decode_i8_bit_exact(dev, M, NK):
+    """Batches of up to 64 tokens run through the weight-streaming kernel where their activation
+    fragments fit in registers (K = 1024, 2048, 4096; 8192 up to 32 tokens) and through the tiled /
+    split-K kernels otherwise; every route returns the reference epilogue bit for bit."""
+    N, Kd = NK
+    a, w = _rand_i8((M, Kd), 131), _rand_i8((N, Kd), 132)
+    s_a = (torch.rand(M, 1, generator=gen(133)) * 0.05 + 1e-3).half()
+    s_w = (torch.rand(N, generator=gen(134)) * 1e-3 + 1e-5).float()
+    bias = (torch.randn(N, generator=gen(135)) * 0.01).half()
+    acc = O.int_gemm(a, w)
+    ref = O.epilogue_ref(acc, s_a, s_w, bias, torch.float16)
+    y = K().gemm_i8_dq(a.to(dev), w.to(dev), s_a.float().to(dev), s_w.to(dev), bias.to(dev),
+                       out_dtype=torch.float16, exact_ref=True)
+    assert torch.equal(y.cpu().view(torch.int16), ref.view(torch.int16))
+    # without a bias the kernels add +0.0 (the reference always adds a bias tensor): equal as values
+    y = K().gemm_i8_dq(a.to(dev), w.to(dev), s_a.float().to(dev), s_w.to(dev), None,
+                       out_dtype=torch.float16, exact_ref=True)
+    assert torch.equal(y.cpu(), O.epilogue_ref(acc, s_a, s_w, None, torch.float16))
+    y32 = K().gemm_i8_dq(a.to(dev), w.to(dev), torch.ones(1, device=dev), torch.ones(1, device=dev), None,
+                         out_dtype=torch.float32, exact_ref=False)
+    assert torch.equal(y32.cpu().double(), acc.double())
+
+
+@pytest.mark.parametrize("M", [17, 32, 40, 64])
+@pytest.mark.parametrize("NK", [(4096, 4096), (520, 1024), (256, 8192)])
+def test_batched_decode_fp8(dev, M, NK):
+    N, Kd = NK
+    a = torch.randint(-8, 9, (M, Kd), generator=gen(141)).float().to(torch.float8_e4m3fn)
+    w = torch.randint(-8, 9, (N, Kd), generator=gen(142)).float().to(torch.float8_e4m3fn)
+    one = torch.ones(1, device=dev)
+    y = K().gemm_fp8_dq(a.to(dev), w.to(dev), one, one, None, out_dtype=torch.float32)
+    assert torch.equal(y.cpu().double(), a.double() @ w.double().t())  # integer-valued operands: exact
+    a, w = _rand_fp8((M, Kd), 143, 2.0), _rand_fp8((N, Kd), 144, 0.5)
+    s_a = torch.rand(M, generator=gen(145)) * 0.05 + 1e-3
+    s_w = torch.rand(N, generator=gen(146)) * 0.01 + 1e-4
+    bias = (torch.randn(N, generator=gen(147)) * 0.1).bfloat16()
+    exact = (a.double() @ w.double().t()) * s_a.double()[:, None] * s_w.double()[None, :] + bias.double()
+    y = K().gemm_fp8_dq(a.to(dev), w.to(dev), s_a.to(dev), s_w.to(dev), bias.to(dev), out_dtype=torch.bfloat16)
+    torch.testing.assert_close(y.cpu().double(), exact, rtol=1e-2, atol=1e-2 * exact.abs().max().item())
