@@ -192,7 +192,7 @@ def main():
 
 
 def extras(torch, K, dev):
-    """FP8 GEMMs (Granite-3-8B-like shapes, M=2048), decode shapes (M in 1,4,16), the Mixtral-style
+    """FP8 GEMMs (Granite-3-8B-like shapes, M=2048), decode shapes (M in 1 .. 128), the Mixtral-style
     grouped expert GEMMs and the chunk-truncate emulation; reported in addition to the headline
     value."""
     from fms_mo_amd import _lib as L
@@ -229,7 +229,7 @@ def extras(torch, K, dev):
         copies = max(3, (300 * 1024 * 1024 + wbytes - 1) // wbytes)
         ws_i8 = [torch.randint(-127, 128, (n, k), dtype=torch.int8, device=dev) for _ in range(copies)]
         wsc = torch.rand(n, device=dev) * 1e-3
-        for M in (1, 4, 16):
+        for M in (1, 4, 16, 32, 64, 128):  # decode kernels up to 64 (K <= 4096), tiled / split-K above
             x = torch.randn(M, k, device=dev).bfloat16()
             q, s = K.quant_act_i8_pertoken(x)
             side = torch.cuda.Stream()
