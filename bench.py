@@ -257,6 +257,53 @@ def extras(torch, K, dev):
             res[f"decode_i8_M{M}_{name}"] = {"us": round(ms * 1e3, 2), "GBps": round(gbs, 1), "frac_hbm": round(gbs / PEAK_HBM_GBS, 4)}
             del graph
         del ws_i8
+    # a whole decode-step linear from fp16 activations (SmoothQuant divide, per-token quantizer,
+    # weight-streaming matmul, dequantizing epilogue): two launches against the fused one
+    for name, k, n in LLAMA3_8B:
+        wbytes = k * n
+        copies = max(3, (300 * 1024 * 1024 + wbytes - 1) // wbytes)
+        ws_i8 = [torch.randint(-127, 128, (n, k), dtype=torch.int8, device=dev) for _ in range(copies)]
+        wsc = torch.rand(n, device=dev) * 1e-3
+        sm = (torch.rand(k, device=dev) + 0.5).half()
+        for M in (1,):
+            x = torch.randn(M, k, device=dev).half()
+
+            def two(w):
+                q, s = K.quant_act_i8_pertoken(x, sm)
+                return K.gemm_i8_dq(q, w, s, wsc, None, out_dtype=torch.float16, exact_ref=True)
+
+            def one(w):  # the fused launch where it is served (K <= 8192), else the same two
+                if not K.decode_linear_ok(x, sm, k):
+                    return two(w)
+                return K.decode_linear_i8(x, w, wsc, None, sm, out_dtype=torch.float16, exact_ref=True)[0]
+
+            us = {}
+            for label, fn in (("two_launches", two), ("fused", one)):
+                side = torch.cuda.Stream()
+                with torch.cuda.stream(side):
+                    for w in ws_i8:
+                        fn(w)
+                    torch.cuda.synchronize()
+                    graph = torch.cuda.CUDAGraph()
+                    with torch.cuda.graph(graph, stream=side):
+                        for _ in range(3):
+                            for w in ws_i8:
+                                fn(w)
+                    graph.replay()
+                    torch.cuda.synchronize()
+                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    e0.record()
+                    for _ in range(5):
+                        graph.replay()
+                    e1.record()
+                    torch.cuda.synchronize()
+                us[label] = e0.elapsed_time(e1) / (5 * 3 * copies) * 1e3
+                del graph
+            res[f"decode_linear_fp16_in_M{M}_{name}"] = {
+                "two_launches_us": round(us["two_launches"], 2), "fused_us": round(us["fused"], 2),
+                "fused_GBps": round(wbytes / us["fused"] / 1e3, 1),
+                "frac_hbm": round(wbytes / us["fused"] / 1e3 / PEAK_HBM_GBS, 4)}
+        del ws_i8
     # Mixtral-style MoE (8 experts, 4096 tokens routed top-2 with uniform-random logits) in one
     # grouped launch per projection, and the chunk-truncate emulation on one expert's w2
     E, T, H, I = 8, 4096, 4096, 14336

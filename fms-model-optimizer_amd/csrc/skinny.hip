@@ -12,7 +12,7 @@
 //     do the dot products, so the vector ALUs stay free and the loop is pure load + MFMA;
 //   * the NW partial 16x16 blocks are reduced through LDS and dequantized by the first 256
 //     threads.
-#include "common.hpp"
+#include "quant_math.hpp"
 
 namespace fmsmo {
 
@@ -30,7 +30,105 @@ struct GemvArgs {
   void* y;
   int y_dtype;
   int64_t ldy;
+  // fused decode linear: the activations arrive unquantized (fp16 / bf16) and every block
+  // quantizes them itself
+  const u16* x16;       // [M,K]
+  int64_t ldx;
+  const u16* smooth;    // [K] SmoothQuant divisors of x's dtype, or NULL
+  int saturate;
+  float* a_scale_out;   // [M] per-token scales (written by block 0), or NULL
 };
+
+// Per-token int8 quantization of up to MAXM token rows by all NT threads of a block, into LDS:
+// the arithmetic of the stand-alone quantizer for a 16-bit compute dtype T (divide by the
+// SmoothQuant scale, row maximum, s = rnd_T(max(amax, rnd_T(1e-5)) / 127), rint(rnd_T(x / s)),
+// exact quotients from reciprocals, rows or divisors outside the fast path's range redone with
+// IEEE divisions).  A decode step has a handful of tokens: quantizing them again in every block
+// costs a few KB of L2 reads and saves a kernel launch in front of every linear layer.
+template <int T, int NT, int KMAX, int MAXM>
+__device__ __forceinline__ void quantize_rows_to_lds(const GemvArgs& g, uint8_t (*xq)[KMAX], float* sc,
+                                                     float* red) {
+  constexpr int NCH = (KMAX / AQ_VEC + NT - 1) / NT;
+  const int nchunk = g.K / AQ_VEC;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  constexpr uint32_t INF_BITS = T == FMSMO_F16 ? 0x7c00u : 0x7f80u;
+  const float floor_T = cvt16<T>(to16<T>(1e-5f));
+  const float sat_hi = g.saturate ? 127.0f : 3.0e38f;
+  for (int m = 0; m < g.M; ++m) {
+    const u16* xr = g.x16 + (size_t)m * g.ldx;
+    v4i cur[NCH];
+    int bad = 0;
+    us2 amax2 = {0, 0};
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      const int c = threadIdx.x + i * NT;
+      if (c < nchunk) {
+        cur[i] = *(const v4i*)(xr + (size_t)c * AQ_VEC);
+        if (g.smooth) {
+          const v4i sm = *(const v4i*)(g.smooth + (size_t)c * AQ_VEC);
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const uint32_t w = (uint32_t)cur[i][j], d = (uint32_t)sm[j];
+            const float dl = cvt16<T>((u16)(d & 0xffff)), dh = cvt16<T>((u16)(d >> 16));
+            if constexpr (T == FMSMO_BF16)
+              bad |= !(fabsf(dl) >= 8.6736174e-19f && fabsf(dl) <= 1.1529215e18f) ||
+                     !(fabsf(dh) >= 8.6736174e-19f && fabsf(dh) <= 1.1529215e18f);
+            const u16 el = to16<T>(div16<T, false>(cvt16<T>((u16)(w & 0xffff)), dl, __builtin_amdgcn_rcpf(dl)));
+            const u16 eh = to16<T>(div16<T, false>(cvt16<T>((u16)(w >> 16)), dh, __builtin_amdgcn_rcpf(dh)));
+            cur[i][j] = (int)((uint32_t)el | ((uint32_t)eh << 16));
+          }
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const uint32_t mag = (uint32_t)cur[i][j] & 0x7fff7fffu;
+          us2 m2;
+          __builtin_memcpy(&m2, &mag, 4);
+          amax2 = __builtin_elementwise_max(amax2, m2);
+        }
+      }
+    }
+    // non-negative floats order like their bit patterns (a NaN outranks inf)
+    // (a divisor outside the fast path's range marks the row for the IEEE routine)
+    float v = wave_max(__uint_as_float(bad ? 0xffffu : (uint32_t)(amax2[0] > amax2[1] ? amax2[0] : amax2[1])));
+    if (lane == 0) red[wave] = v;
+    __syncthreads();
+    v = red[0];
+#pragma unroll
+    for (int w = 1; w < NT / 64; ++w) v = fmaxf(v, red[w]);
+    __syncthreads();
+    const uint32_t abits = __float_as_uint(v);
+    if (abits >= INF_BITS) {
+      quant_i8_row_ieee16<T, NT>(xr, g.smooth, g.saturate, (int8_t*)xq[m], sc + m, g.K, red);
+      continue;
+    }
+    const float s = cvt16<T>(to16<T>(fmaxf(cvt16<T>((u16)abits), floor_T) / 127.0f));
+    const float rs = __builtin_amdgcn_rcpf(s);
+    if (threadIdx.x == 0) sc[m] = s;
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      const int c = threadIdx.x + i * NT;
+      if (c < nchunk) {
+        uint32_t code[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const uint32_t w = (uint32_t)cur[i][j];
+          float ql = div16<T, false>(cvt16<T>((u16)(w & 0xffff)), s, rs);
+          float qh = div16<T, false>(cvt16<T>((u16)(w >> 16)), s, rs);
+          if (g.saturate) {
+            ql = fminf(fmaxf(ql, -sat_hi), sat_hi);
+            qh = fminf(fmaxf(qh, -sat_hi), sat_hi);
+          }
+          code[j] = rint_codes<T>(to16<T>(ql), to16<T>(qh));
+        }
+        const uint32_t o0 = __builtin_amdgcn_perm(code[1], code[0], 0x06040200u);
+        const uint32_t o1 = __builtin_amdgcn_perm(code[3], code[2], 0x06040200u);
+        *(uint2*)(&xq[m][(size_t)c * AQ_VEC]) = make_uint2(o0, o1);
+      }
+    }
+  }
+  __syncthreads();
+  if (blockIdx.x == 0 && g.a_scale_out && threadIdx.x < g.M) g.a_scale_out[threadIdx.x] = sc[threadIdx.x];
+}
 
 template <int OP, int RG, int NW>
 __global__ __launch_bounds__(NW * 64) void gemv_kernel(GemvArgs g) {
@@ -135,7 +233,6 @@ __global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(GemvArgs g, int G)
   typedef AccT Acc4 __attribute__((ext_vector_type(4)));
   __shared__ __attribute__((aligned(16))) uint8_t stage[NW][2][2048];
   __shared__ AccT red[2][NW][256 * MT];
-
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int r = lane & 15, kg = lane >> 4;
@@ -277,13 +374,43 @@ __global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(GemvArgs g, int G)
 // accumulated with FMAs), and reduces the 64 partial sums with a butterfly.  U rows are in
 // flight per wave; rows are dealt to waves so that neighbouring waves read neighbouring rows.
 // KCH = ceil(K / 1024) chunks per lane; chunks past K are zero.
-template <int OP, int MR, int KCH, int U>
+template <int OP, int MR, int KCH, int U, int XT = -1>
 __global__ __launch_bounds__(256) void gemv_rows_kernel(GemvArgs g) {
   typedef typename std::conditional<OP == FMSMO_OP_I8, int, float>::type AccT;
+  // XT >= 0 (FMSMO_F16 / FMSMO_BF16): fused decode linear -- the block first quantizes the
+  // unquantized activations into LDS (quantize_rows_to_lds) and then takes its chunks and token
+  // scales from there instead of from global memory
+  constexpr bool FUSED = XT >= 0;
+  __shared__ __attribute__((aligned(16))) uint8_t xq[FUSED ? MR : 1][FUSED ? KCH * 1024 : 16];
+  __shared__ float xsc[4];
+  __shared__ float xred[4];
   const int lane = threadIdx.x & 63;
   const int wave_g = blockIdx.x * 4 + (threadIdx.x >> 6);
   const int nwaves = gridDim.x * 4;
   const int kchunks = g.K >> 4;
+
+  auto load_w = [&](int n0, v4i (&w)[U][KCH]) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const uint8_t* wp = g.b + (int64_t)min(n0 + u, g.N - 1) * g.ldb;
+#pragma unroll
+      for (int c = 0; c < KCH; ++c) {
+        const int ch = c * 64 + lane;
+        // chunks past K: re-read the row's first chunk; the zero activation chunk cancels it
+        w[u][c] = __builtin_nontemporal_load((const v4i*)(wp + (int64_t)(ch < kchunks ? ch : lane % kchunks) * 16));
+      }
+    }
+  };
+  v4i w[U][KCH];
+  if constexpr (FUSED) {
+    // the weights of the first turn are in flight while the block quantizes its activations
+    load_w(wave_g * U, w);
+    quantize_rows_to_lds<XT, 256, KCH * 1024, MR>(g, xq, xsc, xred);
+    g.a = &xq[0][0];
+    g.lda = KCH * 1024;
+    g.a_scale = xsc;
+    g.a_stride = 1;
+  }
 
   v4i xr[MR][KCH];
 #pragma unroll
@@ -297,17 +424,7 @@ __global__ __launch_bounds__(256) void gemv_rows_kernel(GemvArgs g) {
   }
 
   for (int n0 = wave_g * U; n0 < g.N; n0 += nwaves * U) {
-    v4i w[U][KCH];
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const uint8_t* wp = g.b + (int64_t)min(n0 + u, g.N - 1) * g.ldb;
-#pragma unroll
-      for (int c = 0; c < KCH; ++c) {
-        const int ch = c * 64 + lane;
-        // chunks past K: re-read the row's first chunk; the zero activation chunk cancels it
-        w[u][c] = __builtin_nontemporal_load((const v4i*)(wp + (int64_t)(ch < kchunks ? ch : lane % kchunks) * 16));
-      }
-    }
+    if (!FUSED || n0 != wave_g * U) load_w(n0, w);
     AccT acc[U][MR];
 #pragma unroll
     for (int u = 0; u < U; ++u)
@@ -524,6 +641,65 @@ int fmsmo_gemv_dispatch(int op, const void* a, int64_t lda, const void* b, int64
     else launch_gemv<FMSMO_OP_E4M3, 1>(g, nw, st);
   }
   return fmsmo_check_launch();
+}
+
+// ---------------------------------------------------------------------- fused decode linear
+// One token and K <= 8192 (measured from a HIP graph against the two launches, us: qkv 9.6 -> 8.3,
+// o 8.1 -> 6.3, gate+up 23.4 -> 19.7).  With more tokens or longer rows the quantization every
+// block repeats costs more than the launch it saves (K = 14336: 16.5 -> 19.6; two tokens at
+// K = 4096: 10.3 -> 10.9), so those shapes are left to the two kernels.
+extern "C" int fmsmo_decode_linear_ok(int64_t M, int64_t K) {
+  if (M != 1 || K % 128 || K < 1024) return 0;
+  const int kch = (int)((K + 1023) / 1024);
+  return kch == 1 || kch == 2 || kch == 4 || kch == 8;
+}
+
+template <int XT>
+static int decode_fused_launch(const GemvArgs& g, hipStream_t st) {
+  const int kch = (int)((g.K + 1023) / 1024);
+#define ROWS(KCHV, UV)                                                                            \
+  {                                                                                                \
+    const int64_t blocks = ((int64_t)g.N + 4 * UV - 1) / (4 * UV);                                 \
+    dim3 grid((unsigned)(blocks < 1024 ? blocks : 1024));                                          \
+    hipLaunchKernelGGL((gemv_rows_kernel<FMSMO_OP_I8, 1, KCHV, UV, XT>), grid, dim3(256), 0, st, g); \
+  }
+  switch (kch) {
+    case 1: ROWS(1, 8) break;
+    case 2: ROWS(2, 8) break;
+    case 4: ROWS(4, 4) break;
+    case 8: ROWS(8, 2) break;
+    default: return FMSMO_ERR_UNSUPPORTED;
+  }
+#undef ROWS
+  return fmsmo_check_launch();
+}
+
+extern "C" int fmsmo_decode_linear_i8(const void* x, int x_dtype, int64_t ldx, const void* smooth,
+                                      int saturate, const int8_t* w, int64_t ldw,
+                                      const float* w_scale, int64_t w_scale_n, const void* bias,
+                                      int bias_dtype, int epilogue, void* y, int y_dtype,
+                                      int64_t ldy, float* a_scale_out, int64_t M, int64_t N,
+                                      int64_t K, fmsmo_stream_t stream) {
+  if (!x || !w || !w_scale || !y) return FMSMO_ERR_NULL;
+  if (M <= 0 || N <= 0 || K <= 0 || ldx < K || ldw < K || ldy < N) return FMSMO_ERR_SHAPE;
+  if (w_scale_n != 1 && w_scale_n != N) return FMSMO_ERR_SHAPE;
+  if ((x_dtype != FMSMO_F16 && x_dtype != FMSMO_BF16) || !fmsmo_decode_linear_ok(M, K)) return FMSMO_ERR_UNSUPPORTED;
+  if (N >= (1 << 30) || N * ldw >= (1ll << 40)) return FMSMO_ERR_UNSUPPORTED;
+  if (y_dtype < 0 || y_dtype > 2 || (bias && (bias_dtype < 0 || bias_dtype > 2))) return FMSMO_ERR_UNSUPPORTED;
+  if (epilogue != FMSMO_EPI_REF_F16 && epilogue != FMSMO_EPI_F32) return FMSMO_ERR_UNSUPPORTED;
+  if (ldx % 8 || ldw % 16 || (((uintptr_t)x) & 15) || (((uintptr_t)w) & 15) ||
+      (smooth && (((uintptr_t)smooth) & 15)))
+    return FMSMO_ERR_ALIGN;
+  GemvArgs g{};
+  g.b = (const uint8_t*)w; g.ldb = ldw;
+  g.M = (int)M; g.N = (int)N; g.K = (int)K;
+  g.w_scale = w_scale; g.w_stride = w_scale_n == 1 ? 0 : 1;
+  g.bias = bias; g.bias_dtype = bias_dtype; g.ref_f16 = epilogue == FMSMO_EPI_REF_F16;
+  g.y = y; g.y_dtype = y_dtype; g.ldy = ldy;
+  g.x16 = (const u16*)x; g.ldx = ldx; g.smooth = (const u16*)smooth; g.saturate = saturate;
+  g.a_scale_out = a_scale_out;
+  return x_dtype == FMSMO_F16 ? decode_fused_launch<FMSMO_F16>(g, (hipStream_t)stream)
+                              : decode_fused_launch<FMSMO_BF16>(g, (hipStream_t)stream);
 }
 
 static int check_gemv(const void* a, int64_t lda, const void* b, int64_t ldb, const float* a_scale,

@@ -37,6 +37,7 @@ SIGNATURES = {
     "fmsmo_gemm_fp8_dq_ws": [_P, _L, _P, _L, _P, _L, _P, _L, _P, _I, _P, _I, _L, _L, _L, _L, _P, _L, _P],
     "fmsmo_gemv_i8_dq": [_P, _L, _P, _L, _P, _L, _P, _L, _P, _I, _I, _P, _I, _L, _L, _L, _L, _P],
     "fmsmo_gemv_fp8_dq": [_P, _L, _P, _L, _P, _L, _P, _L, _P, _I, _P, _I, _L, _L, _L, _L, _P],
+    "fmsmo_decode_linear_i8": [_P, _I, _L, _P, _I, _P, _L, _P, _L, _P, _I, _I, _P, _I, _L, _P, _L, _L, _L, _P],
     "fmsmo_matmul_chunk_i8": [_P, _L, _P, _L, _P, _P, _L, _L, _L, _L, _I, _I, _I, _I, _P],
     "fmsmo_matmul_chunk_fp": [_P, _L, _P, _L, _I, _P, _P, _L, _L, _L, _L, _I, _I, _I, _I, _P],
     "fmsmo_grouped_gemm_i8_dq": [_P, _L, _P, _L, _L, _P, _I, _L, _P, _P, _P, _I, _I, _P, _I, _L,
@@ -53,6 +54,7 @@ OTHER = {
     "fmsmo_status_str": ([c_int], c_char_p),
     "fmsmo_last_error": ([], c_char_p),
     "fmsmo_gemm_workspace_bytes": ([c_int64, c_int64, c_int64], c_int64),
+    "fmsmo_decode_linear_ok": ([c_int64, c_int64], c_int),
 }
 
 _lib = None

@@ -526,3 +526,59 @@ def gemm_fp8_dq(a, w, a_scale, w_scale, bias=None, out_dtype=torch.bfloat16, for
     _need_gpu(a, w, bias)
     return torch.ops.fms_mo_amd.gemm_fp8_dq(a, w, _as_scale(a_scale, a.device), _as_scale(w_scale, a.device),
                                             bias, out_dtype, bool(force_gemv))
+
+
+# ------------------------------------------------------------------------ fused decode linear
+def decode_linear_ok(x, smooth, K):
+    """Can ``decode_linear_i8`` serve these activations?  One token, fp16 / bf16, SmoothQuant
+    divisors of the same dtype (or none), K up to 8192 in one of the decode kernel's sizes."""
+    if x.dim() != 2 or x.dtype not in (torch.float16, torch.bfloat16) or not x.is_cuda:
+        return False
+    if smooth is not None and (smooth.dtype != x.dtype or smooth.numel() != K):
+        return False
+    return bool(L.load().fmsmo_decode_linear_ok(x.shape[0], K))
+
+
+def _decode_linear_i8_impl(x, w, w_scale, bias, smooth, out_dtype, exact_ref, saturate):
+    x = _rows(x)
+    w = _rows(w)
+    M, K = x.shape
+    N = w.shape[0]
+    if w.dtype != torch.int8 or w.shape[1] != K:
+        raise ValueError("w must be int8 [N, K]")
+    w_scale = _scale_vec(w_scale, N, x.device, "w_scale")
+    if smooth is not None:
+        smooth = smooth.detach().reshape(-1).contiguous()
+        if smooth.data_ptr() % 16:
+            smooth = smooth.clone()
+    if bias is not None:
+        bias = bias.detach().reshape(-1).contiguous()
+    y = torch.empty((M, N), dtype=out_dtype, device=x.device)
+    a_scale = torch.empty((M,), dtype=torch.float32, device=x.device)
+    with torch.cuda.device(x.device):
+        L.call("fmsmo_decode_linear_i8", x.data_ptr(), _dt(x), _ld(x), _ptr(smooth), int(bool(saturate)),
+               w.data_ptr(), _ld(w), w_scale.data_ptr(), w_scale.numel(), _ptr(bias),
+               _dt(bias) if bias is not None else 0, L.EPI_REF_F16 if exact_ref else L.EPI_F32,
+               y.data_ptr(), _DT[out_dtype], N, a_scale.data_ptr(), M, N, K, _stream(x))
+    return y, a_scale
+
+
+_register(
+    "decode_linear_i8",
+    "(Tensor x, Tensor w, Tensor w_scale, Tensor? bias, Tensor? smooth, ScalarType out_dtype, "
+    "bool exact_ref, bool saturate) -> (Tensor, Tensor)",
+    lambda x, w, w_scale, bias, smooth, out_dtype, exact_ref, saturate: _decode_linear_i8_impl(
+        x, w, w_scale, bias, smooth, out_dtype, exact_ref, saturate),
+    lambda x, w, w_scale, bias, smooth, out_dtype, exact_ref, saturate: (
+        torch.empty((x.shape[0], w.shape[0]), dtype=out_dtype, device=x.device),
+        torch.empty((x.shape[0],), dtype=torch.float32, device=x.device)),
+)
+
+
+def decode_linear_i8(x, w, w_scale, bias=None, smooth=None, out_dtype=torch.float16, exact_ref=True,
+                     saturate=False):
+    """(y [M,N], per-token scales fp32 [M]) = quantize x per token (see quant_act_i8_pertoken) and
+    multiply with the int8 weights w [N,K], in one launch; check ``decode_linear_ok`` first."""
+    _need_gpu(x, w, bias, smooth)
+    return torch.ops.fms_mo_amd.decode_linear_i8(x, w, _as_scale(w_scale, x.device), bias, smooth,
+                                                 out_dtype, bool(exact_ref), bool(saturate))

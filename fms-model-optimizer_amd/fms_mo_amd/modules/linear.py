@@ -517,6 +517,18 @@ class QLinearINT8Deploy(nn.Linear):
             self._sq_on = bool(torch.all(sq != 1).item())
         return self._sq_on
 
+    def _w_scale_f32(self):
+        """``w_scale`` as the contiguous fp32 vector the kernels read, converted once (the buffer
+        is fp16 in a deployed ``.half()`` module; converting it in every forward costs a launch)."""
+        ws = self.w_scale
+        if torch.compiler.is_compiling():
+            return ws.float().reshape(-1)
+        key = (ws.data_ptr(), ws._version, ws.dtype)
+        if getattr(self, "_ws_key", None) != key:
+            self._ws_key = key
+            self._ws_f32 = ws.detach().float().reshape(-1).contiguous()
+        return self._ws_f32
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         with torch.no_grad():
             org_dtype = x.dtype
@@ -525,14 +537,22 @@ class QLinearINT8Deploy(nn.Linear):
             if not x2.is_cuda:
                 raise RuntimeError("fms_mo_amd.QLinearINT8Deploy runs on an AMD GPU only; there is no CPU path")
             use_sq = self._smoothq_active()
-            if (use_sq and self.useDynMaxQfunc == -1 and self.use_int_kernel
-                    and self.smoothq_scale.numel() == x2.shape[1]
-                    and not (x2.shape[1] > self.chunk_size or self.truncate_lsb > 0)):
-                # fused path: SmoothQuant divide inside the quantizer kernel
-                sq = self.smoothq_scale.reshape(-1)
+            plain = (self.useDynMaxQfunc == -1 and self.use_int_kernel
+                     and not (x2.shape[1] > self.chunk_size or self.truncate_lsb > 0)
+                     and not getattr(self, "use_fake_zero_shift", False))
+            sq = self.smoothq_scale.reshape(-1) if use_sq else None
+            if plain and (sq is None or sq.numel() == x2.shape[1]) and \
+                    kernels.decode_linear_ok(x2, sq, x2.shape[1]):
+                # single-token decode step: quantizer and weight-streaming matmul in one launch
+                y, s = kernels.decode_linear_i8(x2, self.weight, self._w_scale_f32(), self.bias, sq,
+                                                out_dtype=torch.float16, exact_ref=True)
+                self.input_scale = s.reshape(-1, 1)
+                y = y.to(self.acc_dtype)
+            elif plain and use_sq and sq.numel() == x2.shape[1]:
+                # SmoothQuant divide inside the quantizer kernel
                 q, s = kernels.quant_act_i8_pertoken(x2, sq, compute_dtype=_compute_dtype(x2.dtype, sq))
                 self.input_scale = s.reshape(-1, 1)
-                y = kernels.gemm_i8_dq(q, self.weight, s, self.w_scale.float().reshape(-1), self.bias,
+                y = kernels.gemm_i8_dq(q, self.weight, s, self._w_scale_f32(), self.bias,
                                        out_dtype=torch.float16, exact_ref=True).to(self.acc_dtype)
             else:
                 if use_sq:

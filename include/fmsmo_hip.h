@@ -221,6 +221,29 @@ int fmsmo_gemv_fp8_dq(const uint8_t* a, int64_t lda, const uint8_t* b, int64_t l
                       int64_t w_scale_n, const void* bias, int bias_dtype, void* y, int y_dtype,
                       int64_t ldy, int64_t M, int64_t N, int64_t K, fmsmo_stream_t stream);
 
+/*
+ * Fused decode linear for ONE token: y = dequant( quant(x) . W^T ) in one launch.  Every block
+ * quantizes the (tiny) activation row itself -- the arithmetic of fmsmo_quant_act_i8_pertoken for
+ * a 16-bit compute dtype: x fp16 / bf16 [1,K], smooth of x's dtype or NULL -- and then runs the
+ * row-streaming kernel of fmsmo_gemv_i8_dq on the codes, so the result is bit-identical to the
+ * two calls in sequence while a kernel launch and the round trip of the codes through memory are
+ * saved in front of every linear layer of a single-stream decode step.  a_scale_out (fp32 [1],
+ * may be NULL) receives the token's scale (the reference's input_scale side effect).
+ * fmsmo_decode_linear_ok(M, K) != 0 tells whether a shape is served: M == 1 and K <= 8192 in one
+ * of the decode kernel's sizes (1024, 2048, 4096, 8192 and what pads to them); with more tokens
+ * or longer rows the quantization that every block repeats costs more than the launch it saves,
+ * and the call returns FMSMO_ERR_UNSUPPORTED: use the two kernels.
+ * x and smooth 16-byte aligned, ldx % 8 == 0, w as for fmsmo_gemv_i8_dq.
+ * Reference: QLinearINT8Deploy.forward for a decode step -- qa_dynamic_max_qfunc followed by
+ * iaddmm_int (fms_mo/modules/linear.py:1085-1100, 1177-1188, 1309-1338); no fused counterpart.
+ */
+int fmsmo_decode_linear_ok(int64_t M, int64_t K);
+int fmsmo_decode_linear_i8(const void* x, int x_dtype, int64_t ldx, const void* smooth,
+                           int saturate, const int8_t* w, int64_t ldw, const float* w_scale,
+                           int64_t w_scale_n, const void* bias, int bias_dtype, int epilogue,
+                           void* y, int y_dtype, int64_t ldy, float* a_scale_out, int64_t M,
+                           int64_t N, int64_t K, fmsmo_stream_t stream);
+
 /* ------------------------------------------------------------------------------------------
  * 4. Chunked reduced-precision accumulation ("chunk-truncate") matmuls.
  *    Per K-chunk of chunk_size: p = dot(a_chunk, b_chunk) in a fresh accumulator; p is

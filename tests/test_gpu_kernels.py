@@ -629,3 +629,68 @@ def test_split_k_gemm_replays_from_a_hip_graph(dev):
             assert torch.equal(out.view(torch.int16), ref.view(torch.int16))
             fn(a)
             torch.cuda.synchronize()
+
+
+# ------------------------------------------------------------------ fused decode linear
+@pytest.mark.parametrize("NK", [(4096, 4096), (6144, 4096), (520, 1024), (1000, 2048), (256, 8192), (28672, 4096),
+                                (96, 1536), (64, 3584)])
+@pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("smooth", [False, True])
+def test_fused_decode_linear_is_bit_identical_to_the_two_kernels(dev, NK, dt, smooth):
+    N, Kd = NK
+    kn = K()
+    x = torch.randn(1, Kd, generator=gen(171)).to(dt)
+    x[:, 5] *= 30.0
+    sm = (torch.rand(Kd, generator=gen(172)) * 3 + 0.2).to(dt) if smooth else None
+    w = _rand_i8((N, Kd), 173).to(dev)
+    s_w = (torch.rand(N, generator=gen(174)) * 1e-3 + 1e-5).to(dev)
+    bias = (torch.randn(N, generator=gen(175)) * 0.01).to(dt).to(dev)
+    xd, smd = x.to(dev), None if sm is None else sm.to(dev)
+    assert kn.decode_linear_ok(xd, smd, Kd)
+    for exact_ref, od in ((True, torch.float16), (False, dt)):
+        q, s = kn.quant_act_i8_pertoken(xd, smd)
+        ref = kn.gemm_i8_dq(q, w, s, s_w, bias, out_dtype=od, exact_ref=exact_ref)
+        y, s_f = kn.decode_linear_i8(xd, w, s_w, bias, smd, out_dtype=od, exact_ref=exact_ref)
+        assert torch.equal(s_f, s)
+        assert torch.equal(y.view(torch.int16), ref.view(torch.int16))
+    # the scale against the oracle as well (the codes are checked through the matmul above)
+    _, s_ref, _ = O.quant_act_pertoken_i8(x if sm is None else x / sm)
+    assert torch.equal(s_f.cpu(), s_ref.reshape(-1).float())
+
+
+@pytest.mark.parametrize("row", ["zeros", "inf", "overflow"])
+def test_fused_decode_linear_special_rows(dev, row):
+    """Rows that leave the fast division path (all zeros, an infinity, an fp16 overflow after the
+    SmoothQuant divide) must come out like the stand-alone quantizer's."""
+    kn = K()
+    Kd, N = 4096, 512
+    x = torch.randn(1, Kd, generator=gen(181)).half()
+    sm = (torch.rand(Kd, generator=gen(182)) * 3 + 0.2).half()
+    if row == "zeros":
+        x[0] = 0.0
+    elif row == "inf":
+        x[0, 100] = float("inf")
+    else:
+        x[0, 7] = 60000.0
+        sm[7] = 0.25  # 60000 / 0.25 overflows fp16
+    w = _rand_i8((N, Kd), 183).to(dev)
+    s_w = (torch.rand(N, generator=gen(184)) * 1e-3 + 1e-5).to(dev)
+    for smd in (None, sm.to(dev)):
+        q, s = kn.quant_act_i8_pertoken(x.to(dev), smd)
+        ref = kn.gemm_i8_dq(q, w, s, s_w, None, out_dtype=torch.float32, exact_ref=False)
+        y, s_f = kn.decode_linear_i8(x.to(dev), w, s_w, None, smd, out_dtype=torch.float32, exact_ref=False)
+        assert torch.equal(s_f.view(torch.int32), s.view(torch.int32))
+        assert torch.equal(y.view(torch.int32), ref.view(torch.int32))
+
+
+def test_fused_decode_linear_rejects_what_it_does_not_serve(dev):
+    kn = K()
+    x = torch.randn(2, 4096, device=dev).half()
+    assert not kn.decode_linear_ok(x, None, 4096)                          # more than one token
+    assert not kn.decode_linear_ok(x[:1].float(), None, 4096)              # fp32 activations
+    assert not kn.decode_linear_ok(torch.randn(1, 14336, device=dev).half(), None, 14336)  # long rows
+    assert not kn.decode_linear_ok(x[:1], torch.ones(4096, device=dev), 4096)  # fp32 divisors
+    assert kn.decode_linear_ok(x[:1], None, 4096)
+    w = torch.zeros(64, 4096, dtype=torch.int8, device=dev)
+    with pytest.raises(RuntimeError):
+        kn.decode_linear_i8(x, w, torch.ones(1, device=dev))

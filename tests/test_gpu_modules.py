@@ -42,7 +42,8 @@ def outlier_x(M, K, seed, dtype=torch.float16):
 
 
 @pytest.mark.parametrize("smoothq", [False, True])
-@pytest.mark.parametrize("shape", [(3, 40, 256, 384), (1, 512, 1024, 512)])
+@pytest.mark.parametrize("shape", [(3, 40, 256, 384), (1, 512, 1024, 512), (1, 1, 4096, 512), (1, 3, 1024, 384),
+                                   (2, 2, 2048, 256)])
 def test_deploy_module_bit_exact_vs_oracle(dev, smoothq, shape):
     """Conversion (offline weight / scale preparation) runs on the CPU like the reference's
     lower_qmodel_cutlass (custom_ext_kernels/utils.py:830); the forward runs on the GPU."""
@@ -316,3 +317,27 @@ def test_operator_twins_agree_with_the_kernels_on_shapes(dev):
                           test_utils=("test_schema", "test_faketensor"))
     torch.library.opcheck(torch.ops.fms_mo_amd.quant_act_i8_static.default, (x, 0.05, 128, 0),
                           test_utils=("test_schema", "test_faketensor"))
+
+
+@pytest.mark.parametrize("smoothq", [False, True])
+@pytest.mark.parametrize("K,N", [(4096, 1024), (14336, 512), (1024, 768)])
+def test_decode_step_equals_the_rows_of_a_larger_batch(dev, smoothq, K, N):
+    """The deployed fp16 module takes the fused one-launch path for a single token.  Per-token
+    quantization makes every output row a function of its own input row only, so the decode step
+    must reproduce, bit for bit, the corresponding rows of a 40-token batch (which runs the
+    quantizer and the GEMM as two kernels)."""
+    from fms_mo_amd.modules.linear import QLinearINT8Deploy
+
+    m = make_qlinear(None, K, N, smoothq=smoothq, seed=7)
+    x = outlier_x(40, K, 9)
+    if smoothq:
+        m.set_act_scale(x.float().abs().amax(dim=0))
+    dep = QLinearINT8Deploy.from_fms_mo(m, use_int_kernel="cutlass", use_dynamic_max_act_Qfunc=-1,
+                                        recalc_clipvals=False, target_device="cpu").half().to(dev)
+    xd = x.to(dev)
+    full = dep(xd).clone()
+    full_scale = dep.input_scale.clone()
+    for M in (1, 2, 4):  # one token: the fused launch; more: quantizer and decode kernel
+        y = dep(xd[:M])
+        assert torch.equal(y.view(torch.int16), full[:M].view(torch.int16))
+        assert torch.equal(dep.input_scale.reshape(-1), full_scale.reshape(-1)[:M])
