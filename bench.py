@@ -141,26 +141,6 @@ def main():
     gemm_ops = [2.0 * M_TOKENS * k * n for _, k, n in LLAMA3_8B]
     per_shape = {name: round(o / (ms * 1e-3) / 1e12, 1) for (name, _, _), o, ms in zip(LLAMA3_8B, gemm_ops, gemm_ms)}
     achieved = sum(gemm_ops) / (sum(gemm_ms) * 1e-3) / 1e12
-    # Outside the timed region: the same four GEMM launches on all-zero operands.  Nothing toggles
-    # in the multipliers then, the clock stays up, and the figure shows how far the kernel's
-    # instruction stream can go when the power limit does not hold it back.
-    zero_ms = []
-    for L in layers:
-        qz = torch.zeros((M_TOKENS, L["w"].shape[1]), dtype=torch.int8, device=dev)
-        wz = torch.zeros_like(L["w"])
-        sz = torch.ones(M_TOKENS, device=dev)
-        for _ in range(3):
-            K.gemm_i8_dq(qz, wz, sz, L["w_scale"], L["bias"], out_dtype=torch.float16, exact_ref=True)
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(5):
-            K.gemm_i8_dq(qz, wz, sz, L["w_scale"], L["bias"], out_dtype=torch.float16, exact_ref=True)
-        e1.record()
-        torch.cuda.synchronize()
-        zero_ms.append(e0.elapsed_time(e1) / 5)
-        del qz, wz
-    zero_tops = sum(gemm_ops) / (sum(zero_ms) * 1e-3) / 1e12
-
     traffic = None
     tfile = os.path.join(ROOT, "profiles", "gemm_i8_traffic.json")
     if os.path.exists(tfile):
@@ -181,7 +161,6 @@ def main():
                      "unit": "TFLOP/s", "frac": round(achieved / PEAK_INT8_TOPS, 4),
                      "traffic": traffic, "kernel": "gemm_rs_kernel<int8, dequant epilogue> (4 launches per step)",
                      "per_shape_tops": per_shape,
-                     "same_launches_on_zero_operands_tops": round(zero_tops, 1),
                      "avg_launch_ms": {n: round(ms, 4) for (n, _, _), ms in zip(LLAMA3_8B, gemm_ms)}},
     }
     if not args.no_cpu_baseline:
@@ -257,6 +236,22 @@ def extras(torch, K, dev):
             res[f"decode_i8_M{M}_{name}"] = {"us": round(ms * 1e3, 2), "GBps": round(gbs, 1), "frac_hbm": round(gbs / PEAK_HBM_GBS, 4)}
             del graph
         del ws_i8
+    # the four int8 GEMMs of the headline workload on all-zero operands: nothing toggles in the
+    # multipliers, the clock stays up, and the figure shows how far the kernel's instruction
+    # stream goes when the power limit does not hold it back
+    zero_ms, zero_ops = 0.0, 0.0
+    for name, k, n in LLAMA3_8B:
+        qz = torch.zeros((M_TOKENS, k), dtype=torch.int8, device=dev)
+        wz = torch.zeros((n, k), dtype=torch.int8, device=dev)
+        sz = torch.ones(M_TOKENS, device=dev)
+        wsz = torch.ones(n, device=dev)
+        ms = timeit(lambda: K.gemm_i8_dq(qz, wz, sz, wsz, None, out_dtype=torch.float16, exact_ref=True), iters=10, warm=3)
+        zero_ms += ms
+        zero_ops += 2.0 * M_TOKENS * k * n
+        res[f"gemm_i8_zero_operands_M4096_{name}"] = {"ms": round(ms, 4), "tops": round(2.0 * M_TOKENS * k * n / ms / 1e9, 1)}
+        del qz, wz
+    res["gemm_i8_zero_operands_M4096_all"] = {"tops": round(zero_ops / zero_ms / 1e9, 1),
+                                             "frac_peak": round(zero_ops / zero_ms / 1e9 / PEAK_INT8_TOPS, 4)}
     # a whole decode-step linear from fp16 activations (SmoothQuant divide, per-token quantizer,
     # weight-streaming matmul, dequantizing epilogue): two launches against the fused one
     for name, k, n in LLAMA3_8B:
