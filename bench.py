@@ -166,11 +166,11 @@ def main():
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(torch, layers[1])
     if args.extras:
-        out["extras"] = extras(torch, K, dev)
+        out["extras"] = extras(torch, K, dev, layers[1])
     print(json.dumps(out))
 
 
-def extras(torch, K, dev):
+def extras(torch, K, dev, o_layer):
     """FP8 GEMMs (Granite-3-8B-like shapes, M=2048), decode shapes (M in 1 .. 128), the Mixtral-style
     grouped expert GEMMs and the chunk-truncate emulation; reported in addition to the headline
     value."""
@@ -190,6 +190,37 @@ def extras(torch, K, dev):
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) / iters
 
+    # the sample the CPU baseline is timed on (first 512 tokens of the o projection), on the GPU:
+    # SmoothQuant act-quant + int8 GEMM + dequant (512 x 4096 x 4096 splits its reduction in two)
+    x512 = o_layer["x"][:512]
+
+    def c1_step():
+        q, sc = K.quant_act_i8_pertoken(x512, o_layer["smooth"])
+        return K.gemm_i8_dq(q, o_layer["w"], sc, o_layer["w_scale"], o_layer["bias"], out_dtype=torch.float16,
+                            exact_ref=True)
+
+    def graph_time(fn, reps=20, replays=5):  # device time: launches replayed from a HIP graph
+        side = torch.cuda.Stream()
+        with torch.cuda.stream(side):
+            fn()
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=side):
+                for _ in range(reps):
+                    fn()
+            graph.replay()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(replays):
+                graph.replay()
+            e1.record()
+            torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / (reps * replays)
+
+    ms_eager, ms = timeit(c1_step), graph_time(c1_step)
+    res["cpu_baseline_sample_on_gpu_o_M512"] = {"us": round(ms * 1e3, 1), "eager_us": round(ms_eager * 1e3, 1),
+                                                "tops": round(2.0 * 512 * 4096 * 4096 / ms / 1e9, 1)}
     g = torch.Generator().manual_seed(3)
     M = 2048
     for name, k, n in [("qkv", 4096, 6144), ("o", 4096, 4096), ("gate_up", 4096, 25600), ("down", 12800, 4096)]:
