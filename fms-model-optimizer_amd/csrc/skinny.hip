@@ -130,6 +130,71 @@ __device__ __forceinline__ void quantize_rows_to_lds(const GemvArgs& g, uint8_t 
   if (blockIdx.x == 0 && g.a_scale_out && threadIdx.x < g.M) g.a_scale_out[threadIdx.x] = sc[threadIdx.x];
 }
 
+// The FP8Linear recipe for one token row by all NT threads of a block, into LDS:
+// s = max(amax / 448, 1e-12) in fp32, q = e4m3( clamp(f32(x) / s, -448, 448) ), IEEE divisions
+// (a row is a few thousand elements); rows whose maximum is inf / NaN use the software encoder,
+// like the stand-alone quantizer.
+template <int XT, int NT, int KMAX>
+__device__ __forceinline__ void quantize_row_fp8_to_lds(const GemvArgs& g, uint8_t (*xq)[KMAX], float* sc,
+                                                        float* red) {
+  constexpr int NCH = (KMAX / AQ_VEC + NT - 1) / NT;
+  const int nchunk = g.K / AQ_VEC;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  constexpr uint32_t INF_BITS = XT == FMSMO_F16 ? 0x7c00u : 0x7f80u;
+  v4i cur[NCH];
+  us2 amax2 = {0, 0};
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) {
+    const int c = threadIdx.x + i * NT;
+    if (c < nchunk) {
+      cur[i] = *(const v4i*)(g.x16 + (size_t)c * AQ_VEC);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const uint32_t mag = (uint32_t)cur[i][j] & 0x7fff7fffu;
+        us2 m2;
+        __builtin_memcpy(&m2, &mag, 4);
+        amax2 = __builtin_elementwise_max(amax2, m2);
+      }
+    }
+  }
+  float v = wave_max(__uint_as_float((uint32_t)(amax2[0] > amax2[1] ? amax2[0] : amax2[1])));
+  if (lane == 0) red[wave] = v;
+  __syncthreads();
+  v = red[0];
+#pragma unroll
+  for (int w = 1; w < NT / 64; ++w) v = fmaxf(v, red[w]);
+  const uint32_t abits = __float_as_uint(v);
+  const float s = fmaxf(cvt16<XT>((u16)abits) / 448.0f, 1e-12f);
+  if (threadIdx.x == 0) sc[0] = s;
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) {
+    const int c = threadIdx.x + i * NT;
+    if (c < nchunk) {
+      float t[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float xv = cvt16<XT>((u16)((uint32_t)cur[i][j >> 1] >> ((j & 1) * 16)));
+        t[j] = fminf(fmaxf(xv / s, -448.0f), 448.0f);
+      }
+      if (abits < INF_BITS) {
+        int o0 = 0, o1 = 0;
+        o0 = __builtin_amdgcn_cvt_pk_fp8_f32(t[0], t[1], o0, false);
+        o0 = __builtin_amdgcn_cvt_pk_fp8_f32(t[2], t[3], o0, true);
+        o1 = __builtin_amdgcn_cvt_pk_fp8_f32(t[4], t[5], o1, false);
+        o1 = __builtin_amdgcn_cvt_pk_fp8_f32(t[6], t[7], o1, true);
+        *(uint2*)(&xq[0][(size_t)c * AQ_VEC]) = make_uint2((uint32_t)o0, (uint32_t)o1);
+      } else {
+        uint8_t b[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) b[j] = f32_to_e4m3_sw(t[j]);
+        store8(&xq[0][0], (size_t)c * AQ_VEC, b);
+      }
+    }
+  }
+  __syncthreads();
+  if (blockIdx.x == 0 && g.a_scale_out && threadIdx.x == 0) g.a_scale_out[0] = sc[0];
+}
+
 template <int OP, int RG, int NW>
 __global__ __launch_bounds__(NW * 64) void gemv_kernel(GemvArgs g) {
   typedef typename std::conditional<OP == FMSMO_OP_I8, int, float>::type AccT;
@@ -405,7 +470,8 @@ __global__ __launch_bounds__(256) void gemv_rows_kernel(GemvArgs g) {
   if constexpr (FUSED) {
     // the weights of the first turn are in flight while the block quantizes its activations
     load_w(wave_g * U, w);
-    quantize_rows_to_lds<XT, 256, KCH * 1024, MR>(g, xq, xsc, xred);
+    if constexpr (OP == FMSMO_OP_I8) quantize_rows_to_lds<XT, 256, KCH * 1024, MR>(g, xq, xsc, xred);
+    else quantize_row_fp8_to_lds<XT, 256, KCH * 1024>(g, xq, xsc, xred);
     g.a = &xq[0][0];
     g.lda = KCH * 1024;
     g.a_scale = xsc;
@@ -654,14 +720,14 @@ extern "C" int fmsmo_decode_linear_ok(int64_t M, int64_t K) {
   return kch == 1 || kch == 2 || kch == 4 || kch == 8;
 }
 
-template <int XT>
+template <int OP, int XT>
 static int decode_fused_launch(const GemvArgs& g, hipStream_t st) {
   const int kch = (int)((g.K + 1023) / 1024);
 #define ROWS(KCHV, UV)                                                                            \
   {                                                                                                \
     const int64_t blocks = ((int64_t)g.N + 4 * UV - 1) / (4 * UV);                                 \
     dim3 grid((unsigned)(blocks < 1024 ? blocks : 1024));                                          \
-    hipLaunchKernelGGL((gemv_rows_kernel<FMSMO_OP_I8, 1, KCHV, UV, XT>), grid, dim3(256), 0, st, g); \
+    hipLaunchKernelGGL((gemv_rows_kernel<OP, 1, KCHV, UV, XT>), grid, dim3(256), 0, st, g);         \
   }
   switch (kch) {
     case 1: ROWS(1, 8) break;
@@ -698,8 +764,32 @@ extern "C" int fmsmo_decode_linear_i8(const void* x, int x_dtype, int64_t ldx, c
   g.y = y; g.y_dtype = y_dtype; g.ldy = ldy;
   g.x16 = (const u16*)x; g.ldx = ldx; g.smooth = (const u16*)smooth; g.saturate = saturate;
   g.a_scale_out = a_scale_out;
-  return x_dtype == FMSMO_F16 ? decode_fused_launch<FMSMO_F16>(g, (hipStream_t)stream)
-                              : decode_fused_launch<FMSMO_BF16>(g, (hipStream_t)stream);
+  return x_dtype == FMSMO_F16 ? decode_fused_launch<FMSMO_OP_I8, FMSMO_F16>(g, (hipStream_t)stream)
+                              : decode_fused_launch<FMSMO_OP_I8, FMSMO_BF16>(g, (hipStream_t)stream);
+}
+
+extern "C" int fmsmo_decode_linear_fp8(const void* x, int x_dtype, int64_t ldx, const uint8_t* w,
+                                       int64_t ldw, const float* w_scale, int64_t w_scale_n,
+                                       const void* bias, int bias_dtype, void* y, int y_dtype,
+                                       int64_t ldy, float* a_scale_out, int64_t M, int64_t N,
+                                       int64_t K, fmsmo_stream_t stream) {
+  if (!x || !w || !w_scale || !y) return FMSMO_ERR_NULL;
+  if (M <= 0 || N <= 0 || K <= 0 || ldx < K || ldw < K || ldy < N) return FMSMO_ERR_SHAPE;
+  if (w_scale_n != 1 && w_scale_n != N) return FMSMO_ERR_SHAPE;
+  if ((x_dtype != FMSMO_F16 && x_dtype != FMSMO_BF16) || !fmsmo_decode_linear_ok(M, K)) return FMSMO_ERR_UNSUPPORTED;
+  if (N >= (1 << 30) || N * ldw >= (1ll << 40)) return FMSMO_ERR_UNSUPPORTED;
+  if (y_dtype < 0 || y_dtype > 2 || (bias && (bias_dtype < 0 || bias_dtype > 2))) return FMSMO_ERR_UNSUPPORTED;
+  if (ldx % 8 || ldw % 16 || (((uintptr_t)x) & 15) || (((uintptr_t)w) & 15)) return FMSMO_ERR_ALIGN;
+  GemvArgs g{};
+  g.b = w; g.ldb = ldw;
+  g.M = (int)M; g.N = (int)N; g.K = (int)K;
+  g.w_scale = w_scale; g.w_stride = w_scale_n == 1 ? 0 : 1;
+  g.bias = bias; g.bias_dtype = bias_dtype; g.ref_f16 = 0;
+  g.y = y; g.y_dtype = y_dtype; g.ldy = ldy;
+  g.x16 = (const u16*)x; g.ldx = ldx;
+  g.a_scale_out = a_scale_out;
+  return x_dtype == FMSMO_F16 ? decode_fused_launch<FMSMO_OP_E4M3, FMSMO_F16>(g, (hipStream_t)stream)
+                              : decode_fused_launch<FMSMO_OP_E4M3, FMSMO_BF16>(g, (hipStream_t)stream);
 }
 
 static int check_gemv(const void* a, int64_t lda, const void* b, int64_t ldb, const float* a_scale,

@@ -38,6 +38,7 @@ SIGNATURES = {
     "fmsmo_gemv_i8_dq": [_P, _L, _P, _L, _P, _L, _P, _L, _P, _I, _I, _P, _I, _L, _L, _L, _L, _P],
     "fmsmo_gemv_fp8_dq": [_P, _L, _P, _L, _P, _L, _P, _L, _P, _I, _P, _I, _L, _L, _L, _L, _P],
     "fmsmo_decode_linear_i8": [_P, _I, _L, _P, _I, _P, _L, _P, _L, _P, _I, _I, _P, _I, _L, _P, _L, _L, _L, _P],
+    "fmsmo_decode_linear_fp8": [_P, _I, _L, _P, _L, _P, _L, _P, _I, _P, _I, _L, _P, _L, _L, _L, _P],
     "fmsmo_matmul_chunk_i8": [_P, _L, _P, _L, _P, _P, _L, _L, _L, _L, _I, _I, _I, _I, _P],
     "fmsmo_matmul_chunk_fp": [_P, _L, _P, _L, _I, _P, _P, _L, _L, _L, _L, _I, _I, _I, _I, _P],
     "fmsmo_grouped_gemm_i8_dq": [_P, _L, _P, _L, _L, _P, _I, _L, _P, _P, _P, _I, _I, _P, _I, _L,

@@ -582,3 +582,39 @@ def decode_linear_i8(x, w, w_scale, bias=None, smooth=None, out_dtype=torch.floa
     _need_gpu(x, w, bias, smooth)
     return torch.ops.fms_mo_amd.decode_linear_i8(x, w, _as_scale(w_scale, x.device), bias, smooth,
                                                  out_dtype, bool(exact_ref), bool(saturate))
+
+
+def _decode_linear_fp8_impl(x, w, w_scale, bias, out_dtype):
+    x = _rows(x)
+    w = _rows(w)
+    M, K = x.shape
+    N = w.shape[0]
+    if w.dtype != torch.float8_e4m3fn or w.shape[1] != K:
+        raise ValueError("w must be float8_e4m3fn [N, K]")
+    w_scale = _scale_vec(w_scale, N, x.device, "w_scale")
+    if bias is not None:
+        bias = bias.detach().reshape(-1).contiguous()
+    y = torch.empty((M, N), dtype=out_dtype, device=x.device)
+    a_scale = torch.empty((M,), dtype=torch.float32, device=x.device)
+    with torch.cuda.device(x.device):
+        L.call("fmsmo_decode_linear_fp8", x.data_ptr(), _dt(x), _ld(x), w.data_ptr(), _ld(w),
+               w_scale.data_ptr(), w_scale.numel(), _ptr(bias), _dt(bias) if bias is not None else 0,
+               y.data_ptr(), _DT[out_dtype], N, a_scale.data_ptr(), M, N, K, _stream(x))
+    return y, a_scale
+
+
+_register(
+    "decode_linear_fp8",
+    "(Tensor x, Tensor w, Tensor w_scale, Tensor? bias, ScalarType out_dtype) -> (Tensor, Tensor)",
+    lambda x, w, w_scale, bias, out_dtype: _decode_linear_fp8_impl(x, w, w_scale, bias, out_dtype),
+    lambda x, w, w_scale, bias, out_dtype: (
+        torch.empty((x.shape[0], w.shape[0]), dtype=out_dtype, device=x.device),
+        torch.empty((x.shape[0],), dtype=torch.float32, device=x.device)),
+)
+
+
+def decode_linear_fp8(x, w, w_scale, bias=None, out_dtype=torch.bfloat16):
+    """(y [1,N], token scale fp32 [1]): dynamic per-token e4m3 quantizer (the FP8Linear recipe) and
+    the e4m3 weight-streaming matmul in one launch; check ``decode_linear_ok(x, None, K)`` first."""
+    _need_gpu(x, w, bias)
+    return torch.ops.fms_mo_amd.decode_linear_fp8(x, w, _as_scale(w_scale, x.device), bias, out_dtype)

@@ -243,6 +243,17 @@ int fmsmo_decode_linear_i8(const void* x, int x_dtype, int64_t ldx, const void* 
                            int64_t w_scale_n, const void* bias, int bias_dtype, int epilogue,
                            void* y, int y_dtype, int64_t ldy, float* a_scale_out, int64_t M,
                            int64_t N, int64_t K, fmsmo_stream_t stream);
+/*
+ * The same for e4m3 weights: the block quantizes the token with the dynamic per-token recipe of
+ * fmsmo_quant_act_fp8_pertoken(FMSMO_FP8_LINEAR) and runs fmsmo_gemv_fp8_dq's kernel on it;
+ * bit-identical to the two calls.  Served shapes as told by fmsmo_decode_linear_ok.
+ * Reference: FP8Linear.forward with dynamic activation scales
+ * (fms_mo/aiu_addons/fp8/fp8_linear.py:217-283) on one token.
+ */
+int fmsmo_decode_linear_fp8(const void* x, int x_dtype, int64_t ldx, const uint8_t* w, int64_t ldw,
+                            const float* w_scale, int64_t w_scale_n, const void* bias,
+                            int bias_dtype, void* y, int y_dtype, int64_t ldy, float* a_scale_out,
+                            int64_t M, int64_t N, int64_t K, fmsmo_stream_t stream);
 
 /* ------------------------------------------------------------------------------------------
  * 4. Chunked reduced-precision accumulation ("chunk-truncate") matmuls.

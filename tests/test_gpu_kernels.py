@@ -694,3 +694,31 @@ def test_fused_decode_linear_rejects_what_it_does_not_serve(dev):
     w = torch.zeros(64, 4096, dtype=torch.int8, device=dev)
     with pytest.raises(RuntimeError):
         kn.decode_linear_i8(x, w, torch.ones(1, device=dev))
+
+
+@pytest.mark.parametrize("NK", [(4096, 4096), (6144, 4096), (520, 1024), (1000, 2048), (256, 8192), (96, 1536)])
+@pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("special", [None, "zeros", "inf"])
+def test_fused_decode_linear_fp8_is_bit_identical_to_the_two_kernels(dev, NK, dt, special):
+    from fms_mo_amd import _lib as L
+
+    N, Kd = NK
+    kn = K()
+    x = (2.0 * torch.randn(1, Kd, generator=gen(191))).to(dt)
+    x[0, 3] = -0.0
+    if special == "zeros":
+        x[0] = 0.0
+    elif special == "inf":
+        x[0, 9] = float("inf")
+    w = _rand_fp8((N, Kd), 192, 0.5).to(dev)
+    s_w = (torch.rand(N, generator=gen(193)) * 0.01 + 1e-4).to(dev)
+    bias = (torch.randn(N, generator=gen(194)) * 0.1).to(dt).to(dev)
+    xd = x.to(dev)
+    assert kn.decode_linear_ok(xd, None, Kd)
+    for od in (dt, torch.float32):
+        q, s = kn.quant_act_fp8_pertoken(xd, L.FP8_LINEAR)
+        ref = kn.gemm_fp8_dq(q, w, s, s_w, bias, out_dtype=od)
+        y, s_f = kn.decode_linear_fp8(xd, w, s_w, bias, out_dtype=od)
+        assert torch.equal(s_f.view(torch.int32), s.view(torch.int32))
+        bits = torch.int32 if od == torch.float32 else torch.int16
+        assert torch.equal(y.view(bits), ref.view(bits))
