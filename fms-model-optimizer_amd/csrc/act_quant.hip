@@ -146,6 +146,7 @@ __global__ __launch_bounds__(TH) void quant_i8_pertoken16_kernel(
     if constexpr (T == FMSMO_BF16) ieee_block = __syncthreads_or(bad) != 0;
   }
 
+  const float nz = opaque_neg_zero();
   v4i cur[NCH], nxt[NCH];
   auto load_row = [&](int row, v4i (&dst)[NCH]) {
     const u16* xr = x + (size_t)row * ldx;
@@ -177,9 +178,7 @@ __global__ __launch_bounds__(TH) void quant_i8_pertoken16_kernel(
           } else {
             rl = __builtin_amdgcn_rcpf(dl), rh = __builtin_amdgcn_rcpf(dh);
           }
-          const u16 el = to16<T>(div16<T, false>(lo, dl, rl));
-          const u16 eh = to16<T>(div16<T, false>(hi, dh, rh));
-          cur[i][j] = (int)((uint32_t)el | ((uint32_t)eh << 16));
+          cur[i][j] = (int)pack16<T>(div16_mix<T>(lo, dl, rl, nz), div16_mix<T>(hi, dh, rh, nz));
         }
       }
       __builtin_amdgcn_sched_barrier(0);  // one chunk at a time: keeps the live ranges short
@@ -203,23 +202,23 @@ __global__ __launch_bounds__(TH) void quant_i8_pertoken16_kernel(
         }
       }
     }
-    // non-negative floats order like their bit patterns: reduce as floats of the raw bits
-    float v = wave_max(__uint_as_float((uint32_t)(amax2[0] > amax2[1] ? amax2[0] : amax2[1])));
+    uint32_t v = wave_max_u32((uint32_t)(amax2[0] > amax2[1] ? amax2[0] : amax2[1]));
     float* rb = red[parity];
     parity ^= 1;
-    if (lane == 0) rb[wave] = v;
+    if (lane == 0) rb[wave] = __uint_as_float(v);
     __syncthreads();
-    v = rb[0];
 #pragma unroll
-    for (int w = 1; w < TH / 64; ++w) v = fmaxf(v, rb[w]);
-    return __float_as_uint(v);
+    for (int w = 0; w < TH / 64; ++w) {
+      const uint32_t o = __float_as_uint(rb[w]);
+      v = o > v ? o : v;
+    }
+    return v;
   };
   constexpr uint32_t INF_BITS = T == FMSMO_F16 ? 0x7c00u : 0x7f80u;
 
   int row = blockIdx.x;
   if (row < M) load_row(row, cur);
   const float floor_T = cvt16<T>(to16<T>(1e-5f));
-  const float sat_hi = saturate ? 127.0f : 3.0e38f;
   for (; row < M; row += gridDim.x) {
     const int nrow = row + gridDim.x;
     if (nrow < M) load_row(nrow, nxt);
@@ -255,13 +254,9 @@ __global__ __launch_bounds__(TH) void quant_i8_pertoken16_kernel(
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
             const uint32_t w = (uint32_t)cur[i][j];
-            float ql = div16<T, false>(cvt16<T>((u16)(w & 0xffff)), s, rs);
-            float qh = div16<T, false>(cvt16<T>((u16)(w >> 16)), s, rs);
-            if (saturate) {  // clamp before rounding: the bounds are integers
-              ql = fminf(fmaxf(ql, -sat_hi), sat_hi);
-              qh = fminf(fmaxf(qh, -sat_hi), sat_hi);
-            }
-            code[j] = rint_codes<T>(to16<T>(ql), to16<T>(qh));
+            const float ql = div16_mix<T>(cvt16<T>((u16)(w & 0xffff)), s, rs, nz);
+            const float qh = div16_mix<T>(cvt16<T>((u16)(w >> 16)), s, rs, nz);
+            code[j] = rint_codes_packed<T>(pack16<T>(ql, qh), saturate != 0);
           }
           // bytes 0 and 2 of each code word -> 8 consecutive int8
           const uint32_t o0 = __builtin_amdgcn_perm(code[1], code[0], 0x06040200u);
@@ -370,8 +365,7 @@ __global__ __launch_bounds__(TH) void quant_i8_pertoken_f16x_f32s_kernel(
   auto block_amax = [&](float v) -> float {
     // NaN must survive the reduction (it selects the IEEE path): compare bit patterns of |v|
     uint32_t b = __float_as_uint(v) & 0x7fffffffu;
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) b = max(b, (uint32_t)__shfl_xor((int)b, o, 64));
+    b = wave_max_u32(b);
     float* rb = red[parity];
     parity ^= 1;
     if (lane == 0) rb[wave] = __uint_as_float(b);
@@ -744,12 +738,13 @@ __global__ __launch_bounds__(AQ_THREADS) void quant_fp8_pertoken16_kernel(
         }
       }
     }
-    float v = wave_max(__uint_as_float((uint32_t)(amax2[0] > amax2[1] ? amax2[0] : amax2[1])));
+    const uint32_t v = wave_max_u32((uint32_t)(amax2[0] > amax2[1] ? amax2[0] : amax2[1]));
     float* rb = red[parity];
     parity ^= 1;
-    if (lane == 0) rb[wave] = v;
+    if (lane == 0) rb[wave] = __uint_as_float(v);
     __syncthreads();
-    const uint32_t abits = __float_as_uint(fmaxf(fmaxf(rb[0], rb[1]), fmaxf(rb[2], rb[3])));
+    const uint32_t abits = max(max(__float_as_uint(rb[0]), __float_as_uint(rb[1])),
+                               max(__float_as_uint(rb[2]), __float_as_uint(rb[3])));
     const float amax = cvt16<XT>((u16)abits);
 
     float s;

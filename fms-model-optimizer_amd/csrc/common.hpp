@@ -64,10 +64,42 @@ __device__ __forceinline__ void store_from_f32(void* p, size_t i, float v) {
   else ((float*)p)[i] = v;
 }
 
+// Maximum of an unsigned value over the 64 lanes of the wave (all active), same result in every
+// lane.  Cross-lane
+// moves are DPP modifiers of the max instructions themselves (no LDS round trips): pairs and quads
+// by quad permutes, 8 and 16 lanes by the mirror patterns, then lane 15 / 31 broadcast into the
+// following rows, after which lane 63 holds the maximum of all.
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t x) {
+#define FMSMO_DPP_MAX(ctrl, rows)                                                             \
+  {                                                                                            \
+    const uint32_t y = (uint32_t)__builtin_amdgcn_update_dpp((int)x, (int)x, ctrl, rows, 0xf, false); \
+    x = y > x ? y : x;                                                                         \
+  }
+  FMSMO_DPP_MAX(0xb1, 0xf)   // quad_perm [1,0,3,2]
+  FMSMO_DPP_MAX(0x4e, 0xf)   // quad_perm [2,3,0,1]
+  FMSMO_DPP_MAX(0x141, 0xf)  // row_half_mirror
+  FMSMO_DPP_MAX(0x140, 0xf)  // row_mirror
+  FMSMO_DPP_MAX(0x142, 0xa)  // row_bcast15 into rows 1 and 3
+  FMSMO_DPP_MAX(0x143, 0xc)  // row_bcast31 into rows 2 and 3
+#undef FMSMO_DPP_MAX
+  return (uint32_t)__builtin_amdgcn_readlane((int)x, 63);
+}
+
+// The same for floats (fmaxf semantics: a NaN loses against a number).  All 64 lanes must be active.
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
-  return v;
+#define FMSMO_DPP_FMAX(ctrl, rows)                                                            \
+  {                                                                                            \
+    const int b = __float_as_int(v);                                                           \
+    v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(b, b, ctrl, rows, 0xf, false)));   \
+  }
+  FMSMO_DPP_FMAX(0xb1, 0xf)
+  FMSMO_DPP_FMAX(0x4e, 0xf)
+  FMSMO_DPP_FMAX(0x141, 0xf)
+  FMSMO_DPP_FMAX(0x140, 0xf)
+  FMSMO_DPP_FMAX(0x142, 0xa)
+  FMSMO_DPP_FMAX(0x143, 0xc)
+#undef FMSMO_DPP_FMAX
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
 }
 
 // OCP e4m3fn encode of one float, RNE, the way torch's float->float8_e4m3fn cast does it:

@@ -46,6 +46,19 @@ __device__ __forceinline__ float div16(float e, float s, float r) {
     return __builtin_fmaf(__builtin_fmaf(-q0, s, e), r, q0);
   }
 }
+// -0.0f the compiler cannot see through: fma(e, r, nz) is e * r bit for bit, and for e widened
+// from fp16 the widening folds into v_fma_mix_f32, where a plain product needs its own conversion.
+__device__ __forceinline__ float opaque_neg_zero() {
+  float z = -0.0f;
+  asm volatile("" : "+s"(z));
+  return z;
+}
+// div16<T, false> with the first product written as that fma (fp16 only; bf16 widens by a shift)
+template <int T>
+__device__ __forceinline__ float div16_mix(float e, float s, float r, float nz) {
+  const float q0 = T == FMSMO_F16 ? __builtin_fmaf(e, r, nz) : __fmul_rn(e, r);
+  return __builtin_fmaf(__builtin_fmaf(-q0, s, e), r, q0);
+}
 template <int T>
 __device__ __forceinline__ float cvt16(u16 h) {
   if constexpr (T == FMSMO_F16) return f16_to_f32(h);
@@ -59,10 +72,59 @@ __device__ __forceinline__ u16 to16(float f) {
 
 typedef unsigned short us2 __attribute__((ext_vector_type(2)));
 typedef _Float16 hf2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+typedef float f2 __attribute__((ext_vector_type(2)));
+
+// two floats rounded to T (nearest even), low and high half of one word, by one packed
+// conversion.  For fp16 the empty asm keeps the conversion apart from the arithmetic that feeds
+// it (see f32_to_f16).
+template <int T>
+__device__ __forceinline__ uint32_t pack16(float lo, float hi) {
+  if constexpr (T == FMSMO_F16) {
+    asm volatile("" : "+v"(lo), "+v"(hi));
+    const hf2 h = {(_Float16)lo, (_Float16)hi};
+    uint32_t r;
+    __builtin_memcpy(&r, &h, 4);
+    return r;
+  } else {
+    const f2 v = {lo, hi};
+    const bf2 h = __builtin_convertvector(v, bf2);  // v_cvt_pk_bf16_f32: RNE, NaN stays NaN
+    uint32_t r;
+    __builtin_memcpy(&r, &h, 4);
+    return r;
+  }
+}
 
 // int8 code of rint(h) for a 16-bit value h with |h| <= 511, in the low byte of each half:
 // h + 1536 lands in [1024, 2048), where the fp16 grid is the integers, so the addition itself
 // rounds to nearest-even and the low mantissa bits are the two's-complement integer.
+template <int T>
+__device__ __forceinline__ uint32_t rint_codes(u16 lo, u16 hi);
+// the same on a packed pair, optionally clamped to +-127 first (the bounds are integers, so
+// clamping before or after the rounding gives the same code)
+template <int T>
+__device__ __forceinline__ uint32_t rint_codes_packed(uint32_t packed, bool saturate) {
+  if constexpr (T == FMSMO_F16) {
+    hf2 h;
+    __builtin_memcpy(&h, &packed, 4);
+    if (saturate) {
+      const hf2 hi = {(_Float16)127.0f, (_Float16)127.0f};
+      h = __builtin_elementwise_min(__builtin_elementwise_max(h, -hi), hi);
+    }
+    const hf2 magic = {(_Float16)1536.0f, (_Float16)1536.0f};
+    h = h + magic;
+    uint32_t r;
+    __builtin_memcpy(&r, &h, 4);
+    return r;
+  } else {
+    float lo = bf16_to_f32((u16)(packed & 0xffff)), hi = bf16_to_f32((u16)(packed >> 16));
+    if (saturate) {
+      lo = fminf(fmaxf(lo, -127.0f), 127.0f);
+      hi = fminf(fmaxf(hi, -127.0f), 127.0f);
+    }
+    return rint_codes<T>(f32_to_bf16(lo), f32_to_bf16(hi));
+  }
+}
 template <int T>
 __device__ __forceinline__ uint32_t rint_codes(u16 lo, u16 hi) {
   if constexpr (T == FMSMO_F16) {
