@@ -39,19 +39,21 @@ struct TileWide { static constexpr int BM = 128, BN = 256, BK = 64, NST = 4, WGM
 struct TileMid { static constexpr int BM = 128, BN = 128, BK = 64, NST = 4, WGM = 2, WGN = 2; };
 
 // Pick the tile shape by (relative kernel efficiency) x (fill of the last round of tiles over
-// the 256 compute units).  The efficiencies are measured loop efficiencies of the three shapes
-// (bigger tiles move fewer bytes per MFMA); 128x128 tiles fit two blocks per CU.
-int pick_tile(int M, int N) {
-  static const char* force = getenv("FMSMO_TILE");  // tuning aid: 0 = 256x256, 1 = 128x256, 2 = 128x128
-  if (force && force[0] >= '0' && force[0] <= '2') return force[0] - '0';
+// the 256 compute units).  The efficiencies are measured loop efficiencies of the shapes
+// (bigger tiles move fewer bytes per MFMA); 128x128 tiles fit two blocks per CU.  Shape 3 is the
+// register-staged kernel with 256x192 tiles (K % 128 == 0 only): 8 % slower per operation than
+// 256x256, but e.g. N = 6144 at M = 4096 then makes 512 tiles, two full rounds, instead of 384.
+int pick_tile(int M, int N, bool rs192_ok) {
+  static const char* force = getenv("FMSMO_TILE");  // tuning aid: 0 = 256x256, 1 = 128x256, 2 = 128x128, 3 = 256x192
+  if (force && force[0] >= '0' && force[0] <= '3') return force[0] - '0';
   // Fitted to measurements on the Llama / Granite shapes: relative loop efficiency of the three
   // tile shapes, and a sub-linear penalty for a partially filled last round (idle CUs leave
   // power, hence clock, to the busy ones).
-  const double eff[3] = {1.0, 0.76, 0.70};
-  const int bm[3] = {256, 128, 128}, bn[3] = {256, 256, 128};
+  const double eff[4] = {1.0, 0.76, 0.70, 0.92};
+  const int bm[4] = {256, 128, 128, 256}, bn[4] = {256, 256, 128, 192};
   int best = 0;
   double best_score = -1;
-  for (int t = 0; t < 3; ++t) {
+  for (int t = 0; t < (rs192_ok ? 4 : 3); ++t) {
     const long tiles = (long)div_up(M, bm[t]) * div_up(N, bn[t]);
     const long slots = (t == 2 && tiles > 256) ? 512 : 256;  // two 128x128 blocks fit per CU
     const long rounds = (tiles + slots - 1) / slots;
@@ -84,14 +86,14 @@ static bool use_register_staged(int op) {
   (void)op;
   return true;
 }
-template <int OP, bool GROUPED = false, class Epi>
+template <int OP, bool GROUPED = false, int BN = 256, class Epi>
 void launch_rs(const GemmArgs& g0, const Epi& epi, hipStream_t st) {
   GemmArgs g = g0;
-  g.grid_n = div_up(g.N, 256);
+  g.grid_n = div_up(g.N, BN);
   if (!GROUPED) g.grid_m = div_up(g.M, 256);
   g.group_m = 4;
   dim3 grid((unsigned)(g.grid_m * g.grid_n)), block(256);
-  hipLaunchKernelGGL((gemm_rs_kernel<OP, Epi, GROUPED>), grid, block, 0, st, g, epi);
+  hipLaunchKernelGGL((gemm_rs_kernel<OP, Epi, GROUPED, BN>), grid, block, 0, st, g, epi);
 }
 
 // Generic fallback (any K % 16 == 0): one thread per output element, 4-byte dot products.
@@ -125,12 +127,16 @@ __global__ void gemm_simple_kernel(GemmArgs g, Epi epi) {
 template <int OP, class Epi>
 void launch_any(const GemmArgs& g, const Epi& epi, hipStream_t st) {
   if (g.K % 64 == 0) {
-    switch (pick_tile(g.M, g.N)) {
+    switch (pick_tile(g.M, g.N, g.K % 128 == 0 && use_register_staged(OP))) {
       case 0:
         if (g.K % 128 == 0 && use_register_staged(OP)) launch_rs<OP>(g, epi, st);
         else launch_tile<TileBig, OP, false>(g, epi, st);
         break;
       case 1: launch_tile<TileWide, OP, false>(g, epi, st); break;
+      case 3:
+        if (g.K % 128 == 0 && use_register_staged(OP)) launch_rs<OP, false, 192>(g, epi, st);
+        else launch_tile<TileBig, OP, false>(g, epi, st);
+        break;
       default: launch_tile<TileMid, OP, false>(g, epi, st); break;
     }
   } else {

@@ -19,18 +19,19 @@
 
 namespace fmsmo {
 
-template <int OP, class Epi, bool GROUPED = false>
+template <int OP, class Epi, bool GROUPED = false, int BN_ = 256>
 __global__ __launch_bounds__(256) void gemm_rs_kernel(GemmArgs g, Epi epi) {
 #if defined(__HIP_DEVICE_COMPILE__)
   typedef Mma<OP> MM;
   typedef typename MM::Frag Frag;
   typedef typename MM::Acc Acc;
-  constexpr int BM = 256, BN = 256, BK = 128, CPR = 8;
-  constexpr int TM = 128, TN = 128, FM = 4, FN = 4;
+  static_assert(BN_ == 256 || BN_ == 192, "tile width");
+  constexpr int BM = 256, BN = BN_, BK = 128, CPR = 8;
+  constexpr int TM = 128, TN = BN / 2, FM = 4, FN = TN / 32;
   constexpr int NKS = BK / MM::KSTEP;   // MFMA k-steps per slab (int8 4, e4m3 2)
   constexpr int CL = MM::KSTEP / 32;    // 16-byte chunks per lane per k-step
-  constexpr int SLAB = (BM + BN) * BK;  // 64 KiB
-  constexpr int NJ = 8;                 // row groups of 32 per operand and thread
+  constexpr int SLAB = (BM + BN) * BK;  // 64 KiB (56 KiB for the 192-column tile)
+  constexpr int NJ = BM / 32, NJB = BN / 32;  // row groups of 32 per thread: A, B
   static_assert(NKS % 2 == 0, "fragment buffers alternate per k-step");
   __shared__ __attribute__((aligned(16))) uint8_t lds[2 * SLAB];
 
@@ -96,7 +97,7 @@ __global__ __launch_bounds__(256) void gemm_rs_kernel(GemmArgs g, Epi epi) {
   const int vb = (col_lo + ld_row) * (int)g.ldb + ld_chunk * 16;
   const int sa32 = 32 * (int)g.lda, sb32 = 32 * (int)g.ldb;
   const int nslab = g.K / BK;
-  v4i sta[NJ], stb[NJ];
+  v4i sta[NJ], stb[NJB];
   // The loads keep their program order (a scheduling barrier that only memory instructions may
   // not cross follows each one): the compiler's vmcnt bookkeeping is exact only if the order in
   // the prologue and in the loop is the same.
@@ -114,7 +115,7 @@ __global__ __launch_bounds__(256) void gemm_rs_kernel(GemmArgs g, Epi epi) {
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
       load_a(j, k0);
-      load_b(j, k0);
+      if (j < NJB) load_b(j, k0);
     }
   };
   // LDS position of the thread's chunk: row-major [row][128 B], chunk c of row r at c ^ swz(r);
@@ -124,7 +125,7 @@ __global__ __launch_bounds__(256) void gemm_rs_kernel(GemmArgs g, Epi epi) {
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
       *(v4i*)(buf + wr + j * 32 * BK) = sta[j];
-      *(v4i*)(buf + BM * BK + wr + j * 32 * BK) = stb[j];
+      if (j < NJB) *(v4i*)(buf + BM * BK + wr + j * 32 * BK) = stb[j];
     }
   };
 
@@ -185,7 +186,7 @@ __global__ __launch_bounds__(256) void gemm_rs_kernel(GemmArgs g, Epi epi) {
 
   // One k-step in explicit order.  Behind MFMA r (a full scheduling barrier closes every group):
   // read r of the fragments for the following k-step (from `rd_ls`, k-step `RS`, into buffer RB)
-  // and the staging pairs [P0, P1) spread evenly over the 16 MFMAs.  A pair = write one staged
+  // and the staging pairs [P0, P1) spread evenly over the FM x FN MFMAs.  A pair = write one staged
   // 16-byte chunk into `wr_buf`, then re-load its registers from slab `k0`.  Pair p < NJ is
   // operand A row group p, pair p >= NJ operand B row group p - NJ.
   auto pair = [&](uint8_t* wr_buf, int k0, auto p_c) {
@@ -221,10 +222,10 @@ __global__ __launch_bounds__(256) void gemm_rs_kernel(GemmArgs g, Epi epi) {
           ...);
     }(std::make_integer_sequence<int, NMMA>{});
   };
-  // Staging pairs [0, NP0) are handled in the last k-step of a slab, [NP0, 16) in the first
+  // Staging pairs [0, NP0) are handled in the last k-step of a slab, [NP0, NPAIR) in the first
   // k-step of the next one (int8 MFMAs are half as long as e4m3 ones: 16 of them cannot hide 16
   // buffer loads and 16 LDS writes).
-  constexpr int NPAIR = 2 * NJ;
+  constexpr int NPAIR = NJ + NJB;
   constexpr int NP0 = OP == MMA_I8 ? NPAIR / 2 : NPAIR;
   auto pairs_now = [&](uint8_t* wr_buf, int k0, auto p0_c, auto p1_c) {  // no MFMAs to hide behind
     [&]<int... P>(std::integer_sequence<int, P...>) {
@@ -238,17 +239,18 @@ __global__ __launch_bounds__(256) void gemm_rs_kernel(GemmArgs g, Epi epi) {
   auto slab_k0 = [&](int s) { return min(s, nslab - 1) * BK; };  // slabs past the end: never used
 
   // ---- prologue: slab 0 into LDS; slab 1: pairs [0, NP0) into LDS and their registers re-loaded
-  // with slab 2, pairs [NP0, 16) still staged (the first k-step of the loop writes them)
+  // with slab 2, pairs [NP0, NPAIR) still staged (the first k-step of the loop writes them)
   // (slabs 0 and 1 are fetched together: the accumulators and fragments are not live yet, so
   // there are registers for a second staging set)
   {
     load_slab(0);
-    v4i ta[NJ], tb[NJ];
+    v4i ta[NJ], tb[NJB];
     const int k1 = slab_k0(1);
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
       ta[j] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, va, j * sa32 + k1, 0));
-      tb[j] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, vb, j * sb32 + k1, 0));
+      if (j < NJB)
+        tb[j] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, vb, j * sb32 + k1, 0));
     }
     store_slab(lds);
     // slab 1: pairs [0, NP0) go to LDS, the rest stay staged

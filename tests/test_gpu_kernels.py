@@ -244,8 +244,9 @@ def _rand_i8(shape, seed):
 @pytest.mark.parametrize("shape", [(512, 4096, 4096), (300, 520, 1024), (256, 256, 64),
                                    (17, 4096, 4096), (1000, 1200, 256), (129, 130, 80),
                                    (64, 72, 4112), (2048, 2304, 512),
-                                   # large ragged shapes: 256x256 tiles, K in whole 128-byte slabs
-                                   (4000, 4100, 384), (4097, 4095, 128), (3900, 4352, 256)])
+                                   # large ragged shapes, K in whole 128-byte slabs: the first three
+                                   # run 256x192 tiles (fuller last round), the last one 256x256
+                                   (4000, 4100, 384), (4097, 4095, 128), (3900, 4352, 256), (4000, 4000, 384)])
 def test_gemm_i8_i32_exact(dev, shape):
     M, N, Kd = shape
     a, w = _rand_i8((M, Kd), 11), _rand_i8((N, Kd), 12)
@@ -266,7 +267,8 @@ def test_gemm_i8_i32_strided_rows(dev):
 
 
 @pytest.mark.parametrize("out_dtype", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("shape", [(512, 4096, 4096), (300, 520, 1024), (16, 512, 1024), (1, 256, 128)])
+@pytest.mark.parametrize("shape", [(512, 4096, 4096), (300, 520, 1024), (16, 512, 1024), (1, 256, 128),
+                                   (2048, 6100, 256)])  # 256x192 tiles, ragged last column tile
 def test_gemm_i8_dq_reference_epilogue_bit_exact(dev, shape, out_dtype):
     M, N, Kd = shape
     a, w = _rand_i8((M, Kd), 21), _rand_i8((N, Kd), 22)
@@ -357,11 +359,11 @@ def test_gemm_fp8_dq(dev, M):
     torch.testing.assert_close(y.cpu().float(), ref.float(), rtol=2e-2, atol=2e-2)
 
 
-@pytest.mark.parametrize("shape", [(256, 512, 1024), (4000, 4100, 384), (4097, 4095, 128)])
+@pytest.mark.parametrize("shape", [(256, 512, 1024), (4000, 4100, 384), (4097, 4095, 128), (4000, 4000, 384)])
 def test_gemm_fp8_integer_valued_is_exact(dev, shape):
     # small-integer operands: every product and partial sum is exact in fp32, so any MFMA
-    # summation order must give the exact integer result (the large ragged shapes run 256x256
-    # tiles with K in whole 128-byte slabs)
+    # summation order must give the exact integer result (the large ragged shapes run 256x192
+    # tiles, the last one 256x256, with K in whole 128-byte slabs)
     M, N, Kd = shape
     a = torch.randint(-4, 5, (M, Kd), generator=gen(46)).float().to(torch.float8_e4m3fn)
     w = torch.randint(-4, 5, (N, Kd), generator=gen(47)).float().to(torch.float8_e4m3fn)
