@@ -103,10 +103,14 @@ def main():
     layers = [make_layer(torch, dev, k, n, seed=1 + i) for i, (_, k, n) in enumerate(LLAMA3_8B)]
     total_ops = sum(2.0 * M_TOKENS * k * n for _, k, n in LLAMA3_8B)
 
+    clk = [torch.zeros(6, dtype=torch.int64, device=dev) for _ in layers]
+
     def step(events=None):
         for i, L in enumerate(layers):
             q, s = K.quant_act_i8_pertoken(L["x"], L["smooth"])
             if events is not None:
+                # block 0 of this launch stores its clock readings (core clock the GEMM ran at)
+                K.clock_probe(clk[i])
                 e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
                 e0.record()
             y = K.gemm_i8_dq(q, L["w"], s, L["w_scale"], L["bias"], out_dtype=torch.float16,
@@ -134,6 +138,7 @@ def main():
         step(events)
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
+    K.clock_probe(None)
     ms_per_step = dt / args.steps * 1e3
     value = total_ops / (dt / args.steps) / 1e12
 
@@ -141,6 +146,11 @@ def main():
     gemm_ops = [2.0 * M_TOKENS * k * n for _, k, n in LLAMA3_8B]
     per_shape = {name: round(o / (ms * 1e-3) / 1e12, 1) for (name, _, _), o, ms in zip(LLAMA3_8B, gemm_ops, gemm_ms)}
     achieved = sum(gemm_ops) / (sum(gemm_ms) * 1e-3) / 1e12
+    # Core clock of block 0 of the last timed launch of each shape.  The published peak is
+    # 2400 MHz x the MFMA rate; the operands' switching activity decides how far below that the
+    # power cap lets the clock settle, so the peak at the measured clock is reported beside it.
+    mhz = [K.core_clock_mhz(c) for c in clk]
+    peak_at_clock = sum(gemm_ops) / sum(o / (PEAK_INT8_TOPS * m / 2400.0) for o, m in zip(gemm_ops, mhz))
     traffic = None
     tfile = os.path.join(ROOT, "profiles", "gemm_i8_traffic.json")
     if os.path.exists(tfile):
@@ -161,7 +171,10 @@ def main():
                      "unit": "TFLOP/s", "frac": round(achieved / PEAK_INT8_TOPS, 4),
                      "traffic": traffic, "kernel": "gemm_rs_kernel<int8, dequant epilogue> (4 launches per step)",
                      "per_shape_tops": per_shape,
-                     "avg_launch_ms": {n: round(ms, 4) for (n, _, _), ms in zip(LLAMA3_8B, gemm_ms)}},
+                     "avg_launch_ms": {n: round(ms, 4) for (n, _, _), ms in zip(LLAMA3_8B, gemm_ms)},
+                     "core_clock_mhz": {n: round(m) for (n, _, _), m in zip(LLAMA3_8B, mhz)},
+                     "peak_at_measured_clock": round(peak_at_clock, 1),
+                     "frac_at_measured_clock": round(achieved / peak_at_clock, 4)},
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(torch, layers[1])

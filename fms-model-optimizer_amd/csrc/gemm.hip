@@ -11,6 +11,16 @@ int fmsmo_check_launch() {
   return FMSMO_ERR_LAUNCH;
 }
 
+unsigned long long*& fmsmo_clock_probe() {
+  static thread_local unsigned long long* probe = nullptr;
+  return probe;
+}
+extern "C" int fmsmo_debug_clock_probe(uint64_t* dev6) {
+  if (((uintptr_t)dev6) & 7) return FMSMO_ERR_ALIGN;
+  fmsmo_clock_probe() = (unsigned long long*)dev6;
+  return FMSMO_OK;
+}
+
 extern "C" int fmsmo_abi_version(void) { return FMSMO_ABI_VERSION; }
 extern "C" const char* fmsmo_last_error(void) { return g_fmsmo_last_error; }
 extern "C" const char* fmsmo_status_str(int s) {

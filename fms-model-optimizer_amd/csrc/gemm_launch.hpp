@@ -8,6 +8,9 @@
 using namespace fmsmo;
 
 int fmsmo_check_launch();
+// Device buffer of 6 x 64 bit that later register-staged GEMM launches of this thread fill with
+// block 0's clock readings (null = off); defined in gemm.hip.
+unsigned long long*& fmsmo_clock_probe();
 bool fmsmo_gemv_batch_ok(int64_t M, int64_t K);
 int fmsmo_gemv_dispatch(int op, const void* a, int64_t lda, const void* b, int64_t ldb,
                         const float* a_scale, int64_t a_scale_n, const float* w_scale,
@@ -89,6 +92,7 @@ static bool use_register_staged(int op) {
 template <int OP, bool GROUPED = false, int BN = 256, class Epi>
 void launch_rs(const GemmArgs& g0, const Epi& epi, hipStream_t st) {
   GemmArgs g = g0;
+  g.clk = fmsmo_clock_probe();
   g.grid_n = div_up(g.N, BN);
   if (!GROUPED) g.grid_m = div_up(g.M, 256);
   g.group_m = 4;

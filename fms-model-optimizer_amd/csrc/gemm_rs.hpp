@@ -83,9 +83,7 @@ __global__ __launch_bounds__(256) void gemm_rs_kernel(GemmArgs g, Epi epi) {
   }
   const int col_lo = tile_n * BN;
 
-#ifdef FMSMO_CLK
   if (blockIdx.x == 0 && tid == 0 && g.clk) { g.clk[0] = clock64(); g.clk[1] = wall_clock64(); }
-#endif
   // ---- global -> register staging: thread -> (row = tid / 8 + 32 j, 16-byte chunk = tid % 8)
   const int ld_row = tid >> 3, ld_chunk = tid & 7;
   const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
@@ -300,9 +298,7 @@ __global__ __launch_bounds__(256) void gemm_rs_kernel(GemmArgs g, Epi epi) {
     kstep(std::integral_constant<int, (NKS - 1) & 1>{}, nxt, C0{}, C0{}, cur, slab_k0(s + 3), C0{}, CNP0{});
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-#ifdef FMSMO_CLK
   if (blockIdx.x == 0 && tid == 0 && g.clk) { g.clk[2] = clock64(); g.clk[3] = wall_clock64(); }
-#endif
 
   // ---- epilogue: acc[i][j][v] is C(row, col) with
   //      row = 32 i + 8 (v / 4) + 4 (lane / 32) + v % 4,   col = 32 j + lane % 32
@@ -339,9 +335,7 @@ __global__ __launch_bounds__(256) void gemm_rs_kernel(GemmArgs g, Epi epi) {
       }
     }
   }
-#ifdef FMSMO_CLK
   if (blockIdx.x == 0 && tid == 0 && g.clk) { g.clk[4] = clock64(); g.clk[5] = wall_clock64(); }
-#endif
 #endif  // __HIP_DEVICE_COMPILE__
 }
 

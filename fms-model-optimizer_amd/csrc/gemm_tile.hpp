@@ -39,9 +39,9 @@ struct GemmArgs {
   int rows_per_group;  // > 0: every group owns this many rows (batched matmul, split K), offsets unused
   int64_t lda_e;       // uniform groups: bytes between groups in A (rows * lda for stacked batches,
                        // the K slice length when the groups are slices of one reduction)
-#ifdef FMSMO_CLK
-  unsigned long long* clk;  // harness only: {core clock, 100 MHz wall clock} at start / end
-#endif
+  // optional clock probe (register-staged kernel): block 0 stores {core clock counter, 100 MHz
+  // wall clock} at its start, after its K loop and after its epilogue; null = off
+  unsigned long long* clk;
 };
 
 // 16-byte chunk c of row r is stored at chunk position c ^ swz(r).  Depends on r & 15 only.

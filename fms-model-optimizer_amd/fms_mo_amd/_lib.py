@@ -49,6 +49,7 @@ SIGNATURES = {
     "fmsmo_bmm_i8_dq": [_P, _L, _P, _L, _L, _P, _P, _P, _P, _I, _L, _L, _L, _L, _L, _P],
     "fmsmo_bmm_fp8_dq": [_P, _L, _P, _L, _L, _P, _P, _P, _P, _I, _L, _L, _L, _L, _L, _P],
     "fmsmo_zero_shift_bias": [_P, _L, _P, _L, _P, _F, _P, _I, _P, _L, _L, _P],
+    "fmsmo_debug_clock_probe": [_P],
 }
 OTHER = {
     "fmsmo_abi_version": ([], c_int),

@@ -151,6 +151,26 @@ def _workspace(M, N, K, device):
     return torch.empty((nbytes,), dtype=torch.uint8, device=device) if nbytes > 0 else None
 
 
+def clock_probe(buf):
+    """Diagnostic: have block 0 of the following 256-row-tile GEMM launches store its clock
+    readings into `buf` (int64 [6] on the GPU), or switch the probe off with None.  See
+    fmsmo_debug_clock_probe; `core_clock_mhz` turns a filled buffer into a frequency."""
+    if buf is None:
+        L.call("fmsmo_debug_clock_probe", None)
+        return
+    _need_gpu(buf)
+    if buf.dtype != torch.int64 or buf.numel() < 6 or not buf.is_contiguous():
+        raise ValueError("the probe buffer must be a contiguous int64 tensor of 6 elements")
+    L.call("fmsmo_debug_clock_probe", buf.data_ptr())
+
+
+def core_clock_mhz(buf):
+    """Average core clock (MHz) over the life of the probed block: core cycles per tick of the
+    constant 100 MHz counter, start of the block to the end of its epilogue."""
+    c = buf.cpu().tolist()
+    return (c[4] - c[0]) / ((c[5] - c[1]) / 100.0)
+
+
 def _check_ab(a, w, dtype):
     _need_gpu(a, w)
     if a.dtype != dtype or w.dtype != dtype:

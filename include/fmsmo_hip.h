@@ -59,6 +59,19 @@ const char* fmsmo_status_str(int status);
 /* hipGetLastError text of the most recent FMSMO_ERR_LAUNCH on this thread ("" if none). */
 const char* fmsmo_last_error(void);
 
+/*
+ * Diagnostic with no counterpart in the reference: the core clock a GEMM really ran at.  After
+ * this call every 256-row-tile (register-staged) GEMM launched from the calling thread has its
+ * block 0 store six 64-bit values into dev6 (device memory, 8-byte aligned, valid until the probe
+ * is switched off with NULL and the launches have finished):
+ *   dev6[0], dev6[1]  core clock counter and constant 100 MHz counter when the block starts,
+ *   dev6[2], dev6[3]  after its K loop,  dev6[4], dev6[5]  after its epilogue.
+ * (dev6[4] - dev6[0]) / ((dev6[5] - dev6[1]) / 100) is the average core clock in MHz over the
+ * block's life.  MFMA throughput scales with that clock; the published peak assumes 2400 MHz.
+ * The pointer is read at launch time, so consecutive launches may be given different buffers.
+ */
+int fmsmo_debug_clock_probe(uint64_t* dev6);
+
 /* ------------------------------------------------------------------------------------------
  * 1. Activation quantizers (one pass over x: read 2-4 B, write 1 B per element).
  * ------------------------------------------------------------------------------------------ */

@@ -476,6 +476,28 @@ def test_grouped_gemm_equals_per_expert_linear(dev):
 
 
 # ------------------------------------------------------------------------------ error behaviour
+def test_clock_probe_reports_a_plausible_core_clock(dev):
+    # diagnostic entry point: block 0 of a 256-row-tile GEMM stores {core, 100 MHz} counter pairs
+    a, w = _rand_i8((4096, 256), 71).to(dev), _rand_i8((4096, 256), 72).to(dev)
+    buf = torch.zeros(6, dtype=torch.int64, device=dev)
+    K().clock_probe(buf)
+    try:
+        c = K().gemm_i8_i32(a, w)
+    finally:
+        K().clock_probe(None)
+    torch.cuda.synchronize()
+    t = buf.cpu().tolist()
+    assert t[0] < t[2] < t[4] and t[1] <= t[3] <= t[5] and t[5] > t[1]
+    assert 300.0 < K().core_clock_mhz(buf) < 2700.0
+    # switched off: the buffer stays as it is, the result is the same
+    buf.zero_()
+    c2 = K().gemm_i8_i32(a, w)
+    torch.cuda.synchronize()
+    assert int(buf.abs().sum()) == 0 and torch.equal(c, c2)
+    with pytest.raises(ValueError):
+        K().clock_probe(torch.zeros(6, dtype=torch.int32, device=dev))
+
+
 def test_errors_are_raised_not_swallowed(dev):
     from fms_mo_amd._lib import FmsMoHipError
 
