@@ -108,6 +108,39 @@ extern "C" int64_t fmsmo_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   return plan_split_k(M, N, K).ws_bytes;
 }
 
+extern "C" int fmsmo_gemm_plan(int64_t M, int64_t N, int64_t K, int with_workspace, int* kernel,
+                               int* tile_m, int* tile_n, int* splits) {
+  if (!kernel || !tile_m || !tile_n || !splits) return FMSMO_ERR_NULL;
+  if (M <= 0 || N <= 0 || K <= 0 || M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff)
+    return FMSMO_ERR_SHAPE;
+  if (K % 16) return FMSMO_ERR_ALIGN;
+  *tile_m = *tile_n = 0;
+  *splits = 1;
+  if ((M <= 16 && K % 128 == 0) || fmsmo_gemv_batch_ok(M, K)) {
+    *kernel = FMSMO_PLAN_DECODE;
+    return FMSMO_OK;
+  }
+  const SplitPlan plan = plan_split_k(M, N, K);
+  if (with_workspace && plan.splits > 1) {
+    *kernel = FMSMO_PLAN_TILE_LDS_DMA;
+    *tile_m = TileMid::BM;
+    *tile_n = TileMid::BN;
+    *splits = plan.splits;
+    return FMSMO_OK;
+  }
+  if (K % 64) {
+    *kernel = FMSMO_PLAN_GENERIC;
+    return FMSMO_OK;
+  }
+  const bool rs = K % 128 == 0 && use_register_staged(MMA_I8);
+  const int bm[4] = {256, 128, 128, 256}, bn[4] = {256, 256, 128, 192};
+  const int t = pick_tile((int)M, (int)N, rs);
+  *kernel = (rs && (t == 0 || t == 3)) ? FMSMO_PLAN_TILE_REGISTER_STAGED : FMSMO_PLAN_TILE_LDS_DMA;
+  *tile_m = bm[t];
+  *tile_n = (t == 3 && !rs) ? 256 : bn[t];
+  return FMSMO_OK;
+}
+
 extern "C" int fmsmo_grouped_gemm_i8_dq(const int8_t* a, int64_t lda, const int8_t* b,
                                         int64_t ldb, int64_t ldb_e, const int32_t* offsets,
                                         int num_experts, int64_t total_rows, const float* a_scale,

@@ -21,6 +21,7 @@ FP8_LINEAR, FP8_FPXACC, FP8_FPXACC_DL8 = 0, 1, 2
 WQ_MUL, WQ_DIV = 0, 1
 MS_PER_TOKEN, MS_SYMM, MS_ASYMM = 0, 1, 2
 ABI_VERSION = 1
+PLAN_DECODE, PLAN_TILE_REGISTER_STAGED, PLAN_TILE_LDS_DMA, PLAN_GENERIC = 0, 1, 2, 3
 
 _P, _I, _L, _F = c_void_p, c_int, c_int64, c_float
 
@@ -50,6 +51,7 @@ SIGNATURES = {
     "fmsmo_bmm_fp8_dq": [_P, _L, _P, _L, _L, _P, _P, _P, _P, _I, _L, _L, _L, _L, _L, _P],
     "fmsmo_zero_shift_bias": [_P, _L, _P, _L, _P, _F, _P, _I, _P, _L, _L, _P],
     "fmsmo_debug_clock_probe": [_P],
+    "fmsmo_gemm_plan": [_L, _L, _L, _I, _P, _P, _P, _P],
 }
 OTHER = {
     "fmsmo_abi_version": ([], c_int),

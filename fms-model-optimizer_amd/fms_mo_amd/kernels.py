@@ -151,6 +151,16 @@ def _workspace(M, N, K, device):
     return torch.empty((nbytes,), dtype=torch.uint8, device=device) if nbytes > 0 else None
 
 
+def gemm_plan(M, N, K, with_workspace=False):
+    """(kernel, tile_m, tile_n, splits) the *_dq GEMMs use for a shape; no GPU needed
+    (kernel is one of L.PLAN_*; see fmsmo_gemm_plan)."""
+    import ctypes
+
+    out = [ctypes.c_int(0) for _ in range(4)]
+    L.call("fmsmo_gemm_plan", M, N, K, int(bool(with_workspace)), *[ctypes.byref(o) for o in out])
+    return tuple(o.value for o in out)
+
+
 def clock_probe(buf):
     """Diagnostic: have block 0 of the following 256-row-tile GEMM launches store its clock
     readings into `buf` (int64 [6] on the GPU), or switch the probe off with None.  See

@@ -209,6 +209,24 @@ int fmsmo_gemm_fp8_dq(const uint8_t* a, int64_t lda, const uint8_t* b, int64_t l
  * No counterpart in the reference (its GEMMs are single launches of CUTLASS / cuBLASLt kernels).
  */
 int64_t fmsmo_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
+
+/*
+ * Which kernel the *_dq GEMMs run for a shape, without launching anything (host-only; for tests,
+ * tuning and capacity planning).  with_workspace != 0 describes the *_dq_ws calls given a
+ * sufficient workspace.  tile_m / tile_n are 0 for the decode and generic kernels; splits is the
+ * number of K slices (1 = single pass).  The choice weighs the measured efficiency of each tile
+ * shape against how full the last round of tiles leaves the 256 compute units, e.g.
+ * 4096 x 6144 runs 512 tiles of 256 x 192 (two full rounds) rather than 384 of 256 x 256.
+ * No counterpart in the reference (CUTLASS / cuBLASLt choose internally).
+ */
+enum fmsmo_plan_kernel {
+  FMSMO_PLAN_DECODE = 0,                /* skinny-M weight-streaming kernels */
+  FMSMO_PLAN_TILE_REGISTER_STAGED = 1,  /* MFMA tiles, 128-byte K slabs staged through registers */
+  FMSMO_PLAN_TILE_LDS_DMA = 2,          /* MFMA tiles, 64-byte K stages loaded straight into LDS */
+  FMSMO_PLAN_GENERIC = 3                /* K % 64 != 0: one thread per output element */
+};
+int fmsmo_gemm_plan(int64_t M, int64_t N, int64_t K, int with_workspace, int* kernel, int* tile_m,
+                    int* tile_n, int* splits);
 int fmsmo_gemm_i8_dq_ws(const int8_t* a, int64_t lda, const int8_t* b, int64_t ldb,
                         const float* a_scale, int64_t a_scale_n, const float* w_scale,
                         int64_t w_scale_n, const void* bias, int bias_dtype, int epilogue, void* y,

@@ -24,7 +24,7 @@ def test_header_declares_the_expected_entry_points():
               "fmsmo_grouped_gemm_i8_dq", "fmsmo_quant_weight_i8", "fmsmo_absmax_cols",
               "fmsmo_quant_act_i8_mulscale", "fmsmo_zero_shift_bias", "fmsmo_quant_i8_affine",
               "fmsmo_bmm_i8_dq", "fmsmo_bmm_fp8_dq", "fmsmo_gemm_i8_dq_ws", "fmsmo_gemm_fp8_dq_ws",
-              "fmsmo_gemm_workspace_bytes", "fmsmo_decode_linear_i8", "fmsmo_decode_linear_fp8", "fmsmo_decode_linear_ok", "fmsmo_debug_clock_probe", "fmsmo_abi_version", "fmsmo_status_str", "fmsmo_last_error"]:
+              "fmsmo_gemm_workspace_bytes", "fmsmo_decode_linear_i8", "fmsmo_decode_linear_fp8", "fmsmo_decode_linear_ok", "fmsmo_debug_clock_probe", "fmsmo_gemm_plan", "fmsmo_abi_version", "fmsmo_status_str", "fmsmo_last_error"]:
         assert s in syms
 
 
@@ -108,3 +108,38 @@ def test_workspace_plan_is_host_logic():
     assert b > 0 and b % (64 * 4096 * 4) == 0
     s = b // (64 * 4096 * 4)
     assert 2 <= s <= 8 and 14336 % (s * 128) == 0 and 14336 // s >= 512
+
+
+def test_gemm_plan_is_host_logic():
+    """Kernel and tile choice per shape, queried without a GPU: decode kernels for skinny M,
+    256 x 192 tiles where 256 x 256 would leave the last round of tiles half empty, split
+    reductions only with a workspace, the generic kernel when K is not a multiple of 64."""
+    from fms_mo_amd import _lib, kernels as K
+
+    if os.environ.get("FMSMO_TILE") or os.environ.get("FMSMO_RS") or os.environ.get("FMSMO_SPLIT_K"):
+        pytest.skip("tuning overrides are set")
+    RS, DMA = _lib.PLAN_TILE_REGISTER_STAGED, _lib.PLAN_TILE_LDS_DMA
+    # the four linears of a Llama-3-8B layer at 4096 tokens
+    assert K.gemm_plan(4096, 6144, 4096) == (RS, 256, 192, 1)     # 512 tiles = 2 full rounds
+    assert K.gemm_plan(4096, 4096, 4096) == (RS, 256, 256, 1)     # 256 tiles = 1 round
+    assert K.gemm_plan(4096, 28672, 4096) == (RS, 256, 256, 1)    # 1792 tiles = 7 rounds
+    assert K.gemm_plan(4096, 4096, 14336) == (RS, 256, 256, 1)
+    # decode and batched decode
+    assert K.gemm_plan(1, 4096, 4096)[0] == _lib.PLAN_DECODE
+    assert K.gemm_plan(16, 28672, 4096)[0] == _lib.PLAN_DECODE
+    assert K.gemm_plan(32, 4096, 8192)[0] == _lib.PLAN_DECODE
+    assert K.gemm_plan(64, 4096, 4096)[0] == _lib.PLAN_DECODE
+    assert K.gemm_plan(64, 4096, 8192)[0] != _lib.PLAN_DECODE
+    # a few tokens through a long reduction: split only when a workspace is offered
+    k, tm, tn, s = K.gemm_plan(17, 4096, 14336, with_workspace=True)
+    assert (k, tm, tn) == (DMA, 128, 128) and s >= 2 and 14336 % (s * 128) == 0
+    assert K.gemm_plan(17, 4096, 14336, with_workspace=False)[3] == 1
+    # K in 64-byte stages only: no register-staged kernel; K % 64 != 0: generic kernel
+    assert K.gemm_plan(4096, 4096, 4160)[0] == DMA
+    assert K.gemm_plan(300, 520, 1040) == (_lib.PLAN_GENERIC, 0, 0, 1)
+    # small problems take small tiles
+    assert K.gemm_plan(300, 520, 1024)[1:3] == (128, 128)
+    with pytest.raises(_lib.FmsMoHipError):
+        K.gemm_plan(0, 4096, 4096)
+    with pytest.raises(_lib.FmsMoHipError):
+        K.gemm_plan(128, 128, 100)
