@@ -255,6 +255,31 @@ def test_gemm_i8_i32_exact(dev, shape):
     assert torch.equal(c.cpu(), ref)
 
 
+def test_gemm_i8_i32_random_shapes_cover_every_kernel_choice(dev):
+    """Forty seeded shapes between 17 and ~4500 rows / columns: whatever kernel and tile shape the
+    library picks for a shape (fmsmo_gemm_plan names it), the int32 result must equal the exact
+    product, here taken in float64 on the GPU (|acc| < 2^53) so that large shapes stay cheap."""
+    import random
+
+    rng = random.Random(1234)
+    seen = set()
+    for case in range(40):
+        M = rng.choice([rng.randint(17, 300), rng.randint(300, 2100), rng.randint(2100, 4500)])
+        N = rng.choice([rng.randint(8, 300), rng.randint(300, 2100), rng.randint(2100, 6200)])
+        Kd = rng.choice([16 * rng.randint(1, 40), 64 * rng.randint(1, 24), 128 * rng.randint(1, 16)])
+        g = torch.Generator(device=dev).manual_seed(100 + case)
+        a = torch.randint(-128, 128, (M, Kd), generator=g, dtype=torch.int8, device=dev)
+        w = torch.randint(-128, 128, (N, Kd), generator=g, dtype=torch.int8, device=dev)
+        plan = K().gemm_plan(M, N, Kd)
+        seen.add(plan[:3])
+        c = K().gemm_i8_i32(a, w)
+        ref = (a.double() @ w.double().t()).to(torch.int32)
+        assert torch.equal(c, ref), f"M={M} N={N} K={Kd} plan={plan}"
+    # the sample reaches the generic kernel, both MFMA pipelines and all four tile shapes
+    assert {p[0] for p in seen} >= {1, 2, 3}
+    assert {p[1:] for p in seen if p[0] in (1, 2)} >= {(256, 256), (256, 192), (128, 256), (128, 128)}
+
+
 def test_gemm_i8_i32_strided_rows(dev):
     big_a, big_w = _rand_i8((200, 2048 + 64), 13), _rand_i8((300, 2048 + 128), 14)
     a, w = big_a[:, :2048], big_w[:, :2048]
