@@ -292,6 +292,14 @@ __device__ __forceinline__ float div32_fast(float x, float s, float r1) {
   q = __builtin_fmaf(__builtin_fmaf(-s, q, x), r1, q);
   return q;
 }
+// the same for x widened from fp16: with the first product written as fma(x, r1, -0) (nz: see
+// opaque_neg_zero) all three uses of x fold into v_fma_mix_f32 and no conversion is issued
+__device__ __forceinline__ float div32_fast_mix(float x, float s, float r1, float nz) {
+  float q = __builtin_fmaf(x, r1, nz);
+  q = __builtin_fmaf(__builtin_fmaf(-s, q, x), r1, q);
+  q = __builtin_fmaf(__builtin_fmaf(-s, q, x), r1, q);
+  return q;
+}
 
 template <int NCH, bool KEEP, int TH = AQ_THREADS>
 __global__ __launch_bounds__(TH) void quant_i8_pertoken_f16x_f32s_kernel(
@@ -325,6 +333,7 @@ __global__ __launch_bounds__(TH) void quant_i8_pertoken_f16x_f32s_kernel(
   }
   const bool ieee_block = __syncthreads_or(bad) != 0;
 
+  const float nz = opaque_neg_zero();
   v4i cur[NCH], nxt[NCH];
   float e[NCH][8];
   auto load_row = [&](int row, v4i (&dst)[NCH]) {
@@ -353,8 +362,8 @@ __global__ __launch_bounds__(TH) void quant_i8_pertoken_f16x_f32s_kernel(
         for (int j = 0; j < 8; ++j) {
           const float xv = f16_to_f32((u16)((uint32_t)cur[i][j >> 1] >> ((j & 1) * 16)));
           if constexpr (IEEE) e[i][j] = xv / d[j];
-          else if constexpr (KEEP) e[i][j] = div32_fast(xv, sv[i][j], sr[i][j]);
-          else e[i][j] = div32_fast(xv, d[j], rcp_refined(d[j]));
+          else if constexpr (KEEP) e[i][j] = div32_fast_mix(xv, sv[i][j], sr[i][j], nz);
+          else e[i][j] = div32_fast_mix(xv, d[j], rcp_refined(d[j]), nz);
           amax = fmaxf(amax, fabsf(e[i][j]));
         }
       }
@@ -401,14 +410,23 @@ __global__ __launch_bounds__(TH) void quant_i8_pertoken_f16x_f32s_kernel(
     for (int i = 0; i < NCH; ++i) {
       const int c = threadIdx.x + i * TH;
       if (c < nchunk) {
-        uint32_t o[2] = {0, 0};
+        uint32_t code[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-          float r = __builtin_rintf(ieee ? e[i][j] / s : div32_fast(e[i][j], s, rs));
-          if (saturate) r = fminf(fmaxf(r, -127.0f), 127.0f);
-          // |r| <= 128 in every finite row: r + 1.5 * 2^23 holds the two's-complement integer in
-          // its low mantissa bits
-          o[j >> 2] |= (__float_as_uint(r + 12582912.0f) & 0xffu) << ((j & 3) * 8);
+          float r = ieee ? e[i][j] / s : div32_fast(e[i][j], s, rs);
+          if (saturate) r = fminf(fmaxf(r, -127.0f), 127.0f);  // the bounds are integers
+          // |r| <= 128.5 in every finite row: the addition of 1.5 * 2^23 itself rounds r to the
+          // nearest integer, ties to even, and leaves it in two's complement in the low mantissa
+          // bits
+          code[j] = __float_as_uint(r + 12582912.0f);
+        }
+        // byte 0 of each code word -> 8 consecutive int8
+        uint32_t o[2];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const uint32_t lo = __builtin_amdgcn_perm(code[4 * h + 1], code[4 * h], 0x0c0c0400u);
+          const uint32_t hi = __builtin_amdgcn_perm(code[4 * h + 3], code[4 * h + 2], 0x0c0c0400u);
+          o[h] = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
         }
         *(uint2*)(qr + (size_t)c * AQ_VEC) = make_uint2(o[0], o[1]);
       }
