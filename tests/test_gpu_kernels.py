@@ -38,6 +38,27 @@ def test_quant_act_i8_pertoken(dev, dtype, shape):
     assert torch.equal(q.cpu(), q_ref)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("Kd", [64, 4096, 14336])
+def test_quant_act_row_maximum_found_in_every_lane_and_wave(dev, dtype, Kd):
+    """The row maximum is reduced across lanes with DPP row operations and across waves through
+    LDS: one row per 16-byte chunk position, its only large element inside that chunk, so a lane,
+    row of lanes or wave that the reduction skipped shows up as a wrong scale in its rows."""
+    nchunk = Kd // 8
+    rows = torch.arange(nchunk)
+    x = torch.full((nchunk, Kd), 0.001)
+    x[rows, rows * 8 + rows % 8] = (rows % 7 + 1).float() * torch.where(rows % 2 == 0, 1.0, -1.0)
+    x = x.to(dtype)
+    sm = (torch.rand(Kd, generator=gen(5)) + 0.5).to(dtype)
+    for smooth in (None, sm):
+        q_ref, s_ref, _ = O.quant_act_pertoken_i8(x, smooth)
+        q, s = K().quant_act_i8_pertoken(x.to(dev), None if smooth is None else smooth.to(dev))
+        assert torch.equal(s.cpu(), s_ref.float().reshape(-1))
+        assert torch.equal(q.cpu(), q_ref)
+    q8, s8 = K().quant_act_fp8_pertoken(x.to(dev))
+    assert torch.equal(s8.cpu(), O.fp8_dynamic_scale(x).reshape(-1))
+
+
 def test_quant_act_i8_bf16_wraps_like_reference(dev):
     # amax = 0.0103759765625 in bfloat16 quantises to 127.5 -> rint 128 -> int8 -128
     x = torch.zeros(2, 64, dtype=torch.bfloat16)
