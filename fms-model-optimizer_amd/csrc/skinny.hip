@@ -291,13 +291,20 @@ __global__ __launch_bounds__(NW * 64) void gemv_kernel(GemvArgs g) {
 // MT > 1: batches of up to 16 MT tokens.  The weight stream is the same; every step feeds MT
 // MFMAs (one per tile of 16 tokens) from the same weight fragment, so up to 64 tokens cost little
 // more than 16 as long as their activation fragments fit in registers (MT * STEPS * 8 VGPRs).
-template <int OP, int STEPS, int NW, int D, int MT = 1>
+// XL > 0: long rows with at most XL tokens.  The activation rows live in LDS (XL rows of K + 32
+// bytes: the pad puts the rows 8 banks apart) instead of STEPS * 8 registers per lane, which makes
+// room to keep every load of the wave's K slice in flight at once (D = STEPS).
+template <int OP, int STEPS, int NW, int D, int MT = 1, int XL = 0>
 __global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(GemvArgs g, int G) {
   static_assert(STEPS % D == 0, "pipeline depth must divide the steps per group");
+  static_assert(XL == 0 || MT == 1, "activations in LDS: one tile of tokens");
   typedef typename std::conditional<OP == FMSMO_OP_I8, int, float>::type AccT;
   typedef AccT Acc4 __attribute__((ext_vector_type(4)));
+  constexpr int XPITCH = 128 * STEPS * NW + 32;
+  constexpr int NRED = XL ? 1 : 2;  // exchange buffers (one and a second barrier when LDS is short)
   __shared__ __attribute__((aligned(16))) uint8_t stage[NW][2][2048];
-  __shared__ AccT red[2][NW][256 * MT];
+  __shared__ AccT red[NRED][NW][256 * MT];
+  __shared__ __attribute__((aligned(16))) uint8_t xs[XL ? XL * XPITCH : 16];
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int r = lane & 15, kg = lane >> 4;
@@ -307,14 +314,27 @@ __global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(GemvArgs g, int G)
   const int kwave = wave * (STEPS * 128);
 
   // activation fragments: lane (m = r, kg) holds x[m][kwave + s*128 + (h*4 + kg)*16 ...]
-  v4i xf[MT][STEPS][2];
+  v4i xf[XL ? 1 : MT][XL ? 1 : STEPS][2];
+  // XL: the block's copy of x, 16-byte chunks dealt round-robin to the threads; fetched before
+  // the weights so that it arrives first (loads complete in order)
+  constexpr int XCH = 8 * STEPS * NW;                                  // chunks per row
+  constexpr int XPT = XL ? (XL * XCH + NW * 64 - 1) / (NW * 64) : 1;  // chunks per thread
+  v4i xcp[XPT];
+  if constexpr (XL) {
 #pragma unroll
-  for (int t = 0; t < MT; ++t) {
-    const uint8_t* xp = g.a + (int64_t)min(t * 16 + r, g.M - 1) * g.lda + kwave + kg * 16;
+    for (int i = 0; i < XPT; ++i) {
+      const int c = min((int)threadIdx.x + i * NW * 64, g.M * XCH - 1);
+      xcp[i] = *(const v4i*)(g.a + (int64_t)(c / XCH) * g.lda + (c % XCH) * 16);
+    }
+  } else {
 #pragma unroll
-    for (int s = 0; s < STEPS; ++s) {
-      xf[t][s][0] = *(const v4i*)(xp + s * 128);
-      xf[t][s][1] = *(const v4i*)(xp + s * 128 + 64);
+    for (int t = 0; t < MT; ++t) {
+      const uint8_t* xp = g.a + (int64_t)min(t * 16 + r, g.M - 1) * g.lda + kwave + kg * 16;
+#pragma unroll
+      for (int s = 0; s < STEPS; ++s) {
+        xf[t][s][0] = *(const v4i*)(xp + s * 128);
+        xf[t][s][1] = *(const v4i*)(xp + s * 128 + 64);
+      }
     }
   }
   // weight loads: lane -> (row = lane / 8 [+8], 16-byte chunk = lane % 8): 8 rows x 128 B each
@@ -340,6 +360,15 @@ __global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(GemvArgs g, int G)
   v4i wb[D][2];
 #pragma unroll
   for (int j = 0; j < D; ++j) load_item(false, j, wb[j]);
+  const int xrd = min(r, g.M - 1) * XPITCH + kwave + kg * 16;
+  if constexpr (XL) {
+#pragma unroll
+    for (int i = 0; i < XPT; ++i) {
+      const int c = (int)threadIdx.x + i * NW * 64;
+      if (c < g.M * XCH) *(v4i*)(xs + (c / XCH) * XPITCH + (c % XCH) * 16) = xcp[i];
+    }
+    __syncthreads();
+  }
 
   // epilogue operands of output element e = threadIdx.x (n = e / 16, m = e % 16 of the group) are
   // fetched at the top of each group so that their latency hides behind the weight stream
@@ -373,13 +402,19 @@ __global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(GemvArgs g, int G)
       const v4i w1 = *(const v4i*)(st + rd1);
 #pragma unroll
       for (int t = 0; t < MT; ++t) {
+        v4i x0, x1;
+        if constexpr (XL) {
+          x0 = *(const v4i*)(xs + xrd + s * 128);
+          x1 = *(const v4i*)(xs + xrd + s * 128 + 64);
+        } else {
+          x0 = xf[t][s][0], x1 = xf[t][s][1];
+        }
         if constexpr (OP == FMSMO_OP_I8) {
-          acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w0, xf[t][s][0], acc[t], 0, 0, 0);
-          acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w1, xf[t][s][1], acc[t], 0, 0, 0);
+          acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w0, x0, acc[t], 0, 0, 0);
+          acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w1, x1, acc[t], 0, 0, 0);
         } else {
           const v8i wv = {w0[0], w0[1], w0[2], w0[3], w1[0], w1[1], w1[2], w1[3]};
-          const v8i xv = {xf[t][s][0][0], xf[t][s][0][1], xf[t][s][0][2], xf[t][s][0][3],
-                          xf[t][s][1][0], xf[t][s][1][1], xf[t][s][1][2], xf[t][s][1][3]};
+          const v8i xv = {x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
           acc[t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wv, xv, acc[t], 0, 0, 0, 0, 0, 0);
         }
       }
@@ -391,16 +426,16 @@ __global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(GemvArgs g, int G)
       pc[0] = pn[0], pc[1] = pn[1];
       pn[0] = rowptr(gi + 2, 0), pn[1] = rowptr(gi + 2, 1);
     }
-    AccT* mine = &red[gi & 1][wave][0];
+    AccT* mine = &red[gi % NRED][wave][0];
 #pragma unroll
     for (int t = 0; t < MT; ++t)
 #pragma unroll
       for (int v = 0; v < 4; ++v) mine[t * 256 + (kg * 4 + v) * 16 + r] = acc[t][v];
     __syncthreads();
     auto finish = [&](int e, float as_e, float ws_e, float bv_e) {
-      AccT sum = red[gi & 1][0][e];
+      AccT sum = red[gi % NRED][0][e];
 #pragma unroll
-      for (int w = 1; w < NW; ++w) sum += red[gi & 1][w][e];
+      for (int w = 1; w < NW; ++w) sum += red[gi % NRED][w][e];
       const int n = (group0 + gi) * 16 + ((e >> 4) & 15), m = (e >> 8) * 16 + (e & 15);
       if (n < g.N && m < g.M) {
         float out;
@@ -427,6 +462,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(GemvArgs g, int G)
         finish(e, g.a_scale[g.a_stride ? m : 0], ws, bv);
       }
     }
+    if constexpr (NRED == 1 && !LAST) __syncthreads();  // the next group reuses the exchange buffer
   };
   for (int gi = 0; gi + 1 < gcount; ++gi) do_group(std::false_type{}, gi);
   do_group(std::true_type{}, gcount - 1);
@@ -672,6 +708,15 @@ int fmsmo_gemv_dispatch(int op, const void* a, int64_t lda, const void* b, int64
     if (G > 64) G = 64;
     dim3 grid((unsigned)((groups + G - 1) / G)), block(NW * 64);
     bool handled = true;
+    // K = 14336 with 3 .. 8 tokens: activations in LDS, all 14 steps of loads in flight
+    // (N = 4096, us at M = 3 / 4 / 8: 15.8 -> 15.0, 15.9 -> 14.7, 17.0 -> 15.4)
+    if (M >= 3 && M <= 8 && NW == 8 && STEPS == 14) {
+      if (op == FMSMO_OP_I8)
+        hipLaunchKernelGGL((gemv_stream_kernel<FMSMO_OP_I8, 14, 8, 14, 1, 8>), grid, block, 0, st, g, G);
+      else
+        hipLaunchKernelGGL((gemv_stream_kernel<FMSMO_OP_E4M3, 14, 8, 14, 1, 8>), grid, block, 0, st, g, G);
+      return fmsmo_check_launch();
+    }
 #define GEMV_STREAM(OPV, NWV, ST, DV)                                                             \
   if (M <= 16) hipLaunchKernelGGL((gemv_stream_kernel<OPV, ST, NWV, DV>), grid, block, 0, st, g, G); \
   else if constexpr (NWV == 8 && ST <= 8) {                                                        \

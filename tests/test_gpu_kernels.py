@@ -385,6 +385,30 @@ def test_gemv_i8_matches_gemm_semantics(dev, M, NK):
     assert torch.equal(y_auto.cpu().view(torch.int16), ref.view(torch.int16))
 
 
+@pytest.mark.parametrize("M", [3, 5, 8, 9])
+@pytest.mark.parametrize("N", [1000, 8200])
+def test_decode_long_rows_with_activations_in_lds(dev, M, N):
+    """K = 14336 with 3 .. 8 tokens keeps the activation rows in LDS (9 tokens: registers again).
+    N = 1000: ragged last group of 16 weight rows; N = 8200: several groups per block, which
+    reuse one exchange buffer behind a second barrier.  int8 bit-exact, e4m3 exact on small
+    integers."""
+    Kd = 14336
+    a, w = _rand_i8((M, Kd), 36), _rand_i8((N, Kd), 37)
+    s_a = (torch.rand(M, 1, generator=gen(38)) * 0.05 + 1e-3).half()
+    s_w = (torch.rand(N, generator=gen(39)) * 1e-3 + 1e-5).float()
+    bias = (torch.randn(N, generator=gen(40)) * 0.01).half()
+    ref = O.epilogue_ref(O.int_gemm(a, w), s_a, s_w, bias, torch.float16)
+    y = K().gemm_i8_dq(a.to(dev), w.to(dev), s_a.float().to(dev), s_w.to(dev), bias.to(dev),
+                       out_dtype=torch.float16, exact_ref=True)
+    assert torch.equal(y.cpu().view(torch.int16), ref.view(torch.int16))
+    a8 = torch.randint(-3, 4, (M, Kd), generator=gen(41)).float()
+    w8 = torch.randint(-3, 4, (N, Kd), generator=gen(42)).float()
+    one = torch.ones(1, device=dev)
+    y8 = K().gemm_fp8_dq(a8.to(torch.float8_e4m3fn).to(dev), w8.to(torch.float8_e4m3fn).to(dev), one, one,
+                         None, out_dtype=torch.float32)
+    assert torch.equal(y8.cpu(), a8 @ w8.t())
+
+
 def _rand_fp8(shape, seed, scale=1.0):
     return (torch.randn(shape, generator=gen(seed)) * scale).clamp(-448, 448).to(torch.float8_e4m3fn)
 
