@@ -865,11 +865,11 @@ extern "C" int fmsmo_quant_act_i8_pertoken(const void* x, int x_dtype, int64_t l
   if (M == 0) return FMSMO_OK;
   hipStream_t st = (hipStream_t)stream;
   // 16-bit fast path: x, the divisor and the compute dtype all fp16 (or all bf16), row cached in
-  // registers (K <= 16384)
+  // registers (K <= 32768)
   if (x_dtype != FMSMO_F32 && compute_dtype == x_dtype && (!smooth || smooth_dtype == x_dtype) &&
-      K <= AQ_MAXCHUNK * AQ_THREADS * AQ_VEC) {
+      K <= 2 * AQ_MAXCHUNK * AQ_THREADS * AQ_VEC) {
     const int64_t per_thread = div_up(K, AQ_THREADS * AQ_VEC);
-    const int nch = per_thread <= 1 ? 1 : per_thread <= 2 ? 2 : per_thread <= 4 ? 4 : 8;
+    const int nch = per_thread <= 1 ? 1 : per_thread <= 2 ? 2 : per_thread <= 4 ? 4 : per_thread <= 8 ? 8 : 16;
     // rows longer than 8192 elements: 512-thread blocks with 4 chunks per thread (more, shorter
     // lanes: 45 vs 49 us at K = 14336 with the SmoothQuant divide, 34 vs 38 us without)
 #define LAUNCH16(T, NCH, SM, TH, KEEP)                                                           \
@@ -886,8 +886,9 @@ extern "C" int fmsmo_quant_act_i8_pertoken(const void* x, int x_dtype, int64_t l
     case 2: LAUNCH16(T, 1, false, 256, true); break;  case 3: LAUNCH16(T, 1, true, 256, true); break;   \
     case 4: LAUNCH16(T, 2, false, 256, true); break;  case 5: LAUNCH16(T, 2, true, 256, true); break;   \
     case 8: LAUNCH16(T, 4, false, 256, true); break;  case 9: LAUNCH16(T, 4, true, 256, true); break;   \
-    case 16: LAUNCH16(T, 4, false, 512, true); break;                                                   \
-    default: LAUNCH16(T, 4, true, 512, false); break;                                                   \
+    case 16: LAUNCH16(T, 4, false, 512, true); break; case 17: LAUNCH16(T, 4, true, 512, false); break; \
+    case 32: LAUNCH16(T, 8, false, 512, true); break;                                                   \
+    default: LAUNCH16(T, 8, true, 512, false); break; /* 16384 < K <= 32768 */                          \
   }
     if (x_dtype == FMSMO_F16) { PICK16(FMSMO_F16) } else { PICK16(FMSMO_BF16) }
 #undef PICK16

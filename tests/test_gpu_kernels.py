@@ -89,7 +89,7 @@ def test_quant_act_i8_smoothquant(dev, sdtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("shape", [(4133, 64), (2500, 4096), (530, 14336)])
+@pytest.mark.parametrize("shape", [(4133, 64), (2500, 4096), (530, 14336), (300, 28672), (70, 32768)])
 def test_quant_act_i8_rows_walked_by_one_block(dev, dtype, shape):
     """More rows than resident blocks (each block quantizes several rows, prefetching the next),
     16-bit SmoothQuant divisors with a narrow range so that every x / smooth rounding shows in q."""
