@@ -672,7 +672,9 @@ int fmsmo_gemv_dispatch(int op, const void* a, int64_t lda, const void* b, int64
     case 1: GEMV_ROWS_M(OPV, 1, 8) break;                       \
     case 2: GEMV_ROWS_M(OPV, 2, 8) break;                       \
     case 4: GEMV_ROWS_M(OPV, 4, 4) break;                       \
+    case 5: GEMV_ROWS_M(OPV, 5, 2) break;                       \
     case 8: GEMV_ROWS_M(OPV, 8, 2) break;                       \
+    case 11: GEMV_ROWS_M(OPV, 11, 1) break;                     \
     case 13: GEMV_ROWS_M(OPV, 13, 1) break;                     \
     case 14: GEMV_ROWS_M(OPV, 14, 1) break;                     \
     case 16: GEMV_ROWS_M(OPV, 16, 1) break;                     \
@@ -729,6 +731,7 @@ int fmsmo_gemv_dispatch(int op, const void* a, int64_t lda, const void* b, int64
     case 801: GEMV_STREAM(OPV, 8, 1, 1); break;                     \
     case 802: GEMV_STREAM(OPV, 8, 2, 2); break;                     \
     case 804: GEMV_STREAM(OPV, 8, 4, 4); break;                     \
+    case 805: GEMV_STREAM(OPV, 8, 5, 5); break;                     \
     case 808: GEMV_STREAM(OPV, 8, 8, 4); break;                     \
     case 814: GEMV_STREAM(OPV, 8, 14, 7); break;                    \
     case 816: GEMV_STREAM(OPV, 8, 16, 4); break;                    \

@@ -367,8 +367,9 @@ def test_c1_config_deploy_forward(dev):
 
 
 # ------------------------------------------------------------------------------ skinny (decode)
-@pytest.mark.parametrize("M", [1, 4, 16, 7])
-@pytest.mark.parametrize("NK", [(4096, 4096), (6144, 4096), (4096, 14336), (1000, 384)])
+@pytest.mark.parametrize("M", [1, 2, 4, 16, 7])
+@pytest.mark.parametrize("NK", [(4096, 4096), (6144, 4096), (4096, 14336), (1000, 384),
+                                (1000, 5120), (520, 11008), (300, 13824)])  # Llama-2 reduction lengths
 def test_gemv_i8_matches_gemm_semantics(dev, M, NK):
     N, Kd = NK
     a, w = _rand_i8((M, Kd), 31), _rand_i8((N, Kd), 32)
