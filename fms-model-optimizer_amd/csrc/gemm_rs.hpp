@@ -19,7 +19,11 @@
 
 namespace fmsmo {
 
-template <int OP, class Epi, bool GROUPED = false, int BN_ = 256>
+//
+// ONE_SLAB: K == 128 (attention scores: head dimension 128).  The tile is one slab, so nothing is
+// prefetched: without the flag the pipeline would fetch slabs "1", "2" and "3" (clamped re-reads
+// of slab 0, 256 KiB per tile) and write them to LDS in front of the epilogue's stores.
+template <int OP, class Epi, bool GROUPED = false, int BN_ = 256, bool ONE_SLAB = false>
 __global__ __launch_bounds__(256) void gemm_rs_kernel(GemmArgs g, Epi epi) {
 #if defined(__HIP_DEVICE_COMPILE__)
   typedef Mma<OP> MM;
@@ -240,7 +244,10 @@ __global__ __launch_bounds__(256) void gemm_rs_kernel(GemmArgs g, Epi epi) {
   // with slab 2, pairs [NP0, NPAIR) still staged (the first k-step of the loop writes them)
   // (slabs 0 and 1 are fetched together: the accumulators and fragments are not live yet, so
   // there are registers for a second staging set)
-  {
+  if constexpr (ONE_SLAB) {
+    load_slab(0);
+    store_slab(lds);
+  } else {
     load_slab(0);
     v4i ta[NJ], tb[NJB];
     const int k1 = slab_k0(1);
@@ -279,6 +286,22 @@ __global__ __launch_bounds__(256) void gemm_rs_kernel(GemmArgs g, Epi epi) {
   __syncthreads();
   read_all(lds, 0, 0);
 
+  if constexpr (ONE_SLAB) {
+    // the k-steps of the only slab, nothing staged (the last one reads no further fragments)
+    [&]<int... KS>(std::integer_sequence<int, KS...>) {
+      (kstep(std::integral_constant<int, KS & 1>{}, lds, std::integral_constant<int, KS + 1>{},
+             std::integral_constant<int, (KS + 1) & 1>{}, lds, 0, C0{}, C0{}),
+       ...);
+    }(std::make_integer_sequence<int, NKS - 1>{});
+    [&]<int... R>(std::integer_sequence<int, R...>) {
+      (
+          [&] {
+            constexpr int I = R / FN, J = R % FN;
+            acc[I][J] = MM::mma(frag_a((NKS - 1) & 1, I), frag_b((NKS - 1) & 1, J), acc[I][J]);
+          }(),
+          ...);
+    }(std::make_integer_sequence<int, NMMA>{});
+  } else
   for (int s = 0; s < nslab; ++s) {
     uint8_t* cur = lds + (s & 1) * SLAB;
     uint8_t* nxt = lds + ((s + 1) & 1) * SLAB;
