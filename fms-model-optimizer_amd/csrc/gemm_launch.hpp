@@ -89,15 +89,15 @@ static bool use_register_staged(int op) {
   (void)op;
   return true;
 }
-template <int OP, bool GROUPED = false, int BN = 256, bool ONE_SLAB = false, class Epi>
+template <int OP, bool GROUPED = false, int BN = 256, bool ONE_SLAB = false, int BM = 256, class Epi>
 void launch_rs(const GemmArgs& g0, const Epi& epi, hipStream_t st) {
   GemmArgs g = g0;
   g.clk = fmsmo_clock_probe();
   g.grid_n = div_up(g.N, BN);
-  if (!GROUPED) g.grid_m = div_up(g.M, 256);
+  if (!GROUPED) g.grid_m = div_up(g.M, BM);
   g.group_m = 4;
   dim3 grid((unsigned)(g.grid_m * g.grid_n)), block(256);
-  hipLaunchKernelGGL((gemm_rs_kernel<OP, Epi, GROUPED, BN, ONE_SLAB>), grid, block, 0, st, g, epi);
+  hipLaunchKernelGGL((gemm_rs_kernel<OP, Epi, GROUPED, BN, ONE_SLAB, BM>), grid, block, 0, st, g, epi);
 }
 
 // Generic fallback (any K % 16 == 0): one thread per output element, 4-byte dot products.
@@ -304,7 +304,10 @@ int launch_bmm(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t s
       launch_tile<TileMid, OP, true>(g, epi, st);                                           \
     } else {                                                                                \
       g.grid_m = (int)batch * div_up(M, 256);                                               \
-      if (K == 128 && use_register_staged(OP)) launch_rs<OP, true, 256, true>(g, epi, st);  \
+      if (K == 128 && use_register_staged(OP)) {                                            \
+        g.grid_m = (int)batch * div_up(M, 128);                                             \
+        launch_rs<OP, true, 256, true, 128>(g, epi, st);                                    \
+      }                                                                                     \
       else if (K % 128 == 0 && use_register_staged(OP)) launch_rs<OP, true>(g, epi, st);    \
       else launch_tile<TileBig, OP, true>(g, epi, st);                                      \
     }                                                                                       \

@@ -23,21 +23,24 @@ namespace fmsmo {
 // ONE_SLAB: K == 128 (attention scores: head dimension 128).  The tile is one slab, so nothing is
 // prefetched: without the flag the pipeline would fetch slabs "1", "2" and "3" (clamped re-reads
 // of slab 0, 256 KiB per tile) and write them to LDS in front of the epilogue's stores.
-template <int OP, class Epi, bool GROUPED = false, int BN_ = 256, bool ONE_SLAB = false>
-__global__ __launch_bounds__(256) void gemm_rs_kernel(GemmArgs g, Epi epi) {
+// With BM_ = 128 (wave tile 64 x 128, 128 accumulator registers, one 48 KiB slab) two blocks
+// share a compute unit, so that the load, multiply and store phases of neighbouring tiles overlap.
+template <int OP, class Epi, bool GROUPED = false, int BN_ = 256, bool ONE_SLAB = false, int BM_ = 256>
+__global__ __launch_bounds__(256, BM_ == 128 ? 2 : 1) void gemm_rs_kernel(GemmArgs g, Epi epi) {
 #if defined(__HIP_DEVICE_COMPILE__)
   typedef Mma<OP> MM;
   typedef typename MM::Frag Frag;
   typedef typename MM::Acc Acc;
   static_assert(BN_ == 256 || BN_ == 192, "tile width");
-  constexpr int BM = 256, BN = BN_, BK = 128, CPR = 8;
-  constexpr int TM = 128, TN = BN / 2, FM = 4, FN = TN / 32;
+  static_assert(BM_ == 256 || (BM_ == 128 && ONE_SLAB), "tile height (128 rows: single-slab mode only)");
+  constexpr int BM = BM_, BN = BN_, BK = 128, CPR = 8;
+  constexpr int TM = BM / 2, TN = BN / 2, FM = TM / 32, FN = TN / 32;
   constexpr int NKS = BK / MM::KSTEP;   // MFMA k-steps per slab (int8 4, e4m3 2)
   constexpr int CL = MM::KSTEP / 32;    // 16-byte chunks per lane per k-step
   constexpr int SLAB = (BM + BN) * BK;  // 64 KiB (56 KiB for the 192-column tile)
   constexpr int NJ = BM / 32, NJB = BN / 32;  // row groups of 32 per thread: A, B
   static_assert(NKS % 2 == 0, "fragment buffers alternate per k-step");
-  __shared__ __attribute__((aligned(16))) uint8_t lds[2 * SLAB];
+  __shared__ __attribute__((aligned(16))) uint8_t lds[(ONE_SLAB ? 1 : 2) * SLAB];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -115,8 +118,8 @@ __global__ __launch_bounds__(256) void gemm_rs_kernel(GemmArgs g, Epi epi) {
   auto load_slab = [&](int s) {
     const int k0 = min(s, nslab - 1) * BK;  // slabs past the end re-read the last one (never used)
 #pragma unroll
-    for (int j = 0; j < NJ; ++j) {
-      load_a(j, k0);
+    for (int j = 0; j < (NJ > NJB ? NJ : NJB); ++j) {
+      if (j < NJ) load_a(j, k0);
       if (j < NJB) load_b(j, k0);
     }
   };
@@ -125,8 +128,8 @@ __global__ __launch_bounds__(256) void gemm_rs_kernel(GemmArgs g, Epi epi) {
   const int wr = ld_row * BK + ((ld_chunk ^ swz<CPR, 1>(ld_row)) * 16);
   auto store_slab = [&](uint8_t* buf) {
 #pragma unroll
-    for (int j = 0; j < NJ; ++j) {
-      *(v4i*)(buf + wr + j * 32 * BK) = sta[j];
+    for (int j = 0; j < (NJ > NJB ? NJ : NJB); ++j) {
+      if (j < NJ) *(v4i*)(buf + wr + j * 32 * BK) = sta[j];
       if (j < NJB) *(v4i*)(buf + BM * BK + wr + j * 32 * BK) = stb[j];
     }
   };

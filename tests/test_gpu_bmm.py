@@ -50,7 +50,7 @@ def test_affine_quantizer_strided_input(dev):
     assert torch.equal(q[..., :40], O.qbmm_quant(x[..., 3:43], scale, zp).reshape(8, 50, 40))
 
 
-@pytest.mark.parametrize("shape", [(4, 256, 256, 128), (3, 100, 77, 64), (2, 300, 128, 320),
+@pytest.mark.parametrize("shape", [(4, 256, 256, 128), (3, 300, 333, 128), (3, 100, 77, 64), (2, 300, 128, 320),
                                    (5, 64, 40, 192), (1, 513, 700, 256)])
 @pytest.mark.parametrize("with_bias", [False, True])
 def test_bmm_i8_exact(dev, shape, with_bias):
@@ -68,7 +68,7 @@ def test_bmm_i8_exact(dev, shape, with_bias):
     torch.testing.assert_close(y.double(), ref, rtol=2e-7, atol=1e-6)
 
 
-@pytest.mark.parametrize("shape", [(4, 256, 256, 128), (3, 100, 77, 64), (2, 130, 128, 384)])
+@pytest.mark.parametrize("shape", [(4, 256, 256, 128), (3, 300, 333, 128), (3, 100, 77, 64), (2, 130, 128, 384)])
 def test_bmm_fp8_exact_on_integer_operands(dev, shape):
     B, M, N, Kd = shape
     g = gen(10)
