@@ -296,10 +296,22 @@ int launch_bmm(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t s
   g.lda_e = M * lda;
   // small per-batch outputs (attention heads: N or M of 128) take the 128x128 tile
   const bool mid = N <= 128 || M <= 128;
+  // probabilities x values: many rows, one head dimension of columns, a long reduction whose
+  // A operand is read exactly once -- 256 x 128 tiles of the register-staged pipeline (whole
+  // 128-byte lines of P), every block starting its reduction at a different slab: with all blocks
+  // sweeping K in step, rows a power of two apart ask for the same memory channels at the same
+  // time (4096 x 128 x 4096 per head, 32 heads: 0.144 ms in step, 0.118 ms staggered).  Operands
+  // that several tiles share (the large GEMMs) want the opposite: their tiles meet in L2 because
+  // they sweep K together (K = 14336: 205 -> 255 us when staggered).
+  const bool tall = N > 64 && N <= 128 && M >= 256 && K % 128 == 0 && K >= 512 && use_register_staged(OP);
+  g.k_rotate = tall ? 5 : 0;
 #define GO(OUT)                                                                             \
   {                                                                                         \
     EpiDequant<OUT, FMSMO_F32, false, AccT> epi{y, ldy, a_scale, b_scale, bias, 0, 0};      \
-    if (mid) {                                                                              \
+    if (tall) {                                                                             \
+      g.grid_m = (int)batch * div_up(M, 256);                                               \
+      launch_rs<OP, true, 128>(g, epi, st);                                                 \
+    } else if (mid) {                                                                       \
       g.grid_m = (int)batch * div_up(M, TileMid::BM);                                       \
       launch_tile<TileMid, OP, true>(g, epi, st);                                           \
     } else {                                                                                \

@@ -31,7 +31,7 @@ __global__ __launch_bounds__(256, BM_ == 128 ? 2 : 1) void gemm_rs_kernel(GemmAr
   typedef Mma<OP> MM;
   typedef typename MM::Frag Frag;
   typedef typename MM::Acc Acc;
-  static_assert(BN_ == 256 || BN_ == 192, "tile width");
+  static_assert(BN_ == 256 || BN_ == 192 || BN_ == 128, "tile width");
   static_assert(BM_ == 256 || (BM_ == 128 && ONE_SLAB), "tile height (128 rows: single-slab mode only)");
   constexpr int BM = BM_, BN = BN_, BK = 128, CPR = 8;
   constexpr int TM = BM / 2, TN = BN / 2, FM = TM / 32, FN = TN / 32;
@@ -102,6 +102,15 @@ __global__ __launch_bounds__(256, BM_ == 128 ? 2 : 1) void gemm_rs_kernel(GemmAr
   const int vb = (col_lo + ld_row) * (int)g.ldb + ld_chunk * 16;
   const int sa32 = 32 * (int)g.lda, sb32 = 32 * (int)g.ldb;
   const int nslab = g.K / BK;
+  // slabs past the end: never used.  With k_rotate the block walks the slabs from its own
+  // starting point (all blocks sweeping K in step would ask for the same address bits 7.. of
+  // rows a power of two apart at the same time).
+  const int s0 = g.k_rotate ? (int)((blockIdx.x * (unsigned)g.k_rotate) % (unsigned)nslab) : 0;
+  auto slab_k0 = [&](int s) {
+    int t = min(s, nslab - 1) + s0;
+    if (t >= nslab) t -= nslab;
+    return t * BK;
+  };
   v4i sta[NJ], stb[NJB];
   // The loads keep their program order (a scheduling barrier that only memory instructions may
   // not cross follows each one): the compiler's vmcnt bookkeeping is exact only if the order in
@@ -116,7 +125,7 @@ __global__ __launch_bounds__(256, BM_ == 128 ? 2 : 1) void gemm_rs_kernel(GemmAr
     __builtin_amdgcn_sched_barrier(NOT_VMEM);
   };
   auto load_slab = [&](int s) {
-    const int k0 = min(s, nslab - 1) * BK;  // slabs past the end re-read the last one (never used)
+    const int k0 = slab_k0(s);
 #pragma unroll
     for (int j = 0; j < (NJ > NJB ? NJ : NJB); ++j) {
       if (j < NJ) load_a(j, k0);
@@ -241,7 +250,6 @@ __global__ __launch_bounds__(256, BM_ == 128 ? 2 : 1) void gemm_rs_kernel(GemmAr
   typedef std::integral_constant<int, 1> C1;
   typedef std::integral_constant<int, NP0> CNP0;
   typedef std::integral_constant<int, NPAIR> CNP;
-  auto slab_k0 = [&](int s) { return min(s, nslab - 1) * BK; };  // slabs past the end: never used
 
   // ---- prologue: slab 0 into LDS; slab 1: pairs [0, NP0) into LDS and their registers re-loaded
   // with slab 2, pairs [NP0, NPAIR) still staged (the first k-step of the loop writes them)

@@ -39,6 +39,7 @@ struct GemmArgs {
   int rows_per_group;  // > 0: every group owns this many rows (batched matmul, split K), offsets unused
   int64_t lda_e;       // uniform groups: bytes between groups in A (rows * lda for stacked batches,
                        // the K slice length when the groups are slices of one reduction)
+  int k_rotate;  // register-staged kernel: block b starts its reduction at slab (b * k_rotate) % slabs
   // optional clock probe (register-staged kernel): block 0 stores {core clock counter, 100 MHz
   // wall clock} at its start, after its K loop and after its epilogue; null = off
   unsigned long long* clk;

@@ -51,6 +51,7 @@ def test_affine_quantizer_strided_input(dev):
 
 
 @pytest.mark.parametrize("shape", [(4, 256, 256, 128), (3, 300, 333, 128), (3, 100, 77, 64), (2, 300, 128, 320),
+                                   (3, 300, 100, 640), (2, 700, 128, 1024),  # tall tiles, staggered reduction
                                    (5, 64, 40, 192), (1, 513, 700, 256)])
 @pytest.mark.parametrize("with_bias", [False, True])
 def test_bmm_i8_exact(dev, shape, with_bias):
@@ -68,7 +69,8 @@ def test_bmm_i8_exact(dev, shape, with_bias):
     torch.testing.assert_close(y.double(), ref, rtol=2e-7, atol=1e-6)
 
 
-@pytest.mark.parametrize("shape", [(4, 256, 256, 128), (3, 300, 333, 128), (3, 100, 77, 64), (2, 130, 128, 384)])
+@pytest.mark.parametrize("shape", [(4, 256, 256, 128), (3, 300, 333, 128), (3, 100, 77, 64), (2, 130, 128, 384),
+                                   (3, 300, 100, 640)])
 def test_bmm_fp8_exact_on_integer_operands(dev, shape):
     B, M, N, Kd = shape
     g = gen(10)
