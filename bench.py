@@ -455,11 +455,14 @@ def extras(torch, K, dev, layers):
                                    "GBps": round(byts / ms / 1e6, 1), "frac_hbm": round(byts / ms / 1e6 / PEAK_HBM_GBS, 4)}
     del pi
     pf = torch.rand(h, sq, sq, device=dev).half()
-    ms = timeit(lambda: K.quant_i8_affine(pf, 1.0 / 127, -64.0, torch.float16), iters=5, warm=2)
+    # the quantizer's scale is a tensor of the compute dtype in the module, i.e. an fp16 value here
+    s_p = float(torch.tensor(1.0 / 127).half())
+    s_v = float(torch.tensor(0.03).half())
+    ms = timeit(lambda: K.quant_i8_affine(pf, s_p, -64.0, torch.float16), iters=5, warm=2)
     byts = h * sq * sq * 3
     res["attn_quant_scores_fp16_S4096"] = {"ms": round(ms, 4), "GBps": round(byts / ms / 1e6, 1), "frac_hbm": round(byts / ms / 1e6 / PEAK_HBM_GBS, 4)}
     vf = torch.randn(h, sq, d, device=dev).half()
-    ms = timeit(lambda: K.quant_i8_affine(vf, 0.03, 0.0, torch.float16, transpose=True), iters=10, warm=3)
+    ms = timeit(lambda: K.quant_i8_affine(vf, s_v, 0.0, torch.float16, transpose=True), iters=10, warm=3)
     byts = h * sq * d * 3
     res["attn_quant_v_transposed_fp16_S4096"] = {"us": round(ms * 1e3, 1), "GBps": round(byts / ms / 1e6, 1), "frac_hbm": round(byts / ms / 1e6 / PEAK_HBM_GBS, 4)}
     return res

@@ -577,9 +577,40 @@ __global__ __launch_bounds__(AQ_THREADS) void quant_i8_mulscale_kernel(
 // q [batch][C][ldq] (q[c][r] = code of x[r][c]) so that an operand stored with its reduction
 // dimension outermost becomes reduction-contiguous for the MFMA kernels.  Columns of q past the
 // data are filled with zeros (they pad the reduction dimension of the matmul).
+// The division by the (scalar) scale without the IEEE sequence where that is exact: the 16-bit
+// quotient of quant_i8_pertoken16_kernel when the scale is itself a value of T, the refined fp32
+// quotient of the fp16-x / fp32-scale kernel when x is fp16; both need a scale of 2^-60 .. 2^60.
+// A quotient that comes out inf or NaN (non-finite x, overflow) is redone with the IEEE division.
+struct AffineDiv {
+  float s, r;
+  bool fast;
+};
+template <int XT, int T>
+__device__ __forceinline__ AffineDiv affine_div(float scale) {
+  AffineDiv d;
+  d.s = scale;
+  const float m = fabsf(scale);
+  d.fast = m >= 8.6736174e-19f && m <= 1.1529215e18f;
+  if constexpr (T == FMSMO_F32) {
+    d.fast = d.fast && XT == FMSMO_F16;
+    d.r = rcp_refined(scale);
+  } else {
+    d.fast = d.fast && XT == T && round_to<T>(scale) == scale;
+    d.r = __builtin_amdgcn_rcpf(scale);
+  }
+  return d;
+}
 template <int T>
-__device__ __forceinline__ float affine_code(float e, float scale, float offset) {
-  const float t = round_to<T>(__fadd_rn(round_to<T>(e / scale), offset));
+__device__ __forceinline__ float affine_code(float e, const AffineDiv& d, float offset) {
+  float q;
+  if (d.fast) {
+    if constexpr (T == FMSMO_F32) q = div32_fast(e, d.s, d.r);
+    else q = div16<T, false>(e, d.s, d.r);
+    if (__builtin_expect(!(fabsf(q) < __builtin_inff()), 0)) q = e / d.s;
+  } else {
+    q = e / d.s;
+  }
+  const float t = round_to<T>(__fadd_rn(round_to<T>(q), offset));
   return fminf(fmaxf(__builtin_rintf(t), -128.0f), 127.0f);
 }
 
@@ -601,6 +632,7 @@ __global__ __launch_bounds__(AQ_THREADS) void quant_i8_affine_kernel(
     int8_t* __restrict__ q, int64_t ldq, int64_t stride_q, int C) {
   const size_t xrow = (size_t)blockIdx.y * stride_x + (size_t)blockIdx.x * ldx;
   uint8_t* qrow = (uint8_t*)q + (size_t)blockIdx.y * stride_q + (size_t)blockIdx.x * ldq;
+  const AffineDiv dv = affine_div<XT, T>(scale);
   for (int c = threadIdx.x * 8; c < (int)ldq; c += AQ_THREADS * 8) {
     uint8_t b[8] = {0, 0, 0, 0, 0, 0, 0, 0};
     if (c < C) {
@@ -608,7 +640,7 @@ __global__ __launch_bounds__(AQ_THREADS) void quant_i8_affine_kernel(
       load8_guard<XT>(x, xrow, c, C, vec, e);
 #pragma unroll
       for (int j = 0; j < 8; ++j)
-        b[j] = (c + j < C) ? (uint8_t)(int)affine_code<T>(e[j], scale, offset) : (uint8_t)0;
+        b[j] = (c + j < C) ? (uint8_t)(int)affine_code<T>(e[j], dv, offset) : (uint8_t)0;
     }
     store8(qrow, (size_t)c, b);
   }
@@ -622,6 +654,7 @@ __global__ __launch_bounds__(256) void quant_i8_affine_t_kernel(
   const int r0 = blockIdx.x * 64, c0 = blockIdx.y * 64;
   const size_t xb = (size_t)blockIdx.z * stride_x;
   const int cl = (threadIdx.x & 7) * 8;
+  const AffineDiv dv = affine_div<XT, T>(scale);
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
     const int rl = (threadIdx.x >> 3) + 32 * i;
@@ -631,7 +664,7 @@ __global__ __launch_bounds__(256) void quant_i8_affine_t_kernel(
 #pragma unroll
     for (int j = 0; j < 8; ++j)
       tile[cl + j][rl] =
-          (r < R && c + j < C) ? (uint8_t)(int)affine_code<T>(e[j], scale, offset) : (uint8_t)0;
+          (r < R && c + j < C) ? (uint8_t)(int)affine_code<T>(e[j], dv, offset) : (uint8_t)0;
   }
   __syncthreads();
   const int oc = threadIdx.x >> 2, chunk = threadIdx.x & 3;

@@ -41,6 +41,28 @@ def test_affine_quantizer_bit_exact(dev, xdt, sdt, shape, transpose):
         assert torch.all(q[..., inner:] == 0)
 
 
+@pytest.mark.parametrize("xdt", [torch.float16, torch.bfloat16])
+def test_affine_quantizer_every_16_bit_pattern(dev, xdt):
+    """The scalar division runs without the IEEE sequence where that is exact (scale a value of
+    the compute dtype, or fp16 x with an fp32 scale): every 16-bit pattern of x except NaN, whose
+    int8 cast is undefined in the reference -- zeros of both signs, subnormals, the largest finite
+    values, both infinities -- against scales from 2^-20 to 600 and two zero points."""
+    bits = torch.arange(65536, dtype=torch.int32).to(torch.int16)
+    x = bits.view(xdt)
+    x = x[~torch.isnan(x)]
+    x = x[: x.numel() // 64 * 64].reshape(1, -1, 64)
+    scales = [0.0371, 1.0, 2.0 ** -20, 600.0, 3.0517578125e-05, 0.3333]
+    for sdt in (xdt, torch.float32):
+        if sdt == torch.float32 and xdt == torch.bfloat16:
+            continue  # promoted to fp32 with bf16 x: plain IEEE path, covered above
+        for sv in scales:
+            scale = torch.tensor([sv], dtype=sdt)
+            for zp in (0, -91):
+                ref = O.qbmm_quant(x, scale, torch.tensor([zp], dtype=torch.int))
+                q = K().quant_i8_affine(x.to(dev), float(scale), float(zp), torch.promote_types(xdt, sdt)).cpu()
+                assert torch.equal(q[..., :64], ref), f"scale {sv} ({sdt}) zp {zp}"
+
+
 def test_affine_quantizer_strided_input(dev):
     """A [b, h, s, d] tensor viewed as K^T ([.., d, s], unit stride along d): the module quantizes
     the untransposed view, a slice along the last dimension takes the scalar path."""
