@@ -444,10 +444,36 @@ __global__ __launch_bounds__(AQ_THREADS) void quant_i8_static_kernel(
   const int row = blockIdx.x;
   const int nchunk = K / AQ_VEC;
   const float inv_scale = 1.0f / scale;
+  // x / scale: the IEEE fp32 sequence is r1 = refined rcp, q = x r1, two residual corrections,
+  // wrapped in range scaling and a special-case fix-up.  Without the wrapping the same operations
+  // give the same quotient whenever no intermediate leaves the normal range: |scale| within
+  // 2^-20 .. 2^20 and x zero or within 2^-100 .. 2^100 (always, for fp16 x) with a finite result.
+  const float r1 = rcp_refined(scale);
+  const bool fast = fabsf(scale) >= 9.5367431640625e-07f && fabsf(scale) <= 1048576.0f;
   for (int c = threadIdx.x; c < nchunk; c += AQ_THREADS) {
     float e[8];
     load8<XT>(x, (size_t)row * ldx + (size_t)c * AQ_VEC, e);
     uint8_t b[8];
+    float qv[8];
+    if (!pt_native) {
+      bool ok = fast;
+      if (fast) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          qv[j] = div32_fast(e[j], scale, r1);
+          ok = ok && fabsf(qv[j]) < __builtin_inff();
+          if constexpr (XT != FMSMO_F16) {
+            // |x| in [2^-100, 2^100): one unsigned compare on the exponent field
+            const uint32_t mag = __float_as_uint(e[j]) & 0x7fffffffu;
+            ok = ok && (mag == 0u || mag - 0x0d800000u < 0x64000000u);
+          }
+        }
+      }
+      if (__builtin_expect(!ok, 0)) {  // one rarely taken branch per 8 elements
+#pragma unroll
+        for (int j = 0; j < 8; ++j) qv[j] = e[j] / scale;
+      }
+    }
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       // ((x/s + zp) - 128) + sym, each step rounded to fp32, then round-half-even and clamp
@@ -455,7 +481,7 @@ __global__ __launch_bounds__(AQ_THREADS) void quant_i8_static_kernel(
       if (pt_native)  // torch.quantize_per_tensor: rint(x * (1/scale)) + zero_point
         t = __builtin_rintf(__fmul_rn(e[j], inv_scale)) + (zp - 128.0f + sym);
       else
-        t = __builtin_rintf(__fadd_rn(__fadd_rn(__fadd_rn(e[j] / scale, zp), -128.0f), sym));
+        t = __builtin_rintf(__fadd_rn(__fadd_rn(__fadd_rn(qv[j], zp), -128.0f), sym));
       t = fminf(fmaxf(t, -128.0f), 127.0f);
       b[j] = (uint8_t)(int)t;
     }

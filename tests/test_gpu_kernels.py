@@ -174,6 +174,29 @@ def test_quant_act_i8_static(dev):
         assert torch.equal(q.cpu(), q_ref)
 
 
+@pytest.mark.parametrize("xdt", [torch.float16, torch.bfloat16, torch.float32])
+def test_quant_act_i8_static_every_pattern_and_range(dev, xdt):
+    """x / scale runs without the range scaling and fix-up of the IEEE sequence where the plain
+    operations give the same quotient; outside that range, and for non-finite x, it falls back.
+    Every 16-bit pattern except NaN (fp32: random values over the whole exponent range, zeros and
+    infinities), scales inside and outside the fast range."""
+    if xdt == torch.float32:
+        g = gen(77)
+        mant = torch.rand(65536, generator=g) + 1.0
+        expo = torch.randint(-140, 128, (65536,), generator=g).float()
+        x = mant * torch.exp2(expo) * torch.where(torch.rand(65536, generator=g) < 0.5, -1.0, 1.0)
+        x[:4] = torch.tensor([0.0, -0.0, float("inf"), float("-inf")])
+    else:
+        x = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(xdt)
+        x = x[~torch.isnan(x)]
+    x = x[: x.numel() // 64 * 64].reshape(-1, 64)
+    for scale in (0.0371, 1.0, 2.0 ** -19, 2.0 ** -30, 3.0e5, 7.0e7, 1.1e-3):
+        for zp, sym in ((128, 1), (117, 0)):
+            q_ref = O.quant_act_static_raw(x, torch.tensor([scale]), zp, sym)
+            q = K().quant_act_i8_static(x.to(dev), scale, zp, sym)
+            assert torch.equal(q.cpu(), q_ref), f"scale {scale} zp {zp} sym {sym}"
+
+
 # ------------------------------------------------------------------------------ act quant fp8
 def test_fp8_cast_all_codes_and_midpoints(dev):
     codes = torch.arange(256, dtype=torch.uint8).view(torch.float8_e4m3fn).float()
