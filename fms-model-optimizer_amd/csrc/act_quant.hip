@@ -301,7 +301,11 @@ __device__ __forceinline__ float div32_fast_mix(float x, float s, float r1, floa
   return q;
 }
 
-template <int NCH, bool KEEP, int TH = AQ_THREADS>
+// bf16 x (XT = FMSMO_BF16) reaches below fp16's range: a row whose maximum quotient is under
+// 2^-80 (and not zero) also takes the IEEE division, because the residuals of its corrections
+// could fall below the smallest fp32 subnormal; elements that small inside an ordinary row
+// quantize to zero whichever way their last bit is rounded.
+template <int NCH, bool KEEP, int TH = AQ_THREADS, int XT = FMSMO_F16>
 __global__ __launch_bounds__(TH) void quant_i8_pertoken_f16x_f32s_kernel(
     const u16* __restrict__ x, int64_t ldx, const float* __restrict__ smooth, int saturate,
     int8_t* __restrict__ q, int64_t ldq, float* __restrict__ scale, int M, int K) {
@@ -360,7 +364,7 @@ __global__ __launch_bounds__(TH) void quant_i8_pertoken_f16x_f32s_kernel(
         }
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-          const float xv = f16_to_f32((u16)((uint32_t)cur[i][j >> 1] >> ((j & 1) * 16)));
+          const float xv = cvt16<XT>((u16)((uint32_t)cur[i][j >> 1] >> ((j & 1) * 16)));
           if constexpr (IEEE) e[i][j] = xv / d[j];
           else if constexpr (KEEP) e[i][j] = div32_fast_mix(xv, sv[i][j], sr[i][j], nz);
           else e[i][j] = div32_fast_mix(xv, d[j], rcp_refined(d[j]), nz);
@@ -396,6 +400,7 @@ __global__ __launch_bounds__(TH) void quant_i8_pertoken_f16x_f32s_kernel(
     if (!ieee) {
       amax = block_amax(divide_row(std::false_type{}));
       ieee = !(amax < __builtin_inff());  // inf or NaN somewhere in the row
+      if constexpr (XT == FMSMO_BF16) ieee = ieee || (amax != 0.0f && amax < 8.271806e-25f);
     }
     if (ieee) {
       // fmaxf drops NaN like the generic kernel does
@@ -954,18 +959,27 @@ extern "C" int fmsmo_quant_act_i8_pertoken(const void* x, int x_dtype, int64_t l
 #undef LAUNCH16
     return fmsmo_check_launch();
   }
-  // fp16 x promoted to fp32 by an fp32 SmoothQuant scale
-  if (x_dtype == FMSMO_F16 && smooth && smooth_dtype == FMSMO_F32 && compute_dtype == FMSMO_F32 &&
+  // fp16 / bf16 x promoted to fp32 by an fp32 SmoothQuant scale
+  if (x_dtype != FMSMO_F32 && smooth && smooth_dtype == FMSMO_F32 && compute_dtype == FMSMO_F32 &&
       K <= AQ_MAXCHUNK * AQ_THREADS * AQ_VEC) {
     const int64_t per_thread = div_up(K, AQ_THREADS * AQ_VEC);
 #define LAUNCH32(NCH, KEEP, TH)                                                                   \
   {                                                                                               \
-    const int64_t resident =                                                                      \
-        resident_blocks((const void*)quant_i8_pertoken_f16x_f32s_kernel<NCH, KEEP, TH>, TH);      \
-    dim3 grid32((unsigned)(M < resident ? M : resident)), block32(TH);                            \
-    hipLaunchKernelGGL((quant_i8_pertoken_f16x_f32s_kernel<NCH, KEEP, TH>), grid32, block32, 0,   \
-                       st, (const u16*)x, ldx, (const float*)smooth, saturate, q, ldq, scale,     \
-                       (int)M, (int)K);                                                           \
+    if (x_dtype == FMSMO_F16) {                                                                   \
+      const int64_t resident =                                                                    \
+          resident_blocks((const void*)quant_i8_pertoken_f16x_f32s_kernel<NCH, KEEP, TH>, TH);    \
+      dim3 grid32((unsigned)(M < resident ? M : resident)), block32(TH);                          \
+      hipLaunchKernelGGL((quant_i8_pertoken_f16x_f32s_kernel<NCH, KEEP, TH>), grid32, block32, 0, \
+                         st, (const u16*)x, ldx, (const float*)smooth, saturate, q, ldq, scale,   \
+                         (int)M, (int)K);                                                         \
+    } else {                                                                                      \
+      const int64_t resident = resident_blocks(                                                   \
+          (const void*)quant_i8_pertoken_f16x_f32s_kernel<NCH, KEEP, TH, FMSMO_BF16>, TH);        \
+      dim3 grid32((unsigned)(M < resident ? M : resident)), block32(TH);                          \
+      hipLaunchKernelGGL((quant_i8_pertoken_f16x_f32s_kernel<NCH, KEEP, TH, FMSMO_BF16>), grid32, \
+                         block32, 0, st, (const u16*)x, ldx, (const float*)smooth, saturate, q,   \
+                         ldq, scale, (int)M, (int)K);                                             \
+    }                                                                                             \
   }
     if (per_thread <= 1) LAUNCH32(1, true, 256)
     else if (per_thread <= 2) LAUNCH32(2, true, 256)

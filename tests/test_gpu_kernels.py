@@ -147,6 +147,34 @@ def test_quant_act_i8_fp16_x_fp32_smooth_rows(dev, shape):
         assert torch.equal(q.cpu()[ok], q_ref[ok]), variant
 
 
+@pytest.mark.parametrize("shape", [(2500, 4096), (300, 6144), (530, 14336)])
+def test_quant_act_i8_bf16_x_fp32_smooth_rows(dev, shape):
+    """bf16 x with an fp32 SmoothQuant scale (a bf16 model with fp32 quantizer buffers): fp32
+    arithmetic as above, plus what bf16's range adds -- rows of tiny values (maximum below 2^-80:
+    IEEE path), tiny and huge elements inside ordinary rows, rows that overflow."""
+    M, Kd = shape
+    g = gen(13)
+    x = ((torch.rand(M, Kd, generator=g) * 3 + 0.01) * torch.sign(torch.randn(M, Kd, generator=g))).bfloat16()
+    x = _special_rows(x)
+    x[5, 3] = 3.0e38                                   # overflows after the divide: scale inf
+    x[6] = (x[6].float() * 1e-30).bfloat16()           # whole row tiny: maximum ~3e-30 < 2^-80
+    x[7] = (x[7].float() * 2.0 ** -110).bfloat16()     # and deeper still
+    x[8, ::5] = (x[8, ::5].float() * 1e-36).bfloat16() # tiny elements in an ordinary row
+    x[9, 11] = 1.0e30                                  # one huge, finite element
+    base = torch.rand(Kd, generator=g) * 1.5 + 0.5
+    for variant in ("plain", "tiny_divisor", "huge_divisor"):
+        smooth = base.clone()
+        if variant == "tiny_divisor":
+            smooth[7] = 1e-30
+        if variant == "huge_divisor":
+            smooth[9] = 3e30
+        q_ref, s_ref, _ = O.quant_act_pertoken_i8(x, smooth.reshape(1, -1))
+        q, s = K().quant_act_i8_pertoken(x.to(dev), smooth.to(dev))
+        ok = torch.isfinite(s_ref.float().reshape(-1))
+        assert torch.equal(s.cpu()[ok], s_ref.float().reshape(-1)[ok]), variant
+        assert torch.equal(q.cpu()[ok], q_ref[ok]), variant
+
+
 def test_quant_act_i8_fp16_division_ties_and_subnormals(dev):
     """Every finite fp16 bit pattern as x against divisors that make exact ties (powers of two on
     subnormal quotients), tiny and huge quotients: x / smooth must round like torch's fp16
