@@ -283,36 +283,49 @@ def extras(torch, K, dev, layers):
     for name, k, n in LLAMA3_8B:
         wbytes = k * n
         copies = max(3, (300 * 1024 * 1024 + wbytes - 1) // wbytes)
-        ws_i8 = [torch.randint(-127, 128, (n, k), dtype=torch.int8, device=dev) for _ in range(copies)]
         wsc = torch.rand(n, device=dev) * 1e-3
-        for M in (1, 4, 16, 32, 64, 128):  # decode kernels up to 64 (K <= 4096), tiled / split-K above
-            x = torch.randn(M, k, device=dev).bfloat16()
-            q, s = K.quant_act_i8_pertoken(x)
-            side = torch.cuda.Stream()
-            reps, replays = 3, 5
-            with torch.cuda.stream(side):
-                for w in ws_i8:
-                    K.gemm_i8_dq(q, w, s, wsc, None, out_dtype=torch.bfloat16, exact_ref=True)
-                torch.cuda.synchronize()
-                graph = torch.cuda.CUDAGraph()
-                with torch.cuda.graph(graph, stream=side):
-                    for _ in range(reps):
-                        for w in ws_i8:
-                            K.gemm_i8_dq(q, w, s, wsc, None, out_dtype=torch.bfloat16, exact_ref=True)
-                graph.replay()
-                torch.cuda.synchronize()
-                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                e0.record()
-                for _ in range(replays):
+        for op in ("i8", "fp8"):
+            if op == "i8":
+                ws_q = [torch.randint(-127, 128, (n, k), dtype=torch.int8, device=dev) for _ in range(copies)]
+                m_list = (1, 4, 16, 32, 64, 128)  # decode kernels up to 64 (K <= 4096), tiled / split-K above
+            else:  # e4m3 weights whose codes cover the format's range (per-channel-scaled Gaussian)
+                ws_q = [torch.randn(n, k, device=dev).mul_(448.0 / 4.5).clamp_(-448, 448).to(torch.float8_e4m3fn)
+                        for _ in range(copies)]
+                m_list = (1, 4, 16)
+            for M in m_list:
+                x = torch.randn(M, k, device=dev).bfloat16()
+                if op == "i8":
+                    q, s = K.quant_act_i8_pertoken(x)
+                    run = lambda w: K.gemm_i8_dq(q, w, s, wsc, None, out_dtype=torch.bfloat16, exact_ref=True)  # noqa: E731
+                else:
+                    q, s = K.quant_act_fp8_pertoken(x, L.FP8_LINEAR)
+                    run = lambda w: K.gemm_fp8_dq(q, w, s, wsc, None, out_dtype=torch.bfloat16)  # noqa: E731
+                side = torch.cuda.Stream()
+                reps, replays = 3, 5
+                with torch.cuda.stream(side):
+                    for w in ws_q:
+                        run(w)
+                    torch.cuda.synchronize()
+                    graph = torch.cuda.CUDAGraph()
+                    with torch.cuda.graph(graph, stream=side):
+                        for _ in range(reps):
+                            for w in ws_q:
+                                run(w)
                     graph.replay()
-                e1.record()
-                torch.cuda.synchronize()
-            ms = e0.elapsed_time(e1) / (replays * reps * copies)
-            byts = wbytes + M * k + M * n * 2 + 4 * n
-            gbs = byts / (ms * 1e-3) / 1e9
-            res[f"decode_i8_M{M}_{name}"] = {"us": round(ms * 1e3, 2), "GBps": round(gbs, 1), "frac_hbm": round(gbs / PEAK_HBM_GBS, 4)}
-            del graph
-        del ws_i8
+                    torch.cuda.synchronize()
+                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    e0.record()
+                    for _ in range(replays):
+                        graph.replay()
+                    e1.record()
+                    torch.cuda.synchronize()
+                ms = e0.elapsed_time(e1) / (replays * reps * copies)
+                byts = wbytes + M * k + M * n * 2 + 4 * n
+                gbs = byts / (ms * 1e-3) / 1e9
+                res[f"decode_{op}_M{M}_{name}"] = {"us": round(ms * 1e3, 2), "GBps": round(gbs, 1),
+                                                  "frac_hbm": round(gbs / PEAK_HBM_GBS, 4)}
+                del graph
+            del ws_q
     # the four int8 GEMMs of the headline workload on all-zero operands: nothing toggles in the
     # multipliers, the clock stays up, and the figure shows how far the kernel's instruction
     # stream goes when the power limit does not hold it back

@@ -525,6 +525,25 @@ __global__ __launch_bounds__(256) void gemv_rows_kernel(GemvArgs g) {
     }
   }
 
+  // e4m3: every code is an fp16 value and a product of two fp16 values is exact in fp32, so the
+  // codes are widened two at a time to packed fp16 and multiplied by v_dot2_f32_f16 (fp32
+  // accumulation): 6 vector instructions per 4 weight bytes, 4 where the activation chunks are
+  // kept widened (XH: at most 64 registers), against 8 for conversions to fp32 and FMAs.
+  constexpr bool XH = OP != FMSMO_OP_I8 && MR * KCH <= 8;
+  typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+  h2 xh[XH ? MR : 1][XH ? KCH : 1][8];
+  if constexpr (XH) {
+#pragma unroll
+    for (int m = 0; m < MR; ++m)
+#pragma unroll
+      for (int c = 0; c < KCH; ++c)
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+          xh[m][c][2 * d] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(xr[m][c][d], 1.0f, false);
+          xh[m][c][2 * d + 1] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(xr[m][c][d], 1.0f, true);
+        }
+  }
+
   for (int n0 = wave_g * U; n0 < g.N; n0 += nwaves * U) {
     if (!FUSED || n0 != wave_g * U) load_w(n0, w);
     AccT acc[U][MR];
@@ -540,14 +559,18 @@ __global__ __launch_bounds__(256) void gemv_rows_kernel(GemvArgs g) {
             if constexpr (OP == FMSMO_OP_I8) {
               a = __builtin_amdgcn_sdot4(w[u][c][d], xr[m][c][d], a, false);
             } else {
-              const auto w0 = __builtin_amdgcn_cvt_pk_f32_fp8(w[u][c][d], false);
-              const auto w1 = __builtin_amdgcn_cvt_pk_f32_fp8(w[u][c][d], true);
-              const auto x0 = __builtin_amdgcn_cvt_pk_f32_fp8(xr[m][c][d], false);
-              const auto x1 = __builtin_amdgcn_cvt_pk_f32_fp8(xr[m][c][d], true);
-              a = __builtin_fmaf(w0[0], x0[0], a);
-              a = __builtin_fmaf(w0[1], x0[1], a);
-              a = __builtin_fmaf(w1[0], x1[0], a);
-              a = __builtin_fmaf(w1[1], x1[1], a);
+              const h2 w0 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w[u][c][d], 1.0f, false);
+              const h2 w1 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w[u][c][d], 1.0f, true);
+              h2 x0, x1;
+              if constexpr (XH) {
+                x0 = xh[m][c][2 * d];
+                x1 = xh[m][c][2 * d + 1];
+              } else {
+                x0 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(xr[m][c][d], 1.0f, false);
+                x1 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(xr[m][c][d], 1.0f, true);
+              }
+              a = __builtin_amdgcn_fdot2(w0, x0, a, false);
+              a = __builtin_amdgcn_fdot2(w1, x1, a, false);
             }
           }
         }
@@ -653,7 +676,10 @@ int fmsmo_gemv_dispatch(int op, const void* a, int64_t lda, const void* b, int64
     static const int env_kind = getenv("FMSMO_GEMV_KIND") ? atoi(getenv("FMSMO_GEMV_KIND")) : 0;
     const int kch = (int)((K + 1023) / 1024);
     const int mr = M <= 1 ? 1 : 2;
-    bool handled = env_kind != 1 && M <= 2 && K >= 1024;
+    // two e4m3 tokens double the widening work per weight byte and the MFMA streaming kernel is
+    // faster on every shape measured (us, rows -> streaming: qkv 7.7 -> 6.9, o 6.2 -> 5.9,
+    // gate+up 23.7 -> 20.9, down 22.3 -> 19.2 and less with the activations in LDS)
+    bool handled = env_kind != 1 && M <= 2 && K >= 1024 && !(op != FMSMO_OP_I8 && M == 2);
     if (handled) {
       // 16 waves per CU resident (register use allows it), rows dealt round-robin to waves
       const int64_t waves_needed = N;  // at U = 1
@@ -710,9 +736,10 @@ int fmsmo_gemv_dispatch(int op, const void* a, int64_t lda, const void* b, int64
     if (G > 64) G = 64;
     dim3 grid((unsigned)((groups + G - 1) / G)), block(NW * 64);
     bool handled = true;
-    // K = 14336 with 3 .. 8 tokens: activations in LDS, all 14 steps of loads in flight
+    // K = 14336 with at most 8 tokens (one or two int8 tokens went to the row kernel above):
+    // activations in LDS, all 14 steps of loads in flight
     // (N = 4096, us at M = 3 / 4 / 8: 15.8 -> 15.0, 15.9 -> 14.7, 17.0 -> 15.4)
-    if (M >= 3 && M <= 8 && NW == 8 && STEPS == 14) {
+    if (M <= 8 && NW == 8 && STEPS == 14) {
       if (op == FMSMO_OP_I8)
         hipLaunchKernelGGL((gemv_stream_kernel<FMSMO_OP_I8, 14, 8, 14, 1, 8>), grid, block, 0, st, g, G);
       else

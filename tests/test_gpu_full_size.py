@@ -98,7 +98,7 @@ def test_decode_shapes_full_size_equal_exact_product(dev, name, Kd, N, M):
 
 
 @pytest.mark.parametrize("name,Kd,N", LLAMA)
-@pytest.mark.parametrize("M", [1, 4, 16])
+@pytest.mark.parametrize("M", [1, 2, 4, 16])
 def test_decode_shapes_full_size_fp8(dev, name, Kd, N, M):
     """Config 3, fp8: e4m3 operands with small-integer values make every product and partial sum
     exact in fp32, so any summation order must give the same result; random operands are held
