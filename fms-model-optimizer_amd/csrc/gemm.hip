@@ -133,9 +133,9 @@ extern "C" int fmsmo_gemm_plan(int64_t M, int64_t N, int64_t K, int with_workspa
     return FMSMO_OK;
   }
   const bool rs = K % 128 == 0 && use_register_staged(MMA_I8);
-  const int bm[4] = {256, 128, 128, 256}, bn[4] = {256, 256, 128, 192};
+  const int bm[5] = {256, 128, 128, 256, 256}, bn[5] = {256, 256, 128, 192, 128};
   const int t = pick_tile((int)M, (int)N, rs);
-  *kernel = (rs && (t == 0 || t == 3)) ? FMSMO_PLAN_TILE_REGISTER_STAGED : FMSMO_PLAN_TILE_LDS_DMA;
+  *kernel = (rs && (t == 0 || t >= 3)) ? FMSMO_PLAN_TILE_REGISTER_STAGED : FMSMO_PLAN_TILE_LDS_DMA;
   *tile_m = bm[t];
   *tile_n = (t == 3 && !rs) ? 256 : bn[t];
   return FMSMO_OK;

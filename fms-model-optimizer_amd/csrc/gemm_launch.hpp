@@ -46,17 +46,22 @@ struct TileMid { static constexpr int BM = 128, BN = 128, BK = 64, NST = 4, WGM 
 // (bigger tiles move fewer bytes per MFMA); 128x128 tiles fit two blocks per CU.  Shape 3 is the
 // register-staged kernel with 256x192 tiles (K % 128 == 0 only): 8 % slower per operation than
 // 256x256, but e.g. N = 6144 at M = 4096 then makes 512 tiles, two full rounds, instead of 384.
+// Shape 4 is the same kernel with 256x128 tiles (the tile of the probabilities x values batched
+// matmul): 0.85 of the 256x256 rate where both fill their rounds (4096 x 4096 x 4096: 73 -> 85 us),
+// but 2048 rows x 4096 columns make 256 tiles instead of 128 (us, int8 / e4m3: K = 4096 45.8 ->
+// 43.4 / 42.2 -> 38.7, K = 12800 141 -> 123 / 130 -> 114).
+constexpr double EFF_RS128 = 0.85;
 int pick_tile(int M, int N, bool rs192_ok) {
-  static const char* force = getenv("FMSMO_TILE");  // tuning aid: 0 = 256x256, 1 = 128x256, 2 = 128x128, 3 = 256x192
-  if (force && force[0] >= '0' && force[0] <= '3') return force[0] - '0';
+  static const char* force = getenv("FMSMO_TILE");  // tuning aid: 0 = 256x256, 1 = 128x256, 2 = 128x128, 3 = 256x192, 4 = 256x128
+  if (force && force[0] >= '0' && force[0] <= '4') return (force[0] == '4' && !rs192_ok) ? 2 : force[0] - '0';
   // Fitted to measurements on the Llama / Granite shapes: relative loop efficiency of the three
   // tile shapes, and a sub-linear penalty for a partially filled last round (idle CUs leave
   // power, hence clock, to the busy ones).
-  const double eff[4] = {1.0, 0.76, 0.70, 0.92};
-  const int bm[4] = {256, 128, 128, 256}, bn[4] = {256, 256, 128, 192};
+  const double eff[5] = {1.0, 0.76, 0.70, 0.92, EFF_RS128};
+  const int bm[5] = {256, 128, 128, 256, 256}, bn[5] = {256, 256, 128, 192, 128};
   int best = 0;
   double best_score = -1;
-  for (int t = 0; t < (rs192_ok ? 4 : 3); ++t) {
+  for (int t = 0; t < (rs192_ok ? 5 : 3); ++t) {
     const long tiles = (long)div_up(M, bm[t]) * div_up(N, bn[t]);
     const long slots = (t == 2 && tiles > 256) ? 512 : 256;  // two 128x128 blocks fit per CU
     const long rounds = (tiles + slots - 1) / slots;
@@ -141,6 +146,7 @@ void launch_any(const GemmArgs& g, const Epi& epi, hipStream_t st) {
         if (g.K % 128 == 0 && use_register_staged(OP)) launch_rs<OP, false, 192>(g, epi, st);
         else launch_tile<TileBig, OP, false>(g, epi, st);
         break;
+      case 4: launch_rs<OP, false, 128>(g, epi, st); break;  // only offered when K % 128 == 0
       default: launch_tile<TileMid, OP, false>(g, epi, st); break;
     }
   } else {

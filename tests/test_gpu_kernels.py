@@ -347,9 +347,9 @@ def test_gemm_i8_i32_random_shapes_cover_every_kernel_choice(dev):
         c = K().gemm_i8_i32(a, w)
         ref = (a.double() @ w.double().t()).to(torch.int32)
         assert torch.equal(c, ref), f"M={M} N={N} K={Kd} plan={plan}"
-    # the sample reaches the generic kernel, both MFMA pipelines and all four tile shapes
+    # the sample reaches the generic kernel, both MFMA pipelines and all five tile shapes
     assert {p[0] for p in seen} >= {1, 2, 3}
-    assert {p[1:] for p in seen if p[0] in (1, 2)} >= {(256, 256), (256, 192), (128, 256), (128, 128)}
+    assert {p[1:] for p in seen if p[0] in (1, 2)} >= {(256, 256), (256, 192), (256, 128), (128, 256), (128, 128)}
 
 
 def test_gemm_i8_i32_strided_rows(dev):
@@ -365,7 +365,8 @@ def test_gemm_i8_i32_strided_rows(dev):
 
 @pytest.mark.parametrize("out_dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("shape", [(512, 4096, 4096), (300, 520, 1024), (16, 512, 1024), (1, 256, 128),
-                                   (2048, 6100, 256)])  # 256x192 tiles, ragged last column tile
+                                   (2048, 6100, 256),   # 256x192 tiles, ragged last column tile
+                                   (2000, 4090, 384)])  # 256x128 tiles, ragged last row and column tiles
 def test_gemm_i8_dq_reference_epilogue_bit_exact(dev, shape, out_dtype):
     M, N, Kd = shape
     a, w = _rand_i8((M, Kd), 21), _rand_i8((N, Kd), 22)

@@ -124,6 +124,12 @@ def test_gemm_plan_is_host_logic():
     assert K.gemm_plan(4096, 4096, 4096) == (RS, 256, 256, 1)     # 256 tiles = 1 round
     assert K.gemm_plan(4096, 28672, 4096) == (RS, 256, 256, 1)    # 1792 tiles = 7 rounds
     assert K.gemm_plan(4096, 4096, 14336) == (RS, 256, 256, 1)
+    # Granite-3-8B linears with 4096 output columns at 2048 tokens: 256 x 256 tiles would fill half
+    # the compute units, 256 x 128 tiles of the same pipeline fill them all
+    assert K.gemm_plan(2048, 4096, 4096) == (RS, 256, 128, 1)
+    assert K.gemm_plan(2048, 4096, 12800) == (RS, 256, 128, 1)
+    assert K.gemm_plan(2048, 6144, 4096) == (RS, 256, 192, 1)
+    assert K.gemm_plan(2048, 25600, 4096) == (RS, 256, 256, 1)
     # decode and batched decode
     assert K.gemm_plan(1, 4096, 4096)[0] == _lib.PLAN_DECODE
     assert K.gemm_plan(16, 28672, 4096)[0] == _lib.PLAN_DECODE
