@@ -291,20 +291,21 @@ __global__ __launch_bounds__(NW * 64) void gemv_kernel(GemvArgs g) {
 // MT > 1: batches of up to 16 MT tokens.  The weight stream is the same; every step feeds MT
 // MFMAs (one per tile of 16 tokens) from the same weight fragment, so up to 64 tokens cost little
 // more than 16 as long as their activation fragments fit in registers (MT * STEPS * 8 VGPRs).
-// XL > 0: long rows with at most XL tokens.  The activation rows live in LDS (XL rows of K + 32
-// bytes: the pad puts the rows 8 banks apart) instead of STEPS * 8 registers per lane, which makes
-// room to keep every load of the wave's K slice in flight at once (D = STEPS).
-template <int OP, int STEPS, int NW, int D, int MT = 1, int XL = 0>
+// D steps of weight loads are in flight per wave.  Long rows want a shallow pipeline: the
+// activation fragments of K = 14336 take 112 registers per lane, and with 7 of the 14 steps in
+// flight the kernel spilled (12 / 32 registers for int8 / e4m3 at the 256-register limit); D = 2
+// fits and is faster at every token count (us at N = 4096, 16 tokens: int8 18.9 -> 15.4, e4m3
+// 23.5 -> 16.1; 4 tokens 15.8 -> 12.5; K = 12800 as 10 waves x 10 steps, D = 5 -> 2: 20.1 ->
+// 11.3 at 4 tokens), also than keeping the activations in LDS with all 14 steps in flight (4
+// tokens: 14.6).
+template <int OP, int STEPS, int NW, int D, int MT = 1>
 __global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(GemvArgs g, int G) {
   static_assert(STEPS % D == 0, "pipeline depth must divide the steps per group");
-  static_assert(XL == 0 || MT == 1, "activations in LDS: one tile of tokens");
   typedef typename std::conditional<OP == FMSMO_OP_I8, int, float>::type AccT;
   typedef AccT Acc4 __attribute__((ext_vector_type(4)));
-  constexpr int XPITCH = 128 * STEPS * NW + 32;
-  constexpr int NRED = XL ? 1 : 2;  // exchange buffers (one and a second barrier when LDS is short)
+  constexpr int NRED = 2;  // exchange buffers alternate, one barrier per group
   __shared__ __attribute__((aligned(16))) uint8_t stage[NW][2][2048];
   __shared__ AccT red[NRED][NW][256 * MT];
-  __shared__ __attribute__((aligned(16))) uint8_t xs[XL ? XL * XPITCH : 16];
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int r = lane & 15, kg = lane >> 4;
@@ -314,19 +315,8 @@ __global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(GemvArgs g, int G)
   const int kwave = wave * (STEPS * 128);
 
   // activation fragments: lane (m = r, kg) holds x[m][kwave + s*128 + (h*4 + kg)*16 ...]
-  v4i xf[XL ? 1 : MT][XL ? 1 : STEPS][2];
-  // XL: the block's copy of x, 16-byte chunks dealt round-robin to the threads; fetched before
-  // the weights so that it arrives first (loads complete in order)
-  constexpr int XCH = 8 * STEPS * NW;                                  // chunks per row
-  constexpr int XPT = XL ? (XL * XCH + NW * 64 - 1) / (NW * 64) : 1;  // chunks per thread
-  v4i xcp[XPT];
-  if constexpr (XL) {
-#pragma unroll
-    for (int i = 0; i < XPT; ++i) {
-      const int c = min((int)threadIdx.x + i * NW * 64, g.M * XCH - 1);
-      xcp[i] = *(const v4i*)(g.a + (int64_t)(c / XCH) * g.lda + (c % XCH) * 16);
-    }
-  } else {
+  v4i xf[MT][STEPS][2];
+  {
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
       const uint8_t* xp = g.a + (int64_t)min(t * 16 + r, g.M - 1) * g.lda + kwave + kg * 16;
@@ -360,15 +350,6 @@ __global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(GemvArgs g, int G)
   v4i wb[D][2];
 #pragma unroll
   for (int j = 0; j < D; ++j) load_item(false, j, wb[j]);
-  const int xrd = min(r, g.M - 1) * XPITCH + kwave + kg * 16;
-  if constexpr (XL) {
-#pragma unroll
-    for (int i = 0; i < XPT; ++i) {
-      const int c = (int)threadIdx.x + i * NW * 64;
-      if (c < g.M * XCH) *(v4i*)(xs + (c / XCH) * XPITCH + (c % XCH) * 16) = xcp[i];
-    }
-    __syncthreads();
-  }
 
   // epilogue operands of output element e = threadIdx.x (n = e / 16, m = e % 16 of the group) are
   // fetched at the top of each group so that their latency hides behind the weight stream
@@ -402,13 +383,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(GemvArgs g, int G)
       const v4i w1 = *(const v4i*)(st + rd1);
 #pragma unroll
       for (int t = 0; t < MT; ++t) {
-        v4i x0, x1;
-        if constexpr (XL) {
-          x0 = *(const v4i*)(xs + xrd + s * 128);
-          x1 = *(const v4i*)(xs + xrd + s * 128 + 64);
-        } else {
-          x0 = xf[t][s][0], x1 = xf[t][s][1];
-        }
+        const v4i x0 = xf[t][s][0], x1 = xf[t][s][1];
         if constexpr (OP == FMSMO_OP_I8) {
           acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w0, x0, acc[t], 0, 0, 0);
           acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w1, x1, acc[t], 0, 0, 0);
@@ -462,7 +437,6 @@ __global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(GemvArgs g, int G)
         finish(e, g.a_scale[g.a_stride ? m : 0], ws, bv);
       }
     }
-    if constexpr (NRED == 1 && !LAST) __syncthreads();  // the next group reuses the exchange buffer
   };
   for (int gi = 0; gi + 1 < gcount; ++gi) do_group(std::false_type{}, gi);
   do_group(std::true_type{}, gcount - 1);
@@ -676,10 +650,18 @@ int fmsmo_gemv_dispatch(int op, const void* a, int64_t lda, const void* b, int64
     static const int env_kind = getenv("FMSMO_GEMV_KIND") ? atoi(getenv("FMSMO_GEMV_KIND")) : 0;
     const int kch = (int)((K + 1023) / 1024);
     const int mr = M <= 1 ? 1 : 2;
-    // two e4m3 tokens double the widening work per weight byte and the MFMA streaming kernel is
-    // faster on every shape measured (us, rows -> streaming: qkv 7.7 -> 6.9, o 6.2 -> 5.9,
-    // gate+up 23.7 -> 20.9, down 22.3 -> 19.2 and less with the activations in LDS)
-    bool handled = env_kind != 1 && M <= 2 && K >= 1024 && !(op != FMSMO_OP_I8 && M == 2);
+    // Where the MFMA streaming kernel below has an instantiation for K it is the faster one for
+    // two e4m3 tokens (twice the widening work per weight byte; us at N = 4096, rows -> streaming:
+    // K = 4096 6.2 -> 5.4, 14336 22.3 -> 12.6), for two int8 tokens from K = 8192 (7.9 -> 7.4;
+    // 14336: 13.7 -> 12.1; 5120: 5.7 against 5.9), for one e4m3 token from K = 12800 (12.6 ->
+    // 11.2; 8192: 7.9 both) and for one int8 token at K = 12800 (11.4 -> 10.8; 14336: 11.8 both,
+    // 16384: 13.0 against 13.8).
+    const int steps128 = K % 128 ? 0 : (int)(K / 128);
+    const bool stream_ok = steps128 == 8 || steps128 == 16 || steps128 == 32 || steps128 == 40 ||
+                           steps128 == 64 || steps128 == 100 || steps128 == 112 || steps128 == 128;
+    const bool prefer_stream =
+        stream_ok && (op == FMSMO_OP_I8 ? (M == 2 ? kch >= 8 : kch == 13) : (M == 2 || kch >= 11));
+    bool handled = env_kind != 1 && M <= 2 && K >= 1024 && !prefer_stream;
     if (handled) {
       // 16 waves per CU resident (register use allows it), rows dealt round-robin to waves
       const int64_t waves_needed = N;  // at U = 1
@@ -728,24 +710,12 @@ int fmsmo_gemv_dispatch(int op, const void* a, int64_t lda, const void* b, int64
     else if (steps_total % 10 == 0) NW = 10;
     // K = 4096 and at most 16 tokens: 16 waves of 2 steps each instead of 8 of 4 (us at M = 4 / 16:
     // o 5.8 -> 5.5 / 6.6 -> 6.0, qkv 7.0 -> 7.0 / 8.2 -> 7.7, gate+up 21.8 -> 20.9 / 22.8 -> 21.8).
-    // K = 14336 as 16 x 7 steps does not fit 128 registers with all 7 loads in flight (spills, 43 us
-    // against 16).
     if (M <= 16 && steps_total == 32) NW = 16;
     const int STEPS = NW ? steps_total / NW : 0;
     int G = env_g > 0 ? env_g : (int)((groups + 255) / 256);
     if (G > 64) G = 64;
     dim3 grid((unsigned)((groups + G - 1) / G)), block(NW * 64);
     bool handled = true;
-    // K = 14336 with at most 8 tokens (one or two int8 tokens went to the row kernel above):
-    // activations in LDS, all 14 steps of loads in flight
-    // (N = 4096, us at M = 3 / 4 / 8: 15.8 -> 15.0, 15.9 -> 14.7, 17.0 -> 15.4)
-    if (M <= 8 && NW == 8 && STEPS == 14) {
-      if (op == FMSMO_OP_I8)
-        hipLaunchKernelGGL((gemv_stream_kernel<FMSMO_OP_I8, 14, 8, 14, 1, 8>), grid, block, 0, st, g, G);
-      else
-        hipLaunchKernelGGL((gemv_stream_kernel<FMSMO_OP_E4M3, 14, 8, 14, 1, 8>), grid, block, 0, st, g, G);
-      return fmsmo_check_launch();
-    }
 #define GEMV_STREAM(OPV, NWV, ST, DV)                                                             \
   if (M <= 16) hipLaunchKernelGGL((gemv_stream_kernel<OPV, ST, NWV, DV>), grid, block, 0, st, g, G); \
   else if constexpr (NWV == 8 && ST <= 8) {                                                        \
@@ -760,9 +730,9 @@ int fmsmo_gemv_dispatch(int op, const void* a, int64_t lda, const void* b, int64
     case 804: GEMV_STREAM(OPV, 8, 4, 4); break;                     \
     case 805: GEMV_STREAM(OPV, 8, 5, 5); break;                     \
     case 808: GEMV_STREAM(OPV, 8, 8, 4); break;                     \
-    case 814: GEMV_STREAM(OPV, 8, 14, 7); break;                    \
+    case 814: GEMV_STREAM(OPV, 8, 14, 2); break;                    \
     case 816: GEMV_STREAM(OPV, 8, 16, 4); break;                    \
-    case 1010: GEMV_STREAM(OPV, 10, 10, 5); break;                  \
+    case 1010: GEMV_STREAM(OPV, 10, 10, 2); break;                  \
     case 1602: GEMV_STREAM(OPV, 16, 2, 2); break;                   \
     default: handled = false; break;                                \
   }

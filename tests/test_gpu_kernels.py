@@ -438,14 +438,14 @@ def test_gemv_i8_matches_gemm_semantics(dev, M, NK):
     assert torch.equal(y_auto.cpu().view(torch.int16), ref.view(torch.int16))
 
 
-@pytest.mark.parametrize("M", [3, 5, 8, 9])
-@pytest.mark.parametrize("N", [1000, 8200])
-def test_decode_long_rows_with_activations_in_lds(dev, M, N):
-    """K = 14336 with 3 .. 8 tokens keeps the activation rows in LDS (9 tokens: registers again).
-    N = 1000: ragged last group of 16 weight rows; N = 8200: several groups per block, which
-    reuse one exchange buffer behind a second barrier.  int8 bit-exact, e4m3 exact on small
-    integers."""
-    Kd = 14336
+@pytest.mark.parametrize("M", [1, 2, 3, 5, 8, 9, 16])
+@pytest.mark.parametrize("NKd", [(1000, 14336), (8200, 14336), (1000, 12800), (520, 8192), (520, 16384)])
+def test_decode_long_rows(dev, M, NKd):
+    """Long reductions (14336 and 12800: the shallow two-step pipeline of the streaming kernel;
+    one or two tokens go to the row kernel or to the streaming kernel depending on K and operand
+    type).  N = 1000: ragged last group of 16 weight rows; N = 8200: several groups per block.
+    int8 bit-exact, e4m3 exact on small integers."""
+    N, Kd = NKd
     a, w = _rand_i8((M, Kd), 36), _rand_i8((N, Kd), 37)
     s_a = (torch.rand(M, 1, generator=gen(38)) * 0.05 + 1e-3).half()
     s_w = (torch.rand(N, generator=gen(39)) * 1e-3 + 1e-5).float()
