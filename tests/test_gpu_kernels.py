@@ -702,7 +702,7 @@ def test_split_k_fp8(dev, shape):
 
 # ------------------------------------------------------------------ 17 .. 64 tokens, one weight pass
 @pytest.mark.parametrize("M", [17, 24, 32, 33, 48, 64])
-@pytest.mark.parametrize("NK", [(4096, 4096), (520, 1024), (1000, 2048), (256, 8192), (6144, 4096)])
+@pytest.mark.parametrize("NK", [(4096, 4096), (520, 1024), (1000, 2048), (256, 8192), (6144, 4096), (1000, 5120)])
 def test_batched_decode_i8_bit_exact(dev, M, NK):
     """Batches of up to 64 tokens run through the weight-streaming kernel where their activation
     fragments fit in registers (K = 1024, 2048, 4096; 8192 up to 32 tokens) and through the tiled /
@@ -727,7 +727,7 @@ def test_batched_decode_i8_bit_exact(dev, M, NK):
 
 
 @pytest.mark.parametrize("M", [17, 32, 40, 64])
-@pytest.mark.parametrize("NK", [(4096, 4096), (520, 1024), (256, 8192)])
+@pytest.mark.parametrize("NK", [(4096, 4096), (520, 1024), (256, 8192), (1000, 5120)])
 def test_batched_decode_fp8(dev, M, NK):
     N, Kd = NK
     a = torch.randint(-8, 9, (M, Kd), generator=gen(141)).float().to(torch.float8_e4m3fn)

@@ -136,6 +136,8 @@ def test_gemm_plan_is_host_logic():
     assert K.gemm_plan(32, 4096, 8192)[0] == _lib.PLAN_DECODE
     assert K.gemm_plan(64, 4096, 4096)[0] == _lib.PLAN_DECODE
     assert K.gemm_plan(64, 4096, 8192)[0] != _lib.PLAN_DECODE
+    assert K.gemm_plan(32, 5120, 5120)[0] == _lib.PLAN_DECODE      # Llama-2-13B hidden size
+    assert K.gemm_plan(33, 5120, 5120)[0] != _lib.PLAN_DECODE
     # a few tokens through a long reduction: split only when a workspace is offered
     k, tm, tn, s = K.gemm_plan(17, 4096, 14336, with_workspace=True)
     assert (k, tm, tn) == (DMA, 128, 128) and s >= 2 and 14336 % (s * 128) == 0
