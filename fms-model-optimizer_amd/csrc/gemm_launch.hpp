@@ -155,11 +155,49 @@ void launch_any(const GemmArgs& g, const Epi& epi, hipStream_t st) {
   }
 }
 
+// A last round of 256x256 tiles that fills at most a quarter of the compute units costs most of
+// a round.  Columns to cut off so that the remaining tiles make full rounds (0 = leave the GEMM
+// whole); the cut columns then run as a second, small GEMM with the tile shape that suits them.
+// Taken only when at least 1024 columns are cut: a narrower second GEMM is a latency-bound launch
+// that costs as much as the sparse round it replaces (us, whole -> cut: 2048 x 25600 x 4096, 32
+// tiles over 3 rounds, int8 263 -> 248, e4m3 224 -> 204; 4096 x 8448 x 8192, 16 tiles over 2
+// rounds, one column tile cut: 316 -> 321).  FMSMO_TAIL_SPLIT=0 switches this off (tuning aid).
+inline int tail_split_columns(int M, int N, int K) {
+  static const char* off = getenv("FMSMO_TAIL_SPLIT");
+  if (off && off[0] == '0') return 0;
+  if (K % 128 || !use_register_staged(0) || pick_tile(M, N, true) != 0) return 0;
+  const long gm = div_up(M, 256), gn = div_up(N, 256), tiles = gm * gn;
+  if (tiles <= 256) return 0;
+  const long last = tiles % 256;
+  if (last == 0 || last > 64) return 0;
+  const long cut = (last + gm - 1) / gm;  // column tiles
+  if (cut < 4 || cut >= gn) return 0;
+  return (int)(N - (gn - cut) * 256);
+}
+
 template <int OP, bool REF, class AccT, bool GROUPED>
 int launch_dq(const GemmArgs& g, const float* a_scale, int a_stride, const float* w_scale,
               int w_stride, const void* bias, int bias_dtype, void* y, int y_dtype, int64_t ldy,
-              hipStream_t st) {
+              hipStream_t st, bool may_split = true) {
   if (!bias) bias_dtype = FMSMO_F32;
+  if constexpr (!GROUPED) {
+    const int tail = may_split ? tail_split_columns(g.M, g.N, g.K) : 0;
+    if (tail > 0) {
+      const int64_t n0 = g.N - tail;
+      GemmArgs g1 = g, g2 = g;
+      g1.N = (int)n0;
+      g2.N = tail;
+      g2.b = g.b + n0 * g.ldb;
+      const int64_t ysz = y_dtype == FMSMO_F32 ? 4 : 2, bsz = bias_dtype == FMSMO_F32 ? 4 : 2;
+      int rc = launch_dq<OP, REF, AccT, false>(g1, a_scale, a_stride, w_scale, w_stride, bias, bias_dtype,
+                                               y, y_dtype, ldy, st, false);
+      if (rc) return rc;
+      return launch_dq<OP, REF, AccT, false>(
+          g2, a_scale, a_stride, w_scale + (w_stride ? n0 : 0), w_stride,
+          bias ? (const void*)((const char*)bias + n0 * bsz) : nullptr, bias_dtype,
+          (void*)((char*)y + n0 * ysz), y_dtype, ldy, st, false);
+    }
+  }
 #define GO(OUT, BIAS)                                                                         \
   {                                                                                           \
     EpiDequant<OUT, BIAS, REF, AccT> epi{y, ldy, a_scale, w_scale, bias, a_stride, w_stride}; \
