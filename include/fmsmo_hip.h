@@ -174,7 +174,7 @@ int fmsmo_gemm_i8_i32(const int8_t* a, int64_t lda, const int8_t* b, int64_t ldb
  * a_scale: fp32 [M] (a_scale_n == M) or one value (a_scale_n == 1); w_scale likewise [N] or 1;
  * bias: [N] of bias_dtype or NULL.  epilogue: FMSMO_EPI_REF_F16 | FMSMO_EPI_F32.
  * M <= 16 is routed to the weight-streaming (HBM-bound) kernel, and so are 17 <= M <= 64 when
- * K is 1024, 2048 or 4096 (8192 up to M = 32).
+ * K is 1024, 2048 or 4096 (5120 and 8192 up to M = 32).
  * Reference: QLinearINT8Deploy.iaddmm_int, plain branch (fms_mo/modules/linear.py:1177-1188),
  * torch.ops.fms_mo.iaddmm (custom_ext_kernels/utils.py:729-737).
  */
@@ -217,6 +217,9 @@ int64_t fmsmo_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
  * number of K slices (1 = single pass).  The choice weighs the measured efficiency of each tile
  * shape against how full the last round of tiles leaves the 256 compute units, e.g.
  * 4096 x 6144 runs 512 tiles of 256 x 192 (two full rounds) rather than 384 of 256 x 256.
+ * 2048 x 4096 runs 256 tiles of 256 x 128 rather than 128 of 256 x 256.  Not reported: when the
+ * last round of 256 x 256 tiles would be nearly empty, the *_dq calls run its columns (at least
+ * 1024) as a second GEMM behind the first.
  * No counterpart in the reference (CUTLASS / cuBLASLt choose internally).
  */
 enum fmsmo_plan_kernel {
