@@ -1,6 +1,7 @@
 // Host launchers of the tiled MFMA GEMMs (int8 -> int32, int8 / e4m3 with fused dequantizing
 // epilogue, grouped mixture-of-experts variant).
 #include "gemm_launch.hpp"
+#include <mutex>
 
 thread_local char g_fmsmo_last_error[256] = {0};
 
@@ -31,6 +32,7 @@ extern "C" const char* fmsmo_status_str(int s) {
     case FMSMO_ERR_ALIGN: return "pointer, K or leading dimension not 16-byte aligned";
     case FMSMO_ERR_UNSUPPORTED: return "unsupported enum value or size";
     case FMSMO_ERR_LAUNCH: return "kernel launch failed";
+    case FMSMO_ERR_SCRATCH: return "shape needs more scratch than the library's static buffer holds";
     default: return "unknown status";
   }
 }
@@ -102,6 +104,66 @@ extern "C" int fmsmo_gemm_i8_dq_ws(const int8_t* a, int64_t lda, const int8_t* b
                                    fmsmo_stream_t stream) {
   return gemm_i8_dq_impl(a, lda, b, ldb, a_scale, a_scale_n, w_scale, w_scale_n, bias, bias_dtype,
                          epilogue, y, y_dtype, ldy, M, N, K, workspace, workspace_bytes, stream);
+}
+
+// ------------------------------------------------------------- entry point that allocates nothing
+// Split-K partial sums in device memory that belongs to the library's code object instead of a
+// caller's workspace.  `scratch` is a host-side stand-in for the array: its device address is
+// looked up once per device (each GPU that loads the library holds its own copy) and only that
+// address is handed to kernels.
+static __device__ __align__(256) unsigned char scratch[FMSMO_STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mu;
+void* g_scratch_ptr[kMaxDevices] = {nullptr};
+
+int static_scratch(void** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e == hipSuccess && (dev < 0 || dev >= kMaxDevices)) e = hipErrorInvalidDevice;
+  if (e == hipSuccess) {
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    if (!g_scratch_ptr[dev]) {
+      void* p = nullptr;
+      e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));  // address on the CURRENT device
+      if (e == hipSuccess && !p) e = hipErrorInvalidSymbol;
+      if (e == hipSuccess) g_scratch_ptr[dev] = p;
+    }
+    if (e == hipSuccess) *out = g_scratch_ptr[dev];
+  }
+  if (e != hipSuccess) {
+    snprintf(g_fmsmo_last_error, sizeof(g_fmsmo_last_error), "static scratch lookup: %s",
+             hipGetErrorString(e));
+    return FMSMO_ERR_LAUNCH;
+  }
+  return FMSMO_OK;
+}
+}  // namespace
+
+extern "C" int fmsmo_gemm_i8_dq_noalloc(const int8_t* a, int64_t lda, const int8_t* b, int64_t ldb,
+                                        const float* a_scale, int64_t a_scale_n,
+                                        const float* w_scale, int64_t w_scale_n, const void* bias,
+                                        int bias_dtype, int epilogue, void* y, int y_dtype,
+                                        int64_t ldy, int64_t M, int64_t N, int64_t K,
+                                        fmsmo_stream_t stream) {
+  const int64_t need = (M > 0 && N > 0 && K > 0) ? plan_split_k(M, N, K).ws_bytes : 0;
+  if (need > (int64_t)FMSMO_STATIC_SCRATCH_BYTES) {
+    snprintf(g_fmsmo_last_error, sizeof(g_fmsmo_last_error),
+             "split-K partial sums of %lld x %lld x %lld need %lld bytes, the static scratch holds %lld",
+             (long long)M, (long long)N, (long long)K, (long long)need,
+             (long long)FMSMO_STATIC_SCRATCH_BYTES);
+    return FMSMO_ERR_SCRATCH;
+  }
+  void* ws = nullptr;
+  if (need > 0) {
+    int rc = static_scratch(&ws);
+    if (rc) return rc;
+  }
+  // every slice's kernel stores its whole M x N block of partial sums before the reduction reads
+  // it, so nothing in the scratch has to start at zero
+  return gemm_i8_dq_impl(a, lda, b, ldb, a_scale, a_scale_n, w_scale, w_scale_n, bias, bias_dtype,
+                         epilogue, y, y_dtype, ldy, M, N, K, ws, need, stream);
 }
 
 extern "C" int64_t fmsmo_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {

@@ -35,6 +35,7 @@ SIGNATURES = {
     "fmsmo_gemm_i8_dq": [_P, _L, _P, _L, _P, _L, _P, _L, _P, _I, _I, _P, _I, _L, _L, _L, _L, _P],
     "fmsmo_gemm_fp8_dq": [_P, _L, _P, _L, _P, _L, _P, _L, _P, _I, _P, _I, _L, _L, _L, _L, _P],
     "fmsmo_gemm_i8_dq_ws": [_P, _L, _P, _L, _P, _L, _P, _L, _P, _I, _I, _P, _I, _L, _L, _L, _L, _P, _L, _P],
+    "fmsmo_gemm_i8_dq_noalloc": [_P, _L, _P, _L, _P, _L, _P, _L, _P, _I, _I, _P, _I, _L, _L, _L, _L, _P],
     "fmsmo_gemm_fp8_dq_ws": [_P, _L, _P, _L, _P, _L, _P, _L, _P, _I, _P, _I, _L, _L, _L, _L, _P, _L, _P],
     "fmsmo_gemv_i8_dq": [_P, _L, _P, _L, _P, _L, _P, _L, _P, _I, _I, _P, _I, _L, _L, _L, _L, _P],
     "fmsmo_gemv_fp8_dq": [_P, _L, _P, _L, _P, _L, _P, _L, _P, _I, _P, _I, _L, _L, _L, _L, _P],
@@ -100,6 +101,6 @@ def call(name: str, *args) -> None:
     rc = getattr(lib, name)(*args)
     if rc != 0:
         msg = lib.fmsmo_status_str(rc).decode()
-        if rc == 5:
+        if rc in (5, 6):
             msg += ": " + lib.fmsmo_last_error().decode()
         raise FmsMoHipError(f"{name} failed with status {rc} ({msg})")

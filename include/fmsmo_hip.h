@@ -40,7 +40,8 @@ enum {
   FMSMO_ERR_SHAPE = 2,       /* negative size, leading dimension too small, ...     */
   FMSMO_ERR_ALIGN = 3,       /* pointer / leading dimension not 16-byte aligned     */
   FMSMO_ERR_UNSUPPORTED = 4, /* enum value or size outside what the kernels handle  */
-  FMSMO_ERR_LAUNCH = 5       /* hipLaunchKernel / hipGetLastError reported an error */
+  FMSMO_ERR_LAUNCH = 5,      /* hipLaunchKernel / hipGetLastError reported an error */
+  FMSMO_ERR_SCRATCH = 6      /* the shape needs more scratch than the static buffer holds */
 };
 
 /* Epilogue arithmetic of the fused int8 GEMM. */
@@ -240,6 +241,33 @@ int fmsmo_gemm_fp8_dq_ws(const uint8_t* a, int64_t lda, const uint8_t* b, int64_
                          int64_t w_scale_n, const void* bias, int bias_dtype, void* y, int y_dtype,
                          int64_t ldy, int64_t M, int64_t N, int64_t K, void* workspace,
                          int64_t workspace_bytes, fmsmo_stream_t stream);
+
+/*
+ * fmsmo_gemm_i8_dq_ws without a workspace argument and without any allocation: the split-K
+ * partial sums live in a device array that is part of the library's code object
+ * (FMSMO_STATIC_SCRATCH_BYTES, resident on every GPU the library is loaded on until the process
+ * ends).  It has NO counterpart in the reference; it is for callers that cannot allocate: code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  The call makes
+ * no hipMalloc / hipFree and uses no allocating library routine; the caller still passes inputs
+ * and outputs.  Results are bit-identical to fmsmo_gemm_i8_dq_ws given a sufficient workspace
+ * (and so to fmsmo_gemm_i8_dq).
+ * A shape whose partial sums would not fit returns FMSMO_ERR_SCRATCH (fmsmo_last_error() says
+ * how many bytes it needs); under the current split policy (16 < M <= 1024, at most 128 tiles of
+ * 128 x 128, up to 256 / tiles slices) the need never exceeds the buffer, so the check guards
+ * changes of that policy.  Shapes that take no split use no scratch at all.
+ * All calls on one GPU share that GPU's array: two calls that overlap in time on the same GPU
+ * (different streams, different threads) race on it; calls on one stream are ordered and safe.
+ * Nothing in the array has to be cleared between calls (every slice stores its whole block of
+ * partial sums before the reduction reads it).  The device address of the array is looked up on
+ * the first call on each device (hipGetSymbolAddress); make that first call outside a graph
+ * capture.
+ */
+#define FMSMO_STATIC_SCRATCH_BYTES (16 << 20)
+int fmsmo_gemm_i8_dq_noalloc(const int8_t* a, int64_t lda, const int8_t* b, int64_t ldb,
+                             const float* a_scale, int64_t a_scale_n, const float* w_scale,
+                             int64_t w_scale_n, const void* bias, int bias_dtype, int epilogue,
+                             void* y, int y_dtype, int64_t ldy, int64_t M, int64_t N, int64_t K,
+                             fmsmo_stream_t stream);
 
 /* ------------------------------------------------------------------------------------------
  * 3. Skinny-M (decode) variants, M <= 16: stream the weights once from HBM.

@@ -23,7 +23,7 @@ def test_header_declares_the_expected_entry_points():
               "fmsmo_gemv_fp8_dq", "fmsmo_matmul_chunk_i8", "fmsmo_matmul_chunk_fp",
               "fmsmo_grouped_gemm_i8_dq", "fmsmo_quant_weight_i8", "fmsmo_absmax_cols",
               "fmsmo_quant_act_i8_mulscale", "fmsmo_zero_shift_bias", "fmsmo_quant_i8_affine",
-              "fmsmo_bmm_i8_dq", "fmsmo_bmm_fp8_dq", "fmsmo_gemm_i8_dq_ws", "fmsmo_gemm_fp8_dq_ws",
+              "fmsmo_bmm_i8_dq", "fmsmo_bmm_fp8_dq", "fmsmo_gemm_i8_dq_ws", "fmsmo_gemm_fp8_dq_ws", "fmsmo_gemm_i8_dq_noalloc",
               "fmsmo_gemm_workspace_bytes", "fmsmo_decode_linear_i8", "fmsmo_decode_linear_fp8", "fmsmo_decode_linear_ok", "fmsmo_debug_clock_probe", "fmsmo_gemm_plan", "fmsmo_abi_version", "fmsmo_status_str", "fmsmo_last_error"]:
         assert s in syms
 
