@@ -61,7 +61,7 @@ static int gemm_i8_dq_impl(const int8_t* a, int64_t lda, const int8_t* b, int64_
   if (rc) return rc;
   rc = check_dq(a_scale, a_scale_n, w_scale, w_scale_n, bias, bias_dtype, y_dtype, M, N);
   if (rc) return rc;
-  if (epilogue != FMSMO_EPI_REF_F16 && epilogue != FMSMO_EPI_F32) return FMSMO_ERR_UNSUPPORTED;
+  if (epilogue < FMSMO_EPI_REF_F16 || epilogue > FMSMO_EPI_F32_MULADD) return FMSMO_ERR_UNSUPPORTED;
   if (M == 0) return FMSMO_OK;
   if ((M <= 16 && K % 128 == 0) || fmsmo_gemv_batch_ok(M, K))
     return fmsmo_gemv_dispatch(FMSMO_OP_I8, a, lda, b, ldb, a_scale, a_scale_n, w_scale, w_scale_n,
@@ -78,13 +78,15 @@ static int gemm_i8_dq_impl(const int8_t* a, int64_t lda, const int8_t* b, int64_
       return launch_split_k<MMA_I8, true, int>(plan, g, workspace, a_scale, as, w_scale, ws, bias,
                                                bias_dtype, y, y_dtype, ldy, (hipStream_t)stream);
     return launch_split_k<MMA_I8, false, int>(plan, g, workspace, a_scale, as, w_scale, ws, bias,
-                                              bias_dtype, y, y_dtype, ldy, (hipStream_t)stream);
+                                              bias_dtype, y, y_dtype, ldy, (hipStream_t)stream,
+                                              epilogue == FMSMO_EPI_F32_MULADD);
   }
   if (epilogue == FMSMO_EPI_REF_F16)
     return launch_dq<MMA_I8, true, int, false>(g, a_scale, as, w_scale, ws, bias, bias_dtype, y,
                                                y_dtype, ldy, (hipStream_t)stream);
   return launch_dq<MMA_I8, false, int, false>(g, a_scale, as, w_scale, ws, bias, bias_dtype, y,
-                                              y_dtype, ldy, (hipStream_t)stream);
+                                              y_dtype, ldy, (hipStream_t)stream, true,
+                                              epilogue == FMSMO_EPI_F32_MULADD);
 }
 
 extern "C" int fmsmo_gemm_i8_dq(const int8_t* a, int64_t lda, const int8_t* b, int64_t ldb,
@@ -170,6 +172,12 @@ extern "C" int64_t fmsmo_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   return plan_split_k(M, N, K).ws_bytes;
 }
 
+extern "C" int64_t fmsmo_gemm_tail_columns(int64_t M, int64_t N, int64_t K) {
+  if (M <= 0 || N <= 0 || K <= 0 || M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff) return 0;
+  if ((M <= 16 && K % 128 == 0) || fmsmo_gemv_batch_ok(M, K)) return 0;
+  return tail_split_columns((int)M, (int)N, (int)K);
+}
+
 extern "C" int fmsmo_gemm_plan(int64_t M, int64_t N, int64_t K, int with_workspace, int* kernel,
                                int* tile_m, int* tile_n, int* splits) {
   if (!kernel || !tile_m || !tile_n || !splits) return FMSMO_ERR_NULL;
@@ -216,7 +224,7 @@ extern "C" int fmsmo_grouped_gemm_i8_dq(const int8_t* a, int64_t lda, const int8
   if ((int64_t)num_experts * ldb_e >= (1ll << 40)) return FMSMO_ERR_UNSUPPORTED;
   if (K % 64 || ldb_e % 16) return FMSMO_ERR_ALIGN;
   if (y_dtype < 0 || y_dtype > 2 || (bias && (bias_dtype < 0 || bias_dtype > 2))) return FMSMO_ERR_UNSUPPORTED;
-  if (epilogue != FMSMO_EPI_REF_F16 && epilogue != FMSMO_EPI_F32) return FMSMO_ERR_UNSUPPORTED;
+  if (epilogue < FMSMO_EPI_REF_F16 || epilogue > FMSMO_EPI_F32_MULADD) return FMSMO_ERR_UNSUPPORTED;
   if (total_rows == 0) return FMSMO_OK;
   GemmArgs g{};
   g.a = (const uint8_t*)a; g.b = (const uint8_t*)b; g.lda = lda; g.ldb = ldb;
@@ -227,7 +235,8 @@ extern "C" int fmsmo_grouped_gemm_i8_dq(const int8_t* a, int64_t lda, const int8
     return launch_dq<MMA_I8, true, int, true>(g, a_scale, 1, w_scale, 1, bias, bias_dtype, y,
                                               y_dtype, ldy, (hipStream_t)stream);
   return launch_dq<MMA_I8, false, int, true>(g, a_scale, 1, w_scale, 1, bias, bias_dtype, y,
-                                             y_dtype, ldy, (hipStream_t)stream);
+                                             y_dtype, ldy, (hipStream_t)stream, true,
+                                             epilogue == FMSMO_EPI_F32_MULADD);
 }
 
 

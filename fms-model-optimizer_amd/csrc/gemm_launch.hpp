@@ -178,7 +178,7 @@ inline int tail_split_columns(int M, int N, int K) {
 template <int OP, bool REF, class AccT, bool GROUPED>
 int launch_dq(const GemmArgs& g, const float* a_scale, int a_stride, const float* w_scale,
               int w_stride, const void* bias, int bias_dtype, void* y, int y_dtype, int64_t ldy,
-              hipStream_t st, bool may_split = true) {
+              hipStream_t st, bool may_split = true, int muladd = 0) {
   if (!bias) bias_dtype = FMSMO_F32;
   if constexpr (!GROUPED) {
     const int tail = may_split ? tail_split_columns(g.M, g.N, g.K) : 0;
@@ -190,17 +190,17 @@ int launch_dq(const GemmArgs& g, const float* a_scale, int a_stride, const float
       g2.b = g.b + n0 * g.ldb;
       const int64_t ysz = y_dtype == FMSMO_F32 ? 4 : 2, bsz = bias_dtype == FMSMO_F32 ? 4 : 2;
       int rc = launch_dq<OP, REF, AccT, false>(g1, a_scale, a_stride, w_scale, w_stride, bias, bias_dtype,
-                                               y, y_dtype, ldy, st, false);
+                                               y, y_dtype, ldy, st, false, muladd);
       if (rc) return rc;
       return launch_dq<OP, REF, AccT, false>(
           g2, a_scale, a_stride, w_scale + (w_stride ? n0 : 0), w_stride,
           bias ? (const void*)((const char*)bias + n0 * bsz) : nullptr, bias_dtype,
-          (void*)((char*)y + n0 * ysz), y_dtype, ldy, st, false);
+          (void*)((char*)y + n0 * ysz), y_dtype, ldy, st, false, muladd);
     }
   }
 #define GO(OUT, BIAS)                                                                         \
   {                                                                                           \
-    EpiDequant<OUT, BIAS, REF, AccT> epi{y, ldy, a_scale, w_scale, bias, a_stride, w_stride}; \
+    EpiDequant<OUT, BIAS, REF, AccT> epi{y, ldy, a_scale, w_scale, bias, a_stride, w_stride, muladd}; \
     if constexpr (GROUPED) {                                                                  \
       if (g.K % 128 == 0 && use_register_staged(OP)) launch_rs<OP, true>(g, epi, st);         \
       else launch_tile<TileBig, OP, true>(g, epi, st);                                        \
@@ -279,7 +279,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const AccT* __restri
 template <int OP, bool REF, class AccT>
 int launch_split_k(const SplitPlan& p, const GemmArgs& g0, void* workspace, const float* a_scale,
                    int a_stride, const float* w_scale, int w_stride, const void* bias,
-                   int bias_dtype, void* y, int y_dtype, int64_t ldy, hipStream_t st) {
+                   int bias_dtype, void* y, int y_dtype, int64_t ldy, hipStream_t st, int muladd = 0) {
   GemmArgs g = g0;
   g.K = (int)p.k_len;
   g.num_experts = p.splits;
@@ -294,7 +294,7 @@ int launch_split_k(const SplitPlan& p, const GemmArgs& g0, void* workspace, cons
   dim3 grid(div_up(g0.N, 256), (unsigned)g0.M), block(256);
 #define GO(OUT, BIAS)                                                                         \
   {                                                                                           \
-    EpiDequant<OUT, BIAS, REF, AccT> epi{y, ldy, a_scale, w_scale, bias, a_stride, w_stride}; \
+    EpiDequant<OUT, BIAS, REF, AccT> epi{y, ldy, a_scale, w_scale, bias, a_stride, w_stride, muladd}; \
     hipLaunchKernelGGL((splitk_reduce_kernel<AccT, decltype(epi)>), grid, block, 0, st,       \
                        (const AccT*)workspace, p.splits, g0.M, g0.N, epi);                    \
   }

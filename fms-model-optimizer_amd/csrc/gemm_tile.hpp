@@ -647,6 +647,7 @@ struct EpiDequant {
   const float* w_scale;
   const void* bias;
   int a_stride, w_stride;  // 0 = one value for all rows / columns, 1 = per row / column
+  int muladd = 0;          // fp32-scale form only: separate multiply and add instead of one fma
   struct Col {
     float ws, b;
   };
@@ -664,14 +665,18 @@ struct EpiDequant {
   __device__ __forceinline__ void store(int m, int n, AccT v, Row r, Col c) const {
     const int64_t idx = (int64_t)m * ldy + n;
     if constexpr (REF_F16) {
-      // separate fp32 multiply and add (no fma), scale product rounded to fp16 first,
-      // result rounded to fp16 before the cast to the output dtype
+      // separate fp32 multiply and add (no fma), scale product rounded to fp16 first; a 16-bit
+      // output is the fp16 accumulator dtype of from_fms_mo cast to the output dtype, an fp32
+      // output is the fp32 accumulator dtype of from_torch_iW (no fp16 rounding of the result)
       const float sc = round_to<FMSMO_F16>(__fmul_rn(r.as, c.ws));
-      const u16 h = f32_to_f16(__fadd_rn(__fmul_rn((float)v, sc), c.b));
-      if constexpr (OUT == FMSMO_F16) ((u16*)y)[idx] = h;
-      else store_from_f32<OUT>(y, idx, f16_to_f32(h));
+      const float t = __fadd_rn(__fmul_rn((float)v, sc), c.b);
+      if constexpr (OUT == FMSMO_F32) ((float*)y)[idx] = t;
+      else if constexpr (OUT == FMSMO_F16) ((u16*)y)[idx] = f32_to_f16(t);
+      else store_from_f32<OUT>(y, idx, f16_to_f32(f32_to_f16(t)));
     } else {
-      store_from_f32<OUT>(y, idx, __fmaf_rn((float)v, __fmul_rn(r.as, c.ws), c.b));
+      const float sc = __fmul_rn(r.as, c.ws);
+      const float t = muladd ? __fadd_rn(__fmul_rn((float)v, sc), c.b) : __fmaf_rn((float)v, sc, c.b);
+      store_from_f32<OUT>(y, idx, t);
     }
   }
 };

@@ -26,7 +26,7 @@ struct GemvArgs {
   int a_stride, w_stride;
   const void* bias;
   int bias_dtype;
-  int ref_f16;
+  int epi;  // FMSMO_EPI_*
   void* y;
   int y_dtype;
   int64_t ldy;
@@ -265,9 +265,12 @@ __global__ __launch_bounds__(NW * 64) void gemv_kernel(GemvArgs g) {
                                          : ((const float*)g.bias)[n];
       }
       float out;
-      if (g.ref_f16) {
+      if (g.epi == FMSMO_EPI_REF_F16) {
         const float sc = round_to<FMSMO_F16>(__fmul_rn(as, ws));
-        out = round_to<FMSMO_F16>(__fadd_rn(__fmul_rn((float)s, sc), b));
+        out = __fadd_rn(__fmul_rn((float)s, sc), b);
+        if (g.y_dtype != FMSMO_F32) out = round_to<FMSMO_F16>(out);
+      } else if (g.epi == FMSMO_EPI_F32_MULADD) {
+        out = __fadd_rn(__fmul_rn((float)s, __fmul_rn(as, ws)), b);
       } else {
         out = __fmaf_rn((float)s, __fmul_rn(as, ws), b);
       }
@@ -414,9 +417,12 @@ __global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(GemvArgs g, int G)
       const int n = (group0 + gi) * 16 + ((e >> 4) & 15), m = (e >> 8) * 16 + (e & 15);
       if (n < g.N && m < g.M) {
         float out;
-        if (g.ref_f16) {
+        if (g.epi == FMSMO_EPI_REF_F16) {
           const float sc = round_to<FMSMO_F16>(__fmul_rn(as_e, ws_e));
-          out = round_to<FMSMO_F16>(__fadd_rn(__fmul_rn((float)sum, sc), bv_e));
+          out = __fadd_rn(__fmul_rn((float)sum, sc), bv_e);
+          if (g.y_dtype != FMSMO_F32) out = round_to<FMSMO_F16>(out);
+        } else if (g.epi == FMSMO_EPI_F32_MULADD) {
+          out = __fadd_rn(__fmul_rn((float)sum, __fmul_rn(as_e, ws_e)), bv_e);
         } else {
           out = __fmaf_rn((float)sum, __fmul_rn(as_e, ws_e), bv_e);
         }
@@ -591,9 +597,12 @@ __global__ __launch_bounds__(256) void gemv_rows_kernel(GemvArgs g) {
                                           : ((const float*)g.bias)[n];
       }
       float out;
-      if (g.ref_f16) {
+      if (g.epi == FMSMO_EPI_REF_F16) {
         const float sc = round_to<FMSMO_F16>(__fmul_rn(as, ws));
-        out = round_to<FMSMO_F16>(__fadd_rn(__fmul_rn((float)sum, sc), bv));
+        out = __fadd_rn(__fmul_rn((float)sum, sc), bv);
+        if (g.y_dtype != FMSMO_F32) out = round_to<FMSMO_F16>(out);
+      } else if (g.epi == FMSMO_EPI_F32_MULADD) {
+        out = __fadd_rn(__fmul_rn((float)sum, __fmul_rn(as, ws)), bv);
       } else {
         out = __fmaf_rn((float)sum, __fmul_rn(as, ws), bv);
       }
@@ -643,7 +652,7 @@ int fmsmo_gemv_dispatch(int op, const void* a, int64_t lda, const void* b, int64
   g.M = (int)M; g.N = (int)N; g.K = (int)K;
   g.a_scale = a_scale; g.w_scale = w_scale;
   g.a_stride = a_scale_n == 1 ? 0 : 1; g.w_stride = w_scale_n == 1 ? 0 : 1;
-  g.bias = bias; g.bias_dtype = bias_dtype; g.ref_f16 = epilogue == FMSMO_EPI_REF_F16;
+  g.bias = bias; g.bias_dtype = bias_dtype; g.epi = epilogue;
   g.y = y; g.y_dtype = y_dtype; g.ldy = ldy;
   // M <= 2: whole-row streaming on the vector ALUs (at M = 4 its register use halves the
   // occupancy and the MFMA streaming kernel below is faster) (FMSMO_GEMV_KIND=1 disables it for tuning)
@@ -804,7 +813,7 @@ extern "C" int fmsmo_decode_linear_i8(const void* x, int x_dtype, int64_t ldx, c
   if ((x_dtype != FMSMO_F16 && x_dtype != FMSMO_BF16) || !fmsmo_decode_linear_ok(M, K)) return FMSMO_ERR_UNSUPPORTED;
   if (N >= (1 << 30) || N * ldw >= (1ll << 40)) return FMSMO_ERR_UNSUPPORTED;
   if (y_dtype < 0 || y_dtype > 2 || (bias && (bias_dtype < 0 || bias_dtype > 2))) return FMSMO_ERR_UNSUPPORTED;
-  if (epilogue != FMSMO_EPI_REF_F16 && epilogue != FMSMO_EPI_F32) return FMSMO_ERR_UNSUPPORTED;
+  if (epilogue < FMSMO_EPI_REF_F16 || epilogue > FMSMO_EPI_F32_MULADD) return FMSMO_ERR_UNSUPPORTED;
   if (ldx % 8 || ldw % 16 || (((uintptr_t)x) & 15) || (((uintptr_t)w) & 15) ||
       (smooth && (((uintptr_t)smooth) & 15)))
     return FMSMO_ERR_ALIGN;
@@ -812,7 +821,7 @@ extern "C" int fmsmo_decode_linear_i8(const void* x, int x_dtype, int64_t ldx, c
   g.b = (const uint8_t*)w; g.ldb = ldw;
   g.M = (int)M; g.N = (int)N; g.K = (int)K;
   g.w_scale = w_scale; g.w_stride = w_scale_n == 1 ? 0 : 1;
-  g.bias = bias; g.bias_dtype = bias_dtype; g.ref_f16 = epilogue == FMSMO_EPI_REF_F16;
+  g.bias = bias; g.bias_dtype = bias_dtype; g.epi = epilogue;
   g.y = y; g.y_dtype = y_dtype; g.ldy = ldy;
   g.x16 = (const u16*)x; g.ldx = ldx; g.smooth = (const u16*)smooth; g.saturate = saturate;
   g.a_scale_out = a_scale_out;
@@ -836,7 +845,7 @@ extern "C" int fmsmo_decode_linear_fp8(const void* x, int x_dtype, int64_t ldx, 
   g.b = w; g.ldb = ldw;
   g.M = (int)M; g.N = (int)N; g.K = (int)K;
   g.w_scale = w_scale; g.w_stride = w_scale_n == 1 ? 0 : 1;
-  g.bias = bias; g.bias_dtype = bias_dtype; g.ref_f16 = 0;
+  g.bias = bias; g.bias_dtype = bias_dtype; g.epi = FMSMO_EPI_F32;
   g.y = y; g.y_dtype = y_dtype; g.ldy = ldy;
   g.x16 = (const u16*)x; g.ldx = ldx;
   g.a_scale_out = a_scale_out;
@@ -866,7 +875,7 @@ extern "C" int fmsmo_gemv_i8_dq(const int8_t* a, int64_t lda, const int8_t* b, i
   int rc = check_gemv(a, lda, b, ldb, a_scale, a_scale_n, w_scale, w_scale_n, bias, bias_dtype, y,
                       y_dtype, ldy, M, N, K);
   if (rc) return rc;
-  if (epilogue != FMSMO_EPI_REF_F16 && epilogue != FMSMO_EPI_F32) return FMSMO_ERR_UNSUPPORTED;
+  if (epilogue < FMSMO_EPI_REF_F16 || epilogue > FMSMO_EPI_F32_MULADD) return FMSMO_ERR_UNSUPPORTED;
   if (M == 0) return FMSMO_OK;
   return fmsmo_gemv_dispatch(FMSMO_OP_I8, a, lda, b, ldb, a_scale, a_scale_n, w_scale, w_scale_n,
                              bias, bias_dtype, epilogue, y, y_dtype, ldy, M, N, K,

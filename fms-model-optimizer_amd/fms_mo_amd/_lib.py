@@ -16,7 +16,10 @@ LIB_PATH = os.path.normpath(os.path.join(_HERE, "..", "lib", "libfmsmo_hip.so"))
 # dtype / enum codes of include/fmsmo_hip.h
 F16, BF16, F32 = 0, 1, 2
 OP_I8, OP_E4M3, OP_F16, OP_BF16, OP_F32 = 0, 1, 2, 3, 4
-EPI_REF_F16, EPI_F32 = 0, 1
+EPI_REF_F16, EPI_F32, EPI_F32_MULADD = 0, 1, 2
+SQ_RAW, SQ_FMO, SQ_U8_SHIFT, SQ_S8_NARROW = 0, 1, 2, 3
+DQ_PER_TENSOR, DQ_PER_COLUMN = 0, 1
+F8E_SAT, F8E_PER_TENSOR, F8E_PER_ROW = 0, 1, 2
 FP8_LINEAR, FP8_FPXACC, FP8_FPXACC_DL8 = 0, 1, 2
 WQ_MUL, WQ_DIV = 0, 1
 MS_PER_TOKEN, MS_SYMM, MS_ASYMM = 0, 1, 2
@@ -29,6 +32,9 @@ _P, _I, _L, _F = c_void_p, c_int, c_int64, c_float
 SIGNATURES = {
     "fmsmo_quant_act_i8_pertoken": [_P, _I, _L, _P, _I, _I, _I, _P, _L, _P, _L, _L, _P],
     "fmsmo_quant_act_i8_static": [_P, _I, _L, _F, _I, _I, _P, _L, _L, _L, _P],
+    "fmsmo_quant_act_i8_static_t": [_P, _I, _L, _I, _I, _F, _F, _I, _F, _F, _P, _L, _L, _L, _P],
+    "fmsmo_quant_act_i8_dynamic": [_P, _I, _L, _P, _I, _I, _I, _P, _L, _P, _L, _L, _P],
+    "fmsmo_fake_quant_fp8": [_P, _I, _L, _I, _P, _P, _L, _P, _L, _P, _P, _L, _L, _P],
     "fmsmo_quant_act_i8_mulscale": [_P, _I, _L, _P, _P, _I, _I, _I, _P, _L, _P, _L, _L, _P],
     "fmsmo_quant_act_fp8_pertoken": [_P, _I, _L, _I, _I, _P, _L, _P, _L, _L, _P],
     "fmsmo_gemm_i8_i32": [_P, _L, _P, _L, _P, _L, _L, _L, _L, _P],
@@ -60,6 +66,7 @@ OTHER = {
     "fmsmo_last_error": ([], c_char_p),
     "fmsmo_gemm_workspace_bytes": ([c_int64, c_int64, c_int64], c_int64),
     "fmsmo_decode_linear_ok": ([c_int64, c_int64], c_int),
+    "fmsmo_gemm_tail_columns": ([c_int64, c_int64, c_int64], c_int64),
 }
 
 _lib = None

@@ -133,60 +133,91 @@ def cublas_ops_load_and_reg(qcfg=None, run_unit_test=False):
     native_gemm_ops_reg()
 
 
-def _swap_linears(mod, make, exam_inp_eval=None):
-    from ..modules.linear import QLinear
-
-    swapped = 0
-    for parent in list(mod.modules()):
-        for name, child in list(parent.named_children()):
-            if isinstance(child, QLinear):
-                setattr(parent, name, make(child))
-                swapped += 1
-    logger.info("swapped %d QLinear modules", swapped)
-    if exam_inp_eval is not None:
-        with torch.no_grad():
-            mod(**exam_inp_eval) if isinstance(exam_inp_eval, dict) else mod(exam_inp_eval)
-    return mod
+def _parent_name(target: str):
+    """'a.b.c' -> ('a.b', 'c') (torch.ao.quantization.utils._parent_name)."""
+    *parent, name = target.rsplit(".", 1)
+    return (parent[0] if parent else ""), name
 
 
-def lower_qmodel_cutlass(mod, exam_inp_eval=None, qcfg=None, use_inductor=False, model_dtype=torch.float16):
-    """Swap every QLinear for QLinearINT8Deploy (the reference first casts the module and all its
-    quantizer buffers to ``model_dtype``, custom_ext_kernels/utils.py:830, which puts the scale
-    arithmetic in that dtype; the same is done here)."""
-    from ..modules.linear import QLinearINT8Deploy
-
-    dev = next(mod.parameters()).device
-    mod.to(model_dtype)
-    _swap_linears(mod, lambda m: QLinearINT8Deploy.from_fms_mo(
-        m, use_int_kernel="cutlass", use_dynamic_max_act_Qfunc=(qcfg or {}).get("dynamic_act", -1),
-        target_device=dev), None)
-    mod.to(dev)
-    if use_inductor:
-        mod = torch.compile(mod)
-    if exam_inp_eval is not None:
-        with torch.no_grad():
-            mod(**exam_inp_eval) if isinstance(exam_inp_eval, dict) else mod(exam_inp_eval)
-    return mod
+def _run_once(mod, exam_inp_eval):
+    if exam_inp_eval is None:
+        return
+    with torch.no_grad():
+        if isinstance(exam_inp_eval, dict):
+            mod(**exam_inp_eval)
+        elif isinstance(exam_inp_eval, (tuple, list)):
+            mod(*exam_inp_eval)
+        else:
+            mod(exam_inp_eval)
 
 
-def lower_qmodel_triton(model, use_dyn_max_act=False, max_acc_bits=32, num_lsb_to_truncate=0,
-                        chunk_size=32, clamp_acc_to_dl16=False, layer_to_exclude=None):
-    """Swap QLinear -> QLinearINT8Deploy(use_int_kernel='triton') and nn.Linear -> LinearFPxAcc
-    is NOT done here; this helper handles the integer branch of the reference's function
-    (custom_ext_kernels/utils.py:869-959)."""
-    from ..modules.linear import QLinearINT8Deploy
+def lower_qmodel_cutlass(mod, exam_inp_eval=None, qcfg=None, use_inductor=False, model_dtype=torch.float16,
+                         **from_fms_mo_kwargs):
+    """In-place swap of every 8-bit QLinear for QLinearINT8Deploy, then optionally torch.compile
+    (fms_mo/custom_ext_kernels/utils.py:805-866).  Like the reference it passes no quantizer choice
+    to from_fms_mo, i.e. the static fms_mo-formula activation quantizer is what the modules get;
+    extra keyword arguments (an extension: e.g. use_dynamic_max_act_Qfunc=-1) are handed through.  As in the reference the model is first moved to
+    the host and cast to ``model_dtype`` together with all quantizer buffers, which puts the
+    offline scale arithmetic in that dtype with the host's roundings; each module is converted on
+    the target device and the model is moved back at the end."""
+    from ..modules.linear import QLinear, QLinearINT8Deploy
 
-    exclude = set(layer_to_exclude or [])
-    for pname, parent in list(model.named_modules()):
-        for name, child in list(parent.named_children()):
-            full = f"{pname}.{name}" if pname else name
-            if full in exclude:
+    curr_dev = getattr(mod, "device", next(mod.parameters()).device)
+    mod.cpu().to(model_dtype)
+    cutlass_ops_load_and_reg(qcfg)
+    for name, m in list(mod.named_modules()):
+        if isinstance(m, QLinear):
+            if m.num_bits_weight != 8 or m.num_bits_feature != 8:
+                logger.warning("Only support INT8 lowering for now, cannot lower %s", name)
                 continue
-            from ..modules.linear import QLinear
+            parent_name, module_name = _parent_name(name)
+            parent_mod = mod.get_submodule(parent_name)
+            m.to(curr_dev)
+            new_module = QLinearINT8Deploy.from_fms_mo(m, target_device=curr_dev, use_inductor=use_inductor,
+                                                       **from_fms_mo_kwargs)
+            setattr(parent_mod, module_name, new_module)
+            m.to("cpu")
+    mod.to(curr_dev)
+    if use_inductor is True:
+        use_inductor = "default"
+    if use_inductor:
+        _run_once(mod, exam_inp_eval)  # the deploy modules cache host-side decisions on an eager call
+        with torch.no_grad():
+            mod = torch.compile(mod, mode=use_inductor)
+            _run_once(mod, exam_inp_eval)
+    logger.info("Model lowered %s.", "and compiled" if use_inductor else "")
+    return mod
 
-            if isinstance(child, QLinear):
-                setattr(parent, name, QLinearINT8Deploy.from_fms_mo(
-                    child, use_int_kernel="triton",
-                    use_dynamic_max_act_Qfunc=use_dyn_max_act if use_dyn_max_act in (-1, -2) else False,
-                    max_acc_bits=max_acc_bits, truncate_lsb=num_lsb_to_truncate, chunk_size=chunk_size))
+
+def lower_qmodel_triton(model, use_dyn_max_act=False, max_acc_bits=32, clamp_acc_to_dl16=False,
+                        num_lsb_to_truncate=0, chunk_size=32, layer_to_exclude=None):
+    """In-place swap QLinear -> QLinearINT8Deploy(use_int_kernel='triton') and nn.Linear ->
+    LinearFPxAcc, both running the chunked-accumulation HIP kernels
+    (fms_mo/custom_ext_kernels/utils.py:869-959): simulation of accumulators with fewer bits
+    (max_acc_bits), LSB truncation per K chunk and the DL16 accumulator range."""
+    from ..modules.linear import LinearFPxAcc, QLinear, QLinearINT8Deploy
+
+    lin_fp_dyn_code = ("per_token" if use_dyn_max_act in [-1, -2]
+                       else "per_tensor" if use_dyn_max_act else False)
+    if layer_to_exclude is None:
+        layer_to_exclude = []
+    elif isinstance(layer_to_exclude, str):
+        layer_to_exclude = [layer_to_exclude]
+    elif not isinstance(layer_to_exclude, (list, tuple)):
+        raise RuntimeError("layer_to_exclude has to be either str, list, or tuple.")
+    for name, m in list(model.named_modules()):
+        if not isinstance(m, (QLinear, torch.nn.Linear)) or name in layer_to_exclude:
+            continue
+        parent_name, module_name = _parent_name(name)
+        parent_mod = model.get_submodule(parent_name)
+        if isinstance(m, QLinear):
+            new_lin = QLinearINT8Deploy.from_fms_mo(
+                m, use_int_kernel="triton", use_dynamic_max_act_Qfunc=use_dyn_max_act,
+                max_acc_bits=max_acc_bits, truncate_lsb=num_lsb_to_truncate, chunk_size=chunk_size)
+        else:
+            new_lin = LinearFPxAcc.from_nn(
+                m, trun_bits=num_lsb_to_truncate, chunk_size=chunk_size, dynamic_fp8=lin_fp_dyn_code,
+                clamp_acc_to_dl16=clamp_acc_to_dl16)
+        setattr(parent_mod, module_name, new_lin)
+    logger.info("Model lowering with the chunked-accumulation kernels is done.")
     return model

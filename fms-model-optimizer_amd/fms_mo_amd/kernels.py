@@ -142,6 +142,58 @@ def quant_act_fp8_pertoken(x, variant=L.FP8_LINEAR, static_scale=None):
     return q, scale
 
 
+def quant_act_i8_static_t(x, mode, compute_dtype, scale, zp, sym=0, clip_lo=0.0, clip_hi=0.0):
+    """int8 [M,K]: the static per-tensor formulas evaluated in ``compute_dtype`` (see
+    fmsmo_quant_act_i8_static_t; mode is one of L.SQ_*).  All parameters are host numbers."""
+    _need_gpu(x)
+    x = _rows(x)
+    M, K = x.shape
+    q = torch.empty((M, K), dtype=torch.int8, device=x.device)
+    with torch.cuda.device(x.device):
+        L.call("fmsmo_quant_act_i8_static_t", x.data_ptr(), _dt(x), _ld(x), int(mode),
+               _DT[compute_dtype], float(scale), float(zp), int(sym), float(clip_lo), float(clip_hi),
+               q.data_ptr(), K, M, K, _stream(x))
+    return q
+
+
+def quant_act_i8_dynamic(x, per_column, levels, zp=0):
+    """(q int8 [M,K], scale fp32 [1] or [K]): dynamic symmetric quantizer with one scale for the
+    whole tensor or one per column, abs-max / levels in x's dtype, codes shifted by zp (see
+    fmsmo_quant_act_i8_dynamic).  Two passes over x: the column abs-max, then the quantizer; nothing
+    is read back to the host."""
+    _need_gpu(x)
+    x = _rows(x)
+    M, K = x.shape
+    col_amax = absmax_cols(x)
+    q = torch.empty((M, K), dtype=torch.int8, device=x.device)
+    scale = torch.empty((K if per_column else 1,), dtype=torch.float32, device=x.device)
+    with torch.cuda.device(x.device):
+        L.call("fmsmo_quant_act_i8_dynamic", x.data_ptr(), _dt(x), _ld(x), col_amax.data_ptr(),
+               L.DQ_PER_COLUMN if per_column else L.DQ_PER_TENSOR, int(levels), int(zp),
+               q.data_ptr(), K, scale.data_ptr(), M, K, _stream(x))
+    return q, scale
+
+
+def fake_quant_fp8(x, mode, want_values=True, want_codes=False):
+    """FP8 (e4m3) emulation quantizer of QLinear on x [M,K] (see fmsmo_fake_quant_fp8; mode is one of
+    L.F8E_*).  Returns (y, q, scale, inv_scale): y the fake-quantized tensor in x's dtype (None
+    unless want_values), q the e4m3 codes (None unless want_codes), scale / inv_scale fp32 [1] or
+    [M] (None for the saturating cast)."""
+    _need_gpu(x)
+    x = _rows(x)
+    M, K = x.shape
+    y = torch.empty((M, K), dtype=x.dtype, device=x.device) if want_values else None
+    q = torch.empty((M, K), dtype=torch.float8_e4m3fn, device=x.device) if want_codes else None
+    n = {L.F8E_SAT: 0, L.F8E_PER_TENSOR: 1, L.F8E_PER_ROW: M}[mode]
+    scale = torch.empty((n,), dtype=torch.float32, device=x.device) if n else None
+    inv = torch.empty((n,), dtype=torch.float32, device=x.device) if n else None
+    col_amax = absmax_cols(x) if mode == L.F8E_PER_TENSOR else None
+    with torch.cuda.device(x.device):
+        L.call("fmsmo_fake_quant_fp8", x.data_ptr(), _dt(x), _ld(x), int(mode), _ptr(col_amax),
+               _ptr(y), K, _ptr(q), K, _ptr(scale), _ptr(inv), M, K, _stream(x))
+    return y, q, scale, inv
+
+
 # ------------------------------------------------------------------------------------ GEMMs
 def _workspace(M, N, K, device):
     """Scratch for the split-K form of the *_dq GEMMs (None when the shape does not use one).  It
@@ -203,7 +255,7 @@ def gemm_i8_i32(a, w):
     return c
 
 
-def gemm_i8_dq(a, w, a_scale, w_scale, bias=None, out_dtype=torch.float16, exact_ref=True,
+def gemm_i8_dq(a, w, a_scale, w_scale, bias=None, out_dtype=torch.float16, epilogue=L.EPI_REF_F16,
                force_gemv=False):
     a, w = _check_ab(a, w, torch.int8)
     M, K = a.shape
@@ -218,7 +270,7 @@ def gemm_i8_dq(a, w, a_scale, w_scale, bias=None, out_dtype=torch.float16, exact
     y = torch.empty((M, N), dtype=out_dtype, device=a.device)
     args = (a.data_ptr(), _ld(a), w.data_ptr(), _ld(w), a_scale.data_ptr(),
             a_scale.numel(), w_scale.data_ptr(), w_scale.numel(), _ptr(bias),
-            _dt(bias) if bias is not None else 0, L.EPI_REF_F16 if exact_ref else L.EPI_F32,
+            _dt(bias) if bias is not None else 0, int(epilogue),
             y.data_ptr(), _DT[out_dtype], N, M, N, K)
     ws = None if force_gemv else _workspace(M, N, K, a.device)
     with torch.cuda.device(a.device):
@@ -238,6 +290,8 @@ def gemm_fp8_dq(a, w, a_scale, w_scale, bias=None, out_dtype=torch.bfloat16, for
     if bias is not None:
         _need_gpu(bias)
         bias = bias.detach().reshape(-1).contiguous()
+        if bias.numel() != N:
+            raise ValueError("bias must have N elements")
     y = torch.empty((M, N), dtype=out_dtype, device=a.device)
     args = (a.data_ptr(), _ld(a), w.data_ptr(), _ld(w), a_scale.data_ptr(),
             a_scale.numel(), w_scale.data_ptr(), w_scale.numel(), _ptr(bias),
@@ -497,10 +551,10 @@ _register(
 _register(
     "gemm_i8_dq",
     "(Tensor a, Tensor w, Tensor a_scale, Tensor w_scale, Tensor? bias, ScalarType out_dtype, "
-    "bool exact_ref, bool force_gemv) -> Tensor",
-    lambda a, w, a_scale, w_scale, bias, out_dtype, exact_ref, force_gemv: _gemm_i8_dq_impl(
-        a, w, a_scale, w_scale, bias, out_dtype, exact_ref, force_gemv),
-    lambda a, w, a_scale, w_scale, bias, out_dtype, exact_ref, force_gemv: torch.empty(
+    "int epilogue, bool force_gemv) -> Tensor",
+    lambda a, w, a_scale, w_scale, bias, out_dtype, epilogue, force_gemv: _gemm_i8_dq_impl(
+        a, w, a_scale, w_scale, bias, out_dtype, epilogue, force_gemv),
+    lambda a, w, a_scale, w_scale, bias, out_dtype, epilogue, force_gemv: torch.empty(
         (a.shape[0], w.shape[0]), dtype=out_dtype, device=a.device),
 )
 _register(
@@ -546,10 +600,14 @@ def quant_act_fp8_pertoken(x, variant=L.FP8_LINEAR, static_scale=None):  # noqa:
 
 
 def gemm_i8_dq(a, w, a_scale, w_scale, bias=None, out_dtype=torch.float16, exact_ref=True,  # noqa: F811
-               force_gemv=False):
+               force_gemv=False, epilogue=None):
+    """y [M,N] = dequant(a int8 [M,K] . w int8 [N,K]^T), see fmsmo_gemm_i8_dq.  ``epilogue`` (one of
+    L.EPI_*) overrides ``exact_ref`` (True = L.EPI_REF_F16, False = L.EPI_F32)."""
     _need_gpu(a, w, bias)
+    if epilogue is None:
+        epilogue = L.EPI_REF_F16 if exact_ref else L.EPI_F32
     return torch.ops.fms_mo_amd.gemm_i8_dq(a, w, _as_scale(a_scale, a.device), _as_scale(w_scale, a.device),
-                                           bias, out_dtype, bool(exact_ref), bool(force_gemv))
+                                           bias, out_dtype, int(epilogue), bool(force_gemv))
 
 
 def gemm_fp8_dq(a, w, a_scale, w_scale, bias=None, out_dtype=torch.bfloat16, force_gemv=False):  # noqa: F811
@@ -559,6 +617,9 @@ def gemm_fp8_dq(a, w, a_scale, w_scale, bias=None, out_dtype=torch.bfloat16, for
 
 
 # ------------------------------------------------------------------------ fused decode linear
+_DECODE_OK = {}
+
+
 def decode_linear_ok(x, smooth, K):
     """Can ``decode_linear_i8`` serve these activations?  One token, fp16 / bf16, SmoothQuant
     divisors of the same dtype (or none), K up to 8192 in one of the decode kernel's sizes."""
@@ -566,7 +627,14 @@ def decode_linear_ok(x, smooth, K):
         return False
     if smooth is not None and (smooth.dtype != x.dtype or smooth.numel() != K):
         return False
-    return bool(L.load().fmsmo_decode_linear_ok(x.shape[0], K))
+    key = (x.shape[0], K)
+    if torch.compiler.is_compiling():
+        # answers of earlier eager calls only (a foreign-function call cannot be traced); a shape
+        # never seen eagerly takes the two-kernel path, which serves every shape
+        return _DECODE_OK.get(key, False)
+    if key not in _DECODE_OK:
+        _DECODE_OK[key] = bool(L.load().fmsmo_decode_linear_ok(x.shape[0], K))
+    return _DECODE_OK[key]
 
 
 def _decode_linear_i8_impl(x, w, w_scale, bias, smooth, out_dtype, exact_ref, saturate):
@@ -578,11 +646,17 @@ def _decode_linear_i8_impl(x, w, w_scale, bias, smooth, out_dtype, exact_ref, sa
         raise ValueError("w must be int8 [N, K]")
     w_scale = _scale_vec(w_scale, N, x.device, "w_scale")
     if smooth is not None:
+        _need_gpu(smooth)
         smooth = smooth.detach().reshape(-1).contiguous()
+        if smooth.numel() != K or smooth.dtype != x.dtype:
+            raise ValueError("smooth must have K elements of x's dtype")
         if smooth.data_ptr() % 16:
             smooth = smooth.clone()
     if bias is not None:
+        _need_gpu(bias)
         bias = bias.detach().reshape(-1).contiguous()
+        if bias.numel() != N:
+            raise ValueError("bias must have N elements")
     y = torch.empty((M, N), dtype=out_dtype, device=x.device)
     a_scale = torch.empty((M,), dtype=torch.float32, device=x.device)
     with torch.cuda.device(x.device):
@@ -623,7 +697,10 @@ def _decode_linear_fp8_impl(x, w, w_scale, bias, out_dtype):
         raise ValueError("w must be float8_e4m3fn [N, K]")
     w_scale = _scale_vec(w_scale, N, x.device, "w_scale")
     if bias is not None:
+        _need_gpu(bias)
         bias = bias.detach().reshape(-1).contiguous()
+        if bias.numel() != N:
+            raise ValueError("bias must have N elements")
     y = torch.empty((M, N), dtype=out_dtype, device=x.device)
     a_scale = torch.empty((M,), dtype=torch.float32, device=x.device)
     with torch.cuda.device(x.device):

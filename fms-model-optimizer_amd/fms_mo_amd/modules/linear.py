@@ -31,6 +31,7 @@ from ..quant.quantizers import (
     Qmax,
     get_activation_quantizer,
     get_weight_quantizer,
+    to_fp8,
 )
 
 logger = logging.getLogger(__name__)
@@ -142,7 +143,9 @@ class QLinear(nn.Linear):
             self.register_buffer("smoothq_act_scale", torch.zeros(self.weight.shape[1]))
             self.register_buffer("smoothq_alpha",
                                  torch.tensor([qcfg.get("smoothq_alpha", 0.5)], dtype=torch.float32))
-        self._wcache = None  # (key, w_int8, w_scale) of the eval-mode integer path
+        self._wcache = None   # (key, quantized weights, weight scales) of the eval-mode kernel paths
+        self._sqcache = None  # (key, SmoothQuant scale or None)
+        self._sq_gen = 0
 
     # -- SmoothQuant ------------------------------------------------------------------------
     def set_act_scale(self, act_scale):
@@ -156,54 +159,122 @@ class QLinear(nn.Linear):
         alpha = self.smoothq_alpha.item() if isinstance(self.smoothq_alpha, torch.Tensor) else self.smoothq_alpha
         return (self.smoothq_act_scale.pow(alpha) / wmax.pow(1.0 - alpha)).clamp(min=1e-5).to(x.dtype)
 
+    def _cached_smoothq_scale(self, x):
+        """get_smoothq_scale(x), recomputed only when the activation statistics, alpha or the
+        weights change: the reference re-reads all of W for a column maximum and synchronizes with
+        the host (``.sum().item()``) on every forward (linear.py:345-368)."""
+        if not self.smoothq:
+            return None
+        a, al, w = self.smoothq_act_scale, self.smoothq_alpha, self.weight
+        key = (a.data_ptr(), a._version, w.data_ptr(), w._version, x.dtype, x.device,
+               (al.data_ptr(), al._version) if torch.is_tensor(al) else al)
+        if self._sqcache is None or self._sqcache[0] != key:
+            scale = self.get_smoothq_scale(x)
+            self._sq_gen += 1  # names this scale in the keys of the weight caches
+            self._sqcache = (key, scale if scale.numel() > 1 else None)
+        return self._sqcache[1]
+
     # -- forward ----------------------------------------------------------------------------
-    def _int_path_ok(self, x):
+    def _eval_path_ok(self, x):
         return (not self.training and self.calib_counter <= 0 and self.ptqmode != "fp32_out"
                 and self.mask is None and x.is_cuda
-                and self.num_bits_feature == 8 and self.num_bits_weight == 8
+                and self.num_bits_feature == 8 and self.num_bits_weight == 8)
+
+    def _int_path_ok(self, x):
+        return (self._eval_path_ok(x)
                 and isinstance(self.quantize_feature, QMaxDynamic)
                 and self.quantize_feature.reduce_dim == -1
                 and isinstance(self.quantize_weight, Qmax))
 
+    def _fp8_path_ok(self, x):
+        return (self._eval_path_ok(x) and x.shape[-1] % 16 == 0
+                and x.dtype in (torch.float16, torch.bfloat16, torch.float32)
+                and isinstance(self.quantize_feature, to_fp8) and self.quantize_feature.emulate
+                and isinstance(self.quantize_weight, to_fp8) and self.quantize_weight.emulate)
+
+    def _weights_key(self, scale):
+        w = self.weight
+        return (w._version, w.data_ptr(), w.dtype, None if scale is None else self._sq_gen)
+
     def _int_weights(self, scale):
         """Integer weights of the fake-quantized W*scale, cached until W, the clip values or the
-        SmoothQuant scale change.  Levels: fake_quantize_per_channel_affine / QmaxSTE, i.e. the
-        stored ``clip_val`` of the weight quantizer defines the grid (eval-mode semantics)."""
+        SmoothQuant scale change (``scale`` is the cached tensor of _cached_smoothq_scale, so its
+        identity stands for the statistics it was computed from).  Levels:
+        fake_quantize_per_channel_affine / QmaxSTE, i.e. the stored ``clip_val`` of the weight
+        quantizer defines the grid (eval-mode semantics)."""
         qw = self.quantize_weight
-        key = (self.weight._version, self.weight.data_ptr(), qw.clip_val._version,
-               None if scale is None else (scale.data_ptr(), scale._version))
+        key = self._weights_key(scale) + (qw.clip_val._version, qw.clip_val.data_ptr())
         if self._wcache is not None and self._wcache[0] == key:
             return self._wcache[1], self._wcache[2]
         with torch.no_grad():
-            ws = self.weight if scale is None else self.weight * scale
-            cv = qw.clip_val.to(ws.device).float()
+            cv = qw.clip_val.to(self.weight.device).float()
             w_scale = cv * 2 / 254
-            if qw.perCh:
-                # torch.fake_quantize_per_channel_affine rounds x * (1/scale)
-                inv = 1.0 / w_scale
-                w_int = torch.clamp(torch.round(ws.float() * inv[:, None]), -127, 127)
+            Kd = self.weight.shape[1]
+            if qw.perCh and Kd % 8 == 0 and self.weight.dtype in (torch.float16, torch.bfloat16, torch.float32):
+                # torch.fake_quantize_per_channel_affine rounds W.float() * (1 / scale): one pass of
+                # the weight-quantizer kernel (SmoothQuant folding W * s in W's dtype included)
+                smooth = None if scale is None else scale.reshape(-1).to(self.weight.dtype).contiguous()
+                w_int8 = kernels.quant_weight_i8(self.weight.detach(), 1.0 / w_scale, smooth, mode="mul")
+            elif qw.perCh:
+                ws = self.weight if scale is None else self.weight * scale
+                w_int8 = torch.clamp(torch.round(ws.float() * (1.0 / w_scale)[:, None]), -127, 127).to(torch.int8)
             else:
+                ws = self.weight if scale is None else self.weight * scale
                 u = ws.mul(1 / cv.to(ws.dtype)).clamp(-1, 1).mul(0.5).add(0.5)
-                w_int = torch.round(254 * u) - 127
-            w_int8 = w_int.to(torch.int8).contiguous()
+                w_int8 = (torch.round(254 * u) - 127).to(torch.int8).contiguous()
         self._wcache = (key, w_int8, w_scale.float().reshape(-1))
         return w_int8, self._wcache[2]
 
+    @staticmethod
+    def _fp8_mode(q):
+        if q.perCh or q.perToken:
+            return L.F8E_PER_ROW
+        return L.F8E_SAT if "_sat" in q.q_mode else L.F8E_PER_TENSOR
+
+    def _fp8_weights(self, scale):
+        """e4m3 codes of the emulation quantizer's W*scale and their dequantizing factors, cached
+        like the integer weights."""
+        key = self._weights_key(scale) + ("fp8", self.quantize_weight.q_mode)
+        if self._wcache is not None and self._wcache[0] == key:
+            return self._wcache[1], self._wcache[2]
+        with torch.no_grad():
+            ws = self.weight.detach() if scale is None else self.weight.detach() * scale
+            _, q, _, inv = kernels.fake_quant_fp8(ws, self._fp8_mode(self.quantize_weight),
+                                                  want_values=False, want_codes=True)
+            if inv is None:
+                inv = torch.ones(1, dtype=torch.float32, device=ws.device)
+        self._wcache = (key, q, inv)
+        return q, inv
+
     def forward(self, x):
-        if self.smoothq:
-            scale = self.get_smoothq_scale(x)
-        else:
-            scale = torch.tensor([1.0]).to(x.dtype).to(x.device)
+        scale = self._cached_smoothq_scale(x) if x.is_cuda else None
         if self._int_path_ok(x):
             x2 = x.reshape(-1, x.shape[-1])
-            smooth = scale.reshape(-1) if scale.numel() > 1 else None
+            smooth = None if scale is None else scale.reshape(-1)
             q, s = kernels.quant_act_i8_pertoken(x2, smooth, compute_dtype=x.dtype)
-            w_int8, w_scale = self._int_weights(scale if scale.numel() > 1 else None)
+            w_int8, w_scale = self._int_weights(scale)
             y = kernels.gemm_i8_dq(q, w_int8, s, w_scale, self.bias, out_dtype=x.dtype, exact_ref=False)
+            self.num_module_called += 1
+            return y.reshape(tuple(x.shape[:-1]) + (self.out_features,))
+        if self._fp8_path_ok(x):
+            # FP8 emulation modes: the reference multiplies the fake-quantized tensors with F.linear;
+            # here the e4m3 codes go through the FP8 MFMA GEMM and the two reciprocal scales are
+            # applied to the fp32 accumulator
+            x2 = x.reshape(-1, x.shape[-1])
+            if scale is not None:
+                x2 = x2 / scale
+            _, q, _, inv = kernels.fake_quant_fp8(x2, self._fp8_mode(self.quantize_feature),
+                                                  want_values=False, want_codes=True)
+            if inv is None:
+                inv = torch.ones(1, dtype=torch.float32, device=x.device)
+            wq, w_inv = self._fp8_weights(scale)
+            y = kernels.gemm_fp8_dq(q, wq, inv, w_inv, self.bias, out_dtype=x.dtype)
             self.num_module_called += 1
             return y.reshape(tuple(x.shape[:-1]) + (self.out_features,))
         if not x.is_cuda:
             raise RuntimeError("fms_mo_amd.QLinear runs on an AMD GPU only; there is no CPU path")
+        if scale is None:
+            scale = torch.tensor([1.0]).to(x.dtype).to(x.device)
         # training / calibration / other quantizer modes: quantizer modules evaluated with torch ops
         if self.calib_counter > 0:
             with torch.no_grad():
@@ -376,7 +447,7 @@ class QLinearINT8Deploy(nn.Linear):
             m.register_buffer("corr_term", corr_term)
             m.register_buffer("zero_shift", zero_s)
             if nnlin_iW.bias is not None:
-                m.bias = nn.Parameter((nnlin_iW.bias - corr_term.to(target_device)).to(m.acc_dtype),
+                m.bias = nn.Parameter((nnlin_iW.bias - corr_term.to(nnlin_iW.bias.device)).to(m.acc_dtype),
                                       requires_grad=False)
                 m.org_mod_has_bias = True
             else:
@@ -387,44 +458,77 @@ class QLinearINT8Deploy(nn.Linear):
         return m.to(target_device)
 
     # -- activation quantizers (device kernels) ----------------------------------------------
+    def _static_params(self, x_dtype):
+        """Host copies of the static quantizer's parameters and the dtype torch would evaluate the
+        formula in, refreshed when a buffer changes (reading them costs a host sync)."""
+        tensors = [self.input_scale, self.input_zp]
+        fmo = not self.usePTnativeQfunc and hasattr(self, "quant_stepsize")
+        if fmo:
+            tensors += [self.quant_stepsize, self.quant_zero_point]
+            tensors += [t for t in self.cvs[:2] if torch.is_tensor(t)]
+        key = (x_dtype,) + tuple((t.data_ptr(), t._version, t.dtype) for t in tensors)
+        if getattr(self, "_sp_key", None) != key:
+            probe = torch.empty((1, 1), dtype=x_dtype)
+            p = {"scale": float(self.input_scale.reshape(-1)[0]), "zp": int(self.input_zp.reshape(-1)[0]),
+                 "T": torch.result_type(probe, self.input_scale.cpu())}
+            if fmo:
+                cvn, cv = (t.detach().cpu() if torch.is_tensor(t) else torch.tensor(float(t)) for t in
+                           (self.cvs[1], self.cvs[0]))
+                clamped = probe.clamp(cvn, cv)                     # torch's own promotion rules
+                quot = clamped / self.quant_stepsize.cpu() - self.quant_zero_point.cpu()
+                p.update(T=quot.dtype, lo=float(cvn.to(clamped.dtype).reshape(-1)[0]),
+                         hi=float(cv.to(clamped.dtype).reshape(-1)[0]),
+                         step=float(self.quant_stepsize.reshape(-1)[0]),
+                         qzp=float(self.quant_zero_point.reshape(-1)[0]))
+            self._sp_key, self._sp = key, p
+        return self._sp
+
     def qa_raw_qfunc(self, x):
-        return kernels.quant_act_i8_static(x, float(self.input_scale.reshape(-1)[0]),
-                                           int(self.input_zp.reshape(-1)[0]), int(self.useSymAct))
+        """clamp(round(x / input_scale + input_zp - 128 + sym), -128, 127) in the dtype torch
+        promotes x and ``input_scale`` to (linear.py:1061-1071)."""
+        p = self._static_params(x.dtype)
+        if p["T"] == torch.float32:
+            return kernels.quant_act_i8_static(x, p["scale"], p["zp"], int(self.useSymAct))
+        return kernels.quant_act_i8_static_t(x, L.SQ_RAW, p["T"], p["scale"], p["zp"], int(self.useSymAct))
 
     def qa_pt_quant_func(self, x):
         """torch.quantize_per_tensor(x.float(), scale, zp - 128 + sym) arithmetic (linear.py:1043-1059)."""
-        return kernels.quant_act_i8_static(x, float(self.input_scale.reshape(-1)[0]),
-                                           int(self.input_zp.reshape(-1)[0]), int(self.useSymAct) | 2)
+        p = self._static_params(x.dtype)
+        return kernels.quant_act_i8_static(x, p["scale"], p["zp"], int(self.useSymAct) | 2)
 
     qa_pt_qfunc_wrapped = qa_pt_quant_func
 
     def qa_fmo_mo_qfunc(self, x):
         """round(clamp(x, cvn, cv) / stepsize - zero_point) - (128 - sym): clamp-then-round with the
-        fms_mo formula (linear.py:1073-1083).  Offline-calibrated static path; torch ops."""
-        xq = torch.round(x.clamp(self.cvs[1], self.cvs[0]) / self.quant_stepsize - self.quant_zero_point) \
-            - (128 - self.useSymAct)
-        return xq.to(torch.int8)
+        fms_mo formula (linear.py:1073-1083), in the dtype torch's promotion gives the chain."""
+        p = self._static_params(x.dtype)
+        return kernels.quant_act_i8_static_t(x, L.SQ_FMO, p["T"], p["step"], p["qzp"], int(self.useSymAct),
+                                             p["lo"], p["hi"])
 
     def qa_dynamic_max_qfunc(self, x):
-        """Per-token (dim -1) dynamic abs-max quantizer; stores ``input_scale`` [M,1] and
-        ``cvs[0:2]`` like the reference."""
+        """Dynamic abs-max quantizer per token (dim -1) or per input channel over the tokens
+        (dim -2); stores ``input_scale`` ([M,1] / [1,K]) and ``cvs[0:2]`` like the reference
+        (linear.py:1085-1100)."""
         if self.useDynMaxQfunc == -2:
-            amax = x.abs().max(dim=-2, keepdim=True)[0]
-            self.cvs[0], self.cvs[1] = amax, -amax
-            self.input_scale = amax.clamp(min=1e-5).div(127)
-            return torch.round(x / self.input_scale).to(torch.int8)
-        smooth = None
-        q, s = kernels.quant_act_i8_pertoken(x, smooth, compute_dtype=x.dtype)
-        self.input_scale = s.reshape(-1, 1)
-        self.cvs[0], self.cvs[1] = s.reshape(-1, 1) * 127, -(s.reshape(-1, 1) * 127)
+            q, s = kernels.quant_act_i8_dynamic(x, True, 2 ** (self.nbits_a - 1) - 1)
+            s = s.reshape(1, -1).to(x.dtype)
+        else:
+            q, s = kernels.quant_act_i8_pertoken(x, None, compute_dtype=x.dtype)
+            s = s.reshape(-1, 1)
+        self.input_scale = s
+        self.cvs[0], self.cvs[1] = s * 127, -(s * 127)
         return q
 
     def qa_dyn_max_fake_zero_shift(self, x):
-        amax = x.abs().max()
-        levels = 2 ** (self.nbits_a - 1) - 1 - self.input_zp
-        self.cvs[0], self.cvs[1] = amax, -amax
-        self.input_scale = amax.clamp(min=1e-5) / levels
-        return (torch.round(x / self.input_scale) + self.input_zp).to(torch.int8)
+        """One dynamic scale amax / (127 - zp) for the whole tensor, codes shifted by zp
+        (linear.py:1102-1113).  The zero point is a construction-time constant."""
+        if getattr(self, "_fzs_zp", None) is None:
+            self._fzs_zp = int(self.input_zp)
+        levels = 2 ** (self.nbits_a - 1) - 1 - self._fzs_zp
+        q, s = kernels.quant_act_i8_dynamic(x, False, levels, self._fzs_zp)
+        self.input_scale = s.reshape(()).to(x.dtype)
+        self.cvs[0], self.cvs[1] = self.input_scale * levels, -(self.input_scale * levels)
+        return q
 
     # -- matmul + dequant ----------------------------------------------------------------------
     def _quantize(self, m1):
@@ -452,12 +556,27 @@ class QLinearINT8Deploy(nn.Linear):
         K = m1.shape[1]
         if K > self.chunk_size and self.use_int_kernel != "triton":
             cs = int(self.chunk_size)
-            if cs < 32 or cs & (cs - 1):
-                raise NotImplementedError("chunk_size must be a power of two >= 32 on this backend")
-            acc = kernels.matmul_chunk(m1, w, None, chunk_size=cs, chunk_trun_bits=int(self.truncate_lsb),
-                                       max_acc_bits=self.max_acc_bits)
-            # acc == 2^t * (the reference's shifted accumulator); (2^t a) * s == a * (2^t s) exactly
-            return (acc * (self.input_scale * self.w_scale) + bias).to(self.acc_dtype)
+            if cs >= 32 and not cs & (cs - 1):
+                acc = kernels.matmul_chunk(m1, w, None, chunk_size=cs, chunk_trun_bits=int(self.truncate_lsb),
+                                           max_acc_bits=self.max_acc_bits)
+                # acc == 2^t * (the reference's shifted accumulator); (2^t a) * s == a * (2^t s) exactly
+                return (acc * (self.input_scale * self.w_scale) + bias).to(self.acc_dtype)
+            # any other chunk size (ragged last chunk included): the reference's serial loop, one
+            # exact int32 GEMM per chunk
+            acc = torch.zeros((m1.shape[0], w.shape[0]), dtype=torch.int, device=m1.device)
+            t = int(self.truncate_lsb)
+            for k0 in range(0, K, cs):
+                a_c, w_c = m1[:, k0:k0 + cs], w[:, k0:k0 + cs]
+                # the GEMM wants 16-byte aligned rows: copy the slices out, zero-padded
+                pad = (-a_c.shape[1]) % 16
+                a_c, w_c = F.pad(a_c, (0, pad)).contiguous(), F.pad(w_c, (0, pad)).contiguous()
+                p = kernels.gemm_i8_i32(a_c, w_c)
+                if self.max_acc_bits < 32:
+                    p = p.clamp(self.accminmax[0], self.accminmax[1])
+                if t > 0:
+                    p = torch.bitwise_right_shift(p + (1 << (t - 1)), t)
+                acc += p
+            return (acc * ((1 << t) * self.input_scale * self.w_scale) + bias).to(self.acc_dtype)
         updated_bias = bias
         if self.use_fake_zero_shift:
             updated_bias = bias - self.input_scale * self.corr_term
@@ -465,10 +584,21 @@ class QLinearINT8Deploy(nn.Linear):
             imm_out = tl_matmul(m1, m2, chunk_trun_bits=int(self.truncate_lsb), chunk_size=int(self.chunk_size))
             return (imm_out.float() * (self.input_scale * self.w_scale).to(torch.float16)
                     + updated_bias).to(self.acc_dtype)
+        # fused epilogue: acc.float() * f16(input_scale * w_scale) + bias, rounded once to the fp16
+        # accumulator dtype of from_fms_mo or left in fp32 for any other (from_torch_iW: fp32)
         ref16 = self.acc_dtype == torch.float16
-        y = kernels.gemm_i8_dq(m1, w, self.input_scale.float().reshape(-1), self.w_scale.float().reshape(-1),
-                               updated_bias, out_dtype=torch.float16 if ref16 else torch.float32,
-                               exact_ref=True)
+        a_scale = self.input_scale.float().reshape(-1)
+        w_scale = self._w_scale_f32()
+        if self.useDynMaxQfunc == -2:
+            # per-input-channel scales [1,K] broadcast against the [M,N] accumulator (K == N): the
+            # product input_scale[n] * w_scale[n] goes in as the column scale
+            if a_scale.numel() != w.shape[0]:
+                raise RuntimeError("per-channel activation scales need in_features == out_features "
+                                   "(the reference's [1,K] scale broadcasts against [M,N])")
+            w_scale = a_scale * w_scale
+            a_scale = torch.ones(1, dtype=torch.float32, device=m1.device)
+        y = kernels.gemm_i8_dq(m1, w, a_scale, w_scale, updated_bias,
+                               out_dtype=torch.float16 if ref16 else torch.float32, exact_ref=True)
         return y if ref16 else y.to(self.acc_dtype)
 
     def iaddmm_FP(self, bias, m1, m2):
@@ -668,7 +798,112 @@ class QLinearINT8Train(torch.nn.Linear):
         return s
 
 
-QLinear_modules = (QLinear, QLinearINT8Deploy, LinearFPxAcc, QLinearINT8Train)
+class QLinearCublasI8I32NT(nn.Linear):
+    """Deploy linear with a STATIC activation quantizer, int8 x int8 -> int32 GEMM and an fp32
+    dequantization ``input_scale * w_scale * acc + bias`` (linear.py:1341-1535).  Asymmetric
+    activations are quantized to uint8 codes stored minus 128 with the zero-point correction
+    folded into the bias.  Here the quantizer is one HIP launch and the GEMM carries the
+    dequantization in its epilogue (``torch.ops.mygemm.gemm_nt_i8i32`` stays registered for callers
+    that want the raw int32 product)."""
+
+    @classmethod
+    def from_reference(cls, ref_qlinear, input_scale, input_zero_point, input_dtype, forceSymA=False):
+        """From a torch.ao reference quantized linear (per-channel weights), linear.py:1349-1427."""
+        m = cls(ref_qlinear.in_features, ref_qlinear.out_features, device="meta")
+        m.forceSymA = forceSymA
+        m.input_dtype = input_dtype
+        m.register_buffer("input_scale", input_scale.clone())
+        m.register_buffer("input_zp", input_zero_point.clone())
+        qweight = ref_qlinear.float().get_quantized_weight()
+        if ref_qlinear.weight_qscheme not in [torch.per_channel_symmetric, torch.per_channel_affine]:
+            raise RuntimeError("QLinear_cublas only supports perCh for now. ")
+        m.register_buffer("w_scale", qweight.q_per_channel_scales().float())
+        m.register_buffer("w_zp", qweight.q_per_channel_zero_points())
+        m.weight = nn.Parameter(qweight.int_repr(), requires_grad=False)
+        m.bias = nn.Parameter(ref_qlinear.bias, requires_grad=False)
+        if input_dtype == torch.quint8:
+            if forceSymA:
+                a_min = -input_zero_point * input_scale
+                a_max = (255 - input_zero_point) * input_scale
+                a_max_new = max(abs(a_min), abs(a_max))
+                m.input_scale.copy_((2 * a_max_new) / (255 - 2))
+                m.input_zp.copy_(0)
+                m.input_dtype = torch.qint8
+            else:
+                corr_term = m.w_scale * input_scale * (input_zero_point - 128) * m.weight.sum(dim=1)
+                corr_term = corr_term.to(ref_qlinear.bias.dtype)
+                m.bias = nn.Parameter(ref_qlinear.bias - corr_term, requires_grad=False)
+        return m
+
+    @classmethod
+    def from_fms_mo(cls, fms_mo_qlinear, **kwargs):
+        """From a QLinear with static (clip_val / clip_valn) activation quantizer and a max weight
+        quantizer (linear.py:1429-1489).  The activation is taken as asymmetric (quint8)."""
+        assert fms_mo_qlinear.num_bits_feature in [4, 8] and fms_mo_qlinear.num_bits_weight in [4, 8], \
+            "Please check nbits setting!"
+        target_device = kwargs.get("target_device", next(fms_mo_qlinear.parameters()).device)
+        m = cls(fms_mo_qlinear.in_features, fms_mo_qlinear.out_features, device="meta")
+        m.input_dtype = torch.quint8
+        with torch.no_grad():
+            Qa = fms_mo_qlinear.quantize_feature
+            input_scale = (Qa.clip_val - Qa.clip_valn) / (2**Qa.num_bits - 1)
+            input_zero_point = torch.round(-Qa.clip_valn / input_scale).to(torch.int)
+            m.register_buffer("input_scale", input_scale)
+            m.register_buffer("input_zp", input_zero_point)
+            Qw = fms_mo_qlinear.quantize_weight
+            w_scale = Qw.clip_val * 2 / (2**Qw.num_bits - 2)
+            m.register_buffer("w_scale", w_scale.float())
+            m.register_buffer("w_zp", torch.zeros_like(w_scale, dtype=torch.int))
+            # the weight quantizer's integer output, cast (truncated) to int8 like the reference
+            Qw.dequantize = False
+            m.weight = nn.Parameter(Qw(fms_mo_qlinear.weight.float()).to(torch.int8), requires_grad=False)
+            corr_term = m.w_scale * input_scale * (input_zero_point - 128) * m.weight.sum(dim=1)
+            corr_term = corr_term.to(fms_mo_qlinear.bias.dtype)
+            m.bias = nn.Parameter(fms_mo_qlinear.bias - corr_term, requires_grad=False)
+        return m.to(target_device)
+
+    def _get_name(self):
+        return "QuantizedLinear_cublasi8i32"
+
+    def _params(self, x_dtype):
+        """Host copies of scale and zero point and the dtype torch evaluates the quantizer in."""
+        key = (x_dtype, self.input_scale.data_ptr(), self.input_scale._version, self.input_scale.dtype,
+               self.input_zp.data_ptr(), self.input_zp._version)
+        if getattr(self, "_p_key", None) != key:
+            probe = torch.empty((1, 1), dtype=x_dtype)
+            T = (probe / self.input_scale.cpu() + self.input_zp.cpu()).dtype
+            self._p_key = key
+            self._p = (float(self.input_scale.reshape(-1)[0]), float(self.input_zp.reshape(-1)[0]), T)
+        return self._p
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        with torch.no_grad():
+            if not x.is_cuda:
+                raise RuntimeError("fms_mo_amd quantized linears run on an AMD GPU only; there is no CPU path")
+            if x.dim() not in (2, 3) and type(self) is QLinearCublasI8I32NT:
+                raise RuntimeError("Input dimension to QLinear is not 2D or batched 2D")
+            in_dtype = x.dtype
+            scale, zp, T = self._params(in_dtype)
+            x2 = x.reshape(-1, x.shape[-1])
+            mode = L.SQ_U8_SHIFT if self.input_dtype == torch.quint8 else L.SQ_S8_NARROW
+            q = kernels.quant_act_i8_static_t(x2, mode, T, scale, zp)
+            # input_scale * w_scale * acc + bias in fp32, product and sum rounded separately
+            y = kernels.gemm_i8_dq(q, self.weight, self.input_scale.float().reshape(-1),
+                                   self.w_scale.float().reshape(-1), self.bias, out_dtype=in_dtype,
+                                   epilogue=L.EPI_F32_MULADD)
+            return y.reshape(tuple(x.shape[:-1]) + (self.weight.shape[0],))
+
+
+class QLinearCutlassI8I32NT(QLinearCublasI8I32NT):
+    """The same module under the name of the CUTLASS variant (linear.py:1538-1583): any number of
+    leading dimensions is accepted."""
+
+    def _get_name(self):
+        return "QuantizedLinear_cutlassi8i32"
+
+
+QLinear_modules = (QLinear, QLinearINT8Deploy, QLinearCublasI8I32NT, QLinearCutlassI8I32NT,
+                   LinearFPxAcc, QLinearINT8Train)
 
 
 def isinstance_qlinear(module):

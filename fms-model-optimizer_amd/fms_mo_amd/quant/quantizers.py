@@ -78,6 +78,17 @@ def _qmax_per_tensor(x, num_bits, dequantize, cv, align_zero):
     return q - levels / 2
 
 
+def _qminmax_per_tensor(x, num_bits, cv, cvn, align_zero):
+    """QminmaxSTE.forward (fms_mo/quant/quantizers.py:3270-3287): asymmetric, always dequantized."""
+    cv, cvn = cv.to(x.dtype), cvn.to(x.dtype)
+    scale = (2**num_bits - 1) / (cv - cvn)
+    zero_point = cvn * scale
+    if align_zero:
+        zero_point = torch.round(zero_point)
+    out = (x.clamp(cvn.item(), cv.item()) - cvn) * scale
+    return (torch.round(out) + zero_point) / scale
+
+
 def _qmax_per_channel(x, num_bits, dequantize, cv):
     nspace = 2**num_bits - 2
     lo = -(2 ** (num_bits - 1)) + 1
@@ -101,27 +112,30 @@ class Qmax(nn.Module):
     def __init__(self, num_bits, dequantize=True, inplace=False, align_zero=False, clipSTE=True,
                  minmax=False, perCh=None, perGp=None, extend_act_range=False):
         super().__init__()
-        if minmax or perGp or extend_act_range:
+        if perGp or extend_act_range or (minmax and perCh):
             raise NotImplementedError(
-                "Qmax variants minmax / perGp / extend_act_range are outside the W8A8 inference path"
+                "Qmax variants perGp / extend_act_range / per-channel minmax are outside the W8A8 "
+                "inference path"
             )
         self.num_bits = num_bits
         self.dequantize = dequantize
         self.inplace = inplace
         self.align_zero = align_zero
         self.clipSTE = clipSTE
-        self.minmax = False
+        self.minmax = minmax
         self.perCh = perCh
         self.perGp = None
         self.extend_act_range = False
-        self.quantizer_name = "Qmax"
+        self.quantizer_name = "Qminmax" if minmax else "Qmax"
         self.movAvgFac = 0.1
         self.Niter = 0
         n = perCh if perCh else 1
         self.register_buffer("clip_val", torch.zeros(n))
         self.register_buffer("clip_valn", torch.zeros(n))
 
-    def _quantize(self, x, cv):
+    def _quantize(self, x, cv, cvn=None):
+        if self.minmax:
+            return _PassThrough.apply(x, lambda t: _qminmax_per_tensor(t, self.num_bits, cv, cvn, self.align_zero))
         if self.perCh:
             return _PassThrough.apply(x, lambda t: _qmax_per_channel(t, self.num_bits, self.dequantize, cv))
         return _PassThrough.apply(
@@ -132,20 +146,22 @@ class Qmax(nn.Module):
         if self.perCh:
             cv_new = torch.max(input_tensor.abs().reshape([self.perCh, -1]), dim=1).values
             assert len(cv_new) == input_tensor.shape[0], "dimension error"
+        elif self.minmax:  # asymmetric
+            cv_new = input_tensor.max().unsqueeze(0)
         else:
             cv_new = input_tensor.abs().max().unsqueeze(0)
-        cvn_new = -cv_new
+        cvn_new = input_tensor.min().unsqueeze(0) if self.minmax else -cv_new
         if self.Niter == 0 and self.training:
             with torch.no_grad():
                 self.clip_val.copy_(cv_new)
                 self.clip_valn.copy_(cvn_new)
         if self.training:
-            out = self._quantize(input_tensor, cv_new)
+            out = self._quantize(input_tensor, cv_new, cvn_new)
             with torch.no_grad():
                 self.clip_val.copy_(self.clip_val * (1.0 - self.movAvgFac) + cv_new * self.movAvgFac)
                 self.clip_valn.copy_(self.clip_valn * (1.0 - self.movAvgFac) + cvn_new * self.movAvgFac)
         else:
-            out = self._quantize(input_tensor, self.clip_val)
+            out = self._quantize(input_tensor, self.clip_val, self.clip_valn)
         self.Niter += 1
         return out
 
@@ -237,7 +253,7 @@ def get_activation_quantizer(qa_mode="PACT", nbits=32, clip_val=None, clip_valn=
         raise NotImplementedError(f"activation quantizer '{qa_mode}' is a training-time quantizer, not built here")
     if "max" in mode:
         if "min" in mode:
-            raise NotImplementedError("minmax activation quantizer is not on the W8A8 path")
+            return Qmax(nbits, align_zero=align_zero, minmax=True)
         if "pertoken" in mode or "perToken" in mode:
             return QMaxDynamic(nbits, dim=-1)
         if "per_channel" in mode or "perCh" in mode:

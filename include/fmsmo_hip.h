@@ -46,13 +46,20 @@ enum {
 
 /* Epilogue arithmetic of the fused int8 GEMM. */
 enum {
-  /* y = f16( f32(acc) * f32( f16(a_scale[m]*w_scale[n]) ) + f32(bias[n]) ): the exact operation
-     order of iaddmm_int's plain branch (fms_mo/modules/linear.py:1185-1188), then a cast to the
-     output dtype (linear.py:1338). */
+  /* t = f32(acc) * f32( f16(a_scale[m]*w_scale[n]) ) + f32(bias[n]), multiply and add rounded
+     separately in fp32: the exact operation order of iaddmm_int's plain branch
+     (fms_mo/modules/linear.py:1185-1188).  A 16-bit output is y = out( f16(t) ): the fp16 acc_dtype
+     that from_fms_mo hard-wires (:777), then the cast to the activations' dtype (:1338).  An fp32
+     output is y = t: the fp32 acc_dtype from_torch_iW defaults to (:955). */
   FMSMO_EPI_REF_F16 = 0,
-  /* y = out( f32(acc) * (a_scale[m]*w_scale[n]) + f32(bias[n]) ) with the scale product kept in
-     fp32 (no fp16 rounding of the scale, single rounding to the output dtype). */
-  FMSMO_EPI_F32 = 1
+  /* y = out( fma( f32(acc), a_scale[m]*w_scale[n], f32(bias[n]) ) ) with the scale product kept
+     in fp32 (no fp16 rounding of the scale, single rounding to the output dtype). */
+  FMSMO_EPI_F32 = 1,
+  /* y = out( f32( f32(acc) * (a_scale[m]*w_scale[n]) ) + f32(bias[n]) ): fp32 scale product,
+     multiply and add rounded separately -- `input_scale * w_scale * acc + bias` of
+     QLinearCublasI8I32NT / QLinearCutlassI8I32NT.forward (fms_mo/modules/linear.py:1533-1535,
+     1581-1583). */
+  FMSMO_EPI_F32_MULADD = 2
 };
 
 int fmsmo_abi_version(void);
@@ -111,6 +118,68 @@ int fmsmo_quant_act_i8_pertoken(const void* x, int x_dtype, int64_t ldx, const v
 int fmsmo_quant_act_i8_static(const void* x, int x_dtype, int64_t ldx, float scale, int zp,
                               int sym, int8_t* q, int64_t ldq, int64_t M, int64_t K,
                               fmsmo_stream_t stream);
+
+/*
+ * Static per-tensor int8 quantizers evaluated in the compute dtype T = compute_dtype (torch's
+ * promotion of x's dtype with the dtype of the module's scale buffer: x's own dtype for a module
+ * cast to the model dtype, fp32 for fp32 quantizer buffers); every intermediate is rounded to T,
+ * divisions are IEEE divisions, rint is half-to-even:
+ *   FMSMO_SQ_RAW        q = clamp( rint( (((x / scale) + zp) - 128) + sym ), -128, 127 )
+ *                       QLinearINT8Deploy.qa_raw_qfunc (fms_mo/modules/linear.py:1061-1071)
+ *   FMSMO_SQ_FMO        q = int8( rint( clamp(x, clip_lo, clip_hi) / scale - zp ) - (128 - sym) )
+ *                       with scale = quant_stepsize, zp = quant_zero_point: clamp before round,
+ *                       QLinearINT8Deploy.qa_fmo_mo_qfunc (linear.py:1073-1083)
+ *   FMSMO_SQ_U8_SHIFT   q = clamp( rint( x / scale + zp ), 0, 255 ) - 128
+ *   FMSMO_SQ_S8_NARROW  q = clamp( rint( x / scale + zp ), -127, 127 )
+ *                       the quint8 / qint8 branches of QLinearCublasI8I32NT.forward and
+ *                       QLinearCutlassI8I32NT.forward (linear.py:1505-1512, 1563-1570)
+ * scale, zp, clip_lo, clip_hi are values of T (or of fp32 when T is fp32) passed as fp32.
+ * x 16-byte aligned, K and ldx multiples of 8 elements.
+ */
+enum { FMSMO_SQ_RAW = 0, FMSMO_SQ_FMO = 1, FMSMO_SQ_U8_SHIFT = 2, FMSMO_SQ_S8_NARROW = 3 };
+int fmsmo_quant_act_i8_static_t(const void* x, int x_dtype, int64_t ldx, int mode,
+                                int compute_dtype, float scale, float zp, int sym, float clip_lo,
+                                float clip_hi, int8_t* q, int64_t ldq, int64_t M, int64_t K,
+                                fmsmo_stream_t stream);
+
+/*
+ * Dynamic symmetric int8 quantizers whose abs-max is taken over the whole tensor or per column
+ * (over the tokens), in x's dtype T.  col_amax: device fp32 [K], the column abs-max of x as
+ * fmsmo_absmax_cols writes it (a separate pass; nothing is read on the host).
+ *   FMSMO_DQ_PER_TENSOR  s = rnd_T( max(max_k col_amax[k], rnd_T(1e-5)) / levels ); scale[0] <- s
+ *   FMSMO_DQ_PER_COLUMN  s_k = rnd_T( max(col_amax[k], rnd_T(1e-5)) / levels );     scale[k] <- s_k
+ *   q = int8( rint( rnd_T(x / s) ) + zp )            (no clamp; the int8 cast wraps like torch's)
+ * PER_TENSOR with levels = 127 - zp: QLinearINT8Deploy.qa_dyn_max_fake_zero_shift
+ * (fms_mo/modules/linear.py:1102-1113); PER_COLUMN with levels = 127, zp = 0:
+ * qa_dynamic_max_qfunc with reduce dim -2 (linear.py:1085-1100).
+ * scale: device fp32, 16-byte aligned, [1] or [K].
+ */
+enum { FMSMO_DQ_PER_TENSOR = 0, FMSMO_DQ_PER_COLUMN = 1 };
+int fmsmo_quant_act_i8_dynamic(const void* x, int x_dtype, int64_t ldx, const float* col_amax,
+                               int granularity, int levels, int zp, int8_t* q, int64_t ldq,
+                               float* scale, int64_t M, int64_t K, fmsmo_stream_t stream);
+
+/*
+ * FP8 (OCP e4m3fn) emulation quantizers of QLinear, in x's dtype T:
+ *   FMSMO_F8E_SAT         y = T( e4m3( clamp(x, -448, 448) ) )                       to_fp8_saturated
+ *   FMSMO_F8E_PER_TENSOR  s = fp8 scale of max |x| (col_amax: device fp32 [K] column abs-max)
+ *   FMSMO_F8E_PER_ROW     s_m = fp8 scale of max_k |x_mk|   (per token for activations, per output
+ *                         channel for weights [N,K])
+ *     fp8 scale(a) = rnd_T( rnd_T( 1 / max(a, rnd_T(1e-12)) ) * 448 ), for T = fp16 clamped to 65504
+ *                    (max_to_scale; torch evaluates "448 / tensor" as reciprocal, then multiply)
+ *     y = rnd_T( T( e4m3( clamp( rnd_T(x * s), -448, 448 ) ) ) / s )
+ * Outputs, each optional except that y or q must be given: y [M,K] of x's dtype (the fake-quantized
+ * tensor the reference feeds to F.linear); q [M,K] the e4m3 codes; scale fp32 [1] / [M] <- s
+ * (required for PER_TENSOR); inv_scale fp32 [1] / [M] <- 1 / s (the dequantizing factor for a
+ * GEMM on the codes).
+ * Reference: to_fp8_saturated, max_to_scale, to_fp8_scaled, to_fp8_scaled_perCh,
+ * to_fp8_scaled_perToken, class to_fp8 (fms_mo/quant/quantizers.py:5309-5488), emulate = True.
+ * x and y 16-byte aligned, K, ldx, ldy, ldq multiples of 8 elements.
+ */
+enum { FMSMO_F8E_SAT = 0, FMSMO_F8E_PER_TENSOR = 1, FMSMO_F8E_PER_ROW = 2 };
+int fmsmo_fake_quant_fp8(const void* x, int x_dtype, int64_t ldx, int mode, const float* col_amax,
+                         void* y, int64_t ldy, uint8_t* q, int64_t ldq, float* scale,
+                         float* inv_scale, int64_t M, int64_t K, fmsmo_stream_t stream);
 
 /*
  * int8 quantizers with a multiplicative scale (the quantize half of the accelerator op
@@ -218,9 +287,9 @@ int64_t fmsmo_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
  * number of K slices (1 = single pass).  The choice weighs the measured efficiency of each tile
  * shape against how full the last round of tiles leaves the 256 compute units, e.g.
  * 4096 x 6144 runs 512 tiles of 256 x 192 (two full rounds) rather than 384 of 256 x 256.
- * 2048 x 4096 runs 256 tiles of 256 x 128 rather than 128 of 256 x 256.  Not reported: when the
- * last round of 256 x 256 tiles would be nearly empty, the *_dq calls run its columns (at least
- * 1024) as a second GEMM behind the first.
+ * 2048 x 4096 runs 256 tiles of 256 x 128 rather than 128 of 256 x 256.  When the last round of
+ * 256 x 256 tiles would be nearly empty, the *_dq calls run its columns (at least 1024) as a second
+ * GEMM behind the first: the plan describes the first, fmsmo_gemm_tail_columns tells the cut.
  * No counterpart in the reference (CUTLASS / cuBLASLt choose internally).
  */
 enum fmsmo_plan_kernel {
@@ -231,6 +300,9 @@ enum fmsmo_plan_kernel {
 };
 int fmsmo_gemm_plan(int64_t M, int64_t N, int64_t K, int with_workspace, int* kernel, int* tile_m,
                     int* tile_n, int* splits);
+/* Columns that the single-pass *_dq GEMMs cut off the end of N and run as a second GEMM behind
+   the first (0: the GEMM runs whole; fmsmo_gemm_plan describes the first, main part).  Host-only. */
+int64_t fmsmo_gemm_tail_columns(int64_t M, int64_t N, int64_t K);
 int fmsmo_gemm_i8_dq_ws(const int8_t* a, int64_t lda, const int8_t* b, int64_t ldb,
                         const float* a_scale, int64_t a_scale_n, const float* w_scale,
                         int64_t w_scale_n, const void* bias, int bias_dtype, int epilogue, void* y,

@@ -30,6 +30,21 @@ How each function is pinned (see tests/test_oracle_*.py):
   * AIU checkpoint conversion, column abs-max
                         -- closed forms (sqrt(a)/sqrt(wmax) at alpha = 0.5, rint(127 W s / cv) away
                            from ties), invariants (|q| <= 127, zero shift = integer row sums)
+  * static / asymmetric deploy branches, from_torch_iW, fake zero shift, per-column dynamic
+    scales, the cuBLAS / CUTLASS style modules
+                        -- the output equals the float64 product of the dequantized operands
+                           ((q - z) s_x) . (w s_w)^T + b (pins sign and size of the correction
+                           term, the zero point's offset of 128 and the dimension of the row
+                           sums); zero point 128 => no correction; clamp-then-round ==
+                           round-then-clamp == torch.quantize_per_tensor away from ties and the
+                           same end codes outside the clip range; the per-column quantizer is the
+                           per-token one of the transposed tensor; the chunk loop equals the
+                           chunked-kernel restatement (tests/test_oracle_pins_deploy.py)
+  * FP8 emulation quantizers (to_fp8*)
+                        -- the scale re-derived with exact rationals and explicit roundings
+                           (reciprocal-then-multiply, fp16 clamp), the cast against the enumerated
+                           e4m3 grid with ties to even, every element of the scaled quantizers
+                           re-derived the same way
   * FP8Linear dynamic scale (computed inside torchao 0.11, not in the reference tree):
                            PARITY UNPINNED -- the rule used is the one of the reference's test
                            helper (tests/aiu_addons/test_fp8_addon.py:65-79).
@@ -100,6 +115,48 @@ def quant_act_static_raw(x: torch.Tensor, scale: torch.Tensor, zp: int, sym: int
     return torch.clamp((x / scale + zp - 128 + sym).round(), -128, 127).to(torch.int8)
 
 
+def quant_act_pt_native(x: torch.Tensor, scale: torch.Tensor, zp: int, sym: int):
+    """qa_pt_quant_func / qa_pt_qfunc_wrapped (linear.py:1025-1059): the library routine itself."""
+    return torch.quantize_per_tensor(x.float(), float(scale.reshape(-1)[0]), int(zp) - 128 + int(sym),
+                                     torch.qint8).int_repr()
+
+
+def quant_act_fmo_mo(x, cvn, cv, quant_stepsize, quant_zero_point, sym: int):
+    """qa_fmo_mo_qfunc (linear.py:1073-1083): clamp first, then round.  The operands are the
+    module's tensors (``cvs``, ``quant_stepsize``, ``quant_zero_point``), so torch's type
+    promotion decides the compute dtype exactly as in the reference."""
+    r = torch.round(x.clamp(cvn, cv) / quant_stepsize - quant_zero_point) - (128 - int(sym))
+    return r.to(torch.int8)
+
+
+def _wrap_int8(r: torch.Tensor) -> torch.Tensor:
+    """float -> int8 the way the reference's ``.to(torch.int8)`` behaves on x86 for integer values
+    a little outside the range: two's-complement wrap (128 -> -128), made explicit."""
+    r = torch.where(r > 127, r - 256, r)
+    r = torch.where(r < -128, r + 256, r)
+    return r.to(torch.int8)
+
+
+def quant_act_dyn_max(x: torch.Tensor, dim: int = -1, nbits: int = 8):
+    """qa_dynamic_max_qfunc (linear.py:1085-1100) for either reduce dimension: -1 = per token
+    (scale [M,1]), -2 = per input channel over the tokens (scale [1,K]).  Returns (q, scale)."""
+    amax = x.abs().max(dim=dim, keepdim=True)[0]
+    levels = 2 ** (nbits - 1) - 1
+    scale = amax.clamp(min=1e-5).div(levels)
+    return _wrap_int8(torch.round(x / scale)), scale
+
+
+def quant_act_fake_zero_shift(x: torch.Tensor, input_zp: torch.Tensor, nbits: int = 8):
+    """qa_dyn_max_fake_zero_shift (linear.py:1102-1113): one dynamic scale for the whole tensor,
+    amax / (127 - zp), codes shifted by zp.  input_zp: the module's 0-dim int tensor.
+    Returns (q, input_scale 0-dim in x's dtype)."""
+    amax = x.abs().max()
+    levels = 2 ** (nbits - 1) - 1 - input_zp
+    scale = amax.clamp(min=1e-5) / levels
+    xq = torch.round(x / scale) + input_zp
+    return _wrap_int8(xq), scale
+
+
 # ------------------------------------------------------------------------------------------
 # Weight quantizers
 # ------------------------------------------------------------------------------------------
@@ -136,12 +193,13 @@ def int_gemm(a_i8: torch.Tensor, w_i8: torch.Tensor) -> torch.Tensor:
 
 
 def epilogue_ref(acc: torch.Tensor, input_scale: torch.Tensor, w_scale: torch.Tensor,
-                 bias: torch.Tensor | None, org_dtype=torch.float16):
-    """iaddmm_int plain branch (linear.py:1185-1188) then ``.to(org_dtype)`` (:1338)."""
+                 bias: torch.Tensor | None, org_dtype=torch.float16, acc_dtype=torch.float16):
+    """iaddmm_int plain branch (linear.py:1185-1188) then ``.to(org_dtype)`` (:1338).  acc_dtype is
+    fp16 in from_fms_mo (:777) and fp32 by default in from_torch_iW (:955)."""
     y = acc.float() * (input_scale * w_scale).to(torch.float16)
     if bias is not None:
         y = y + bias
-    return y.to(torch.float16).to(org_dtype)
+    return y.to(acc_dtype).to(org_dtype)
 
 
 def epilogue_f32(acc, input_scale, w_scale, bias, out_dtype):
@@ -199,6 +257,175 @@ def deploy_forward(x, bufs):
     y = (y + bias) if bias is not None else y
     y = y.to(torch.float16).reshape(tuple(x.shape[:-1]) + (bufs["weight"].shape[0],))
     return {"q_x": q_x, "input_scale": input_scale, "acc": acc, "y": y.to(org_dtype)}
+
+
+def deploy_prepare_general(weight, bias, w_cv, a_cv=None, a_cvn=None, sym_act=True, act_scale=None,
+                           alpha=0.5, use_PT_native_Qfunc=False, use_dynamic_max_act_Qfunc=False):
+    """QLinearINT8Deploy.from_fms_mo (linear.py:717-920) for every activation-quantizer branch:
+    dynamic max (-1 / -2), fake zero shift (1..64), PT-native static, fms_mo-formula static.
+    ``sym_act`` is the reference's useSymAct (:765-769: 'sym' in qa_mode or qa_mode in
+    pertokenmax / max).  a_cv / a_cvn: the activation quantizer's clip_val / clip_valn tensors
+    (shape [1], fp32 as the quantizers register them) -- default 8.0 / -8.0 as at :793-794.
+    Returns the module state as a dict (buffers under the reference's names plus the flags)."""
+    w_dtype = weight.dtype
+    sym = int(bool(sym_act))
+    w_levels, a_levels = 2**8 - 2, 2**8 - 1 - sym
+    a_cv = torch.tensor(8.0) if a_cv is None else a_cv
+    a_cvn = torch.tensor(-8.0) if a_cvn is None else a_cvn
+    sq = torch.tensor([1.0], dtype=w_dtype)
+    if act_scale is not None:
+        sq = smoothq_scale_deploy(weight, act_scale, torch.tensor([alpha], dtype=torch.float32))
+    input_scale = torch.tensor(1.0)
+    w_scale = w_cv * 2 / w_levels
+    st = {"useSymAct": sym, "useDynMaxQfunc": use_dynamic_max_act_Qfunc,
+          "usePTnativeQfunc": use_PT_native_Qfunc, "use_fake_zero_shift": False,
+          "cvs": [a_cv, a_cvn, w_cv], "acc_dtype": torch.float16}
+    if use_dynamic_max_act_Qfunc in [-1, -2]:
+        input_zp = torch.tensor(128 - sym)
+    elif 0 < use_dynamic_max_act_Qfunc < 65:
+        st["use_fake_zero_shift"] = True
+        input_zp = torch.tensor(use_dynamic_max_act_Qfunc)
+    elif use_PT_native_Qfunc:
+        input_scale = torch.tensor([(a_cv - a_cvn) / a_levels])
+        input_zp = torch.round(-a_cvn / input_scale)
+    else:
+        quant_scale = a_levels / torch.tensor([a_cv - a_cvn])
+        quant_stepsize = 1.0 / quant_scale
+        quant_zero_point = torch.round(a_cvn * quant_scale)
+        input_scale = quant_stepsize
+        input_zp = -quant_zero_point
+        w_scale = 1.0 / (w_levels / (w_cv * 2))
+        st.update(quant_scale=quant_scale, quant_stepsize=quant_stepsize,
+                  quant_zero_point=quant_zero_point)
+    input_zp = input_zp.to(torch.int)
+    w_int = torch.round((weight * sq).t() / w_scale).clamp(-w_levels / 2, w_levels / 2).t().to(torch.int)
+    if sym:
+        corr_term_int = 0
+        if st["use_fake_zero_shift"]:
+            corr_term_int = input_zp * (w_int.sum(dim=1))
+    else:
+        corr_term_int = (input_zp - 128) * (w_int.sum(dim=1))
+    corr_term = corr_term_int * w_scale.float() * input_scale.float()
+    new_bias = (bias.float() - corr_term) if bias is not None else -corr_term
+    if st["use_fake_zero_shift"]:
+        new_bias = new_bias + corr_term
+    if not torch.is_tensor(new_bias):  # symmetric, no bias: -0 broadcast to the bias shape
+        new_bias = torch.zeros(weight.shape[0]) + new_bias
+    if new_bias.dim() == 0:
+        new_bias = new_bias.expand(weight.shape[0]).clone()
+    st.update(weight=w_int.to(torch.int8), w_scale=w_scale, smoothq_scale=sq, input_scale=input_scale,
+              input_zp=input_zp, corr_term=corr_term, bias=new_bias.to(w_dtype))
+    return st
+
+
+def deploy_from_torch_iW(w_int, bias, a_cv: float, a_cvn: float, w_cv: float, zero_shift,
+                         use_PT_native_Qfunc=True, acc_dtype=torch.float):
+    """QLinearINT8Deploy.from_torch_iW (linear.py:923-1023): the module state built from integer
+    weights (any dtype holding integers), Python-float clip values and the per-channel
+    ``zero_shift`` (list / tensor of integer row sums, or one float)."""
+    st = {"useSymAct": 0, "useDynMaxQfunc": False, "usePTnativeQfunc": use_PT_native_Qfunc,
+          "use_fake_zero_shift": False, "cvs": [a_cv, a_cvn, w_cv], "acc_dtype": acc_dtype}
+    if use_PT_native_Qfunc:
+        input_scale = torch.Tensor([(a_cv - a_cvn) / (2**8 - 1)])
+        input_zp = torch.round(-a_cvn / input_scale).to(torch.int)
+        w_scale = torch.Tensor([w_cv * 2 / (2**8 - 2)])
+    else:
+        quant_scale = (2**8 - 1) / torch.Tensor([a_cv - a_cvn])
+        quant_stepsize = 1.0 / quant_scale
+        quant_zero_point = torch.round(a_cvn * quant_scale)
+        input_scale = quant_stepsize
+        input_zp = -quant_zero_point
+        w_scale = 1.0 / ((2**8 - 2) / torch.Tensor([w_cv * 2]))
+        st.update(quant_scale=quant_scale, quant_stepsize=quant_stepsize,
+                  quant_zero_point=quant_zero_point)
+    zero_s = torch.Tensor(list(zero_shift)) if not isinstance(zero_shift, (int, float)) else torch.Tensor([zero_shift])
+    corr_term = (input_zp - 128) * zero_s * w_scale * input_scale
+    new_bias = (bias - corr_term).to(acc_dtype) if bias is not None else -corr_term.to(acc_dtype)
+    st.update(weight=w_int.to(torch.int8), w_scale=w_scale, smoothq_scale=torch.tensor([1.0]),
+              input_scale=input_scale, input_zp=input_zp, corr_term=corr_term, zero_shift=zero_s,
+              bias=new_bias)
+    return st
+
+
+def deploy_forward_general(x, st, chunk_size=100000, truncate_lsb=0, max_acc_bits=32):
+    """QLinearINT8Deploy.forward + iaddmm_int (linear.py:1309-1338, 1115-1188) on a module state
+    from deploy_prepare_general / deploy_from_torch_iW: every activation-quantizer branch, the
+    serial chunk loop (:1142-1175) and the plain branch (:1177-1188).  Integer products are exact.
+    Returns {q_x, input_scale, acc, y}."""
+    org_dtype = x.dtype
+    x2 = x.reshape(-1, x.shape[-1])
+    sq = st["smoothq_scale"]
+    if torch.all(sq != 1).item():
+        x2 = x2 / sq
+    input_scale = st["input_scale"]
+    if st["useDynMaxQfunc"] in [-1, -2]:
+        q_x, input_scale = quant_act_dyn_max(x2, st["useDynMaxQfunc"])
+    elif st["use_fake_zero_shift"]:
+        q_x, input_scale = quant_act_fake_zero_shift(x2, st["input_zp"])
+    elif st["usePTnativeQfunc"]:
+        q_x = quant_act_static_raw(x2, input_scale, st["input_zp"], st["useSymAct"])
+    else:
+        q_x = quant_act_fmo_mo(x2, st["cvs"][1], st["cvs"][0], st["quant_stepsize"],
+                               st["quant_zero_point"], st["useSymAct"])
+    w = st["weight"]
+    bias, w_scale = st["bias"], st["w_scale"]
+    K = x2.shape[1]
+    if K > chunk_size:
+        acc = torch.zeros((x2.shape[0], w.shape[0]), dtype=torch.int)
+        trun_scale = 1
+        lo, hi = -(1 << (max_acc_bits - 1)), (1 << (max_acc_bits - 1)) - 1
+        for k0 in range(0, K, chunk_size):
+            p = int_gemm(q_x[:, k0:k0 + chunk_size].contiguous(), w[:, k0:k0 + chunk_size].contiguous())
+            if max_acc_bits < 32:
+                p = p.clamp(lo, hi)
+            if truncate_lsb > 0:
+                trun_scale = 1 << truncate_lsb
+                p = torch.bitwise_right_shift(p + (1 << (truncate_lsb - 1)), truncate_lsb)
+            acc += p
+        y = (acc * (trun_scale * input_scale * w_scale) + bias).to(st["acc_dtype"])
+    else:
+        acc = int_gemm(q_x, w)
+        updated_bias = bias
+        if st["use_fake_zero_shift"]:
+            updated_bias = bias - input_scale * st["corr_term"]
+        y = (acc.float() * (input_scale * w_scale).to(torch.float16) + updated_bias).to(st["acc_dtype"])
+    y = y.reshape(tuple(x.shape[:-1]) + (w.shape[0],)).to(org_dtype)
+    return {"q_x": q_x, "input_scale": input_scale, "acc": acc, "y": y}
+
+
+def i8i32nt_from_fms_mo(weight, bias, a_cv, a_cvn, w_cv):
+    """QLinearCublasI8I32NT.from_fms_mo (linear.py:1429-1489): asymmetric (quint8) activations with
+    the zero-point correction folded into the bias.  The weight integers are what the per-channel
+    max quantizer returns with ``dequantize = False`` (:1466-1469; QmaxPerChSTE.forward,
+    fms_mo/quant/quantizers.py:3190-3224): the fake-quantized fp32 weights divided by the scale
+    again, cast to int8 -- a truncating cast of a quotient that is an integer up to one rounding."""
+    input_scale = (a_cv - a_cvn) / (2**8 - 1)
+    input_zp = torch.round(-a_cvn / input_scale).to(torch.int)
+    scale = w_cv * 2 / (2**8 - 2)
+    w_scale = scale.float()
+    wf = weight.float()
+    fq = torch.fake_quantize_per_channel_affine(wf, scale.float(), torch.zeros_like(scale).float(),
+                                                axis=0, quant_min=-127, quant_max=127).to(wf.dtype)
+    w_i8 = (fq.t() / scale).t().to(torch.int8)
+    corr_term = (w_scale * input_scale * (input_zp - 128) * w_i8.sum(dim=1)).to(bias.dtype)
+    return {"weight": w_i8, "w_scale": w_scale, "input_scale": input_scale, "input_zp": input_zp,
+            "bias": bias - corr_term, "input_dtype": torch.quint8}
+
+
+def i8i32nt_forward(x, st):
+    """QLinearCublasI8I32NT.forward / QLinearCutlassI8I32NT.forward (linear.py:1491-1535,
+    1549-1583): static quantizer (uint8 codes shifted by -128, or int8 clamped to +-127), exact
+    integer GEMM, ``input_scale * w_scale * acc + bias``.  Returns {q_x, acc, y}."""
+    in_dtype = x.dtype
+    if st["input_dtype"] == torch.quint8:
+        q = torch.clamp((x / st["input_scale"] + st["input_zp"]).round(), 0, 255)
+        q = (q.to(torch.int16) - 128).to(torch.int8)
+    else:
+        q = torch.clamp((x / st["input_scale"] + st["input_zp"]).round(), -127, 127).to(torch.int8)
+    tar_shape = x.shape[:-1] + (st["weight"].shape[0],)
+    acc = int_gemm(q.reshape(-1, q.shape[-1]).contiguous(), st["weight"]).reshape(tar_shape)
+    y = st["input_scale"] * st["w_scale"] * acc + st["bias"]
+    return {"q_x": q, "acc": acc, "y": y.to(in_dtype)}
 
 
 def deploy_forward_fp(x, bufs):
@@ -325,6 +552,52 @@ def int8train_forward(x, weight, bias=None, lsb_trun_bits=0, chunk_size=64, max_
     if bias is not None:
         out = out + bias.to(org_dtype)
     return out, x_i8, w_i8, acc
+
+
+def to_fp8_saturated(x, orig_dtype):
+    """to_fp8_saturated, e4m3, emulate=True (fms_mo/quant/quantizers.py:5316-5333)."""
+    x = x.clamp(min=-1 * E4M3_MAX, max=E4M3_MAX)
+    return x.to(torch.float8_e4m3fn).to(orig_dtype)
+
+
+def fp8_max_to_scale(x_max, orig_dtype):
+    """max_to_scale, e4m3 (quantizers.py:5335-5351): 448 / clamp(x_max, 1e-12) in x_max's dtype,
+    clamped to the fp16 maximum for fp16."""
+    scale = torch.empty_like(x_max, dtype=orig_dtype)
+    res = E4M3_MAX / torch.clamp(x_max, min=1e-12)
+    if orig_dtype is torch.float16:
+        res = torch.clamp(res, max=torch.finfo(torch.float16).max)
+    scale.copy_(res)
+    return scale
+
+
+def to_fp8_scaled(x, granularity="tensor"):
+    """to_fp8_scaled / to_fp8_scaled_perCh / to_fp8_scaled_perToken, e4m3, emulate=True
+    (quantizers.py:5353-5421).  granularity: 'tensor' | 'perCh' (max over dim 1, weights [N,K]) |
+    'perToken' (max over dim -1).  Returns (fake-quantized x in x's dtype, scale)."""
+    orig_dtype = x.dtype
+    if granularity == "tensor":
+        x_max = torch.max(torch.abs(x))
+    elif granularity == "perCh":
+        x_max = torch.max(torch.abs(x), dim=1, keepdim=True)[0]
+    else:
+        x_max = torch.max(torch.abs(x), dim=-1, keepdim=True)[0]
+    x_scale = fp8_max_to_scale(x_max, orig_dtype)
+    x_scaled = x * x_scale
+    return (to_fp8_saturated(x_scaled, orig_dtype) / x_scale).to(orig_dtype), x_scale
+
+
+def to_fp8_forward(x, q_mode="fp8_e4m3_sat", perCh=None, perToken=False):
+    """class to_fp8, forward (quantizers.py:5423-5488), emulate=True."""
+    if perCh:
+        return to_fp8_scaled(x, "perCh")[0]
+    if perToken:
+        return to_fp8_scaled(x, "perToken")[0]
+    if "_sat" in q_mode:
+        return to_fp8_saturated(x, x.dtype)
+    if "_scale" in q_mode:
+        return to_fp8_scaled(x, "tensor")[0]
+    return None
 
 
 def fp8_quant_static(x: torch.Tensor, scale: torch.Tensor):

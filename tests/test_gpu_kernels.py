@@ -499,30 +499,47 @@ def test_gemm_fp8_integer_valued_is_exact(dev, shape):
     assert torch.equal(y16.cpu(), exact[:16])
 
 
-@pytest.mark.parametrize("bias_dt", [None, torch.float16, torch.float32])
+@pytest.mark.parametrize("bias_dt", [None, torch.float16, torch.bfloat16, torch.float32])
 def test_gemm_dq_with_columns_cut_off_the_last_round(dev, bias_dt):
-    """1100 x 14080 outputs are 275 tiles of 256 x 256: 19 tiles over a full round of 256, so the
-    library runs the last 1024 columns as a second, small GEMM.  Scales, bias and output of both
-    parts must line up: int8 bit-exact against the reference epilogue, e4m3 exact on small
-    integers with per-column scales that are powers of two.  Without a bias the kernel adds 0.0
-    like the reference, whose deploy module always holds a bias buffer (linear.py:897-911): a
+    """2048 x 25600 outputs are 800 tiles of 256 x 256: three full rounds over 256 compute units
+    and 32 tiles more, so the library runs the last 1024 columns as a second, small GEMM.
+    Per-column scales, bias (every dtype) and output of both parts must line up: int8 bit-exact
+    against the reference epilogue (fp16 and fp32 accumulator dtype) and the fp32 forms, e4m3 exact
+    on small integers with per-column scales that are powers of two.  Without a bias the kernel adds
+    0.0 like the reference, whose deploy module always holds a bias buffer (linear.py:897-911): a
     product of -0.0 comes out as +0.0."""
-    M, N, Kd = 1100, 14080, 128
+    from fms_mo_amd import _lib as L
+
+    M, N, Kd = 2048, 25600, 128
+    if L.load().fmsmo_gemm_tail_columns(M, N, Kd) != 1024:
+        pytest.skip("tuning overrides switch the cut off")
+    assert L.load().fmsmo_gemm_tail_columns(1100, 14080, Kd) == 0   # 128 x 256 tiles: nothing to cut
     a, w = _rand_i8((M, Kd), 51), _rand_i8((N, Kd), 52)
     s_a = (torch.rand(M, 1, generator=gen(53)) * 0.05 + 1e-3).half()
     s_w = (torch.rand(N, generator=gen(54)) * 1e-3 + 1e-5).float()
     bias = None if bias_dt is None else (torch.randn(N, generator=gen(55)) * 0.01).to(bias_dt)
-    ref = O.epilogue_ref(O.int_gemm(a, w), s_a, s_w, torch.zeros(N) if bias is None else bias, torch.float16)
-    y = K().gemm_i8_dq(a.to(dev), w.to(dev), s_a.float().to(dev), s_w.to(dev),
-                       None if bias is None else bias.to(dev), out_dtype=torch.float16, exact_ref=True)
+    bz = torch.zeros(N) if bias is None else bias
+    acc = O.int_gemm(a, w)
+    ad, wd, sad, swd = a.to(dev), w.to(dev), s_a.float().to(dev), s_w.to(dev)
+    bd = None if bias is None else bias.to(dev)
+    ref = O.epilogue_ref(acc, s_a, s_w, bz, torch.float16)
+    y = K().gemm_i8_dq(ad, wd, sad, swd, bd, out_dtype=torch.float16, exact_ref=True)
     assert torch.equal(y.cpu().view(torch.int16), ref.view(torch.int16))
+    ref32 = O.epilogue_ref(acc, s_a, s_w, bz, torch.float32, acc_dtype=torch.float32)
+    y32 = K().gemm_i8_dq(ad, wd, sad, swd, bd, out_dtype=torch.float32, exact_ref=True)
+    assert torch.equal(y32.cpu().view(torch.int32), ref32.view(torch.int32))
+    ref_ma = ((s_a.float() * s_w) * acc + bz.float()).to(torch.bfloat16)
+    y_ma = K().gemm_i8_dq(ad, wd, sad, swd, bd, out_dtype=torch.bfloat16, epilogue=L.EPI_F32_MULADD)
+    assert torch.equal(y_ma.cpu().view(torch.int16), ref_ma.view(torch.int16))
     a8 = torch.randint(-4, 5, (M, Kd), generator=gen(56)).float()
     w8 = torch.randint(-4, 5, (N, Kd), generator=gen(57)).float()
     s8 = torch.tensor([0.5, 1.0, 2.0, 4.0])[torch.randint(0, 4, (N,), generator=gen(58))]
     one = torch.ones(M)
+    b8 = None if bias is None else bias.float().to(bias_dt)
     y8 = K().gemm_fp8_dq(a8.to(torch.float8_e4m3fn).to(dev), w8.to(torch.float8_e4m3fn).to(dev), one.to(dev),
-                         s8.to(dev), None, out_dtype=torch.float32)
-    assert torch.equal(y8.cpu(), (a8 @ w8.t()) * s8[None, :])
+                         s8.to(dev), None if b8 is None else b8.to(dev), out_dtype=torch.float32)
+    exact8 = (a8 @ w8.t()).double() * s8[None, :].double() + (0 if b8 is None else b8.double())
+    assert torch.equal(y8.cpu(), exact8.float())
 
 
 # ------------------------------------------------------------------------- chunked accumulation

@@ -313,7 +313,7 @@ def test_operator_twins_agree_with_the_kernels_on_shapes(dev):
     torch.library.opcheck(torch.ops.fms_mo_amd.quant_act_i8_pertoken.default, (x, sm, torch.float16, False),
                           test_utils=("test_schema", "test_faketensor"))
     torch.library.opcheck(torch.ops.fms_mo_amd.gemm_i8_dq.default,
-                          (q, w, s, ws, None, torch.float16, True, False),
+                          (q, w, s, ws, None, torch.float16, 0, False),
                           test_utils=("test_schema", "test_faketensor"))
     torch.library.opcheck(torch.ops.fms_mo_amd.quant_act_i8_static.default, (x, 0.05, 128, 0),
                           test_utils=("test_schema", "test_faketensor"))

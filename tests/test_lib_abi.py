@@ -24,6 +24,7 @@ def test_header_declares_the_expected_entry_points():
               "fmsmo_grouped_gemm_i8_dq", "fmsmo_quant_weight_i8", "fmsmo_absmax_cols",
               "fmsmo_quant_act_i8_mulscale", "fmsmo_zero_shift_bias", "fmsmo_quant_i8_affine",
               "fmsmo_bmm_i8_dq", "fmsmo_bmm_fp8_dq", "fmsmo_gemm_i8_dq_ws", "fmsmo_gemm_fp8_dq_ws", "fmsmo_gemm_i8_dq_noalloc",
+              "fmsmo_gemm_tail_columns", "fmsmo_quant_act_i8_static_t", "fmsmo_quant_act_i8_dynamic", "fmsmo_fake_quant_fp8",
               "fmsmo_gemm_workspace_bytes", "fmsmo_decode_linear_i8", "fmsmo_decode_linear_fp8", "fmsmo_decode_linear_ok", "fmsmo_debug_clock_probe", "fmsmo_gemm_plan", "fmsmo_abi_version", "fmsmo_status_str", "fmsmo_last_error"]:
         assert s in syms
 
@@ -130,6 +131,14 @@ def test_gemm_plan_is_host_logic():
     assert K.gemm_plan(2048, 4096, 12800) == (RS, 256, 128, 1)
     assert K.gemm_plan(2048, 6144, 4096) == (RS, 256, 192, 1)
     assert K.gemm_plan(2048, 25600, 4096) == (RS, 256, 256, 1)
+    # a nearly empty last round of 256 x 256 tiles is cut off and run as a second GEMM
+    tail = _lib.load().fmsmo_gemm_tail_columns
+    if not os.environ.get("FMSMO_TAIL_SPLIT"):
+        assert tail(2048, 25600, 4096) == 1024 and tail(2048, 25600, 128) == 1024   # 800 tiles
+        assert tail(1100, 14080, 128) == 0        # 128 x 256 tiles win here: no 256 x 256 round to cut
+        assert tail(4096, 28672, 4096) == 0       # 1792 tiles: full rounds
+        assert tail(4096, 8448, 8192) == 0        # one column tile only: too narrow to pay
+        assert tail(16, 25600, 4096) == 0         # decode kernel
     # decode and batched decode
     assert K.gemm_plan(1, 4096, 4096)[0] == _lib.PLAN_DECODE
     assert K.gemm_plan(16, 28672, 4096)[0] == _lib.PLAN_DECODE

@@ -1,0 +1,357 @@
+"""Pins of the oracle's static / asymmetric deploy branches, the cuBLAS / CUTLASS style modules and
+the FP8 emulation quantizers -- by what the mathematics fixes, not by retyping the formulas:
+
+  * every deploy branch is an affine quantizer followed by an exact integer product, so its output
+    must equal the float64 product of the DEQUANTIZED operands, ((q - z) s_x) . (w s_w)^T + b with
+    z the zero point the codes were stored against, to within the roundings of the epilogue.  A
+    wrong sign of the correction term, a zero point off by 128, a row sum over the wrong dimension
+    or a correction that is not folded into the bias each move the result by far more than that;
+  * special cases: zero point 128 makes the correction vanish; the fms_mo clamp-then-round formula
+    and the round-then-clamp formula agree inside the clip range away from ties and saturate to the
+    same end codes outside; torch.quantize_per_tensor is the library routine for the PT-native one;
+    a per-column quantizer is the per-token quantizer of the transposed tensor;
+  * FP8 emulation: the scale re-derived with exact rationals and explicit roundings to the dtype's
+    grid, the cast against the enumerated e4m3 grid with ties to even.
+"""
+from fractions import Fraction
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import qlinear_oracle as O
+
+
+def gen(seed):
+    return torch.Generator().manual_seed(seed)
+
+
+def _layer(N=48, K=96, seed=0, dtype=torch.float16):
+    g = gen(seed)
+    W = (0.05 * torch.randn(N, K, generator=g)).to(dtype)
+    b = (0.1 * torch.randn(N, generator=g)).to(dtype)
+    x = (torch.randn(40, K, generator=g) * 1.5 + 0.7).to(dtype)   # off-centre: asymmetric range
+    w_cv = W.abs().amax(dim=1).float()
+    return W, b, x, w_cv
+
+
+def _dequantized_product(q_x, z, s_x, w_i8, s_w, bias):
+    """float64 ((q - z) s_x) . (w s_w)^T + b."""
+    xd = (q_x.double() - z) * s_x.double()
+    wd = w_i8.double() * s_w.double().reshape(-1, 1)
+    return xd @ wd.t() + (0 if bias is None else bias.double())
+
+
+# --------------------------------------------------------------------------- static branches
+@pytest.mark.parametrize("pt_native", [True, False])
+@pytest.mark.parametrize("with_bias", [True, False])
+def test_static_asymmetric_deploy_equals_dequantized_product(pt_native, with_bias):
+    W, b, x, w_cv = _layer(seed=1)
+    a_cv, a_cvn = torch.tensor([5.5]), torch.tensor([-3.25])
+    st = O.deploy_prepare_general(W, b if with_bias else None, w_cv, a_cv, a_cvn, sym_act=False,
+                                  use_PT_native_Qfunc=pt_native)
+    out = O.deploy_forward_general(x, st)
+    zp = int(st["input_zp"])
+    assert 0 < zp < 255 and zp != 128                       # genuinely asymmetric
+    assert st["corr_term"].abs().max() > 0.05               # and the correction matters
+    # codes are stored minus 128: the real zero point of the int8 codes is zp - 128
+    ref = _dequantized_product(out["q_x"], zp - 128, st["input_scale"], st["weight"], st["w_scale"],
+                               b if with_bias else None)
+    # epilogue roundings: fp16 scale product (2^-11 relative on acc * scale), bias stored in fp16,
+    # fp16 result
+    tol = 2.0 ** -10 * (ref.abs() + st["corr_term"].abs().double() + 1.0)
+    assert ((out["y"].double() - ref).abs() <= tol).all()
+    # the quantizer itself: x within half a step of its dequantized code inside the clip range
+    xin = x.float().clamp(a_cvn, a_cv)
+    deq = (out["q_x"].float() - (zp - 128)) * st["input_scale"]
+    assert ((deq - xin).abs() <= 0.5001 * st["input_scale"] + 1e-6).all()
+    assert out["q_x"].min() == -128 or x.min() > a_cvn      # the range end codes are reachable
+    # sign check made explicit: dropping or flipping the correction is far outside the tolerance
+    wrong = ref + 2 * st["corr_term"].double()
+    assert ((out["y"].double() - wrong).abs() > tol).any()
+
+
+def test_zero_point_128_makes_the_correction_vanish():
+    W, b, x, w_cv = _layer(seed=2)
+    # PT-native: zp = round(-cvn / ((cv - cvn) / 255)); cv = 127, cvn = -128 gives exactly 128
+    st = O.deploy_prepare_general(W, b, w_cv, torch.tensor([127.0]), torch.tensor([-128.0]),
+                                  sym_act=False, use_PT_native_Qfunc=True)
+    assert int(st["input_zp"]) == 128
+    assert torch.count_nonzero(st["corr_term"]) == 0
+    assert torch.equal(st["bias"], b)
+
+
+def test_fms_mo_formula_against_round_then_clamp_and_library_routine():
+    """qa_fmo_mo_qfunc clamps then rounds; qa_raw_qfunc rounds then clamps; quantize_per_tensor
+    multiplies by the reciprocal.  On values strictly inside the clip range whose quotient is not
+    within 1e-3 of a tie all three name the same integer; outside the range the first two give the
+    end codes."""
+    a_cv, a_cvn = torch.tensor([6.0]), torch.tensor([-2.0])
+    W, b, _, w_cv = _layer(seed=3)
+    st_f = O.deploy_prepare_general(W, b, w_cv, a_cv, a_cvn, sym_act=False, use_PT_native_Qfunc=False)
+    st_p = O.deploy_prepare_general(W, b, w_cv, a_cv, a_cvn, sym_act=False, use_PT_native_Qfunc=True)
+    assert int(st_f["input_zp"]) == int(st_p["input_zp"]) == 64      # -(-2)/(8/255) = 63.75 -> 64
+    x = (torch.rand(4000, generator=gen(4)) * 12 - 5).half().reshape(50, 80)
+    q_f = O.quant_act_fmo_mo(x, a_cvn, a_cv, st_f["quant_stepsize"], st_f["quant_zero_point"], 0)
+    q_r = O.quant_act_static_raw(x, st_p["input_scale"], st_p["input_zp"], 0)
+    q_t = O.quant_act_pt_native(x, st_p["input_scale"], st_p["input_zp"], 0)
+    quot = x.double() / (8.0 / 255.0)
+    frac = (quot - torch.floor(quot) - 0.5).abs()
+    inside = (x.float() > -2.0) & (x.float() < 6.0) & (frac > 1e-3)
+    assert inside.sum() > 1000
+    assert torch.equal(q_f[inside], q_r[inside]) and torch.equal(q_r[inside], q_t[inside])
+    # the integer is round(x / step) + 64 - 128 by plain arithmetic
+    expect = torch.round(quot[inside]) + 64 - 128
+    assert torch.equal(q_f[inside].double(), expect)
+    below, above = x.float() <= -2.0, x.float() >= 6.0
+    assert (q_f[below] == -128).all() and (q_r[below] == -128).all()
+    assert (q_f[above] == 127).all() and (q_r[above] == 127).all()
+
+
+def test_per_column_dynamic_quantizer_is_the_per_token_one_transposed():
+    x = (torch.randn(37, 64, generator=gen(5)) * 2).half()
+    q2, s2 = O.quant_act_dyn_max(x, -2)
+    q1, s1, _ = O.quant_act_pertoken_i8(x.t().contiguous())
+    assert s2.shape == (1, 64)
+    assert torch.equal(q2, q1.t()) and torch.equal(s2.reshape(-1), s1.reshape(-1))
+    qa, sa = O.quant_act_dyn_max(x, -1)
+    qb, sb, _ = O.quant_act_pertoken_i8(x)
+    assert torch.equal(qa, qb) and torch.equal(sa, sb)
+
+
+def test_per_column_deploy_forward_on_a_square_layer():
+    """With reduce dim -2 the reference multiplies the accumulator column n by input_scale[n] (the
+    [1,K] scale broadcasts against [M,N], so K must equal N): restated literally, and checked to be
+    that product and not the per-token one."""
+    W, b, _, w_cv = _layer(N=64, K=64, seed=6)
+    x = (torch.randn(24, 64, generator=gen(7)) * torch.linspace(0.2, 3, 64)).half()
+    st = O.deploy_prepare_general(W, b, w_cv, use_dynamic_max_act_Qfunc=-2)
+    out = O.deploy_forward_general(x, st)
+    # (the scale product is an fp16 subnormal here, so its fp16 rounding is part of the definition)
+    sc = (out["input_scale"].float().reshape(1, -1) * st["w_scale"].float()).half().double()
+    lit = out["acc"].double() * sc + b.double()
+    assert ((out["y"].double() - lit).abs() <= 2.0 ** -10 * (lit.abs() + 1)).all()
+
+
+@pytest.mark.parametrize("zp", [1, 17, 64])
+def test_fake_zero_shift_equals_dequantized_product(zp):
+    W, b, x, w_cv = _layer(seed=8)
+    st = O.deploy_prepare_general(W, b, w_cv, use_dynamic_max_act_Qfunc=zp)
+    assert st["use_fake_zero_shift"] and int(st["input_zp"]) == zp
+    # the correction stays out of the stored bias: (b - corr) + corr in fp32, i.e. b up to the
+    # fp32 rounding of the intermediate
+    assert ((st["bias"].float() - b.float()).abs() <= 2.0 ** -22 * st["corr_term"].abs() + 2.0 ** -11 * b.abs().float()).all()
+    out = O.deploy_forward_general(x, st)
+    s = out["input_scale"]
+    assert s.dim() == 0 and s.dtype == torch.float16
+    amax = x.abs().max().double()
+    assert abs(float(s) - float(amax) / (127 - zp)) <= 2.0 ** -11 * float(s)
+    assert out["q_x"].max() <= 127 and out["q_x"].min() >= zp - (127 - zp) - 1
+    ref = _dequantized_product(out["q_x"], zp, s, st["weight"], st["w_scale"], b)
+    # corr_term is stored with input_scale = 1 and multiplied by the dynamic scale in the forward
+    corr = float(s) * st["corr_term"].abs().double()
+    tol = 2.0 ** -10 * (ref.abs() + corr + 1.0)
+    assert ((out["y"].double() - ref).abs() <= tol).all()
+    deq = (out["q_x"].float() - zp) * float(s)
+    # (the quotient is rounded to fp16 before rint: up to 2^-5 of a step on top of the half step)
+    assert ((deq - x.float()).abs() <= 0.54 * float(s) + 1e-6).all()
+
+
+# ------------------------------------------------------------------------------ from_torch_iW
+@pytest.mark.parametrize("pt_native", [True, False])
+def test_from_torch_iW_equals_dequantized_product_and_matches_from_fms_mo(pt_native):
+    W, b, x, _ = _layer(seed=9)
+    w_cv = float(W.abs().max())
+    a_cv, a_cvn = 5.0, -2.5
+    st_ref = O.deploy_prepare_general(W, b, torch.tensor([w_cv]), torch.tensor([a_cv]),
+                                      torch.tensor([a_cvn]), sym_act=False, use_PT_native_Qfunc=pt_native)
+    w_int = st_ref["weight"]
+    zero_shift = w_int.sum(dim=1).float().tolist()
+    st = O.deploy_from_torch_iW(w_int.float(), b.float(), a_cv, a_cvn, w_cv, zero_shift,
+                                use_PT_native_Qfunc=pt_native)
+    assert st["bias"].dtype == torch.float32 and st["acc_dtype"] == torch.float32
+    assert int(st["input_zp"]) == int(st_ref["input_zp"])
+    torch.testing.assert_close(st["input_scale"], st_ref["input_scale"].float(), rtol=1e-6, atol=0)
+    torch.testing.assert_close(st["corr_term"], st_ref["corr_term"], rtol=1e-5, atol=1e-7)
+    out = O.deploy_forward_general(x, st)
+    assert out["y"].dtype == x.dtype
+    zp = int(st["input_zp"])
+    ref = _dequantized_product(out["q_x"], zp - 128, st["input_scale"], w_int, st["w_scale"], b.float())
+    tol = 2.0 ** -10 * (ref.abs() + st["corr_term"].abs().double() + 1.0)
+    assert ((out["y"].double() - ref).abs() <= tol).all()
+    # the same layer through from_fms_mo (fp16 accumulator dtype, fp16 bias) agrees to fp16 rounding
+    out_ref = O.deploy_forward_general(x, st_ref)
+    assert torch.equal(out["q_x"], out_ref["q_x"]) and torch.equal(out["acc"], out_ref["acc"])
+    torch.testing.assert_close(out["y"].float(), out_ref["y"].float(), rtol=4e-3, atol=4e-3)
+    # a scalar zero shift (symmetric checkpoint: no shift) broadcasts
+    st0 = O.deploy_from_torch_iW(w_int.float(), None, a_cv, a_cvn, w_cv, 0.0, use_PT_native_Qfunc=pt_native)
+    assert torch.count_nonzero(st0["corr_term"]) == 0 and torch.count_nonzero(st0["bias"]) == 0
+
+
+def test_acc_dtype_fp32_skips_the_fp16_rounding_of_the_result():
+    acc = torch.tensor([[12345, -7]], dtype=torch.int32)
+    s_a, s_w = torch.tensor([[3.1e-3]]), torch.tensor([1.7e-3, 2.0e-3])
+    y32 = O.epilogue_ref(acc, s_a, s_w, None, torch.float32, acc_dtype=torch.float32)
+    y16 = O.epilogue_ref(acc, s_a, s_w, None, torch.float32, acc_dtype=torch.float16)
+    assert y32.dtype == y16.dtype == torch.float32
+    assert torch.equal(y16, y32.half().float()) and not torch.equal(y16, y32)
+    sc = (s_a * s_w).half().double()
+    assert torch.equal(y32.double(), (acc.double() * sc).float().double())
+
+
+# -------------------------------------------------------------------------- chunked deploy loop
+@pytest.mark.parametrize("cfg", [(32, 0, 32), (64, 3, 32), (32, 2, 12)])
+def test_chunk_loop_of_iaddmm_int_equals_the_chunked_kernel_semantics(cfg):
+    chunk, t, bits = cfg
+    W, b, x, w_cv = _layer(seed=10)
+    st = O.deploy_prepare_general(W, b, w_cv, use_dynamic_max_act_Qfunc=-1)
+    out = O.deploy_forward_general(x, st, chunk_size=chunk, truncate_lsb=t, max_acc_bits=bits)
+    acc_k = O.chunk_matmul_i8(out["q_x"], st["weight"], None, chunk, t, bits)
+    assert torch.equal(out["acc"].to(torch.int64) << t, acc_k.to(torch.int64))
+    if t == 0 and bits == 32:
+        assert torch.equal(out["acc"], O.int_gemm(out["q_x"], st["weight"]))
+
+
+# ------------------------------------------------------------------- cuBLAS / CUTLASS modules
+def test_i8i32nt_module_equals_dequantized_product():
+    W, b, x, w_cv = _layer(seed=11)
+    a_cv, a_cvn = torch.tensor([5.0]), torch.tensor([-3.0])
+    st = O.i8i32nt_from_fms_mo(W, b, a_cv, a_cvn, w_cv)
+    out = O.i8i32nt_forward(x, st)
+    zp = int(st["input_zp"])
+    assert out["q_x"].dtype == torch.int8 and 0 < zp < 255
+    ref = _dequantized_product(out["q_x"], zp - 128, st["input_scale"], st["weight"], st["w_scale"], b)
+    assert ((out["y"].double() - ref).abs() <= 2.0 ** -10 * (ref.abs() + 1.0) + 2e-3).all()
+    # weights: levels of the per-channel fake quantizer
+    # (the truncating cast may land one level low where (q * s) / s rounds below q)
+    fq = O.fake_quant_weight_perch(W.float(), w_cv)
+    lvl = torch.round(fq.double() / st["w_scale"].double()[:, None])
+    diff = lvl - st["weight"].double()
+    assert (diff * lvl.sign() >= 0).all() and diff.abs().max() <= 1 and (diff != 0).float().mean() < 0.1
+    # symmetric branch: clamp to +-127, zero point added before the rounding
+    st_s = dict(st, input_dtype=torch.qint8, input_zp=torch.tensor([0], dtype=torch.int), bias=b)
+    out_s = O.i8i32nt_forward(x, st_s)
+    assert out_s["q_x"].abs().max() <= 127
+    ref_s = _dequantized_product(out_s["q_x"], 0, st["input_scale"], st["weight"], st["w_scale"], b)
+    assert ((out_s["y"].double() - ref_s).abs() <= 2.0 ** -10 * (ref_s.abs() + 1.0) + 2e-3).all()
+
+
+# ----------------------------------------------------------------------------- FP8 emulation
+def _grid(dtype):
+    """(significand bits incl. hidden, min normal exponent) of the dtype's value grid."""
+    return {torch.float16: (11, -14), torch.bfloat16: (8, -126), torch.float32: (24, -126)}[dtype]
+
+
+def _rne(v: Fraction, dtype) -> Fraction:
+    """Round an exact rational to the dtype's grid, ties to even, no overflow handling."""
+    if v == 0:
+        return v
+    p, emin = _grid(dtype)
+    sign = -1 if v < 0 else 1
+    a = abs(v)
+    e = 0
+    while a >= 2:
+        a /= 2; e += 1
+    while a < 1:
+        a *= 2; e -= 1
+    e = max(e, emin)
+    quantum = Fraction(2) ** (e - (p - 1))
+    n = abs(v) / quantum
+    fl = n.numerator // n.denominator
+    rem = n - fl
+    if rem > Fraction(1, 2) or (rem == Fraction(1, 2) and fl % 2 == 1):
+        fl += 1
+    return sign * fl * quantum
+
+
+E4M3_VALUES = sorted({float(torch.tensor([c], dtype=torch.uint8).view(torch.float8_e4m3fn).float())
+                      for c in range(256) if (c & 0x7f) != 0x7f})
+
+
+def _e4m3_nearest_even(v: float) -> float:
+    """Nearest value of the enumerated e4m3 grid, ties to the code with an even mantissa."""
+    arr = np.array(E4M3_VALUES)
+    i = int(np.searchsorted(arr, v))
+    cands = [arr[j] for j in (i - 1, i) if 0 <= j < len(arr)]
+    best = min(cands, key=lambda c: abs(Fraction(float(c)) - Fraction(v)))
+    ties = [c for c in cands if abs(Fraction(float(c)) - Fraction(v)) == abs(Fraction(float(best)) - Fraction(v))]
+    if len(ties) == 2:
+        def mant_even(c):
+            code = int(torch.tensor([float(c)]).to(torch.float8_e4m3fn).view(torch.uint8))
+            return (code & 1) == 0
+        best = [c for c in ties if mant_even(c)][0]
+    return float(best)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+def test_fp8_scale_rederived_with_exact_rationals(dtype):
+    amax = torch.tensor([448.0, 1.0, 3.14159, 0.0123, 1000.0, 7e-4, 0.0, 6e-8, 2.0 ** -20]).to(dtype)
+    s = O.fp8_max_to_scale(amax, dtype)
+    assert s.dtype == dtype
+    fmax16 = Fraction(65504)
+    for a, got in zip(amax.tolist(), s.tolist()):
+        floor = _rne(Fraction(1e-12), dtype) if dtype != torch.float16 else Fraction(0)
+        c = max(Fraction(a), floor)
+        if c == 0:
+            expect = float(fmax16)                       # fp16: 448 / 0 = inf, clamped
+        else:
+            r = _rne(1 / c, dtype)
+            if dtype == torch.float16 and r > fmax16:
+                expect = float(fmax16)                   # reciprocal overflows to inf
+            else:
+                e = _rne(r * 448, dtype)
+                expect = float(min(e, fmax16)) if dtype == torch.float16 else float(e)
+        assert got == expect, (dtype, a, got, expect)
+    # reciprocal-then-multiply is NOT the correctly rounded quotient: the distinction is live
+    t = (torch.rand(5000, generator=gen(12)) * 100 + 1e-2).to(dtype)
+    assert (O.fp8_max_to_scale(t, dtype) != (448.0 / t.double()).to(dtype)).any()
+
+
+def test_fp8_saturating_cast_on_the_whole_grid_midpoints_and_overflow():
+    vals = torch.tensor(E4M3_VALUES)
+    for dtype in (torch.float16, torch.bfloat16, torch.float32):
+        assert torch.equal(O.to_fp8_saturated(vals.to(dtype), dtype).float(), vals)   # idempotent
+    pos = [v for v in E4M3_VALUES if v >= 0]
+    mids = torch.tensor([(a + b) / 2 for a, b in zip(pos[:-1], pos[1:])])
+    got = O.to_fp8_saturated(mids, torch.float32)
+    expect = torch.tensor([_e4m3_nearest_even(float(m)) for m in mids])
+    assert torch.equal(got, expect)
+    assert torch.equal(O.to_fp8_saturated(-mids, torch.float32), -expect)
+    big = torch.tensor([449.0, 464.0, 465.0, 1e6, float("inf")])
+    assert torch.equal(O.to_fp8_saturated(big, torch.float32), torch.full((5,), 448.0))   # clamp first
+    assert torch.equal(O.to_fp8_saturated(-big, torch.float32), torch.full((5,), -448.0))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("gran", ["tensor", "perCh", "perToken"])
+def test_fp8_scaled_quantizers_rederived_elementwise(dtype, gran):
+    x = (torch.randn(6, 40, generator=gen(13)) * torch.tensor([[0.01], [1.0], [30.0], [0.3], [5.0], [100.0]])).to(dtype)
+    y, s = O.to_fp8_scaled(x, gran)
+    assert y.dtype == dtype and y.shape == x.shape
+    assert s.shape == (() if gran == "tensor" else (6, 1))
+    s_full = s.expand(6, 1) if gran != "tensor" else s.reshape(1, 1).expand(6, 1)
+    amax = x.abs().amax() if gran == "tensor" else x.abs().amax(dim=1)
+    for m in range(6):
+        sm = Fraction(float(s_full[m, 0]))
+        a = float(amax if gran == "tensor" else amax[m])
+        assert float(sm) == float(O.fp8_max_to_scale(torch.tensor(a, dtype=dtype), dtype))
+        for k in range(0, 40, 3):
+            xs = _rne(Fraction(float(x[m, k])) * sm, dtype)
+            xs = max(min(xs, Fraction(448)), Fraction(-448))
+            f8 = _e4m3_nearest_even(float(xs))
+            expect = float(_rne(Fraction(f8) / sm, dtype))
+            assert float(y[m, k]) == expect, (m, k)
+    # relative error of an e4m3 grid with 3 mantissa bits, plus the roundings in the dtype
+    big = x.abs().float() * s_full.float() >= 2.0 ** -6
+    rel = ((y.float() - x.float()).abs() / x.abs().float().clamp(min=1e-30))[big]
+    assert rel.max() <= 2.0 ** -4 + 2.0 ** -7
+
+
+def test_to_fp8_module_dispatch():
+    x = (torch.randn(5, 32, generator=gen(14)) * 600).half()
+    assert torch.equal(O.to_fp8_forward(x, "fp8_e4m3_sat"), O.to_fp8_saturated(x, x.dtype))
+    assert O.to_fp8_forward(x, "fp8_e4m3_sat").abs().max() == 448
+    assert torch.equal(O.to_fp8_forward(x, "fp8_e4m3_scale"), O.to_fp8_scaled(x, "tensor")[0])
+    assert torch.equal(O.to_fp8_forward(x, "fp8_e4m3_scale_perCh", perCh=5), O.to_fp8_scaled(x, "perCh")[0])
+    assert torch.equal(O.to_fp8_forward(x, "fp8_e4m3_scale_perToken", perToken=True),
+                       O.to_fp8_scaled(x, "perToken")[0])
