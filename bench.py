@@ -9,9 +9,10 @@ Weights are quantized once, before the timed region (they are constants of the d
 
 Prints ONE JSON line (see the keys below).  `value` is 2*M*N*K summed over the four linears
 divided by the wall time of a step; `roofline` prices the GEMM kernel alone (HIP-event time of
-its launches inside the timed region) against the published dense INT8 MFMA peak; `cpu_baseline`
-is the CPU restatement of the reference's QLinear forward timed on the host cores on a bounded
-sample of the same workload.
+its launches inside the timed region) against the published dense INT8 MFMA peak; `roofline_fp8`
+and `roofline_decode` carry the other two parts of the metric (e4m3 GEMMs against the FP8 MFMA
+peak, M <= 16 decode launches against the HBM peak); `cpu_baseline` is the CPU restatement of the
+reference's QLinear forward timed on the host cores on a bounded sample of the same workload.
 """
 import argparse
 import json
@@ -76,11 +77,172 @@ def cpu_baseline(torch, layers, budget_s=30.0):
     times.sort()
     med = times[len(times) // 2]
     ops = sum(2.0 * rows * layer["W_cpu"].shape[0] * layer["W_cpu"].shape[1] for layer in layers)
-    return {"value": ops / med / 1e12, "unit": "TOPS", "cores": torch.get_num_threads(),
-            "kind": "port",
-            "sample": f"QLinear fake-quant forward (act Q/dQ, per-call weight Q/dQ, fp16 F.linear) of all four "
-                      f"linears, first {rows} of 4096 tokens, median of {len(times)} passes, "
-                      f"{med:.2f} s each"}
+    res = {"value": ops / med / 1e12, "unit": "TOPS", "cores": torch.get_num_threads(),
+           "kind": "port",
+           "sample": f"QLinear fake-quant forward (act Q/dQ, per-call weight Q/dQ, fp16 F.linear) of all four "
+                     f"linears, first {rows} of 4096 tokens, median of {len(times)} passes, "
+                     f"{med:.2f} s each"}
+    # second leg: the deployed module's CPU fallback, QLinearINT8Deploy.forward with iaddmm_FP
+    # (fms_mo/modules/linear.py:1190-1211, 1309-1338): weights already int8, per-token quantizer,
+    # matmul on the dequantized operands in fp16 -- needs every buffer in x's dtype
+    bufs = []
+    for layer in layers:
+        b = O.deploy_prepare(layer["W_cpu"], layer["b_cpu"], layer["W_cpu"].abs().amax(dim=1).float(),
+                             layer["act_scale_cpu"], 0.5)
+        bufs.append({k: (v.half() if v.is_floating_point() else v) for k, v in b.items()})
+
+    def fp_pass():
+        for layer, b in zip(layers, bufs):
+            O.deploy_forward_fp(layer["x_cpu"][:rows], b)
+
+    fp_pass()
+    t_fp = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        fp_pass()
+        t_fp.append(time.perf_counter() - t0)
+    t_fp.sort()
+    res["deploy_iaddmm_FP"] = {"value": ops / t_fp[1] / 1e12, "unit": "TOPS",
+                               "sample": f"QLinearINT8Deploy forward with the iaddmm_FP fallback, same "
+                                         f"{rows} tokens and linears, median of 3 passes, {t_fp[1]:.2f} s each"}
+    return res
+
+GRANITE_8B = [("qkv", 4096, 6144), ("o", 4096, 4096), ("gate_up", 4096, 25600), ("down", 12800, 4096)]
+
+
+def time_events(torch, fn, iters=30, warm=5):
+    """Average HIP-event time (ms) of fn over iters eager calls on the current stream."""
+    for _ in range(warm):
+        fn()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(iters):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / iters
+
+
+def fp8_rooflines(torch, K, dev):
+    """The FP8 half of the metric: e4m3 x e4m3 GEMMs with fp32 accumulation and the dequantizing
+    epilogue (per-token activation scale, bf16 out) against the 5.0 PFLOP/s dense FP8 peak, on the
+    Llama-3-8B shapes at M = 4096 (per-channel weight scales) and the Granite-3-8B-like shapes at
+    M = 2048 (per-tensor weight scale).  Operands are real quantizer outputs (codes over the whole
+    +-448 range), timed over eager launches with HIP events, the GEMM alone."""
+    from fms_mo_amd import _lib as L
+
+    g = torch.Generator().manual_seed(3)
+    out = {"peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s", "bound": "mfma", "dtype": "e4m3 x e4m3 -> fp32"}
+    clk = torch.zeros(6, dtype=torch.int64, device=dev)
+    for label, M, shapes, per_channel in (("llama3_8b_M4096", M_TOKENS, LLAMA3_8B, True),
+                                          ("granite_8b_M2048", 2048, GRANITE_8B, False)):
+        per, tot_ms, tot_ops = {}, 0.0, 0.0
+        for name, k, n in shapes:
+            x = torch.randn(M, k, generator=g).bfloat16().to(dev)
+            w = (0.02 * torch.randn(n, k, generator=g)).to(dev)
+            ws = (w.abs().amax(dim=1) / 448).float() if per_channel else (w.abs().amax() / 448).reshape(1).float()
+            w8 = (w / (ws[:, None] if per_channel else ws)).clamp(-448, 448).to(torch.float8_e4m3fn)
+            q, s = K.quant_act_fp8_pertoken(x, L.FP8_LINEAR)
+            K.clock_probe(clk)
+            ms = time_events(torch, lambda: K.gemm_fp8_dq(q, w8, s, ws, None, out_dtype=torch.bfloat16), iters=20, warm=4)
+            K.clock_probe(None)
+            ops = 2.0 * M * k * n
+            tot_ms += ms
+            tot_ops += ops
+            tf = ops / (ms * 1e-3) / 1e12
+            per[name] = {"ms": round(ms, 4), "tflops": round(tf, 1), "frac": round(tf / PEAK_FP8_TFLOPS, 4),
+                         "core_clock_mhz": round(K.core_clock_mhz(clk))}
+            del x, w, w8, q
+        tf = tot_ops / (tot_ms * 1e-3) / 1e12
+        out[label] = {"per_shape": per, "achieved": round(tf, 1), "frac": round(tf / PEAK_FP8_TFLOPS, 4)}
+    return out
+
+
+def decode_rooflines(torch, K, dev, m_list=(1, 4, 16), ops=("i8", "fp8"), copies_mib=300):
+    """The decode half of the metric: y = dequant(q_x . W_q^T) for M in {1, 4, 16} tokens on the four
+    Llama-3-8B weight shapes, int8 and e4m3 weights, against the 8 TB/s HBM peak.  Algorithmic bytes
+    per launch: N K (weights) + M K (codes) + 2 M N (bf16 out) + 4 N (scales).  Weight copies
+    totalling > 256 MiB are rotated so the memory-side cache cannot hold them.  `us` is device time
+    (the launches replayed from a HIP graph); `eager_us` is the time per call of the same launches
+    issued one by one from Python through the operator wrapper (host launch cost included)."""
+    from fms_mo_amd import _lib as L
+
+    out = {"peak": PEAK_HBM_GBS, "unit": "GB/s", "bound": "hbm"}
+    for name, k, n in LLAMA3_8B:
+        wbytes = k * n
+        copies = max(3, (copies_mib * 1024 * 1024 + wbytes - 1) // wbytes)
+        wsc = torch.rand(n, device=dev) * 1e-3
+        for op in ops:
+            if op == "i8":
+                ws_q = [torch.randint(-127, 128, (n, k), dtype=torch.int8, device=dev) for _ in range(copies)]
+            else:  # e4m3 weights whose codes cover the format's range (per-channel-scaled Gaussian)
+                ws_q = [torch.randn(n, k, device=dev).mul_(448.0 / 4.5).clamp_(-448, 448).to(torch.float8_e4m3fn)
+                        for _ in range(copies)]
+            for M in m_list:
+                x = torch.randn(M, k, device=dev).bfloat16()
+                if op == "i8":
+                    q, s = K.quant_act_i8_pertoken(x)
+                    run = lambda w: K.gemm_i8_dq(q, w, s, wsc, None, out_dtype=torch.bfloat16, exact_ref=True)  # noqa: E731
+                else:
+                    q, s = K.quant_act_fp8_pertoken(x, L.FP8_LINEAR)
+                    run = lambda w: K.gemm_fp8_dq(q, w, s, wsc, None, out_dtype=torch.bfloat16)  # noqa: E731
+                side = torch.cuda.Stream()
+                reps, replays = 3, 5
+                with torch.cuda.stream(side):
+                    for w in ws_q:
+                        run(w)
+                    torch.cuda.synchronize()
+                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    e0.record()
+                    for _ in range(reps):
+                        for w in ws_q:
+                            run(w)
+                    e1.record()
+                    torch.cuda.synchronize()
+                    eager_ms = e0.elapsed_time(e1) / (reps * copies)
+                    graph = torch.cuda.CUDAGraph()
+                    with torch.cuda.graph(graph, stream=side):
+                        for _ in range(reps):
+                            for w in ws_q:
+                                run(w)
+                    graph.replay()
+                    torch.cuda.synchronize()
+                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    e0.record()
+                    for _ in range(replays):
+                        graph.replay()
+                    e1.record()
+                    torch.cuda.synchronize()
+                ms = e0.elapsed_time(e1) / (replays * reps * copies)
+                byts = wbytes + M * k + M * n * 2 + 4 * n
+                gbs = byts / (ms * 1e-3) / 1e9
+                out[f"{op}_M{M}_{name}"] = {"us": round(ms * 1e3, 2), "eager_us": round(eager_ms * 1e3, 2),
+                                            "GBps": round(gbs, 1), "frac": round(gbs / PEAK_HBM_GBS, 4)}
+                del graph
+            del ws_q
+    fr = [v["frac"] for kk, v in out.items() if isinstance(v, dict)]
+    out["frac_min"], out["frac_max"] = min(fr), max(fr)
+    return out
+
+
+def vendor_int_mm(torch, K, layers):
+    """The vendor library's int8 GEMM (torch._int_mm -> hipBLASLt, int32 out, no epilogue) on the
+    SAME quantized operands as the headline step, same event timing, beside this library's raw
+    int32 GEMM: how much of the distance to the published peak is the part's, not the kernel's."""
+    res = {}
+    for (name, k, n), L in zip(LLAMA3_8B, layers):
+        q, _ = K.quant_act_i8_pertoken(L["x"], L["smooth"])
+        wt = L["w"].t()
+        ops = 2.0 * M_TOKENS * k * n
+        try:
+            ms_v = time_events(torch, lambda: torch._int_mm(q, wt), iters=20, warm=4)
+            v = {"ms": round(ms_v, 4), "tops": round(ops / ms_v / 1e9, 1)}
+        except Exception as e:  # the vendor path is evidence, not a dependency
+            v = {"error": str(e)[:200]}
+        ms_o = time_events(torch, lambda: K.gemm_i8_i32(q, L["w"]), iters=20, warm=4)
+        res[name] = {"torch_int_mm": v, "fmsmo_gemm_i8_i32": {"ms": round(ms_o, 4), "tops": round(ops / ms_o / 1e9, 1)}}
+    return res
 
 
 def main():
@@ -89,7 +251,10 @@ def main():
     ap.add_argument("--steps", type=int, default=30)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--extras", action="store_true", help="also time FP8 GEMMs and decode shapes")
+    ap.add_argument("--no-fp8-decode", action="store_true",
+                    help="skip the FP8 GEMM and decode rooflines (profiling runs of the INT8 step)")
+    ap.add_argument("--extras", action="store_true",
+                    help="also time the vendor GEMM, mid-size batches, MoE, chunk-truncate, side kernels")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no collectives are part of it); "
@@ -180,6 +345,9 @@ def main():
                      "peak_at_measured_clock": round(peak_at_clock, 1),
                      "frac_at_measured_clock": round(achieved / peak_at_clock, 4)},
     }
+    if not args.no_fp8_decode:
+        out["roofline_fp8"] = fp8_rooflines(torch, K, dev)
+        out["roofline_decode"] = decode_rooflines(torch, K, dev)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(torch, layers)
     if args.extras:
@@ -188,24 +356,15 @@ def main():
 
 
 def extras(torch, K, dev, layers):
-    """FP8 GEMMs (Granite-3-8B-like shapes, M=2048), decode shapes (M in 1 .. 128), the Mixtral-style
-    grouped expert GEMMs and the chunk-truncate emulation; reported in addition to the headline
-    value."""
+    """The vendor GEMM on the same operands, mid-size batches (M in 32 .. 128), the Mixtral-style
+    grouped expert GEMMs, the chunk-truncate emulation and the side kernels; reported in addition
+    to the headline value and the FP8 / decode rooflines of the default run."""
     from fms_mo_amd import _lib as L
 
     res = {}
 
     def timeit(fn, iters=30, warm=5):
-        for _ in range(warm):
-            fn()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        torch.cuda.synchronize()
-        e0.record()
-        for _ in range(iters):
-            fn()
-        e1.record()
-        torch.cuda.synchronize()
-        return e0.elapsed_time(e1) / iters
+        return time_events(torch, fn, iters, warm)
 
     # the reference's CPU-runnable configuration (512 tokens through a 4096 -> 4096 linear) on the
     # GPU: SmoothQuant act-quant + int8 GEMM + dequant (512 x 4096 x 4096 splits its reduction in two)
@@ -249,83 +408,11 @@ def extras(torch, K, dev, layers):
     ms = timeit(cpu_sample_step)
     sample_ops = sum(2.0 * 2048 * k * n for _, k, n in LLAMA3_8B)
     res["cpu_baseline_sample_on_gpu_M2048"] = {"ms": round(ms, 4), "tops": round(sample_ops / ms / 1e9, 1)}
-    g = torch.Generator().manual_seed(3)
-    M = 2048
-    for name, k, n in [("qkv", 4096, 6144), ("o", 4096, 4096), ("gate_up", 4096, 25600), ("down", 12800, 4096)]:
-        x = torch.randn(M, k, generator=g).bfloat16().to(dev)
-        w = (0.02 * torch.randn(n, k, generator=g)).to(dev)
-        ws = (w.abs().amax() / 448).reshape(1).float()
-        w8 = (w / ws).clamp(-448, 448).to(torch.float8_e4m3fn)
-        q, s = K.quant_act_fp8_pertoken(x, L.FP8_LINEAR)
-        ms = timeit(lambda: K.gemm_fp8_dq(q, w8, s, ws, None, out_dtype=torch.bfloat16))
-        tf = 2.0 * M * k * n / (ms * 1e-3) / 1e12
-        res[f"fp8_M2048_{name}"] = {"ms": round(ms, 4), "tflops": round(tf, 1), "frac_peak": round(tf / PEAK_FP8_TFLOPS, 4)}
-    # the headline workload's four shapes with e4m3 operands (per-token act scale, per-channel weight scale)
-    tot_ms, fp8_clk = 0.0, torch.zeros(6, dtype=torch.int64, device=dev)
-    for name, k, n in LLAMA3_8B:
-        x = torch.randn(M_TOKENS, k, generator=g).bfloat16().to(dev)
-        w = (0.02 * torch.randn(n, k, generator=g)).to(dev)
-        ws = (w.abs().amax(dim=1) / 448).float()
-        w8 = (w / ws[:, None]).clamp(-448, 448).to(torch.float8_e4m3fn)
-        q, s = K.quant_act_fp8_pertoken(x, L.FP8_LINEAR)
-        K.clock_probe(fp8_clk)
-        ms = timeit(lambda: K.gemm_fp8_dq(q, w8, s, ws, None, out_dtype=torch.bfloat16))
-        K.clock_probe(None)
-        tot_ms += ms
-        tf = 2.0 * M_TOKENS * k * n / (ms * 1e-3) / 1e12
-        res[f"fp8_M4096_{name}"] = {"ms": round(ms, 4), "tflops": round(tf, 1), "frac_peak": round(tf / PEAK_FP8_TFLOPS, 4),
-                                    "core_clock_mhz": round(K.core_clock_mhz(fp8_clk))}
-        del x, w, w8, q
-    tf = sum(2.0 * M_TOKENS * k * n for _, k, n in LLAMA3_8B) / (tot_ms * 1e-3) / 1e12
-    res["fp8_M4096_all_four"] = {"ms": round(tot_ms, 4), "tflops": round(tf, 1), "frac_peak": round(tf / PEAK_FP8_TFLOPS, 4)}
-    # decode: rotate weight copies totalling > 256 MiB so the Infinity Cache cannot hold them;
-    # the launches are replayed from a HIP graph so that host launch overhead is not what is timed
-    for name, k, n in LLAMA3_8B:
-        wbytes = k * n
-        copies = max(3, (300 * 1024 * 1024 + wbytes - 1) // wbytes)
-        wsc = torch.rand(n, device=dev) * 1e-3
-        for op in ("i8", "fp8"):
-            if op == "i8":
-                ws_q = [torch.randint(-127, 128, (n, k), dtype=torch.int8, device=dev) for _ in range(copies)]
-                m_list = (1, 4, 16, 32, 64, 128)  # decode kernels up to 64 (K <= 4096), tiled / split-K above
-            else:  # e4m3 weights whose codes cover the format's range (per-channel-scaled Gaussian)
-                ws_q = [torch.randn(n, k, device=dev).mul_(448.0 / 4.5).clamp_(-448, 448).to(torch.float8_e4m3fn)
-                        for _ in range(copies)]
-                m_list = (1, 4, 16)
-            for M in m_list:
-                x = torch.randn(M, k, device=dev).bfloat16()
-                if op == "i8":
-                    q, s = K.quant_act_i8_pertoken(x)
-                    run = lambda w: K.gemm_i8_dq(q, w, s, wsc, None, out_dtype=torch.bfloat16, exact_ref=True)  # noqa: E731
-                else:
-                    q, s = K.quant_act_fp8_pertoken(x, L.FP8_LINEAR)
-                    run = lambda w: K.gemm_fp8_dq(q, w, s, wsc, None, out_dtype=torch.bfloat16)  # noqa: E731
-                side = torch.cuda.Stream()
-                reps, replays = 3, 5
-                with torch.cuda.stream(side):
-                    for w in ws_q:
-                        run(w)
-                    torch.cuda.synchronize()
-                    graph = torch.cuda.CUDAGraph()
-                    with torch.cuda.graph(graph, stream=side):
-                        for _ in range(reps):
-                            for w in ws_q:
-                                run(w)
-                    graph.replay()
-                    torch.cuda.synchronize()
-                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                    e0.record()
-                    for _ in range(replays):
-                        graph.replay()
-                    e1.record()
-                    torch.cuda.synchronize()
-                ms = e0.elapsed_time(e1) / (replays * reps * copies)
-                byts = wbytes + M * k + M * n * 2 + 4 * n
-                gbs = byts / (ms * 1e-3) / 1e9
-                res[f"decode_{op}_M{M}_{name}"] = {"us": round(ms * 1e3, 2), "GBps": round(gbs, 1),
-                                                  "frac_hbm": round(gbs / PEAK_HBM_GBS, 4)}
-                del graph
-            del ws_q
+    res["vendor"] = vendor_int_mm(torch, K, layers)
+    # batches between decode and the large GEMMs (decode kernels up to 64 tokens at K <= 4096,
+    # tiled / split-K above), int8, same protocol as the decode rooflines
+    mid = decode_rooflines(torch, K, dev, m_list=(32, 64, 128), ops=("i8",))
+    res.update({f"decode_{k_}": v for k_, v in mid.items() if isinstance(v, dict)})
     # the four int8 GEMMs of the headline workload on all-zero operands: nothing toggles in the
     # multipliers, the clock stays up, and the figure shows how far the kernel's instruction
     # stream goes when the power limit does not hold it back
