@@ -503,6 +503,14 @@ def extras(torch, K, dev, layers):
         ms = timeit(lambda: K.matmul_chunk(a, w, chunk_size=64, chunk_trun_bits=t), iters=10, warm=3)
         tops = 2.0 * m_e * I * H / (ms * 1e-3) / 1e12
         res[f"chunk64_trunc{t}_i8_w2_M{m_e}"] = {"ms": round(ms, 4), "tops": round(tops, 1), "frac_peak": round(tops / PEAK_INT8_TOPS, 4)}
+    # the same on 4096 rows (1024 tiles of 128 x 128: whole rounds over the compute units, where one
+    # expert's 1069 rows make 288 tiles for 256 units), chunk sizes 32 / 64 / 128
+    a4 = torch.randint(-127, 128, (4096, I), dtype=torch.int8, device=dev)
+    for cs in (32, 64, 128):
+        ms = timeit(lambda: K.matmul_chunk(a4, w, chunk_size=cs, chunk_trun_bits=7), iters=10, warm=3)
+        tops = 2.0 * 4096 * I * H / (ms * 1e-3) / 1e12
+        res[f"chunk{cs}_trunc7_i8_w2_M4096"] = {"ms": round(ms, 4), "tops": round(tops, 1), "frac_peak": round(tops / PEAK_INT8_TOPS, 4)}
+    del a4
     # the steps either side of the hot path: offline weight quantizer, SmoothQuant statistics, the
     # accelerator op's quantizer (HBM bound; inputs rotated so the Infinity Cache cannot hold them)
     # and the accelerator op end to end

@@ -257,7 +257,26 @@ static bool launch_chunk_tile(const ChunkArgs& c, const Epi& epi, hipStream_t st
   k.post = c.dl16 || k.t > 0 || c.max_acc_bits < 32;
   k.dl16 = c.dl16; k.tta = c.tta; k.c_in = c.c_in; k.ldc = c.ldd;
   dim3 grid((unsigned)(g.grid_m * g.grid_n)), block(256);
-  if (fast) {
+  // the schedules that round one block while the matrix unit multiplies the others: a chunk of one
+  // 64-byte stage (every operand type), of several stages or of one 32-byte k-step (int8)
+  const int sched = !fast ? 0 : c.chunk_bytes == 64 ? 1 : MMA != MMA_I8 ? 0 : c.chunk_bytes == 32 ? 3
+                    : c.chunk_bytes % 64 == 0 ? 2 : 0;
+#define LAUNCH_SCHED(SV)                                                                             \
+  {                                                                                                  \
+    ChunkTrunc<true, SV> kf{};                                                                       \
+    kf.chunk_ks = k.chunk_ks; kf.t = k.t; kf.round_bit = k.round_bit; kf.mask = k.mask;              \
+    kf.lo = k.lo; kf.hi = k.hi; kf.post = k.post; kf.dl16 = 0; kf.tta = 1;                           \
+    kf.c_in = k.c_in; kf.ldc = k.ldc;                                                                \
+    hipLaunchKernelGGL((gemm_tile_kernel<128, 128, 64, 4, 2, 2, MMA, 1, false, Epi, ChunkTrunc<true, SV>>), \
+                       grid, block, 0, st, g, epi, kf);                                              \
+  }
+  if (sched == 1) {
+    LAUNCH_SCHED(1)
+  } else if (sched == 2) {
+    if constexpr (MMA == MMA_I8) LAUNCH_SCHED(2)
+  } else if (sched == 3) {
+    if constexpr (MMA == MMA_I8) LAUNCH_SCHED(3)
+  } else if (fast) {
     ChunkTrunc<true> kf{};
     kf.chunk_ks = k.chunk_ks; kf.t = k.t; kf.round_bit = k.round_bit; kf.mask = k.mask;
     kf.lo = k.lo; kf.hi = k.hi; kf.post = k.post; kf.dl16 = 0; kf.tta = 1;

@@ -147,13 +147,22 @@ struct Mma<MMA_F32> {
 struct NoChunk {
   static constexpr bool enabled = false;
   static constexpr bool fast = false;
+  static constexpr bool one_stage = false;
 };
 // FAST = the common configuration (truncate-then-accumulate, no integer clamp, no DL16 clamp):
 // three vector ALU operations per accumulator element and chunk.
-template <bool FAST>
+// ONE_STAGE (with FAST) = the schedules that interleave the rounding of one 32x32 block with the
+// MFMAs of the others inside one wave (see the loop in gemm_tile_kernel): integers with any chunk
+// of one k-step or of whole LDS stages, floating point with a chunk of exactly one stage.
+// SCHED: 1 = a chunk is one stage, 2 = several whole stages, 3 = one k-step (integers only); each is
+// a kernel of its own (one kernel holding all three loops runs out of registers).
+template <bool FAST, int SCHED = 0>
 struct ChunkTrunc {
+  static_assert(FAST || SCHED == 0, "the interleaved schedules exist for the fast configuration only");
   static constexpr bool enabled = true;
   static constexpr bool fast = FAST;
+  static constexpr bool one_stage = SCHED != 0;
+  static constexpr int sched = SCHED;
   int chunk_ks;           // MFMA k-steps (32 bytes of K) per chunk
   int t, lo, hi;          // LSBs to round away; integer clamp range
   unsigned round_bit, mask;
@@ -543,6 +552,209 @@ __global__ __launch_bounds__(WGM* WGN * 64, (Chk::enabled && (OP == MMA_I8 || Ch
     issue_part(st, min(st, nk - 1) * BK, std::integral_constant<int, 0>{},
                std::integral_constant<int, NLD>{});
   asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"((NSTAGE - 2) * NLD) : "memory");
+  if constexpr (Chk::one_stage) {
+    // Chunk == stage: the fragments of all k-steps of a chunk are register resident (two sets:
+    // the stage being multiplied and the one being read), and the rounding of one 32x32 block is
+    // issued between the MFMAs of the others, so that one wave keeps both units busy.  With all
+    // MFMAs of a chunk issued before any rounding (the generic schedule) the units take turns, and
+    // only a second resident wave overlaps them -- which a problem with about one tile per compute
+    // unit does not have.
+    Frag ca[2][NKS][FM], cb[2][NKS][FN];
+    constexpr bool INT = std::is_same<Elem, int>::value;
+    auto stage_top = [&](int kt, auto par_c) {
+      constexpr int PAR = decltype(par_c)::value;
+      // stage kt + 1 has landed for every wave; its fragments go to the other register set, and
+      // the buffer of stage kt - 1 (last read a stage ago) is refilled with stage kt + 3
+      asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"((NSTAGE - 3) * NLD) : "memory");
+      const uint8_t* ls = &lds[0][0] + ((kt + 1) % NSTAGE) * STAGE_BYTES;
+#pragma unroll
+      for (int ks = 0; ks < NKS; ++ks) read_frags(ls, ks, ca[PAR ^ 1][ks], cb[PAR ^ 1][ks]);
+      issue_part((kt + NSTAGE - 1) % NSTAGE, min(kt + NSTAGE - 1, nk - 1) * BK,
+                 std::integral_constant<int, 0>{}, std::integral_constant<int, NLD>{});
+      __builtin_amdgcn_sched_barrier(0);
+    };
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks) read_frags(&lds[0][0], ks, ca[0][ks], cb[0][ks]);
+    if constexpr (INT) {
+      // Integers: with R the running sum (a multiple of 2^t) and r the rounding bit, a chunk's
+      // MFMAs started from C = R + r leave W = R + p + r, and (W & mask) = R + ((p + r) & mask) is
+      // the new running sum: ONE operation per element and chunk, W <- (W & mask) | r, turns the
+      // accumulator into the next chunk's C operand (low bits are zero, so OR adds r), and the
+      // matrix unit does the accumulation.  8 such operations take as long as one MFMA, and a
+      // chunk has 8 MFMAs and 64 elements per lane: the steady state below issues 8 operations in
+      // front of every MFMA.  Block b's k-steps are two MFMA slots apart, its 16 operations follow
+      // its second MFMA by a slot or more and are complete before its next first MFMA:
+      //   slot       0       1       2       3       4       5       6       7
+      //   rounding   b1 hi'  b2 lo'  b2 hi'  b3 lo'  b3 hi'  b0 lo   b0 hi   b1 lo    (' = previous chunk)
+      //   MFMA       b0 k0   b1 k0   b0 k1   b1 k1   b2 k0   b3 k0   b2 k1   b3 k1
+      // (a chunk of several stages rounds behind its last stage only; a chunk of one k-step has a
+      // table of its own below)
+      // Rounding an accumulator that holds C = R + r changes nothing, so the first chunk runs the
+      // same code.  An initial accumulator enters as its multiple of 2^t; its low bits are added
+      // at the end (adding a multiple of 2^t commutes with clearing the low bits).
+      static_assert(NKS == 2 && FM == 2 && FN == 2, "the slot table is written for 2 k-steps x 4 blocks");
+#pragma unroll
+      for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int jj = 0; jj < FN; ++jj)
+#pragma unroll
+          for (int v = 0; v < 16; ++v)
+            work[i][jj][v] = (int)(((unsigned)acc[i][jj][v] & chk.mask) | chk.round_bit);
+      // (one v_and_or_b32: the instruction takes a single scalar operand, so the rounding bit
+      // lives in a vector register)
+      unsigned rbv = chk.round_bit;
+      asm volatile("" : "+v"(rbv));
+      auto rnd = [&](auto b_c, auto h_c) {
+        constexpr int I = decltype(b_c)::value / FN, J = decltype(b_c)::value % FN, H = decltype(h_c)::value;
+#pragma unroll
+        for (int v = H * 8; v < H * 8 + 8; ++v)
+          work[I][J][v] = (int)(((unsigned)work[I][J][v] & chk.mask) | rbv);
+        __builtin_amdgcn_sched_barrier(0);
+      };
+      auto mm = [&](auto par_c, auto b_c, auto ks_c) {
+        constexpr int PAR = decltype(par_c)::value, KS = decltype(ks_c)::value;
+        constexpr int I = decltype(b_c)::value / FN, J = decltype(b_c)::value % FN;
+        work[I][J] = MM::mma(ca[PAR][KS][I], cb[PAR][KS][J], work[I][J]);
+        __builtin_amdgcn_sched_barrier(0);
+      };
+      typedef std::integral_constant<int, 0> I0;
+      typedef std::integral_constant<int, 1> I1;
+      typedef std::integral_constant<int, 2> I2;
+      typedef std::integral_constant<int, 3> I3;
+      if constexpr (Chk::sched == 1) {
+        // a chunk is one stage: the table as it stands
+        auto chunk_stage = [&](int kt, auto par_c) {
+          stage_top(kt, par_c);
+          rnd(I1{}, I1{}); mm(par_c, I0{}, I0{});
+          rnd(I2{}, I0{}); mm(par_c, I1{}, I0{});
+          rnd(I2{}, I1{}); mm(par_c, I0{}, I1{});
+          rnd(I3{}, I0{}); mm(par_c, I1{}, I1{});
+          rnd(I3{}, I1{}); mm(par_c, I2{}, I0{});
+          rnd(I0{}, I0{}); mm(par_c, I3{}, I0{});
+          rnd(I0{}, I1{}); mm(par_c, I2{}, I1{});
+          rnd(I1{}, I0{}); mm(par_c, I3{}, I1{});
+        };
+        int kt = 0;
+        for (; kt + 1 < nk; kt += 2) {
+          chunk_stage(kt, I0{});
+          chunk_stage(kt + 1, I1{});
+        }
+        if (kt < nk) chunk_stage(kt, I0{});
+      } else if constexpr (Chk::sched == 2) {
+        // a chunk is several whole stages: the roundings run only behind a chunk's last stage
+        // (slots 5 - 7 of that stage, slots 0 - 4 of the following one)
+        const int spc = chk.chunk_ks / NKS;
+        int phase = 0;  // stage index inside the chunk
+        auto chunk_stage = [&](int kt, auto par_c) {
+          stage_top(kt, par_c);
+          const bool prev_end = phase == 0, this_end = phase + 1 == spc;
+          phase = this_end ? 0 : phase + 1;
+          if (prev_end) rnd(I1{}, I1{});
+          mm(par_c, I0{}, I0{});
+          if (prev_end) rnd(I2{}, I0{});
+          mm(par_c, I1{}, I0{});
+          if (prev_end) rnd(I2{}, I1{});
+          mm(par_c, I0{}, I1{});
+          if (prev_end) rnd(I3{}, I0{});
+          mm(par_c, I1{}, I1{});
+          if (prev_end) rnd(I3{}, I1{});
+          mm(par_c, I2{}, I0{});
+          if (this_end) rnd(I0{}, I0{});
+          mm(par_c, I3{}, I0{});
+          if (this_end) rnd(I0{}, I1{});
+          mm(par_c, I2{}, I1{});
+          if (this_end) rnd(I1{}, I0{});
+          mm(par_c, I3{}, I1{});
+        };
+        int kt = 0;
+        for (; kt + 1 < nk; kt += 2) {
+          chunk_stage(kt, I0{});
+          chunk_stage(kt + 1, I1{});
+        }
+        if (kt < nk) chunk_stage(kt, I0{});
+      } else {
+        // a chunk is one k-step (32 bytes of K): 16 roundings per MFMA, the vector ALU is the
+        // bound (half the MFMA rate at best).  Per k-step: MFMA b0, round b2', MFMA b1, round b3',
+        // MFMA b2, round b0, MFMA b3, round b1 (' = of the previous k-step).
+        auto chunk_stage = [&](int kt, auto par_c) {
+          stage_top(kt, par_c);
+          [&]<int... KS>(std::integer_sequence<int, KS...>) {
+            (
+                [&] {
+                  typedef std::integral_constant<int, KS> CK;
+                  mm(par_c, I0{}, CK{}); rnd(I2{}, I0{}); rnd(I2{}, I1{});
+                  mm(par_c, I1{}, CK{}); rnd(I3{}, I0{}); rnd(I3{}, I1{});
+                  mm(par_c, I2{}, CK{}); rnd(I0{}, I0{}); rnd(I0{}, I1{});
+                  mm(par_c, I3{}, CK{}); rnd(I1{}, I0{}); rnd(I1{}, I1{});
+                }(),
+                ...);
+          }(std::make_integer_sequence<int, NKS>{});
+        };
+        int kt = 0;
+        for (; kt + 1 < nk; kt += 2) {
+          chunk_stage(kt, I0{});
+          chunk_stage(kt + 1, I1{});
+        }
+        if (kt < nk) chunk_stage(kt, I0{});
+      }
+      // the sum of the rounded chunks, plus the low bits of the initial accumulator (read again
+      // here: holding it in registers through the loop would cost 64 of them)
+#pragma unroll
+      for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int jj = 0; jj < FN; ++jj)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) {
+            unsigned low = 0;
+            if (chk.c_in) {
+              const int m = row_lo + wm * TM + i * 32 + (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3);
+              const int n = col_lo + wn * TN + jj * 32 + (lane & 31);
+              if (m < row_hi && n < g.N) low = (unsigned)((const int*)chk.c_in)[(int64_t)m * chk.ldc + n] & ~chk.mask;
+            }
+            acc[i][jj][v] = (int)(((unsigned)work[i][jj][v] & chk.mask) + low);
+          }
+    } else {
+      // Floating point: the rounding works on the bits of the chunk's own sum, which is then added
+      // in fp32 -- three operations per element (integer add, and, float add).  Block b's MFMAs
+      // start from C = 0; block b - 1 is folded into `acc` while they run.
+      Acc zero;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) zero[v] = 0;
+      auto fold = [&](auto b_c) {
+        constexpr int I = decltype(b_c)::value / FN, J = decltype(b_c)::value % FN;
+#pragma unroll
+        for (int v = 0; v < 16; ++v)
+          acc[I][J][v] += __uint_as_float((__float_as_uint(work[I][J][v]) + chk.round_bit) & chk.mask);
+      };
+      auto chunk_stage = [&](int kt, auto par_c) {
+        constexpr int PAR = decltype(par_c)::value;
+        stage_top(kt, par_c);
+        [&]<int... B>(std::integer_sequence<int, B...>) {
+          (
+              [&] {
+                constexpr int I = B / FN, J = B % FN;
+                work[I][J] = MM::mma(ca[PAR][0][I], cb[PAR][0][J], zero);
+#pragma unroll
+                for (int ks = 1; ks < NKS; ++ks)
+                  work[I][J] = MM::mma(ca[PAR][ks][I], cb[PAR][ks][J], work[I][J]);
+                __builtin_amdgcn_sched_barrier(0);
+                // block B - 1 of this chunk, or the last block of the previous one (zeros before
+                // the first chunk: a zero block folds to zero)
+                fold(std::integral_constant<int, (B + NMMA - 1) % NMMA>{});
+                __builtin_amdgcn_sched_barrier(0);
+              }(),
+              ...);
+        }(std::make_integer_sequence<int, NMMA>{});
+      };
+      int kt = 0;
+      for (; kt + 1 < nk; kt += 2) {
+        chunk_stage(kt, std::integral_constant<int, 0>{});
+        chunk_stage(kt + 1, std::integral_constant<int, 1>{});
+      }
+      if (kt < nk) chunk_stage(kt, std::integral_constant<int, 0>{});
+      fold(std::integral_constant<int, NMMA - 1>{});
+    }
+  } else {
   read_frags(&lds[0][0], 0, fa[0], fb[0]);
   {
     int kt = 0;
@@ -556,8 +768,9 @@ __global__ __launch_bounds__(WGM* WGN * 64, (Chk::enabled && (OP == MMA_I8 || Ch
       if (kt < nk) stage(kt, std::integral_constant<int, 0>{});
     }
   }
+  }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no DMA may be in flight when LDS is released
-  if constexpr (Chk::enabled) {
+  if constexpr (Chk::enabled && !Chk::one_stage) {
     if (ks_cnt != 0) finish_any();  // K ended inside a chunk
     if (!chk.tta) {
 #pragma unroll

@@ -301,8 +301,15 @@ __global__ __launch_bounds__(NW * 64) void gemv_kernel(GemvArgs g) {
 // 23.5 -> 16.1; 4 tokens 15.8 -> 12.5; K = 12800 as 10 waves x 10 steps, D = 5 -> 2: 20.1 ->
 // 11.3 at 4 tokens), also than keeping the activations in LDS with all 14 steps in flight (4
 // tokens: 14.6).
-template <int OP, int STEPS, int NW, int D, int MT = 1>
-__global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(GemvArgs g, int G) {
+// Work is dealt to the blocks in units of 8 weight rows (half an MFMA row group): block b owns the
+// half groups [b H / B, (b + 1) H / B) of the H = ceil(N / 8) there are, so that N = 6144 gives
+// each of 256 blocks 24 rows (whole groups only: 192 blocks of 32 rows, a quarter of the compute
+// units idle).  A block walks its rows in groups of 16; when the last one is a half group, its
+// upper 8 rows are neither loaded nor stored.
+// HALF = false: the host has checked that every block owns whole groups only (the loads of the
+// upper rows are then unconditional, which the register allocation of the long-row shapes needs).
+template <int OP, int STEPS, int NW, int D, int MT = 1, bool HALF = false>
+__global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(GemvArgs g, int halves) {
   static_assert(STEPS % D == 0, "pipeline depth must divide the steps per group");
   typedef typename std::conditional<OP == FMSMO_OP_I8, int, float>::type AccT;
   typedef AccT Acc4 __attribute__((ext_vector_type(4)));
@@ -312,9 +319,11 @@ __global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(GemvArgs g, int G)
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int r = lane & 15, kg = lane >> 4;
-  const int group0 = blockIdx.x * G;
-  const int ngroups = (g.N + 15) >> 4;
-  const int gcount = min(G, ngroups - group0);
+  const int h_lo = (int)(((int64_t)blockIdx.x * halves) / gridDim.x);
+  const int h_hi = (int)(((int64_t)(blockIdx.x + 1) * halves) / gridDim.x);
+  const int row_lo = h_lo * 8, row_hi = min(h_hi * 8, g.N);  // this block's weight rows
+  const int gcount = (h_hi - h_lo + 1) >> 1;                 // groups of 16 rows, the last maybe half
+  if (gcount <= 0) return;                                    // more blocks than half groups
   const int kwave = wave * (STEPS * 128);
 
   // activation fragments: lane (m = r, kg) holds x[m][kwave + s*128 + (h*4 + kg)*16 ...]
@@ -335,14 +344,19 @@ __global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(GemvArgs g, int G)
   // per-group row pointers, clamped (branch-free) for prefetch past the end and a ragged last group
   const int64_t kcol = kwave + dpos * 16;
   auto rowptr = [&](int gi, int half) {
-    const int row0 = min(group0 + min(gi, gcount - 1), ngroups - 1) * 16;
+    const int row0 = row_lo + min(gi, gcount - 1) * 16;
     return g.b + (int64_t)min(row0 + half * 8 + drow, g.N - 1) * g.ldb + kcol;
   };
+  // does group gi hold rows in its upper half? (uniform; a half group's upper rows belong to the
+  // next block: not loaded, their products are never stored)
+  auto is_full = [&](int gi) { return !HALF || row_lo + min(gi, gcount - 1) * 16 + 8 < row_hi; };
   const uint8_t* pc[2] = {rowptr(0, 0), rowptr(0, 1)};  // current group
   const uint8_t* pn[2] = {rowptr(1, 0), rowptr(1, 1)};  // next group
+  bool fullc = is_full(0), fulln = is_full(1);
   auto load_item = [&](bool next, int s, v4i (&w)[2]) {
     w[0] = __builtin_nontemporal_load((const v4i*)((next ? pn[0] : pc[0]) + s * 128));
-    w[1] = __builtin_nontemporal_load((const v4i*)((next ? pn[1] : pc[1]) + s * 128));
+    if (!HALF || (next ? fulln : fullc))
+      w[1] = __builtin_nontemporal_load((const v4i*)((next ? pn[1] : pc[1]) + s * 128));
   };
   // staging: row-major [16 rows][128 B], chunk c of row q stored at position c ^ (q % 8)
   const int wr0 = drow * 128 + ((dpos ^ drow) * 16);
@@ -351,6 +365,10 @@ __global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(GemvArgs g, int G)
   const int rd0 = r * 128 + ((kg ^ rr) * 16), rd1 = r * 128 + (((4 + kg) ^ rr) * 16);
 
   v4i wb[D][2];
+  if constexpr (HALF) {  // the upper halves stay unloaded for a block whose only group is a half one
+#pragma unroll
+    for (int j = 0; j < D; ++j) wb[j][1] = v4i{0, 0, 0, 0};
+  }
 #pragma unroll
   for (int j = 0; j < D; ++j) load_item(false, j, wb[j]);
 
@@ -363,7 +381,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(GemvArgs g, int G)
   // rows), so the group body exists twice: streaming (LAST = false) and draining (LAST = true).
   auto do_group = [&](auto last_tag, int gi) {
     constexpr bool LAST = decltype(last_tag)::value;
-    const int en = min((group0 + gi) * 16 + (int)((threadIdx.x >> 4) & 15), g.N - 1);
+    const int en = min(row_lo + gi * 16 + (int)((threadIdx.x >> 4) & 15), g.N - 1);
     const float ws = g.w_scale[g.w_stride ? en : 0];
     float bv = 0.f;
     if (g.bias) {
@@ -403,6 +421,10 @@ __global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(GemvArgs g, int G)
     if (!LAST) {
       pc[0] = pn[0], pc[1] = pn[1];
       pn[0] = rowptr(gi + 2, 0), pn[1] = rowptr(gi + 2, 1);
+      if constexpr (HALF) {
+        fullc = fulln;
+        fulln = is_full(gi + 2);
+      }
     }
     AccT* mine = &red[gi % NRED][wave][0];
 #pragma unroll
@@ -414,8 +436,8 @@ __global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(GemvArgs g, int G)
       AccT sum = red[gi % NRED][0][e];
 #pragma unroll
       for (int w = 1; w < NW; ++w) sum += red[gi % NRED][w][e];
-      const int n = (group0 + gi) * 16 + ((e >> 4) & 15), m = (e >> 8) * 16 + (e & 15);
-      if (n < g.N && m < g.M) {
+      const int n = row_lo + gi * 16 + ((e >> 4) & 15), m = (e >> 8) * 16 + (e & 15);
+      if (n < row_hi && m < g.M) {
         float out;
         if (g.epi == FMSMO_EPI_REF_F16) {
           const float sc = round_to<FMSMO_F16>(__fmul_rn(as_e, ws_e));
@@ -707,7 +729,7 @@ int fmsmo_gemv_dispatch(int op, const void* a, int64_t lda, const void* b, int64
   }
   // Streaming variant when the K steps of 128 split evenly over the waves of a block in one of
   // the instantiated (waves, steps per wave, loads in flight) shapes; other K use the generic
-  // kernel below.  One block per compute unit, each walking G consecutive groups: every block
+  // kernel below.  One block per compute unit, each walking its share of the row groups: every block
   // re-reads the activations and pays one memory latency before its stream starts, so fewer,
   // longer-lived blocks win (measured: N = 28672, K = 4096 runs 26.5 us at G = 1, 21.0 us at
   // G = 7).  FMSMO_GEMV_G overrides G for tuning.
@@ -722,17 +744,26 @@ int fmsmo_gemv_dispatch(int op, const void* a, int64_t lda, const void* b, int64
     // o 5.8 -> 5.5 / 6.6 -> 6.0, qkv 7.0 -> 7.0 / 8.2 -> 7.7, gate+up 21.8 -> 20.9 / 22.8 -> 21.8).
     if (M <= 16 && steps_total == 32) NW = 16;
     const int STEPS = NW ? steps_total / NW : 0;
-    int G = env_g > 0 ? env_g : (int)((groups + 255) / 256);
-    if (G > 64) G = 64;
-    dim3 grid((unsigned)((groups + G - 1) / G)), block(NW * 64);
+    // one block per compute unit, the rows dealt out in units of 8 (FMSMO_GEMV_G = groups of 16
+    // rows per block instead, for tuning)
+    const int halves = (int)((N + 7) / 8);
+    int64_t nblocks = env_g > 0 ? (groups + env_g - 1) / env_g : 256;
+    if (nblocks > halves) nblocks = halves;
+    const int G = halves;  // the kernels' second argument
+    // every block's share begins and ends on a group boundary
+    const bool whole_groups = halves % (2 * nblocks) == 0;
+    dim3 grid((unsigned)nblocks), block(NW * 64);
     bool handled = true;
-#define GEMV_STREAM(OPV, NWV, ST, DV)                                                             \
-  if (M <= 16) hipLaunchKernelGGL((gemv_stream_kernel<OPV, ST, NWV, DV>), grid, block, 0, st, g, G); \
+#define GEMV_STREAM_H(OPV, NWV, ST, DV, HV)                                                       \
+  if (M <= 16) hipLaunchKernelGGL((gemv_stream_kernel<OPV, ST, NWV, DV, 1, HV>), grid, block, 0, st, g, G); \
   else if constexpr (NWV == 8 && ST <= 8) {                                                        \
-    if (M <= 32) hipLaunchKernelGGL((gemv_stream_kernel<OPV, ST, NWV, DV, 2>), grid, block, 0, st, g, G); \
-    else if constexpr (ST <= 4) hipLaunchKernelGGL((gemv_stream_kernel<OPV, ST, NWV, DV, 4>), grid, block, 0, st, g, G); \
+    if (M <= 32) hipLaunchKernelGGL((gemv_stream_kernel<OPV, ST, NWV, DV, 2, HV>), grid, block, 0, st, g, G); \
+    else if constexpr (ST <= 4) hipLaunchKernelGGL((gemv_stream_kernel<OPV, ST, NWV, DV, 4, HV>), grid, block, 0, st, g, G); \
     else handled = false;                                                                          \
   } else handled = false
+#define GEMV_STREAM(OPV, NWV, ST, DV)                     \
+  if (whole_groups) { GEMV_STREAM_H(OPV, NWV, ST, DV, false); } \
+  else { GEMV_STREAM_H(OPV, NWV, ST, DV, true); }
 #define GEMV_SHAPES(OPV)                                            \
   switch (NW * 100 + STEPS) {                                       \
     case 801: GEMV_STREAM(OPV, 8, 1, 1); break;                     \
@@ -749,6 +780,7 @@ int fmsmo_gemv_dispatch(int op, const void* a, int64_t lda, const void* b, int64
     if (op == FMSMO_OP_I8) { GEMV_SHAPES(FMSMO_OP_I8) } else { GEMV_SHAPES(FMSMO_OP_E4M3) }
 #undef GEMV_SHAPES
 #undef GEMV_STREAM
+#undef GEMV_STREAM_H
     if (handled) return fmsmo_check_launch();
   }
   if (M > 16) return FMSMO_ERR_UNSUPPORTED;  // callers ask fmsmo_gemv_batch_ok first
