@@ -165,10 +165,16 @@ def decode_rooflines(torch, K, dev, m_list=(1, 4, 16), ops=("i8", "fp8"), copies
     per launch: N K (weights) + M K (codes) + 2 M N (bf16 out) + 4 N (scales).  Weight copies
     totalling > 256 MiB are rotated so the memory-side cache cannot hold them.  `us` is device time
     (the launches replayed from a HIP graph); `eager_us` is the time per call of the same launches
-    issued one by one from Python through the operator wrapper (host launch cost included)."""
+    issued one by one from Python through the operator wrapper (host launch cost included).
+    `read_only_floor_<shape>`: a launch that only reads the same weight bytes (256 x 1024 threads,
+    16-byte loads, nothing written), timed in the same graph over the same rotation -- what the
+    launch and the memory system leave to any kernel of that size; `floor_over_us` is its share of
+    the decode launch's time."""
     from fms_mo_amd import _lib as L
 
     out = {"peak": PEAK_HBM_GBS, "unit": "GB/s", "bound": "hbm"}
+    sink = torch.zeros(1, dtype=torch.int32, device=dev)
+    floors = {}
     for name, k, n in LLAMA3_8B:
         wbytes = k * n
         copies = max(3, (copies_mib * 1024 * 1024 + wbytes - 1) // wbytes)
@@ -179,9 +185,14 @@ def decode_rooflines(torch, K, dev, m_list=(1, 4, 16), ops=("i8", "fp8"), copies
             else:  # e4m3 weights whose codes cover the format's range (per-channel-scaled Gaussian)
                 ws_q = [torch.randn(n, k, device=dev).mul_(448.0 / 4.5).clamp_(-448, 448).to(torch.float8_e4m3fn)
                         for _ in range(copies)]
-            for M in m_list:
-                x = torch.randn(M, k, device=dev).bfloat16()
-                if op == "i8":
+            for M in (0,) * (name not in floors) + tuple(m_list):
+                if M == 0:  # the floor: a launch that only reads the weight bytes (same graph, same rotation)
+                    run = lambda w: K.stream_read(w, sink)  # noqa: E731
+                else:
+                    x = torch.randn(M, k, device=dev).bfloat16()
+                if M == 0:
+                    pass
+                elif op == "i8":
                     q, s = K.quant_act_i8_pertoken(x)
                     run = lambda w: K.gemm_i8_dq(q, w, s, wsc, None, out_dtype=torch.bfloat16, exact_ref=True)  # noqa: E731
                 else:
@@ -215,13 +226,19 @@ def decode_rooflines(torch, K, dev, m_list=(1, 4, 16), ops=("i8", "fp8"), copies
                     e1.record()
                     torch.cuda.synchronize()
                 ms = e0.elapsed_time(e1) / (replays * reps * copies)
+                del graph
+                if M == 0:
+                    floors[name] = ms
+                    out[f"read_only_floor_{name}"] = {"us": round(ms * 1e3, 2), "GBps": round(wbytes / ms / 1e6, 1),
+                                                      "frac": round(wbytes / ms / 1e6 / PEAK_HBM_GBS, 4)}
+                    continue
                 byts = wbytes + M * k + M * n * 2 + 4 * n
                 gbs = byts / (ms * 1e-3) / 1e9
                 out[f"{op}_M{M}_{name}"] = {"us": round(ms * 1e3, 2), "eager_us": round(eager_ms * 1e3, 2),
-                                            "GBps": round(gbs, 1), "frac": round(gbs / PEAK_HBM_GBS, 4)}
-                del graph
+                                            "GBps": round(gbs, 1), "frac": round(gbs / PEAK_HBM_GBS, 4),
+                                            "floor_over_us": round(floors[name] / ms, 3)}
             del ws_q
-    fr = [v["frac"] for kk, v in out.items() if isinstance(v, dict)]
+    fr = [v["frac"] for kk, v in out.items() if isinstance(v, dict) and not kk.startswith("read_only_floor")]
     out["frac_min"], out["frac_max"] = min(fr), max(fr)
     return out
 

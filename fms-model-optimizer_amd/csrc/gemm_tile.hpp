@@ -884,7 +884,7 @@ struct EpiDequant {
       const float sc = round_to<FMSMO_F16>(__fmul_rn(r.as, c.ws));
       const float t = __fadd_rn(__fmul_rn((float)v, sc), c.b);
       if constexpr (OUT == FMSMO_F32) ((float*)y)[idx] = t;
-      else if constexpr (OUT == FMSMO_F16) ((u16*)y)[idx] = f32_to_f16(t);
+      else if constexpr (OUT == FMSMO_F16) __builtin_nontemporal_store(f32_to_f16(t), &((u16*)y)[idx]);
       else store_from_f32<OUT>(y, idx, f16_to_f32(f32_to_f16(t)));
     } else {
       const float sc = __fmul_rn(r.as, c.ws);

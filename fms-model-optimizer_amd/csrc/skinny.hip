@@ -308,9 +308,10 @@ __global__ __launch_bounds__(NW * 64) void gemv_kernel(GemvArgs g) {
 // upper 8 rows are neither loaded nor stored.
 // HALF = false: the host has checked that every block owns whole groups only (the loads of the
 // upper rows are then unconditional, which the register allocation of the long-row shapes needs).
-template <int OP, int STEPS, int NW, int D, int MT = 1, bool HALF = false>
+template <int OP, int STEPS, int NW, int D, int MT = 1, bool HALF = false, bool XS = false>
 __global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(GemvArgs g, int halves) {
   static_assert(STEPS % D == 0, "pipeline depth must divide the steps per group");
+  static_assert(!XS || MT == 1, "streamed activations: one tile of tokens");
   typedef typename std::conditional<OP == FMSMO_OP_I8, int, float>::type AccT;
   typedef AccT Acc4 __attribute__((ext_vector_type(4)));
   constexpr int NRED = 2;  // exchange buffers alternate, one barrier per group
@@ -326,19 +327,6 @@ __global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(GemvArgs g, int ha
   if (gcount <= 0) return;                                    // more blocks than half groups
   const int kwave = wave * (STEPS * 128);
 
-  // activation fragments: lane (m = r, kg) holds x[m][kwave + s*128 + (h*4 + kg)*16 ...]
-  v4i xf[MT][STEPS][2];
-  {
-#pragma unroll
-    for (int t = 0; t < MT; ++t) {
-      const uint8_t* xp = g.a + (int64_t)min(t * 16 + r, g.M - 1) * g.lda + kwave + kg * 16;
-#pragma unroll
-      for (int s = 0; s < STEPS; ++s) {
-        xf[t][s][0] = *(const v4i*)(xp + s * 128);
-        xf[t][s][1] = *(const v4i*)(xp + s * 128 + 64);
-      }
-    }
-  }
   // weight loads: lane -> (row = lane / 8 [+8], 16-byte chunk = lane % 8): 8 rows x 128 B each
   const int drow = lane >> 3, dpos = lane & 7;
   // per-group row pointers, clamped (branch-free) for prefetch past the end and a ragged last group
@@ -369,6 +357,38 @@ __global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(GemvArgs g, int ha
 #pragma unroll
     for (int j = 0; j < D; ++j) wb[j][1] = v4i{0, 0, 0, 0};
   }
+  // Activation fragments: lane (m = r, kg) holds x[m][kwave + s*128 + (h*4 + kg)*16 ...], fetched
+  // through a buffer descriptor that ends with token row M - 1: the lanes of token rows past M get
+  // zeros without a branch or a clamped address (column m of the MFMA's second operand only
+  // reaches output column m, which is never stored).  Every block re-reads the activations from
+  // L2: 16 K bytes against its (N / blocks) K weight bytes, as much as the weights at N = 4096.
+  // XS = false: the fragments of the wave's whole K slice stay in registers for all the block's
+  // groups.  XS = true (long rows, one group per block, so each fragment is used once): they are
+  // fetched step by step beside the weights, D steps in flight, and the registers they leave free
+  // go to a deeper pipeline (us at N = 4096, K = 14336, int8, 4 / 16 tokens: 12.7 / 15.5 with the
+  // fragments held and two steps in flight, 11.4 / 13.8 streamed with seven; starting the blocks
+  // at different K steps so that they do not all ask L2 for the same lines at once: 11.7 / 14.3).
+  v4i xf[XS ? 1 : MT][XS ? 1 : STEPS][2];
+  v4i xb[XS ? D : 1][2];
+  const __amdgpu_buffer_rsrc_t rsrc_x = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)g.a, 0, (int)((int64_t)(g.M - 1) * g.lda + g.K), 0x00020000);
+  const int vx = r * (int)g.lda + kwave + kg * 16;
+  auto load_x = [&](int t, int s, v4i (&x)[2]) {
+    const int v = vx + t * 16 * (int)g.lda;
+    x[0] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_x, v, s * 128, 0));
+    x[1] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_x, v, s * 128 + 64, 0));
+  };
+  if constexpr (XS) {
+#pragma unroll
+    for (int j = 0; j < D; ++j) load_x(0, j, xb[j]);
+  } else {
+#pragma unroll
+    for (int t = 0; t < MT; ++t)
+#pragma unroll
+      for (int s = 0; s < STEPS; ++s) load_x(t, s, xf[t][s]);
+  }
+  // (the activation loads go first: with the weights ahead of them the kernel measured 2 - 5 %
+  // slower at 16 tokens)
 #pragma unroll
   for (int j = 0; j < D; ++j) load_item(false, j, wb[j]);
 
@@ -404,7 +424,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(GemvArgs g, int ha
       const v4i w1 = *(const v4i*)(st + rd1);
 #pragma unroll
       for (int t = 0; t < MT; ++t) {
-        const v4i x0 = xf[t][s][0], x1 = xf[t][s][1];
+        const v4i x0 = XS ? xb[s % D][0] : xf[t][s][0], x1 = XS ? xb[s % D][1] : xf[t][s][1];
         if constexpr (OP == FMSMO_OP_I8) {
           acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w0, x0, acc[t], 0, 0, 0);
           acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w1, x1, acc[t], 0, 0, 0);
@@ -413,6 +433,11 @@ __global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(GemvArgs g, int ha
           const v8i xv = {x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
           acc[t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wv, xv, acc[t], 0, 0, 0, 0, 0, 0);
         }
+      }
+      if constexpr (XS) {  // the same K offsets serve every group: the refill wraps around
+        __builtin_amdgcn_sched_barrier(0);
+        if (!LAST || s + D < STEPS) load_x(0, (s + D) % STEPS, xb[s % D]);
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
     // acc[v] = partial C(n = 16 (group0+gi) + 4 kg + v, m = r) of this wave's K slice.  The NW
@@ -466,8 +491,10 @@ __global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(GemvArgs g, int ha
       }
     }
   };
-  for (int gi = 0; gi + 1 < gcount; ++gi) do_group(std::false_type{}, gi);
-  do_group(std::true_type{}, gcount - 1);
+  if constexpr (!XS) {
+    for (int gi = 0; gi + 1 < gcount; ++gi) do_group(std::false_type{}, gi);
+  }
+  do_group(std::true_type{}, gcount - 1);  // XS: the host gives every block one group at most
 }
 
 // Row-streaming variant for M <= 2: no MFMA, no LDS.  A wave owns whole weight rows and reads
@@ -691,8 +718,13 @@ int fmsmo_gemv_dispatch(int op, const void* a, int64_t lda, const void* b, int64
     const int steps128 = K % 128 ? 0 : (int)(K / 128);
     const bool stream_ok = steps128 == 8 || steps128 == 16 || steps128 == 32 || steps128 == 40 ||
                            steps128 == 64 || steps128 == 100 || steps128 == 112 || steps128 == 128;
+    // Rows of 14336 where N <= 4096 gives every block of the streaming kernel a single row group
+    // (activations streamed beside the weights, seven steps in flight): one token 11.8 -> 11.2
+    // (int8), 12.7 -> 11.9 (e4m3).
+    const bool one_group = N <= 16 * 256;
     const bool prefer_stream =
-        stream_ok && (op == FMSMO_OP_I8 ? (M == 2 ? kch >= 8 : kch == 13) : (M == 2 || kch >= 11));
+        stream_ok && (op == FMSMO_OP_I8 ? (M == 2 ? kch >= 8 : (kch == 13 || (kch == 14 && one_group)))
+                                        : (M == 2 || kch >= 11));
     bool handled = env_kind != 1 && M <= 2 && K >= 1024 && !prefer_stream;
     if (handled) {
       // 16 waves per CU resident (register use allows it), rows dealt round-robin to waves
@@ -754,6 +786,11 @@ int fmsmo_gemv_dispatch(int op, const void* a, int64_t lda, const void* b, int64
     const bool whole_groups = halves % (2 * nblocks) == 0;
     dim3 grid((unsigned)nblocks), block(NW * 64);
     bool handled = true;
+    // a block that owns one row group gains nothing from keeping the activations in registers
+    // (FMSMO_GEMV_XS = 0 switches the streamed variant off, for tuning)
+    static const int env_xs = getenv("FMSMO_GEMV_XS") ? atoi(getenv("FMSMO_GEMV_XS")) : -1;
+    const bool x_ok = (M - 1) * lda + K < ((int64_t)1 << 31);  // 32-bit offsets into the activations
+    const bool xs = M <= 16 && halves <= 2 * nblocks && env_xs != 0;
 #define GEMV_STREAM_H(OPV, NWV, ST, DV, HV)                                                       \
   if (M <= 16) hipLaunchKernelGGL((gemv_stream_kernel<OPV, ST, NWV, DV, 1, HV>), grid, block, 0, st, g, G); \
   else if constexpr (NWV == 8 && ST <= 8) {                                                        \
@@ -764,21 +801,28 @@ int fmsmo_gemv_dispatch(int op, const void* a, int64_t lda, const void* b, int64
 #define GEMV_STREAM(OPV, NWV, ST, DV)                     \
   if (whole_groups) { GEMV_STREAM_H(OPV, NWV, ST, DV, false); } \
   else { GEMV_STREAM_H(OPV, NWV, ST, DV, true); }
+// long rows: DXS steps of weights and activations in flight where every block owns one group
+#define GEMV_STREAM_L(OPV, NWV, ST, DV, DXS)                                                       \
+  if (xs && whole_groups) hipLaunchKernelGGL((gemv_stream_kernel<OPV, ST, NWV, DXS, 1, false, true>), grid, block, 0, st, g, G); \
+  else if (xs) hipLaunchKernelGGL((gemv_stream_kernel<OPV, ST, NWV, DXS, 1, true, true>), grid, block, 0, st, g, G); \
+  else { GEMV_STREAM(OPV, NWV, ST, DV) }
 #define GEMV_SHAPES(OPV)                                            \
   switch (NW * 100 + STEPS) {                                       \
     case 801: GEMV_STREAM(OPV, 8, 1, 1); break;                     \
     case 802: GEMV_STREAM(OPV, 8, 2, 2); break;                     \
     case 804: GEMV_STREAM(OPV, 8, 4, 4); break;                     \
     case 805: GEMV_STREAM(OPV, 8, 5, 5); break;                     \
-    case 808: GEMV_STREAM(OPV, 8, 8, 4); break;                     \
-    case 814: GEMV_STREAM(OPV, 8, 14, 2); break;                    \
-    case 816: GEMV_STREAM(OPV, 8, 16, 4); break;                    \
-    case 1010: GEMV_STREAM(OPV, 10, 10, 2); break;                  \
+    case 808: GEMV_STREAM_L(OPV, 8, 8, 4, 8); break;                \
+    case 814: GEMV_STREAM_L(OPV, 8, 14, 2, 7); break;               \
+    case 816: GEMV_STREAM_L(OPV, 8, 16, 4, 8); break;               \
+    case 1010: GEMV_STREAM_L(OPV, 10, 10, 2, 5); break;             \
     case 1602: GEMV_STREAM(OPV, 16, 2, 2); break;                   \
     default: handled = false; break;                                \
   }
-    if (op == FMSMO_OP_I8) { GEMV_SHAPES(FMSMO_OP_I8) } else { GEMV_SHAPES(FMSMO_OP_E4M3) }
+    if (!x_ok) handled = false;
+    else if (op == FMSMO_OP_I8) { GEMV_SHAPES(FMSMO_OP_I8) } else { GEMV_SHAPES(FMSMO_OP_E4M3) }
 #undef GEMV_SHAPES
+#undef GEMV_STREAM_L
 #undef GEMV_STREAM
 #undef GEMV_STREAM_H
     if (handled) return fmsmo_check_launch();
@@ -883,6 +927,35 @@ extern "C" int fmsmo_decode_linear_fp8(const void* x, int x_dtype, int64_t ldx, 
   g.a_scale_out = a_scale_out;
   return x_dtype == FMSMO_F16 ? decode_fused_launch<FMSMO_OP_E4M3, FMSMO_F16>(g, (hipStream_t)stream)
                               : decode_fused_launch<FMSMO_OP_E4M3, FMSMO_BF16>(g, (hipStream_t)stream);
+}
+
+namespace fmsmo {
+// pure read of n16 16-byte words, block-contiguous, UNROLL loads in flight per lane
+__global__ __launch_bounds__(1024) void stream_read_kernel(const v4i* __restrict__ p, int64_t n16, int* sink) {
+  constexpr int UNROLL = 4;
+  const int64_t per = (n16 + gridDim.x - 1) / gridDim.x;
+  const int64_t lo = blockIdx.x * per, hi = lo + per < n16 ? lo + per : n16;
+  v4i acc = {0, 0, 0, 0};
+  int64_t i = lo + threadIdx.x;
+  for (; i + (UNROLL - 1) * 1024 < hi; i += UNROLL * 1024) {
+    v4i t[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) t[u] = __builtin_nontemporal_load(&p[i + u * 1024]);
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) acc ^= t[u];
+  }
+  for (; i < hi; i += 1024) acc ^= __builtin_nontemporal_load(&p[i]);
+  if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) == 0x5ca1ab1e) sink[0] = 1;
+}
+}  // namespace fmsmo
+
+extern "C" int fmsmo_debug_stream_read(const void* p, int64_t bytes, int32_t* sink, fmsmo_stream_t stream) {
+  if (!p || !sink) return FMSMO_ERR_NULL;
+  if (bytes <= 0 || bytes % 16) return FMSMO_ERR_SHAPE;
+  if ((uintptr_t)p & 15) return FMSMO_ERR_ALIGN;
+  hipLaunchKernelGGL(stream_read_kernel, dim3(256), dim3(1024), 0, (hipStream_t)stream, (const v4i*)p,
+                     bytes / 16, sink);
+  return fmsmo_check_launch();
 }
 
 static int check_gemv(const void* a, int64_t lda, const void* b, int64_t ldb, const float* a_scale,

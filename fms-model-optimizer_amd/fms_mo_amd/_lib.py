@@ -11,7 +11,8 @@ import os
 from ctypes import c_char_p, c_float, c_int, c_int64, c_void_p
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.normpath(os.path.join(_HERE, "..", "lib", "libfmsmo_hip.so"))
+# FMSMO_LIB names another build of the library (A/B measurements of kernel variants)
+LIB_PATH = os.environ.get("FMSMO_LIB") or os.path.normpath(os.path.join(_HERE, "..", "lib", "libfmsmo_hip.so"))
 
 # dtype / enum codes of include/fmsmo_hip.h
 F16, BF16, F32 = 0, 1, 2
@@ -58,6 +59,7 @@ SIGNATURES = {
     "fmsmo_bmm_fp8_dq": [_P, _L, _P, _L, _L, _P, _P, _P, _P, _I, _L, _L, _L, _L, _L, _P],
     "fmsmo_zero_shift_bias": [_P, _L, _P, _L, _P, _F, _P, _I, _P, _L, _L, _P],
     "fmsmo_debug_clock_probe": [_P],
+    "fmsmo_debug_stream_read": [_P, _L, _P, _P],
     "fmsmo_gemm_plan": [_L, _L, _L, _I, _P, _P, _P, _P],
 }
 OTHER = {

@@ -226,6 +226,18 @@ def clock_probe(buf):
     L.call("fmsmo_debug_clock_probe", buf.data_ptr())
 
 
+def stream_read(t, sink):
+    """Diagnostic: one launch that only reads the bytes of the contiguous tensor `t` from device
+    memory (fmsmo_debug_stream_read); `sink` is an int32 tensor of one element on the same GPU.
+    Timed like a decode linear over the same weights it gives the floor the launch and the
+    memory system set for that linear."""
+    _need_gpu(t)
+    _need_gpu(sink)
+    if not t.is_contiguous() or sink.dtype != torch.int32 or sink.numel() < 1:
+        raise ValueError("stream_read wants a contiguous tensor and an int32 sink")
+    L.call("fmsmo_debug_stream_read", t.data_ptr(), t.numel() * t.element_size(), sink.data_ptr(), _stream(t))
+
+
 def core_clock_mhz(buf):
     """Average core clock (MHz) over the life of the probed block: core cycles per tick of the
     constant 100 MHz counter, start of the block to the end of its epilogue."""

@@ -80,6 +80,17 @@ const char* fmsmo_last_error(void);
  */
 int fmsmo_debug_clock_probe(uint64_t* dev6);
 
+/*
+ * Diagnostic with no counterpart in the reference: the time a launch needs just to pull `bytes`
+ * bytes (a multiple of 16, 16-byte aligned) out of device memory.  256 blocks of 1024 threads
+ * read p once with 16-byte loads, one KiB of consecutive bytes per wave instruction, and write
+ * nothing (sink, 4 bytes of device memory, is written only if the XOR of all words happens to
+ * match a constant).  Timed in the same way as a decode linear over the same weights it gives
+ * the floor that the launch and the memory system set for that linear: the decode kernels add
+ * the activation reads, the reduction over the waves and the output on top of it.
+ */
+int fmsmo_debug_stream_read(const void* p, int64_t bytes, int32_t* sink, fmsmo_stream_t stream);
+
 /* ------------------------------------------------------------------------------------------
  * 1. Activation quantizers (one pass over x: read 2-4 B, write 1 B per element).
  * ------------------------------------------------------------------------------------------ */
