@@ -601,6 +601,255 @@ __global__ __launch_bounds__(AQ_THREADS) void quant_i8_mulscale_kernel(
   }
 }
 
+// ------------------------------------------------------------------ int8, multiplicative scale,
+// 16-bit compute dtype (x, the SmoothQuant scale, the clip values and every intermediate in fp16
+// or in bf16): the row-walking structure of quant_i8_pertoken16_kernel.  Blocks walk rows with a
+// stride of gridDim.x and fetch the next row while they work on the current one; the divisors of
+// the thread's columns stay in registers; the divided row is kept as packed 16-bit values and its
+// maximum is taken on the packed magnitudes.  The division uses the same fast quotient (see there
+// for why it rounds like the IEEE one); rows or blocks it does not cover -- divisors outside its
+// range, a zero or non-finite divisor, inf / NaN anywhere in the divided row, a row maximum whose
+// reciprocal overflows -- take mulscale_row_ieee16, which repeats the generic kernel's arithmetic.
+// The products  rnd_T(e * scale)  are exact in fp32 (two 16-bit significands), so one rounding to T
+// gives the correctly rounded T product; fp16 does it, the zero-point subtraction and the clamp
+// on packed pairs, and rounds to integer by adding 1536 (mode 2: 1536 - 128, which also folds the
+// shift to signed storage into the same single rounding).
+template <int T, int TH>
+__device__ __forceinline__ void mulscale_row_ieee16(const u16* __restrict__ xr, const u16* __restrict__ smooth,
+                                                    int mode, float sx, float zp, int8_t* __restrict__ qr,
+                                                    float* __restrict__ scale_out, int K, float* red) {
+  const int nchunk = K / AQ_VEC;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  auto chunk = [&](int c, float (&e)[8]) {
+    load8<T>(xr, (size_t)c * AQ_VEC, e);
+    if (smooth) {
+      float d[8];
+      load8<T>(smooth, (size_t)c * AQ_VEC, d);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) e[i] = round_to<T>(e[i] / d[i]);
+    }
+  };
+  float lo = -127.0f, hi = 127.0f, shift = 0.0f;
+  if (mode == 2) { lo = 0.0f; hi = 255.0f; shift = 128.0f; }
+  if (mode == 0) {
+    float amax = 0.0f;
+#pragma unroll 1
+    for (int c = threadIdx.x; c < nchunk; c += TH) {
+      float e[8];
+      chunk(c, e);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(e[j]));
+    }
+    amax = wave_max(amax);
+    __syncthreads();
+    if (lane == 0) red[wave] = amax;
+    __syncthreads();
+    amax = red[0];
+#pragma unroll
+    for (int w = 1; w < TH / 64; ++w) amax = fmaxf(amax, red[w]);
+    __syncthreads();
+    sx = amax > 0.0f ? levels_over<T>(127.0f, amax) : 0.0f;
+    if (threadIdx.x == 0) *scale_out = (sx > 0.0f) ? 1.0f / sx : 0.0f;
+  }
+#pragma unroll 1
+  for (int c = threadIdx.x; c < nchunk; c += TH) {
+    float e[8];
+    chunk(c, e);
+    uint8_t b[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      float t = round_to<T>(__fmul_rn(e[j], sx));
+      if (mode == 2) t = round_to<T>(__fsub_rn(t, zp));
+      t = fminf(fmaxf(__builtin_rintf(t), lo), hi) - shift;
+      b[j] = (uint8_t)(int)t;
+    }
+    store8((uint8_t*)qr, (size_t)c * AQ_VEC, b);
+  }
+}
+
+template <int T, int MODE, int NCH, bool SMOOTH, int TH = AQ_THREADS, bool KEEP = true>
+__global__ __launch_bounds__(TH) void quant_i8_mulscale16_kernel(
+    const u16* __restrict__ x, int64_t ldx, const u16* __restrict__ smooth,
+    const u16* __restrict__ clip, int8_t* __restrict__ q, int64_t ldq,
+    float* __restrict__ a_scale, int M, int K) {
+  constexpr bool KEEP_RCP = SMOOTH && KEEP;
+  constexpr int mode = MODE;
+  __shared__ float red[2][TH / 64];
+  const int nchunk = K / AQ_VEC;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+
+  v4i sm[SMOOTH ? NCH : 1];
+  float sr[KEEP_RCP ? NCH : 1][8];
+  bool ieee_block = false;
+  if constexpr (SMOOTH) {
+    int bad = 0;
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      const int c = threadIdx.x + i * TH;
+      if (c < nchunk) {
+        sm[i] = *(const v4i*)(smooth + (size_t)c * AQ_VEC);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const float d = cvt16<T>((u16)((uint32_t)sm[i][j >> 1] >> ((j & 1) * 16)));
+          if constexpr (T == FMSMO_BF16) bad |= !(fabsf(d) >= 8.6736174e-19f && fabsf(d) <= 1.1529215e18f);
+          if constexpr (KEEP_RCP) sr[i][j] = __builtin_amdgcn_rcpf(d);
+        }
+      }
+    }
+    if constexpr (T == FMSMO_BF16) ieee_block = __syncthreads_or(bad) != 0;
+  }
+
+  // per-tensor modes: one scale (and zero point) for all rows
+  float sx = 0.0f, zp = 0.0f;
+  if (mode != 0) {
+    const float cv = cvt16<T>(clip[0]);
+    if (mode == 1) {
+      sx = levels_over<T>(127.0f, cv);
+    } else {
+      const float cvn = cvt16<T>(clip[1]);
+      sx = levels_over<T>(255.0f, round_to<T>(__fsub_rn(cv, cvn)));
+      zp = round_to<T>(__fmul_rn(cvn, sx));
+    }
+    if (blockIdx.x == 0 && threadIdx.x == 0) { a_scale[0] = 1.0f / sx; a_scale[1] = zp; }
+    // clip values that give an infinite or NaN scale or zero point: every row the IEEE way
+    if (!(fabsf(sx) <= 3.0e38f) || !(fabsf(zp) <= 3.0e38f)) ieee_block = true;
+  }
+
+  const float nz = opaque_neg_zero();
+  v4i cur[NCH], nxt[NCH];
+  auto load_row = [&](int row, v4i (&dst)[NCH]) {
+    const u16* xr = x + (size_t)row * ldx;
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      const int c = threadIdx.x + i * TH;
+      if (c < nchunk) dst[i] = __builtin_nontemporal_load((const v4i*)(xr + (size_t)c * AQ_VEC));
+    }
+  };
+  auto divide_row = [&]() {
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      const int c = threadIdx.x + i * TH;
+      if (c < nchunk) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          uint32_t d = (uint32_t)sm[i][j];
+          if constexpr (!KEEP_RCP) asm volatile("" : "+v"(d));
+          const uint32_t w = (uint32_t)cur[i][j];
+          const float lo = cvt16<T>((u16)(w & 0xffff)), hi = cvt16<T>((u16)(w >> 16));
+          const float dl = cvt16<T>((u16)(d & 0xffff)), dh = cvt16<T>((u16)(d >> 16));
+          float rl, rh;
+          if constexpr (KEEP_RCP) {
+            rl = sr[i][2 * j], rh = sr[i][2 * j + 1];
+          } else {
+            rl = __builtin_amdgcn_rcpf(dl), rh = __builtin_amdgcn_rcpf(dh);
+          }
+          cur[i][j] = (int)pack16<T>(div16_mix<T>(lo, dl, rl, nz), div16_mix<T>(hi, dh, rh, nz));
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  int parity = 0;
+  auto row_amax_bits = [&]() -> uint32_t {
+    us2 amax2 = {0, 0};
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      const int c = threadIdx.x + i * TH;
+      if (c < nchunk) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const uint32_t mag = (uint32_t)cur[i][j] & 0x7fff7fffu;
+          us2 m2;
+          __builtin_memcpy(&m2, &mag, 4);
+          amax2 = __builtin_elementwise_max(amax2, m2);
+        }
+      }
+    }
+    uint32_t v = wave_max_u32((uint32_t)(amax2[0] > amax2[1] ? amax2[0] : amax2[1]));
+    float* rb = red[parity];
+    parity ^= 1;
+    if (lane == 0) rb[wave] = __uint_as_float(v);
+    __syncthreads();
+#pragma unroll
+    for (int w = 0; w < TH / 64; ++w) {
+      const uint32_t o = __float_as_uint(rb[w]);
+      v = o > v ? o : v;
+    }
+    return v;
+  };
+  constexpr uint32_t INF_BITS = T == FMSMO_F16 ? 0x7c00u : 0x7f80u;
+
+  int row = blockIdx.x;
+  if (row < M) load_row(row, cur);
+  for (; row < M; row += gridDim.x) {
+    const int nrow = row + gridDim.x;
+    if (nrow < M) load_row(nrow, nxt);
+
+    uint32_t abits = INF_BITS;
+    if (!ieee_block) {
+      if constexpr (SMOOTH) divide_row();
+      abits = row_amax_bits();
+    }
+    float s_row = sx;
+    if (abits < INF_BITS && mode == 0) {
+      const float amax = cvt16<T>((u16)abits);
+      s_row = amax > 0.0f ? levels_over<T>(127.0f, amax) : 0.0f;
+      if (!(s_row <= 3.0e38f)) abits = INF_BITS;  // 1 / amax overflowed T: the IEEE path's business
+    }
+    if (abits >= INF_BITS) {
+      mulscale_row_ieee16<T, TH>(x + (size_t)row * ldx, SMOOTH ? smooth : nullptr, mode, sx, zp,
+                                 q + (size_t)row * ldq, a_scale + row, K, red[0]);
+#pragma unroll
+      for (int i = 0; i < NCH; ++i) cur[i] = nxt[i];
+      continue;
+    }
+    if (mode == 0 && threadIdx.x == 0) a_scale[row] = (s_row > 0.0f) ? 1.0f / s_row : 0.0f;
+    int8_t* qr = q + (size_t)row * ldq;
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      const int c = threadIdx.x + i * TH;
+      if (c < nchunk) {
+        uint32_t code[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const uint32_t w = (uint32_t)cur[i][j];
+          if constexpr (T == FMSMO_F16) {
+            hf2 h;
+            __builtin_memcpy(&h, &w, 4);
+            const _Float16 s16 = (_Float16)s_row, z16 = (_Float16)zp;
+            h = h * hf2{s16, s16};
+            if (mode == 2) h = h - hf2{z16, z16};
+            const _Float16 lo16 = mode == 2 ? (_Float16)0.0f : (_Float16)-127.0f;
+            const _Float16 hi16 = mode == 2 ? (_Float16)255.0f : (_Float16)127.0f;
+            h = __builtin_elementwise_min(__builtin_elementwise_max(h, hf2{lo16, lo16}), hf2{hi16, hi16});
+            const _Float16 magic = mode == 2 ? (_Float16)1408.0f : (_Float16)1536.0f;
+            h = h + hf2{magic, magic};
+            __builtin_memcpy(&code[j], &h, 4);
+          } else {
+            float tl = round_to<T>(__fmul_rn(cvt16<T>((u16)(w & 0xffff)), s_row));
+            float th = round_to<T>(__fmul_rn(cvt16<T>((u16)(w >> 16)), s_row));
+            float lo = -127.0f, hi = 127.0f, shift = 0.0f;
+            if (mode == 2) {
+              tl = round_to<T>(__fsub_rn(tl, zp));
+              th = round_to<T>(__fsub_rn(th, zp));
+              lo = 0.0f; hi = 255.0f; shift = 128.0f;
+            }
+            const int cl = (int)(fminf(fmaxf(__builtin_rintf(tl), lo), hi) - shift);
+            const int ch = (int)(fminf(fmaxf(__builtin_rintf(th), lo), hi) - shift);
+            code[j] = ((uint32_t)cl & 0xffu) | (((uint32_t)ch & 0xffu) << 16);
+          }
+        }
+        const uint32_t o0 = __builtin_amdgcn_perm(code[1], code[0], 0x06040200u);
+        const uint32_t o1 = __builtin_amdgcn_perm(code[3], code[2], 0x06040200u);
+        *(uint2*)(qr + (size_t)c * AQ_VEC) = make_uint2(o0, o1);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) cur[i] = nxt[i];
+  }
+}
+
 // ------------------------------------------------------------------ int8, static per tensor,
 // evaluated in the compute dtype T, for the operands of a batched matmul:
 //   q = clamp( rint( rnd_T( rnd_T(x / scale) + offset ) ), -128, 127 )
@@ -1049,6 +1298,39 @@ extern "C" int fmsmo_quant_act_i8_mulscale(const void* x, int x_dtype, int64_t l
     return FMSMO_ERR_ALIGN;
   if (M == 0) return FMSMO_OK;
   hipStream_t st = (hipStream_t)stream;
+  // 16-bit fast path: x, the metadata and the compute dtype all fp16 (or all bf16)
+  if (x_dtype != FMSMO_F32 && compute_dtype == x_dtype && meta_dtype == x_dtype &&
+      K <= 2 * AQ_MAXCHUNK * AQ_THREADS * AQ_VEC) {
+    const int64_t per_thread = div_up(K, AQ_THREADS * AQ_VEC);
+    const int nch = per_thread <= 1 ? 1 : per_thread <= 2 ? 2 : per_thread <= 4 ? 4 : per_thread <= 8 ? 8 : 16;
+#define LAUNCH16M(T, MD, NCH, SM, TH, KEEP)                                                      \
+  {                                                                                              \
+    const int64_t resident =                                                                     \
+        resident_blocks((const void*)quant_i8_mulscale16_kernel<T, MD, NCH, SM, TH, KEEP>, TH);  \
+    dim3 grid16((unsigned)(M < resident ? M : resident)), block16(TH);                           \
+    hipLaunchKernelGGL((quant_i8_mulscale16_kernel<T, MD, NCH, SM, TH, KEEP>), grid16, block16,  \
+                       0, st, (const u16*)x, ldx, (const u16*)smooth, (const u16*)clip, q, ldq,  \
+                       a_scale, (int)M, (int)K);                                                 \
+  }
+#define LAUNCH16(T, NCH, SM, TH, KEEP)                    \
+  if (mode == 0) LAUNCH16M(T, 0, NCH, SM, TH, KEEP)       \
+  else if (mode == 1) LAUNCH16M(T, 1, NCH, SM, TH, KEEP)  \
+  else LAUNCH16M(T, 2, NCH, SM, TH, KEEP)
+#define PICK16(T)                                                                                        \
+  switch (nch * 2 + (smooth ? 1 : 0)) {                                                                  \
+    case 2: LAUNCH16(T, 1, false, 256, true); break;  case 3: LAUNCH16(T, 1, true, 256, true); break;   \
+    case 4: LAUNCH16(T, 2, false, 256, true); break;  case 5: LAUNCH16(T, 2, true, 256, true); break;   \
+    case 8: LAUNCH16(T, 4, false, 256, true); break;  case 9: LAUNCH16(T, 4, true, 256, true); break;   \
+    case 16: LAUNCH16(T, 4, false, 512, true); break; case 17: LAUNCH16(T, 4, true, 512, false); break; \
+    case 32: LAUNCH16(T, 8, false, 512, true); break;                                                   \
+    default: LAUNCH16(T, 8, true, 512, false); break; /* 16384 < K <= 32768 */                          \
+  }
+    if (x_dtype == FMSMO_F16) { PICK16(FMSMO_F16) } else { PICK16(FMSMO_BF16) }
+#undef PICK16
+#undef LAUNCH16
+#undef LAUNCH16M
+    return fmsmo_check_launch();
+  }
   dim3 grid((unsigned)M), block(AQ_THREADS);
 #define LAUNCH(XT, T)                                                                        \
   hipLaunchKernelGGL((quant_i8_mulscale_kernel<XT, T>), grid, block, 0, st, x, ldx, smooth,  \

@@ -82,6 +82,51 @@ def test_activation_codes_bit_exact(dev, act, xdt, mdt, smooth, shape):
             assert a_meta.cpu()[1].item() == zp_x.float().item()
 
 
+@pytest.mark.parametrize("act", MODES)
+@pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("K", [256, 14336])
+def test_activation_codes_rows_off_the_fast_path(dev, act, dt, K):
+    """Rows the row-walking 16-bit kernel hands to its IEEE routine, between ordinary rows: a
+    quotient x / smooth that overflows the dtype (per-tensor modes: the code saturates), a row whose
+    maximum is so small that 127 / max overflows (per token: every code +-127, output scale 0), a
+    divisor far outside the fast quotient's range (bf16).  All of them are finite in torch's own
+    arithmetic, so the oracle defines them; the neighbours must stay bit-exact too."""
+    from fms_mo_amd import _lib as L
+    from fms_mo_amd import kernels
+
+    g = gen(77)
+    M = 9
+    x = torch.randn(M, K, generator=g).to(dt)
+    sq = (torch.rand(K, generator=g) * 3 + 0.25).to(dt)
+    big = 6.0e4 if dt == torch.float16 else 3.0e38
+    if act == "per_token":
+        tiny = 2.0 ** -24 if dt == torch.float16 else 2.0 ** -130
+        x[4] = torch.where(torch.rand(K, generator=g) < 0.5, -1.0, 1.0).to(dt) * tiny * 3
+        sq[:] = 1.0
+        sq[5] = 0.5
+    else:
+        if dt == torch.bfloat16 and act == "per_tensor_symm":
+            sq[6] = 2.0 ** -70  # outside the fast quotient's divisor range: the whole block goes IEEE
+            x[:, 6] = (torch.randn(M, generator=g) * 2.0 ** -72).to(dt)
+        x[3, 17] = big
+        sq[17] = 0.25  # x / smooth = inf in the compute dtype
+        x[6, 200] = -big
+        sq[200] = 0.5
+    xs = x.float() / sq.float()
+    fin = xs[torch.isfinite(xs) & (xs.abs() < 100)]
+    a_cv = (fin.max() * 0.8).reshape(1).to(dt)
+    a_cvn = -a_cv if act != "per_tensor_asymm" else (fin.min() * 0.6).reshape(1).to(dt)
+    ref_int, scale_x, zp_x = O.i8i8_aiu_quant_act(x, a_cv, a_cvn, sq, act)
+    mode = {"per_token": L.MS_PER_TOKEN, "per_tensor_symm": L.MS_SYMM, "per_tensor_asymm": L.MS_ASYMM}[act]
+    clip = None if act == "per_token" else torch.cat((a_cv, a_cvn)).to(dev)
+    q, a_meta = kernels.quant_act_i8_mulscale(x.to(dev), mode, clip=clip, smooth=sq.to(dev), meta_dtype=dt)
+    got = q.cpu().to(torch.int32) + (128 if act == "per_tensor_asymm" else 0)
+    assert torch.equal(got, ref_int.to(torch.int32))
+    if act == "per_token":
+        assert torch.equal(a_meta.cpu(), (1.0 / scale_x.float()).reshape(-1))
+        assert a_meta[4].item() == 0.0 and torch.all(got[4].abs() == 127)
+
+
 def test_all_zero_row_gives_zero_codes_and_zero_scale(dev):
     from fms_mo_amd import _lib as L
     from fms_mo_amd import kernels
