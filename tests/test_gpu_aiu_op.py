@@ -146,9 +146,12 @@ def test_op_matches_the_reference_vectors(dev, path):
              d["weight_quant_type"], d["activ_quant_type"], d["smoothquant"])
     ref = d["reference_out"]
     assert y.shape == ref.shape and y.dtype == torch.float16
-    # the stored outputs come from the floating-point simulation (fp16 operands, fp16 F.linear);
-    # the integer path agrees within the fp16/bf16 output tolerance of the W8A8 path
-    torch.testing.assert_close(y.cpu().float(), ref.float(), rtol=1e-2, atol=1e-2)
+    # The stored outputs come from the floating-point simulation (fp16 operands, fp16 F.linear with
+    # its own accumulation order), the op here multiplies the integer codes exactly and rounds
+    # once.  Observed on these six vectors (K = 7, |y| up to 10.5): at most 4.3e-3 absolute where
+    # |y| < 8 and one fp16 ulp (7.8e-3) above; the band asserted is that with a small margin, half
+    # the W8A8 path's stated 1e-2 / 1e-2.
+    torch.testing.assert_close(y.cpu().float(), ref.float(), rtol=1e-3, atol=5e-3)
 
 
 def exact_from_oracle_codes(x, w_int, bias, w_cv, a_cv, a_cvn, sq, act):
