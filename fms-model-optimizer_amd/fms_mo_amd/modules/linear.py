@@ -29,6 +29,7 @@ from ..quant.quantizers import (
     Qbypass,
     QMaxDynamic,
     Qmax,
+    SAWB,
     get_activation_quantizer,
     get_weight_quantizer,
     to_fp8,
@@ -385,7 +386,12 @@ class QLinearINT8Deploy(nn.Linear):
             m.register_buffer("w_scale", w_scale)
             m.register_buffer("w_zp", w_zp)
             m.register_buffer("smoothq_scale", smoothq_scale)
-            w_int8 = _quantize_weight_rows(fms_mo_qlinear.weight, smoothq_scale, w_scale).to(torch.int)
+            if isinstance(Qw, SAWB):
+                # the quantizer's own integer output (linear.py:859-861); it stays switched to codes
+                Qw.dequantize = False
+                w_int8 = Qw(fms_mo_qlinear.weight.float() * smoothq_scale).to(torch.int)
+            else:
+                w_int8 = _quantize_weight_rows(fms_mo_qlinear.weight, smoothq_scale, w_scale).to(torch.int)
             m.weight = nn.Parameter(w_int8.to(torch.int8), requires_grad=False)
             if m.useSymAct:
                 corr_term_int = 0

@@ -8,9 +8,10 @@ inference forward of the modules in ``fms_mo_amd.modules.linear`` does not call 
 to the HIP kernels.
 
 Reference: fms_mo/quant/quantizers.py (factories :46-373, Qmax :2990-3141, QmaxSTE :3159,
-QmaxPerChSTE :3190, QMaxDynamic :3504-3537, to_fp8* :5309-5488, Qbypass).  Training-time
-learnable quantizers (PACT, LSQ, SAWB, AdaRound, ...) are outside the inference path and raise
-NotImplementedError here.
+QmaxPerChSTE :3190, QMaxDynamic :3504-3537, to_fp8* :5309-5488, Qbypass, SAWB :377-452 with its
+zero-aligned forward functions :455-630 and the clip rule :633-672 -- forward only, as
+QLinearINT8Deploy.from_fms_mo uses it).  Training-time learnable quantizers (PACT, LSQ, AdaRound,
+...) are outside the inference path and raise NotImplementedError here.
 """
 from __future__ import annotations
 
@@ -171,6 +172,98 @@ class Qmax(nn.Module):
                 f"{per}class={self.__class__.__name__})")
 
 
+SAWB_COEFF = {103: (2.6, -1.71), 403: (12.035, -12.03), 703: (28.24, -30.81), 803: (31.76, -35.04)}
+SAWB_BITS2CODE = {2: 103, 4: 403, 7: 703, 8: 803}
+
+
+def sawb_params_code(num_bits, code, out, perCh=False):
+    """Statistics-aware clip value  c1 * mean|w| + c0 * sqrt(mean w^2)  (quantizers.py:633-672):
+    per tensor -> (clip, 2^bits - 2); per output channel -> (clip vector, None)."""
+    if code not in SAWB_COEFF:
+        raise ValueError(f"SAWB not implemented for code={code}")
+    c0, c1 = SAWB_COEFF[code]
+    with torch.no_grad():
+        if perCh:
+            dims = list(range(1, out.dim()))
+            mu = torch.mean(out.abs(), dim=dims)
+            std = torch.mean(out**2, dim=dims).sqrt()
+            return c1 * mu + c0 * std, None
+        x = out.flatten()
+        mu = x.abs().mean()
+        std = x.mul(x).mean().sqrt()
+        return c1 * mu + c0 * std, 2**num_bits - 2
+
+
+class SAWB(nn.Module):
+    """Statistics-aware weight binning, zero-aligned (symmetric, 2^bits - 1 levels), forward only
+    (quantizers.py:377-452).  In training mode a call recomputes ``clip_val`` from the weight
+    statistics, in eval mode it uses the stored one.  ``dequantize=False`` returns the integer codes
+    in [-(2^(bits-1) - 1), 2^(bits-1) - 1], which is how QLinearINT8Deploy.from_fms_mo takes the
+    weights from it.  clipSTE and perCh select the per-channel formula (quantizers.py:503-572:
+    ``torch.quantize_per_channel`` with scale = 2 clip / (2^bits - 2)); every other combination is
+    per tensor (:455-500, :575-630):  round((clamp(w / clip, -1, 1) / 2 + 1/2) * (2^bits - 2)) - (2^(bits-1) - 1).
+    The variants without zero alignment are training-time only and are not built."""
+
+    def __init__(self, num_bits, dequantize=True, inplace=False, align_zero=False, clipSTE=True, perCh=False,
+                 interp=False):
+        super().__init__()
+        if num_bits not in [2, 4, 8]:
+            raise ValueError("FMS: SAWB supports 2, 4, and 8-bit quantization only.")
+        if not align_zero:
+            raise NotImplementedError("SAWB without zero alignment is a training-time quantizer, not built here")
+        self.num_bits = num_bits
+        self.dequantize = dequantize
+        self.inplace = inplace
+        self.align_zero = align_zero
+        self.clipSTE = clipSTE
+        self.perCh = perCh
+        self.interp = interp
+        self.register_buffer("clip_val", torch.zeros(perCh) if perCh else torch.Tensor([0.0]))
+
+    @property
+    def per_channel_formula(self):
+        return bool(self.clipSTE and self.perCh)
+
+    def forward(self, input_tensor):
+        nb = self.num_bits
+        with torch.no_grad():
+            if self.per_channel_formula:
+                if self.training:
+                    clip_val, _ = sawb_params_code(nb, SAWB_BITS2CODE[nb], input_tensor, perCh=True)
+                else:
+                    clip_val = self.clip_val
+                self.clip_val.copy_(clip_val)
+                int_u = 2 ** (nb - 1) - 1
+                scale = clip_val * 2 / (2**nb - 2)
+                zero_point = torch.zeros_like(scale)
+                if self.dequantize:
+                    return torch.fake_quantize_per_channel_affine(
+                        input_tensor.float(), scale.float(), zero_point.float(), axis=0, quant_min=-int_u,
+                        quant_max=int_u).to(clip_val.dtype)
+                return torch.quantize_per_channel(input_tensor, scale, zero_point, 0, torch.qint8) \
+                    .int_repr().clamp(-int_u, int_u)
+            scale = 2**nb - 2
+            if self.training:
+                clip_val, _ = sawb_params_code(nb, SAWB_BITS2CODE[nb], input_tensor)
+            else:
+                clip_val = self.clip_val
+            if self.clipSTE and clip_val <= 0:  # "sometimes sawb returns negative clipvals" (:481-483)
+                clip_val = input_tensor.abs().max()
+            if clip_val.dim() == 0:
+                clip_val = clip_val.unsqueeze(dim=0)
+            self.clip_val.copy_(clip_val)
+            clip_val = clip_val.to(input_tensor.device)
+            output = input_tensor.mul(1 / clip_val).clamp(-1, 1).mul(0.5).add(0.5)
+            output = torch.round(scale * output - 0.0)
+            if self.dequantize:
+                output = (output + 0.0) / scale
+                return (2 * output - 1) * clip_val
+            return output - scale / 2
+
+    def __repr__(self):
+        return f"{self.__class__.__name__}(num_bits={self.num_bits}, perCh={self.perCh}, clipSTE={self.clipSTE})"
+
+
 def max_to_scale(x_max, float8_dtype, orig_dtype):
     """Multiplicative FP8 scale 448 / clamp(max, 1e-12), stored in the original dtype."""
     if float8_dtype != torch.float8_e4m3fn:
@@ -240,7 +333,7 @@ class to_fp8(nn.Module):
         return f"{self.__class__.__name__}(q_mode={self.q_mode}, emulate={self.emulate})"
 
 
-_OUT_OF_SCOPE = ("pact", "lsq", "qsilu", "dorefa", "fix", "brecq", "sawb", "adaround", "qil", "custom")
+_OUT_OF_SCOPE = ("pact", "lsq", "qsilu", "dorefa", "fix", "brecq", "adaround", "qil", "custom")
 
 
 def get_activation_quantizer(qa_mode="PACT", nbits=32, clip_val=None, clip_valn=None, non_neg=False,
@@ -269,11 +362,14 @@ def get_activation_quantizer(qa_mode="PACT", nbits=32, clip_val=None, clip_valn=
 def get_weight_quantizer(qw_mode="SAWB+", nbits=32, clip_val=None, clip_valn=None, align_zero=True,
                          w_shape=None, use_swcap=False, recompute=False, perGp=None,
                          use_subnormal=False):
-    """Weight quantizer factory: max / maxperCh, fp8_e4m3_{sat,scale}[_perCh]."""
+    """Weight quantizer factory: sawb[+][perCh], max / maxperCh, fp8_e4m3_{sat,scale}[_perCh]."""
     mode = qw_mode or ""
     if use_swcap or any(k in mode.lower() for k in _OUT_OF_SCOPE):
         raise NotImplementedError(f"weight quantizer '{qw_mode}' is a training-time quantizer, not built here")
     nch = w_shape[0] if w_shape is not None and "perCh" in mode else False
+    if "sawb" in mode:  # quantizers.py:256-268
+        return SAWB(nbits, dequantize=True, inplace=False, align_zero=True, clipSTE="+" in mode, perCh=nch,
+                    interp="interp" in mode)
     if "max" in mode:
         if "min" in mode or "perGp" in mode:
             raise NotImplementedError("minmax / per-group weight quantizers are not on the W8A8 path")

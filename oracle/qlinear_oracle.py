@@ -40,6 +40,10 @@ How each function is pinned (see tests/test_oracle_*.py):
                            same end codes outside the clip range; the per-column quantizer is the
                            per-token one of the transposed tensor; the chunk loop equals the
                            chunked-kernel restatement (tests/test_oracle_pins_deploy.py)
+  * SAWB (zero-aligned, forward only) -- the codes equal the index of the nearest of the
+                           2^bits - 1 levels k clip / (2^(bits-1) - 1) found by search, the dequantized
+                           values are those levels, the clip rule against closed-form moments of a
+                           uniform grid and the negative-clip fallback on two-valued weights
   * FP8 emulation quantizers (to_fp8*)
                         -- the scale re-derived with exact rationals and explicit roundings
                            (reciprocal-then-multiply, fp16 clamp), the cast against the enumerated
@@ -181,6 +185,46 @@ def quant_weight_deploy(weight: torch.Tensor, w_cv: torch.Tensor, smoothq_scale:
     return w.to(torch.int).to(torch.int8), w_scale
 
 
+SAWB_COEFF = {103: (2.6, -1.71), 403: (12.035, -12.03), 803: (31.76, -35.04)}
+
+
+def sawb_clip(weight: torch.Tensor, num_bits: int = 8, perCh: bool = False):
+    """sawb_params_code (quantizers.py:633-672) for the zero-aligned codes 103 / 403 / 803:
+    clip = c1 * mean|w| + c0 * sqrt(mean w^2), per tensor or per output channel."""
+    c0, c1 = SAWB_COEFF[{2: 103, 4: 403, 8: 803}[num_bits]]
+    if perCh:
+        dims = list(range(1, weight.dim()))
+        return c1 * torch.mean(weight.abs(), dim=dims) + c0 * torch.mean(weight**2, dim=dims).sqrt()
+    x = weight.flatten()
+    return c1 * x.abs().mean() + c0 * x.mul(x).mean().sqrt()
+
+
+def sawb_zero_forward(x: torch.Tensor, clip_val: torch.Tensor, num_bits: int = 8, dequantize: bool = True):
+    """SAWBPlusZeroSTE / SAWBZeroSTE forward in eval mode (quantizers.py:486-494, 610-617):
+    x / clip clamped to +-1, mapped to [0, 1], rounded onto 2^bits - 2 steps; integer codes
+    (dequantize False) are that minus (2^bits - 2) / 2."""
+    scale = 2**num_bits - 2
+    if clip_val.dim() == 0:
+        clip_val = clip_val.unsqueeze(0)
+    out = x.mul(1 / clip_val).clamp(-1, 1).mul(0.5).add(0.5)
+    out = torch.round(scale * out - 0.0)
+    if dequantize:
+        out = (out + 0.0) / scale
+        return (2 * out - 1) * clip_val
+    return out - scale / 2
+
+
+def sawb_zero_perch_forward(x: torch.Tensor, clip_val: torch.Tensor, num_bits: int = 8, dequantize: bool = True):
+    """SAWBPlusZeroPerChSTE forward in eval mode (quantizers.py:541-565)."""
+    int_u = 2 ** (num_bits - 1) - 1
+    scale = clip_val * 2 / (2**num_bits - 2)
+    zp = torch.zeros_like(scale)
+    if dequantize:
+        return torch.fake_quantize_per_channel_affine(x.float(), scale.float(), zp.float(), axis=0,
+                                                      quant_min=-int_u, quant_max=int_u).to(clip_val.dtype)
+    return torch.quantize_per_channel(x, scale, zp, 0, torch.qint8).int_repr().clamp(-int_u, int_u)
+
+
 # ------------------------------------------------------------------------------------------
 # Integer GEMM and epilogue
 # ------------------------------------------------------------------------------------------
@@ -260,12 +304,14 @@ def deploy_forward(x, bufs):
 
 
 def deploy_prepare_general(weight, bias, w_cv, a_cv=None, a_cvn=None, sym_act=True, act_scale=None,
-                           alpha=0.5, use_PT_native_Qfunc=False, use_dynamic_max_act_Qfunc=False):
+                           alpha=0.5, use_PT_native_Qfunc=False, use_dynamic_max_act_Qfunc=False,
+                           sawb=None):
     """QLinearINT8Deploy.from_fms_mo (linear.py:717-920) for every activation-quantizer branch:
     dynamic max (-1 / -2), fake zero shift (1..64), PT-native static, fms_mo-formula static.
     ``sym_act`` is the reference's useSymAct (:765-769: 'sym' in qa_mode or qa_mode in
     pertokenmax / max).  a_cv / a_cvn: the activation quantizer's clip_val / clip_valn tensors
     (shape [1], fp32 as the quantizers register them) -- default 8.0 / -8.0 as at :793-794.
+    ``sawb``: the weight quantizer is a SAWB (None | "tensor" | "perCh") and supplies the codes.
     Returns the module state as a dict (buffers under the reference's names plus the flags)."""
     w_dtype = weight.dtype
     sym = int(bool(sym_act))
@@ -298,7 +344,11 @@ def deploy_prepare_general(weight, bias, w_cv, a_cv=None, a_cvn=None, sym_act=Tr
         st.update(quant_scale=quant_scale, quant_stepsize=quant_stepsize,
                   quant_zero_point=quant_zero_point)
     input_zp = input_zp.to(torch.int)
-    w_int = torch.round((weight * sq).t() / w_scale).clamp(-w_levels / 2, w_levels / 2).t().to(torch.int)
+    if sawb is None:
+        w_int = torch.round((weight * sq).t() / w_scale).clamp(-w_levels / 2, w_levels / 2).t().to(torch.int)
+    else:  # isinstance(Qw, SAWB) (linear.py:859-861): the quantizer's integer output; sawb = "tensor" | "perCh"
+        fwd = sawb_zero_perch_forward if sawb == "perCh" else sawb_zero_forward
+        w_int = fwd(weight.float() * sq, w_cv, 8, dequantize=False).to(torch.int)
     if sym:
         corr_term_int = 0
         if st["use_fake_zero_shift"]:

@@ -217,6 +217,53 @@ def test_deploy_module_fake_zero_shift_bit_exact(dev, zp):
     assert torch.equal(bits(y.cpu()), bits(ref["y"]))
 
 
+@pytest.mark.parametrize("qw_mode", ["sawb+", "sawb", "sawb+perCh"])
+@pytest.mark.parametrize("smoothq", [False, True])
+def test_deploy_module_from_a_sawb_weight_quantizer(dev, qw_mode, smoothq):
+    """from_fms_mo takes the integer weights from a SAWB quantizer's own output (linear.py:859-861).
+    The clip value comes from one training-mode pass over the weights (quantizers.py:633-672), the
+    conversion runs on the CPU, the forward on the GPU; weights, scales, bias and output against
+    the oracle, bit for bit."""
+    from fms_mo_amd.modules.linear import QLinear, QLinearINT8Deploy
+    from fms_mo_amd.quant.quantizers import SAWB
+
+    K, N, M = 512, 192, 33
+    m = QLinear(K, N, bias=True, num_bits_feature=8, qa_mode="pertokenmax", num_bits_weight=8,
+                qw_mode=qw_mode, qcfg={"smoothq": smoothq, "smoothq_alpha": 0.5}, device="cpu")
+    g = gen(21)
+    with torch.no_grad():
+        m.weight.copy_(0.02 * torch.randn(N, K, generator=g))
+        m.bias.copy_(0.01 * torch.randn(N, generator=g))
+    m.to(torch.float16)
+    Qw = m.quantize_weight
+    assert isinstance(Qw, SAWB) and Qw.per_channel_formula == (qw_mode == "sawb+perCh")
+    Qw.float()
+    act_scale = None
+    if smoothq:
+        act_scale = (torch.rand(K, generator=g) * 4 + 0.1)
+        m.smoothq_act_scale = act_scale.clone()
+        m.smoothq_alpha = m.smoothq_alpha.float()
+    with torch.no_grad():
+        Qw.train()
+        Qw(m.weight.float())
+    m.eval()
+    ref_clip = O.sawb_clip(m.weight.detach().float(), 8, perCh=Qw.per_channel_formula)
+    assert torch.equal(Qw.clip_val.reshape(-1), ref_clip.reshape(-1)) and (ref_clip > 0).all()
+    dep = QLinearINT8Deploy.from_fms_mo(m, use_int_kernel="cutlass", use_dynamic_max_act_Qfunc=-1,
+                                        recalc_clipvals=False, target_device=dev)
+    st = O.deploy_prepare_general(m.weight.detach(), m.bias.detach(), Qw.clip_val, act_scale=act_scale,
+                                  use_dynamic_max_act_Qfunc=-1,
+                                  sawb="perCh" if Qw.per_channel_formula else "tensor")
+    assert torch.equal(dep.weight.cpu(), st["weight"]) and st["weight"].abs().max() == 127
+    assert torch.equal(dep.w_scale.cpu(), st["w_scale"]) and torch.equal(bits(dep.bias.cpu()), bits(st["bias"]))
+    x = static_x(M, K, 22)
+    ref = O.deploy_forward_general(x, st)
+    y = dep(x.to(dev))
+    if not smoothq:  # (with SmoothQuant the division is fused into the forward's quantizer launch)
+        assert torch.equal(dep._quantize(x.to(dev)).cpu(), ref["q_x"])
+    assert torch.equal(bits(y.cpu()), bits(ref["y"]))
+
+
 def test_deploy_module_per_channel_dynamic_bit_exact(dev):
     """use_dynamic_max_act_Qfunc = -2: one scale per input channel over the tokens; the reference's
     [1,K] scale broadcasts against the [M,N] accumulator, so the layer is square."""

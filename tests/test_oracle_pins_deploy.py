@@ -355,3 +355,84 @@ def test_to_fp8_module_dispatch():
     assert torch.equal(O.to_fp8_forward(x, "fp8_e4m3_scale_perCh", perCh=5), O.to_fp8_scaled(x, "perCh")[0])
     assert torch.equal(O.to_fp8_forward(x, "fp8_e4m3_scale_perToken", perToken=True),
                        O.to_fp8_scaled(x, "perToken")[0])
+
+
+# ------------------------------------------------------------------------------------------ SAWB
+def test_sawb_codes_are_the_nearest_level_by_search():
+    """The zero-aligned SAWB forward restated as what it must be: the index of the nearest of the
+    255 (15, 3) levels k * clip / kmax, found by search over all levels (values further than 1e-3
+    of a step from a midpoint, where fp32 rounding of the two formulas may differ)."""
+    for bits in (8, 4, 2):
+        kmax = 2 ** (bits - 1) - 1
+        x = torch.randn(64, 96, generator=gen(31)) * 0.05
+        clip = torch.tensor(0.11)
+        codes = O.sawb_zero_forward(x, clip, bits, dequantize=False)
+        levels = torch.arange(-kmax, kmax + 1).double() * clip.double() / kmax
+        d = (x.double().unsqueeze(-1) - levels).abs()
+        best = d.argmin(-1) - kmax
+        step = clip.double() / kmax
+        frac = (x.double().clamp(-clip.double(), clip.double()) / step) % 1.0
+        safe = (frac - 0.5).abs() > 1e-3
+        assert safe.float().mean() > 0.99
+        assert torch.equal(codes.long()[safe], best[safe])
+        assert codes.abs().max() == kmax                      # values beyond +-clip saturate
+        deq = O.sawb_zero_forward(x, clip, bits, dequantize=True)
+        torch.testing.assert_close(deq.double(), codes.double() * step, rtol=1e-5, atol=1e-7)
+        # the per-channel formula with every row's clip equal is the same quantizer away from ties
+        pc = O.sawb_zero_perch_forward(x, clip.expand(64).clone(), bits, dequantize=False) if bits == 8 else None
+        if pc is not None:
+            assert torch.equal(pc.long()[safe], best[safe])
+
+
+def test_sawb_clip_rule_closed_forms():
+    """clip = c1 mean|w| + c0 rms(w).  A fine uniform grid on [-1, 1] has mean|w| = 1/2 and
+    rms = 1/sqrt(3) (up to 1/n): 8 bits -> 31.76 / sqrt(3) - 35.04 / 2.  Two-valued weights +-a
+    have mean|w| = rms = a, so the rule goes negative (31.76 - 35.04 < 0) and the quantizer falls
+    back on max|w| (quantizers.py:481-483)."""
+    w = torch.linspace(-1, 1, 200001).reshape(3, -1)
+    assert abs(O.sawb_clip(w, 8).item() - (31.76 / 3**0.5 - 35.04 / 2)) < 1e-3
+    assert abs(O.sawb_clip(w, 4).item() - (12.035 / 3**0.5 - 12.03 / 2)) < 1e-3
+    rows = torch.stack([torch.linspace(-1, 1, 100001), 0.5 * torch.linspace(-1, 1, 100001)])
+    pc = O.sawb_clip(rows, 8, perCh=True)
+    assert abs(pc[0].item() - (31.76 / 3**0.5 - 35.04 / 2)) < 1e-3 and abs(pc[1].item() * 2 - pc[0].item()) < 1e-3
+    a = 0.37
+    w2 = torch.where(torch.rand(16, 64, generator=gen(32)) < 0.5, -a, a)
+    assert O.sawb_clip(w2, 8).item() < 0
+
+    import sys, os
+    sys.path.insert(0, os.path.join(os.path.dirname(__file__), "..", "fms-model-optimizer_amd"))
+    from fms_mo_amd.quant.quantizers import SAWB
+
+    q = SAWB(8, align_zero=True, clipSTE=True, perCh=False).train()
+    out = q(w2)
+    assert abs(q.clip_val.item() - a) < 1e-6 and torch.allclose(out, w2)
+    # host class against the restatement: clip values and codes, per tensor and per channel
+    w3 = torch.randn(48, 80, generator=gen(33)) * 0.04
+    for perch in (False, 48):
+        q = SAWB(8, align_zero=True, clipSTE=True, perCh=perch).train()
+        q(w3)
+        ref_clip = O.sawb_clip(w3, 8, perCh=bool(perch))
+        assert torch.equal(q.clip_val.reshape(-1), ref_clip.reshape(-1))
+        q.eval()
+        q.dequantize = False
+        fwd = O.sawb_zero_perch_forward if perch else O.sawb_zero_forward
+        assert torch.equal(q(w3).float(), fwd(w3, ref_clip, 8, dequantize=False).float())
+
+
+def test_deploy_prepare_with_sawb_weights_dequantized_product_identity():
+    """from_fms_mo with a SAWB weight quantizer (linear.py:859-861): the int8 weights times
+    w_scale = 2 clip / 254 are the SAWB levels, so the deployed output equals the float64 product
+    of the dequantized operands like every other branch."""
+    g = gen(34)
+    W = (torch.randn(24, 64, generator=g) * 0.05).half()
+    b = (torch.randn(24, generator=g) * 0.1).half()
+    x = torch.randn(9, 64, generator=g).half()
+    w_cv = O.sawb_clip(W.float(), 8).reshape(1)
+    st = O.deploy_prepare_general(W, b, w_cv, use_dynamic_max_act_Qfunc=-1, sawb="tensor")
+    deq = O.sawb_zero_forward(W.float(), w_cv, 8, dequantize=True)
+    torch.testing.assert_close(st["weight"].double() * st["w_scale"].double(), deq.double(), rtol=1e-6, atol=1e-8)
+    out = O.deploy_forward_general(x, st)
+    q, s = O.quant_act_dyn_max(x, -1)
+    assert torch.equal(out["q_x"], q)
+    exact = (q.double() * s.double()) @ deq.double().t() + b.double()
+    torch.testing.assert_close(out["y"].double(), exact, rtol=2e-3, atol=2e-3)
