@@ -40,9 +40,14 @@ def test_quantizer_factories_and_scope():
     assert Q.get_weight_quantizer("maxperCh", 8, w_shape=(16, 32)).perCh == 16
     assert not Q.get_weight_quantizer("max", 8, w_shape=(16, 32)).perCh
     assert isinstance(Q.get_weight_quantizer("fp8_e4m3_scale_perCh", 8, w_shape=(16, 32)), Q.to_fp8)
-    for mode in ["pact+", "lsq+", "sawb+", "brecq"]:
+    sawb = Q.get_weight_quantizer("sawb+perCh", 8, w_shape=(16, 32))
+    assert isinstance(sawb, Q.SAWB) and sawb.per_channel_formula and sawb.clip_val.shape == (16,)
+    assert not Q.get_weight_quantizer("sawb", 8, w_shape=(16, 32)).per_channel_formula
+    for mode in ["pact+", "lsq+", "brecq"]:
         with pytest.raises(NotImplementedError):
             Q.get_activation_quantizer(mode, 8)
+    with pytest.raises(ValueError):  # SAWB is a weight quantizer only, as in the reference's factory
+        Q.get_activation_quantizer("sawb+", 8)
     with pytest.raises(ValueError):
         Q.get_weight_quantizer("nonsense", 8)
 
