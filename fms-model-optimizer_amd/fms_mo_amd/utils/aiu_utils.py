@@ -7,9 +7,10 @@ asymmetric activations).  The two passes over a weight matrix (column abs-max fo
 scale, quantization + row sums) run as HIP kernels; the vectors of K or N elements between them
 are torch arithmetic on the host, in the order the reference uses.
 
-Not carried over: the SAWB recomputation of narrow weight distributions
-(``recompute_narrow_weights``, aiu_utils.py:125-235) needs the SAWB quantizer, which is a
-training-time quantizer outside this package.
+``recompute_narrow_weights`` (aiu_utils.py:125-235): layers whose integer weights are narrow (standard
+deviation below 20 levels) are re-quantized with a SAWB quantizer's statistics-aware clip value,
+kept only where that clip value lies below the row (tensor) maximum; a one-time host computation
+with torch ops, as in the reference.
 """
 from __future__ import annotations
 
@@ -19,8 +20,11 @@ from pathlib import Path
 import torch
 
 from .. import kernels
+from ..quant.quantizers import SAWB
 
 logger = logging.getLogger(__name__)
+
+STD_THRESHOLD = 20
 
 EXCLUDED_KEYS = ["calib_counter", "num_module_called", "smoothq_act_scale", "smoothq_alpha",
                  "obsrv_w_clipval", "obsrv_clipval", "obsrv_clipvaln"]
@@ -69,12 +73,44 @@ def process_smoothquant(sd: dict, layer_name: str, new_sd: dict, device=None):
     return sq_scale, sq_a_scale
 
 
+def recompute_weight_with_sawb(weight_pre_quant, weight_int_as_fp, weight_per_channel: bool, sq_a_scale,
+                               layer_name: str, new_sd: dict):
+    """aiu_utils.py:125-235.  Returns (integer weights or None, recomputed?); overwrites the layer's
+    weight clip values in ``new_sd`` when it recomputes."""
+    weight_pre_quant = weight_pre_quant.to("cpu")
+    weight_int_as_fp = weight_int_as_fp.to("cpu")
+    if weight_per_channel:
+        recompute = any(w < STD_THRESHOLD for w in weight_int_as_fp.std(dim=-1))
+    else:
+        recompute = weight_int_as_fp.std().item() < STD_THRESHOLD
+    if not recompute:
+        return None, False
+    if sq_a_scale is not None and sum(sq_a_scale) != 0:
+        raise ValueError("Weight recomputation while smoothquant is in use is not yet supported.")
+    quantizer = SAWB(num_bits=8, dequantize=False, align_zero=True,
+                     perCh=weight_int_as_fp.size(0) if weight_per_channel else False)
+    quantizer.training = True  # the quantizer recomputes its clip value(s) from the weights
+    weight_int_sawb = quantizer(weight_pre_quant.to(torch.float32))
+    cv_sawb = quantizer.clip_val.to("cpu").to(torch.float16)
+    if weight_per_channel:
+        # SAWB rows only where the clip value does not exceed the row maximum
+        cv_max = weight_pre_quant.abs().max(dim=-1)[0]
+        weight_int_sawb = torch.where((cv_sawb < cv_max)[:, None], weight_int_sawb, weight_int_as_fp)
+        cv_guarded = torch.where(cv_sawb < cv_max, cv_sawb, cv_max)
+    else:
+        cv_max = weight_pre_quant.abs().max()
+        weight_int_sawb = weight_int_sawb if cv_sawb < cv_max else weight_int_as_fp
+        cv_guarded = torch.min(cv_sawb, cv_max)
+    new_sd[layer_name + ".quantize_weight.clip_val"] = cv_guarded
+    new_sd[layer_name + ".quantize_weight.clip_valn"] = -cv_guarded
+    return weight_int_sawb, True
+
+
 def process_weight(sd: dict, layer_name: str, sq_scale, recompute_narrow_weights: bool, new_sd: dict,
-                   device=None):
+                   device=None, weight_per_channel: bool = False, sq_a_scale=None):
     """aiu_utils.py:237-279: ``clamp(127 / w_cv * (W * sq_scale), -127, 127).round()`` -> int8, in
-    one kernel pass that also returns the integer row sums."""
-    if recompute_narrow_weights:
-        raise NotImplementedError("SAWB recomputation of narrow weights is not part of this package")
+    one kernel pass that also returns the integer row sums.  With ``recompute_narrow_weights`` a
+    layer whose integers are narrow is re-quantized by recompute_weight_with_sawb."""
     if layer_name + ".quantize_weight.clip_val" not in sd:
         return None, None
     w = sd[layer_name + ".weight"]
@@ -86,6 +122,16 @@ def process_weight(sd: dict, layer_name: str, sq_scale, recompute_narrow_weights
     wd = _gpu(w, device)
     smooth = None if sq_scale is None else sq_scale.reshape(-1).to(wd.device)
     q, row_sum = kernels.quant_weight_i8(wd, coef.to(wd.device), smooth, mode="mul", want_row_sum=True)
+    t_sum = w.dtype if sq_scale is None else torch.promote_types(w.dtype, sq_scale.dtype)
+    t_sum = torch.promote_types(t_sum, coef.dtype)
+    if recompute_narrow_weights:
+        w_pre = w if sq_scale is None else w * sq_scale.to(w.device)
+        w_sawb, recomputed = recompute_weight_with_sawb(w_pre, q.to(w_pre.dtype), weight_per_channel, sq_a_scale,
+                                                        layer_name, new_sd)
+        if recomputed:
+            q8 = w_sawb.to(torch.int8)
+            new_sd[layer_name + ".weight"] = q8.to("cpu")
+            return q8, q8.to(torch.int64).sum(dim=-1).to(t_sum)
     new_sd[layer_name + ".weight"] = q.to("cpu")
     # the reference sums the integer-valued weights in the dtype they were computed in (fp32
     # accumulation, one final rounding): round the exact integer sum to that dtype
@@ -115,7 +161,6 @@ def convert_sd_for_aiu(model, recompute_narrow_weights: bool = False, weight_per
     """aiu_utils.py:336-449.  ``model`` is any module whose state dict follows the fms_mo naming
     (``<layer>.weight``, ``<layer>.quantize_weight.clip_val``, ...); the layer identifiers come
     from ``model.config.model_type`` unless given."""
-    del weight_per_channel  # only steers the SAWB recomputation in the reference
     if quantized_layers is None:
         model_type = getattr(getattr(model, "config", None), "model_type", None)
         if not model_type:
@@ -126,9 +171,9 @@ def convert_sd_for_aiu(model, recompute_narrow_weights: bool = False, weight_per
     for k, v in sd.items():
         if k.endswith(".weight") and any(q in k for q in quantized_layers):
             layer_name = k[:-7]
-            sq_scale, _ = process_smoothquant(sd, layer_name, new_sd, device)
+            sq_scale, sq_a_scale = process_smoothquant(sd, layer_name, new_sd, device)
             weight_int, row_sum = process_weight(sd, layer_name, sq_scale, recompute_narrow_weights,
-                                                 new_sd, device)
+                                                 new_sd, device, weight_per_channel, sq_a_scale)
             process_zero_shift(sd, layer_name, weight_int, row_sum, new_sd)
         elif all(ex not in k for ex in EXCLUDED_KEYS):
             if k not in new_sd:

@@ -804,6 +804,34 @@ def aiu_convert_layer(weight, w_cv, sq_a_scale=None, sq_alpha=None, a_cv=None, a
     return out
 
 
+def aiu_recompute_narrow(weight_pre_quant, weight_int_as_fp, per_channel: bool):
+    """recompute_weight_with_sawb (fms_mo/utils/aiu_utils.py:125-235) without SmoothQuant: when the
+    integer weights are narrow (std below 20 levels, any row in per-channel mode) they are
+    re-quantized with a SAWB quantizer in training mode (clip from the statistics, :633-672) and
+    kept where that clip value is below the row (tensor) maximum.  Returns (integers or None,
+    guarded clip value(s) in fp16 or None)."""
+    if per_channel:
+        recompute = any(w < 20 for w in weight_int_as_fp.std(dim=-1))
+    else:
+        recompute = weight_int_as_fp.std().item() < 20
+    if not recompute:
+        return None, None
+    w32 = weight_pre_quant.to(torch.float32)
+    clip = sawb_clip(w32, 8, perCh=per_channel)
+    if per_channel:
+        w_sawb = sawb_zero_perch_forward(w32, clip, 8, dequantize=False)
+        cv_sawb = clip.to(torch.float16)
+        cv_max = weight_pre_quant.abs().max(dim=-1)[0]
+        w_int = torch.where((cv_sawb < cv_max)[:, None], w_sawb, weight_int_as_fp)
+        return w_int, torch.where(cv_sawb < cv_max, cv_sawb, cv_max)
+    if clip <= 0:  # SAWBPlusZeroSTE's safety check (:481-483)
+        clip = w32.abs().max()
+    w_sawb = sawb_zero_forward(w32, clip, 8, dequantize=False)
+    cv_sawb = clip.reshape(1).to(torch.float16)
+    cv_max = weight_pre_quant.abs().max()
+    return (w_sawb if cv_sawb < cv_max else weight_int_as_fp), torch.min(cv_sawb, cv_max)
+
+
 def absmax_cols(x):
     """comming_max of the SmoothQuant statistics hook (fms_mo/quant/ptq.py:2586-2595)."""
     return x.reshape(-1, x.shape[-1]).abs().max(dim=0).values.float()

@@ -155,12 +155,65 @@ def test_checkpoint_writer_matches_oracle_and_reader_runs(dev, smoothq, tmp_path
     assert err < 0.05 * ref.abs().max().item() + 0.02, err
 
 
+@pytest.mark.parametrize("per_channel", [False, True])
+def test_checkpoint_writer_recomputes_narrow_weights_with_sawb(dev, per_channel):
+    """recompute_narrow_weights (aiu_utils.py:125-235): one layer has an outlier weight that makes
+    the max-based integers narrow (std < 20 levels), the other does not.  Integers, clip values and
+    zero shifts against the oracle; the narrow layer's integers get wider and its clip value
+    smaller; with SmoothQuant in use the reference refuses, so does the writer."""
+    from fms_mo_amd.utils import aiu_utils as A
+
+    model = _Toy(False)
+    layers = ("layers.0.self_attn.q_proj", "layers.0.mlp.down_proj")
+    with torch.no_grad():
+        lin = model.layers[0].self_attn.q_proj
+        lin.weight[5, 9] = 1.5                                 # 30 sigma: the maximum no longer fits the bulk
+        if per_channel:
+            for m_ in (lin, model.layers[0].mlp.down_proj):
+                cv = m_.weight.detach().abs().max(dim=1)[0]
+                m_.quantize_weight.clip_val = cv.clone()
+                m_.quantize_weight.clip_valn = -cv.clone()
+        else:
+            lin.quantize_weight.clip_val.fill_(1.5)
+            lin.quantize_weight.clip_valn.fill_(-1.5)
+    sd = A.convert_sd_for_aiu(model, recompute_narrow_weights=True, weight_per_channel=per_channel, device=dev)
+    plain = A.convert_sd_for_aiu(model, recompute_narrow_weights=False, weight_per_channel=per_channel, device=dev)
+    msd = model.state_dict()
+    changed = []
+    for layer in layers:
+        w, cv = msd[layer + ".weight"], msd[layer + ".quantize_weight.clip_val"]
+        base = O.aiu_convert_layer(w, cv, None, None, msd[layer + ".quantize_feature.clip_val"],
+                                   msd[layer + ".quantize_feature.clip_valn"])
+        assert torch.equal(plain[layer + ".weight"], base["weight"])
+        w_int, cv_new = O.aiu_recompute_narrow(w, base["weight"].to(w.dtype), per_channel)
+        if w_int is None:
+            assert torch.equal(sd[layer + ".weight"], base["weight"])
+            assert torch.equal(sd[layer + ".quantize_weight.clip_val"], cv.to(torch.float16))
+            changed.append(False)
+            continue
+        changed.append(True)
+        assert torch.equal(sd[layer + ".weight"], w_int.to(torch.int8))
+        assert torch.equal(sd[layer + ".quantize_weight.clip_val"], cv_new)
+        assert torch.equal(sd[layer + ".quantize_weight.clip_valn"], -cv_new)
+        assert torch.equal(sd[layer + ".zero_shift"], w_int.sum(dim=1).to(torch.float32))
+        if not per_channel:   # (per channel the outlier row itself keeps its integers: SAWB's clip exceeds its maximum)
+            assert sd[layer + ".weight"].float().std() > 3 * plain[layer + ".weight"].float().std()
+        assert (sd[layer + ".quantize_weight.clip_val"].float() <= cv.float() + 1e-3).all()
+    assert changed[0]                                          # the layer with the outlier was recomputed
+    if not per_channel:
+        assert not changed[1]
+    with pytest.raises(ValueError, match="smoothquant"):
+        sq = _Toy(True)
+        with torch.no_grad():
+            sq.layers[0].self_attn.q_proj.weight[5, 9] = 40.0
+            sq.layers[0].self_attn.q_proj.quantize_weight.clip_val.fill_(40.0 * 5)
+        A.convert_sd_for_aiu(sq, recompute_narrow_weights=True, device=dev)
+
+
 def test_writer_rejects_what_it_cannot_do(dev):
     from fms_mo_amd.utils import aiu_utils as A
 
     model = _Toy(False)
-    with pytest.raises(NotImplementedError):
-        A.convert_sd_for_aiu(model, recompute_narrow_weights=True, device=dev)
     with pytest.raises(ValueError):
         A.save_sd_for_aiu(model, {"nbits_w": 4}, device=dev)
     model.config.model_type = "mamba"
