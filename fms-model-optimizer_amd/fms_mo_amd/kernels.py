@@ -22,8 +22,47 @@ def _need_gpu(*ts):
             )
 
 
+_RAW_STREAM = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_CUR_DEVICE = getattr(torch._C, "_cuda_getDevice", None)
+
+
 def _stream(t: torch.Tensor):
+    """The current HIP stream of the tensor's device, as the integer handle the C ABI takes."""
+    if _RAW_STREAM is not None:
+        return _RAW_STREAM(t.get_device())
     return torch.cuda.current_stream(t.device).cuda_stream
+
+
+class _NoSwitch:
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_SWITCH = _NoSwitch()
+
+
+def _dev(t: torch.Tensor):
+    """Context that makes the tensor's GPU current for a launch; nothing to do (and nothing paid:
+    entering torch.cuda.device costs about a microsecond each way) when it already is."""
+    idx = t.get_device()
+    if _CUR_DEVICE is not None and _CUR_DEVICE() == idx:
+        return _NO_SWITCH
+    return torch.cuda.device(idx)
+
+
+def _eager(*ts) -> bool:
+    """True when the call can go straight to the implementation: plain tensors outside a compiler
+    trace.  Otherwise the registered ``torch.ops.fms_mo_amd`` operator is called, whose shape-only
+    twin serves tracing (going through the dispatcher costs about 3 us per call)."""
+    if torch.compiler.is_compiling():
+        return False
+    for t in ts:
+        if t is not None and type(t) is not torch.Tensor and type(t) is not torch.nn.Parameter:
+            return False
+    return True
 
 
 def _ptr(t):
@@ -51,6 +90,10 @@ def _ld(t: torch.Tensor) -> int:
 
 
 def _scale_vec(s, n, device, name):
+    if (type(s) is torch.Tensor and s.dtype is torch.float32 and s.dim() == 1 and s.is_cuda
+            and s.is_contiguous() and not s.requires_grad and s.get_device() == device.index
+            and s.numel() in (1, n)):
+        return s  # the usual case: already the vector the kernels take
     if not torch.is_tensor(s):
         s = torch.tensor([float(s)], dtype=torch.float32, device=device)
     s = s.detach().to(device=device, dtype=torch.float32).reshape(-1).contiguous()
@@ -75,7 +118,7 @@ def quant_act_i8_pertoken(x, smooth=None, compute_dtype=None, saturate=False):
         compute_dtype = x.dtype if smooth is None else torch.promote_types(x.dtype, smooth.dtype)
     q = torch.empty((M, K), dtype=torch.int8, device=x.device)
     scale = torch.empty((M,), dtype=torch.float32, device=x.device)
-    with torch.cuda.device(x.device):
+    with _dev(x):
         L.call("fmsmo_quant_act_i8_pertoken", x.data_ptr(), _dt(x), _ld(x), _ptr(smooth),
                _dt(smooth) if smooth is not None else 0, _DT[compute_dtype], int(bool(saturate)),
                q.data_ptr(), K, scale.data_ptr(), M, K, _stream(x))
@@ -87,7 +130,7 @@ def quant_act_i8_static(x, scale: float, zp: int, sym: int):
     x = _rows(x)
     M, K = x.shape
     q = torch.empty((M, K), dtype=torch.int8, device=x.device)
-    with torch.cuda.device(x.device):
+    with _dev(x):
         L.call("fmsmo_quant_act_i8_static", x.data_ptr(), _dt(x), _ld(x), float(scale), int(zp),
                int(sym), q.data_ptr(), K, M, K, _stream(x))
     return q
@@ -119,7 +162,7 @@ def quant_act_i8_mulscale(x, mode, clip=None, smooth=None, meta_dtype=None):
     q = torch.empty((M, K), dtype=torch.int8, device=x.device)
     a_scale = torch.empty((M if mode == L.MS_PER_TOKEN else 2,), dtype=torch.float32,
                           device=x.device)
-    with torch.cuda.device(x.device):
+    with _dev(x):
         L.call("fmsmo_quant_act_i8_mulscale", x.data_ptr(), _dt(x), _ld(x), _ptr(smooth),
                _ptr(clip), _DT[meta_dtype] if meta_dtype is not None else _dt(x), _DT[compute_dtype],
                int(mode), q.data_ptr(), K, a_scale.data_ptr(), M, K, _stream(x))
@@ -136,7 +179,7 @@ def quant_act_fp8_pertoken(x, variant=L.FP8_LINEAR, static_scale=None):
         scale = _scale_vec(static_scale, 1, x.device, "static_scale")[:1].contiguous()
     else:
         scale = torch.empty((M,), dtype=torch.float32, device=x.device)
-    with torch.cuda.device(x.device):
+    with _dev(x):
         L.call("fmsmo_quant_act_fp8_pertoken", x.data_ptr(), _dt(x), _ld(x), int(variant),
                int(static_scale is not None), q.data_ptr(), K, scale.data_ptr(), M, K, _stream(x))
     return q, scale
@@ -149,7 +192,7 @@ def quant_act_i8_static_t(x, mode, compute_dtype, scale, zp, sym=0, clip_lo=0.0,
     x = _rows(x)
     M, K = x.shape
     q = torch.empty((M, K), dtype=torch.int8, device=x.device)
-    with torch.cuda.device(x.device):
+    with _dev(x):
         L.call("fmsmo_quant_act_i8_static_t", x.data_ptr(), _dt(x), _ld(x), int(mode),
                _DT[compute_dtype], float(scale), float(zp), int(sym), float(clip_lo), float(clip_hi),
                q.data_ptr(), K, M, K, _stream(x))
@@ -167,7 +210,7 @@ def quant_act_i8_dynamic(x, per_column, levels, zp=0):
     col_amax = absmax_cols(x)
     q = torch.empty((M, K), dtype=torch.int8, device=x.device)
     scale = torch.empty((K if per_column else 1,), dtype=torch.float32, device=x.device)
-    with torch.cuda.device(x.device):
+    with _dev(x):
         L.call("fmsmo_quant_act_i8_dynamic", x.data_ptr(), _dt(x), _ld(x), col_amax.data_ptr(),
                L.DQ_PER_COLUMN if per_column else L.DQ_PER_TENSOR, int(levels), int(zp),
                q.data_ptr(), K, scale.data_ptr(), M, K, _stream(x))
@@ -188,18 +231,24 @@ def fake_quant_fp8(x, mode, want_values=True, want_codes=False):
     scale = torch.empty((n,), dtype=torch.float32, device=x.device) if n else None
     inv = torch.empty((n,), dtype=torch.float32, device=x.device) if n else None
     col_amax = absmax_cols(x) if mode == L.F8E_PER_TENSOR else None
-    with torch.cuda.device(x.device):
+    with _dev(x):
         L.call("fmsmo_fake_quant_fp8", x.data_ptr(), _dt(x), _ld(x), int(mode), _ptr(col_amax),
                _ptr(y), K, _ptr(q), K, _ptr(scale), _ptr(inv), M, K, _stream(x))
     return y, q, scale, inv
 
 
 # ------------------------------------------------------------------------------------ GEMMs
+_WS_BYTES: dict = {}
+
+
 def _workspace(M, N, K, device):
     """Scratch for the split-K form of the *_dq GEMMs (None when the shape does not use one).  It
     comes from torch's caching allocator like every output, so it is also valid under graph
     capture; the library itself never allocates."""
-    nbytes = L.load().fmsmo_gemm_workspace_bytes(M, N, K)
+    key = (M, N, K)
+    nbytes = _WS_BYTES.get(key)
+    if nbytes is None:  # the policy is fixed for the life of the process: ask the library once per shape
+        nbytes = _WS_BYTES[key] = L.load().fmsmo_gemm_workspace_bytes(M, N, K)
     return torch.empty((nbytes,), dtype=torch.uint8, device=device) if nbytes > 0 else None
 
 
@@ -261,7 +310,7 @@ def gemm_i8_i32(a, w):
     M, K = a.shape
     N = w.shape[0]
     c = torch.empty((M, N), dtype=torch.int32, device=a.device)
-    with torch.cuda.device(a.device):
+    with _dev(a):
         L.call("fmsmo_gemm_i8_i32", a.data_ptr(), _ld(a), w.data_ptr(), _ld(w), c.data_ptr(), N,
                M, N, K, _stream(a))
     return c
@@ -285,7 +334,7 @@ def gemm_i8_dq(a, w, a_scale, w_scale, bias=None, out_dtype=torch.float16, epilo
             _dt(bias) if bias is not None else 0, int(epilogue),
             y.data_ptr(), _DT[out_dtype], N, M, N, K)
     ws = None if force_gemv else _workspace(M, N, K, a.device)
-    with torch.cuda.device(a.device):
+    with _dev(a):
         if ws is not None:
             L.call("fmsmo_gemm_i8_dq_ws", *args, ws.data_ptr(), ws.numel(), _stream(a))
         else:
@@ -309,7 +358,7 @@ def gemm_fp8_dq(a, w, a_scale, w_scale, bias=None, out_dtype=torch.bfloat16, for
             a_scale.numel(), w_scale.data_ptr(), w_scale.numel(), _ptr(bias),
             _dt(bias) if bias is not None else 0, y.data_ptr(), _DT[out_dtype], N, M, N, K)
     ws = None if force_gemv else _workspace(M, N, K, a.device)
-    with torch.cuda.device(a.device):
+    with _dev(a):
         if ws is not None:
             L.call("fmsmo_gemm_fp8_dq_ws", *args, ws.data_ptr(), ws.numel(), _stream(a))
         else:
@@ -339,7 +388,7 @@ def grouped_gemm_i8_dq(a, w, offsets, a_scale, w_scale, bias=None, out_dtype=tor
         if bias.numel() != E * N:
             raise ValueError("bias must be [E,N]")
     y = torch.empty((T, N), dtype=out_dtype, device=a.device)
-    with torch.cuda.device(a.device):
+    with _dev(a):
         L.call("fmsmo_grouped_gemm_i8_dq", a.data_ptr(), _ld(a), w.data_ptr(), K, N * K,
                offsets.contiguous().data_ptr(), E, T, a_scale.data_ptr(), w_scale.data_ptr(),
                _ptr(bias), _dt(bias) if bias is not None else 0,
@@ -373,7 +422,7 @@ def matmul_chunk(a, w, c=None, chunk_size=64, chunk_trun_bits=0, max_acc_bits=32
         if c.shape != (M, N):
             raise ValueError("C shape is inconsistent with A B.")
         c = c.to(acc_dtype).contiguous()
-    with torch.cuda.device(a.device):
+    with _dev(a):
         if a.dtype == torch.int8:
             L.call("fmsmo_matmul_chunk_i8", a.data_ptr(), _ld(a), w.data_ptr(), _ld(w), _ptr(c),
                    d.data_ptr(), N, M, N, K, int(chunk_size), int(chunk_trun_bits),
@@ -407,7 +456,7 @@ def quant_weight_i8(w, coef, smooth=None, mode="mul", want_row_sum=False):
             smooth = smooth.clone()
     q = torch.empty((N, K), dtype=torch.int8, device=w.device)
     rs = torch.empty((N,), dtype=torch.int32, device=w.device) if want_row_sum else None
-    with torch.cuda.device(w.device):
+    with _dev(w):
         L.call("fmsmo_quant_weight_i8", w.data_ptr(), _dt(w), _ld(w), _ptr(smooth),
                _dt(smooth) if smooth is not None else 0, coef.data_ptr(), _dt(coef), coef.numel(),
                L.WQ_MUL if mode == "mul" else L.WQ_DIV, q.data_ptr(), K, _ptr(rs), N, K, _stream(w))
@@ -424,7 +473,7 @@ def absmax_cols(x, running=None):
         running = torch.zeros((K,), dtype=torch.float32, device=x.device)
     elif running.dtype != torch.float32 or running.numel() != K or not running.is_contiguous():
         raise ValueError("running must be a contiguous fp32 tensor with K elements")
-    with torch.cuda.device(x.device):
+    with _dev(x):
         L.call("fmsmo_absmax_cols", x.data_ptr(), _dt(x), _ld(x), M, K, running.data_ptr(), _stream(x))
     return running
 
@@ -445,7 +494,7 @@ def zero_shift_bias(w, w_scale, a_meta, bias=None, offset=128.0):
         if bias.numel() != N:
             raise ValueError("bias must have N elements")
     out = torch.empty((N,), dtype=torch.float32, device=w.device)
-    with torch.cuda.device(w.device):
+    with _dev(w):
         L.call("fmsmo_zero_shift_bias", w.data_ptr(), _ld(w), w_scale.data_ptr(), w_scale.numel(),
                a_meta.contiguous().data_ptr(), float(offset), _ptr(bias),
                _dt(bias) if bias is not None else 0, out.data_ptr(), N, K, _stream(w))
@@ -472,7 +521,7 @@ def quant_i8_affine(x, scale: float, offset: float, compute_dtype=None, transpos
     inner = R if transpose else C
     ldq = (inner + pad_to - 1) // pad_to * pad_to
     q = torch.empty((B, C if transpose else R, ldq), dtype=torch.int8, device=x.device)
-    with torch.cuda.device(x.device):
+    with _dev(x):
         L.call("fmsmo_quant_i8_affine", x3.data_ptr(), _dt(x3), x3.stride(1) if R > 1 else C,
                x3.stride(0) if B > 1 else R * C, float(scale), float(offset), _DT[compute_dtype],
                int(bool(transpose)), q.data_ptr(), ldq, q.stride(0), B, R, C, _stream(x))
@@ -497,7 +546,7 @@ def _bmm(fn, dtype, a, b, a_scale, b_scale, bias, out_dtype):
         if bias.numel() != B * N:
             raise ValueError("bias must be [batch, N]")
     y = torch.empty((B, M, N), dtype=out_dtype, device=a.device)
-    with torch.cuda.device(a.device):
+    with _dev(a):
         L.call(fn, a.data_ptr(), K, b.data_ptr(), b.stride(1) if N > 1 else K,
                b.stride(0) if B > 1 else N * K, a_scale.data_ptr(), b_scale.data_ptr(), _ptr(bias),
                y.data_ptr(), _DT[out_dtype], N, B, M, N, K, _stream(a))
@@ -591,6 +640,8 @@ def quant_act_i8_pertoken(x, smooth=None, compute_dtype=None, saturate=False):  
     _need_gpu(x, smooth)
     if x.dim() != 2:
         raise ValueError("expected a 2-D tensor")
+    if _eager(x, smooth):
+        return _quant_act_i8_pertoken_impl(x, smooth, compute_dtype, bool(saturate))
     return torch.ops.fms_mo_amd.quant_act_i8_pertoken(x, smooth, compute_dtype, bool(saturate))
 
 
@@ -598,6 +649,8 @@ def quant_act_i8_static(x, scale: float, zp: int, sym: int):  # noqa: F811
     _need_gpu(x)
     if x.dim() != 2:
         raise ValueError("expected a 2-D tensor")
+    if _eager(x):
+        return _quant_act_i8_static_impl(x, float(scale), int(zp), int(sym))
     return torch.ops.fms_mo_amd.quant_act_i8_static(x, float(scale), int(zp), int(sym))
 
 
@@ -608,6 +661,8 @@ def quant_act_fp8_pertoken(x, variant=L.FP8_LINEAR, static_scale=None):  # noqa:
         raise ValueError("expected a 2-D tensor")
     if static_scale is not None:
         static_scale = _as_scale(static_scale, x.device)
+    if _eager(x, static_scale):
+        return _quant_act_fp8_pertoken_impl(x, int(variant), static_scale)
     return torch.ops.fms_mo_amd.quant_act_fp8_pertoken(x, int(variant), static_scale)
 
 
@@ -618,12 +673,18 @@ def gemm_i8_dq(a, w, a_scale, w_scale, bias=None, out_dtype=torch.float16, exact
     _need_gpu(a, w, bias)
     if epilogue is None:
         epilogue = L.EPI_REF_F16 if exact_ref else L.EPI_F32
+    if _eager(a, w, bias) and (not torch.is_tensor(a_scale) or _eager(a_scale)) \
+            and (not torch.is_tensor(w_scale) or _eager(w_scale)):
+        return _gemm_i8_dq_impl(a, w, a_scale, w_scale, bias, out_dtype, int(epilogue), bool(force_gemv))
     return torch.ops.fms_mo_amd.gemm_i8_dq(a, w, _as_scale(a_scale, a.device), _as_scale(w_scale, a.device),
                                            bias, out_dtype, int(epilogue), bool(force_gemv))
 
 
 def gemm_fp8_dq(a, w, a_scale, w_scale, bias=None, out_dtype=torch.bfloat16, force_gemv=False):  # noqa: F811
     _need_gpu(a, w, bias)
+    if _eager(a, w, bias) and (not torch.is_tensor(a_scale) or _eager(a_scale)) \
+            and (not torch.is_tensor(w_scale) or _eager(w_scale)):
+        return _gemm_fp8_dq_impl(a, w, a_scale, w_scale, bias, out_dtype, bool(force_gemv))
     return torch.ops.fms_mo_amd.gemm_fp8_dq(a, w, _as_scale(a_scale, a.device), _as_scale(w_scale, a.device),
                                             bias, out_dtype, bool(force_gemv))
 
@@ -671,7 +732,7 @@ def _decode_linear_i8_impl(x, w, w_scale, bias, smooth, out_dtype, exact_ref, sa
             raise ValueError("bias must have N elements")
     y = torch.empty((M, N), dtype=out_dtype, device=x.device)
     a_scale = torch.empty((M,), dtype=torch.float32, device=x.device)
-    with torch.cuda.device(x.device):
+    with _dev(x):
         L.call("fmsmo_decode_linear_i8", x.data_ptr(), _dt(x), _ld(x), _ptr(smooth), int(bool(saturate)),
                w.data_ptr(), _ld(w), w_scale.data_ptr(), w_scale.numel(), _ptr(bias),
                _dt(bias) if bias is not None else 0, L.EPI_REF_F16 if exact_ref else L.EPI_F32,
@@ -696,6 +757,8 @@ def decode_linear_i8(x, w, w_scale, bias=None, smooth=None, out_dtype=torch.floa
     """(y [M,N], per-token scales fp32 [M]) = quantize x per token (see quant_act_i8_pertoken) and
     multiply with the int8 weights w [N,K], in one launch; check ``decode_linear_ok`` first."""
     _need_gpu(x, w, bias, smooth)
+    if _eager(x, w, bias, smooth) and (not torch.is_tensor(w_scale) or _eager(w_scale)):
+        return _decode_linear_i8_impl(x, w, w_scale, bias, smooth, out_dtype, bool(exact_ref), bool(saturate))
     return torch.ops.fms_mo_amd.decode_linear_i8(x, w, _as_scale(w_scale, x.device), bias, smooth,
                                                  out_dtype, bool(exact_ref), bool(saturate))
 
@@ -715,7 +778,7 @@ def _decode_linear_fp8_impl(x, w, w_scale, bias, out_dtype):
             raise ValueError("bias must have N elements")
     y = torch.empty((M, N), dtype=out_dtype, device=x.device)
     a_scale = torch.empty((M,), dtype=torch.float32, device=x.device)
-    with torch.cuda.device(x.device):
+    with _dev(x):
         L.call("fmsmo_decode_linear_fp8", x.data_ptr(), _dt(x), _ld(x), w.data_ptr(), _ld(w),
                w_scale.data_ptr(), w_scale.numel(), _ptr(bias), _dt(bias) if bias is not None else 0,
                y.data_ptr(), _DT[out_dtype], N, a_scale.data_ptr(), M, N, K, _stream(x))
@@ -736,4 +799,6 @@ def decode_linear_fp8(x, w, w_scale, bias=None, out_dtype=torch.bfloat16):
     """(y [1,N], token scale fp32 [1]): dynamic per-token e4m3 quantizer (the FP8Linear recipe) and
     the e4m3 weight-streaming matmul in one launch; check ``decode_linear_ok(x, None, K)`` first."""
     _need_gpu(x, w, bias)
+    if _eager(x, w, bias) and (not torch.is_tensor(w_scale) or _eager(w_scale)):
+        return _decode_linear_fp8_impl(x, w, w_scale, bias, out_dtype)
     return torch.ops.fms_mo_amd.decode_linear_fp8(x, w, _as_scale(w_scale, x.device), bias, out_dtype)
