@@ -2,6 +2,7 @@
 // compiled separately to keep the build parallel): argument checks, tile choice, launchers.
 #pragma once
 #include "gemm_rs.hpp"
+#include "gemm_k128.hpp"
 #include <cmath>
 #include <cstdlib>
 
@@ -103,6 +104,21 @@ void launch_rs(const GemmArgs& g0, const Epi& epi, hipStream_t st) {
   g.group_m = 4;
   dim3 grid((unsigned)(g.grid_m * g.grid_n)), block(256);
   hipLaunchKernelGGL((gemm_rs_kernel<OP, Epi, GROUPED, BN, ONE_SLAB, BM>), grid, block, 0, st, g, epi);
+}
+
+// Reduction of exactly 128 bytes (attention scores): persistent blocks over 128 x 256 tiles, two
+// per compute unit (FMSMO_K128_BLOCKS sets the grid, for tuning).
+template <int OP, class Epi>
+void launch_k128(const GemmArgs& g0, int batch, int M, const Epi& epi, hipStream_t st) {
+  GemmArgs g = g0;
+  g.grid_n = div_up(g.N, 256);
+  g.grid_m = batch * div_up(M, 128);
+  g.group_m = 4;
+  static const int env_blocks = getenv("FMSMO_K128_BLOCKS") ? atoi(getenv("FMSMO_K128_BLOCKS")) : 0;
+  const long tiles = (long)g.grid_m * g.grid_n;
+  long blocks = env_blocks > 0 ? env_blocks : 512;
+  if (blocks > tiles) blocks = tiles;
+  hipLaunchKernelGGL((gemm_k128_kernel<OP, Epi>), dim3((unsigned)blocks), dim3(256), 0, st, g, epi);
 }
 
 // Generic fallback (any K % 16 == 0): one thread per output element, 4-byte dot products.
@@ -361,8 +377,7 @@ int launch_bmm(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t s
     } else {                                                                                \
       g.grid_m = (int)batch * div_up(M, 256);                                               \
       if (K == 128 && use_register_staged(OP)) {                                            \
-        g.grid_m = (int)batch * div_up(M, 128);                                             \
-        launch_rs<OP, true, 256, true, 128>(g, epi, st);                                    \
+        launch_k128<OP>(g, (int)batch, (int)M, EpiScaleBias<OUT, AccT>{y, ldy, a_scale, b_scale, bias}, st); \
       }                                                                                     \
       else if (K % 128 == 0 && use_register_staged(OP)) launch_rs<OP, true>(g, epi, st);    \
       else launch_tile<TileBig, OP, true>(g, epi, st);                                      \

@@ -854,6 +854,7 @@ struct EpiStoreF32 {
 // y = acc * (a_scale[m] x w_scale[n]) + bias[n], see FMSMO_EPI_* in fmsmo_hip.h.
 template <int OUT, int BIAS, bool REF_F16, class AccT>
 struct EpiDequant {
+  static constexpr bool UNIFORM_ROWS = false;
   void* y;
   int64_t ldy;
   const float* a_scale;
@@ -891,6 +892,33 @@ struct EpiDequant {
       const float t = muladd ? __fadd_rn(__fmul_rn((float)v, sc), c.b) : __fmaf_rn((float)v, sc, c.b);
       store_from_f32<OUT>(y, idx, t);
     }
+  }
+};
+
+// y = acc * (a_scale[0] * w_scale[0]) + bias[n]: the batched matmuls' epilogue, one scale for the
+// whole batch (EpiDequant's fp32-scale arithmetic with nothing to fetch per row).
+template <int OUT, class AccT>
+struct EpiScaleBias {
+  static constexpr bool UNIFORM_ROWS = true;
+  static constexpr int OUT_DT = OUT;
+  void* y;
+  int64_t ldy;
+  const float* a_scale;
+  const float* w_scale;
+  const float* bias;
+  struct Col {
+    float b;
+  };
+  struct Row {
+    float sc;
+  };
+  __device__ __forceinline__ Col col(int n, int expert, int N) const {
+    return Col{bias ? bias[(int64_t)expert * N + n] : 0.0f};
+  }
+  __device__ __forceinline__ Row row(int) const { return Row{__fmul_rn(a_scale[0], w_scale[0])}; }
+  __device__ __forceinline__ float value(AccT v, Row r, Col c) const { return __fmaf_rn((float)v, r.sc, c.b); }
+  __device__ __forceinline__ void store(int m, int n, AccT v, Row r, Col c) const {
+    store_from_f32<OUT>(y, (int64_t)m * ldy + n, value(v, r, c));
   }
 };
 
