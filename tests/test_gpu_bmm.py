@@ -74,7 +74,8 @@ def test_affine_quantizer_strided_input(dev):
 
 @pytest.mark.parametrize("shape", [(4, 256, 256, 128), (3, 300, 333, 128), (3, 100, 77, 64), (2, 300, 128, 320),
                                    (3, 300, 100, 640), (2, 700, 128, 1024),  # tall tiles, staggered reduction
-                                   (5, 64, 40, 192), (1, 513, 700, 256)])
+                                   (5, 64, 40, 192), (1, 513, 700, 256),
+                                   (40, 520, 700, 128)])  # 600 ragged tiles of the K = 128 kernel: its blocks walk several
 @pytest.mark.parametrize("with_bias", [False, True])
 def test_bmm_i8_exact(dev, shape, with_bias):
     B, M, N, Kd = shape
@@ -92,7 +93,7 @@ def test_bmm_i8_exact(dev, shape, with_bias):
 
 
 @pytest.mark.parametrize("shape", [(4, 256, 256, 128), (3, 300, 333, 128), (3, 100, 77, 64), (2, 130, 128, 384),
-                                   (3, 300, 100, 640)])
+                                   (3, 300, 100, 640), (40, 520, 700, 128)])
 def test_bmm_fp8_exact_on_integer_operands(dev, shape):
     B, M, N, Kd = shape
     g = gen(10)
