@@ -33,7 +33,7 @@ M_TOKENS = 4096
 
 
 def make_layer(torch, dev, K, N, seed):
-    """BASELINE config 2 inputs: x ~ N(0,1) with 1 % of the input channels scaled x50, W ~ N(0,0.02),
+    """Inputs of the headline configuration: x ~ N(0,1) with 1 % of the input channels scaled x50, W ~ N(0,0.02),
     SmoothQuant alpha = 0.5 with a_k = max_m |x_mk|.  Generated on the CPU from a seeded generator
     (so the CPU baseline sees the same bits), quantized offline with the deploy-module recipe."""
     from fms_mo_amd.modules.linear import prepare_deploy_weights

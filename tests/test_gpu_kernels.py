@@ -386,7 +386,7 @@ def test_gemm_i8_dq_reference_epilogue_bit_exact(dev, shape, out_dtype):
 
 
 def test_c1_config_deploy_forward(dev):
-    """BASELINE config 1: x fp16 [512,4096] ~N(0,1), W fp16 [4096,4096] ~N(0,0.02), bias
+    """The reference's CPU-runnable configuration: x fp16 [512,4096] ~N(0,1), W fp16 [4096,4096] ~N(0,0.02), bias
     ~N(0,0.01), per-token act / per-channel weight int8, seed 0."""
     g = gen(0)
     x = torch.randn(512, 4096, generator=g).half()
