@@ -70,6 +70,19 @@ def test_argument_validation_without_a_gpu():
     assert lib.fmsmo_matmul_chunk_fp(p, 64, p, 64, 1, None, p, 64, 1, 1, 64, 64, 23, 0, 1, None) == 4  # t > 22
     # empty problems are accepted without a launch
     assert lib.fmsmo_gemm_i8_i32(p, 64, p, 64, p, 64, 0, 1, 64, None) == 0
+    # the later entry points validate the same way
+    assert lib.fmsmo_debug_stream_read(None, 64, p, None) == 1
+    assert lib.fmsmo_debug_stream_read(p, 24, p, None) == 2 and lib.fmsmo_debug_stream_read(p, 0, p, None) == 2
+    assert lib.fmsmo_debug_stream_read(p + 1, 64, p, None) == 3
+    assert lib.fmsmo_quant_act_i8_static_t(None, 0, 64, 0, 0, 1.0, 0.0, 0, 0.0, 0.0, p, 64, 1, 64, None) == 1
+    assert lib.fmsmo_quant_act_i8_static_t(p, 0, 64, 9, 0, 1.0, 0.0, 0, 0.0, 0.0, p, 64, 1, 64, None) == 4  # mode
+    assert lib.fmsmo_quant_act_i8_static_t(p, 0, 32, 0, 0, 1.0, 0.0, 0, 0.0, 0.0, p, 64, 1, 64, None) == 2  # ldx < K
+    assert lib.fmsmo_quant_act_i8_dynamic(None, 0, 64, p, 0, 127, 0, p, 64, p, 1, 64, None) == 1
+    assert lib.fmsmo_quant_act_i8_dynamic(p, 0, 64, p, 5, 127, 0, p, 64, p, 1, 64, None) == 4  # granularity
+    assert lib.fmsmo_fake_quant_fp8(None, 0, 64, 0, None, p, 64, None, 0, None, None, 1, 64, None) == 1
+    assert lib.fmsmo_fake_quant_fp8(p, 0, 64, 7, None, p, 64, None, 0, None, None, 1, 64, None) == 4  # mode
+    assert lib.fmsmo_gemm_i8_dq_noalloc(None, 64, p, 64, p, 1, p, 1, None, 0, 0, p, 0, 64, 1, 1, 64, None) == 1
+    assert lib.fmsmo_gemm_i8_dq_noalloc(p, 64, p, 64, p, 1, p, 1, None, 0, 9, p, 0, 64, 1, 1, 64, None) == 4  # epilogue
 
 
 def test_python_wrapper_raises_on_cpu_tensors():
