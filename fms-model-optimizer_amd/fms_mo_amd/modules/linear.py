@@ -665,6 +665,16 @@ class QLinearINT8Deploy(nn.Linear):
             self._ws_f32 = ws.detach().float().reshape(-1).contiguous()
         return self._ws_f32
 
+    def _set_input_scale(self, s):
+        """Replace the ``input_scale`` buffer (the reference assigns it in every dynamic forward,
+        linear.py:1074-1082).  Eagerly the entry of the buffer table is swapped directly:
+        ``Module.__setattr__`` spends several microseconds per call on its checks, as much as a
+        decode kernel runs."""
+        if torch.compiler.is_compiling() or "input_scale" not in self._buffers:
+            self.input_scale = s
+        else:
+            self._buffers["input_scale"] = s
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         with torch.no_grad():
             org_dtype = x.dtype
@@ -682,12 +692,12 @@ class QLinearINT8Deploy(nn.Linear):
                 # single-token decode step: quantizer and weight-streaming matmul in one launch
                 y, s = kernels.decode_linear_i8(x2, self.weight, self._w_scale_f32(), self.bias, sq,
                                                 out_dtype=torch.float16, exact_ref=True)
-                self.input_scale = s.reshape(-1, 1)
+                self._set_input_scale(s.reshape(-1, 1))
                 y = y.to(self.acc_dtype)
             elif plain and use_sq and sq.numel() == x2.shape[1]:
                 # SmoothQuant divide inside the quantizer kernel
                 q, s = kernels.quant_act_i8_pertoken(x2, sq, compute_dtype=_compute_dtype(x2.dtype, sq))
-                self.input_scale = s.reshape(-1, 1)
+                self._set_input_scale(s.reshape(-1, 1))
                 y = kernels.gemm_i8_dq(q, self.weight, s, self._w_scale_f32(), self.bias,
                                        out_dtype=torch.float16, exact_ref=True).to(self.acc_dtype)
             else:
