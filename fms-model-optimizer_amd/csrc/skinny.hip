@@ -195,6 +195,154 @@ __device__ __forceinline__ void quantize_row_fp8_to_lds(const GemvArgs& g, uint8
   if (blockIdx.x == 0 && g.a_scale_out && threadIdx.x == 0) g.a_scale_out[0] = sc[0];
 }
 
+// The two quantizers above for ONE token row, split in two so that the caller can issue other
+// loads (the head of a weight stream) between the row's loads and their use: row_request() issues
+// the loads, row_finish_i8 / row_finish_fp8 do the arithmetic and leave codes and scale in LDS
+// (they end with a barrier).  Chunks past the row hold zeros.
+template <int NT, int NCH>
+__device__ __forceinline__ void row_request(const GemvArgs& g, v4i (&cur)[NCH], v4i (&sm)[NCH]) {
+  const int nchunk = g.K / AQ_VEC;
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) {
+    const int c = threadIdx.x + i * NT;
+    cur[i] = v4i{0, 0, 0, 0};
+    sm[i] = v4i{0, 0, 0, 0};
+    if (c < nchunk) {
+      cur[i] = *(const v4i*)(g.x16 + (size_t)c * AQ_VEC);
+      if (g.smooth) sm[i] = *(const v4i*)(g.smooth + (size_t)c * AQ_VEC);
+    }
+  }
+}
+
+template <int T, int NT, int NCH>
+__device__ __forceinline__ void row_finish_i8(const GemvArgs& g, v4i (&cur)[NCH], const v4i (&sm)[NCH],
+                                              uint8_t* xq, float* sc, float* red) {
+  const int nchunk = g.K / AQ_VEC;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  constexpr uint32_t INF_BITS = T == FMSMO_F16 ? 0x7c00u : 0x7f80u;
+  const float floor_T = cvt16<T>(to16<T>(1e-5f));
+  int bad = 0;
+  us2 amax2 = {0, 0};
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) {
+    const int c = threadIdx.x + i * NT;
+    if (c < nchunk) {
+      if (g.smooth) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const uint32_t w = (uint32_t)cur[i][j], d = (uint32_t)sm[i][j];
+          const float dl = cvt16<T>((u16)(d & 0xffff)), dh = cvt16<T>((u16)(d >> 16));
+          if constexpr (T == FMSMO_BF16)
+            bad |= !(fabsf(dl) >= 8.6736174e-19f && fabsf(dl) <= 1.1529215e18f) ||
+                   !(fabsf(dh) >= 8.6736174e-19f && fabsf(dh) <= 1.1529215e18f);
+          const u16 el = to16<T>(div16<T, false>(cvt16<T>((u16)(w & 0xffff)), dl, __builtin_amdgcn_rcpf(dl)));
+          const u16 eh = to16<T>(div16<T, false>(cvt16<T>((u16)(w >> 16)), dh, __builtin_amdgcn_rcpf(dh)));
+          cur[i][j] = (int)((uint32_t)el | ((uint32_t)eh << 16));
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const uint32_t mag = (uint32_t)cur[i][j] & 0x7fff7fffu;
+        us2 m2;
+        __builtin_memcpy(&m2, &mag, 4);
+        amax2 = __builtin_elementwise_max(amax2, m2);
+      }
+    }
+  }
+  float v = wave_max(__uint_as_float(bad ? 0xffffu : (uint32_t)(amax2[0] > amax2[1] ? amax2[0] : amax2[1])));
+  if (lane == 0) red[wave] = v;
+  __syncthreads();
+  v = red[0];
+#pragma unroll
+  for (int w = 1; w < NT / 64; ++w) v = fmaxf(v, red[w]);
+  __syncthreads();
+  const uint32_t abits = __float_as_uint(v);
+  if (abits >= INF_BITS) {
+    quant_i8_row_ieee16<T, NT>(g.x16, g.smooth, g.saturate, (int8_t*)xq, sc, g.K, red);
+  } else {
+    const float s = cvt16<T>(to16<T>(fmaxf(cvt16<T>((u16)abits), floor_T) / 127.0f));
+    const float rs = __builtin_amdgcn_rcpf(s);
+    if (threadIdx.x == 0) sc[0] = s;
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      const int c = threadIdx.x + i * NT;
+      if (c < nchunk) {
+        uint32_t code[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const uint32_t w = (uint32_t)cur[i][j];
+          float ql = div16<T, false>(cvt16<T>((u16)(w & 0xffff)), s, rs);
+          float qh = div16<T, false>(cvt16<T>((u16)(w >> 16)), s, rs);
+          if (g.saturate) {
+            ql = fminf(fmaxf(ql, -127.0f), 127.0f);
+            qh = fminf(fmaxf(qh, -127.0f), 127.0f);
+          }
+          code[j] = rint_codes<T>(to16<T>(ql), to16<T>(qh));
+        }
+        const uint32_t o0 = __builtin_amdgcn_perm(code[1], code[0], 0x06040200u);
+        const uint32_t o1 = __builtin_amdgcn_perm(code[3], code[2], 0x06040200u);
+        *(uint2*)(xq + (size_t)c * AQ_VEC) = make_uint2(o0, o1);
+      }
+    }
+  }
+  __syncthreads();
+  if (blockIdx.x == 0 && g.a_scale_out && threadIdx.x == 0) g.a_scale_out[0] = sc[0];
+}
+
+template <int XT, int NT, int NCH>
+__device__ __forceinline__ void row_finish_fp8(const GemvArgs& g, const v4i (&cur)[NCH], uint8_t* xq, float* sc,
+                                               float* red) {
+  const int nchunk = g.K / AQ_VEC;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  constexpr uint32_t INF_BITS = XT == FMSMO_F16 ? 0x7c00u : 0x7f80u;
+  us2 amax2 = {0, 0};
+#pragma unroll
+  for (int i = 0; i < NCH; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {  // (chunks past the row are zero)
+      const uint32_t mag = (uint32_t)cur[i][j] & 0x7fff7fffu;
+      us2 m2;
+      __builtin_memcpy(&m2, &mag, 4);
+      amax2 = __builtin_elementwise_max(amax2, m2);
+    }
+  float v = wave_max(__uint_as_float((uint32_t)(amax2[0] > amax2[1] ? amax2[0] : amax2[1])));
+  if (lane == 0) red[wave] = v;
+  __syncthreads();
+  v = red[0];
+#pragma unroll
+  for (int w = 1; w < NT / 64; ++w) v = fmaxf(v, red[w]);
+  const uint32_t abits = __float_as_uint(v);
+  const float s = fmaxf(cvt16<XT>((u16)abits) / 448.0f, 1e-12f);
+  if (threadIdx.x == 0) sc[0] = s;
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) {
+    const int c = threadIdx.x + i * NT;
+    if (c < nchunk) {
+      float t[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float xv = cvt16<XT>((u16)((uint32_t)cur[i][j >> 1] >> ((j & 1) * 16)));
+        t[j] = fminf(fmaxf(xv / s, -448.0f), 448.0f);
+      }
+      if (abits < INF_BITS) {
+        int o0 = 0, o1 = 0;
+        o0 = __builtin_amdgcn_cvt_pk_fp8_f32(t[0], t[1], o0, false);
+        o0 = __builtin_amdgcn_cvt_pk_fp8_f32(t[2], t[3], o0, true);
+        o1 = __builtin_amdgcn_cvt_pk_fp8_f32(t[4], t[5], o1, false);
+        o1 = __builtin_amdgcn_cvt_pk_fp8_f32(t[6], t[7], o1, true);
+        *(uint2*)(xq + (size_t)c * AQ_VEC) = make_uint2((uint32_t)o0, (uint32_t)o1);
+      } else {
+        uint8_t b[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) b[j] = f32_to_e4m3_sw(t[j]);
+        store8(xq, (size_t)c * AQ_VEC, b);
+      }
+    }
+  }
+  __syncthreads();
+  if (blockIdx.x == 0 && g.a_scale_out && threadIdx.x == 0) g.a_scale_out[0] = sc[0];
+}
+
 template <int OP, int RG, int NW>
 __global__ __launch_bounds__(NW * 64) void gemv_kernel(GemvArgs g) {
   typedef typename std::conditional<OP == FMSMO_OP_I8, int, float>::type AccT;
@@ -308,10 +456,21 @@ __global__ __launch_bounds__(NW * 64) void gemv_kernel(GemvArgs g) {
 // upper 8 rows are neither loaded nor stored.
 // HALF = false: the host has checked that every block owns whole groups only (the loads of the
 // upper rows are then unconditional, which the register allocation of the long-row shapes needs).
-template <int OP, int STEPS, int NW, int D, int MT = 1, bool HALF = false, bool XS = false>
+// XT >= 0 (fused decode linear, one token of dtype XT, with XS): the block quantizes the token
+// row itself, into LDS -- its loads are issued first, the head of the weight stream next, and the
+// quantizer's arithmetic runs while those weights are in flight -- and the activation fragments
+// are read from there (token rows 1..15 of the MFMA operand are zeros).
+template <int OP, int STEPS, int NW, int D, int MT = 1, bool HALF = false, bool XS = false, int XT = -1>
 __global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(GemvArgs g, int halves) {
   static_assert(STEPS % D == 0, "pipeline depth must divide the steps per group");
   static_assert(!XS || MT == 1, "streamed activations: one tile of tokens");
+  constexpr bool FUSED = XT >= 0;
+  static_assert(!FUSED || XS, "the fused form streams its activations");
+  constexpr int KROW = NW * STEPS * 128;
+  constexpr int QCH = (KROW / AQ_VEC + NW * 64 - 1) / (NW * 64);  // 16-byte chunks of the row per thread
+  __shared__ __attribute__((aligned(16))) uint8_t xq[FUSED ? KROW : 16];
+  __shared__ float xsc[1];
+  __shared__ float xred[NW];
   typedef typename std::conditional<OP == FMSMO_OP_I8, int, float>::type AccT;
   typedef AccT Acc4 __attribute__((ext_vector_type(4)));
   constexpr int NRED = 2;  // exchange buffers alternate, one barrier per group
@@ -369,16 +528,19 @@ __global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(GemvArgs g, int ha
   // fragments held and two steps in flight, 11.4 / 13.8 streamed with seven; starting the blocks
   // at different K steps so that they do not all ask L2 for the same lines at once: 11.7 / 14.3).
   v4i xf[XS ? 1 : MT][XS ? 1 : STEPS][2];
-  v4i xb[XS ? D : 1][2];
+  v4i xb[XS && !FUSED ? D : 1][2];
+  v4i qcur[FUSED ? QCH : 1], qsm[FUSED ? QCH : 1];
   const __amdgpu_buffer_rsrc_t rsrc_x = __builtin_amdgcn_make_buffer_rsrc(
-      (void*)g.a, 0, (int)((int64_t)(g.M - 1) * g.lda + g.K), 0x00020000);
+      (void*)g.a, 0, FUSED ? 0 : (int)((int64_t)(g.M - 1) * g.lda + g.K), 0x00020000);
   const int vx = r * (int)g.lda + kwave + kg * 16;
   auto load_x = [&](int t, int s, v4i (&x)[2]) {
     const int v = vx + t * 16 * (int)g.lda;
     x[0] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_x, v, s * 128, 0));
     x[1] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_x, v, s * 128 + 64, 0));
   };
-  if constexpr (XS) {
+  if constexpr (FUSED) {
+    row_request<NW * 64, QCH>(g, qcur, qsm);
+  } else if constexpr (XS) {
 #pragma unroll
     for (int j = 0; j < D; ++j) load_x(0, j, xb[j]);
   } else {
@@ -395,7 +557,17 @@ __global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(GemvArgs g, int ha
   // epilogue operands of output element e = threadIdx.x (n = e / 16, m = e % 16 of the group) are
   // fetched at the top of each group so that their latency hides behind the weight stream
   const int em = min((int)(threadIdx.x & 15), g.M - 1);
-  const float as = g.a_scale[g.a_stride ? em : 0];
+  float as;
+  if constexpr (FUSED) {
+    if constexpr (OP == FMSMO_OP_I8) row_finish_i8<XT, NW * 64, QCH>(g, qcur, qsm, xq, xsc, xred);
+    else row_finish_fp8<XT, NW * 64, QCH>(g, qcur, xq, xsc, xred);
+    as = xsc[0];
+  } else {
+    as = g.a_scale[g.a_stride ? em : 0];
+  }
+  // fused: the token's codes of this lane's K positions (lanes of token rows 1..15 read zeros)
+  const uint8_t* xl = xq + (FUSED ? kwave + kg * 16 : 0);
+  const bool xrow0 = r == 0;
 
   // The last group of a block refills nothing (its prefetches would fall into the next block's
   // rows), so the group body exists twice: streaming (LAST = false) and draining (LAST = true).
@@ -424,7 +596,14 @@ __global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(GemvArgs g, int ha
       const v4i w1 = *(const v4i*)(st + rd1);
 #pragma unroll
       for (int t = 0; t < MT; ++t) {
-        const v4i x0 = XS ? xb[s % D][0] : xf[t][s][0], x1 = XS ? xb[s % D][1] : xf[t][s][1];
+        v4i x0, x1;
+        if constexpr (FUSED) {
+          const v4i z = {0, 0, 0, 0};
+          x0 = *(const v4i*)(xl + s * 128), x1 = *(const v4i*)(xl + s * 128 + 64);
+          x0 = xrow0 ? x0 : z, x1 = xrow0 ? x1 : z;
+        } else {
+          x0 = XS ? xb[s % D][0] : xf[t][s][0], x1 = XS ? xb[s % D][1] : xf[t][s][1];
+        }
         if constexpr (OP == FMSMO_OP_I8) {
           acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w0, x0, acc[t], 0, 0, 0);
           acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w1, x1, acc[t], 0, 0, 0);
@@ -434,7 +613,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(GemvArgs g, int ha
           acc[t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wv, xv, acc[t], 0, 0, 0, 0, 0, 0);
         }
       }
-      if constexpr (XS) {  // the same K offsets serve every group: the refill wraps around
+      if constexpr (XS && !FUSED) {  // the same K offsets serve every group: the refill wraps around
         __builtin_amdgcn_sched_barrier(0);
         if (!LAST || s + D < STEPS) load_x(0, (s + D) % STEPS, xb[s % D]);
         __builtin_amdgcn_sched_barrier(0);
@@ -847,18 +1026,39 @@ int fmsmo_gemv_dispatch(int op, const void* a, int64_t lda, const void* b, int64
 }
 
 // ---------------------------------------------------------------------- fused decode linear
-// One token and K <= 8192 (measured from a HIP graph against the two launches, us: qkv 9.6 -> 8.3,
-// o 8.1 -> 6.3, gate+up 23.4 -> 19.7).  With more tokens or longer rows the quantization every
-// block repeats costs more than the launch it saves (K = 14336: 16.5 -> 19.6; two tokens at
-// K = 4096: 10.3 -> 10.9), so those shapes are left to the two kernels.
+// One token.  K <= 8192: the row kernel quantizes the token in every block (measured from a HIP
+// graph against the two launches, us: qkv 9.6 -> 8.3, o 8.1 -> 6.3, gate+up 23.4 -> 19.7).  With
+// longer rows the quantization its 1024 small blocks repeat costs more than the launch it saves
+// (K = 14336: 16.5 -> 19.6), so K = 14336 and K = 12800 take the streaming kernel's fused form:
+// 256 blocks of 8 / 10 waves quantize the row once each while the head of their weight stream is
+// in flight (N = 4096, int8 from fp16 / bf16 with SmoothQuant / e4m3: K = 14336 14.5 -> 11.4,
+// 16.6 -> 12.7, 17.5 -> 12.2; K = 12800 13.6 -> 10.6, 15.6 -> 11.6, 16.6 -> 11.9).  Two tokens at
+// K = 4096 lose (10.3 -> 10.9): more tokens are left to the two kernels.
 extern "C" int fmsmo_decode_linear_ok(int64_t M, int64_t K) {
   if (M != 1 || K % 128 || K < 1024) return 0;
+  if (K == 14336 || K == 12800) return 1;  // the streaming kernel's fused form
   const int kch = (int)((K + 1023) / 1024);
   return kch == 1 || kch == 2 || kch == 4 || kch == 8;
 }
 
 template <int OP, int XT>
 static int decode_fused_launch(const GemvArgs& g, hipStream_t st) {
+  if (g.K == 14336 || g.K == 12800) {
+    // one group of 16 weight rows per block at most (the fused form streams its activations)
+    const int halves = (g.N + 7) / 8;
+    int nblocks = halves < 256 ? halves : 256;
+    if (2 * nblocks < halves) nblocks = (halves + 1) / 2;
+    const bool whole_groups = halves % (2 * nblocks) == 0;
+    dim3 grid((unsigned)nblocks);
+#define STREAM_F(NWV, ST, DV)                                                                        \
+  if (whole_groups)                                                                                  \
+    hipLaunchKernelGGL((gemv_stream_kernel<OP, ST, NWV, DV, 1, false, true, XT>), grid, dim3(NWV * 64), 0, st, g, halves); \
+  else                                                                                               \
+    hipLaunchKernelGGL((gemv_stream_kernel<OP, ST, NWV, DV, 1, true, true, XT>), grid, dim3(NWV * 64), 0, st, g, halves)
+    if (g.K == 14336) { STREAM_F(8, 14, 7); } else { STREAM_F(10, 10, 5); }
+#undef STREAM_F
+    return fmsmo_check_launch();
+  }
   const int kch = (int)((g.K + 1023) / 1024);
 #define ROWS(KCHV, UV)                                                                            \
   {                                                                                                \

@@ -374,10 +374,11 @@ int fmsmo_gemv_fp8_dq(const uint8_t* a, int64_t lda, const uint8_t* b, int64_t l
  * two calls in sequence while a kernel launch and the round trip of the codes through memory are
  * saved in front of every linear layer of a single-stream decode step.  a_scale_out (fp32 [1],
  * may be NULL) receives the token's scale (the reference's input_scale side effect).
- * fmsmo_decode_linear_ok(M, K) != 0 tells whether a shape is served: M == 1 and K <= 8192 in one
- * of the decode kernel's sizes (1024, 2048, 4096, 8192 and what pads to them); with more tokens
- * or longer rows the quantization that every block repeats costs more than the launch it saves,
- * and the call returns FMSMO_ERR_UNSUPPORTED: use the two kernels.
+ * fmsmo_decode_linear_ok(M, K) != 0 tells whether a shape is served: M == 1 and either K <= 8192
+ * in one of the row kernel's sizes (1024, 2048, 4096, 8192 and what pads to them) or K = 14336 /
+ * 12800 (the streaming kernel quantizes the row while the head of its weight stream is in
+ * flight); with more tokens or other row lengths the quantization that every block repeats costs
+ * more than the launch it saves, and the call returns FMSMO_ERR_UNSUPPORTED: use the two kernels.
  * x and smooth 16-byte aligned, ldx % 8 == 0, w as for fmsmo_gemv_i8_dq.
  * Reference: QLinearINT8Deploy.forward for a decode step -- qa_dynamic_max_qfunc followed by
  * iaddmm_int (fms_mo/modules/linear.py:1085-1100, 1177-1188, 1309-1338); no fused counterpart.
@@ -390,8 +391,10 @@ int fmsmo_decode_linear_i8(const void* x, int x_dtype, int64_t ldx, const void* 
                            int64_t N, int64_t K, fmsmo_stream_t stream);
 /*
  * The same for e4m3 weights: the block quantizes the token with the dynamic per-token recipe of
- * fmsmo_quant_act_fp8_pertoken(FMSMO_FP8_LINEAR) and runs fmsmo_gemv_fp8_dq's kernel on it;
- * bit-identical to the two calls.  Served shapes as told by fmsmo_decode_linear_ok.
+ * fmsmo_quant_act_fp8_pertoken(FMSMO_FP8_LINEAR) and runs fmsmo_gemv_fp8_dq's kernel on it:
+ * scale and codes are the quantizer's bit for bit, and so is the result wherever the two-call
+ * path streams the weights in the same shape (K <= 8192; K = 14336 with N <= 4096); elsewhere the
+ * fp32 partial sums are added in another order.  Served shapes as told by fmsmo_decode_linear_ok.
  * Reference: FP8Linear.forward with dynamic activation scales
  * (fms_mo/aiu_addons/fp8/fp8_linear.py:217-283) on one token.
  */

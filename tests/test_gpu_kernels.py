@@ -823,7 +823,11 @@ def test_split_k_gemm_replays_from_a_hip_graph(dev):
 
 # ------------------------------------------------------------------ fused decode linear
 @pytest.mark.parametrize("NK", [(4096, 4096), (6144, 4096), (520, 1024), (1000, 2048), (256, 8192), (28672, 4096),
-                                (96, 1536), (64, 3584)])
+                                (96, 1536), (64, 3584),
+                                # long rows: the streaming kernel's fused form (whole and half row
+                                # groups, fewer and more than one group per compute unit)
+                                (4096, 14336), (1000, 14336), (4104, 14336), (8200, 14336), (24, 14336),
+                                (4096, 12800), (1016, 12800)])
 @pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("smooth", [False, True])
 def test_fused_decode_linear_is_bit_identical_to_the_two_kernels(dev, NK, dt, smooth):
@@ -849,11 +853,12 @@ def test_fused_decode_linear_is_bit_identical_to_the_two_kernels(dev, NK, dt, sm
 
 
 @pytest.mark.parametrize("row", ["zeros", "inf", "overflow"])
-def test_fused_decode_linear_special_rows(dev, row):
+@pytest.mark.parametrize("Kd", [4096, 14336])
+def test_fused_decode_linear_special_rows(dev, row, Kd):
     """Rows that leave the fast division path (all zeros, an infinity, an fp16 overflow after the
     SmoothQuant divide) must come out like the stand-alone quantizer's."""
     kn = K()
-    Kd, N = 4096, 512
+    N = 512
     x = torch.randn(1, Kd, generator=gen(181)).half()
     sm = (torch.rand(Kd, generator=gen(182)) * 3 + 0.2).half()
     if row == "zeros":
@@ -878,7 +883,9 @@ def test_fused_decode_linear_rejects_what_it_does_not_serve(dev):
     x = torch.randn(2, 4096, device=dev).half()
     assert not kn.decode_linear_ok(x, None, 4096)                          # more than one token
     assert not kn.decode_linear_ok(x[:1].float(), None, 4096)              # fp32 activations
-    assert not kn.decode_linear_ok(torch.randn(1, 14336, device=dev).half(), None, 14336)  # long rows
+    assert not kn.decode_linear_ok(torch.randn(1, 16384, device=dev).half(), None, 16384)  # long rows
+    assert not kn.decode_linear_ok(torch.randn(4, 14336, device=dev).half(), None, 14336)
+    assert kn.decode_linear_ok(torch.randn(1, 14336, device=dev).half(), None, 14336)
     assert not kn.decode_linear_ok(x[:1], torch.ones(4096, device=dev), 4096)  # fp32 divisors
     assert kn.decode_linear_ok(x[:1], None, 4096)
     w = torch.zeros(64, 4096, dtype=torch.int8, device=dev)
@@ -912,3 +919,47 @@ def test_fused_decode_linear_fp8_is_bit_identical_to_the_two_kernels(dev, NK, dt
         assert torch.equal(s_f.view(torch.int32), s.view(torch.int32))
         bits = torch.int32 if od == torch.float32 else torch.int16
         assert torch.equal(y.view(bits), ref.view(bits))
+
+
+@pytest.mark.parametrize("NK", [(4096, 14336), (1000, 14336), (8200, 14336), (4096, 12800), (1016, 12800)])
+@pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("special", [None, "zeros", "inf"])
+def test_fused_decode_linear_fp8_long_rows(dev, NK, dt, special):
+    """Long rows take the streaming kernel's fused form.  The quantized token is the stand-alone
+    quantizer's bit for bit (scale; codes through an exact product with power-of-two weights);
+    the product with random weights equals the two kernels' up to the order of the fp32 sums,
+    which differs where they stream the weights in another shape (rtol 1e-5 on fp32 outputs)."""
+    from fms_mo_amd import _lib as L
+
+    N, Kd = NK
+    kn = K()
+    x = (2.0 * torch.randn(1, Kd, generator=gen(195))).to(dt)
+    x[0, 3] = -0.0
+    if special == "zeros":
+        x[0] = 0.0
+    elif special == "inf":
+        x[0, 9] = float("inf")
+    xd = x.to(dev)
+    assert kn.decode_linear_ok(xd, None, Kd)
+    q, s = kn.quant_act_fp8_pertoken(xd, L.FP8_LINEAR)
+    # (a) codes: weight row n = one power of two at column n (mod Kd) -> y[n] is code n exactly
+    n_id = min(N, Kd)
+    w_id = torch.zeros(N, Kd)
+    w_id[torch.arange(n_id), torch.arange(n_id)] = 1.0
+    w_id = w_id.to(torch.float8_e4m3fn).to(dev)
+    ones = torch.ones(N, device=dev)
+    y_id, s_f = kn.decode_linear_fp8(xd, w_id, ones, None, out_dtype=torch.float32)
+    assert torch.equal(s_f.view(torch.int32), s.view(torch.int32))
+    want = q.float()[0, :n_id] * s
+    got = y_id[0, :n_id]
+    assert torch.equal(torch.nan_to_num(got, nan=7.0), torch.nan_to_num(want, nan=7.0))
+    # (b) random weights against the two kernels
+    w = _rand_fp8((N, Kd), 196, 0.5).to(dev)
+    s_w = (torch.rand(N, generator=gen(197)) * 0.01 + 1e-4).to(dev)
+    bias = (torch.randn(N, generator=gen(198)) * 0.1).to(dt).to(dev)
+    ref = kn.gemm_fp8_dq(q, w, s, s_w, bias, out_dtype=torch.float32)
+    y, _ = kn.decode_linear_fp8(xd, w, s_w, bias, out_dtype=torch.float32)
+    if special == "inf":
+        assert torch.equal(torch.isnan(y), torch.isnan(ref))
+    else:
+        torch.testing.assert_close(y, ref, rtol=1e-5, atol=1e-5)
