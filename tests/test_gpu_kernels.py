@@ -827,7 +827,7 @@ def test_split_k_gemm_replays_from_a_hip_graph(dev):
                                 # long rows: the streaming kernel's fused form (whole and half row
                                 # groups, fewer and more than one group per compute unit)
                                 (4096, 14336), (1000, 14336), (4104, 14336), (8200, 14336), (24, 14336),
-                                (4096, 12800), (1016, 12800)])
+                                (4096, 12800), (1016, 12800), (1024, 4096), (1000, 4096), (4104, 4096)])
 @pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("smooth", [False, True])
 def test_fused_decode_linear_is_bit_identical_to_the_two_kernels(dev, NK, dt, smooth):
