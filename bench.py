@@ -460,14 +460,14 @@ def extras(torch, K, dev, layers):
         ws_i8 = [torch.randint(-127, 128, (n, k), dtype=torch.int8, device=dev) for _ in range(copies)]
         wsc = torch.rand(n, device=dev) * 1e-3
         sm = (torch.rand(k, device=dev) + 0.5).half()
-        for M in (1,):
+        for M in (1, 2, 4):
             x = torch.randn(M, k, device=dev).half()
 
             def two(w):
                 q, s = K.quant_act_i8_pertoken(x, sm)
                 return K.gemm_i8_dq(q, w, s, wsc, None, out_dtype=torch.float16, exact_ref=True)
 
-            def one(w):  # the fused launch where it is served (K <= 8192), else the same two
+            def one(w):  # the fused launch where it is served, else the same two
                 if not K.decode_linear_ok(x, sm, k):
                     return two(w)
                 return K.decode_linear_i8(x, w, wsc, None, sm, out_dtype=torch.float16, exact_ref=True)[0]

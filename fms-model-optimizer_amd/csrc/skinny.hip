@@ -195,152 +195,218 @@ __device__ __forceinline__ void quantize_row_fp8_to_lds(const GemvArgs& g, uint8
   if (blockIdx.x == 0 && g.a_scale_out && threadIdx.x == 0) g.a_scale_out[0] = sc[0];
 }
 
-// The two quantizers above for ONE token row, split in two so that the caller can issue other
-// loads (the head of a weight stream) between the row's loads and their use: row_request() issues
-// the loads, row_finish_i8 / row_finish_fp8 do the arithmetic and leave codes and scale in LDS
-// (they end with a barrier).  Chunks past the row hold zeros.
-template <int NT, int NCH>
-__device__ __forceinline__ void row_request(const GemvArgs& g, v4i (&cur)[NCH], v4i (&sm)[NCH]) {
-  const int nchunk = g.K / AQ_VEC;
+// The two quantizers above for up to MAXM token rows of KROW elements, split in two so that the
+// caller can issue other loads (the head of a weight stream) between the rows' loads and their
+// use: rows_request() issues the loads, rows_finish_i8 / rows_finish_fp8 do the arithmetic and
+// leave codes (row stride xstride bytes) and scales in LDS; they end with a barrier.
+// Threads are dealt to the rows so that a wave stays inside one row: with at least as many threads
+// as a row has 16-byte chunks, RPP rows are worked on at once, one chunk per thread; otherwise
+// every thread takes QCH chunks of one row at a time.
+template <int NT, int KROW, int MAXM_>
+struct RowsPlan {
+  static constexpr int MAXM = MAXM_;
+  static constexpr int CPR = KROW / AQ_VEC;            // chunks per row
+  static constexpr int TPR = NT >= CPR ? CPR : NT;     // threads per row
+  static constexpr int RPP = NT / TPR;                 // rows per pass
+  static constexpr int QCH = (CPR + TPR - 1) / TPR;    // chunks per thread and row
+  static constexpr int NPASS = (MAXM + RPP - 1) / RPP;
+  static constexpr int WPR = TPR / 64;                 // waves per row
+  static constexpr int NTHREADS = NT;
+  static_assert(TPR % 64 == 0 && NT % TPR == 0 && KROW % AQ_VEC == 0, "a wave stays inside one row");
+};
+
+template <class P>
+__device__ __forceinline__ void rows_request(const GemvArgs& g, v4i (&cur)[P::NPASS][P::QCH], v4i (&sm)[P::QCH]) {
+  const int tr = threadIdx.x % P::TPR, rs = threadIdx.x / P::TPR;
 #pragma unroll
-  for (int i = 0; i < NCH; ++i) {
-    const int c = threadIdx.x + i * NT;
-    cur[i] = v4i{0, 0, 0, 0};
+  for (int i = 0; i < P::QCH; ++i) {
+    const int c = tr + i * P::TPR;
     sm[i] = v4i{0, 0, 0, 0};
-    if (c < nchunk) {
-      cur[i] = *(const v4i*)(g.x16 + (size_t)c * AQ_VEC);
-      if (g.smooth) sm[i] = *(const v4i*)(g.smooth + (size_t)c * AQ_VEC);
+    if (c < P::CPR && g.smooth) sm[i] = *(const v4i*)(g.smooth + (size_t)c * AQ_VEC);
+  }
+#pragma unroll
+  for (int j = 0; j < P::NPASS; ++j) {
+    const int m = j * P::RPP + rs;
+#pragma unroll
+    for (int i = 0; i < P::QCH; ++i) {
+      const int c = tr + i * P::TPR;
+      cur[j][i] = v4i{0, 0, 0, 0};
+      if (m < g.M && c < P::CPR) cur[j][i] = *(const v4i*)(g.x16 + (size_t)m * g.ldx + (size_t)c * AQ_VEC);
     }
   }
 }
 
-template <int T, int NT, int NCH>
-__device__ __forceinline__ void row_finish_i8(const GemvArgs& g, v4i (&cur)[NCH], const v4i (&sm)[NCH],
-                                              uint8_t* xq, float* sc, float* red) {
-  const int nchunk = g.K / AQ_VEC;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+// red: P::MAXM * P::WPR floats, followed by NT / 64 for the IEEE routine; sc: P::MAXM
+template <int T, class P>
+__device__ __forceinline__ void rows_finish_i8(const GemvArgs& g, v4i (&cur)[P::NPASS][P::QCH],
+                                               const v4i (&sm)[P::QCH], uint8_t* xq, int xstride, float* sc,
+                                               float* red) {
+  const int tr = threadIdx.x % P::TPR, rs = threadIdx.x / P::TPR;
+  const int lane = threadIdx.x & 63, wrow = tr >> 6;
   constexpr uint32_t INF_BITS = T == FMSMO_F16 ? 0x7c00u : 0x7f80u;
   const float floor_T = cvt16<T>(to16<T>(1e-5f));
-  int bad = 0;
-  us2 amax2 = {0, 0};
 #pragma unroll
-  for (int i = 0; i < NCH; ++i) {
-    const int c = threadIdx.x + i * NT;
-    if (c < nchunk) {
-      if (g.smooth) {
+  for (int j = 0; j < P::NPASS; ++j) {
+    const int m = j * P::RPP + rs;  // uniform in a wave
+    int bad = 0;
+    us2 amax2 = {0, 0};
+    if (m < g.M) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const uint32_t w = (uint32_t)cur[i][j], d = (uint32_t)sm[i][j];
-          const float dl = cvt16<T>((u16)(d & 0xffff)), dh = cvt16<T>((u16)(d >> 16));
-          if constexpr (T == FMSMO_BF16)
-            bad |= !(fabsf(dl) >= 8.6736174e-19f && fabsf(dl) <= 1.1529215e18f) ||
-                   !(fabsf(dh) >= 8.6736174e-19f && fabsf(dh) <= 1.1529215e18f);
-          const u16 el = to16<T>(div16<T, false>(cvt16<T>((u16)(w & 0xffff)), dl, __builtin_amdgcn_rcpf(dl)));
-          const u16 eh = to16<T>(div16<T, false>(cvt16<T>((u16)(w >> 16)), dh, __builtin_amdgcn_rcpf(dh)));
-          cur[i][j] = (int)((uint32_t)el | ((uint32_t)eh << 16));
-        }
-      }
+      for (int i = 0; i < P::QCH; ++i) {
+        const int c = tr + i * P::TPR;
+        if (c < P::CPR) {
+          if (g.smooth) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const uint32_t mag = (uint32_t)cur[i][j] & 0x7fff7fffu;
-        us2 m2;
-        __builtin_memcpy(&m2, &mag, 4);
-        amax2 = __builtin_elementwise_max(amax2, m2);
-      }
-    }
-  }
-  float v = wave_max(__uint_as_float(bad ? 0xffffu : (uint32_t)(amax2[0] > amax2[1] ? amax2[0] : amax2[1])));
-  if (lane == 0) red[wave] = v;
-  __syncthreads();
-  v = red[0];
-#pragma unroll
-  for (int w = 1; w < NT / 64; ++w) v = fmaxf(v, red[w]);
-  __syncthreads();
-  const uint32_t abits = __float_as_uint(v);
-  if (abits >= INF_BITS) {
-    quant_i8_row_ieee16<T, NT>(g.x16, g.smooth, g.saturate, (int8_t*)xq, sc, g.K, red);
-  } else {
-    const float s = cvt16<T>(to16<T>(fmaxf(cvt16<T>((u16)abits), floor_T) / 127.0f));
-    const float rs = __builtin_amdgcn_rcpf(s);
-    if (threadIdx.x == 0) sc[0] = s;
-#pragma unroll
-    for (int i = 0; i < NCH; ++i) {
-      const int c = threadIdx.x + i * NT;
-      if (c < nchunk) {
-        uint32_t code[4];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const uint32_t w = (uint32_t)cur[i][j];
-          float ql = div16<T, false>(cvt16<T>((u16)(w & 0xffff)), s, rs);
-          float qh = div16<T, false>(cvt16<T>((u16)(w >> 16)), s, rs);
-          if (g.saturate) {
-            ql = fminf(fmaxf(ql, -127.0f), 127.0f);
-            qh = fminf(fmaxf(qh, -127.0f), 127.0f);
+            for (int q = 0; q < 4; ++q) {
+              const uint32_t w = (uint32_t)cur[j][i][q], d = (uint32_t)sm[i][q];
+              const float dl = cvt16<T>((u16)(d & 0xffff)), dh = cvt16<T>((u16)(d >> 16));
+              if constexpr (T == FMSMO_BF16)
+                bad |= !(fabsf(dl) >= 8.6736174e-19f && fabsf(dl) <= 1.1529215e18f) ||
+                       !(fabsf(dh) >= 8.6736174e-19f && fabsf(dh) <= 1.1529215e18f);
+              const u16 el = to16<T>(div16<T, false>(cvt16<T>((u16)(w & 0xffff)), dl, __builtin_amdgcn_rcpf(dl)));
+              const u16 eh = to16<T>(div16<T, false>(cvt16<T>((u16)(w >> 16)), dh, __builtin_amdgcn_rcpf(dh)));
+              cur[j][i][q] = (int)((uint32_t)el | ((uint32_t)eh << 16));
+            }
           }
-          code[j] = rint_codes<T>(to16<T>(ql), to16<T>(qh));
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const uint32_t mag = (uint32_t)cur[j][i][q] & 0x7fff7fffu;
+            us2 m2;
+            __builtin_memcpy(&m2, &mag, 4);
+            amax2 = __builtin_elementwise_max(amax2, m2);
+          }
         }
-        const uint32_t o0 = __builtin_amdgcn_perm(code[1], code[0], 0x06040200u);
-        const uint32_t o1 = __builtin_amdgcn_perm(code[3], code[2], 0x06040200u);
-        *(uint2*)(xq + (size_t)c * AQ_VEC) = make_uint2(o0, o1);
+      }
+      // non-negative floats order like their bit patterns (a NaN outranks inf; a divisor outside
+      // the fast path's range marks the row for the IEEE routine)
+      const float v = wave_max(__uint_as_float(bad ? 0xffffu : (uint32_t)(amax2[0] > amax2[1] ? amax2[0] : amax2[1])));
+      if (lane == 0) red[m * P::WPR + wrow] = v;
+    }
+  }
+  __syncthreads();
+  // every thread forms every row's maximum itself (broadcast reads; no second barrier)
+  uint32_t rowbits[P::MAXM];
+  uint32_t off_fast = 0;  // (uniform) rows for the IEEE routine
+#pragma unroll
+  for (int m = 0; m < P::MAXM; ++m) {
+    rowbits[m] = 0;
+    if (m < g.M) {
+      float v = red[m * P::WPR];
+#pragma unroll
+      for (int w = 1; w < P::WPR; ++w) v = fmaxf(v, red[m * P::WPR + w]);
+      rowbits[m] = __float_as_uint(v);
+      if (rowbits[m] >= INF_BITS) off_fast |= 1u << m;
+    }
+  }
+  if (off_fast)
+    for (int m = 0; m < g.M; ++m)  // by the whole block, with scratch of their own
+      if (off_fast >> m & 1)
+        quant_i8_row_ieee16<T, P::NTHREADS>(g.x16 + (size_t)m * g.ldx, g.smooth, g.saturate,
+                                            (int8_t*)(xq + (size_t)m * xstride), sc + m, g.K, red + P::MAXM * P::WPR);
+#pragma unroll
+  for (int j = 0; j < P::NPASS; ++j) {
+    const int m = j * P::RPP + rs;
+    uint32_t abits = 0;
+#pragma unroll
+    for (int q = 0; q < P::RPP; ++q)
+      if (j * P::RPP + q < P::MAXM && rs == q) abits = rowbits[j * P::RPP + q];
+    if (m < g.M && abits < INF_BITS) {
+      const float s = cvt16<T>(to16<T>(fmaxf(cvt16<T>((u16)abits), floor_T) / 127.0f));
+      const float rcp_s = __builtin_amdgcn_rcpf(s);
+      if (tr == 0) sc[m] = s;
+#pragma unroll
+      for (int i = 0; i < P::QCH; ++i) {
+        const int c = tr + i * P::TPR;
+        if (c < P::CPR) {
+          uint32_t code[4];
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const uint32_t w = (uint32_t)cur[j][i][q];
+            float ql = div16<T, false>(cvt16<T>((u16)(w & 0xffff)), s, rcp_s);
+            float qh = div16<T, false>(cvt16<T>((u16)(w >> 16)), s, rcp_s);
+            if (g.saturate) {
+              ql = fminf(fmaxf(ql, -127.0f), 127.0f);
+              qh = fminf(fmaxf(qh, -127.0f), 127.0f);
+            }
+            code[q] = rint_codes<T>(to16<T>(ql), to16<T>(qh));
+          }
+          const uint32_t o0 = __builtin_amdgcn_perm(code[1], code[0], 0x06040200u);
+          const uint32_t o1 = __builtin_amdgcn_perm(code[3], code[2], 0x06040200u);
+          *(uint2*)(xq + (size_t)m * xstride + (size_t)c * AQ_VEC) = make_uint2(o0, o1);
+        }
       }
     }
   }
   __syncthreads();
-  if (blockIdx.x == 0 && g.a_scale_out && threadIdx.x == 0) g.a_scale_out[0] = sc[0];
+  if (blockIdx.x == 0 && g.a_scale_out && (int)threadIdx.x < g.M) g.a_scale_out[threadIdx.x] = sc[threadIdx.x];
 }
 
-template <int XT, int NT, int NCH>
-__device__ __forceinline__ void row_finish_fp8(const GemvArgs& g, const v4i (&cur)[NCH], uint8_t* xq, float* sc,
-                                               float* red) {
-  const int nchunk = g.K / AQ_VEC;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+template <int XT, class P>
+__device__ __forceinline__ void rows_finish_fp8(const GemvArgs& g, const v4i (&cur)[P::NPASS][P::QCH], uint8_t* xq,
+                                                int xstride, float* sc, float* red) {
+  const int tr = threadIdx.x % P::TPR, rs = threadIdx.x / P::TPR;
+  const int lane = threadIdx.x & 63, wrow = tr >> 6;
   constexpr uint32_t INF_BITS = XT == FMSMO_F16 ? 0x7c00u : 0x7f80u;
-  us2 amax2 = {0, 0};
 #pragma unroll
-  for (int i = 0; i < NCH; ++i)
+  for (int j = 0; j < P::NPASS; ++j) {
+    const int m = j * P::RPP + rs;
+    if (m < g.M) {
+      us2 amax2 = {0, 0};
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {  // (chunks past the row are zero)
-      const uint32_t mag = (uint32_t)cur[i][j] & 0x7fff7fffu;
-      us2 m2;
-      __builtin_memcpy(&m2, &mag, 4);
-      amax2 = __builtin_elementwise_max(amax2, m2);
+      for (int i = 0; i < P::QCH; ++i)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {  // (chunks past the row are zero)
+          const uint32_t mag = (uint32_t)cur[j][i][q] & 0x7fff7fffu;
+          us2 m2;
+          __builtin_memcpy(&m2, &mag, 4);
+          amax2 = __builtin_elementwise_max(amax2, m2);
+        }
+      const float v = wave_max(__uint_as_float((uint32_t)(amax2[0] > amax2[1] ? amax2[0] : amax2[1])));
+      if (lane == 0) red[m * P::WPR + wrow] = v;
     }
-  float v = wave_max(__uint_as_float((uint32_t)(amax2[0] > amax2[1] ? amax2[0] : amax2[1])));
-  if (lane == 0) red[wave] = v;
+  }
   __syncthreads();
-  v = red[0];
 #pragma unroll
-  for (int w = 1; w < NT / 64; ++w) v = fmaxf(v, red[w]);
-  const uint32_t abits = __float_as_uint(v);
-  const float s = fmaxf(cvt16<XT>((u16)abits) / 448.0f, 1e-12f);
-  if (threadIdx.x == 0) sc[0] = s;
+  for (int j = 0; j < P::NPASS; ++j) {
+    const int m = j * P::RPP + rs;
+    if (m < g.M) {
+      float v = red[m * P::WPR];
 #pragma unroll
-  for (int i = 0; i < NCH; ++i) {
-    const int c = threadIdx.x + i * NT;
-    if (c < nchunk) {
-      float t[8];
+      for (int w = 1; w < P::WPR; ++w) v = fmaxf(v, red[m * P::WPR + w]);
+      const uint32_t abits = __float_as_uint(v);
+      const float s = fmaxf(cvt16<XT>((u16)abits) / 448.0f, 1e-12f);
+      if (tr == 0) sc[m] = s;
+      const bool finite = abits < INF_BITS;
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const float xv = cvt16<XT>((u16)((uint32_t)cur[i][j >> 1] >> ((j & 1) * 16)));
-        t[j] = fminf(fmaxf(xv / s, -448.0f), 448.0f);
-      }
-      if (abits < INF_BITS) {
-        int o0 = 0, o1 = 0;
-        o0 = __builtin_amdgcn_cvt_pk_fp8_f32(t[0], t[1], o0, false);
-        o0 = __builtin_amdgcn_cvt_pk_fp8_f32(t[2], t[3], o0, true);
-        o1 = __builtin_amdgcn_cvt_pk_fp8_f32(t[4], t[5], o1, false);
-        o1 = __builtin_amdgcn_cvt_pk_fp8_f32(t[6], t[7], o1, true);
-        *(uint2*)(xq + (size_t)c * AQ_VEC) = make_uint2((uint32_t)o0, (uint32_t)o1);
-      } else {
-        uint8_t b[8];
+      for (int i = 0; i < P::QCH; ++i) {
+        const int c = tr + i * P::TPR;
+        if (c < P::CPR) {
+          float t[8];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) b[j] = f32_to_e4m3_sw(t[j]);
-        store8(xq, (size_t)c * AQ_VEC, b);
+          for (int q = 0; q < 8; ++q) {
+            const float xv = cvt16<XT>((u16)((uint32_t)cur[j][i][q >> 1] >> ((q & 1) * 16)));
+            t[q] = fminf(fmaxf(xv / s, -448.0f), 448.0f);
+          }
+          uint8_t* dst = xq + (size_t)m * xstride;
+          if (finite) {
+            int o0 = 0, o1 = 0;
+            o0 = __builtin_amdgcn_cvt_pk_fp8_f32(t[0], t[1], o0, false);
+            o0 = __builtin_amdgcn_cvt_pk_fp8_f32(t[2], t[3], o0, true);
+            o1 = __builtin_amdgcn_cvt_pk_fp8_f32(t[4], t[5], o1, false);
+            o1 = __builtin_amdgcn_cvt_pk_fp8_f32(t[6], t[7], o1, true);
+            *(uint2*)(dst + (size_t)c * AQ_VEC) = make_uint2((uint32_t)o0, (uint32_t)o1);
+          } else {
+            uint8_t b[8];
+#pragma unroll
+            for (int q = 0; q < 8; ++q) b[q] = f32_to_e4m3_sw(t[q]);
+            store8(dst, (size_t)c * AQ_VEC, b);
+          }
+        }
       }
     }
   }
   __syncthreads();
-  if (blockIdx.x == 0 && g.a_scale_out && threadIdx.x == 0) g.a_scale_out[0] = sc[0];
+  if (blockIdx.x == 0 && g.a_scale_out && (int)threadIdx.x < g.M) g.a_scale_out[threadIdx.x] = sc[threadIdx.x];
 }
 
 template <int OP, int RG, int NW>
@@ -456,21 +522,26 @@ __global__ __launch_bounds__(NW * 64) void gemv_kernel(GemvArgs g) {
 // upper 8 rows are neither loaded nor stored.
 // HALF = false: the host has checked that every block owns whole groups only (the loads of the
 // upper rows are then unconditional, which the register allocation of the long-row shapes needs).
-// XT >= 0 (fused decode linear, one token of dtype XT, with XS): the block quantizes the token
-// row itself, into LDS -- its loads are issued first, the head of the weight stream next, and the
-// quantizer's arithmetic runs while those weights are in flight -- and the activation fragments
-// are read from there (token rows 1..15 of the MFMA operand are zeros).
-template <int OP, int STEPS, int NW, int D, int MT = 1, bool HALF = false, bool XS = false, int XT = -1>
+// XT >= 0 (fused decode linear, up to MAXM tokens of dtype XT, K = NW * STEPS * 128): the block
+// quantizes the token rows itself, into LDS -- their loads are issued first, the head of the
+// weight stream next, and the quantizer's arithmetic runs while those weights are in flight --
+// and the activation fragments of every step are read from there (rows of 16 bytes more than K,
+// so that the 16 token rows of a fragment read fall into different banks; the lanes of token rows
+// past M substitute zeros).  No activation registers: the weight pipeline can be as deep as with
+// XS, for any number of row groups per block.
+template <int OP, int STEPS, int NW, int D, int MT = 1, bool HALF = false, bool XS = false, int XT = -1,
+          int MAXM = 1>
 __global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(GemvArgs g, int halves) {
   static_assert(STEPS % D == 0, "pipeline depth must divide the steps per group");
   static_assert(!XS || MT == 1, "streamed activations: one tile of tokens");
   constexpr bool FUSED = XT >= 0;
-  static_assert(!FUSED || XS, "the fused form streams its activations");
+  static_assert(!FUSED || (MT == 1 && MAXM <= 16), "the fused form serves one tile of tokens");
   constexpr int KROW = NW * STEPS * 128;
-  constexpr int QCH = (KROW / AQ_VEC + NW * 64 - 1) / (NW * 64);  // 16-byte chunks of the row per thread
-  __shared__ __attribute__((aligned(16))) uint8_t xq[FUSED ? KROW : 16];
-  __shared__ float xsc[1];
-  __shared__ float xred[NW];
+  constexpr int XSTRIDE = KROW + 16;
+  typedef RowsPlan<NW * 64, KROW, MAXM> QP;
+  __shared__ __attribute__((aligned(16))) uint8_t xq[FUSED ? MAXM * XSTRIDE : 16];
+  __shared__ float xsc[FUSED ? MAXM : 1];
+  __shared__ float xred[FUSED ? MAXM * QP::WPR + NW : 1];
   typedef typename std::conditional<OP == FMSMO_OP_I8, int, float>::type AccT;
   typedef AccT Acc4 __attribute__((ext_vector_type(4)));
   constexpr int NRED = 2;  // exchange buffers alternate, one barrier per group
@@ -527,9 +598,9 @@ __global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(GemvArgs g, int ha
   // go to a deeper pipeline (us at N = 4096, K = 14336, int8, 4 / 16 tokens: 12.7 / 15.5 with the
   // fragments held and two steps in flight, 11.4 / 13.8 streamed with seven; starting the blocks
   // at different K steps so that they do not all ask L2 for the same lines at once: 11.7 / 14.3).
-  v4i xf[XS ? 1 : MT][XS ? 1 : STEPS][2];
+  v4i xf[XS || FUSED ? 1 : MT][XS || FUSED ? 1 : STEPS][2];
   v4i xb[XS && !FUSED ? D : 1][2];
-  v4i qcur[FUSED ? QCH : 1], qsm[FUSED ? QCH : 1];
+  v4i qcur[FUSED ? QP::NPASS : 1][FUSED ? QP::QCH : 1], qsm[FUSED ? QP::QCH : 1];
   const __amdgpu_buffer_rsrc_t rsrc_x = __builtin_amdgcn_make_buffer_rsrc(
       (void*)g.a, 0, FUSED ? 0 : (int)((int64_t)(g.M - 1) * g.lda + g.K), 0x00020000);
   const int vx = r * (int)g.lda + kwave + kg * 16;
@@ -539,7 +610,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(GemvArgs g, int ha
     x[1] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_x, v, s * 128 + 64, 0));
   };
   if constexpr (FUSED) {
-    row_request<NW * 64, QCH>(g, qcur, qsm);
+    rows_request<QP>(g, qcur, qsm);
   } else if constexpr (XS) {
 #pragma unroll
     for (int j = 0; j < D; ++j) load_x(0, j, xb[j]);
@@ -559,15 +630,15 @@ __global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(GemvArgs g, int ha
   const int em = min((int)(threadIdx.x & 15), g.M - 1);
   float as;
   if constexpr (FUSED) {
-    if constexpr (OP == FMSMO_OP_I8) row_finish_i8<XT, NW * 64, QCH>(g, qcur, qsm, xq, xsc, xred);
-    else row_finish_fp8<XT, NW * 64, QCH>(g, qcur, xq, xsc, xred);
-    as = xsc[0];
+    if constexpr (OP == FMSMO_OP_I8) rows_finish_i8<XT, QP>(g, qcur, qsm, xq, XSTRIDE, xsc, xred);
+    else rows_finish_fp8<XT, QP>(g, qcur, xq, XSTRIDE, xsc, xred);
+    as = xsc[em];
   } else {
     as = g.a_scale[g.a_stride ? em : 0];
   }
-  // fused: the token's codes of this lane's K positions (lanes of token rows 1..15 read zeros)
-  const uint8_t* xl = xq + (FUSED ? kwave + kg * 16 : 0);
-  const bool xrow0 = r == 0;
+  // fused: the codes of this lane's token row and K positions (token rows past M: zeros)
+  const bool xrow = r < g.M;
+  const uint8_t* xl = xq + (FUSED ? (xrow ? r : 0) * XSTRIDE + kwave + kg * 16 : 0);
 
   // The last group of a block refills nothing (its prefetches would fall into the next block's
   // rows), so the group body exists twice: streaming (LAST = false) and draining (LAST = true).
@@ -600,7 +671,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(GemvArgs g, int ha
         if constexpr (FUSED) {
           const v4i z = {0, 0, 0, 0};
           x0 = *(const v4i*)(xl + s * 128), x1 = *(const v4i*)(xl + s * 128 + 64);
-          x0 = xrow0 ? x0 : z, x1 = xrow0 ? x1 : z;
+          x0 = xrow ? x0 : z, x1 = xrow ? x1 : z;
         } else {
           x0 = XS ? xb[s % D][0] : xf[t][s][0], x1 = XS ? xb[s % D][1] : xf[t][s][1];
         }
@@ -1026,39 +1097,55 @@ int fmsmo_gemv_dispatch(int op, const void* a, int64_t lda, const void* b, int64
 }
 
 // ---------------------------------------------------------------------- fused decode linear
-// One token.  K <= 8192: the row kernel quantizes the token in every block (measured from a HIP
+// One token, K <= 8192: the row kernel quantizes the token in every block (measured from a HIP
 // graph against the two launches, us: qkv 9.6 -> 8.3, o 8.1 -> 6.3, gate+up 23.4 -> 19.7).  With
 // longer rows the quantization its 1024 small blocks repeat costs more than the launch it saves
 // (K = 14336: 16.5 -> 19.6), so K = 14336 and K = 12800 take the streaming kernel's fused form:
 // 256 blocks of 8 / 10 waves quantize the row once each while the head of their weight stream is
 // in flight (N = 4096, int8 from fp16 / bf16 with SmoothQuant / e4m3: K = 14336 14.5 -> 11.4,
-// 16.6 -> 12.7, 17.5 -> 12.2; K = 12800 13.6 -> 10.6, 15.6 -> 11.6, 16.6 -> 11.9).  Two tokens at
-// K = 4096 lose (10.3 -> 10.9): more tokens are left to the two kernels.
+// 16.6 -> 12.7, 17.5 -> 12.2; K = 12800 13.6 -> 10.6, 15.6 -> 11.6, 16.6 -> 11.9).
+// A few tokens take the same form while the quantization that all 256 blocks repeat costs less
+// than the launch it saves (us, two launches -> fused, int8 from fp16 with SmoothQuant, 2 / 3 / 4
+// tokens: o 8.8 -> 7.9, 9.3 -> 7.6, 8.9 -> 8.3; qkv 10.3 -> 8.5, 9.9 -> 8.8, 9.9 -> 9.3; gate+up
+// 24.8 -> 21.8, 23.9 -> 22.1, 23.8 -> 22.8; down 15.8 -> 13.7, 15.9 -> 15.6, four tokens 15.9 ->
+// 17.8; six tokens at K = 4096 lose as well: 8.8 -> 9.3, 10.1 -> 10.4).
 extern "C" int fmsmo_decode_linear_ok(int64_t M, int64_t K) {
-  if (M != 1 || K % 128 || K < 1024) return 0;
-  if (K == 14336 || K == 12800) return 1;  // the streaming kernel's fused form
+  if (M < 1 || M > 4 || K % 128 || K < 1024) return 0;
+  if (M > 1) return K == 4096 || (M <= 3 && (K == 14336 || K == 12800));  // the streaming kernel's fused form
+  if (K == 14336 || K == 12800) return 1;
   const int kch = (int)((K + 1023) / 1024);
   return kch == 1 || kch == 2 || kch == 4 || kch == 8;
 }
 
 template <int OP, int XT>
 static int decode_fused_launch(const GemvArgs& g, hipStream_t st) {
-  // (int8, K = 4096 with at most one row group per compute unit: the same form instead of the row
-  // kernel's, us at N = 4096 / 1024 from bf16 with SmoothQuant: 6.6 -> 6.3 / 5.3 -> 4.6; e4m3
-  // stays with the row kernel there, whose fp32 sums are those of the two-call path)
-  if (g.K == 14336 || g.K == 12800 || (OP == FMSMO_OP_I8 && g.K == 4096 && g.N <= 4096)) {
-    // one group of 16 weight rows per block at most (the fused form streams its activations)
+  // the streaming kernel's fused form: (waves, steps per wave, loads in flight, most tokens)
+  int shape = 0;
+  if (g.K == 14336) shape = 814;
+  else if (g.K == 12800) shape = 1010;
+  else if (g.K == 4096 && g.M > 1) shape = 1602;
+  // (int8, one token, K = 4096 with at most one row group per compute unit: this form instead of
+  // the row kernel's, us at N = 4096 / 1024 from bf16 with SmoothQuant: 6.6 -> 6.3 / 5.3 -> 4.6;
+  // e4m3 stays with the row kernel there, whose fp32 sums are those of the two-call path)
+  else if (g.K == 4096 && OP == FMSMO_OP_I8 && g.N <= 4096) shape = 1602;
+  if (shape) {
     const int halves = (g.N + 7) / 8;
-    int nblocks = halves < 256 ? halves : 256;
-    if (2 * nblocks < halves) nblocks = (halves + 1) / 2;
+    const int nblocks = halves < 256 ? halves : 256;
     const bool whole_groups = halves % (2 * nblocks) == 0;
+    const bool one_group = halves == 2 * nblocks;  // the kernel without its loop over row groups
     dim3 grid((unsigned)nblocks);
-#define STREAM_F(NWV, ST, DV)                                                                        \
-  if (whole_groups)                                                                                  \
-    hipLaunchKernelGGL((gemv_stream_kernel<OP, ST, NWV, DV, 1, false, true, XT>), grid, dim3(NWV * 64), 0, st, g, halves); \
+#define STREAM_F(NWV, ST, DV, MM)                                                                    \
+  if (whole_groups && one_group)                                                                     \
+    hipLaunchKernelGGL((gemv_stream_kernel<OP, ST, NWV, DV, 1, false, true, XT, MM>), grid, dim3(NWV * 64), 0, st, g, halves); \
+  else if (whole_groups)                                                                             \
+    hipLaunchKernelGGL((gemv_stream_kernel<OP, ST, NWV, DV, 1, false, false, XT, MM>), grid, dim3(NWV * 64), 0, st, g, halves); \
   else                                                                                               \
-    hipLaunchKernelGGL((gemv_stream_kernel<OP, ST, NWV, DV, 1, true, true, XT>), grid, dim3(NWV * 64), 0, st, g, halves)
-    if (g.K == 14336) { STREAM_F(8, 14, 7); } else if (g.K == 4096) { STREAM_F(16, 2, 2); } else { STREAM_F(10, 10, 5); }
+    hipLaunchKernelGGL((gemv_stream_kernel<OP, ST, NWV, DV, 1, true, false, XT, MM>), grid, dim3(NWV * 64), 0, st, g, halves)
+    switch (shape) {
+      case 814: if (g.M == 1) { STREAM_F(8, 14, 7, 1); } else { STREAM_F(8, 14, 7, 4); } break;
+      case 1010: if (g.M == 1) { STREAM_F(10, 10, 5, 1); } else { STREAM_F(10, 10, 5, 4); } break;
+      default: if (g.M == 1) { STREAM_F(16, 2, 2, 1); } else { STREAM_F(16, 2, 2, 4); } break;
+    }
 #undef STREAM_F
     return fmsmo_check_launch();
   }

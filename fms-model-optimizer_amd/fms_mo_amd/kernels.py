@@ -694,9 +694,9 @@ _DECODE_OK = {}
 
 
 def decode_linear_ok(x, smooth, K):
-    """Can ``decode_linear_i8`` serve these activations?  One token, fp16 / bf16, SmoothQuant
-    divisors of the same dtype (or none), K up to 8192 in one of the decode kernel's sizes, or
-    14336 / 12800."""
+    """Can ``decode_linear_i8`` serve these activations?  fp16 / bf16, SmoothQuant divisors of the
+    same dtype (or none); one token at K up to 8192 in one of the decode kernel's sizes or at
+    14336 / 12800, up to four tokens at K = 4096, up to three at 14336 / 12800."""
     if x.dim() != 2 or x.dtype not in (torch.float16, torch.bfloat16) or not x.is_cuda:
         return False
     if smooth is not None and (smooth.dtype != x.dtype or smooth.numel() != K):

@@ -86,7 +86,7 @@ class FP8Linear(nn.Module):
                 s_t = (x2.abs().amax().float() / 448.0).clamp(min=1e-12)
                 q, s = kernels.quant_act_fp8_pertoken(x2, L.FP8_LINEAR, static_scale=s_t)
             elif kernels.decode_linear_ok(x2, None, x2.shape[1]):
-                # single-token decode step: quantizer and weight-streaming matmul in one launch
+                # decode step of a few tokens: quantizer and weight-streaming matmul in one launch
                 y, _ = kernels.decode_linear_fp8(x2, self.weight, w_scale, bias, out_dtype=x.dtype)
                 return y.reshape(out_shape)
             else:

@@ -689,7 +689,7 @@ class QLinearINT8Deploy(nn.Linear):
             sq = self.smoothq_scale.reshape(-1) if use_sq else None
             if plain and (sq is None or sq.numel() == x2.shape[1]) and \
                     kernels.decode_linear_ok(x2, sq, x2.shape[1]):
-                # single-token decode step: quantizer and weight-streaming matmul in one launch
+                # decode step of a few tokens: quantizer and weight-streaming matmul in one launch
                 y, s = kernels.decode_linear_i8(x2, self.weight, self._w_scale_f32(), self.bias, sq,
                                                 out_dtype=torch.float16, exact_ref=True)
                 self._set_input_scale(s.reshape(-1, 1))

@@ -367,18 +367,20 @@ int fmsmo_gemv_fp8_dq(const uint8_t* a, int64_t lda, const uint8_t* b, int64_t l
                       int64_t ldy, int64_t M, int64_t N, int64_t K, fmsmo_stream_t stream);
 
 /*
- * Fused decode linear for ONE token: y = dequant( quant(x) . W^T ) in one launch.  Every block
- * quantizes the (tiny) activation row itself -- the arithmetic of fmsmo_quant_act_i8_pertoken for
- * a 16-bit compute dtype: x fp16 / bf16 [1,K], smooth of x's dtype or NULL -- and then runs the
- * row-streaming kernel of fmsmo_gemv_i8_dq on the codes, so the result is bit-identical to the
- * two calls in sequence while a kernel launch and the round trip of the codes through memory are
- * saved in front of every linear layer of a single-stream decode step.  a_scale_out (fp32 [1],
- * may be NULL) receives the token's scale (the reference's input_scale side effect).
+ * Fused decode linear for a decode step of one to four tokens: y = dequant( quant(x) . W^T ) in
+ * one launch.  Every block quantizes the (tiny) activation rows itself -- the arithmetic of
+ * fmsmo_quant_act_i8_pertoken for a 16-bit compute dtype: x fp16 / bf16 [M,K], smooth of x's dtype
+ * or NULL -- and then runs a weight-streaming kernel of fmsmo_gemv_i8_dq on the codes, so the
+ * result is bit-identical to the two calls in sequence while a kernel launch and the round trip
+ * of the codes through memory are saved in front of every linear layer of a single-stream decode
+ * step.  a_scale_out (fp32 [M], may be NULL) receives the tokens' scales (the reference's
+ * input_scale side effect).
  * fmsmo_decode_linear_ok(M, K) != 0 tells whether a shape is served: M == 1 and either K <= 8192
  * in one of the row kernel's sizes (1024, 2048, 4096, 8192 and what pads to them) or K = 14336 /
- * 12800 (the streaming kernel quantizes the row while the head of its weight stream is in
- * flight); with more tokens or other row lengths the quantization that every block repeats costs
- * more than the launch it saves, and the call returns FMSMO_ERR_UNSUPPORTED: use the two kernels.
+ * 12800 (the streaming kernel quantizes the rows while the head of its weight stream is in
+ * flight); M <= 4 at K = 4096 and M <= 3 at K = 14336 / 12800 (the same kernel).  With more
+ * tokens or other row lengths the quantization that every block repeats costs more than the
+ * launch it saves, and the call returns FMSMO_ERR_UNSUPPORTED: use the two kernels.
  * x and smooth 16-byte aligned, ldx % 8 == 0, w as for fmsmo_gemv_i8_dq.
  * Reference: QLinearINT8Deploy.forward for a decode step -- qa_dynamic_max_qfunc followed by
  * iaddmm_int (fms_mo/modules/linear.py:1085-1100, 1177-1188, 1309-1338); no fused counterpart.
@@ -390,11 +392,12 @@ int fmsmo_decode_linear_i8(const void* x, int x_dtype, int64_t ldx, const void* 
                            void* y, int y_dtype, int64_t ldy, float* a_scale_out, int64_t M,
                            int64_t N, int64_t K, fmsmo_stream_t stream);
 /*
- * The same for e4m3 weights: the block quantizes the token with the dynamic per-token recipe of
- * fmsmo_quant_act_fp8_pertoken(FMSMO_FP8_LINEAR) and runs fmsmo_gemv_fp8_dq's kernel on it:
- * scale and codes are the quantizer's bit for bit, and so is the result wherever the two-call
- * path streams the weights in the same shape (K <= 8192; K = 14336 with N <= 4096); elsewhere the
- * fp32 partial sums are added in another order.  Served shapes as told by fmsmo_decode_linear_ok.
+ * The same for e4m3 weights: the block quantizes the tokens with the dynamic per-token recipe of
+ * fmsmo_quant_act_fp8_pertoken(FMSMO_FP8_LINEAR) and runs fmsmo_gemv_fp8_dq's kernel on them:
+ * scales and codes are the quantizer's bit for bit, and so is the result wherever the two-call
+ * path streams the weights in the same shape (one token: K <= 8192; K = 14336 with N <= 4096);
+ * elsewhere the fp32 partial sums are added in another order.  Served shapes as told by
+ * fmsmo_decode_linear_ok.
  * Reference: FP8Linear.forward with dynamic activation scales
  * (fms_mo/aiu_addons/fp8/fp8_linear.py:217-283) on one token.
  */

@@ -852,6 +852,91 @@ def test_fused_decode_linear_is_bit_identical_to_the_two_kernels(dev, NK, dt, sm
     assert torch.equal(s_f.cpu(), s_ref.reshape(-1).float())
 
 
+@pytest.mark.parametrize("NK", [(4096, 4096), (6144, 4096), (28672, 4096), (1000, 4096), (24, 4096),
+                                (4096, 14336), (1000, 14336), (8200, 14336), (4104, 12800)])
+@pytest.mark.parametrize("M", [2, 3, 4])
+@pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("smooth", [False, True])
+def test_fused_decode_linear_several_tokens(dev, NK, M, dt, smooth):
+    """A decode step of a few sequences: the streaming kernel quantizes all token rows itself.
+    Rows off the quantizer's fast path (zeros, an infinity, an overflow after the SmoothQuant
+    divide) sit between ordinary ones.  Scales and outputs are the two kernels' bit for bit."""
+    N, Kd = NK
+    kn = K()
+    x = torch.randn(M, Kd, generator=gen(176)).to(dt)
+    x[:, 5] *= 30.0
+    x[M - 1] *= 0.01
+    sm = (torch.rand(Kd, generator=gen(177)) * 3 + 0.2).to(dt) if smooth else None
+    if M >= 3:
+        x[1] = 0.0
+    if M == 4 or Kd == 12800:
+        x[2 if M > 2 else 0, 100] = float("inf")
+    overflow = M == 3 and dt == torch.float16 and smooth
+    if overflow:
+        x[2, 7] = 60000.0
+        sm[7] = 0.25  # 60000 / 0.25 overflows fp16
+    xd, smd = x.to(dev), None if sm is None else sm.to(dev)
+    if not kn.decode_linear_ok(xd, smd, Kd):
+        assert M > 3 and Kd > 4096  # long rows are served up to three tokens
+        return
+    w = _rand_i8((N, Kd), 178).to(dev)
+    s_w = (torch.rand(N, generator=gen(179)) * 1e-3 + 1e-5).to(dev)
+    bias = (torch.randn(N, generator=gen(180)) * 0.01).to(dt).to(dev)
+    for exact_ref, od in ((True, torch.float16), (False, torch.float32)):
+        q, s = kn.quant_act_i8_pertoken(xd, smd)
+        ref = kn.gemm_i8_dq(q, w, s, s_w, bias, out_dtype=od, exact_ref=exact_ref)
+        y, s_f = kn.decode_linear_i8(xd, w, s_w, bias, smd, out_dtype=od, exact_ref=exact_ref)
+        assert torch.equal(s_f.view(torch.int32), s.view(torch.int32))
+        bits = torch.int32 if od == torch.float32 else torch.int16
+        assert torch.equal(y.view(bits), ref.view(bits))
+    if not (M == 4 or Kd == 12800 or overflow):
+        _, s_ref, _ = O.quant_act_pertoken_i8(x if sm is None else x / sm)
+        assert torch.equal(s_f.cpu(), s_ref.reshape(-1).float())
+
+
+@pytest.mark.parametrize("NK", [(4096, 4096), (6144, 4096), (1000, 4096), (4096, 14336), (1016, 12800)])
+@pytest.mark.parametrize("M", [2, 3, 4])
+@pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
+def test_fused_decode_linear_fp8_several_tokens(dev, NK, M, dt):
+    """The same for e4m3 weights: scales and codes are the stand-alone quantizer's bit for bit
+    (codes through an exact product with weight rows that hold a single one); with random weights
+    the fp32 sums may be added in another order than by the two kernels (rtol 1e-5)."""
+    from fms_mo_amd import _lib as L
+
+    N, Kd = NK
+    kn = K()
+    x = (2.0 * torch.randn(M, Kd, generator=gen(186))).to(dt)
+    x[0, 3] = -0.0
+    x[M - 1] = 0.0
+    if M >= 3:
+        x[1, 9] = float("inf")
+    xd = x.to(dev)
+    if not kn.decode_linear_ok(xd, None, Kd):
+        assert M > 3 and Kd > 4096  # long rows are served up to three tokens
+        return
+    q, s = kn.quant_act_fp8_pertoken(xd, L.FP8_LINEAR)
+    n_id = min(N, Kd)
+    w_id = torch.zeros(N, Kd)
+    w_id[torch.arange(n_id), torch.arange(n_id)] = 1.0
+    w_id = w_id.to(torch.float8_e4m3fn).to(dev)
+    y_id, s_f = kn.decode_linear_fp8(xd, w_id, torch.ones(N, device=dev), None, out_dtype=torch.float32)
+    assert torch.equal(s_f.view(torch.int32), s.view(torch.int32))
+    want = q.float()[:, :n_id] * s.reshape(-1, 1)
+    fin = torch.ones(M, dtype=torch.bool)
+    if M >= 3:
+        fin[1] = False
+    flat = lambda t: torch.nan_to_num(t, nan=7.0, posinf=1e30, neginf=-1e30)
+    # (the row with the infinity has the scale inf: its outputs are NaN = 0 * inf but for column 9)
+    assert torch.equal(flat(y_id[:, :n_id]), flat(want))
+    w = _rand_fp8((N, Kd), 187, 0.5).to(dev)
+    s_w = (torch.rand(N, generator=gen(188)) * 0.01 + 1e-4).to(dev)
+    bias = (torch.randn(N, generator=gen(189)) * 0.1).to(dt).to(dev)
+    ref = kn.gemm_fp8_dq(q, w, s, s_w, bias, out_dtype=torch.float32)
+    y, _ = kn.decode_linear_fp8(xd, w, s_w, bias, out_dtype=torch.float32)
+    torch.testing.assert_close(y[fin.to(dev)], ref[fin.to(dev)], rtol=1e-5, atol=1e-5)
+    assert torch.equal(flat(y[~fin.to(dev)]), flat(ref[~fin.to(dev)]))
+
+
 @pytest.mark.parametrize("row", ["zeros", "inf", "overflow"])
 @pytest.mark.parametrize("Kd", [4096, 14336])
 def test_fused_decode_linear_special_rows(dev, row, Kd):
@@ -881,16 +966,19 @@ def test_fused_decode_linear_special_rows(dev, row, Kd):
 def test_fused_decode_linear_rejects_what_it_does_not_serve(dev):
     kn = K()
     x = torch.randn(2, 4096, device=dev).half()
-    assert not kn.decode_linear_ok(x, None, 4096)                          # more than one token
+    assert kn.decode_linear_ok(x, None, 4096)                              # a few tokens at K = 4096
+    assert not kn.decode_linear_ok(torch.randn(5, 4096, device=dev).half(), None, 4096)
+    assert not kn.decode_linear_ok(torch.randn(2, 2048, device=dev).half(), None, 2048)
     assert not kn.decode_linear_ok(x[:1].float(), None, 4096)              # fp32 activations
     assert not kn.decode_linear_ok(torch.randn(1, 16384, device=dev).half(), None, 16384)  # long rows
+    assert kn.decode_linear_ok(torch.randn(3, 14336, device=dev).half(), None, 14336)
     assert not kn.decode_linear_ok(torch.randn(4, 14336, device=dev).half(), None, 14336)
     assert kn.decode_linear_ok(torch.randn(1, 14336, device=dev).half(), None, 14336)
     assert not kn.decode_linear_ok(x[:1], torch.ones(4096, device=dev), 4096)  # fp32 divisors
     assert kn.decode_linear_ok(x[:1], None, 4096)
-    w = torch.zeros(64, 4096, dtype=torch.int8, device=dev)
+    w = torch.zeros(64, 2048, dtype=torch.int8, device=dev)
     with pytest.raises(RuntimeError):
-        kn.decode_linear_i8(x, w, torch.ones(1, device=dev))
+        kn.decode_linear_i8(x[:, :2048].contiguous(), w, torch.ones(1, device=dev))
 
 
 @pytest.mark.parametrize("NK", [(4096, 4096), (6144, 4096), (520, 1024), (1000, 2048), (256, 8192), (96, 1536)])
