@@ -16,6 +16,10 @@ typedef _Float16 h8 __attribute__((ext_vector_type(8)));
 typedef short s8v __attribute__((ext_vector_type(8)));
 typedef unsigned short u16;
 
+// internal epilogue code of the decode kernels: store the int32 sums themselves (beside the public
+// FMSMO_EPI_* values)
+constexpr int EPI_RAW_I32 = 100;
+
 #define FMSMO_GPTR(p) ((const __attribute__((address_space(1))) void*)(p))
 #define FMSMO_LPTR(p) ((__attribute__((address_space(3))) void*)(p))
 

@@ -38,18 +38,33 @@ extern "C" const char* fmsmo_status_str(int s) {
 }
 
 
-extern "C" int fmsmo_gemm_i8_i32(const int8_t* a, int64_t lda, const int8_t* b, int64_t ldb,
-                                 int32_t* c, int64_t ldc, int64_t M, int64_t N, int64_t K,
-                                 fmsmo_stream_t stream) {
+extern "C" int fmsmo_gemm_i8_i32_ws(const int8_t* a, int64_t lda, const int8_t* b, int64_t ldb,
+                                    int32_t* c, int64_t ldc, int64_t M, int64_t N, int64_t K,
+                                    void* workspace, int64_t workspace_bytes, fmsmo_stream_t stream) {
   int rc = check_gemm(a, lda, b, ldb, c, ldc, M, N, K);
   if (rc) return rc;
   if (M == 0) return FMSMO_OK;
+  // a few tokens: the weight-streaming decode kernels, storing their int32 sums
+  if ((M <= 16 && K % 128 == 0) || fmsmo_gemv_batch_ok(M, K))
+    return fmsmo_gemv_dispatch(FMSMO_OP_I8, a, lda, b, ldb, nullptr, 1, nullptr, 1, nullptr, FMSMO_F32,
+                               EPI_RAW_I32, c, FMSMO_F32, ldc, M, N, K, (hipStream_t)stream);
   GemmArgs g{};
   g.a = (const uint8_t*)a; g.b = (const uint8_t*)b; g.lda = lda; g.ldb = ldb;
   g.M = (int)M; g.N = (int)N; g.K = (int)K;
+  // few output tiles and a long reduction: K slices into the workspace, added in a fixed order
+  const SplitPlan plan = plan_split_k(M, N, K);
+  if (plan.splits > 1 && workspace && workspace_bytes >= plan.ws_bytes && aligned16(workspace) &&
+      plan.splits * M * lda < (1ll << 31))
+    return launch_split_k_i32(plan, g, workspace, c, ldc, (hipStream_t)stream);
   EpiStoreI32 epi{c, ldc};
   launch_any<MMA_I8>(g, epi, (hipStream_t)stream);
   return fmsmo_check_launch();
+}
+
+extern "C" int fmsmo_gemm_i8_i32(const int8_t* a, int64_t lda, const int8_t* b, int64_t ldb,
+                                 int32_t* c, int64_t ldc, int64_t M, int64_t N, int64_t K,
+                                 fmsmo_stream_t stream) {
+  return fmsmo_gemm_i8_i32_ws(a, lda, b, ldb, c, ldc, M, N, K, nullptr, 0, stream);
 }
 
 static int gemm_i8_dq_impl(const int8_t* a, int64_t lda, const int8_t* b, int64_t ldb,

@@ -291,6 +291,25 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const AccT* __restri
   epi.store(m, n, sum, epi.row(m), epi.col(n, 0, N));
 }
 
+// c = sum over K slices (int32, exact), see above.  The caller has checked the operands.
+inline int launch_split_k_i32(const SplitPlan& p, const GemmArgs& g0, void* workspace, int32_t* c, int64_t ldc,
+                              hipStream_t st) {
+  GemmArgs g = g0;
+  g.K = (int)p.k_len;
+  g.num_experts = p.splits;
+  g.rows_per_group = g0.M;
+  g.M = p.splits * g0.M;
+  g.lda_e = p.k_len;
+  g.ldb_e = p.k_len;
+  g.grid_m = p.splits * div_up(g0.M, TileMid::BM);
+  launch_tile<TileMid, MMA_I8, true>(g, EpiStoreI32{(int32_t*)workspace, g0.N}, st);
+  dim3 grid(div_up(g0.N, 256), (unsigned)g0.M), block(256);
+  EpiStoreI32 epi{c, ldc};
+  hipLaunchKernelGGL((splitk_reduce_kernel<int, EpiStoreI32>), grid, block, 0, st, (const int*)workspace,
+                     p.splits, g0.M, g0.N, epi);
+  return fmsmo_check_launch();
+}
+
 // y = epilogue( sum over K slices ), see above.  The caller has checked the operands.
 template <int OP, bool REF, class AccT>
 int launch_split_k(const SplitPlan& p, const GemmArgs& g0, void* workspace, const float* a_scale,

@@ -471,7 +471,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_kernel(GemvArgs g) {
     for (int w = 1; w < NW; ++w) s += red[w][i][e];
     const int n = n0 + i * 16 + (e >> 4), m = e & 15;
     if (n < g.N && m < g.M) {
-      const float as = g.a_scale[g.a_stride ? m : 0], ws = g.w_scale[g.w_stride ? n : 0];
+      const float as = g.a_scale ? g.a_scale[g.a_stride ? m : 0] : 1.f, ws = g.w_scale ? g.w_scale[g.w_stride ? n : 0] : 1.f;
       float b = 0.f;
       if (g.bias) {
         b = g.bias_dtype == FMSMO_F16 ? f16_to_f32(((const u16*)g.bias)[n])
@@ -489,7 +489,8 @@ __global__ __launch_bounds__(NW * 64) void gemv_kernel(GemvArgs g) {
         out = __fmaf_rn((float)s, __fmul_rn(as, ws), b);
       }
       const int64_t idx = (int64_t)m * g.ldy + n;
-      if (g.y_dtype == FMSMO_F16) ((u16*)g.y)[idx] = f32_to_f16(out);
+      if (g.epi == EPI_RAW_I32) ((int*)g.y)[idx] = (int)s;
+      else if (g.y_dtype == FMSMO_F16) ((u16*)g.y)[idx] = f32_to_f16(out);
       else if (g.y_dtype == FMSMO_BF16) ((u16*)g.y)[idx] = f32_to_bf16(out);
       else ((float*)g.y)[idx] = out;
     }
@@ -634,7 +635,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(GemvArgs g, int ha
     else rows_finish_fp8<XT, QP>(g, qcur, xq, XSTRIDE, xsc, xred);
     as = xsc[em];
   } else {
-    as = g.a_scale[g.a_stride ? em : 0];
+    as = g.a_scale ? g.a_scale[g.a_stride ? em : 0] : 1.f;
   }
   // fused: the codes of this lane's token row and K positions (token rows past M: zeros)
   const bool xrow = r < g.M;
@@ -645,7 +646,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(GemvArgs g, int ha
   auto do_group = [&](auto last_tag, int gi) {
     constexpr bool LAST = decltype(last_tag)::value;
     const int en = min(row_lo + gi * 16 + (int)((threadIdx.x >> 4) & 15), g.N - 1);
-    const float ws = g.w_scale[g.w_stride ? en : 0];
+    const float ws = g.w_scale ? g.w_scale[g.w_stride ? en : 0] : 1.f;
     float bv = 0.f;
     if (g.bias) {
       bv = g.bias_dtype == FMSMO_F16 ? f16_to_f32(((const u16*)g.bias)[en])
@@ -724,7 +725,8 @@ __global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(GemvArgs g, int ha
           out = __fmaf_rn((float)sum, __fmul_rn(as_e, ws_e), bv_e);
         }
         const int64_t idx = (int64_t)m * g.ldy + n;
-        if (g.y_dtype == FMSMO_F16) ((u16*)g.y)[idx] = f32_to_f16(out);
+        if (g.epi == EPI_RAW_I32) ((int*)g.y)[idx] = (int)sum;
+        else if (g.y_dtype == FMSMO_F16) ((u16*)g.y)[idx] = f32_to_f16(out);
         else if (g.y_dtype == FMSMO_BF16) ((u16*)g.y)[idx] = f32_to_bf16(out);
         else ((float*)g.y)[idx] = out;
       }
@@ -737,7 +739,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(GemvArgs g, int ha
       static_assert(MT == 1 || (NW * 64) % 256 == 0, "outputs of a thread must share its column");
       for (int e = threadIdx.x; e < 256 * MT; e += NW * 64) {
         const int m = min((e >> 8) * 16 + (e & 15), g.M - 1);
-        finish(e, g.a_scale[g.a_stride ? m : 0], ws, bv);
+        finish(e, g.a_scale ? g.a_scale[g.a_stride ? m : 0] : 1.f, ws, bv);
       }
     }
   };
@@ -888,7 +890,7 @@ __global__ __launch_bounds__(256) void gemv_rows_kernel(GemvArgs g) {
     constexpr int SHARE = 64 / V;  // lanes holding the same total; the first of them writes it
     const int n = n0 + eu;
     if ((lane & (SHARE - 1)) == 0 && n < g.N && em < g.M) {
-      const float as = g.a_scale[g.a_stride ? em : 0], ws = g.w_scale[g.w_stride ? n : 0];
+      const float as = g.a_scale ? g.a_scale[g.a_stride ? em : 0] : 1.f, ws = g.w_scale ? g.w_scale[g.w_stride ? n : 0] : 1.f;
       float bv = 0.f;
       if (g.bias) {
         bv = g.bias_dtype == FMSMO_F16 ? f16_to_f32(((const u16*)g.bias)[n])
@@ -906,7 +908,8 @@ __global__ __launch_bounds__(256) void gemv_rows_kernel(GemvArgs g) {
         out = __fmaf_rn((float)sum, __fmul_rn(as, ws), bv);
       }
       const int64_t idx = (int64_t)em * g.ldy + n;
-      if (g.y_dtype == FMSMO_F16) ((u16*)g.y)[idx] = f32_to_f16(out);
+      if (g.epi == EPI_RAW_I32) ((int*)g.y)[idx] = (int)sum;
+      else if (g.y_dtype == FMSMO_F16) ((u16*)g.y)[idx] = f32_to_f16(out);
       else if (g.y_dtype == FMSMO_BF16) ((u16*)g.y)[idx] = f32_to_bf16(out);
       else ((float*)g.y)[idx] = out;
     }

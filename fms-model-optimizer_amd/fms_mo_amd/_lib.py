@@ -39,6 +39,7 @@ SIGNATURES = {
     "fmsmo_quant_act_i8_mulscale": [_P, _I, _L, _P, _P, _I, _I, _I, _P, _L, _P, _L, _L, _P],
     "fmsmo_quant_act_fp8_pertoken": [_P, _I, _L, _I, _I, _P, _L, _P, _L, _L, _P],
     "fmsmo_gemm_i8_i32": [_P, _L, _P, _L, _P, _L, _L, _L, _L, _P],
+    "fmsmo_gemm_i8_i32_ws": [_P, _L, _P, _L, _P, _L, _L, _L, _L, _P, _L, _P],
     "fmsmo_gemm_i8_dq": [_P, _L, _P, _L, _P, _L, _P, _L, _P, _I, _I, _P, _I, _L, _L, _L, _L, _P],
     "fmsmo_gemm_fp8_dq": [_P, _L, _P, _L, _P, _L, _P, _L, _P, _I, _P, _I, _L, _L, _L, _L, _P],
     "fmsmo_gemm_i8_dq_ws": [_P, _L, _P, _L, _P, _L, _P, _L, _P, _I, _I, _P, _I, _L, _L, _L, _L, _P, _L, _P],

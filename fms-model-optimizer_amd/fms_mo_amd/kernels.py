@@ -310,9 +310,14 @@ def gemm_i8_i32(a, w):
     M, K = a.shape
     N = w.shape[0]
     c = torch.empty((M, N), dtype=torch.int32, device=a.device)
+    ws = _workspace(M, N, K, a.device)
     with _dev(a):
-        L.call("fmsmo_gemm_i8_i32", a.data_ptr(), _ld(a), w.data_ptr(), _ld(w), c.data_ptr(), N,
-               M, N, K, _stream(a))
+        if ws is not None:
+            L.call("fmsmo_gemm_i8_i32_ws", a.data_ptr(), _ld(a), w.data_ptr(), _ld(w), c.data_ptr(), N,
+                   M, N, K, ws.data_ptr(), ws.numel(), _stream(a))
+        else:
+            L.call("fmsmo_gemm_i8_i32", a.data_ptr(), _ld(a), w.data_ptr(), _ld(w), c.data_ptr(), N,
+                   M, N, K, _stream(a))
     return c
 
 

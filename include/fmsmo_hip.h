@@ -249,6 +249,18 @@ int fmsmo_quant_act_fp8_pertoken(const void* x, int x_dtype, int64_t ldx, int va
  */
 int fmsmo_gemm_i8_i32(const int8_t* a, int64_t lda, const int8_t* b, int64_t ldb, int32_t* c,
                       int64_t ldc, int64_t M, int64_t N, int64_t K, fmsmo_stream_t stream);
+/*
+ * The same with an optional scratch buffer, as for fmsmo_gemm_i8_dq_ws below: shapes with few
+ * output tiles and a long reduction run as K slices whose int32 partial sums are added in a fixed
+ * order (exact, so the result is the single-pass one bit for bit); fmsmo_gemm_workspace_bytes
+ * tells the bytes a shape can use, workspace == NULL or fewer bytes runs the single pass.
+ * Up to 16 rows (and the batches of up to 64 rows that fmsmo_gemm_i8_dq sends there) run on the
+ * weight-streaming kernels with either call.
+ * Same reference interfaces as fmsmo_gemm_i8_i32; the workspace has no counterpart there.
+ */
+int fmsmo_gemm_i8_i32_ws(const int8_t* a, int64_t lda, const int8_t* b, int64_t ldb, int32_t* c,
+                         int64_t ldc, int64_t M, int64_t N, int64_t K, void* workspace,
+                         int64_t workspace_bytes, fmsmo_stream_t stream);
 
 /*
  * int8 GEMM with the dequantizing epilogue fused:  y = acc * (a_scale x w_scale) + bias.

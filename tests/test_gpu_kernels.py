@@ -327,6 +327,49 @@ def test_gemm_i8_i32_exact(dev, shape):
     assert torch.equal(c.cpu(), ref)
 
 
+@pytest.mark.parametrize("shape", [
+    # a few rows: the weight-streaming decode kernels store their int32 sums (row kernel, MFMA
+    # streaming kernel with whole and half row groups, streamed activations, generic decode kernel,
+    # batches of up to 64 rows)
+    (1, 4096, 4096), (2, 1000, 4096), (1, 520, 14336), (3, 4096, 14336), (4, 6144, 4096), (9, 264, 12800),
+    (16, 4096, 4096), (16, 1000, 2048), (5, 300, 384), (16, 4104, 14336), (24, 4096, 4096), (33, 520, 2048),
+    (64, 6144, 4096), (32, 1000, 8192),
+    # few output tiles, long reduction: K slices through the workspace
+    (17, 4096, 14336), (128, 4096, 4096), (100, 1000, 8192), (512, 4096, 4096), (300, 520, 14336),
+    (1024, 2048, 4096)])
+def test_gemm_i8_i32_small_batches(dev, shape):
+    M, N, Kd = shape
+    g = torch.Generator(device=dev).manual_seed(M + N + Kd)
+    a = torch.randint(-128, 128, (M, Kd), generator=g, dtype=torch.int8, device=dev)
+    w = torch.randint(-128, 128, (N, Kd), generator=g, dtype=torch.int8, device=dev)
+    ref = (a.double() @ w.double().t()).to(torch.int32)
+    c = K().gemm_i8_i32(a, w)
+    assert c.dtype == torch.int32 and torch.equal(c, ref)
+    if M * N * Kd <= 2 ** 28:  # the oracle itself on the smaller ones
+        assert torch.equal(c.cpu(), O.int_gemm(a.cpu(), w.cpu()))
+
+
+def test_gemm_i8_i32_with_and_without_workspace(dev):
+    """The C entry points: with a workspace the K slices, without one the single pass; the same
+    bits, and a workspace that is too small or NULL is simply not used."""
+    from fms_mo_amd import _lib as L
+
+    lib = L.load()
+    M, N, Kd = 100, 1024, 8192
+    a, w = _rand_i8((M, Kd), 15).to(dev), _rand_i8((N, Kd), 16).to(dev)
+    ref = O.int_gemm(a.cpu(), w.cpu())
+    need = lib.fmsmo_gemm_workspace_bytes(M, N, Kd)
+    assert need > 0
+    st = torch.cuda.current_stream().cuda_stream
+    for nbytes in (need, need - 16, 0):
+        ws = torch.empty((max(nbytes, 16),), dtype=torch.uint8, device=dev)
+        c = torch.full((M, N), -7, dtype=torch.int32, device=dev)
+        L.call("fmsmo_gemm_i8_i32_ws", a.data_ptr(), Kd, w.data_ptr(), Kd, c.data_ptr(), N, M, N, Kd,
+               ws.data_ptr() if nbytes else None, nbytes, st)
+        torch.cuda.synchronize()
+        assert torch.equal(c.cpu(), ref)
+
+
 def test_gemm_i8_i32_random_shapes_cover_every_kernel_choice(dev):
     """Forty seeded shapes between 17 and ~4500 rows / columns: whatever kernel and tile shape the
     library picks for a shape (fmsmo_gemm_plan names it), the int32 result must equal the exact

@@ -19,7 +19,7 @@ def declared_symbols():
 def test_header_declares_the_expected_entry_points():
     syms = declared_symbols()
     for s in ["fmsmo_quant_act_i8_pertoken", "fmsmo_quant_act_i8_static", "fmsmo_quant_act_fp8_pertoken",
-              "fmsmo_gemm_i8_i32", "fmsmo_gemm_i8_dq", "fmsmo_gemm_fp8_dq", "fmsmo_gemv_i8_dq",
+              "fmsmo_gemm_i8_i32", "fmsmo_gemm_i8_i32_ws", "fmsmo_gemm_i8_dq", "fmsmo_gemm_fp8_dq", "fmsmo_gemv_i8_dq",
               "fmsmo_gemv_fp8_dq", "fmsmo_matmul_chunk_i8", "fmsmo_matmul_chunk_fp",
               "fmsmo_grouped_gemm_i8_dq", "fmsmo_quant_weight_i8", "fmsmo_absmax_cols",
               "fmsmo_quant_act_i8_mulscale", "fmsmo_zero_shift_bias", "fmsmo_quant_i8_affine",
