@@ -684,6 +684,47 @@ def test_grouped_gemm_equals_per_expert_linear(dev):
         assert torch.equal(y[lo:hi].view(torch.int16), ref.view(torch.int16)), e
 
 
+@pytest.mark.parametrize("counts", [
+    # rows beyond an expert's last whole 256-row tile: none, 1, 64, 65, 128, 129, 255; empty and
+    # tiny experts; an expert of exactly one tile
+    [256, 257, 320, 321, 384, 385, 511, 0],
+    [0, 0, 5, 0, 130, 64, 1, 0],
+    [1069, 1029, 997, 985],
+    [128, 128, 128, 128, 128, 128],
+    [700]])
+@pytest.mark.parametrize("NK", [(520, 256), (256, 1088)])
+@pytest.mark.parametrize("exact_ref,out_dtype", [(True, torch.float16), (False, torch.float32)])
+def test_grouped_gemm_row_remainders(dev, counts, NK, exact_ref, out_dtype):
+    """Every row of every expert must come out exactly once and equal the per-expert product,
+    whatever the split of the rows (K in whole 128-byte slabs and not: both grouped kernels)."""
+    N, Kd = NK
+    E = len(counts)
+    offsets = torch.zeros(E + 1, dtype=torch.int32)
+    offsets[1:] = torch.tensor(counts).cumsum(0)
+    T = int(offsets[-1])
+    a = _rand_i8((T, Kd), 76)
+    w = _rand_i8((E, N, Kd), 77)
+    s_a = (torch.rand(T, generator=gen(78)) * 0.05 + 1e-3).float()
+    s_w = (torch.rand(E, N, generator=gen(79)) * 1e-3 + 1e-5).float()
+    bias = (torch.randn(E, N, generator=gen(80)) * 0.01).half()
+    y = K().grouped_gemm_i8_dq(a.to(dev), w.to(dev), offsets.to(dev), s_a.to(dev), s_w.to(dev), bias.to(dev),
+                               out_dtype=out_dtype, exact_ref=exact_ref).cpu()
+    bits = torch.int32 if out_dtype == torch.float32 else torch.int16
+    for e in range(E):
+        lo, hi = int(offsets[e]), int(offsets[e + 1])
+        if hi == lo:
+            continue
+        ref = K().gemm_i8_dq(a[lo:hi].to(dev), w[e].to(dev), s_a[lo:hi].to(dev), s_w[e].to(dev), bias[e].to(dev),
+                             out_dtype=out_dtype, exact_ref=exact_ref).cpu()
+        assert torch.equal(y[lo:hi].view(bits), ref.view(bits)), e
+        if exact_ref and hi - lo <= 400:
+            acc = O.int_gemm(a[lo:hi], w[e])
+            want = O.epilogue_ref(acc, s_a[lo:hi, None].half(), s_w[e], bias[e], torch.float16)
+            # (the oracle takes the token scales in fp16, the kernel in fp32: compare where equal)
+            same = s_a[lo:hi].half().float() == s_a[lo:hi]
+            assert torch.equal(y[lo:hi][same].view(bits), want[same].view(bits))
+
+
 # ------------------------------------------------------------------------------ error behaviour
 def test_clock_probe_reports_a_plausible_core_clock(dev):
     # diagnostic entry point: block 0 of a 256-row-tile GEMM stores {core, 100 MHz} counter pairs
