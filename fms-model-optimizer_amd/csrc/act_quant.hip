@@ -282,25 +282,6 @@ __global__ __launch_bounds__(TH) void quant_i8_pertoken16_kernel(
 // a block that sees a divisor outside that range, or a row whose maximum is not finite, takes
 // the plain IEEE division instead.  Quotients by the row scale only feed rint(); where they
 // underflow they are far below 0.5.
-__device__ __forceinline__ float rcp_refined(float s) {
-  const float r0 = __builtin_amdgcn_rcpf(s);
-  return __builtin_fmaf(__builtin_fmaf(-s, r0, 1.0f), r0, r0);
-}
-__device__ __forceinline__ float div32_fast(float x, float s, float r1) {
-  float q = __fmul_rn(x, r1);
-  q = __builtin_fmaf(__builtin_fmaf(-s, q, x), r1, q);
-  q = __builtin_fmaf(__builtin_fmaf(-s, q, x), r1, q);
-  return q;
-}
-// the same for x widened from fp16: with the first product written as fma(x, r1, -0) (nz: see
-// opaque_neg_zero) all three uses of x fold into v_fma_mix_f32 and no conversion is issued
-__device__ __forceinline__ float div32_fast_mix(float x, float s, float r1, float nz) {
-  float q = __builtin_fmaf(x, r1, nz);
-  q = __builtin_fmaf(__builtin_fmaf(-s, q, x), r1, q);
-  q = __builtin_fmaf(__builtin_fmaf(-s, q, x), r1, q);
-  return q;
-}
-
 // bf16 x (XT = FMSMO_BF16) reaches below fp16's range: a row whose maximum quotient is under
 // 2^-80 (and not zero) also takes the IEEE division, because the residuals of its corrections
 // could fall below the smallest fp32 subnormal; elements that small inside an ordinary row

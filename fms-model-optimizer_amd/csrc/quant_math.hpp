@@ -59,6 +59,28 @@ __device__ __forceinline__ float div16_mix(float e, float s, float r, float nz) 
   const float q0 = T == FMSMO_F16 ? __builtin_fmaf(e, r, nz) : __fmul_rn(e, r);
   return __builtin_fmaf(__builtin_fmaf(-q0, s, e), r, q0);
 }
+// fp32 division without the IEEE sequence's range scaling and fix-up: a refined reciprocal and two
+// residual corrections give the correctly rounded quotient whenever no intermediate leaves the
+// normal range (the callers check the ranges of their operands).
+__device__ __forceinline__ float rcp_refined(float s) {
+  const float r0 = __builtin_amdgcn_rcpf(s);
+  return __builtin_fmaf(__builtin_fmaf(-s, r0, 1.0f), r0, r0);
+}
+__device__ __forceinline__ float div32_fast(float x, float s, float r1) {
+  float q = __fmul_rn(x, r1);
+  q = __builtin_fmaf(__builtin_fmaf(-s, q, x), r1, q);
+  q = __builtin_fmaf(__builtin_fmaf(-s, q, x), r1, q);
+  return q;
+}
+// the same for x widened from fp16: with the first product written as fma(x, r1, -0) (nz: see
+// opaque_neg_zero) all three uses of x fold into v_fma_mix_f32 and no conversion is issued
+__device__ __forceinline__ float div32_fast_mix(float x, float s, float r1, float nz) {
+  float q = __builtin_fmaf(x, r1, nz);
+  q = __builtin_fmaf(__builtin_fmaf(-s, q, x), r1, q);
+  q = __builtin_fmaf(__builtin_fmaf(-s, q, x), r1, q);
+  return q;
+}
+
 template <int T>
 __device__ __forceinline__ float cvt16(u16 h) {
   if constexpr (T == FMSMO_F16) return f16_to_f32(h);

@@ -34,7 +34,8 @@ struct GemvArgs {
   // quantizes them itself
   const u16* x16;       // [M,K]
   int64_t ldx;
-  const u16* smooth;    // [K] SmoothQuant divisors of x's dtype, or NULL
+  const u16* smooth;    // [K] SmoothQuant divisors of x's dtype (fp32 when smooth_f32), or NULL
+  int smooth_f32;
   int saturate;
   float* a_scale_out;   // [M] per-token scales (written by block 0), or NULL
 };
@@ -341,6 +342,167 @@ __device__ __forceinline__ void rows_finish_i8(const GemvArgs& g, v4i (&cur)[P::
   if (blockIdx.x == 0 && g.a_scale_out && (int)threadIdx.x < g.M) g.a_scale_out[threadIdx.x] = sc[threadIdx.x];
 }
 
+// fp32 SmoothQuant divisors: torch promotes x / smooth to fp32 and the whole quantizer then runs in
+// fp32 (scale max(amax, 1e-5) / 127, quotients, rint), as in the stand-alone quantizer's kernel for
+// that case: fast correctly rounded divisions while every divisor lies in 2^-60 .. 2^60 and the
+// row maximum is finite (for bf16 x: and not below 2^-80), IEEE divisions otherwise.
+template <class P>
+__device__ __forceinline__ void rows_request_f32s(const GemvArgs& g, v4i (&cur)[P::NPASS][P::QCH],
+                                                  float (&sd)[P::QCH][8]) {
+  const int tr = threadIdx.x % P::TPR, rs = threadIdx.x / P::TPR;
+  const float* smooth = (const float*)g.smooth;
+#pragma unroll
+  for (int i = 0; i < P::QCH; ++i) {
+    const int c = tr + i * P::TPR;
+#pragma unroll
+    for (int q = 0; q < 8; ++q) sd[i][q] = 1.0f;
+    if (c < P::CPR) {
+      const float4 a = *(const float4*)(smooth + (size_t)c * AQ_VEC);
+      const float4 b = *(const float4*)(smooth + (size_t)c * AQ_VEC + 4);
+      sd[i][0] = a.x, sd[i][1] = a.y, sd[i][2] = a.z, sd[i][3] = a.w;
+      sd[i][4] = b.x, sd[i][5] = b.y, sd[i][6] = b.z, sd[i][7] = b.w;
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < P::NPASS; ++j) {
+    const int m = j * P::RPP + rs;
+#pragma unroll
+    for (int i = 0; i < P::QCH; ++i) {
+      const int c = tr + i * P::TPR;
+      cur[j][i] = v4i{0, 0, 0, 0};
+      if (m < g.M && c < P::CPR) cur[j][i] = *(const v4i*)(g.x16 + (size_t)m * g.ldx + (size_t)c * AQ_VEC);
+    }
+  }
+}
+
+// red: 2 * P::MAXM * P::WPR floats; sc: P::MAXM
+template <int XT, class P>
+__device__ __forceinline__ void rows_finish_i8_f32s(const GemvArgs& g, const v4i (&cur)[P::NPASS][P::QCH],
+                                                    const float (&sd)[P::QCH][8], uint8_t* xq, int xstride,
+                                                    float* sc, float* red) {
+  const int tr = threadIdx.x % P::TPR, rs = threadIdx.x / P::TPR;
+  const int lane = threadIdx.x & 63, wrow = tr >> 6;
+  const float nz = opaque_neg_zero();
+  int bad = 0;
+#pragma unroll
+  for (int i = 0; i < P::QCH; ++i)
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {  // (chunks past the row hold ones)
+      const float a = fabsf(sd[i][q]);
+      bad |= !(a >= 8.6736174e-19f && a <= 1.1529215e18f);  // outside 2^-60 .. 2^60, or NaN
+    }
+  const bool ieee_block = __syncthreads_or(bad) != 0;
+  float e[P::NPASS][P::QCH][8];
+  // e <- x / smooth of the thread's rows; the waves' maxima of |e| (a thread's maximum drops NaN,
+  // bit patterns of non-negative floats order like the floats)
+  auto divide = [&](int j, bool ieee) -> float {
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < P::QCH; ++i) {
+      const int c = tr + i * P::TPR;
+      if (c < P::CPR) {
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+          const float xv = cvt16<XT>((u16)((uint32_t)cur[j][i][q >> 1] >> ((q & 1) * 16)));
+          e[j][i][q] = ieee ? xv / sd[i][q] : div32_fast_mix(xv, sd[i][q], rcp_refined(sd[i][q]), nz);
+          amax = fmaxf(amax, fabsf(e[j][i][q]));
+        }
+      }
+    }
+    return amax;
+  };
+  auto row_maxima = [&](float* buf, uint32_t (&rowbits)[P::MAXM]) {
+    __syncthreads();
+#pragma unroll
+    for (int m = 0; m < P::MAXM; ++m) {
+      rowbits[m] = 0;
+      if (m < g.M) {
+        uint32_t v = __float_as_uint(buf[m * P::WPR]);
+#pragma unroll
+        for (int w = 1; w < P::WPR; ++w) v = max(v, __float_as_uint(buf[m * P::WPR + w]));
+        rowbits[m] = v;
+      }
+    }
+  };
+#pragma unroll
+  for (int j = 0; j < P::NPASS; ++j) {
+    const int m = j * P::RPP + rs;  // uniform in a wave
+    if (m < g.M) {
+      const uint32_t b = wave_max_u32(__float_as_uint(divide(j, ieee_block)) & 0x7fffffffu);
+      if (lane == 0) red[m * P::WPR + wrow] = __uint_as_float(b);
+    }
+  }
+  uint32_t rowbits[P::MAXM];
+  row_maxima(red, rowbits);
+  // rows that take the IEEE divisions (uniform over the block)
+  uint32_t ieee_rows = 0;
+#pragma unroll
+  for (int m = 0; m < P::MAXM; ++m) {
+    const float amax = __uint_as_float(rowbits[m]);
+    bool ieee = ieee_block || !(amax < __builtin_inff());
+    if constexpr (XT == FMSMO_BF16) ieee = ieee || (amax != 0.0f && amax < 8.271806e-25f);
+    if (m < g.M && ieee) ieee_rows |= 1u << m;
+  }
+  if (ieee_rows && !ieee_block) {  // redo those rows (with every divisor in range the first pass was the fast one)
+    float* red2 = red + P::MAXM * P::WPR;
+#pragma unroll
+    for (int j = 0; j < P::NPASS; ++j) {
+      const int m = j * P::RPP + rs;
+      if (m < g.M && (ieee_rows >> m & 1)) {
+        const uint32_t b = wave_max_u32(__float_as_uint(divide(j, true)) & 0x7fffffffu);
+        if (lane == 0) red2[m * P::WPR + wrow] = __uint_as_float(b);
+      }
+    }
+    uint32_t again[P::MAXM];
+    row_maxima(red2, again);
+#pragma unroll
+    for (int m = 0; m < P::MAXM; ++m)
+      if (ieee_rows >> m & 1) rowbits[m] = again[m];
+  }
+#pragma unroll
+  for (int j = 0; j < P::NPASS; ++j) {
+    const int m = j * P::RPP + rs;
+    uint32_t abits = 0;
+    bool ieee = false;
+#pragma unroll
+    for (int q = 0; q < P::RPP; ++q)
+      if (j * P::RPP + q < P::MAXM && rs == q) {
+        abits = rowbits[j * P::RPP + q];
+        ieee = ieee_rows >> (j * P::RPP + q) & 1;
+      }
+    if (m < g.M) {
+      const float s = fmaxf(__uint_as_float(abits), 1e-5f) / 127.0f;
+      const float rcp_s = rcp_refined(s);
+      if (tr == 0) sc[m] = s;
+#pragma unroll
+      for (int i = 0; i < P::QCH; ++i) {
+        const int c = tr + i * P::TPR;
+        if (c < P::CPR) {
+          uint32_t code[8];
+#pragma unroll
+          for (int q = 0; q < 8; ++q) {
+            float r = ieee ? e[j][i][q] / s : div32_fast(e[j][i][q], s, rcp_s);
+            if (g.saturate) r = fminf(fmaxf(r, -127.0f), 127.0f);
+            // |r| <= 128.5 in every finite row: adding 1.5 * 2^23 rounds to the nearest integer,
+            // ties to even, and leaves it in two's complement in the low mantissa bits
+            code[q] = __float_as_uint(r + 12582912.0f);
+          }
+          uint32_t o[2];
+#pragma unroll
+          for (int h = 0; h < 2; ++h) {
+            const uint32_t lo = __builtin_amdgcn_perm(code[4 * h + 1], code[4 * h], 0x0c0c0400u);
+            const uint32_t hi = __builtin_amdgcn_perm(code[4 * h + 3], code[4 * h + 2], 0x0c0c0400u);
+            o[h] = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+          }
+          *(uint2*)(xq + (size_t)m * xstride + (size_t)c * AQ_VEC) = make_uint2(o[0], o[1]);
+        }
+      }
+    }
+  }
+  __syncthreads();
+  if (blockIdx.x == 0 && g.a_scale_out && (int)threadIdx.x < g.M) g.a_scale_out[threadIdx.x] = sc[threadIdx.x];
+}
+
 template <int XT, class P>
 __device__ __forceinline__ void rows_finish_fp8(const GemvArgs& g, const v4i (&cur)[P::NPASS][P::QCH], uint8_t* xq,
                                                 int xstride, float* sc, float* red) {
@@ -530,8 +692,9 @@ __global__ __launch_bounds__(NW * 64) void gemv_kernel(GemvArgs g) {
 // so that the 16 token rows of a fragment read fall into different banks; the lanes of token rows
 // past M substitute zeros).  No activation registers: the weight pipeline can be as deep as with
 // XS, for any number of row groups per block.
+// SF32: the fused form with fp32 SmoothQuant divisors (int8 only).
 template <int OP, int STEPS, int NW, int D, int MT = 1, bool HALF = false, bool XS = false, int XT = -1,
-          int MAXM = 1>
+          int MAXM = 1, bool SF32 = false>
 __global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(GemvArgs g, int halves) {
   static_assert(STEPS % D == 0, "pipeline depth must divide the steps per group");
   static_assert(!XS || MT == 1, "streamed activations: one tile of tokens");
@@ -542,7 +705,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(GemvArgs g, int ha
   typedef RowsPlan<NW * 64, KROW, MAXM> QP;
   __shared__ __attribute__((aligned(16))) uint8_t xq[FUSED ? MAXM * XSTRIDE : 16];
   __shared__ float xsc[FUSED ? MAXM : 1];
-  __shared__ float xred[FUSED ? MAXM * QP::WPR + NW : 1];
+  __shared__ float xred[FUSED ? 2 * MAXM * QP::WPR + NW : 1];
   typedef typename std::conditional<OP == FMSMO_OP_I8, int, float>::type AccT;
   typedef AccT Acc4 __attribute__((ext_vector_type(4)));
   constexpr int NRED = 2;  // exchange buffers alternate, one barrier per group
@@ -601,7 +764,8 @@ __global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(GemvArgs g, int ha
   // at different K steps so that they do not all ask L2 for the same lines at once: 11.7 / 14.3).
   v4i xf[XS || FUSED ? 1 : MT][XS || FUSED ? 1 : STEPS][2];
   v4i xb[XS && !FUSED ? D : 1][2];
-  v4i qcur[FUSED ? QP::NPASS : 1][FUSED ? QP::QCH : 1], qsm[FUSED ? QP::QCH : 1];
+  v4i qcur[FUSED ? QP::NPASS : 1][FUSED ? QP::QCH : 1], qsm[FUSED && !SF32 ? QP::QCH : 1];
+  float qsd[SF32 ? QP::QCH : 1][8];
   const __amdgpu_buffer_rsrc_t rsrc_x = __builtin_amdgcn_make_buffer_rsrc(
       (void*)g.a, 0, FUSED ? 0 : (int)((int64_t)(g.M - 1) * g.lda + g.K), 0x00020000);
   const int vx = r * (int)g.lda + kwave + kg * 16;
@@ -610,7 +774,9 @@ __global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(GemvArgs g, int ha
     x[0] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_x, v, s * 128, 0));
     x[1] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_x, v, s * 128 + 64, 0));
   };
-  if constexpr (FUSED) {
+  if constexpr (SF32) {
+    rows_request_f32s<QP>(g, qcur, qsd);
+  } else if constexpr (FUSED) {
     rows_request<QP>(g, qcur, qsm);
   } else if constexpr (XS) {
 #pragma unroll
@@ -631,7 +797,8 @@ __global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(GemvArgs g, int ha
   const int em = min((int)(threadIdx.x & 15), g.M - 1);
   float as;
   if constexpr (FUSED) {
-    if constexpr (OP == FMSMO_OP_I8) rows_finish_i8<XT, QP>(g, qcur, qsm, xq, XSTRIDE, xsc, xred);
+    if constexpr (SF32) rows_finish_i8_f32s<XT, QP>(g, qcur, qsd, xq, XSTRIDE, xsc, xred);
+    else if constexpr (OP == FMSMO_OP_I8) rows_finish_i8<XT, QP>(g, qcur, qsm, xq, XSTRIDE, xsc, xred);
     else rows_finish_fp8<XT, QP>(g, qcur, xq, XSTRIDE, xsc, xred);
     as = xsc[em];
   } else {
@@ -1119,37 +1286,59 @@ extern "C" int fmsmo_decode_linear_ok(int64_t M, int64_t K) {
   const int kch = (int)((K + 1023) / 1024);
   return kch == 1 || kch == 2 || kch == 4 || kch == 8;
 }
+// the same with fp32 SmoothQuant divisors (the streaming kernel's fused form only; the fp32
+// quantizer is heavier: us, two launches -> fused at 1 / 2 / 4 tokens: o 8.7 -> 8.1, 9.5 -> 9.2,
+// 9.6 -> 10.2; qkv 10.5 -> 8.9, 11.1 -> 9.9, 10.9 -> 11.5; gate+up 24.7 -> 23.3, 26.0 -> 23.3,
+// 24.7 -> 24.7; down, one token, 17.2 -> 14.5)
+extern "C" int fmsmo_decode_linear_f32s_ok(int64_t M, int64_t K) {
+  if (M < 1 || M > 2) return 0;
+  return K == 4096 || (M == 1 && (K == 14336 || K == 12800));
+}
 
 template <int OP, int XT>
 static int decode_fused_launch(const GemvArgs& g, hipStream_t st) {
   // the streaming kernel's fused form: (waves, steps per wave, loads in flight, most tokens)
+  const bool sf32 = g.smooth && g.smooth_f32;
   int shape = 0;
   if (g.K == 14336) shape = 814;
   else if (g.K == 12800) shape = 1010;
-  else if (g.K == 4096 && g.M > 1) shape = 1602;
+  else if (g.K == 4096 && (g.M > 1 || sf32)) shape = 1602;
   // (int8, one token, K = 4096 with at most one row group per compute unit: this form instead of
   // the row kernel's, us at N = 4096 / 1024 from bf16 with SmoothQuant: 6.6 -> 6.3 / 5.3 -> 4.6;
   // e4m3 stays with the row kernel there, whose fp32 sums are those of the two-call path)
   else if (g.K == 4096 && OP == FMSMO_OP_I8 && g.N <= 4096) shape = 1602;
+  if (sf32 && (!shape || OP != FMSMO_OP_I8)) return FMSMO_ERR_UNSUPPORTED;
   if (shape) {
     const int halves = (g.N + 7) / 8;
     const int nblocks = halves < 256 ? halves : 256;
     const bool whole_groups = halves % (2 * nblocks) == 0;
     const bool one_group = halves == 2 * nblocks;  // the kernel without its loop over row groups
     dim3 grid((unsigned)nblocks);
-#define STREAM_F(NWV, ST, DV, MM)                                                                    \
+#define STREAM_G(NWV, ST, DV, MM, SF)                                                                \
   if (whole_groups && one_group)                                                                     \
-    hipLaunchKernelGGL((gemv_stream_kernel<OP, ST, NWV, DV, 1, false, true, XT, MM>), grid, dim3(NWV * 64), 0, st, g, halves); \
+    hipLaunchKernelGGL((gemv_stream_kernel<OP, ST, NWV, DV, 1, false, true, XT, MM, SF>), grid, dim3(NWV * 64), 0, st, g, halves); \
   else if (whole_groups)                                                                             \
-    hipLaunchKernelGGL((gemv_stream_kernel<OP, ST, NWV, DV, 1, false, false, XT, MM>), grid, dim3(NWV * 64), 0, st, g, halves); \
+    hipLaunchKernelGGL((gemv_stream_kernel<OP, ST, NWV, DV, 1, false, false, XT, MM, SF>), grid, dim3(NWV * 64), 0, st, g, halves); \
   else                                                                                               \
-    hipLaunchKernelGGL((gemv_stream_kernel<OP, ST, NWV, DV, 1, true, false, XT, MM>), grid, dim3(NWV * 64), 0, st, g, halves)
+    hipLaunchKernelGGL((gemv_stream_kernel<OP, ST, NWV, DV, 1, true, false, XT, MM, SF>), grid, dim3(NWV * 64), 0, st, g, halves)
+#define STREAM_F(NWV, ST, DV, MM)                                       \
+  if constexpr (OP == FMSMO_OP_I8) {                                    \
+    if (sf32) { STREAM_G(NWV, ST, DV, MM, true); }                      \
+    else { STREAM_G(NWV, ST, DV, MM, false); }                          \
+  } else { STREAM_G(NWV, ST, DV, MM, false); }
     switch (shape) {
-      case 814: if (g.M == 1) { STREAM_F(8, 14, 7, 1); } else { STREAM_F(8, 14, 7, 4); } break;
-      case 1010: if (g.M == 1) { STREAM_F(10, 10, 5, 1); } else { STREAM_F(10, 10, 5, 4); } break;
-      default: if (g.M == 1) { STREAM_F(16, 2, 2, 1); } else { STREAM_F(16, 2, 2, 4); } break;
+      case 814:
+        if (g.M == 1) { STREAM_F(8, 14, 7, 1) } else if (sf32) return FMSMO_ERR_UNSUPPORTED; else { STREAM_G(8, 14, 7, 4, false); }
+        break;
+      case 1010:
+        if (g.M == 1) { STREAM_F(10, 10, 5, 1) } else if (sf32) return FMSMO_ERR_UNSUPPORTED; else { STREAM_G(10, 10, 5, 4, false); }
+        break;
+      default:
+        if (g.M == 1) { STREAM_F(16, 2, 2, 1) } else { STREAM_F(16, 2, 2, 4) }
+        break;
     }
 #undef STREAM_F
+#undef STREAM_G
     return fmsmo_check_launch();
   }
   const int kch = (int)((g.K + 1023) / 1024);
@@ -1171,7 +1360,7 @@ static int decode_fused_launch(const GemvArgs& g, hipStream_t st) {
 }
 
 extern "C" int fmsmo_decode_linear_i8(const void* x, int x_dtype, int64_t ldx, const void* smooth,
-                                      int saturate, const int8_t* w, int64_t ldw,
+                                      int smooth_dtype, int saturate, const int8_t* w, int64_t ldw,
                                       const float* w_scale, int64_t w_scale_n, const void* bias,
                                       int bias_dtype, int epilogue, void* y, int y_dtype,
                                       int64_t ldy, float* a_scale_out, int64_t M, int64_t N,
@@ -1179,7 +1368,10 @@ extern "C" int fmsmo_decode_linear_i8(const void* x, int x_dtype, int64_t ldx, c
   if (!x || !w || !w_scale || !y) return FMSMO_ERR_NULL;
   if (M <= 0 || N <= 0 || K <= 0 || ldx < K || ldw < K || ldy < N) return FMSMO_ERR_SHAPE;
   if (w_scale_n != 1 && w_scale_n != N) return FMSMO_ERR_SHAPE;
-  if ((x_dtype != FMSMO_F16 && x_dtype != FMSMO_BF16) || !fmsmo_decode_linear_ok(M, K)) return FMSMO_ERR_UNSUPPORTED;
+  if (x_dtype != FMSMO_F16 && x_dtype != FMSMO_BF16) return FMSMO_ERR_UNSUPPORTED;
+  const bool sf32 = smooth && smooth_dtype == FMSMO_F32;
+  if (smooth && !sf32 && smooth_dtype != x_dtype) return FMSMO_ERR_UNSUPPORTED;
+  if (!(sf32 ? fmsmo_decode_linear_f32s_ok(M, K) : fmsmo_decode_linear_ok(M, K))) return FMSMO_ERR_UNSUPPORTED;
   if (N >= (1 << 30) || N * ldw >= (1ll << 40)) return FMSMO_ERR_UNSUPPORTED;
   if (y_dtype < 0 || y_dtype > 2 || (bias && (bias_dtype < 0 || bias_dtype > 2))) return FMSMO_ERR_UNSUPPORTED;
   if (epilogue < FMSMO_EPI_REF_F16 || epilogue > FMSMO_EPI_F32_MULADD) return FMSMO_ERR_UNSUPPORTED;
@@ -1193,6 +1385,7 @@ extern "C" int fmsmo_decode_linear_i8(const void* x, int x_dtype, int64_t ldx, c
   g.bias = bias; g.bias_dtype = bias_dtype; g.epi = epilogue;
   g.y = y; g.y_dtype = y_dtype; g.ldy = ldy;
   g.x16 = (const u16*)x; g.ldx = ldx; g.smooth = (const u16*)smooth; g.saturate = saturate;
+  g.smooth_f32 = sf32 ? 1 : 0;
   g.a_scale_out = a_scale_out;
   return x_dtype == FMSMO_F16 ? decode_fused_launch<FMSMO_OP_I8, FMSMO_F16>(g, (hipStream_t)stream)
                               : decode_fused_launch<FMSMO_OP_I8, FMSMO_BF16>(g, (hipStream_t)stream);

@@ -24,7 +24,7 @@ F8E_SAT, F8E_PER_TENSOR, F8E_PER_ROW = 0, 1, 2
 FP8_LINEAR, FP8_FPXACC, FP8_FPXACC_DL8 = 0, 1, 2
 WQ_MUL, WQ_DIV = 0, 1
 MS_PER_TOKEN, MS_SYMM, MS_ASYMM = 0, 1, 2
-ABI_VERSION = 1
+ABI_VERSION = 2
 PLAN_DECODE, PLAN_TILE_REGISTER_STAGED, PLAN_TILE_LDS_DMA, PLAN_GENERIC = 0, 1, 2, 3
 
 _P, _I, _L, _F = c_void_p, c_int, c_int64, c_float
@@ -47,7 +47,7 @@ SIGNATURES = {
     "fmsmo_gemm_fp8_dq_ws": [_P, _L, _P, _L, _P, _L, _P, _L, _P, _I, _P, _I, _L, _L, _L, _L, _P, _L, _P],
     "fmsmo_gemv_i8_dq": [_P, _L, _P, _L, _P, _L, _P, _L, _P, _I, _I, _P, _I, _L, _L, _L, _L, _P],
     "fmsmo_gemv_fp8_dq": [_P, _L, _P, _L, _P, _L, _P, _L, _P, _I, _P, _I, _L, _L, _L, _L, _P],
-    "fmsmo_decode_linear_i8": [_P, _I, _L, _P, _I, _P, _L, _P, _L, _P, _I, _I, _P, _I, _L, _P, _L, _L, _L, _P],
+    "fmsmo_decode_linear_i8": [_P, _I, _L, _P, _I, _I, _P, _L, _P, _L, _P, _I, _I, _P, _I, _L, _P, _L, _L, _L, _P],
     "fmsmo_decode_linear_fp8": [_P, _I, _L, _P, _L, _P, _L, _P, _I, _P, _I, _L, _P, _L, _L, _L, _P],
     "fmsmo_matmul_chunk_i8": [_P, _L, _P, _L, _P, _P, _L, _L, _L, _L, _I, _I, _I, _I, _P],
     "fmsmo_matmul_chunk_fp": [_P, _L, _P, _L, _I, _P, _P, _L, _L, _L, _L, _I, _I, _I, _I, _P],
@@ -69,6 +69,7 @@ OTHER = {
     "fmsmo_last_error": ([], c_char_p),
     "fmsmo_gemm_workspace_bytes": ([c_int64, c_int64, c_int64], c_int64),
     "fmsmo_decode_linear_ok": ([c_int64, c_int64], c_int),
+    "fmsmo_decode_linear_f32s_ok": ([c_int64, c_int64], c_int),
     "fmsmo_gemm_tail_columns": ([c_int64, c_int64, c_int64], c_int64),
 }
 

@@ -700,19 +700,23 @@ _DECODE_OK = {}
 
 def decode_linear_ok(x, smooth, K):
     """Can ``decode_linear_i8`` serve these activations?  fp16 / bf16, SmoothQuant divisors of the
-    same dtype (or none); one token at K up to 8192 in one of the decode kernel's sizes or at
-    14336 / 12800, up to four tokens at K = 4096, up to three at 14336 / 12800."""
+    same dtype (or none): one token at K up to 8192 in one of the decode kernel's sizes or at
+    14336 / 12800, up to four tokens at K = 4096, up to three at 14336 / 12800.  fp32 divisors
+    (the quantizer then runs in fp32): K = 4096 up to two tokens, 14336 / 12800 one token."""
     if x.dim() != 2 or x.dtype not in (torch.float16, torch.bfloat16) or not x.is_cuda:
         return False
-    if smooth is not None and (smooth.dtype != x.dtype or smooth.numel() != K):
+    f32s = smooth is not None and smooth.dtype == torch.float32
+    if smooth is not None and ((smooth.dtype != x.dtype and not f32s) or smooth.numel() != K):
         return False
-    key = (x.shape[0], K)
+    key = (x.shape[0], K, f32s)
     if torch.compiler.is_compiling():
         # answers of earlier eager calls only (a foreign-function call cannot be traced); a shape
         # never seen eagerly takes the two-kernel path, which serves every shape
         return _DECODE_OK.get(key, False)
     if key not in _DECODE_OK:
-        _DECODE_OK[key] = bool(L.load().fmsmo_decode_linear_ok(x.shape[0], K))
+        lib = L.load()
+        ok = lib.fmsmo_decode_linear_f32s_ok if f32s else lib.fmsmo_decode_linear_ok
+        _DECODE_OK[key] = bool(ok(x.shape[0], K))
     return _DECODE_OK[key]
 
 
@@ -727,8 +731,8 @@ def _decode_linear_i8_impl(x, w, w_scale, bias, smooth, out_dtype, exact_ref, sa
     if smooth is not None:
         _need_gpu(smooth)
         smooth = smooth.detach().reshape(-1).contiguous()
-        if smooth.numel() != K or smooth.dtype != x.dtype:
-            raise ValueError("smooth must have K elements of x's dtype")
+        if smooth.numel() != K or smooth.dtype not in (x.dtype, torch.float32):
+            raise ValueError("smooth must have K elements of x's dtype or fp32")
         if smooth.data_ptr() % 16:
             smooth = smooth.clone()
     if bias is not None:
@@ -739,7 +743,8 @@ def _decode_linear_i8_impl(x, w, w_scale, bias, smooth, out_dtype, exact_ref, sa
     y = torch.empty((M, N), dtype=out_dtype, device=x.device)
     a_scale = torch.empty((M,), dtype=torch.float32, device=x.device)
     with _dev(x):
-        L.call("fmsmo_decode_linear_i8", x.data_ptr(), _dt(x), _ld(x), _ptr(smooth), int(bool(saturate)),
+        L.call("fmsmo_decode_linear_i8", x.data_ptr(), _dt(x), _ld(x), _ptr(smooth),
+               _dt(smooth) if smooth is not None else 0, int(bool(saturate)),
                w.data_ptr(), _ld(w), w_scale.data_ptr(), w_scale.numel(), _ptr(bias),
                _dt(bias) if bias is not None else 0, L.EPI_REF_F16 if exact_ref else L.EPI_F32,
                y.data_ptr(), _DT[out_dtype], N, a_scale.data_ptr(), M, N, K, _stream(x))

@@ -23,7 +23,7 @@
 extern "C" {
 #endif
 
-#define FMSMO_ABI_VERSION 1
+#define FMSMO_ABI_VERSION 2
 
 typedef void* fmsmo_stream_t; /* hipStream_t */
 
@@ -393,13 +393,18 @@ int fmsmo_gemv_fp8_dq(const uint8_t* a, int64_t lda, const uint8_t* b, int64_t l
  * flight); M <= 4 at K = 4096 and M <= 3 at K = 14336 / 12800 (the same kernel).  With more
  * tokens or other row lengths the quantization that every block repeats costs more than the
  * launch it saves, and the call returns FMSMO_ERR_UNSUPPORTED: use the two kernels.
+ * smooth_dtype = FMSMO_F32 (x fp16 / bf16 with fp32 divisors: torch promotes the whole quantizer
+ * to fp32, the arithmetic of fmsmo_quant_act_i8_pertoken with compute_dtype FMSMO_F32) is served
+ * by the streaming kernel where fmsmo_decode_linear_f32s_ok(M, K) != 0: K = 4096 up to two tokens,
+ * K = 14336 / 12800 one token; otherwise smooth_dtype must equal x_dtype.
  * x and smooth 16-byte aligned, ldx % 8 == 0, w as for fmsmo_gemv_i8_dq.
  * Reference: QLinearINT8Deploy.forward for a decode step -- qa_dynamic_max_qfunc followed by
  * iaddmm_int (fms_mo/modules/linear.py:1085-1100, 1177-1188, 1309-1338); no fused counterpart.
  */
 int fmsmo_decode_linear_ok(int64_t M, int64_t K);
+int fmsmo_decode_linear_f32s_ok(int64_t M, int64_t K);
 int fmsmo_decode_linear_i8(const void* x, int x_dtype, int64_t ldx, const void* smooth,
-                           int saturate, const int8_t* w, int64_t ldw, const float* w_scale,
+                           int smooth_dtype, int saturate, const int8_t* w, int64_t ldw, const float* w_scale,
                            int64_t w_scale_n, const void* bias, int bias_dtype, int epilogue,
                            void* y, int y_dtype, int64_t ldy, float* a_scale_out, int64_t M,
                            int64_t N, int64_t K, fmsmo_stream_t stream);

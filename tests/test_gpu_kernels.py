@@ -1021,6 +1021,61 @@ def test_fused_decode_linear_fp8_several_tokens(dev, NK, M, dt):
     assert torch.equal(flat(y[~fin.to(dev)]), flat(ref[~fin.to(dev)]))
 
 
+@pytest.mark.parametrize("NK", [(4096, 4096), (6144, 4096), (28672, 4096), (1000, 4096), (24, 4096),
+                                (4096, 14336), (1000, 14336), (8200, 14336), (4104, 12800)])
+@pytest.mark.parametrize("M", [1, 2, 3])
+@pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("special", [None, "rows", "divisor"])
+def test_fused_decode_linear_fp32_divisors(dev, NK, M, dt, special):
+    """fp16 / bf16 activations with fp32 SmoothQuant divisors (quantizer buffers left in fp32 under
+    a 16-bit model): torch promotes the quantizer to fp32.  Scales, codes (through the exact int32
+    product) and outputs equal the two kernels' bit for bit; the scales equal the oracle's.  Rows
+    and divisors off the fast division path (zeros, an infinity, a tiny bf16 row; a divisor
+    outside 2^-60 .. 2^60) take IEEE divisions in both."""
+    N, Kd = NK
+    kn = K()
+    x = torch.randn(M, Kd, generator=gen(201)).to(dt)
+    x[:, 5] *= 30.0
+    sm = (torch.rand(Kd, generator=gen(202)) * 3 + 0.2).float()
+    if special == "rows":
+        if M == 1:
+            x[0, 100] = float("inf")
+        elif dt == torch.bfloat16:
+            x[0] = x[0] * 1e-30  # a row whose largest quotient lies under 2^-80
+            x[1] = 0.0
+        else:
+            x[0, 100] = float("inf")
+            x[1] = 0.0
+    elif special == "divisor":
+        sm[11] = 1e-20
+    xd, smd = x.to(dev), sm.to(dev)
+    if not kn.decode_linear_ok(xd, smd, Kd):
+        assert M > 2 or (M > 1 and Kd > 4096)  # fp32 divisors: two tokens at K = 4096, one at long rows
+        return
+    w = _rand_i8((N, Kd), 203).to(dev)
+    s_w = (torch.rand(N, generator=gen(204)) * 1e-3 + 1e-5).to(dev)
+    bias = (torch.randn(N, generator=gen(205)) * 0.01).to(dt).to(dev)
+    q, s = kn.quant_act_i8_pertoken(xd, smd, compute_dtype=torch.float32)
+    for exact_ref, od in ((True, torch.float16), (False, torch.float32)):
+        ref = kn.gemm_i8_dq(q, w, s, s_w, bias, out_dtype=od, exact_ref=exact_ref)
+        y, s_f = kn.decode_linear_i8(xd, w, s_w, bias, smd, out_dtype=od, exact_ref=exact_ref)
+        assert torch.equal(s_f.view(torch.int32), s.view(torch.int32))
+        bits = torch.int32 if od == torch.float32 else torch.int16
+        assert torch.equal(y.view(bits), ref.view(bits))
+    # the codes themselves, through the exact integer product with rows that hold a single one
+    n_id = min(N, Kd)
+    w_id = torch.zeros(N, Kd, dtype=torch.int8)
+    w_id[torch.arange(n_id), torch.arange(n_id)] = 1
+    y_id, _ = kn.decode_linear_i8(xd, w_id.to(dev), torch.ones(N, device=dev), None, smd, out_dtype=torch.float32,
+                                  exact_ref=False)
+    fin = torch.isfinite(s)
+    want = q.float()[:, :n_id] * s.reshape(-1, 1)
+    assert torch.equal(y_id[:, :n_id][fin], want[fin])
+    if special is None:
+        _, s_ref, _ = O.quant_act_pertoken_i8(x, sm)
+        assert s_ref.dtype == torch.float32 and torch.equal(s_f.cpu(), s_ref.reshape(-1))
+
+
 @pytest.mark.parametrize("row", ["zeros", "inf", "overflow"])
 @pytest.mark.parametrize("Kd", [4096, 14336])
 def test_fused_decode_linear_special_rows(dev, row, Kd):
@@ -1058,7 +1113,9 @@ def test_fused_decode_linear_rejects_what_it_does_not_serve(dev):
     assert kn.decode_linear_ok(torch.randn(3, 14336, device=dev).half(), None, 14336)
     assert not kn.decode_linear_ok(torch.randn(4, 14336, device=dev).half(), None, 14336)
     assert kn.decode_linear_ok(torch.randn(1, 14336, device=dev).half(), None, 14336)
-    assert not kn.decode_linear_ok(x[:1], torch.ones(4096, device=dev), 4096)  # fp32 divisors
+    assert kn.decode_linear_ok(x[:1], torch.ones(4096, device=dev), 4096)      # fp32 divisors: K = 4096 ...
+    assert not kn.decode_linear_ok(torch.randn(1, 2048, device=dev).half(), torch.ones(2048, device=dev), 2048)
+    assert not kn.decode_linear_ok(torch.randn(2, 14336, device=dev).half(), torch.ones(14336, device=dev), 14336)
     assert kn.decode_linear_ok(x[:1], None, 4096)
     w = torch.zeros(64, 2048, dtype=torch.int8, device=dev)
     with pytest.raises(RuntimeError):

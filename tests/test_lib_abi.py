@@ -25,7 +25,7 @@ def test_header_declares_the_expected_entry_points():
               "fmsmo_quant_act_i8_mulscale", "fmsmo_zero_shift_bias", "fmsmo_quant_i8_affine",
               "fmsmo_bmm_i8_dq", "fmsmo_bmm_fp8_dq", "fmsmo_gemm_i8_dq_ws", "fmsmo_gemm_fp8_dq_ws", "fmsmo_gemm_i8_dq_noalloc",
               "fmsmo_gemm_tail_columns", "fmsmo_quant_act_i8_static_t", "fmsmo_quant_act_i8_dynamic", "fmsmo_fake_quant_fp8",
-              "fmsmo_gemm_workspace_bytes", "fmsmo_decode_linear_i8", "fmsmo_decode_linear_fp8", "fmsmo_decode_linear_ok", "fmsmo_debug_clock_probe", "fmsmo_debug_stream_read", "fmsmo_gemm_plan", "fmsmo_abi_version", "fmsmo_status_str", "fmsmo_last_error"]:
+              "fmsmo_gemm_workspace_bytes", "fmsmo_decode_linear_i8", "fmsmo_decode_linear_fp8", "fmsmo_decode_linear_ok", "fmsmo_decode_linear_f32s_ok", "fmsmo_debug_clock_probe", "fmsmo_debug_stream_read", "fmsmo_gemm_plan", "fmsmo_abi_version", "fmsmo_status_str", "fmsmo_last_error"]:
         assert s in syms
 
 
@@ -36,7 +36,7 @@ def test_library_exports_every_declared_symbol():
     for s in declared_symbols():
         assert hasattr(lib, s), f"{s} declared in include/fmsmo_hip.h but not exported"
     assert set(_lib.SIGNATURES) | set(_lib.OTHER) == set(declared_symbols())
-    assert lib.fmsmo_abi_version() == 1
+    assert lib.fmsmo_abi_version() == 2
     assert lib.fmsmo_status_str(0) == b"ok"
 
 
