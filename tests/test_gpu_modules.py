@@ -320,12 +320,15 @@ def test_operator_twins_agree_with_the_kernels_on_shapes(dev):
 
 
 @pytest.mark.parametrize("smoothq", [False, True])
+@pytest.mark.parametrize("buffers", ["fp16", "fp32"])
 @pytest.mark.parametrize("K,N", [(4096, 1024), (14336, 512), (1024, 768)])
-def test_decode_step_equals_the_rows_of_a_larger_batch(dev, smoothq, K, N):
-    """The deployed fp16 module takes the fused one-launch path for a single token.  Per-token
-    quantization makes every output row a function of its own input row only, so the decode step
-    must reproduce, bit for bit, the corresponding rows of a 40-token batch (which runs the
-    quantizer and the GEMM as two kernels)."""
+def test_decode_step_equals_the_rows_of_a_larger_batch(dev, smoothq, buffers, K, N):
+    """The deployed module takes the fused one-launch path for a decode step of a few tokens, with
+    its buffers cast to fp16 (the lowering helper's flow) or left in fp32 under fp16 activations
+    (the SmoothQuant divide then promotes the quantizer to fp32).  Per-token quantization makes
+    every output row a function of its own input row only, so the decode step must reproduce, bit
+    for bit, the corresponding rows of a 40-token batch (which runs the quantizer and the GEMM as
+    two kernels)."""
     from fms_mo_amd.modules.linear import QLinearINT8Deploy
 
     m = make_qlinear(None, K, N, smoothq=smoothq, seed=7)
@@ -333,11 +336,14 @@ def test_decode_step_equals_the_rows_of_a_larger_batch(dev, smoothq, K, N):
     if smoothq:
         m.set_act_scale(x.float().abs().amax(dim=0))
     dep = QLinearINT8Deploy.from_fms_mo(m, use_int_kernel="cutlass", use_dynamic_max_act_Qfunc=-1,
-                                        recalc_clipvals=False, target_device="cpu").half().to(dev)
+                                        recalc_clipvals=False, target_device="cpu")
+    dep = dep.half().to(dev) if buffers == "fp16" else dep.to(dev)
+    if smoothq:
+        assert dep.smoothq_scale.dtype == (torch.float16 if buffers == "fp16" else torch.float32)
     xd = x.to(dev)
     full = dep(xd).clone()
     full_scale = dep.input_scale.clone()
-    for M in (1, 2, 4):  # one token: the fused launch; more: quantizer and decode kernel
+    for M in (1, 2, 4):  # fused launch where it is served; else quantizer and decode kernel
         y = dep(xd[:M])
         assert torch.equal(y.view(torch.int16), full[:M].view(torch.int16))
         assert torch.equal(dep.input_scale.reshape(-1), full_scale.reshape(-1)[:M])
