@@ -95,15 +95,15 @@ static bool use_register_staged(int op) {
   (void)op;
   return true;
 }
-template <int OP, bool GROUPED = false, int BN = 256, bool ONE_SLAB = false, int BM = 256, class Epi>
+template <int OP, bool GROUPED = false, int BN = 256, class Epi>
 void launch_rs(const GemmArgs& g0, const Epi& epi, hipStream_t st) {
   GemmArgs g = g0;
   g.clk = fmsmo_clock_probe();
   g.grid_n = div_up(g.N, BN);
-  if (!GROUPED) g.grid_m = div_up(g.M, BM);
+  if (!GROUPED) g.grid_m = div_up(g.M, 256);
   g.group_m = 4;
   dim3 grid((unsigned)(g.grid_m * g.grid_n)), block(256);
-  hipLaunchKernelGGL((gemm_rs_kernel<OP, Epi, GROUPED, BN, ONE_SLAB, BM>), grid, block, 0, st, g, epi);
+  hipLaunchKernelGGL((gemm_rs_kernel<OP, Epi, GROUPED, BN>), grid, block, 0, st, g, epi);
 }
 
 // Reduction of exactly 128 bytes (attention scores): persistent blocks over 128 x 256 tiles, two

@@ -19,28 +19,22 @@
 
 namespace fmsmo {
 
-//
-// ONE_SLAB: K == 128 (attention scores: head dimension 128).  The tile is one slab, so nothing is
-// prefetched: without the flag the pipeline would fetch slabs "1", "2" and "3" (clamped re-reads
-// of slab 0, 256 KiB per tile) and write them to LDS in front of the epilogue's stores.
-// With BM_ = 128 (wave tile 64 x 128, 128 accumulator registers, one 48 KiB slab) two blocks
-// share a compute unit, so that the load, multiply and store phases of neighbouring tiles overlap.
-template <int OP, class Epi, bool GROUPED = false, int BN_ = 256, bool ONE_SLAB = false, int BM_ = 256>
-__global__ __launch_bounds__(256, BM_ == 128 ? 2 : 1) void gemm_rs_kernel(GemmArgs g, Epi epi) {
+// (A reduction of a single slab, K == 128, has its own kernel: gemm_k128.hpp.)
+template <int OP, class Epi, bool GROUPED = false, int BN_ = 256>
+__global__ __launch_bounds__(256, 1) void gemm_rs_kernel(GemmArgs g, Epi epi) {
 #if defined(__HIP_DEVICE_COMPILE__)
   typedef Mma<OP> MM;
   typedef typename MM::Frag Frag;
   typedef typename MM::Acc Acc;
   static_assert(BN_ == 256 || BN_ == 192 || BN_ == 128, "tile width");
-  static_assert(BM_ == 256 || (BM_ == 128 && ONE_SLAB), "tile height (128 rows: single-slab mode only)");
-  constexpr int BM = BM_, BN = BN_, BK = 128, CPR = 8;
+  constexpr int BM = 256, BN = BN_, BK = 128, CPR = 8;
   constexpr int TM = BM / 2, TN = BN / 2, FM = TM / 32, FN = TN / 32;
   constexpr int NKS = BK / MM::KSTEP;   // MFMA k-steps per slab (int8 4, e4m3 2)
   constexpr int CL = MM::KSTEP / 32;    // 16-byte chunks per lane per k-step
   constexpr int SLAB = (BM + BN) * BK;  // 64 KiB (56 KiB for the 192-column tile)
   constexpr int NJ = BM / 32, NJB = BN / 32;  // row groups of 32 per thread: A, B
   static_assert(NKS % 2 == 0, "fragment buffers alternate per k-step");
-  __shared__ __attribute__((aligned(16))) uint8_t lds[(ONE_SLAB ? 1 : 2) * SLAB];
+  __shared__ __attribute__((aligned(16))) uint8_t lds[2 * SLAB];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -255,10 +249,7 @@ __global__ __launch_bounds__(256, BM_ == 128 ? 2 : 1) void gemm_rs_kernel(GemmAr
   // with slab 2, pairs [NP0, NPAIR) still staged (the first k-step of the loop writes them)
   // (slabs 0 and 1 are fetched together: the accumulators and fragments are not live yet, so
   // there are registers for a second staging set)
-  if constexpr (ONE_SLAB) {
-    load_slab(0);
-    store_slab(lds);
-  } else {
+  {
     load_slab(0);
     v4i ta[NJ], tb[NJB];
     const int k1 = slab_k0(1);
@@ -297,22 +288,6 @@ __global__ __launch_bounds__(256, BM_ == 128 ? 2 : 1) void gemm_rs_kernel(GemmAr
   __syncthreads();
   read_all(lds, 0, 0);
 
-  if constexpr (ONE_SLAB) {
-    // the k-steps of the only slab, nothing staged (the last one reads no further fragments)
-    [&]<int... KS>(std::integer_sequence<int, KS...>) {
-      (kstep(std::integral_constant<int, KS & 1>{}, lds, std::integral_constant<int, KS + 1>{},
-             std::integral_constant<int, (KS + 1) & 1>{}, lds, 0, C0{}, C0{}),
-       ...);
-    }(std::make_integer_sequence<int, NKS - 1>{});
-    [&]<int... R>(std::integer_sequence<int, R...>) {
-      (
-          [&] {
-            constexpr int I = R / FN, J = R % FN;
-            acc[I][J] = MM::mma(frag_a((NKS - 1) & 1, I), frag_b((NKS - 1) & 1, J), acc[I][J]);
-          }(),
-          ...);
-    }(std::make_integer_sequence<int, NMMA>{});
-  } else
   for (int s = 0; s < nslab; ++s) {
     uint8_t* cur = lds + (s & 1) * SLAB;
     uint8_t* nxt = lds + ((s + 1) & 1) * SLAB;
