@@ -106,12 +106,21 @@ def load() -> ctypes.CDLL:
     return lib
 
 
+def raise_status(name: str, rc: int) -> None:
+    lib = load()
+    msg = lib.fmsmo_status_str(rc).decode()
+    if rc in (5, 6):
+        msg += ": " + lib.fmsmo_last_error().decode()
+    raise FmsMoHipError(f"{name} failed with status {rc} ({msg})")
+
+
 def call(name: str, *args) -> None:
     """Invoke an entry point and raise on a non-zero status."""
-    lib = load()
-    rc = getattr(lib, name)(*args)
+    rc = getattr(load(), name)(*args)
     if rc != 0:
-        msg = lib.fmsmo_status_str(rc).decode()
-        if rc in (5, 6):
-            msg += ": " + lib.fmsmo_last_error().decode()
-        raise FmsMoHipError(f"{name} failed with status {rc} ({msg})")
+        raise_status(name, rc)
+
+
+def entry(name: str):
+    """The bound entry point itself (returns the status), for callers that keep it."""
+    return getattr(load(), name)

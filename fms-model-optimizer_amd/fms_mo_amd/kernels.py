@@ -640,8 +640,156 @@ def _as_scale(s, device):
     return torch.tensor([float(s)], dtype=torch.float32, device=device)
 
 
+# Lean forms of the three calls a decode step makes.  An eager call of a 5 us kernel is bound by
+# what the host does per launch; the general wrappers above spend about 60 Python-level calls on
+# argument handling.  These take the common case only -- plain, well-formed tensors on the current
+# GPU, outside a compiler trace -- with the checks written inline, and return None for anything
+# else, which then goes through the general path (and gets its error messages there).
+_T, _P = torch.Tensor, torch.nn.Parameter
+_COMPILING = torch.compiler.is_compiling
+_F32, _I8 = torch.float32, torch.int8
+_FN = {}
+
+
+def _fn(name):
+    f = _FN.get(name)
+    if f is None:
+        f = _FN[name] = L.entry(name)
+    return f
+
+
+def _mat(t, dtype):
+    """(rows, cols, row stride) of a plain 2-D CUDA tensor of `dtype` with unit inner stride on
+    the current GPU, else None."""
+    tt = type(t)
+    if (tt is not _T and tt is not _P) or t.dtype is not dtype or not t.is_cuda or t.dim() != 2:
+        return None
+    r, c = t.shape
+    s0, s1 = t.stride()
+    if s1 != 1 or (r > 1 and s0 < c):
+        return None
+    return r, c, (s0 if r > 1 else max(c, s0))
+
+
+def _vec32(t, n):
+    return (type(t) is _T and t.dtype is _F32 and t.is_cuda and t.dim() == 1 and t.is_contiguous()
+            and (t.numel() == n or t.numel() == 1) and not t.requires_grad)
+
+
+def _gemm_i8_dq_lean(a, w, a_scale, w_scale, bias, out_dtype, epilogue):
+    if _COMPILING() or _RAW_STREAM is None:
+        return None
+    ma, mw = _mat(a, _I8), _mat(w, _I8)
+    if ma is None or mw is None or ma[1] != mw[1] or not _vec32(a_scale, ma[0]) or not _vec32(w_scale, mw[0]):
+        return None
+    M, K, lda = ma
+    N, _, ldw = mw
+    if bias is not None:
+        tb = type(bias)
+        if ((tb is not _T and tb is not _P) or not bias.is_cuda or bias.dim() != 1 or bias.numel() != N
+                or not bias.is_contiguous() or bias.dtype not in _DT):
+            return None
+        bptr, bdt = bias.data_ptr(), _DT[bias.dtype]
+    else:
+        bptr, bdt = None, 0
+    idx = a.get_device()
+    if _CUR_DEVICE() != idx or out_dtype not in _DT:
+        return None
+    y = torch.empty((M, N), dtype=out_dtype, device=a.device)
+    nbytes = _WS_BYTES.get((M, N, K))
+    if nbytes is None:
+        nbytes = _WS_BYTES[(M, N, K)] = L.load().fmsmo_gemm_workspace_bytes(M, N, K)
+    if nbytes > 0:
+        ws = torch.empty((nbytes,), dtype=torch.uint8, device=a.device)
+        rc = _fn("fmsmo_gemm_i8_dq_ws")(a.data_ptr(), lda, w.data_ptr(), ldw, a_scale.data_ptr(), a_scale.numel(),
+                                        w_scale.data_ptr(), w_scale.numel(), bptr, bdt, epilogue, y.data_ptr(),
+                                        _DT[out_dtype], N, M, N, K, ws.data_ptr(), nbytes, _RAW_STREAM(idx))
+    else:
+        rc = _fn("fmsmo_gemm_i8_dq")(a.data_ptr(), lda, w.data_ptr(), ldw, a_scale.data_ptr(), a_scale.numel(),
+                                     w_scale.data_ptr(), w_scale.numel(), bptr, bdt, epilogue, y.data_ptr(),
+                                     _DT[out_dtype], N, M, N, K, _RAW_STREAM(idx))
+    if rc:
+        L.raise_status("fmsmo_gemm_i8_dq", rc)
+    return y
+
+
+def _smooth_ok(smooth, K):
+    ts = type(smooth)
+    return ((ts is _T or ts is _P) and smooth.is_cuda and smooth.dim() == 1 and smooth.numel() == K
+            and smooth.is_contiguous() and smooth.dtype in _DT and smooth.data_ptr() % 16 == 0)
+
+
+def _quant_act_i8_pertoken_lean(x, smooth, compute_dtype, saturate):
+    if _COMPILING() or _RAW_STREAM is None or x.dtype not in _DT:
+        return None
+    mx = _mat(x, x.dtype)
+    if mx is None:
+        return None
+    M, K, ldx = mx
+    if smooth is not None:
+        if not _smooth_ok(smooth, K):
+            return None
+        sptr, sdt = smooth.data_ptr(), _DT[smooth.dtype]
+        if compute_dtype is None:
+            compute_dtype = x.dtype if smooth.dtype is x.dtype else torch.promote_types(x.dtype, smooth.dtype)
+    else:
+        sptr, sdt = None, 0
+        if compute_dtype is None:
+            compute_dtype = x.dtype
+    idx = x.get_device()
+    if _CUR_DEVICE() != idx or compute_dtype not in _DT:
+        return None
+    q = torch.empty((M, K), dtype=_I8, device=x.device)
+    scale = torch.empty((M,), dtype=_F32, device=x.device)
+    rc = _fn("fmsmo_quant_act_i8_pertoken")(x.data_ptr(), _DT[x.dtype], ldx, sptr, sdt, _DT[compute_dtype],
+                                            1 if saturate else 0, q.data_ptr(), K, scale.data_ptr(), M, K,
+                                            _RAW_STREAM(idx))
+    if rc:
+        L.raise_status("fmsmo_quant_act_i8_pertoken", rc)
+    return q, scale
+
+
+def _decode_linear_i8_lean(x, w, w_scale, bias, smooth, out_dtype, exact_ref, saturate):
+    if _COMPILING() or _RAW_STREAM is None or x.dtype not in _DT:
+        return None
+    mx, mw = _mat(x, x.dtype), _mat(w, _I8)
+    if mx is None or mw is None or mx[1] != mw[1] or not _vec32(w_scale, mw[0]):
+        return None
+    M, K, ldx = mx
+    N, _, ldw = mw
+    if smooth is not None:
+        if not _smooth_ok(smooth, K):
+            return None
+        sptr, sdt = smooth.data_ptr(), _DT[smooth.dtype]
+    else:
+        sptr, sdt = None, 0
+    if bias is not None:
+        tb = type(bias)
+        if ((tb is not _T and tb is not _P) or not bias.is_cuda or bias.dim() != 1 or bias.numel() != N
+                or not bias.is_contiguous() or bias.dtype not in _DT):
+            return None
+        bptr, bdt = bias.data_ptr(), _DT[bias.dtype]
+    else:
+        bptr, bdt = None, 0
+    idx = x.get_device()
+    if _CUR_DEVICE() != idx or out_dtype not in _DT:
+        return None
+    y = torch.empty((M, N), dtype=out_dtype, device=x.device)
+    a_scale = torch.empty((M,), dtype=_F32, device=x.device)
+    rc = _fn("fmsmo_decode_linear_i8")(x.data_ptr(), _DT[x.dtype], ldx, sptr, sdt, 1 if saturate else 0, w.data_ptr(),
+                                       ldw, w_scale.data_ptr(), w_scale.numel(), bptr, bdt,
+                                       L.EPI_REF_F16 if exact_ref else L.EPI_F32, y.data_ptr(), _DT[out_dtype], N,
+                                       a_scale.data_ptr(), M, N, K, _RAW_STREAM(idx))
+    if rc:
+        L.raise_status("fmsmo_decode_linear_i8", rc)
+    return y, a_scale
+
+
 def quant_act_i8_pertoken(x, smooth=None, compute_dtype=None, saturate=False):  # noqa: F811
     """(q int8 [M,K], scale fp32 [M]) -- see fmsmo_quant_act_i8_pertoken."""
+    r = _quant_act_i8_pertoken_lean(x, smooth, compute_dtype, saturate)
+    if r is not None:
+        return r
     _need_gpu(x, smooth)
     if x.dim() != 2:
         raise ValueError("expected a 2-D tensor")
@@ -675,9 +823,13 @@ def gemm_i8_dq(a, w, a_scale, w_scale, bias=None, out_dtype=torch.float16, exact
                force_gemv=False, epilogue=None):
     """y [M,N] = dequant(a int8 [M,K] . w int8 [N,K]^T), see fmsmo_gemm_i8_dq.  ``epilogue`` (one of
     L.EPI_*) overrides ``exact_ref`` (True = L.EPI_REF_F16, False = L.EPI_F32)."""
-    _need_gpu(a, w, bias)
     if epilogue is None:
         epilogue = L.EPI_REF_F16 if exact_ref else L.EPI_F32
+    if not force_gemv:
+        y = _gemm_i8_dq_lean(a, w, a_scale, w_scale, bias, out_dtype, int(epilogue))
+        if y is not None:
+            return y
+    _need_gpu(a, w, bias)
     if _eager(a, w, bias) and (not torch.is_tensor(a_scale) or _eager(a_scale)) \
             and (not torch.is_tensor(w_scale) or _eager(w_scale)):
         return _gemm_i8_dq_impl(a, w, a_scale, w_scale, bias, out_dtype, int(epilogue), bool(force_gemv))
@@ -767,6 +919,9 @@ def decode_linear_i8(x, w, w_scale, bias=None, smooth=None, out_dtype=torch.floa
                      saturate=False):
     """(y [M,N], per-token scales fp32 [M]) = quantize x per token (see quant_act_i8_pertoken) and
     multiply with the int8 weights w [N,K], in one launch; check ``decode_linear_ok`` first."""
+    r = _decode_linear_i8_lean(x, w, w_scale, bias, smooth, out_dtype, exact_ref, saturate)
+    if r is not None:
+        return r
     _need_gpu(x, w, bias, smooth)
     if _eager(x, w, bias, smooth) and (not torch.is_tensor(w_scale) or _eager(w_scale)):
         return _decode_linear_i8_impl(x, w, w_scale, bias, smooth, out_dtype, bool(exact_ref), bool(saturate))
