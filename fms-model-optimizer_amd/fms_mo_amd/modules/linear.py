@@ -676,35 +676,41 @@ class QLinearINT8Deploy(nn.Linear):
             self._buffers["input_scale"] = s
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        with torch.no_grad():
-            org_dtype = x.dtype
-            tar_shape = tuple(x.shape[:-1]) + (self.weight.shape[0],)
-            x2 = x.reshape(-1, x.shape[-1])
-            if not x2.is_cuda:
-                raise RuntimeError("fms_mo_amd.QLinearINT8Deploy runs on an AMD GPU only; there is no CPU path")
-            use_sq = self._smoothq_active()
-            plain = (self.useDynMaxQfunc == -1 and self.use_int_kernel
-                     and not (x2.shape[1] > self.chunk_size or self.truncate_lsb > 0)
-                     and not getattr(self, "use_fake_zero_shift", False))
-            sq = self.smoothq_scale.reshape(-1) if use_sq else None
-            if plain and (sq is None or sq.numel() == x2.shape[1]) and \
-                    kernels.decode_linear_ok(x2, sq, x2.shape[1]):
-                # decode step of a few tokens: quantizer and weight-streaming matmul in one launch
-                y, s = kernels.decode_linear_i8(x2, self.weight, self._w_scale_f32(), self.bias, sq,
-                                                out_dtype=torch.float16, exact_ref=True)
-                self._set_input_scale(s.reshape(-1, 1))
-                y = y.to(self.acc_dtype)
-            elif plain and use_sq and sq.numel() == x2.shape[1]:
-                # SmoothQuant divide inside the quantizer kernel
-                q, s = kernels.quant_act_i8_pertoken(x2, sq, compute_dtype=_compute_dtype(x2.dtype, sq))
-                self._set_input_scale(s.reshape(-1, 1))
-                y = kernels.gemm_i8_dq(q, self.weight, s, self._w_scale_f32(), self.bias,
-                                       out_dtype=torch.float16, exact_ref=True).to(self.acc_dtype)
-            else:
+        # (the reference runs this forward under torch.no_grad; the kernel paths below create their
+        # outputs outside autograd anyway, and the torch-op branch enters no_grad itself -- an eager
+        # decode step is bound by what the host does per call, so nothing is done twice here)
+        org_dtype = x.dtype
+        K = x.shape[-1]
+        two_d = x.dim() == 2
+        x2 = x if two_d else x.reshape(-1, K)
+        if not x2.is_cuda:
+            raise RuntimeError("fms_mo_amd.QLinearINT8Deploy runs on an AMD GPU only; there is no CPU path")
+        use_sq = self._smoothq_active()
+        plain = (self.useDynMaxQfunc == -1 and self.use_int_kernel
+                 and not (K > self.chunk_size or self.truncate_lsb > 0)
+                 and not getattr(self, "use_fake_zero_shift", False))
+        sq = self.smoothq_scale.reshape(-1) if use_sq else None
+        if plain and (sq is None or sq.numel() == K) and kernels.decode_linear_ok(x2, sq, K):
+            # decode step of a few tokens: quantizer and weight-streaming matmul in one launch
+            y, s = kernels.decode_linear_i8(x2, self.weight, self._w_scale_f32(), self.bias, sq,
+                                            out_dtype=torch.float16, exact_ref=True)
+            self._set_input_scale(s.reshape(-1, 1))
+        elif plain and use_sq and sq.numel() == K:
+            # SmoothQuant divide inside the quantizer kernel
+            q, s = kernels.quant_act_i8_pertoken(x2, sq, compute_dtype=_compute_dtype(x2.dtype, sq))
+            self._set_input_scale(s.reshape(-1, 1))
+            y = kernels.gemm_i8_dq(q, self.weight, s, self._w_scale_f32(), self.bias,
+                                   out_dtype=torch.float16, exact_ref=True)
+        else:
+            with torch.no_grad():
                 if use_sq:
                     x2 = x2 / self.smoothq_scale
                 y = self.iaddmm(self.bias, x2, self.weight.t())
-            return y.reshape(tar_shape).to(org_dtype)
+        if y.dtype != self.acc_dtype:
+            y = y.to(self.acc_dtype)
+        if not two_d:
+            y = y.reshape(tuple(x.shape[:-1]) + (y.shape[-1],))
+        return y if y.dtype == org_dtype else y.to(org_dtype)
 
 
 class LinearFPxAcc(torch.nn.Linear):
