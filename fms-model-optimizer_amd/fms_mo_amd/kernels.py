@@ -785,6 +785,77 @@ def _decode_linear_i8_lean(x, w, w_scale, bias, smooth, out_dtype, exact_ref, sa
     return y, a_scale
 
 
+_E4M3 = torch.float8_e4m3fn
+
+
+def _bias_ok(bias, N):
+    tb = type(bias)
+    return ((tb is _T or tb is _P) and bias.is_cuda and bias.dim() == 1 and bias.numel() == N
+            and bias.is_contiguous() and bias.dtype in _DT)
+
+
+def _gemm_fp8_dq_lean(a, w, a_scale, w_scale, bias, out_dtype):
+    if _COMPILING() or _RAW_STREAM is None:
+        return None
+    ma, mw = _mat(a, _E4M3), _mat(w, _E4M3)
+    if ma is None or mw is None or ma[1] != mw[1] or not _vec32(a_scale, ma[0]) or not _vec32(w_scale, mw[0]):
+        return None
+    M, K, lda = ma
+    N, _, ldw = mw
+    if bias is not None:
+        if not _bias_ok(bias, N):
+            return None
+        bptr, bdt = bias.data_ptr(), _DT[bias.dtype]
+    else:
+        bptr, bdt = None, 0
+    idx = a.get_device()
+    if _CUR_DEVICE() != idx or out_dtype not in _DT:
+        return None
+    y = torch.empty((M, N), dtype=out_dtype, device=a.device)
+    nbytes = _WS_BYTES.get((M, N, K))
+    if nbytes is None:
+        nbytes = _WS_BYTES[(M, N, K)] = L.load().fmsmo_gemm_workspace_bytes(M, N, K)
+    if nbytes > 0:
+        ws = torch.empty((nbytes,), dtype=torch.uint8, device=a.device)
+        rc = _fn("fmsmo_gemm_fp8_dq_ws")(a.data_ptr(), lda, w.data_ptr(), ldw, a_scale.data_ptr(), a_scale.numel(),
+                                         w_scale.data_ptr(), w_scale.numel(), bptr, bdt, y.data_ptr(),
+                                         _DT[out_dtype], N, M, N, K, ws.data_ptr(), nbytes, _RAW_STREAM(idx))
+    else:
+        rc = _fn("fmsmo_gemm_fp8_dq")(a.data_ptr(), lda, w.data_ptr(), ldw, a_scale.data_ptr(), a_scale.numel(),
+                                      w_scale.data_ptr(), w_scale.numel(), bptr, bdt, y.data_ptr(),
+                                      _DT[out_dtype], N, M, N, K, _RAW_STREAM(idx))
+    if rc:
+        L.raise_status("fmsmo_gemm_fp8_dq", rc)
+    return y
+
+
+def _decode_linear_fp8_lean(x, w, w_scale, bias, out_dtype):
+    if _COMPILING() or _RAW_STREAM is None or x.dtype not in _DT:
+        return None
+    mx, mw = _mat(x, x.dtype), _mat(w, _E4M3)
+    if mx is None or mw is None or mx[1] != mw[1] or not _vec32(w_scale, mw[0]):
+        return None
+    M, K, ldx = mx
+    N, _, ldw = mw
+    if bias is not None:
+        if not _bias_ok(bias, N):
+            return None
+        bptr, bdt = bias.data_ptr(), _DT[bias.dtype]
+    else:
+        bptr, bdt = None, 0
+    idx = x.get_device()
+    if _CUR_DEVICE() != idx or out_dtype not in _DT:
+        return None
+    y = torch.empty((M, N), dtype=out_dtype, device=x.device)
+    a_scale = torch.empty((M,), dtype=_F32, device=x.device)
+    rc = _fn("fmsmo_decode_linear_fp8")(x.data_ptr(), _DT[x.dtype], ldx, w.data_ptr(), ldw, w_scale.data_ptr(),
+                                        w_scale.numel(), bptr, bdt, y.data_ptr(), _DT[out_dtype], N,
+                                        a_scale.data_ptr(), M, N, K, _RAW_STREAM(idx))
+    if rc:
+        L.raise_status("fmsmo_decode_linear_fp8", rc)
+    return y, a_scale
+
+
 def quant_act_i8_pertoken(x, smooth=None, compute_dtype=None, saturate=False):  # noqa: F811
     """(q int8 [M,K], scale fp32 [M]) -- see fmsmo_quant_act_i8_pertoken."""
     r = _quant_act_i8_pertoken_lean(x, smooth, compute_dtype, saturate)
@@ -838,6 +909,10 @@ def gemm_i8_dq(a, w, a_scale, w_scale, bias=None, out_dtype=torch.float16, exact
 
 
 def gemm_fp8_dq(a, w, a_scale, w_scale, bias=None, out_dtype=torch.bfloat16, force_gemv=False):  # noqa: F811
+    if not force_gemv:
+        y = _gemm_fp8_dq_lean(a, w, a_scale, w_scale, bias, out_dtype)
+        if y is not None:
+            return y
     _need_gpu(a, w, bias)
     if _eager(a, w, bias) and (not torch.is_tensor(a_scale) or _eager(a_scale)) \
             and (not torch.is_tensor(w_scale) or _eager(w_scale)):
@@ -962,8 +1037,11 @@ _register(
 
 
 def decode_linear_fp8(x, w, w_scale, bias=None, out_dtype=torch.bfloat16):
-    """(y [1,N], token scale fp32 [1]): dynamic per-token e4m3 quantizer (the FP8Linear recipe) and
+    """(y [M,N], token scales fp32 [M]): dynamic per-token e4m3 quantizer (the FP8Linear recipe) and
     the e4m3 weight-streaming matmul in one launch; check ``decode_linear_ok(x, None, K)`` first."""
+    r = _decode_linear_fp8_lean(x, w, w_scale, bias, out_dtype)
+    if r is not None:
+        return r
     _need_gpu(x, w, bias)
     if _eager(x, w, bias) and (not torch.is_tensor(w_scale) or _eager(w_scale)):
         return _decode_linear_fp8_impl(x, w, w_scale, bias, out_dtype)
