@@ -978,6 +978,33 @@ def test_fused_decode_linear_several_tokens(dev, NK, M, dt, smooth):
         assert torch.equal(s_f.cpu(), s_ref.reshape(-1).float())
 
 
+@pytest.mark.parametrize("NK", [(4096, 4096), (520, 4096), (4096, 14336), (264, 12800)])
+@pytest.mark.parametrize("M", [1, 2, 3, 4])
+def test_fused_decode_linear_bf16_divisor_outside_the_fast_range(dev, NK, M):
+    """A bf16 SmoothQuant divisor outside 2^-60 .. 2^60 sends every row through the IEEE division
+    routine (the fast quotient's residual could leave the normal range); scales and outputs must
+    still be the stand-alone quantizer's."""
+    N, Kd = NK
+    kn = K()
+    x = torch.randn(M, Kd, generator=gen(211)).bfloat16()
+    sm = (torch.rand(Kd, generator=gen(212)) * 3 + 0.2).bfloat16()
+    sm[11] = 1e-20
+    sm[Kd - 3] = 3e19
+    xd, smd = x.to(dev), sm.to(dev)
+    if not kn.decode_linear_ok(xd, smd, Kd):
+        assert M > 3 and Kd > 4096
+        return
+    w = _rand_i8((N, Kd), 213).to(dev)
+    s_w = (torch.rand(N, generator=gen(214)) * 1e-3 + 1e-5).to(dev)
+    q, s = kn.quant_act_i8_pertoken(xd, smd)
+    ref = kn.gemm_i8_dq(q, w, s, s_w, None, out_dtype=torch.float32, exact_ref=False)
+    y, s_f = kn.decode_linear_i8(xd, w, s_w, None, smd, out_dtype=torch.float32, exact_ref=False)
+    assert torch.equal(s_f.view(torch.int32), s.view(torch.int32))
+    assert torch.equal(y.view(torch.int32), ref.view(torch.int32))
+    _, s_ref, _ = O.quant_act_pertoken_i8(x, sm)
+    assert torch.equal(s_f.cpu(), s_ref.reshape(-1).float())
+
+
 @pytest.mark.parametrize("NK", [(4096, 4096), (6144, 4096), (1000, 4096), (4096, 14336), (1016, 12800)])
 @pytest.mark.parametrize("M", [2, 3, 4])
 @pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
