@@ -978,6 +978,30 @@ def test_fused_decode_linear_several_tokens(dev, NK, M, dt, smooth):
         assert torch.equal(s_f.cpu(), s_ref.reshape(-1).float())
 
 
+@pytest.mark.parametrize("NK", [(1000, 4096), (4096, 14336), (256, 2048)])
+@pytest.mark.parametrize("M", [1, 3])
+@pytest.mark.parametrize("smooth", [None, "same", "fp32"])
+def test_fused_decode_linear_strided_operands(dev, NK, M, smooth):
+    """Token rows and weight rows that are slices of wider buffers (row stride larger than K)."""
+    N, Kd = NK
+    kn = K()
+    xb = torch.randn(M, Kd + 64, generator=gen(221)).half().to(dev)
+    wb = _rand_i8((N, Kd + 128), 222).to(dev)
+    x, w = xb[:, :Kd], wb[:, :Kd]
+    assert x.stride(0) == Kd + 64 and w.stride(0) == Kd + 128
+    sm = None
+    if smooth is not None:
+        sm = (torch.rand(Kd, generator=gen(223)) * 3 + 0.2).to(torch.float16 if smooth == "same" else torch.float32).to(dev)
+    if not kn.decode_linear_ok(x, sm, Kd):
+        return
+    s_w = (torch.rand(N, generator=gen(224)) * 1e-3 + 1e-5).to(dev)
+    q, s = kn.quant_act_i8_pertoken(x.contiguous(), sm)
+    ref = kn.gemm_i8_dq(q, w.contiguous(), s, s_w, None, out_dtype=torch.float16, exact_ref=True)
+    y, s_f = kn.decode_linear_i8(x, w, s_w, None, sm, out_dtype=torch.float16, exact_ref=True)
+    assert torch.equal(s_f.view(torch.int32), s.view(torch.int32))
+    assert torch.equal(y.view(torch.int16), ref.view(torch.int16))
+
+
 @pytest.mark.parametrize("NK", [(4096, 4096), (520, 4096), (4096, 14336), (264, 12800)])
 @pytest.mark.parametrize("M", [1, 2, 3, 4])
 def test_fused_decode_linear_bf16_divisor_outside_the_fast_range(dev, NK, M):
