@@ -207,9 +207,9 @@ extern "C" int fmsmo_gemm_plan(int64_t M, int64_t N, int64_t K, int with_workspa
   }
   const SplitPlan plan = plan_split_k(M, N, K);
   if (with_workspace && plan.splits > 1) {
-    *kernel = FMSMO_PLAN_TILE_LDS_DMA;
-    *tile_m = TileMid::BM;
-    *tile_n = TileMid::BN;
+    *kernel = plan.rs ? FMSMO_PLAN_TILE_REGISTER_STAGED : FMSMO_PLAN_TILE_LDS_DMA;
+    *tile_m = plan.rs ? 256 : TileMid::BM;
+    *tile_n = plan.rs ? 128 : TileMid::BN;
     *splits = plan.splits;
     return FMSMO_OK;
   }

@@ -263,13 +263,32 @@ namespace {
 struct SplitPlan {
   int splits;
   int64_t k_len, ws_bytes;
+  bool rs;  // 256 x 128 tiles of the register-staged kernel instead of 128 x 128 LDS-DMA tiles
 };
 
 inline SplitPlan plan_split_k(int64_t M, int64_t N, int64_t K) {
-  SplitPlan p{1, K, 0};
+  SplitPlan p{1, K, 0, false};
   static const char* off = getenv("FMSMO_SPLIT_K");  // FMSMO_SPLIT_K=0 disables (tuning aid)
   if (off && off[0] == '0') return p;
   if (M <= 16 || M > 1024 || K % 128) return p;
+  // Long reductions under a few hundred rows: 256 x 128 tiles of the register-staged kernel carry
+  // the slices (us, 128 x 128 LDS-DMA tiles -> these, N = 4096, K = 14336: M = 384 51.4 -> 49.0,
+  // 512 54.6 -> 48.3, 768 84.7 -> 68.2, 1024 87.6 -> 77.8; at K = 4096 they lose, M = 512 25.5 ->
+  // 27.7, and below 384 rows their 256-row tiles are half empty)
+  if (K >= 8192 && M >= 384 && use_register_staged(0)) {
+    const int64_t t = (int64_t)div_up(M, 256) * div_up(N, 128);
+    if (t <= 128) {
+      int s = (int)(256 / t);
+      while (s > 1 && (K % (s * 128) != 0 || K / s < 512)) --s;
+      if (s >= 2) {
+        p.splits = s;
+        p.k_len = K / s;
+        p.ws_bytes = (int64_t)s * M * N * 4;
+        p.rs = true;
+        return p;
+      }
+    }
+  }
   const int64_t tiles = (int64_t)div_up(M, TileMid::BM) * div_up(N, TileMid::BN);
   if (tiles > 128) return p;
   int s = (int)(256 / tiles);  // one block per compute unit; 512 and 1024 blocks measured slower
@@ -322,8 +341,11 @@ int launch_split_k(const SplitPlan& p, const GemmArgs& g0, void* workspace, cons
   g.M = p.splits * g0.M;
   g.lda_e = p.k_len;
   g.ldb_e = p.k_len;
-  g.grid_m = p.splits * div_up(g0.M, TileMid::BM);
-  if constexpr (OP == MMA_I8) launch_tile<TileMid, OP, true>(g, EpiStoreI32{(int32_t*)workspace, g0.N}, st);
+  g.grid_m = p.splits * div_up(g0.M, p.rs ? 256 : TileMid::BM);
+  if (p.rs) {
+    if constexpr (OP == MMA_I8) launch_rs<OP, true, 128>(g, EpiStoreI32{(int32_t*)workspace, g0.N}, st);
+    else launch_rs<OP, true, 128>(g, EpiStoreF32{(float*)workspace, g0.N}, st);
+  } else if constexpr (OP == MMA_I8) launch_tile<TileMid, OP, true>(g, EpiStoreI32{(int32_t*)workspace, g0.N}, st);
   else launch_tile<TileMid, OP, true>(g, EpiStoreF32{(float*)workspace, g0.N}, st);
   if (!bias) bias_dtype = FMSMO_F32;
   dim3 grid(div_up(g0.N, 256), (unsigned)g0.M), block(256);

@@ -778,7 +778,9 @@ def _plain_i8_dq(a, w, a_s, w_s, bias, out_dtype, exact_ref):
 
 
 @pytest.mark.parametrize("shape", [(17, 4096, 14336), (64, 4096, 4096), (200, 1024, 1536), (512, 4096, 4096),
-                                   (100, 520, 2048), (128, 6144, 4096), (1000, 1024, 14336)])
+                                   (100, 520, 2048), (128, 6144, 4096), (1000, 1024, 14336),
+                                   # long reductions from 384 rows: register-staged 256 x 128 tiles
+                                   (384, 4096, 14336), (700, 1000, 8192), (1024, 4096, 14336), (513, 264, 12800)])
 @pytest.mark.parametrize("exact_ref,out_dtype", [(True, torch.float16), (False, torch.bfloat16), (False, torch.float32)])
 def test_split_k_int8_is_bit_identical_to_single_pass(dev, shape, exact_ref, out_dtype):
     from fms_mo_amd import _lib as L
@@ -804,7 +806,8 @@ def test_split_k_int8_is_bit_identical_to_single_pass(dev, shape, exact_ref, out
     torch.testing.assert_close(y[:5].cpu().double(), exact, rtol=1e-6, atol=1e-6)
 
 
-@pytest.mark.parametrize("shape", [(17, 4096, 14336), (64, 4096, 4096), (200, 1024, 1536), (100, 520, 2048)])
+@pytest.mark.parametrize("shape", [(17, 4096, 14336), (64, 4096, 4096), (200, 1024, 1536), (100, 520, 2048),
+                                   (512, 4096, 14336), (700, 1000, 8192)])
 def test_split_k_fp8(dev, shape):
     from fms_mo_amd import kernels as Kn
 

@@ -164,6 +164,12 @@ def test_gemm_plan_is_host_logic():
     k, tm, tn, s = K.gemm_plan(17, 4096, 14336, with_workspace=True)
     assert (k, tm, tn) == (DMA, 128, 128) and s >= 2 and 14336 % (s * 128) == 0
     assert K.gemm_plan(17, 4096, 14336, with_workspace=False)[3] == 1
+    # a few hundred rows through a long reduction: the slices run on register-staged 256 x 128 tiles
+    if not os.environ.get("FMSMO_RS"):
+        assert K.gemm_plan(512, 4096, 14336, with_workspace=True) == (RS, 256, 128, 4)
+        assert K.gemm_plan(1024, 4096, 14336, with_workspace=True) == (RS, 256, 128, 2)
+    assert K.gemm_plan(256, 4096, 14336, with_workspace=True)[:3] == (DMA, 128, 128)
+    assert K.gemm_plan(512, 4096, 4096, with_workspace=True)[:3] == (DMA, 128, 128)
     # K in 64-byte stages only: no register-staged kernel; K % 64 != 0: generic kernel
     assert K.gemm_plan(4096, 4096, 4160)[0] == DMA
     assert K.gemm_plan(300, 520, 1040) == (_lib.PLAN_GENERIC, 0, 0, 1)
