@@ -426,6 +426,27 @@ def extras(torch, K, dev, layers):
     sample_ops = sum(2.0 * 2048 * k * n for _, k, n in LLAMA3_8B)
     res["cpu_baseline_sample_on_gpu_M2048"] = {"ms": round(ms, 4), "tops": round(sample_ops / ms / 1e9, 1)}
     res["vendor"] = vendor_int_mm(torch, K, layers)
+    # batches of a few hundred rows (split-K territory) beside the vendor GEMM, launches replayed
+    # from a HIP graph, weights rotated over > 300 MB: this library's fused-dequant GEMM, its raw
+    # int32 GEMM and torch._int_mm (int32 out, no dequantization) on the same operands
+    for (name, k, n), L_ in ((LLAMA3_8B[1], layers[1]), (LLAMA3_8B[3], layers[3])):
+        copies = max(3, (300 * 1024 * 1024) // (k * n) + 1)
+        ws = [L_["w"]] + [torch.randint(-127, 128, (n, k), dtype=torch.int8, device=dev) for _ in range(copies - 1)]
+        for M in (128, 512, 1024):
+            q, sc = K.quant_act_i8_pertoken(L_["x"][:M], L_["smooth"])
+            row = {}
+            for label, fn in (("fmsmo_gemm_i8_dq", lambda w: K.gemm_i8_dq(q, w, sc, L_["w_scale"], L_["bias"],
+                                                                              out_dtype=torch.float16, exact_ref=True)),
+                              ("fmsmo_gemm_i8_i32", lambda w: K.gemm_i8_i32(q, w)),
+                              ("torch_int_mm", lambda w: torch._int_mm(q, w.t()))):
+                try:
+                    it = iter(range(10 ** 9))
+                    ms = graph_time(lambda: fn(ws[next(it) % copies]), reps=2 * copies, replays=5)
+                    row[label + "_us"] = round(ms * 1e3, 1)
+                except Exception as e:  # the vendor path is evidence, not a dependency
+                    row[label + "_us"] = str(e)[:120]
+            res[f"mid_batch_M{M}_{name}"] = row
+        del ws
     # batches between decode and the large GEMMs (decode kernels up to 64 tokens at K <= 4096,
     # tiled / split-K above), int8, same protocol as the decode rooflines
     mid = decode_rooflines(torch, K, dev, m_list=(32, 64, 128), ops=("i8",))

@@ -320,8 +320,9 @@ inline int launch_split_k_i32(const SplitPlan& p, const GemmArgs& g0, void* work
   g.M = p.splits * g0.M;
   g.lda_e = p.k_len;
   g.ldb_e = p.k_len;
-  g.grid_m = p.splits * div_up(g0.M, TileMid::BM);
-  launch_tile<TileMid, MMA_I8, true>(g, EpiStoreI32{(int32_t*)workspace, g0.N}, st);
+  g.grid_m = p.splits * div_up(g0.M, p.rs ? 256 : TileMid::BM);
+  if (p.rs) launch_rs<MMA_I8, true, 128>(g, EpiStoreI32{(int32_t*)workspace, g0.N}, st);
+  else launch_tile<TileMid, MMA_I8, true>(g, EpiStoreI32{(int32_t*)workspace, g0.N}, st);
   dim3 grid(div_up(g0.N, 256), (unsigned)g0.M), block(256);
   EpiStoreI32 epi{c, ldc};
   hipLaunchKernelGGL((splitk_reduce_kernel<int, EpiStoreI32>), grid, block, 0, st, (const int*)workspace,
