@@ -52,7 +52,7 @@ extern "C" int fmsmo_gemm_i8_i32_ws(const int8_t* a, int64_t lda, const int8_t* 
   g.a = (const uint8_t*)a; g.b = (const uint8_t*)b; g.lda = lda; g.ldb = ldb;
   g.M = (int)M; g.N = (int)N; g.K = (int)K;
   // few output tiles and a long reduction: K slices into the workspace, added in a fixed order
-  const SplitPlan plan = plan_split_k(M, N, K);
+  const SplitPlan plan = plan_split_k(M, N, K, workspace ? workspace_bytes : 0);
   if (plan.splits > 1 && workspace && workspace_bytes >= plan.ws_bytes && aligned16(workspace) &&
       plan.splits * M * lda < (1ll << 31))
     return launch_split_k_i32(plan, g, workspace, c, ldc, (hipStream_t)stream);
@@ -86,7 +86,7 @@ static int gemm_i8_dq_impl(const int8_t* a, int64_t lda, const int8_t* b, int64_
   g.a = (const uint8_t*)a; g.b = (const uint8_t*)b; g.lda = lda; g.ldb = ldb;
   g.M = (int)M; g.N = (int)N; g.K = (int)K;
   const int as = a_scale_n == 1 ? 0 : 1, ws = w_scale_n == 1 ? 0 : 1;
-  const SplitPlan plan = plan_split_k(M, N, K);
+  const SplitPlan plan = plan_split_k(M, N, K, workspace ? workspace_bytes : 0);
   if (plan.splits > 1 && workspace && workspace_bytes >= plan.ws_bytes && aligned16(workspace) &&
       plan.splits * M * lda < (1ll << 31)) {
     if (epilogue == FMSMO_EPI_REF_F16)
@@ -164,7 +164,8 @@ extern "C" int fmsmo_gemm_i8_dq_noalloc(const int8_t* a, int64_t lda, const int8
                                         int bias_dtype, int epilogue, void* y, int y_dtype,
                                         int64_t ldy, int64_t M, int64_t N, int64_t K,
                                         fmsmo_stream_t stream) {
-  const int64_t need = (M > 0 && N > 0 && K > 0) ? plan_split_k(M, N, K).ws_bytes : 0;
+  // (the plan that fits the scratch, if one does: else the preferred plan's size is reported)
+  int64_t need = (M > 0 && N > 0 && K > 0) ? plan_split_k(M, N, K, (int64_t)FMSMO_STATIC_SCRATCH_BYTES).ws_bytes : 0;
   if (need > (int64_t)FMSMO_STATIC_SCRATCH_BYTES) {
     snprintf(g_fmsmo_last_error, sizeof(g_fmsmo_last_error),
              "split-K partial sums of %lld x %lld x %lld need %lld bytes, the static scratch holds %lld",

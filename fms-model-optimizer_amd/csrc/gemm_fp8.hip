@@ -19,7 +19,7 @@ static int gemm_fp8_dq_impl(const uint8_t* a, int64_t lda, const uint8_t* b, int
   g.a = a; g.b = b; g.lda = lda; g.ldb = ldb;
   g.M = (int)M; g.N = (int)N; g.K = (int)K;
   const int as = a_scale_n == 1 ? 0 : 1, ws = w_scale_n == 1 ? 0 : 1;
-  const SplitPlan plan = plan_split_k(M, N, K);
+  const SplitPlan plan = plan_split_k(M, N, K, workspace ? workspace_bytes : 0);
   if (plan.splits > 1 && workspace && workspace_bytes >= plan.ws_bytes && aligned16(workspace) &&
       plan.splits * M * lda < (1ll << 31))
     return launch_split_k<MMA_FP8, false, float>(plan, g, workspace, a_scale, as, w_scale, ws, bias,

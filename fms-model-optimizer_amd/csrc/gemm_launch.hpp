@@ -266,7 +266,9 @@ struct SplitPlan {
   bool rs;  // 256 x 128 tiles of the register-staged kernel instead of 128 x 128 LDS-DMA tiles
 };
 
-inline SplitPlan plan_split_k(int64_t M, int64_t N, int64_t K) {
+// `limit` > 0: the workspace at hand; a plan that needs more is passed over for the next one (the
+// register-staged slices need more partial sums than the 128 x 128 ones: more, shorter slices).
+inline SplitPlan plan_split_k(int64_t M, int64_t N, int64_t K, int64_t limit = 0) {
   SplitPlan p{1, K, 0, false};
   static const char* off = getenv("FMSMO_SPLIT_K");  // FMSMO_SPLIT_K=0 disables (tuning aid)
   if (off && off[0] == '0') return p;
@@ -280,7 +282,7 @@ inline SplitPlan plan_split_k(int64_t M, int64_t N, int64_t K) {
     if (t <= 128) {
       int s = (int)(256 / t);
       while (s > 1 && (K % (s * 128) != 0 || K / s < 512)) --s;
-      if (s >= 2) {
+      if (s >= 2 && (limit <= 0 || (int64_t)s * M * N * 4 <= limit)) {
         p.splits = s;
         p.k_len = K / s;
         p.ws_bytes = (int64_t)s * M * N * 4;

@@ -296,8 +296,11 @@ int fmsmo_gemm_fp8_dq(const uint8_t* a, int64_t lda, const uint8_t* b, int64_t l
  * slices in a fixed order and applies the epilogue: 17 x 4096 x 14336 runs on 256 compute units
  * instead of 32.  int32 partial sums are exact, so the int8 result is bit-identical to
  * fmsmo_gemm_i8_dq's; the e4m3 result differs from fmsmo_gemm_fp8_dq's only by the order of the
- * fp32 additions.  fmsmo_gemm_workspace_bytes returns the bytes a shape can use (0: no split);
- * with workspace == NULL or fewer bytes the call is fmsmo_gemm_*_dq.  workspace: 16-byte aligned
+ * fp32 additions.  From 384 rows and K >= 8192 the slices run on 256 x 128 tiles of the
+ * register-staged kernel (more, shorter slices: more partial sums).  fmsmo_gemm_workspace_bytes
+ * returns the bytes a shape can use at most (0: no split); with fewer bytes the call takes the
+ * split that fits them (the 128 x 128 tiles' never needs more than 16 MiB), with none or
+ * workspace == NULL it is fmsmo_gemm_*_dq.  workspace: 16-byte aligned
  * device memory, contents undefined before and after, private to the call while it runs.
  * No counterpart in the reference (its GEMMs are single launches of CUTLASS / cuBLASLt kernels).
  */
@@ -346,10 +349,12 @@ int fmsmo_gemm_fp8_dq_ws(const uint8_t* a, int64_t lda, const uint8_t* b, int64_
  * no hipMalloc / hipFree and uses no allocating library routine; the caller still passes inputs
  * and outputs.  Results are bit-identical to fmsmo_gemm_i8_dq_ws given a sufficient workspace
  * (and so to fmsmo_gemm_i8_dq).
- * A shape whose partial sums would not fit returns FMSMO_ERR_SCRATCH (fmsmo_last_error() says
- * how many bytes it needs); under the current split policy (16 < M <= 1024, at most 128 tiles of
- * 128 x 128, up to 256 / tiles slices) the need never exceeds the buffer, so the check guards
- * changes of that policy.  Shapes that take no split use no scratch at all.
+ * The call takes the split that fits the array: where the preferred one (register-staged slices
+ * of a long reduction) needs more, the 128 x 128 tiles' split, whose need never exceeds the array
+ * under the current policy (16 < M <= 1024, at most 128 such tiles, up to 256 / tiles slices).
+ * A shape none of whose splits would fit returns FMSMO_ERR_SCRATCH (fmsmo_last_error() says how
+ * many bytes it needs): the check guards changes of that policy.  Shapes that take no split use
+ * no scratch at all.
  * All calls on one GPU share that GPU's array: two calls that overlap in time on the same GPU
  * (different streams, different threads) race on it; calls on one stream are ordered and safe.
  * Nothing in the array has to be cleared between calls (every slice stores its whole block of

@@ -63,6 +63,34 @@ def test_noalloc_entry_point_matches_workspace_entry_point(dev):
     assert seen_split >= 3
 
 
+def test_noalloc_entry_point_takes_the_plan_that_fits(dev):
+    """512 x 4096 x 14336: the preferred plan (four slices on register-staged tiles) needs 32 MiB of
+    partial sums; the static array holds 16 MiB, which two slices on 128 x 128 tiles fit exactly.
+    Same bits as with a caller's workspace of either size, and as the single pass."""
+    from fms_mo_amd import _lib as L
+
+    lib = L.load()
+    M, N, K = 512, 4096, 14336
+    need = lib.fmsmo_gemm_workspace_bytes(M, N, K)
+    assert need == 32 << 20
+    ops = _operands(M, N, K, 300, dev, torch.float16)
+    y_big = _run("fmsmo_gemm_i8_dq_ws", ops, M, N, K, 0, torch.float16, torch.empty(need, dtype=torch.uint8, device=dev))
+    y_small = _run("fmsmo_gemm_i8_dq_ws", ops, M, N, K, 0, torch.float16,
+                   torch.empty(16 << 20, dtype=torch.uint8, device=dev))
+    y_none = _run("fmsmo_gemm_i8_dq", ops, M, N, K, 0, torch.float16)
+    y = _run("fmsmo_gemm_i8_dq_noalloc", ops, M, N, K, 0, torch.float16)
+    torch.cuda.synchronize()
+    for other in (y_big, y_small, y_none):
+        assert torch.equal(y.view(torch.int16), other.view(torch.int16))
+    # 1024 rows: the preferred plan needs 32 MiB and the 128 x 128 tiles do not split (256 tiles):
+    # the call runs the single pass
+    ops = _operands(1024, N, K, 301, dev, None)
+    y_none = _run("fmsmo_gemm_i8_dq", ops, 1024, N, K, 0, torch.float16)
+    y = _run("fmsmo_gemm_i8_dq_noalloc", ops, 1024, N, K, 0, torch.float16)
+    torch.cuda.synchronize()
+    assert torch.equal(y.view(torch.int16), y_none.view(torch.int16))
+
+
 def test_noalloc_entry_point_allocates_nothing_and_repeats(dev):
     """Two calls in a row, the second smaller, with no device allocation in between (torch's
     allocator statistics do not move and the driver reports the same free memory), and the
