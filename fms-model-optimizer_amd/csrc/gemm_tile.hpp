@@ -872,7 +872,7 @@ struct EpiDequant {
     Col c;
     const int64_t o = (int64_t)expert * N + n;
     c.ws = w_scale[w_stride ? o : 0];
-    c.b = bias ? load_as_f32<BIAS>(bias, o) : 0.0f;
+    c.b = bias ? load_as_f32<BIAS>(bias, o) : -0.0f;  // no bias: x + (-0) == x, the sign of a zero product included
     return c;
   }
   __device__ __forceinline__ Row row(int m) const { return Row{a_scale[a_stride ? m : 0]}; }
@@ -913,7 +913,7 @@ struct EpiScaleBias {
     float sc;
   };
   __device__ __forceinline__ Col col(int n, int expert, int N) const {
-    return Col{bias ? bias[(int64_t)expert * N + n] : 0.0f};
+    return Col{bias ? bias[(int64_t)expert * N + n] : -0.0f};
   }
   __device__ __forceinline__ Row row(int) const { return Row{__fmul_rn(a_scale[0], w_scale[0])}; }
   __device__ __forceinline__ float value(AccT v, Row r, Col c) const { return __fmaf_rn((float)v, r.sc, c.b); }

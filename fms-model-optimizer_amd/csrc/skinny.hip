@@ -634,7 +634,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_kernel(GemvArgs g) {
     const int n = n0 + i * 16 + (e >> 4), m = e & 15;
     if (n < g.N && m < g.M) {
       const float as = g.a_scale ? g.a_scale[g.a_stride ? m : 0] : 1.f, ws = g.w_scale ? g.w_scale[g.w_stride ? n : 0] : 1.f;
-      float b = 0.f;
+      float b = -0.f;  // no bias: adding -0 changes nothing, not even the sign of a zero product
       if (g.bias) {
         b = g.bias_dtype == FMSMO_F16 ? f16_to_f32(((const u16*)g.bias)[n])
             : g.bias_dtype == FMSMO_BF16 ? bf16_to_f32(((const u16*)g.bias)[n])
@@ -814,7 +814,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_stream_kernel(GemvArgs g, int ha
     constexpr bool LAST = decltype(last_tag)::value;
     const int en = min(row_lo + gi * 16 + (int)((threadIdx.x >> 4) & 15), g.N - 1);
     const float ws = g.w_scale ? g.w_scale[g.w_stride ? en : 0] : 1.f;
-    float bv = 0.f;
+    float bv = -0.f;  // no bias: adding -0 changes nothing, not even the sign of a zero product
     if (g.bias) {
       bv = g.bias_dtype == FMSMO_F16 ? f16_to_f32(((const u16*)g.bias)[en])
            : g.bias_dtype == FMSMO_BF16 ? bf16_to_f32(((const u16*)g.bias)[en])
@@ -1058,7 +1058,7 @@ __global__ __launch_bounds__(256) void gemv_rows_kernel(GemvArgs g) {
     const int n = n0 + eu;
     if ((lane & (SHARE - 1)) == 0 && n < g.N && em < g.M) {
       const float as = g.a_scale ? g.a_scale[g.a_stride ? em : 0] : 1.f, ws = g.w_scale ? g.w_scale[g.w_stride ? n : 0] : 1.f;
-      float bv = 0.f;
+      float bv = -0.f;  // no bias: adding -0 changes nothing, not even the sign of a zero product
       if (g.bias) {
         bv = g.bias_dtype == FMSMO_F16 ? f16_to_f32(((const u16*)g.bias)[n])
              : g.bias_dtype == FMSMO_BF16 ? bf16_to_f32(((const u16*)g.bias)[n])

@@ -265,7 +265,9 @@ int fmsmo_gemm_i8_i32_ws(const int8_t* a, int64_t lda, const int8_t* b, int64_t 
 /*
  * int8 GEMM with the dequantizing epilogue fused:  y = acc * (a_scale x w_scale) + bias.
  * a_scale: fp32 [M] (a_scale_n == M) or one value (a_scale_n == 1); w_scale likewise [N] or 1;
- * bias: [N] of bias_dtype or NULL.  epilogue: FMSMO_EPI_REF_F16 | FMSMO_EPI_F32.
+ * bias: [N] of bias_dtype or NULL (nothing is added then: a zero product keeps its sign, as with
+ * the -0.0 bias buffer the reference's module holds for a layer without bias, linear.py:897-911).
+ * epilogue: FMSMO_EPI_REF_F16 | FMSMO_EPI_F32.
  * M <= 16 is routed to the weight-streaming (HBM-bound) kernel, and so are 17 <= M <= 64 when
  * K is 1024, 2048 or 4096 (5120 and 8192 up to M = 32).
  * Reference: QLinearINT8Deploy.iaddmm_int, plain branch (fms_mo/modules/linear.py:1177-1188),

@@ -505,6 +505,52 @@ def test_decode_long_rows(dev, M, NKd):
     assert torch.equal(y8.cpu(), a8 @ w8.t())
 
 
+def test_decode_range_random_shapes(dev):
+    """Sixty seeded shapes with 1..64 tokens: whichever decode kernel serves a shape (row kernel,
+    streaming kernel in any of its instantiations, generic kernel, K slices), the int32 sums are
+    the exact product, the reference epilogue gives the oracle's bits, e4m3 is exact on small
+    integers, and the fused linear (where it serves the shape) equals quantizer + matmul."""
+    import random
+
+    rng = random.Random(4321)
+    kn = K()
+    for case in range(60):
+        M = rng.choice([1, 2, 3, 4, rng.randint(5, 16), rng.randint(17, 32), rng.randint(33, 64)])
+        N = rng.choice([rng.randint(1, 64), rng.randint(65, 3000), 8 * rng.randint(1, 800), 16 * rng.randint(1, 400)])
+        Kd = rng.choice([16 * rng.randint(1, 64), 128 * rng.randint(1, 128),
+                         1024 * rng.choice([1, 2, 4, 5, 8, 11, 13, 14, 16]), 12800, 14336])
+        tag = f"case {case}: M={M} N={N} K={Kd}"
+        g = torch.Generator(device=dev).manual_seed(500 + case)
+        a = torch.randint(-128, 128, (M, Kd), generator=g, dtype=torch.int8, device=dev)
+        w = torch.randint(-128, 128, (N, Kd), generator=g, dtype=torch.int8, device=dev)
+        acc = (a.double() @ w.double().t()).to(torch.int32)
+        assert torch.equal(kn.gemm_i8_i32(a, w), acc), tag
+        s_a = (torch.rand(M, 1, generator=gen(600 + case)) * 0.05 + 1e-3).half()
+        s_w = (torch.rand(N, generator=gen(700 + case)) * 1e-3 + 1e-5).float()
+        bias = (torch.randn(N, generator=gen(800 + case)) * 0.01).half() if case % 3 else None
+        ref = O.epilogue_ref(acc.cpu(), s_a, s_w, bias, torch.float16)
+        y = kn.gemm_i8_dq(a, w, s_a.float().to(dev), s_w.to(dev), None if bias is None else bias.to(dev),
+                          out_dtype=torch.float16, exact_ref=True)
+        assert torch.equal(y.cpu().view(torch.int16), ref.view(torch.int16)), tag
+        a8 = torch.randint(-3, 4, (M, Kd), generator=g, device=dev).float()
+        w8 = torch.randint(-3, 4, (N, Kd), generator=g, device=dev).float()
+        one = torch.ones(1, device=dev)
+        y8 = kn.gemm_fp8_dq(a8.to(torch.float8_e4m3fn), w8.to(torch.float8_e4m3fn), one, one, None,
+                            out_dtype=torch.float32)
+        assert torch.equal(y8, a8 @ w8.t()), tag
+        if M <= 4:
+            dt = torch.float16 if case % 2 else torch.bfloat16
+            x = (torch.randn(M, Kd, generator=gen(900 + case)) * 2).to(dt).to(dev)
+            sm = (torch.rand(Kd, generator=gen(1000 + case)) * 3 + 0.2).to(dt).to(dev) if case % 4 < 2 else None
+            if kn.decode_linear_ok(x, sm, Kd):
+                b16 = None if bias is None else bias.to(dt).to(dev)
+                q, s = kn.quant_act_i8_pertoken(x, sm)
+                r2 = kn.gemm_i8_dq(q, w, s, s_w.to(dev), b16, out_dtype=dt, exact_ref=False)
+                y2, s2 = kn.decode_linear_i8(x, w, s_w.to(dev), b16, sm, out_dtype=dt, exact_ref=False)
+                assert torch.equal(s2.view(torch.int32), s.view(torch.int32)), tag
+                assert torch.equal(y2.view(torch.int16), r2.view(torch.int16)), tag
+
+
 def _rand_fp8(shape, seed, scale=1.0):
     return (torch.randn(shape, generator=gen(seed)) * scale).clamp(-448, 448).to(torch.float8_e4m3fn)
 
@@ -548,9 +594,10 @@ def test_gemm_dq_with_columns_cut_off_the_last_round(dev, bias_dt):
     and 32 tiles more, so the library runs the last 1024 columns as a second, small GEMM.
     Per-column scales, bias (every dtype) and output of both parts must line up: int8 bit-exact
     against the reference epilogue (fp16 and fp32 accumulator dtype) and the fp32 forms, e4m3 exact
-    on small integers with per-column scales that are powers of two.  Without a bias the kernel adds
-    0.0 like the reference, whose deploy module always holds a bias buffer (linear.py:897-911): a
-    product of -0.0 comes out as +0.0."""
+    on small integers with per-column scales that are powers of two.  Without a bias nothing is
+    added: a product of -0.0 (a scale product that underflows in fp16, a negative sum) stays -0.0,
+    as in the reference, whose deploy module then holds -corr_term = -0.0 as its bias buffer
+    (linear.py:897-911)."""
     from fms_mo_amd import _lib as L
 
     M, N, Kd = 2048, 25600, 128
@@ -561,7 +608,7 @@ def test_gemm_dq_with_columns_cut_off_the_last_round(dev, bias_dt):
     s_a = (torch.rand(M, 1, generator=gen(53)) * 0.05 + 1e-3).half()
     s_w = (torch.rand(N, generator=gen(54)) * 1e-3 + 1e-5).float()
     bias = None if bias_dt is None else (torch.randn(N, generator=gen(55)) * 0.01).to(bias_dt)
-    bz = torch.zeros(N) if bias is None else bias
+    bz = torch.full((N,), -0.0) if bias is None else bias
     acc = O.int_gemm(a, w)
     ad, wd, sad, swd = a.to(dev), w.to(dev), s_a.float().to(dev), s_w.to(dev)
     bd = None if bias is None else bias.to(dev)
@@ -847,10 +894,10 @@ def test_batched_decode_i8_bit_exact(dev, M, NK):
     y = K().gemm_i8_dq(a.to(dev), w.to(dev), s_a.float().to(dev), s_w.to(dev), bias.to(dev),
                        out_dtype=torch.float16, exact_ref=True)
     assert torch.equal(y.cpu().view(torch.int16), ref.view(torch.int16))
-    # without a bias the kernels add +0.0 (the reference always adds a bias tensor): equal as values
+    # without a bias nothing is added: the same bits, the sign of a zero product included
     y = K().gemm_i8_dq(a.to(dev), w.to(dev), s_a.float().to(dev), s_w.to(dev), None,
                        out_dtype=torch.float16, exact_ref=True)
-    assert torch.equal(y.cpu(), O.epilogue_ref(acc, s_a, s_w, None, torch.float16))
+    assert torch.equal(y.cpu().view(torch.int16), O.epilogue_ref(acc, s_a, s_w, None, torch.float16).view(torch.int16))
     y32 = K().gemm_i8_dq(a.to(dev), w.to(dev), torch.ones(1, device=dev), torch.ones(1, device=dev), None,
                          out_dtype=torch.float32, exact_ref=False)
     assert torch.equal(y32.cpu().double(), acc.double())
