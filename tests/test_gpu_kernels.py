@@ -308,6 +308,49 @@ def test_quant_act_fp8_fpxacc(dev, dtype, dl8):
     assert torch.equal(q.cpu().view(torch.uint8), q_ref.view(torch.uint8))
 
 
+def test_quantizers_random_shapes_dtypes_and_magnitudes(dev):
+    """Eighty seeded cases over row counts, row lengths (any multiple of 8), dtypes, divisor
+    dtypes and magnitudes from 1e-3 to 1e3: whichever quantizer kernel serves a case (packed
+    16-bit row walker in any chunk count, fp32-divisor walker, generic one-row-per-block), codes
+    and scales are the oracle's, for the int8, the e4m3 and the static int8 quantizers."""
+    import random
+
+    from fms_mo_amd import _lib as L
+
+    rng = random.Random(2468)
+    kn = K()
+    for case in range(80):
+        M = rng.choice([rng.randint(1, 8), rng.randint(9, 300), rng.randint(300, 3000)])
+        Kd = 8 * rng.choice([rng.randint(1, 64), rng.randint(64, 1024), rng.randint(1024, 4200)])
+        if M > 300:
+            Kd = min(Kd, 8 * 640)
+        dt = rng.choice([torch.float16, torch.bfloat16, torch.float32])
+        mag = 10.0 ** rng.uniform(-3, 3 if dt != torch.float16 else 2)
+        tag = f"case {case}: M={M} K={Kd} {dt} mag={mag:.3g}"
+        g = gen(3000 + case)
+        x = (torch.randn(M, Kd, generator=g) * mag).to(dt)
+        if M >= 3:
+            x = _special_rows(x)
+        kind = rng.choice(["none", "same", "f32"])
+        sm = None
+        if kind != "none":
+            sm = (torch.rand(Kd, generator=g) * 3 + 0.1).to(dt if kind == "same" else torch.float32)
+        q_ref, s_ref, _ = O.quant_act_pertoken_i8(x, None if sm is None else sm.reshape(1, -1))
+        q, s = kn.quant_act_i8_pertoken(x.to(dev), None if sm is None else sm.to(dev))
+        assert torch.equal(s.cpu(), s_ref.float().reshape(-1)), tag + f" smooth={kind}"
+        assert torch.equal(q.cpu(), q_ref), tag + f" smooth={kind}"
+        s8_ref = O.fp8_dynamic_scale(x)
+        q8_ref = O.fp8_quant_static(x, s8_ref)
+        q8, s8 = kn.quant_act_fp8_pertoken(x.to(dev), L.FP8_LINEAR)
+        assert torch.equal(s8.cpu(), s8_ref.reshape(-1)), tag
+        assert torch.equal(q8.cpu().view(torch.uint8), q8_ref.view(torch.uint8)), tag
+        scale = mag * rng.uniform(0.01, 0.05)
+        zp, sym = rng.choice([(128, 1), (rng.randint(100, 156), 0)])
+        qs_ref = O.quant_act_static_raw(x, torch.tensor([scale]), zp, sym)
+        qs = kn.quant_act_i8_static(x.to(dev), scale, zp, sym)
+        assert torch.equal(qs.cpu(), qs_ref), tag + f" static scale={scale:.4g} zp={zp} sym={sym}"
+
+
 # ---------------------------------------------------------------------------------- int8 GEMM
 def _rand_i8(shape, seed):
     return torch.randint(-128, 128, shape, generator=gen(seed), dtype=torch.int8)
@@ -393,6 +436,50 @@ def test_gemm_i8_i32_random_shapes_cover_every_kernel_choice(dev):
     # the sample reaches the generic kernel, both MFMA pipelines and all five tile shapes
     assert {p[0] for p in seen} >= {1, 2, 3}
     assert {p[1:] for p in seen if p[0] in (1, 2)} >= {(256, 256), (256, 192), (256, 128), (128, 256), (128, 128)}
+
+
+def test_gemm_i8_dq_random_shapes_scales_and_epilogues(dev):
+    """Thirty seeded shapes from 17 rows up: per-row or single activation scale, per-column or
+    single weight scale, bias of any dtype or none, 16-bit and fp32 outputs, the reference epilogue
+    (bit-exact against the oracle) and both fp32-scale forms."""
+    import random
+
+    from fms_mo_amd import _lib as L
+
+    rng = random.Random(9753)
+    kn = K()
+    for case in range(30):
+        M = rng.choice([rng.randint(17, 300), rng.randint(300, 2100), rng.randint(2100, 4500)])
+        N = rng.choice([rng.randint(8, 300), rng.randint(300, 2100), rng.randint(2100, 6200)])
+        Kd = rng.choice([16 * rng.randint(1, 40), 64 * rng.randint(1, 24), 128 * rng.randint(1, 40)])
+        g = torch.Generator(device=dev).manual_seed(4000 + case)
+        a = torch.randint(-128, 128, (M, Kd), generator=g, dtype=torch.int8, device=dev)
+        w = torch.randint(-128, 128, (N, Kd), generator=g, dtype=torch.int8, device=dev)
+        acc = (a.double() @ w.double().t()).to(torch.int32).cpu()
+        an, wn = rng.choice([1, M]), rng.choice([1, N])
+        s_a = (torch.rand(an, 1, generator=gen(4100 + case)) * 0.05 + 1e-3).half()
+        s_w = (torch.rand(wn, generator=gen(4200 + case)) * 1e-2 + 1e-4).float()
+        bdt = rng.choice([None, torch.float16, torch.bfloat16, torch.float32])
+        bias = None if bdt is None else (torch.randn(N, generator=gen(4300 + case)) * 0.1).to(bdt)
+        bd = None if bias is None else bias.to(dev)
+        odt = rng.choice([torch.float16, torch.bfloat16, torch.float32])
+        tag = f"case {case}: M={M} N={N} K={Kd} a_scales={an} w_scales={wn} bias={bdt} out={odt} plan={kn.gemm_plan(M, N, Kd)}"
+        sad, swd = s_a.float().reshape(-1).to(dev), s_w.to(dev)
+        acc_dt = torch.float32 if odt == torch.float32 else torch.float16
+        ref = O.epilogue_ref(acc, s_a, s_w, bias, odt, acc_dtype=acc_dt)
+        y = kn.gemm_i8_dq(a, w, sad, swd, bd, out_dtype=odt, exact_ref=True).cpu()
+        bits = torch.int32 if odt == torch.float32 else torch.int16
+        assert torch.equal(y.view(bits), ref.view(bits)), tag
+        ref2 = O.epilogue_f32(acc, s_a, s_w, bias, odt)
+        y2 = kn.gemm_i8_dq(a, w, sad, swd, bd, out_dtype=odt, exact_ref=False).cpu()
+        # (the oracle's fma is emulated in float64: a rare double rounding may differ by one ulp)
+        torch.testing.assert_close(y2.float(), ref2.float(), rtol=1e-2, atol=1e-2, msg=tag + " fp32-scale fma")
+        assert (y2.view(bits) != ref2.view(bits)).float().mean().item() < 1e-5, tag + " fp32-scale fma"
+        ref3 = (acc.float() * (s_a.float() * s_w.float()))
+        if bias is not None:
+            ref3 = ref3 + bias.float()
+        y3 = kn.gemm_i8_dq(a, w, sad, swd, bd, out_dtype=odt, epilogue=L.EPI_F32_MULADD).cpu()
+        assert torch.equal(y3.view(bits), ref3.to(odt).view(bits)), tag + " fp32-scale mul+add"
 
 
 def test_gemm_i8_i32_strided_rows(dev):
@@ -651,6 +738,30 @@ def test_chunk_i8_bit_exact(dev, cfg, shape):
     assert torch.equal(d.cpu(), ref)
 
 
+def test_chunk_i8_random_shapes_and_settings(dev):
+    """Twenty-five seeded cases: any M and N, K a multiple of 16 (ragged last chunk included),
+    every chunk size, truncation from 0 to 12 bits, accumulator widths from 14 to 32 bits, both
+    orders of truncation and accumulation, with and without an initial accumulator."""
+    import random
+
+    rng = random.Random(1357)
+    for case in range(25):
+        M, N = rng.randint(1, 300), rng.randint(1, 300)
+        Kd = 16 * rng.randint(2, 200)
+        cfg = dict(chunk_size=rng.choice([32, 64, 128, 256]), chunk_trun_bits=rng.randint(0, 12),
+                   max_acc_bits=rng.choice([14, 16, 18, 20, 24, 32]),
+                   truncate_then_accumulate=rng.random() < 0.7)
+        g = gen(5000 + case)
+        a = torch.randint(-128, 128, (M, Kd), generator=g, dtype=torch.int8)
+        w = torch.randint(-128, 128, (N, Kd), generator=g, dtype=torch.int8)
+        c = torch.randint(-10**6, 10**6, (M, N), generator=g, dtype=torch.int32) if case % 3 == 0 else None
+        ocfg = dict(cfg)
+        ocfg["trun_bits"] = ocfg.pop("chunk_trun_bits")
+        ref = O.chunk_matmul_i8(a, w, c, **ocfg)
+        d = K().matmul_chunk(a.to(dev), w.to(dev), None if c is None else c.to(dev), **cfg)
+        assert torch.equal(d.cpu(), ref), f"case {case}: M={M} N={N} K={Kd} {cfg} c={'yes' if c is not None else 'no'}"
+
+
 def test_chunk_i8_initial_accumulator(dev):
     a, w = _rand_i8((100, 512), 53), _rand_i8((90, 512), 54)
     c = torch.randint(-10**6, 10**6, (100, 90), generator=gen(55), dtype=torch.int32)
@@ -770,6 +881,41 @@ def test_grouped_gemm_row_remainders(dev, counts, NK, exact_ref, out_dtype):
             # (the oracle takes the token scales in fp16, the kernel in fp32: compare where equal)
             same = s_a[lo:hi].half().float() == s_a[lo:hi]
             assert torch.equal(y[lo:hi][same].view(bits), want[same].view(bits))
+
+
+def test_grouped_gemm_random_expert_splits(dev):
+    """Twelve seeded cases: 1 to 12 experts, a random split of the rows (empty experts included),
+    any N, K in whole 128-byte slabs and not, per-expert bias or none: every expert's rows equal
+    the plain GEMM on that expert's rows and weights, bit for bit."""
+    import random
+
+    rng = random.Random(8642)
+    for case in range(12):
+        E = rng.randint(1, 12)
+        counts = [rng.choice([0, rng.randint(1, 40), rng.randint(40, 700)]) for _ in range(E)]
+        if sum(counts) == 0:
+            counts[0] = 33
+        N = rng.choice([rng.randint(8, 200), rng.randint(200, 1500)])
+        Kd = rng.choice([64 * rng.randint(1, 30), 128 * rng.randint(1, 24)])
+        exact_ref = case % 2 == 0
+        out_dtype = torch.float16 if exact_ref else rng.choice([torch.float32, torch.bfloat16])
+        offsets = torch.zeros(E + 1, dtype=torch.int32)
+        offsets[1:] = torch.tensor(counts).cumsum(0)
+        T = int(offsets[-1])
+        a = _rand_i8((T, Kd), 6000 + case).to(dev)
+        w = _rand_i8((E, N, Kd), 6100 + case).to(dev)
+        s_a = (torch.rand(T, generator=gen(6200 + case)) * 0.05 + 1e-3).float().to(dev)
+        s_w = (torch.rand(E, N, generator=gen(6300 + case)) * 1e-3 + 1e-5).float().to(dev)
+        bias = (torch.randn(E, N, generator=gen(6400 + case)) * 0.01).half().to(dev) if case % 3 else None
+        y = K().grouped_gemm_i8_dq(a, w, offsets.to(dev), s_a, s_w, bias, out_dtype=out_dtype, exact_ref=exact_ref)
+        bits = torch.int32 if out_dtype == torch.float32 else torch.int16
+        for e in range(E):
+            lo, hi = int(offsets[e]), int(offsets[e + 1])
+            if hi == lo:
+                continue
+            ref = K().gemm_i8_dq(a[lo:hi], w[e], s_a[lo:hi], s_w[e], None if bias is None else bias[e],
+                                 out_dtype=out_dtype, exact_ref=exact_ref)
+            assert torch.equal(y[lo:hi].view(bits), ref.view(bits)), f"case {case}: counts={counts} N={N} K={Kd} expert {e}"
 
 
 # ------------------------------------------------------------------------------ error behaviour

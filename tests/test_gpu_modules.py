@@ -67,6 +67,38 @@ def test_deploy_module_bit_exact_vs_oracle(dev, smoothq, shape):
     assert torch.equal(y.cpu().view(torch.int16), ref["y"].view(torch.int16))
 
 
+def test_deploy_module_random_layers_bit_exact_vs_oracle(dev):
+    """Fourteen seeded layers: any batch shape from one token to a few hundred, K and N off the
+    tile sizes, with and without bias, with and without SmoothQuant: buffers, input scales and
+    outputs are the oracle's, bit for bit (a layer without bias keeps the sign of a zero output)."""
+    import random
+
+    from fms_mo_amd.modules.linear import QLinearINT8Deploy
+
+    rng = random.Random(7531)
+    for case in range(14):
+        B, S = rng.choice([(1, 1), (1, rng.randint(2, 16)), (rng.randint(2, 4), rng.randint(1, 90))])
+        K = rng.choice([64 * rng.randint(1, 40), 128 * rng.randint(1, 40), 1024 * rng.choice([1, 2, 4])])
+        N = rng.choice([8 * rng.randint(1, 100), rng.randint(10, 1200)])
+        smoothq, bias = rng.random() < 0.5, rng.random() < 0.6
+        tag = f"case {case}: B={B} S={S} K={K} N={N} smoothq={smoothq} bias={bias}"
+        m = make_qlinear(None, K, N, smoothq=smoothq, bias=bias, seed=case)
+        x = outlier_x(B * S, K, 7000 + case).reshape(B, S, K)
+        act_scale = None
+        if smoothq:
+            act_scale = x.reshape(-1, K).float().abs().amax(dim=0)
+            m.set_act_scale(act_scale)
+        dep = QLinearINT8Deploy.from_fms_mo(m, use_int_kernel="cutlass", use_dynamic_max_act_Qfunc=-1,
+                                            recalc_clipvals=False, target_device=dev)
+        y = dep(x.to(dev))
+        bufs = O.deploy_prepare(m.weight.detach(), m.bias.detach() if bias else None,
+                                m.quantize_weight.clip_val, act_scale, 0.5)
+        ref = O.deploy_forward(x, bufs)
+        assert torch.equal(dep.weight.cpu(), bufs["weight"]) and torch.equal(dep.w_scale.cpu(), bufs["w_scale"]), tag
+        assert torch.equal(dep.input_scale.cpu().reshape(-1), ref["input_scale"].float().reshape(-1)), tag
+        assert torch.equal(y.cpu().view(torch.int16), ref["y"].view(torch.int16)), tag
+
+
 def test_deploy_module_converted_on_gpu_matches_within_tolerance(dev):
     """Converting on the GPU uses the GPU's pow / division roundings for the offline scales, so it
     is only tolerance-equal to the CPU-converted module."""
