@@ -191,6 +191,42 @@ def test_op_against_oracle(dev, act, per_channel, xdt, mdt, smooth, shape):
     assert torch.all((y.cpu().float() - sim.float()).abs() <= 1e-2 * sim.float().abs() + 1e-2 * scale)
 
 
+def test_random_nodes_codes_bit_exact_and_outputs_within_an_ulp(dev):
+    """Forty seeded nodes over all three activation modes, both weight modes, the dtype pairs the
+    op serves, any M, K a multiple of 64 and any N a multiple of 8: the integer activation codes
+    are the oracle's and the output is the exact value of those integers within the output cast."""
+    import random
+
+    from fms_mo_amd import _lib as L
+    from fms_mo_amd import kernels
+
+    rng = random.Random(97531)
+    for case in range(40):
+        act = rng.choice(MODES)
+        per_channel, smooth = rng.random() < 0.5, rng.random() < 0.5
+        xdt, mdt = rng.choice([(torch.float16, torch.float16), (torch.bfloat16, torch.bfloat16),
+                               (torch.float16, torch.float32)])
+        M = rng.choice([1, rng.randint(2, 16), rng.randint(17, 400)])
+        K = 64 * rng.choice([rng.randint(1, 16), rng.randint(16, 230)])
+        N = 8 * rng.randint(1, 150)
+        tag = f"case {case}: {act} per_channel={per_channel} smooth={smooth} {xdt}/{mdt} M={M} K={K} N={N}"
+        x, w_int, bias, qdata, w_cv, a_cv, a_cvn, sq = make_case(8000 + case, M, K, N, xdt, mdt, per_channel,
+                                                                 act, smooth)
+        ref_int, scale_x, zp_x = O.i8i8_aiu_quant_act(x, a_cv, a_cvn, sq, act)
+        mode = {"per_token": L.MS_PER_TOKEN, "per_tensor_symm": L.MS_SYMM, "per_tensor_asymm": L.MS_ASYMM}[act]
+        clip = None if act == "per_token" else torch.cat((a_cv, a_cvn)).to(dev)
+        q, _ = kernels.quant_act_i8_mulscale(x.to(dev), mode, clip=clip, smooth=sq.to(dev) if smooth else None,
+                                             meta_dtype=mdt)
+        got = q.cpu().to(torch.int32) + (128 if act == "per_tensor_asymm" else 0)
+        assert torch.equal(got, ref_int.to(torch.int32)), tag
+        y = op()(x.to(dev), w_int.to(dev), bias.to(dev), qdata.to(dev),
+                 "per_channel" if per_channel else "per_tensor", act, smooth)
+        exact = exact_from_oracle_codes(x, w_int, bias, w_cv, a_cv, a_cvn, sq, act)
+        ulp = 2.0 ** -8 if xdt == torch.bfloat16 else 2.0 ** -11
+        err = (y.cpu().double() - exact).abs()
+        assert torch.all(err <= 1.1 * ulp * exact.abs() + 1e-3 * exact.abs().max() * ulp + 1e-6), tag
+
+
 def test_three_dimensional_input_and_dummy_bias(dev):
     x, w_int, _, qdata, *_ = make_case(31, 6 * 5, 128, 64, torch.float16, torch.float16, True,
                                        "per_token", False)

@@ -105,6 +105,38 @@ def test_bmm_fp8_exact_on_integer_operands(dev, shape):
     assert torch.equal(y.double(), ref)
 
 
+def test_bmm_random_shapes_exact(dev):
+    """Thirty seeded batched products: any batch count, M and N, K a multiple of 64 up to 1024,
+    with and without the per-column bias: int8 exact up to the fp32 conversion (power-of-two
+    scales), e4m3 exact on small integers; whichever batched kernel serves the shape."""
+    import random
+
+    rng = random.Random(86420)
+    for case in range(30):
+        B = rng.choice([1, rng.randint(2, 8), rng.randint(8, 48)])
+        M, N = rng.choice([1, rng.randint(2, 130), rng.randint(130, 700)]), rng.randint(1, 700)
+        Kd = 64 * rng.randint(1, 16)
+        if B * M * N > 12e6:
+            B = max(1, int(12e6 // (M * N)))
+        tag = f"case {case}: B={B} M={M} N={N} K={Kd}"
+        g = gen(9000 + case)
+        a = torch.randint(-128, 128, (B, M, Kd), generator=g, dtype=torch.int32).to(torch.int8)
+        b = torch.randint(-128, 128, (B, N, Kd), generator=g, dtype=torch.int32).to(torch.int8)
+        bias = torch.randn(B, N, generator=g) if case % 2 else None
+        sa, sb = torch.tensor([2.0 ** -7]), torch.tensor([2.0 ** -9])
+        y = K().bmm_i8_dq(a.to(dev), b.to(dev), sa.to(dev), sb.to(dev),
+                          bias=None if bias is None else bias.to(dev), out_dtype=torch.float32).cpu()
+        acc = torch.matmul(a.to(dev).double(), b.to(dev).double().transpose(1, 2)).cpu()
+        ref = acc * 2.0 ** -16 + (bias.double().unsqueeze(1) if bias is not None else 0.0)
+        torch.testing.assert_close(y.double(), ref, rtol=2e-7, atol=1e-6, msg=tag)
+        a8 = torch.randint(-8, 9, (B, M, Kd), generator=g).float().to(torch.float8_e4m3fn)
+        b8 = torch.randint(-8, 9, (B, N, Kd), generator=g).float().to(torch.float8_e4m3fn)
+        s = torch.tensor([0.5])
+        y8 = K().bmm_fp8_dq(a8.to(dev), b8.to(dev), s.to(dev), s.to(dev), out_dtype=torch.float32).cpu()
+        ref8 = torch.matmul(a8.to(dev).double(), b8.to(dev).double().transpose(1, 2)).cpu() * 0.25
+        assert torch.equal(y8.double(), ref8), tag
+
+
 def stub_qbmm(clip1, clipn1, clip2, mode="asym", nbits1=8, dtype=torch.float32):
     m = torch.nn.Module()
     m.num_bits_m1, m.num_bits_m2, m.qm1_mode = nbits1, 8, mode

@@ -158,6 +158,41 @@ def test_deploy_module_static_branches_bit_exact(dev, pt_native, regime, qa):
         assert torch.equal(qt.cpu(), O.quant_act_pt_native(x, st["input_scale"], st["input_zp"], st["useSymAct"]))
 
 
+def test_deploy_module_static_branches_random_layers(dev):
+    """Sixteen seeded layers through the static branches: random clip values (asymmetric and
+    symmetric), both formulas, both buffer regimes, with and without bias, any M, K a multiple of
+    64, N a multiple of 8: buffers, integer codes and outputs are the oracle's bit for bit."""
+    import random
+
+    from fms_mo_amd.modules.linear import QLinearINT8Deploy
+
+    rng = random.Random(13579)
+    for case in range(16):
+        sym = rng.random() < 0.4
+        a_cv = round(rng.uniform(2.0, 8.0), 3)
+        a_cvn = -a_cv if sym else -round(rng.uniform(0.5, 6.0), 3)
+        pt_native, fp32_buffers, bias = rng.random() < 0.5, rng.random() < 0.5, rng.random() < 0.7
+        K, N = 64 * rng.randint(1, 40), 8 * rng.randint(1, 120)
+        M = rng.choice([1, rng.randint(2, 16), rng.randint(17, 300)])
+        tag = (f"case {case}: sym={sym} cv={a_cv}/{a_cvn} pt_native={pt_native} fp32_buffers={fp32_buffers} "
+               f"bias={bias} M={M} K={K} N={N}")
+        m = make_static_qlinear(K, N, "max" if sym else "minmax", a_cv, a_cvn, seed=100 + case, bias=bias,
+                                buffers_fp32=fp32_buffers)
+        x = static_x(M, K, 200 + case)
+        dep = QLinearINT8Deploy.from_fms_mo(m, use_int_kernel="cutlass", use_PT_native_Qfunc=pt_native,
+                                            recalc_clipvals=False, target_device=dev)
+        Qa, Qw = m.quantize_feature, m.quantize_weight
+        st = O.deploy_prepare_general(m.weight.detach(), m.bias.detach() if bias else None, Qw.clip_val,
+                                      Qa.clip_val, Qa.clip_valn, sym_act=sym, use_PT_native_Qfunc=pt_native)
+        assert torch.equal(dep.weight.cpu(), st["weight"]) and int(dep.input_zp) == int(st["input_zp"]), tag
+        assert torch.equal(bits(dep.corr_term.cpu()), bits(st["corr_term"])), tag
+        assert torch.equal(bits(dep.bias.cpu()), bits(st["bias"])), tag
+        ref = O.deploy_forward_general(x, st)
+        assert torch.equal(dep._quantize(x.to(dev)).cpu(), ref["q_x"]), tag
+        y = dep(x.to(dev))
+        assert torch.equal(bits(y.cpu()), bits(ref["y"])), tag
+
+
 @pytest.mark.parametrize("pt_native", [True, False])
 @pytest.mark.parametrize("acc_dtype", [torch.float32, torch.float16])
 @pytest.mark.parametrize("with_bias", [True, False])
