@@ -124,6 +124,27 @@ def test_noalloc_entry_point_allocates_nothing_and_repeats(dev):
         assert torch.equal(y.view(torch.int16), y_ref.view(torch.int16))
 
 
+def test_noalloc_entry_point_random_sequence_of_calls(dev):
+    """Twenty-four seeded calls in a row through the shared array, shapes on both sides of every
+    routing boundary (decode kernels, K slices of either tile kind, plans that had to shrink to
+    fit, single pass): each equals the plain entry point's result bit for bit."""
+    import random
+
+    rng = random.Random(24680)
+    for case in range(24):
+        M = rng.choice([rng.randint(1, 16), rng.randint(17, 128), rng.randint(129, 700), rng.randint(700, 1500)])
+        N = rng.choice([8 * rng.randint(1, 64), 128 * rng.randint(1, 48), rng.randint(100, 5000)])
+        K = rng.choice([128 * rng.randint(4, 128), 1024 * rng.choice([1, 2, 4, 8, 14]), 64 * rng.randint(1, 64)])
+        epi = rng.choice([0, 1])
+        odt = torch.float16 if epi == 0 else rng.choice([torch.float16, torch.bfloat16, torch.float32])
+        bdt = rng.choice([None, torch.float16, torch.float32])
+        ops = _operands(M, N, K, 500 + case, dev, bdt)
+        y_ref = _run("fmsmo_gemm_i8_dq", ops, M, N, K, epi, odt)
+        y = _run("fmsmo_gemm_i8_dq_noalloc", ops, M, N, K, epi, odt)
+        torch.cuda.synchronize()
+        assert torch.equal(y.view(torch.uint8), y_ref.view(torch.uint8)), f"case {case}: M={M} N={N} K={K} epi={epi} {odt} bias={bdt}"
+
+
 def test_noalloc_entry_point_validates_like_the_others(dev):
     from fms_mo_amd import _lib as L
 
