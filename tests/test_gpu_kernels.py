@@ -658,6 +658,53 @@ def test_gemm_fp8_dq(dev, M):
     torch.testing.assert_close(y.cpu().float(), ref.float(), rtol=2e-2, atol=2e-2)
 
 
+def test_gemm_fp8_random_shapes_and_fused_decode(dev):
+    """Forty seeded e4m3 products from one row to a few thousand: every route (decode kernels, K
+    slices, tiles) against the float64 product of the same codes within the stated tolerance,
+    single or per-row / per-column scales, any bias dtype; where the fused decode linear serves a
+    shape it returns the quantizer's scales and the GEMM's outputs bit for bit."""
+    import random
+
+    from fms_mo_amd import _lib as L
+
+    rng = random.Random(11235)
+    kn = K()
+    for case in range(40):
+        M = rng.choice([1, 2, 3, 4, rng.randint(5, 64), rng.randint(65, 600), rng.randint(600, 3000)])
+        N = rng.choice([rng.randint(8, 300), 16 * rng.randint(1, 300), rng.randint(300, 5000)])
+        Kd = rng.choice([64 * rng.randint(1, 32), 128 * rng.randint(1, 112), 1024 * rng.choice([1, 2, 4, 8, 14]), 12800])
+        if M > 600:
+            Kd = min(Kd, 4096)
+        an, wn = rng.choice([1, M]), rng.choice([1, N])
+        bdt = rng.choice([None, torch.float16, torch.bfloat16, torch.float32])
+        odt = rng.choice([torch.float16, torch.bfloat16, torch.float32])
+        tag = f"case {case}: M={M} N={N} K={Kd} a_scales={an} w_scales={wn} bias={bdt} out={odt}"
+        a = _rand_fp8((M, Kd), 7000 + case, 2.0).to(dev)
+        w = _rand_fp8((N, Kd), 7100 + case, 0.5).to(dev)
+        s_a = (torch.rand(an, generator=gen(7200 + case)) * 0.05 + 1e-3).to(dev)
+        s_w = (torch.rand(wn, generator=gen(7300 + case)) * 0.01 + 1e-4).to(dev)
+        bias = None if bdt is None else (torch.randn(N, generator=gen(7400 + case)) * 0.1).to(bdt).to(dev)
+        exact = (a.double() @ w.double().t()) * s_a.double()[:, None] * s_w.double()[None, :]
+        if bias is not None:
+            exact = exact + bias.double()
+        y = kn.gemm_fp8_dq(a, w, s_a, s_w, bias, out_dtype=odt)
+        torch.testing.assert_close(y.double(), exact, rtol=1e-2, atol=1e-2, msg=tag)
+        # fp32 accumulation: far inside the tolerance when the output is fp32
+        if odt == torch.float32:
+            torch.testing.assert_close(y.double(), exact, rtol=1e-4, atol=1e-4 * exact.abs().max().item(), msg=tag)
+        if M <= 4:
+            dt = torch.float16 if case % 2 else torch.bfloat16
+            x = (2.0 * torch.randn(M, Kd, generator=gen(7500 + case))).to(dt).to(dev)
+            if kn.decode_linear_ok(x, None, Kd):
+                b16 = None if bias is None else bias.to(dt)
+                sw_n = s_w if wn == N else s_w.expand(N).contiguous()
+                q, s = kn.quant_act_fp8_pertoken(x, L.FP8_LINEAR)
+                ref = kn.gemm_fp8_dq(q, w, s, sw_n, b16, out_dtype=dt)
+                y2, s2 = kn.decode_linear_fp8(x, w, sw_n, b16, out_dtype=dt)
+                assert torch.equal(s2.view(torch.int32), s.view(torch.int32)), tag
+                assert torch.equal(y2.view(torch.int16), ref.view(torch.int16)), tag
+
+
 @pytest.mark.parametrize("shape", [(256, 512, 1024), (4000, 4100, 384), (4097, 4095, 128), (4000, 4000, 384)])
 def test_gemm_fp8_integer_valued_is_exact(dev, shape):
     # small-integer operands: every product and partial sum is exact in fp32, so any MFMA
