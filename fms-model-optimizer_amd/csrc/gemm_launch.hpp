@@ -295,6 +295,12 @@ inline SplitPlan plan_split_k(int64_t M, int64_t N, int64_t K, int64_t limit = 0
   if (tiles > 128) return p;
   int s = (int)(256 / tiles);  // one block per compute unit; 512 and 1024 blocks measured slower
   while (s > 1 && (K % (s * 128) != 0 || K / s < 512)) --s;
+  // Slices of 512 are mostly prologue and partial-sum traffic (as many bytes as the weights at
+  // 128 rows): from K = 4096 on, half as many slices of 1024 are faster while 64 blocks remain
+  // (us, M = 65 / 100 / 128: N = 4096, K = 4096 16.4 / 18.8 / 18.1 -> 15.8 / 17.2 / 16.5; N = 2048
+  // 13.8 / 15.1 / 14.1 -> 13.2 / 13.5 / 11.8; N = 1024, K = 8192 15.5 / 16.7 / 15.4 -> 14.2 / 14.6 /
+  // 13.1; N = 1000, K = 4096, where 32 blocks would remain, 12.7 -> 14.1; K = 2048 no difference)
+  if (K >= 4096 && K / s <= 512 && s >= 4 && s % 2 == 0 && tiles * (s / 2) >= 64) s /= 2;
   if (s < 2) return p;
   p.splits = s;
   p.k_len = K / s;

@@ -122,6 +122,10 @@ def test_workspace_plan_is_host_logic():
     assert b > 0 and b % (64 * 4096 * 4) == 0
     s = b // (64 * 4096 * 4)
     assert 2 <= s <= 8 and 14336 % (s * 128) == 0 and 14336 // s >= 512
+    # from K = 4096 on, slices of 1024 instead of 512 while at least 64 blocks remain
+    assert lib.fmsmo_gemm_workspace_bytes(128, 4096, 4096) == 4 * 128 * 4096 * 4    # 32 tiles x 4
+    assert lib.fmsmo_gemm_workspace_bytes(128, 1000, 4096) == 8 * 128 * 1000 * 4    # 8 tiles x 8
+    assert lib.fmsmo_gemm_workspace_bytes(128, 4096, 2048) == 4 * 128 * 4096 * 4    # K < 4096: 512
 
 
 def test_gemm_plan_is_host_logic():
