@@ -453,8 +453,10 @@ def test_gemm_i8_dq_random_shapes_scales_and_epilogues(dev):
         N = rng.choice([rng.randint(8, 300), rng.randint(300, 2100), rng.randint(2100, 6200)])
         Kd = rng.choice([16 * rng.randint(1, 40), 64 * rng.randint(1, 24), 128 * rng.randint(1, 40)])
         g = torch.Generator(device=dev).manual_seed(4000 + case)
-        a = torch.randint(-128, 128, (M, Kd), generator=g, dtype=torch.int8, device=dev)
-        w = torch.randint(-128, 128, (N, Kd), generator=g, dtype=torch.int8, device=dev)
+        # every third case: operands that are column slices of wider buffers (row stride > K)
+        pa, pw = (16 * rng.randint(1, 8), 16 * rng.randint(1, 8)) if case % 3 == 2 else (0, 0)
+        a = torch.randint(-128, 128, (M, Kd + pa), generator=g, dtype=torch.int8, device=dev)[:, :Kd]
+        w = torch.randint(-128, 128, (N, Kd + pw), generator=g, dtype=torch.int8, device=dev)[:, :Kd]
         acc = (a.double() @ w.double().t()).to(torch.int32).cpu()
         an, wn = rng.choice([1, M]), rng.choice([1, N])
         s_a = (torch.rand(an, 1, generator=gen(4100 + case)) * 0.05 + 1e-3).half()
@@ -608,8 +610,10 @@ def test_decode_range_random_shapes(dev):
                          1024 * rng.choice([1, 2, 4, 5, 8, 11, 13, 14, 16]), 12800, 14336])
         tag = f"case {case}: M={M} N={N} K={Kd}"
         g = torch.Generator(device=dev).manual_seed(500 + case)
-        a = torch.randint(-128, 128, (M, Kd), generator=g, dtype=torch.int8, device=dev)
-        w = torch.randint(-128, 128, (N, Kd), generator=g, dtype=torch.int8, device=dev)
+        # every third case: operands that are column slices of wider buffers (row stride > K)
+        pa, pw = (16 * rng.randint(1, 8), 16 * rng.randint(1, 8)) if case % 3 == 2 else (0, 0)
+        a = torch.randint(-128, 128, (M, Kd + pa), generator=g, dtype=torch.int8, device=dev)[:, :Kd]
+        w = torch.randint(-128, 128, (N, Kd + pw), generator=g, dtype=torch.int8, device=dev)[:, :Kd]
         acc = (a.double() @ w.double().t()).to(torch.int32)
         assert torch.equal(kn.gemm_i8_i32(a, w), acc), tag
         s_a = (torch.rand(M, 1, generator=gen(600 + case)) * 0.05 + 1e-3).half()
