@@ -206,6 +206,12 @@ extern "C" int fmsmo_gemm_plan(int64_t M, int64_t N, int64_t K, int with_workspa
     *kernel = FMSMO_PLAN_DECODE;
     return FMSMO_OK;
   }
+  if (use_tall_tiles(M, N, K)) {  // one pass of 128 x 64 tiles, with or without a workspace
+    *kernel = FMSMO_PLAN_TILE_LDS_DMA;
+    *tile_m = TileTallK::BM;
+    *tile_n = TileTallK::BN;
+    return FMSMO_OK;
+  }
   const SplitPlan plan = plan_split_k(M, N, K);
   if (with_workspace && plan.splits > 1) {
     *kernel = plan.rs ? FMSMO_PLAN_TILE_REGISTER_STAGED : FMSMO_PLAN_TILE_LDS_DMA;

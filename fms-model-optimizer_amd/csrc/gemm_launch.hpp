@@ -41,6 +41,30 @@ int check_gemm(const void* a, int64_t lda, const void* b, int64_t ldb, const voi
 struct TileBig { static constexpr int BM = 256, BN = 256, BK = 64, NST = 4, WGM = 2, WGN = 2; };
 struct TileWide { static constexpr int BM = 128, BN = 256, BK = 64, NST = 4, WGM = 2, WGN = 2; };
 struct TileMid { static constexpr int BM = 128, BN = 128, BK = 64, NST = 4, WGM = 2, WGN = 2; };
+// The same tiles with stages of 128 bytes of K (whole 128-byte lines per row and request, half as
+// many barriers): K % 128 == 0, one block per compute unit (128 / 120 KiB of LDS).  Pipelines of
+// three stages lose a third against five; six (tall) and five (square) change nothing.
+struct TileMidK { static constexpr int BM = 128, BN = 128, BK = 128, NST = 4, WGM = 2, WGN = 2; };
+struct TileTallK { static constexpr int BM = 128, BN = 64, BK = 128, NST = 5, WGM = 2, WGN = 2; };
+
+// A few hundred rows through a projection whose 128 x 64 tiles fill half a round of the 256
+// compute units or more run as ONE pass of those tiles rather than as K slices with a second
+// kernel: no partial sums to write and read back.  A block walks K in ~0.41 us per 1024 (one
+// round: 4.4 us + 3.3 us per 1024 of K whatever the rows), so the slices win again on long
+// reductions.  us from a HIP graph, int8, before -> after (e4m3 within 5 % of these):
+//   N = 4096, K = 4096: M = 129 17.5 -> 14.7, 256 21.4 -> 17.0, 512 25.7 -> 18.3 (vendor GEMM, int32
+//   out: 18.1); N = 6144: 129 20.9 -> 16.1, 256 22.1 -> 17.3; N = 2048: 512 22.6 -> 16.1, 1024 25.9 ->
+//   17.5; N = 1024: 1024 21.9 -> 15.6; K = 2048, N = 4096: 129 / 256 / 512 14.4 / 18.2 / 22.9 -> 9.5 /
+//   10.7 / 11.3; K = 8192: 512 36.4 -> 31.6; half a round at K = 5120 / 8192 loses (256 rows: 21.1 ->
+//   22.8, 24.5 -> 29.1) and so does K = 14336 (512 rows 48.2 -> 51.3): those keep the slices.
+inline bool use_tall_tiles(int64_t M, int64_t N, int64_t K) {
+  static const char* off = getenv("FMSMO_TALL");  // FMSMO_TALL=0 disables (tuning aid)
+  if (off && off[0] == '0') return false;
+  if (M <= 128 || M > 1024 || K % 128) return false;
+  const int64_t tiles = (int64_t)div_up(M, TileTallK::BM) * div_up(N, TileTallK::BN);
+  if (tiles > 256) return false;
+  return tiles >= 192 ? K <= 8192 : (tiles >= 96 && K <= 4096);
+}
 
 // Pick the tile shape by (relative kernel efficiency) x (fill of the last round of tiles over
 // the 256 compute units).  The efficiencies are measured loop efficiencies of the shapes
@@ -151,7 +175,9 @@ __global__ void gemm_simple_kernel(GemmArgs g, Epi epi) {
 
 template <int OP, class Epi>
 void launch_any(const GemmArgs& g, const Epi& epi, hipStream_t st) {
-  if (g.K % 64 == 0) {
+  if (use_tall_tiles(g.M, g.N, g.K)) {
+    launch_tile<TileTallK, OP, false>(g, epi, st);
+  } else if (g.K % 64 == 0) {
     switch (pick_tile(g.M, g.N, g.K % 128 == 0 && use_register_staged(OP))) {
       case 0:
         if (g.K % 128 == 0 && use_register_staged(OP)) launch_rs<OP>(g, epi, st);
@@ -163,7 +189,15 @@ void launch_any(const GemmArgs& g, const Epi& epi, hipStream_t st) {
         else launch_tile<TileBig, OP, false>(g, epi, st);
         break;
       case 4: launch_rs<OP, false, 128>(g, epi, st); break;  // only offered when K % 128 == 0
-      default: launch_tile<TileMid, OP, false>(g, epi, st); break;
+      default:
+        // one round of 128 x 128 tiles: stages of 128 bytes (us, 1024 rows, N = 4096: K = 4096 29.0 ->
+        // 25.6, 5120 36.8 -> 31.2; 512 rows, N = 6144, K = 4096: 28.0 -> 23.5); more than a round keeps
+        // the 64-byte stages, whose blocks fit two to a compute unit
+        if (g.K % 128 == 0 && (long)div_up(g.M, TileMidK::BM) * div_up(g.N, TileMidK::BN) <= 256)
+          launch_tile<TileMidK, OP, false>(g, epi, st);
+        else
+          launch_tile<TileMid, OP, false>(g, epi, st);
+        break;
     }
   } else {
     dim3 grid(div_up(g.N, 64), (unsigned)g.M), block(64);
@@ -272,14 +306,17 @@ inline SplitPlan plan_split_k(int64_t M, int64_t N, int64_t K, int64_t limit = 0
   SplitPlan p{1, K, 0, false};
   static const char* off = getenv("FMSMO_SPLIT_K");  // FMSMO_SPLIT_K=0 disables (tuning aid)
   if (off && off[0] == '0') return p;
-  if (M <= 16 || M > 1024 || K % 128) return p;
+  if (M <= 16 || M > 1024 || K % 128 || use_tall_tiles(M, N, K)) return p;
   // Long reductions under a few hundred rows: 256 x 128 tiles of the register-staged kernel carry
   // the slices (us, 128 x 128 LDS-DMA tiles -> these, N = 4096, K = 14336: M = 384 51.4 -> 49.0,
   // 512 54.6 -> 48.3, 768 84.7 -> 68.2, 1024 87.6 -> 77.8; at K = 4096 they lose, M = 512 25.5 ->
   // 27.7, and below 384 rows their 256-row tiles are half empty)
   if (K >= 8192 && M >= 384 && use_register_staged(0)) {
     const int64_t t = (int64_t)div_up(M, 256) * div_up(N, 128);
-    if (t <= 128) {
+    // a full round of 128 x 128 tiles runs faster in one pass with 128-byte stages than as two
+    // slices (1024 x 4096, us: K = 8192 53.4 -> 42.6, K = 14336 80.0 -> 72.5)
+    const bool full_round = (int64_t)div_up(M, TileMidK::BM) * div_up(N, TileMidK::BN) == 256;
+    if (t <= 128 && !full_round) {
       int s = (int)(256 / t);
       while (s > 1 && (K % (s * 128) != 0 || K / s < 512)) --s;
       if (s >= 2 && (limit <= 0 || (int64_t)s * M * N * 4 <= limit)) {

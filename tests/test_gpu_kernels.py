@@ -1021,10 +1021,10 @@ def _plain_i8_dq(a, w, a_s, w_s, bias, out_dtype, exact_ref):
     return y
 
 
-@pytest.mark.parametrize("shape", [(17, 4096, 14336), (64, 4096, 4096), (200, 1024, 1536), (512, 4096, 4096),
+@pytest.mark.parametrize("shape", [(17, 4096, 14336), (64, 4096, 4096), (200, 1024, 1536), (128, 4096, 4096),
                                    (100, 520, 2048), (128, 6144, 4096), (1000, 1024, 14336),
                                    # long reductions from 384 rows: register-staged 256 x 128 tiles
-                                   (384, 4096, 14336), (700, 1000, 8192), (1024, 4096, 14336), (513, 264, 12800)])
+                                   (384, 4096, 14336), (700, 1000, 8192), (768, 4096, 14336), (513, 264, 12800)])
 @pytest.mark.parametrize("exact_ref,out_dtype", [(True, torch.float16), (False, torch.bfloat16), (False, torch.float32)])
 def test_split_k_int8_is_bit_identical_to_single_pass(dev, shape, exact_ref, out_dtype):
     from fms_mo_amd import _lib as L
@@ -1048,6 +1048,39 @@ def test_split_k_int8_is_bit_identical_to_single_pass(dev, shape, exact_ref, out
     exact = acc.double() * a_s[:5].cpu().double()[:, None] * w_s.cpu().double()[None, :]
     y = Kn.gemm_i8_dq(a, w, a_s, w_s, None, out_dtype=torch.float32, exact_ref=False)
     torch.testing.assert_close(y[:5].cpu().double(), exact, rtol=1e-6, atol=1e-6)
+
+
+@pytest.mark.parametrize("shape", [(512, 4096, 4096), (129, 4096, 4096), (256, 6144, 4096), (1024, 2000, 4096),
+                                   (500, 4090, 8192), (300, 4096, 2048),     # 128 x 64 tiles, 128-byte stages
+                                   (1024, 4096, 8192), (512, 6144, 4096), (1000, 4000, 1152),  # 128 x 128
+                                   (200, 13824, 5120)])
+def test_one_pass_tiles_with_128_byte_stages(dev, shape):
+    """A few hundred rows through a projection that fills half a round of 128 x 64 tiles or more
+    (and a round of 128 x 128 tiles) run in one pass even when a workspace is offered: int8
+    bit-exact against the oracle's epilogue on the exact product, e4m3 exact on small integers,
+    ragged last tiles included."""
+    M, N, Kd = shape
+    kn = K()
+    plan = kn.gemm_plan(M, N, Kd, with_workspace=True)
+    assert plan[3] == 1 and plan[1] == 128, plan
+    g = torch.Generator(device=dev).manual_seed(M + N)
+    a = torch.randint(-128, 128, (M, Kd), generator=g, dtype=torch.int8, device=dev)
+    w = torch.randint(-128, 128, (N, Kd), generator=g, dtype=torch.int8, device=dev)
+    acc = (a.double() @ w.double().t()).to(torch.int32)
+    assert torch.equal(kn.gemm_i8_i32(a, w), acc)
+    s_a = (torch.rand(M, 1, generator=gen(61)) * 0.05 + 1e-3).half()
+    s_w = (torch.rand(N, generator=gen(62)) * 1e-3 + 1e-5).float()
+    bias = (torch.randn(N, generator=gen(63)) * 0.01).half()
+    ref = O.epilogue_ref(acc.cpu(), s_a, s_w, bias, torch.float16)
+    y = kn.gemm_i8_dq(a, w, s_a.float().reshape(-1).to(dev), s_w.to(dev), bias.to(dev), out_dtype=torch.float16,
+                      exact_ref=True)
+    assert torch.equal(y.cpu().view(torch.int16), ref.view(torch.int16))
+    a8 = torch.randint(-4, 5, (M, Kd), generator=g, device=dev).float()
+    w8 = torch.randint(-4, 5, (N, Kd), generator=g, device=dev).float()
+    one = torch.ones(1, device=dev)
+    y8 = kn.gemm_fp8_dq(a8.to(torch.float8_e4m3fn), w8.to(torch.float8_e4m3fn), one, one, None,
+                        out_dtype=torch.float32)
+    assert torch.equal(y8, a8 @ w8.t())
 
 
 @pytest.mark.parametrize("shape", [(17, 4096, 14336), (64, 4096, 4096), (200, 1024, 1536), (100, 520, 2048),

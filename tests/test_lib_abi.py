@@ -171,9 +171,20 @@ def test_gemm_plan_is_host_logic():
     # a few hundred rows through a long reduction: the slices run on register-staged 256 x 128 tiles
     if not os.environ.get("FMSMO_RS"):
         assert K.gemm_plan(512, 4096, 14336, with_workspace=True) == (RS, 256, 128, 4)
-        assert K.gemm_plan(1024, 4096, 14336, with_workspace=True) == (RS, 256, 128, 2)
+        assert K.gemm_plan(768, 4096, 14336, with_workspace=True) == (RS, 256, 128, 2)
+    # a full round of 128 x 128 tiles runs in one pass
+    assert K.gemm_plan(1024, 4096, 14336, with_workspace=True) == (DMA, 128, 128, 1)
     assert K.gemm_plan(256, 4096, 14336, with_workspace=True)[:3] == (DMA, 128, 128)
-    assert K.gemm_plan(512, 4096, 4096, with_workspace=True)[:3] == (DMA, 128, 128)
+    # half a round or more of 128 x 64 tiles and a short reduction: one pass of those, no slices
+    if not os.environ.get("FMSMO_TALL"):
+        for shape in ((512, 4096, 4096), (256, 4096, 4096), (256, 6144, 4096), (1024, 2048, 4096),
+                      (512, 4096, 8192), (300, 4096, 2048)):
+            assert K.gemm_plan(*shape, with_workspace=True) == (DMA, 128, 64, 1), shape
+            assert _lib.load().fmsmo_gemm_workspace_bytes(*shape) == 0
+        # long reductions and half-filled rounds of longer ones keep the slices
+        for shape in ((512, 4096, 14336), (256, 4096, 8192), (256, 4096, 5120), (128, 4096, 4096),
+                      (256, 1024, 4096)):
+            assert K.gemm_plan(*shape, with_workspace=True)[3] >= 2, shape
     # K in 64-byte stages only: no register-staged kernel; K % 64 != 0: generic kernel
     assert K.gemm_plan(4096, 4096, 4160)[0] == DMA
     assert K.gemm_plan(300, 520, 1040) == (_lib.PLAN_GENERIC, 0, 0, 1)

@@ -82,8 +82,7 @@ def test_noalloc_entry_point_takes_the_plan_that_fits(dev):
     torch.cuda.synchronize()
     for other in (y_big, y_small, y_none):
         assert torch.equal(y.view(torch.int16), other.view(torch.int16))
-    # 1024 rows: the preferred plan needs 32 MiB and the 128 x 128 tiles do not split (256 tiles):
-    # the call runs the single pass
+    # 1024 rows: a full round of 128 x 128 tiles, one pass with every entry point
     ops = _operands(1024, N, K, 301, dev, None)
     y_none = _run("fmsmo_gemm_i8_dq", ops, 1024, N, K, 0, torch.float16)
     y = _run("fmsmo_gemm_i8_dq_noalloc", ops, 1024, N, K, 0, torch.float16)
