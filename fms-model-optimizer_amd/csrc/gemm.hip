@@ -216,7 +216,7 @@ extern "C" int fmsmo_gemm_plan(int64_t M, int64_t N, int64_t K, int with_workspa
   if (with_workspace && plan.splits > 1) {
     *kernel = plan.rs ? FMSMO_PLAN_TILE_REGISTER_STAGED : FMSMO_PLAN_TILE_LDS_DMA;
     *tile_m = plan.rs ? 256 : TileMid::BM;
-    *tile_n = plan.rs ? 128 : TileMid::BN;
+    *tile_n = plan.rs ? 128 : plan.tall ? TileTallK::BN : TileMid::BN;
     *splits = plan.splits;
     return FMSMO_OK;
   }

@@ -298,6 +298,7 @@ struct SplitPlan {
   int splits;
   int64_t k_len, ws_bytes;
   bool rs;  // 256 x 128 tiles of the register-staged kernel instead of 128 x 128 LDS-DMA tiles
+  bool tall = false;  // 128 x 64 tiles with 128-byte stages
 };
 
 // `limit` > 0: the workspace at hand; a plan that needs more is passed over for the next one (the
@@ -328,6 +329,27 @@ inline SplitPlan plan_split_k(int64_t M, int64_t N, int64_t K, int64_t limit = 0
       }
     }
   }
+  // Slices of at least 1024 on 128 x 64 tiles with 128-byte stages: twice the blocks of the
+  // 128 x 128 tiles for the same partial sums, or the same blocks for half of them (us, 128 x 128
+  // tiles with 64-byte stages -> these, M = 65 / 100 / 128: N = 4096, K = 4096 15.8 / 16.9 / 16.5 ->
+  // 13.4 / 14.2 / 14.9; N = 2048 13.2 / 13.5 / 11.9 -> 9.4 / 9.9 / 9.7; N = 1000 12.6 / 13.0 / 12.7 ->
+  // 10.3 / 10.8 / 10.7; N = 4096, K = 2048 12.8 / 14.4 / 13.6 -> 10.1 / 11.5 / 11.4; K = 5120 17.3 /
+  // 19.4 / 17.9 -> 13.8 / 15.5 / 16.3; K = 8192 18.9 / 19.6 / 18.3 -> 17.4 / 18.5 / 17.2; N = 1024,
+  // K = 8192 14.3 / 14.6 / 13.1 -> 10.6 / 11.2 / 11.2; K = 14336, N = 4096, M = 33 / 128 / 256 22.7 /
+  // 25.1 / 34.1 -> 22.1 / 24.3 / 33.0).  At most 256 blocks of 128 x 64 partial sums: 8 MiB.
+  const int64_t tiles_t = (int64_t)div_up(M, TileTallK::BM) * div_up(N, TileTallK::BN);
+  if (tiles_t <= 128) {
+    int s = (int)(256 / tiles_t);
+    while (s > 1 && (K % (s * 128) != 0 || K / s < 1024)) --s;
+    if (s >= 2) {
+      p.splits = s;
+      p.k_len = K / s;
+      p.ws_bytes = (int64_t)s * M * N * 4;
+      p.tall = true;
+      return p;
+    }
+  }
+  // shorter reductions: 128 x 128 tiles, slices of at least 512
   const int64_t tiles = (int64_t)div_up(M, TileMid::BM) * div_up(N, TileMid::BN);
   if (tiles > 128) return p;
   int s = (int)(256 / tiles);  // one block per compute unit; 512 and 1024 blocks measured slower
@@ -367,6 +389,7 @@ inline int launch_split_k_i32(const SplitPlan& p, const GemmArgs& g0, void* work
   g.ldb_e = p.k_len;
   g.grid_m = p.splits * div_up(g0.M, p.rs ? 256 : TileMid::BM);
   if (p.rs) launch_rs<MMA_I8, true, 128>(g, EpiStoreI32{(int32_t*)workspace, g0.N}, st);
+  else if (p.tall) launch_tile<TileTallK, MMA_I8, true>(g, EpiStoreI32{(int32_t*)workspace, g0.N}, st);
   else launch_tile<TileMid, MMA_I8, true>(g, EpiStoreI32{(int32_t*)workspace, g0.N}, st);
   dim3 grid(div_up(g0.N, 256), (unsigned)g0.M), block(256);
   EpiStoreI32 epi{c, ldc};
@@ -391,6 +414,9 @@ int launch_split_k(const SplitPlan& p, const GemmArgs& g0, void* workspace, cons
   if (p.rs) {
     if constexpr (OP == MMA_I8) launch_rs<OP, true, 128>(g, EpiStoreI32{(int32_t*)workspace, g0.N}, st);
     else launch_rs<OP, true, 128>(g, EpiStoreF32{(float*)workspace, g0.N}, st);
+  } else if (p.tall) {
+    if constexpr (OP == MMA_I8) launch_tile<TileTallK, OP, true>(g, EpiStoreI32{(int32_t*)workspace, g0.N}, st);
+    else launch_tile<TileTallK, OP, true>(g, EpiStoreF32{(float*)workspace, g0.N}, st);
   } else if constexpr (OP == MMA_I8) launch_tile<TileMid, OP, true>(g, EpiStoreI32{(int32_t*)workspace, g0.N}, st);
   else launch_tile<TileMid, OP, true>(g, EpiStoreF32{(float*)workspace, g0.N}, st);
   if (!bias) bias_dtype = FMSMO_F32;

@@ -122,10 +122,12 @@ def test_workspace_plan_is_host_logic():
     assert b > 0 and b % (64 * 4096 * 4) == 0
     s = b // (64 * 4096 * 4)
     assert 2 <= s <= 8 and 14336 % (s * 128) == 0 and 14336 // s >= 512
-    # from K = 4096 on, slices of 1024 instead of 512 while at least 64 blocks remain
-    assert lib.fmsmo_gemm_workspace_bytes(128, 4096, 4096) == 4 * 128 * 4096 * 4    # 32 tiles x 4
-    assert lib.fmsmo_gemm_workspace_bytes(128, 1000, 4096) == 8 * 128 * 1000 * 4    # 8 tiles x 8
-    assert lib.fmsmo_gemm_workspace_bytes(128, 4096, 2048) == 4 * 128 * 4096 * 4    # K < 4096: 512
+    # slices of at least 1024 on 128 x 64 tiles, at most 256 blocks
+    assert lib.fmsmo_gemm_workspace_bytes(128, 4096, 4096) == 4 * 128 * 4096 * 4    # 64 tiles x 4
+    assert lib.fmsmo_gemm_workspace_bytes(128, 1000, 4096) == 4 * 128 * 1000 * 4    # 16 tiles x 4
+    assert lib.fmsmo_gemm_workspace_bytes(128, 4096, 2048) == 2 * 128 * 4096 * 4
+    # reductions under 2048: 128 x 128 tiles, slices of at least 512
+    assert lib.fmsmo_gemm_workspace_bytes(200, 1024, 1536) == 3 * 200 * 1024 * 4
 
 
 def test_gemm_plan_is_host_logic():
@@ -166,7 +168,7 @@ def test_gemm_plan_is_host_logic():
     assert K.gemm_plan(33, 5120, 5120)[0] != _lib.PLAN_DECODE
     # a few tokens through a long reduction: split only when a workspace is offered
     k, tm, tn, s = K.gemm_plan(17, 4096, 14336, with_workspace=True)
-    assert (k, tm, tn) == (DMA, 128, 128) and s >= 2 and 14336 % (s * 128) == 0
+    assert (k, tm, tn) == (DMA, 128, 64) and s >= 2 and 14336 % (s * 128) == 0
     assert K.gemm_plan(17, 4096, 14336, with_workspace=False)[3] == 1
     # a few hundred rows through a long reduction: the slices run on register-staged 256 x 128 tiles
     if not os.environ.get("FMSMO_RS"):
@@ -174,7 +176,8 @@ def test_gemm_plan_is_host_logic():
         assert K.gemm_plan(768, 4096, 14336, with_workspace=True) == (RS, 256, 128, 2)
     # a full round of 128 x 128 tiles runs in one pass
     assert K.gemm_plan(1024, 4096, 14336, with_workspace=True) == (DMA, 128, 128, 1)
-    assert K.gemm_plan(256, 4096, 14336, with_workspace=True)[:3] == (DMA, 128, 128)
+    assert K.gemm_plan(256, 4096, 14336, with_workspace=True)[:3] == (DMA, 128, 64)
+    assert K.gemm_plan(200, 1024, 1536, with_workspace=True) == (DMA, 128, 128, 3)
     # half a round or more of 128 x 64 tiles and a short reduction: one pass of those, no slices
     if not os.environ.get("FMSMO_TALL"):
         for shape in ((512, 4096, 4096), (256, 4096, 4096), (256, 6144, 4096), (1024, 2048, 4096),

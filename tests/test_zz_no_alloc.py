@@ -35,9 +35,9 @@ def _run(name, ops, M, N, K, epilogue, out_dtype, workspace=None):
 
 CALLS = [
     # (M, N, K, epilogue, out dtype, bias dtype); splits and scratch bytes in the comments
-    (128, 4096, 14336, 0, torch.float16, torch.float16),   # 8 slices, 16 MiB: the whole array
+    (128, 4096, 14336, 0, torch.float16, torch.float16),   # 4 slices on 128 x 64 tiles, 8 MiB
     (17, 4096, 4096, 0, torch.float16, None),              # decode-batch kernel: no scratch used
-    (300, 1024, 2048, 1, torch.bfloat16, torch.float32),   # 4 slices of 512
+    (300, 1024, 2048, 1, torch.bfloat16, torch.float32),   # 2 slices of 1024
     (2048, 512, 1024, 1, torch.float32, None),             # no split: no scratch used
     (40, 6144, 4096, 0, torch.float16, torch.bfloat16),    # decode-batch kernel: no scratch used
 ]
