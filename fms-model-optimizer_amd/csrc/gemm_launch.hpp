@@ -49,7 +49,7 @@ struct TileTallK { static constexpr int BM = 128, BN = 64, BK = 128, NST = 5, WG
 
 // A few hundred rows through a projection whose 128 x 64 tiles fill half a round of the 256
 // compute units or more run as ONE pass of those tiles rather than as K slices with a second
-// kernel: no partial sums to write and read back.  A block walks K in ~0.41 us per 1024 (one
+// kernel: no partial sums to write and read back.  A block walks K in ~0.41 us per 128-byte stage (one
 // round: 4.4 us + 3.3 us per 1024 of K whatever the rows), so the slices win again on long
 // reductions.  us from a HIP graph, int8, before -> after (e4m3 within 5 % of these):
 //   N = 4096, K = 4096: M = 129 17.5 -> 14.7, 256 21.4 -> 17.0, 512 25.7 -> 18.3 (vendor GEMM, int32
