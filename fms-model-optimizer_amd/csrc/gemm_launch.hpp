@@ -60,10 +60,15 @@ struct TileTallK { static constexpr int BM = 128, BN = 64, BK = 128, NST = 5, WG
 inline bool use_tall_tiles(int64_t M, int64_t N, int64_t K) {
   static const char* off = getenv("FMSMO_TALL");  // FMSMO_TALL=0 disables (tuning aid)
   if (off && off[0] == '0') return false;
-  if (M <= 128 || M > 1024 || K % 128) return false;
+  if (M <= 16 || M > 1024 || K % 128) return false;
   const int64_t tiles = (int64_t)div_up(M, TileTallK::BM) * div_up(N, TileTallK::BN);
   if (tiles > 256) return false;
-  return tiles >= 192 ? K <= 8192 : (tiles >= 96 && K <= 4096);
+  // three quarters of a round or more: also for a single row of tiles (batches of 17 .. 128 tokens
+  // that the decode kernels do not take, through a wide projection; us, M = 33 / 64 / 128: N = 14336,
+  // K = 8192 39.4 / 39.6 / 42.5 -> 32.2 / 33.8 / 38.3; N = 13824, K = 5120 26.2 / 28.1 -> 20.7 / 23.2;
+  // N = 14336, K = 4096, M = 65 / 128 23.7 / 25.1 -> 19.6 / 20.1)
+  if (tiles >= 192) return K <= 8192;
+  return M > 128 && tiles >= 96 && K <= 4096;
 }
 
 // Pick the tile shape by (relative kernel efficiency) x (fill of the last round of tiles over

@@ -300,8 +300,8 @@ int fmsmo_gemm_fp8_dq(const uint8_t* a, int64_t lda, const uint8_t* b, int64_t l
  * fmsmo_gemm_i8_dq's; the e4m3 result differs from fmsmo_gemm_fp8_dq's only by the order of the
  * fp32 additions.  From 384 rows and K >= 8192 the slices run on 256 x 128 tiles of the
  * register-staged kernel (more, shorter slices: more partial sums).  Shapes whose 128 x 64 tiles
- * fill half a round of the compute units or more with a short reduction (128 < M <= 1024; 192-256
- * tiles and K <= 8192, or 96-191 tiles and K <= 4096), and a full round of 128 x 128 tiles, run in
+ * fill half a round of the compute units or more with a short reduction (192-256 tiles and
+ * K <= 8192, or M > 128, 96-191 tiles and K <= 4096), and a full round of 128 x 128 tiles, run in
  * one pass instead and ask for no workspace.  fmsmo_gemm_workspace_bytes
  * returns the bytes a shape can use at most (0: no split); with fewer bytes the call takes the
  * split that fits them (the 128 x 128 tiles' never needs more than 16 MiB), with none or

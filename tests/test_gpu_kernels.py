@@ -1053,7 +1053,8 @@ def test_split_k_int8_is_bit_identical_to_single_pass(dev, shape, exact_ref, out
 @pytest.mark.parametrize("shape", [(512, 4096, 4096), (129, 4096, 4096), (256, 6144, 4096), (1024, 2000, 4096),
                                    (500, 4090, 8192), (300, 4096, 2048),     # 128 x 64 tiles, 128-byte stages
                                    (1024, 4096, 8192), (512, 6144, 4096), (1000, 4000, 1152),  # 128 x 128
-                                   (200, 13824, 5120)])
+                                   (200, 13824, 5120),
+                                   (100, 14336, 4096), (48, 13824, 5120), (33, 14330, 8192)])  # one row of 128 x 64 tiles
 def test_one_pass_tiles_with_128_byte_stages(dev, shape):
     """A few hundred rows through a projection that fills half a round of 128 x 64 tiles or more
     (and a round of 128 x 128 tiles) run in one pass even when a workspace is offered: int8

@@ -181,7 +181,7 @@ def test_gemm_plan_is_host_logic():
     # half a round or more of 128 x 64 tiles and a short reduction: one pass of those, no slices
     if not os.environ.get("FMSMO_TALL"):
         for shape in ((512, 4096, 4096), (256, 4096, 4096), (256, 6144, 4096), (1024, 2048, 4096),
-                      (512, 4096, 8192), (300, 4096, 2048)):
+                      (512, 4096, 8192), (300, 4096, 2048), (100, 14336, 4096), (48, 13824, 5120)):
             assert K.gemm_plan(*shape, with_workspace=True) == (DMA, 128, 64, 1), shape
             assert _lib.load().fmsmo_gemm_workspace_bytes(*shape) == 0
         # long reductions and half-filled rounds of longer ones keep the slices
