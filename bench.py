@@ -107,6 +107,18 @@ def cpu_baseline(torch, layers, budget_s=30.0):
                                          f"{rows} tokens and linears, median of 3 passes, {t_fp[1]:.2f} s each"}
     return res
 
+def gemm_sources_sha16():
+    """Names the GEMM kernel sources a counter profile belongs to."""
+    import hashlib
+
+    h = hashlib.sha256()
+    csrc = os.path.join(ROOT, "fms-model-optimizer_amd", "csrc")
+    for name in ("common.hpp", "gemm_tile.hpp", "gemm_rs.hpp", "gemm_launch.hpp", "gemm.hip"):
+        with open(os.path.join(csrc, name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
 GRANITE_8B = [("qkv", 4096, 6144), ("o", 4096, 4096), ("gate_up", 4096, 25600), ("down", 12800, 4096)]
 
 
@@ -137,7 +149,7 @@ def fp8_rooflines(torch, K, dev):
     clk = torch.zeros(6, dtype=torch.int64, device=dev)
     for label, M, shapes, per_channel in (("llama3_8b_M4096", M_TOKENS, LLAMA3_8B, True),
                                           ("granite_8b_M2048", 2048, GRANITE_8B, False)):
-        per, tot_ms, tot_ops = {}, 0.0, 0.0
+        per, tot_ms, tot_ops, vend = {}, 0.0, 0.0, {}
         for name, k, n in shapes:
             x = torch.randn(M, k, generator=g).bfloat16().to(dev)
             w = (0.02 * torch.randn(n, k, generator=g)).to(dev)
@@ -153,9 +165,28 @@ def fp8_rooflines(torch, K, dev):
             tf = ops / (ms * 1e-3) / 1e12
             per[name] = {"ms": round(ms, 4), "tflops": round(tf, 1), "frac": round(tf / PEAK_FP8_TFLOPS, 4),
                          "core_clock_mhz": round(K.core_clock_mhz(clk))}
+            # the vendor library on the SAME codes, same event timing, same run: torch._scaled_mm
+            # (hipBLASLt), what the reference's FP8Linear calls on a GPU
+            # (fms_mo/aiu_addons/fp8/fp8_linear.py:275-283), with row-wise scales (per token x per
+            # channel, this kernel's epilogue) and with one scale per tensor
+            sa_row = s.reshape(-1, 1).contiguous()
+            sb_row = (ws if per_channel else ws.expand(n)).reshape(1, -1).contiguous()
+            one = torch.ones((), device=dev)
+            for vlabel, sa, sb in (("vendor_scaled_mm_rowwise", sa_row, sb_row), ("vendor_scaled_mm_tensorwise", one, one)):
+                try:
+                    vms = time_events(torch, lambda: torch._scaled_mm(q, w8.t(), scale_a=sa, scale_b=sb,
+                                                                       out_dtype=torch.bfloat16), iters=20, warm=4)
+                    per[name][vlabel] = {"ms": round(vms, 4), "tflops": round(ops / (vms * 1e-3) / 1e12, 1)}
+                    vend[vlabel] = vend.get(vlabel, 0.0) + vms
+                except Exception as e:  # the vendor path is evidence, not a dependency
+                    per[name][vlabel] = {"error": str(e)[:160]}
+                    vend[vlabel] = float("nan")
             del x, w, w8, q
         tf = tot_ops / (tot_ms * 1e-3) / 1e12
         out[label] = {"per_shape": per, "achieved": round(tf, 1), "frac": round(tf / PEAK_FP8_TFLOPS, 4)}
+        for vlabel, vms in vend.items():
+            if vms == vms:
+                out[label][vlabel + "_tflops"] = round(tot_ops / (vms * 1e-3) / 1e12, 1)
     return out
 
 
@@ -337,11 +368,20 @@ def main():
     # power cap lets the clock settle, so the peak at the measured clock is reported beside it.
     mhz = [K.core_clock_mhz(c) for c in clk]
     peak_at_clock = sum(gemm_ops) / sum(o / (PEAK_INT8_TOPS * m / 2400.0) for o, m in zip(gemm_ops, mhz))
-    traffic = None
+    # HBM traffic per launch is a counter figure (two rocprofv3 --pmc runs of this command), not
+    # something this process can measure: it is read from the committed profile and reported only
+    # while the GEMM sources are the ones that profile was collected with
+    traffic, traffic_source = None, None
     tfile = os.path.join(ROOT, "profiles", "gemm_i8_traffic.json")
     if os.path.exists(tfile):
         with open(tfile) as f:
-            traffic = json.load(f).get("hbm_bytes_per_launch_avg")
+            tj = json.load(f)
+        if tj.get("gemm_sources_sha16") == gemm_sources_sha16():
+            traffic = tj.get("hbm_bytes_per_launch_avg")
+            traffic_source = "profiles/gemm_i8_traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of " \
+                             "this command; GEMM sources unchanged since: sha16 " + tj["gemm_sources_sha16"] + ")"
+        else:
+            traffic_source = "profiles/gemm_i8_traffic.json is older than the GEMM sources: not reported"
 
     out = {
         "metric": "W8A8 INT8 linear (SmoothQuant act-quant + int8 MFMA GEMM + dequant) throughput, "
@@ -355,7 +395,7 @@ def main():
                    "tokens": M_TOKENS},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_INT8_TOPS,
                      "unit": "TFLOP/s", "frac": round(achieved / PEAK_INT8_TOPS, 4),
-                     "traffic": traffic, "kernel": "gemm_rs_kernel<int8, dequant epilogue> (4 launches per step)",
+                     "traffic": traffic, "traffic_source": traffic_source, "kernel": "gemm_rs_kernel<int8, dequant epilogue> (4 launches per step)",
                      "per_shape_tops": per_shape,
                      "avg_launch_ms": {n: round(ms, 4) for (n, _, _), ms in zip(LLAMA3_8B, gemm_ms)},
                      "core_clock_mhz": {n: round(m) for (n, _, _), m in zip(LLAMA3_8B, mhz)},

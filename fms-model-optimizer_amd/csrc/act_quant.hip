@@ -935,10 +935,39 @@ __global__ __launch_bounds__(256) void quant_i8_affine_t_kernel(
 }
 
 // ------------------------------------------------------------------ e4m3, per token
+// Dynamic scale from an abs-max (a value of x's dtype XT): max(amax / 448, floor), formed in
+// fp32 or -- in_xt -- with quotient and floor both rounded to XT (a python-scalar clamp bound
+// leaves a tensor in its dtype, so the bound acts as its rounded value).
+template <int XT>
+__device__ __forceinline__ float fp8_dynamic_scale(float amax, float floor_v, int in_xt) {
+  if (in_xt) return fmaxf(round_to<XT>(amax / 448.0f), round_to<XT>(floor_v));
+  return fmaxf(amax / 448.0f, floor_v);
+}
+
+// scale[0] <- dynamic per-tensor scale from the per-column abs-max vector (one block).
+template <int XT>
+__global__ __launch_bounds__(AQ_THREADS) void fp8_tensor_scale_kernel(
+    const float* __restrict__ col_amax, int K, float scale_floor, int scale_in_xt,
+    float* __restrict__ scale) {
+  __shared__ float red[AQ_THREADS / 64];
+  // NaN abs-max entries order above inf as unsigned bit patterns, like torch's amax propagates them
+  uint32_t b = 0;
+  for (int k = threadIdx.x; k < K; k += AQ_THREADS) b = max(b, __float_as_uint(col_amax[k]));
+  b = wave_max_u32(b);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = __uint_as_float(b);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    uint32_t m = 0;
+    for (int w = 0; w < AQ_THREADS / 64; ++w) m = max(m, __float_as_uint(red[w]));
+    scale[0] = fp8_dynamic_scale<XT>(__uint_as_float(m), scale_floor, scale_in_xt);
+  }
+}
+
 template <int XT>
 __global__ __launch_bounds__(AQ_THREADS) void quant_fp8_pertoken_kernel(
     const void* __restrict__ x, int64_t ldx, int variant, int static_scale,
-    uint8_t* __restrict__ q, int64_t ldq, float* __restrict__ scale, int K) {
+    uint8_t* __restrict__ q, int64_t ldq, float* __restrict__ scale, int K, float scale_floor,
+    int scale_in_xt) {
   __shared__ float red[AQ_THREADS / 64];
   const int row = blockIdx.x;
   const size_t xrow = (size_t)row * ldx;
@@ -965,13 +994,7 @@ __global__ __launch_bounds__(AQ_THREADS) void quant_fp8_pertoken_kernel(
       for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(e[j]));
     }
     amax = block_max(amax, red);
-    if (variant == FMSMO_FP8_LINEAR) {
-      s = fmaxf(amax / 448.0f, 1e-12f);
-    } else {
-      // (amax / 448) in x's dtype, then clamp(min=1e-5): the clamp bound is a python scalar,
-      // so the result stays in x's dtype -> max against 1e-5 rounded to that dtype
-      s = fmaxf(round_to<XT>(amax / 448.0f), round_to<XT>(1e-5f));
-    }
+    s = fp8_dynamic_scale<XT>(amax, scale_floor, scale_in_xt);
     if (threadIdx.x == 0) scale[row] = s;
   }
   auto emit = [&](int c, const float (&e)[8]) {
@@ -1013,11 +1036,15 @@ __global__ __launch_bounds__(AQ_THREADS) void quant_fp8_pertoken_kernel(
 template <int XT, int NCH>
 __global__ __launch_bounds__(AQ_THREADS) void quant_fp8_pertoken16_kernel(
     const u16* __restrict__ x, int64_t ldx, int variant, uint8_t* __restrict__ q, int64_t ldq,
-    float* __restrict__ scale, int M, int K) {
+    float* __restrict__ scale, int M, int K, float scale_floor, int scale_in_xt,
+    int fixed_scale) {
   __shared__ float red[2][AQ_THREADS / 64];
   const int nchunk = K / AQ_VEC;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   constexpr uint32_t INF_BITS = XT == FMSMO_F16 ? 0x7c00u : 0x7f80u;
+  // fixed_scale: one scale for every row, read from scale[0] (nothing is written there); the row
+  // maximum still decides between the fast quotients and the IEEE route of non-finite rows
+  const float s_fixed = fixed_scale ? scale[0] : 0.0f;
 
   v4i cur[NCH], nxt[NCH];
   auto load_row = [&](int row, v4i (&dst)[NCH]) {
@@ -1031,7 +1058,6 @@ __global__ __launch_bounds__(AQ_THREADS) void quant_fp8_pertoken16_kernel(
   int parity = 0;
   int row = blockIdx.x;
   if (row < M) load_row(row, cur);
-  const float floor_X = cvt16<XT>(to16<XT>(1e-5f));
   for (; row < M; row += gridDim.x) {
     const int nrow = row + gridDim.x;
     if (nrow < M) load_row(nrow, nxt);
@@ -1059,13 +1085,17 @@ __global__ __launch_bounds__(AQ_THREADS) void quant_fp8_pertoken16_kernel(
                                max(__float_as_uint(rb[2]), __float_as_uint(rb[3])));
     const float amax = cvt16<XT>((u16)abits);
 
-    float s;
-    if (variant == FMSMO_FP8_LINEAR) s = fmaxf(amax / 448.0f, 1e-12f);
-    else s = fmaxf(cvt16<XT>(to16<XT>(amax / 448.0f)), floor_X);
-    if (threadIdx.x == 0) scale[row] = s;
+    float s = s_fixed;
+    if (!fixed_scale) {
+      s = fp8_dynamic_scale<XT>(amax, scale_floor, scale_in_xt);
+      if (threadIdx.x == 0) scale[row] = s;
+    }
     uint8_t* qr = q + (size_t)row * ldq;
 
-    if (abits < INF_BITS) {
+    // a fixed scale outside the range where the refined reciprocal is exact takes the IEEE route
+    const bool fast = abits < INF_BITS &&
+                      (!fixed_scale || (s >= 0x1p-60f && s <= 0x1p60f && amax <= s * 0x1p100f));
+    if (fast) {
       const float r1 = rcp_refined(s);
       const bool dl8 = variant == FMSMO_FP8_FPXACC_DL8;
 #pragma unroll
@@ -1376,17 +1406,18 @@ extern "C" int fmsmo_quant_i8_affine(const void* x, int x_dtype, int64_t ldx, in
   return fmsmo_check_launch();
 }
 
-extern "C" int fmsmo_quant_act_fp8_pertoken(const void* x, int x_dtype, int64_t ldx, int variant,
-                                            int static_scale, uint8_t* q, int64_t ldq,
-                                            float* scale, int64_t M, int64_t K,
-                                            fmsmo_stream_t stream) {
-  if (!x || !q || !scale) return FMSMO_ERR_NULL;
-  if (M < 0 || K <= 0 || ldx < K || ldq < K || M > 0x7fffffff || K > 0x7fffffff) return FMSMO_ERR_SHAPE;
-  if (x_dtype < 0 || x_dtype > 2 || variant < 0 || variant > 2) return FMSMO_ERR_UNSUPPORTED;
-  if (K % 8 || ldx % 8 || ldq % 8 || !aligned16(x) || (((uintptr_t)q) & 7)) return FMSMO_ERR_ALIGN;
-  if (M == 0) return FMSMO_OK;
-  hipStream_t st = (hipStream_t)stream;
-  if (x_dtype != FMSMO_F32 && !static_scale && K <= AQ_MAXCHUNK * AQ_THREADS * AQ_VEC) {
+// Shared launcher of the e4m3 quantizer entry points.  scale_mode: 0 one dynamic scale per row
+// (written to scale[M]); 1 scale[0] given by the caller, any value; 2 scale[0] is a dynamic
+// per-tensor scale that fp8_tensor_scale_kernel has left there (a value the variant's own rule
+// produces from the tensor's abs-max, so no quotient exceeds the e4m3 range).
+static int launch_quant_fp8(const void* x, int x_dtype, int64_t ldx, int variant, int scale_mode,
+                            float scale_floor, int scale_in_xt, uint8_t* q, int64_t ldq,
+                            float* scale, int64_t M, int64_t K, hipStream_t st) {
+  // the row-walking kernel clamps to +-448 before the hardware conversion: right for the
+  // FP8Linear recipe with any scale, and for the unclamped FPx recipe when the scale comes from
+  // the data's own maximum
+  const bool walk_ok = scale_mode == 0 || scale_mode == 2 || variant == FMSMO_FP8_LINEAR;
+  if (x_dtype != FMSMO_F32 && walk_ok && K <= AQ_MAXCHUNK * AQ_THREADS * AQ_VEC) {
     const int64_t per_thread = div_up(K, AQ_THREADS * AQ_VEC);
     dim3 block16(AQ_THREADS);
 #define LAUNCH8(XT, NCH)                                                                          \
@@ -1394,7 +1425,8 @@ extern "C" int fmsmo_quant_act_fp8_pertoken(const void* x, int x_dtype, int64_t 
     const int64_t resident = resident_blocks((const void*)quant_fp8_pertoken16_kernel<XT, NCH>);  \
     dim3 grid16((unsigned)(M < resident ? M : resident));                                         \
     hipLaunchKernelGGL((quant_fp8_pertoken16_kernel<XT, NCH>), grid16, block16, 0, st,            \
-                       (const u16*)x, ldx, variant, q, ldq, scale, (int)M, (int)K);               \
+                       (const u16*)x, ldx, variant, q, ldq, scale, (int)M, (int)K, scale_floor,   \
+                       scale_in_xt, scale_mode != 0);                                             \
   }
 #define PICK8(XT)                                  \
   if (per_thread <= 1) LAUNCH8(XT, 1)              \
@@ -1409,7 +1441,7 @@ extern "C" int fmsmo_quant_act_fp8_pertoken(const void* x, int x_dtype, int64_t 
   dim3 grid((unsigned)M), block(AQ_THREADS);
 #define LAUNCH(XT)                                                                             \
   hipLaunchKernelGGL((quant_fp8_pertoken_kernel<XT>), grid, block, 0, st, x, ldx, variant,     \
-                     static_scale, q, ldq, scale, (int)K)
+                     (int)(scale_mode != 0), q, ldq, scale, (int)K, scale_floor, scale_in_xt)
   switch (x_dtype) {
     case FMSMO_F16: LAUNCH(FMSMO_F16); break;
     case FMSMO_BF16: LAUNCH(FMSMO_BF16); break;
@@ -1417,4 +1449,56 @@ extern "C" int fmsmo_quant_act_fp8_pertoken(const void* x, int x_dtype, int64_t 
   }
 #undef LAUNCH
   return fmsmo_check_launch();
+}
+
+static int check_quant_fp8(const void* x, int x_dtype, int64_t ldx, int variant, const uint8_t* q,
+                           int64_t ldq, const float* scale, int64_t M, int64_t K) {
+  if (!x || !q || !scale) return FMSMO_ERR_NULL;
+  if (M < 0 || K <= 0 || ldx < K || ldq < K || M > 0x7fffffff || K > 0x7fffffff) return FMSMO_ERR_SHAPE;
+  if (x_dtype < 0 || x_dtype > 2 || variant < 0 || variant > 2) return FMSMO_ERR_UNSUPPORTED;
+  if (K % 8 || ldx % 8 || ldq % 8 || !aligned16(x) || (((uintptr_t)q) & 7)) return FMSMO_ERR_ALIGN;
+  return FMSMO_OK;
+}
+
+extern "C" int fmsmo_quant_act_fp8_pertoken(const void* x, int x_dtype, int64_t ldx, int variant,
+                                            int static_scale, uint8_t* q, int64_t ldq,
+                                            float* scale, int64_t M, int64_t K,
+                                            fmsmo_stream_t stream) {
+  if (const int e = check_quant_fp8(x, x_dtype, ldx, variant, q, ldq, scale, M, K)) return e;
+  if (M == 0) return FMSMO_OK;
+  // the rule each variant's reference states: fp32 amax / 448 floored at 1e-12 for the FP8Linear
+  // recipe, the quotient in x's dtype floored at 1e-5 for the FPx recipes
+  const bool lin = variant == FMSMO_FP8_LINEAR;
+  return launch_quant_fp8(x, x_dtype, ldx, variant, static_scale ? 1 : 0, lin ? 1e-12f : 1e-5f,
+                          lin ? 0 : 1, q, ldq, scale, M, K, (hipStream_t)stream);
+}
+
+extern "C" int fmsmo_quant_act_fp8_dynamic(const void* x, int x_dtype, int64_t ldx, int variant,
+                                           int per_tensor, const float* col_amax,
+                                           float scale_floor, int scale_dtype, uint8_t* q,
+                                           int64_t ldq, float* scale, int64_t M, int64_t K,
+                                           fmsmo_stream_t stream) {
+  if (const int e = check_quant_fp8(x, x_dtype, ldx, variant, q, ldq, scale, M, K)) return e;
+  if (per_tensor && !col_amax) return FMSMO_ERR_NULL;
+  if (scale_dtype != FMSMO_F32 && scale_dtype != x_dtype) return FMSMO_ERR_UNSUPPORTED;
+  if (!(scale_floor > 0.0f) || !(scale_floor < 0x1p60f)) return FMSMO_ERR_UNSUPPORTED;
+  // a floor that rounds to zero in x's dtype would let a zero row divide by zero
+  if (scale_dtype == FMSMO_F16 && scale_floor <= 0x1p-25f) return FMSMO_ERR_UNSUPPORTED;
+  if (scale_dtype == FMSMO_BF16 && scale_floor < 0x1p-126f) return FMSMO_ERR_UNSUPPORTED;
+  if (M == 0) return FMSMO_OK;
+  hipStream_t st = (hipStream_t)stream;
+  const int in_xt = scale_dtype != FMSMO_F32;
+  if (per_tensor) {
+#define LAUNCH(XT)                                                                            \
+  hipLaunchKernelGGL((fp8_tensor_scale_kernel<XT>), dim3(1), dim3(AQ_THREADS), 0, st, col_amax, \
+                     (int)K, scale_floor, in_xt, scale)
+    switch (x_dtype) {
+      case FMSMO_F16: LAUNCH(FMSMO_F16); break;
+      case FMSMO_BF16: LAUNCH(FMSMO_BF16); break;
+      default: LAUNCH(FMSMO_F32); break;
+    }
+#undef LAUNCH
+  }
+  return launch_quant_fp8(x, x_dtype, ldx, variant, per_tensor ? 2 : 0, scale_floor, in_xt, q, ldq,
+                          scale, M, K, st);
 }

@@ -29,8 +29,76 @@ struct ChunkArgs {
   int chunk_bytes;
   int trun_bits, max_acc_bits, dl16, tta;
   const void* c_in;
-  void* d;
-  int64_t ldd;
+  int64_t ldc;  // row stride of c_in (elements)
+};
+
+// What happens to a finished accumulator element.  One functor type per accumulator type with the
+// mode, the output dtype and the bias dtype as run-time fields: the switch is on wave-uniform
+// values in a 64-element epilogue behind a K loop of thousands of MFMAs, and it keeps the number
+// of instantiations of the pipelined kernel (operand types x interleaving schedules) unchanged.
+//   CHUNK_EPI_RAW        d[m,n] = acc                                  (int32 / fp32 out)
+//   FMSMO_EPI_REF_F16    f16( f32(acc) * f16(as ws) + b )              (iaddmm_int's plain branch)
+//   FMSMO_EPI_F32        fma( f32(acc), as ws, b )
+//   FMSMO_EPI_F32_MULADD ( f32(acc) * (as ws) ) + b, every step rounded (iaddmm_int's chunk loop)
+//   FMSMO_EPI_SEQ_OUT    T( T( (f32(acc) * as) * ws ) + T(b) ), T = output dtype
+//                        (LinearFuncFPxFwdBwd / LinearFuncINT8FwdFP32Bwd: descale, cast, add bias)
+enum { CHUNK_EPI_RAW = -1 };
+template <class AccT>
+struct EpiChunk {
+  static constexpr bool UNIFORM_ROWS = false;
+  void* y;
+  int64_t ldy;
+  const float* a_scale;
+  const float* w_scale;
+  const void* bias;
+  int a_stride, w_stride;
+  int mode, out_dt, bias_dt;
+  struct Col {
+    float ws, b;
+  };
+  struct Row {
+    float as;
+  };
+  __device__ __forceinline__ float to_out_grid(float v) const {
+    return out_dt == FMSMO_F16 ? round_to<FMSMO_F16>(v) : out_dt == FMSMO_BF16 ? round_to<FMSMO_BF16>(v) : v;
+  }
+  __device__ __forceinline__ Col col(int n, int, int) const {
+    Col c{1.0f, -0.0f};
+    if (mode == CHUNK_EPI_RAW) return c;
+    c.ws = w_scale[w_stride ? n : 0];
+    if (bias) {
+      c.b = bias_dt == FMSMO_F16 ? load_as_f32<FMSMO_F16>(bias, n)
+            : bias_dt == FMSMO_BF16 ? load_as_f32<FMSMO_BF16>(bias, n) : load_as_f32<FMSMO_F32>(bias, n);
+      if (mode == FMSMO_EPI_SEQ_OUT) c.b = to_out_grid(c.b);
+    }
+    return c;
+  }
+  __device__ __forceinline__ Row row(int m) const {
+    return Row{mode == CHUNK_EPI_RAW ? 1.0f : a_scale[a_stride ? m : 0]};
+  }
+  __device__ __forceinline__ void store(int m, int n, AccT v, Row r, Col c) const {
+    const int64_t idx = (int64_t)m * ldy + n;
+    if (mode == CHUNK_EPI_RAW) {
+      ((AccT*)y)[idx] = v;
+      return;
+    }
+    float t;
+    if (mode == FMSMO_EPI_REF_F16) {
+      const float sc = round_to<FMSMO_F16>(__fmul_rn(r.as, c.ws));
+      t = __fadd_rn(__fmul_rn((float)v, sc), c.b);
+      if (out_dt != FMSMO_F32) t = round_to<FMSMO_F16>(t);  // the fp16 accumulator dtype, then the output dtype
+    } else if (mode == FMSMO_EPI_F32) {
+      t = __fmaf_rn((float)v, __fmul_rn(r.as, c.ws), c.b);
+    } else if (mode == FMSMO_EPI_F32_MULADD) {
+      t = __fadd_rn(__fmul_rn((float)v, __fmul_rn(r.as, c.ws)), c.b);
+    } else {
+      t = to_out_grid(__fmul_rn(__fmul_rn((float)v, r.as), c.ws));
+      if (bias) t = __fadd_rn(t, c.b);
+    }
+    if (out_dt == FMSMO_F16) store_from_f32<FMSMO_F16>(y, idx, t);
+    else if (out_dt == FMSMO_BF16) store_from_f32<FMSMO_BF16>(y, idx, t);
+    else ((float*)y)[idx] = t;
+  }
 };
 
 template <int OP>
@@ -91,7 +159,7 @@ struct ChunkMma<FMSMO_OP_F32> {
 };
 
 template <int OP>
-__global__ __launch_bounds__(256) void chunk_matmul_kernel(ChunkArgs g) {
+__global__ __launch_bounds__(256) void chunk_matmul_kernel(ChunkArgs g, EpiChunk<typename ChunkMma<OP>::Elem> epi) {
   typedef ChunkMma<OP> MM;
   typedef typename MM::Acc Acc;
   typedef typename MM::Elem Elem;
@@ -140,7 +208,7 @@ __global__ __launch_bounds__(256) void chunk_matmul_kernel(ChunkArgs g) {
         if (g.c_in) {
           const int m = row0 + wm * 64 + i * 32 + (v >> 2) * 8 + fg * 4 + (v & 3);
           const int n = col0 + wn * 64 + j * 32 + fr;
-          if (m < g.M && n < g.N) init = ((const Elem*)g.c_in)[(int64_t)m * g.ldd + n];
+          if (m < g.M && n < g.N) init = ((const Elem*)g.c_in)[(int64_t)m * g.ldc + n];
         }
         acc[i][j][v] = init;
       }
@@ -220,10 +288,11 @@ __global__ __launch_bounds__(256) void chunk_matmul_kernel(ChunkArgs g) {
     for (int v = 0; v < 16; ++v) {
       const int m = row0 + wm * 64 + i * 32 + (v >> 2) * 8 + fg * 4 + (v & 3);
       if (m < g.M) {
+        const auto rowctx = epi.row(m);
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
           const int n = col0 + wn * 64 + j * 32 + fr;
-          if (n < g.N) ((Elem*)g.d)[(int64_t)m * g.ldd + n] = acc[i][j][v];
+          if (n < g.N) epi.store(m, n, acc[i][j][v], rowctx, epi.col(n, 0, g.N));
         }
       }
     }
@@ -255,7 +324,7 @@ static bool launch_chunk_tile(const ChunkArgs& c, const Epi& epi, hipStream_t st
   k.lo = c.max_acc_bits < 32 ? -(1 << (c.max_acc_bits - 1)) : (int)0x80000000;
   k.hi = c.max_acc_bits < 32 ? (1 << (c.max_acc_bits - 1)) - 1 : 0x7fffffff;
   k.post = c.dl16 || k.t > 0 || c.max_acc_bits < 32;
-  k.dl16 = c.dl16; k.tta = c.tta; k.c_in = c.c_in; k.ldc = c.ldd;
+  k.dl16 = c.dl16; k.tta = c.tta; k.c_in = c.c_in; k.ldc = c.ldc;
   dim3 grid((unsigned)(g.grid_m * g.grid_n)), block(256);
   // the schedules that round one block while the matrix unit multiplies the others: a chunk of one
   // 64-byte stage (every operand type), of several stages or of one 32-byte k-step (int8)
@@ -303,6 +372,52 @@ static int check_chunk(const void* a, int64_t lda, const void* b, int64_t ldb, c
   return FMSMO_OK;
 }
 
+static int check_chunk_dq(const float* a_scale, int64_t a_scale_n, const float* w_scale,
+                          int64_t w_scale_n, const void* bias, int bias_dtype, int epilogue,
+                          int y_dtype, int64_t M, int64_t N) {
+  if (!a_scale || !w_scale) return FMSMO_ERR_NULL;
+  if ((a_scale_n != 1 && a_scale_n != M) || (w_scale_n != 1 && w_scale_n != N)) return FMSMO_ERR_SHAPE;
+  if (y_dtype < 0 || y_dtype > 2 || (bias && (bias_dtype < 0 || bias_dtype > 2))) return FMSMO_ERR_UNSUPPORTED;
+  if (epilogue < FMSMO_EPI_REF_F16 || epilogue > FMSMO_EPI_SEQ_OUT) return FMSMO_ERR_UNSUPPORTED;
+  return FMSMO_OK;
+}
+
+static int run_chunk_i8(const ChunkArgs& g, const EpiChunk<int>& epi, hipStream_t st) {
+  if (launch_chunk_tile<MMA_I8>(g, epi, st)) return fmsmo_check_launch();
+  dim3 grid(div_up(g.N, 128), div_up(g.M, 128));
+  hipLaunchKernelGGL((chunk_matmul_kernel<FMSMO_OP_I8>), grid, dim3(256), 0, st, g, epi);
+  return fmsmo_check_launch();
+}
+
+static int run_chunk_fp(int op_dtype, const ChunkArgs& g, const EpiChunk<float>& epi, hipStream_t st) {
+  const bool done = op_dtype == FMSMO_OP_E4M3 ? launch_chunk_tile<MMA_FP8_K32>(g, epi, st)
+                    : op_dtype == FMSMO_OP_F16 ? launch_chunk_tile<MMA_F16>(g, epi, st)
+                    : op_dtype == FMSMO_OP_BF16 ? launch_chunk_tile<MMA_BF16>(g, epi, st)
+                                                : launch_chunk_tile<MMA_F32>(g, epi, st);
+  if (done) return fmsmo_check_launch();
+  dim3 grid(div_up(g.N, 128), div_up(g.M, 128));
+  if (op_dtype == FMSMO_OP_E4M3)
+    hipLaunchKernelGGL((chunk_matmul_kernel<FMSMO_OP_E4M3>), grid, dim3(256), 0, st, g, epi);
+  else if (op_dtype == FMSMO_OP_F16)
+    hipLaunchKernelGGL((chunk_matmul_kernel<FMSMO_OP_F16>), grid, dim3(256), 0, st, g, epi);
+  else if (op_dtype == FMSMO_OP_F32)
+    hipLaunchKernelGGL((chunk_matmul_kernel<FMSMO_OP_F32>), grid, dim3(256), 0, st, g, epi);
+  else
+    hipLaunchKernelGGL((chunk_matmul_kernel<FMSMO_OP_BF16>), grid, dim3(256), 0, st, g, epi);
+  return fmsmo_check_launch();
+}
+
+static ChunkArgs chunk_args_i8(const int8_t* a, int64_t lda, const int8_t* b, int64_t ldb, int64_t M,
+                               int64_t N, int64_t K, int chunk_size, int chunk_trun_bits,
+                               int max_acc_bits, int tta, const void* c_in, int64_t ldc) {
+  ChunkArgs g{};
+  g.a = (const uint8_t*)a; g.b = (const uint8_t*)b; g.lda = lda; g.ldb = ldb;
+  g.M = (int)M; g.N = (int)N; g.Kb = (int)K; g.chunk_bytes = chunk_size;
+  g.trun_bits = chunk_trun_bits; g.max_acc_bits = max_acc_bits; g.dl16 = 0;
+  g.tta = tta != 0; g.c_in = c_in; g.ldc = ldc;
+  return g;
+}
+
 extern "C" int fmsmo_matmul_chunk_i8(const int8_t* a, int64_t lda, const int8_t* b, int64_t ldb,
                                      const int32_t* c_in, int32_t* d, int64_t ldd, int64_t M,
                                      int64_t N, int64_t K, int chunk_size, int chunk_trun_bits,
@@ -317,22 +432,42 @@ extern "C" int fmsmo_matmul_chunk_i8(const int8_t* a, int64_t lda, const int8_t*
   // the plain int32 GEMM.
   if (chunk_trun_bits == 0 && max_acc_bits == 32 && !c_in)
     return fmsmo_gemm_i8_i32(a, lda, b, ldb, d, ldd, M, N, K, stream);
-  ChunkArgs g{};
-  g.a = (const uint8_t*)a; g.b = (const uint8_t*)b; g.lda = lda; g.ldb = ldb;
-  g.M = (int)M; g.N = (int)N; g.Kb = (int)K; g.chunk_bytes = chunk_size;
-  g.trun_bits = chunk_trun_bits; g.max_acc_bits = max_acc_bits; g.dl16 = 0;
-  g.tta = truncate_then_accumulate != 0; g.c_in = c_in; g.d = d; g.ldd = ldd;
-  if (launch_chunk_tile<MMA_I8>(g, EpiStoreI32{d, ldd}, (hipStream_t)stream)) return fmsmo_check_launch();
-  dim3 grid(div_up(N, 128), div_up(M, 128));
-  hipLaunchKernelGGL((chunk_matmul_kernel<FMSMO_OP_I8>), grid, dim3(256), 0, (hipStream_t)stream, g);
-  return fmsmo_check_launch();
+  const ChunkArgs g = chunk_args_i8(a, lda, b, ldb, M, N, K, chunk_size, chunk_trun_bits, max_acc_bits,
+                                    truncate_then_accumulate, c_in, ldd);
+  EpiChunk<int> epi{};
+  epi.y = d; epi.ldy = ldd; epi.mode = CHUNK_EPI_RAW;
+  return run_chunk_i8(g, epi, (hipStream_t)stream);
 }
 
-extern "C" int fmsmo_matmul_chunk_fp(const void* a, int64_t lda, const void* b, int64_t ldb,
-                                     int op_dtype, const float* c_in, float* d, int64_t ldd,
-                                     int64_t M, int64_t N, int64_t K, int chunk_size,
-                                     int chunk_trun_bits, int clamp_dl16,
-                                     int truncate_then_accumulate, fmsmo_stream_t stream) {
+extern "C" int fmsmo_matmul_chunk_i8_dq(const int8_t* a, int64_t lda, const int8_t* b, int64_t ldb,
+                                        const float* a_scale, int64_t a_scale_n,
+                                        const float* w_scale, int64_t w_scale_n, const void* bias,
+                                        int bias_dtype, int epilogue, void* y, int y_dtype,
+                                        int64_t ldy, int64_t M, int64_t N, int64_t K,
+                                        int chunk_size, int chunk_trun_bits, int max_acc_bits,
+                                        int truncate_then_accumulate, fmsmo_stream_t stream) {
+  int rc = check_chunk(a, lda, b, ldb, y, ldy, M, N, K, 1, chunk_size, 32);
+  if (rc) return rc;
+  rc = check_chunk_dq(a_scale, a_scale_n, w_scale, w_scale_n, bias, bias_dtype, epilogue, y_dtype, M, N);
+  if (rc) return rc;
+  if (chunk_trun_bits < 0 || chunk_trun_bits > 31 || max_acc_bits < 2 || max_acc_bits > 32)
+    return FMSMO_ERR_UNSUPPORTED;
+  if (M == 0) return FMSMO_OK;
+  // nothing to round or clamp: the plain int8 GEMM with the same epilogue, where it has it
+  if (chunk_trun_bits == 0 && max_acc_bits == 32 && epilogue != FMSMO_EPI_SEQ_OUT && K % 16 == 0)
+    return fmsmo_gemm_i8_dq(a, lda, b, ldb, a_scale, a_scale_n, w_scale, w_scale_n, bias, bias_dtype,
+                            epilogue, y, y_dtype, ldy, M, N, K, stream);
+  const ChunkArgs g = chunk_args_i8(a, lda, b, ldb, M, N, K, chunk_size, chunk_trun_bits, max_acc_bits,
+                                    truncate_then_accumulate, nullptr, 0);
+  EpiChunk<int> epi{y, ldy, a_scale, w_scale, bias, a_scale_n == 1 ? 0 : 1, w_scale_n == 1 ? 0 : 1,
+                    epilogue, y_dtype, bias ? bias_dtype : FMSMO_F32};
+  return run_chunk_i8(g, epi, (hipStream_t)stream);
+}
+
+static int chunk_args_fp(const void* a, int64_t lda, const void* b, int64_t ldb, int op_dtype,
+                         const void* d, int64_t ldd, int64_t M, int64_t N, int64_t K, int chunk_size,
+                         int chunk_trun_bits, int clamp_dl16, int tta, const void* c_in, int64_t ldc,
+                         ChunkArgs* out) {
   if (op_dtype != FMSMO_OP_E4M3 && op_dtype != FMSMO_OP_F16 && op_dtype != FMSMO_OP_BF16 &&
       op_dtype != FMSMO_OP_F32)
     return FMSMO_ERR_UNSUPPORTED;
@@ -340,29 +475,45 @@ extern "C" int fmsmo_matmul_chunk_fp(const void* a, int64_t lda, const void* b, 
   int rc = check_chunk(a, lda, b, ldb, d, ldd, M, N, K, esz, chunk_size, esz == 1 ? 32 : 16);
   if (rc) return rc;
   if (chunk_trun_bits < 0 || chunk_trun_bits > 22) return FMSMO_ERR_UNSUPPORTED;
-  if (M == 0) return FMSMO_OK;
   ChunkArgs g{};
   g.a = (const uint8_t*)a; g.b = (const uint8_t*)b; g.lda = lda * esz; g.ldb = ldb * esz;
   g.M = (int)M; g.N = (int)N; g.Kb = (int)(K * esz); g.chunk_bytes = chunk_size * esz;
   g.trun_bits = chunk_trun_bits; g.max_acc_bits = 32; g.dl16 = clamp_dl16 != 0;
-  g.tta = truncate_then_accumulate != 0; g.c_in = c_in; g.d = d; g.ldd = ldd;
-  hipStream_t st = (hipStream_t)stream;
-  {
-    const EpiStoreF32 epi{d, ldd};
-    const bool done = op_dtype == FMSMO_OP_E4M3 ? launch_chunk_tile<MMA_FP8_K32>(g, epi, st)
-                      : op_dtype == FMSMO_OP_F16 ? launch_chunk_tile<MMA_F16>(g, epi, st)
-                      : op_dtype == FMSMO_OP_BF16 ? launch_chunk_tile<MMA_BF16>(g, epi, st)
-                                                  : launch_chunk_tile<MMA_F32>(g, epi, st);
-    if (done) return fmsmo_check_launch();
-  }
-  dim3 grid(div_up(N, 128), div_up(M, 128));
-  if (op_dtype == FMSMO_OP_E4M3)
-    hipLaunchKernelGGL((chunk_matmul_kernel<FMSMO_OP_E4M3>), grid, dim3(256), 0, st, g);
-  else if (op_dtype == FMSMO_OP_F16)
-    hipLaunchKernelGGL((chunk_matmul_kernel<FMSMO_OP_F16>), grid, dim3(256), 0, st, g);
-  else if (op_dtype == FMSMO_OP_F32)
-    hipLaunchKernelGGL((chunk_matmul_kernel<FMSMO_OP_F32>), grid, dim3(256), 0, st, g);
-  else
-    hipLaunchKernelGGL((chunk_matmul_kernel<FMSMO_OP_BF16>), grid, dim3(256), 0, st, g);
-  return fmsmo_check_launch();
+  g.tta = tta != 0; g.c_in = c_in; g.ldc = ldc;
+  *out = g;
+  return FMSMO_OK;
+}
+
+extern "C" int fmsmo_matmul_chunk_fp(const void* a, int64_t lda, const void* b, int64_t ldb,
+                                     int op_dtype, const float* c_in, float* d, int64_t ldd,
+                                     int64_t M, int64_t N, int64_t K, int chunk_size,
+                                     int chunk_trun_bits, int clamp_dl16,
+                                     int truncate_then_accumulate, fmsmo_stream_t stream) {
+  ChunkArgs g{};
+  int rc = chunk_args_fp(a, lda, b, ldb, op_dtype, d, ldd, M, N, K, chunk_size, chunk_trun_bits,
+                         clamp_dl16, truncate_then_accumulate, c_in, ldd, &g);
+  if (rc) return rc;
+  if (M == 0) return FMSMO_OK;
+  EpiChunk<float> epi{};
+  epi.y = d; epi.ldy = ldd; epi.mode = CHUNK_EPI_RAW;
+  return run_chunk_fp(op_dtype, g, epi, (hipStream_t)stream);
+}
+
+extern "C" int fmsmo_matmul_chunk_fp_dq(const void* a, int64_t lda, const void* b, int64_t ldb,
+                                        int op_dtype, const float* a_scale, int64_t a_scale_n,
+                                        const float* w_scale, int64_t w_scale_n, const void* bias,
+                                        int bias_dtype, int epilogue, void* y, int y_dtype,
+                                        int64_t ldy, int64_t M, int64_t N, int64_t K,
+                                        int chunk_size, int chunk_trun_bits, int clamp_dl16,
+                                        int truncate_then_accumulate, fmsmo_stream_t stream) {
+  ChunkArgs g{};
+  int rc = chunk_args_fp(a, lda, b, ldb, op_dtype, y, ldy, M, N, K, chunk_size, chunk_trun_bits,
+                         clamp_dl16, truncate_then_accumulate, nullptr, 0, &g);
+  if (rc) return rc;
+  rc = check_chunk_dq(a_scale, a_scale_n, w_scale, w_scale_n, bias, bias_dtype, epilogue, y_dtype, M, N);
+  if (rc) return rc;
+  if (M == 0) return FMSMO_OK;
+  EpiChunk<float> epi{y, ldy, a_scale, w_scale, bias, a_scale_n == 1 ? 0 : 1, w_scale_n == 1 ? 0 : 1,
+                      epilogue, y_dtype, bias ? bias_dtype : FMSMO_F32};
+  return run_chunk_fp(op_dtype, g, epi, (hipStream_t)stream);
 }

@@ -164,8 +164,17 @@ extern "C" int fmsmo_gemm_i8_dq_noalloc(const int8_t* a, int64_t lda, const int8
                                         int bias_dtype, int epilogue, void* y, int y_dtype,
                                         int64_t ldy, int64_t M, int64_t N, int64_t K,
                                         fmsmo_stream_t stream) {
+  // arguments first: a rejected call touches nothing, not even the scratch lookup
+  int rc0 = check_gemm(a, lda, b, ldb, y, ldy, M, N, K);
+  if (rc0) return rc0;
+  rc0 = check_dq(a_scale, a_scale_n, w_scale, w_scale_n, bias, bias_dtype, y_dtype, M, N);
+  if (rc0) return rc0;
+  if (epilogue < FMSMO_EPI_REF_F16 || epilogue > FMSMO_EPI_F32_MULADD) return FMSMO_ERR_UNSUPPORTED;
+  if (M == 0) return FMSMO_OK;
+  // the weight-streaming decode kernels use no scratch
+  const bool decode = (M <= 16 && K % 128 == 0) || fmsmo_gemv_batch_ok(M, K);
   // (the plan that fits the scratch, if one does: else the preferred plan's size is reported)
-  int64_t need = (M > 0 && N > 0 && K > 0) ? plan_split_k(M, N, K, (int64_t)FMSMO_STATIC_SCRATCH_BYTES).ws_bytes : 0;
+  int64_t need = decode ? 0 : plan_split_k(M, N, K, (int64_t)FMSMO_STATIC_SCRATCH_BYTES).ws_bytes;
   if (need > (int64_t)FMSMO_STATIC_SCRATCH_BYTES) {
     snprintf(g_fmsmo_last_error, sizeof(g_fmsmo_last_error),
              "split-K partial sums of %lld x %lld x %lld need %lld bytes, the static scratch holds %lld",
@@ -212,7 +221,10 @@ extern "C" int fmsmo_gemm_plan(int64_t M, int64_t N, int64_t K, int with_workspa
     *tile_n = TileTallK::BN;
     return FMSMO_OK;
   }
-  const SplitPlan plan = plan_split_k(M, N, K);
+  const SplitPlan plan = with_workspace == 2 ? plan_split_k(M, N, K, (int64_t)FMSMO_STATIC_SCRATCH_BYTES)
+                                             : plan_split_k(M, N, K);
+  if (with_workspace == 2 && plan.ws_bytes > (int64_t)FMSMO_STATIC_SCRATCH_BYTES)
+    return FMSMO_ERR_SCRATCH;  // what the noalloc entry point returns for this shape
   if (with_workspace && plan.splits > 1) {
     *kernel = plan.rs ? FMSMO_PLAN_TILE_REGISTER_STAGED : FMSMO_PLAN_TILE_LDS_DMA;
     *tile_m = plan.rs ? 256 : TileMid::BM;

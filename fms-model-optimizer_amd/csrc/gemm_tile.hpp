@@ -40,6 +40,8 @@ struct GemmArgs {
   int64_t lda_e;       // uniform groups: bytes between groups in A (rows * lda for stacked batches,
                        // the K slice length when the groups are slices of one reduction)
   int k_rotate;  // register-staged kernel: block b starts its reduction at slab (b * k_rotate) % slabs
+  int skew;      // register-staged kernel: the blocks of the first round start (b / 8 % 8) * skew * 256
+                 // clock cycles late, so that the compute units do not all store their tiles at once
   // optional clock probe (register-staged kernel): block 0 stores {core clock counter, 100 MHz
   // wall clock} at its start, after its K loop and after its epilogue; null = off
   unsigned long long* clk;
@@ -230,9 +232,6 @@ __global__ __launch_bounds__(WGM* WGN * 64, (Chk::enabled && (OP == MMA_I8 || Ch
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / WGN, wn = wave % WGN;
 
-#ifdef FMSMO_CLK
-  if (blockIdx.x == 0 && tid == 0 && g.clk) { g.clk[0] = clock64(); g.clk[1] = wall_clock64(); }
-#endif
   int tile_m, tile_n;
   int row_lo = 0, row_hi = g.M, expert = 0;
   int64_t a_adj = 0;
@@ -415,9 +414,6 @@ __global__ __launch_bounds__(WGM* WGN * 64, (Chk::enabled && (OP == MMA_I8 || Ch
   };
 
   auto read_frags = [&](const uint8_t* ls, int s, Frag* af, Frag* bf) {
-#ifdef FMSMO_ABLATE_NO_LDSREAD
-    if (g.K > 0) return;
-#endif
 #pragma unroll
     for (int i = 0; i < FM; ++i) {
       if constexpr (CL == 1) {
@@ -440,9 +436,6 @@ __global__ __launch_bounds__(WGM* WGN * 64, (Chk::enabled && (OP == MMA_I8 || Ch
     }
   };
   auto mma_step = [&](const Frag* af, const Frag* bf) {
-#ifdef FMSMO_ABLATE_NO_MMA
-    if (g.K > 0) return;
-#endif
 #pragma unroll
     for (int i = 0; i < FM; ++i)
 #pragma unroll
@@ -516,9 +509,6 @@ __global__ __launch_bounds__(WGM* WGN * 64, (Chk::enabled && (OP == MMA_I8 || Ch
     const uint8_t* ls = &lds[0][0] + cur * STAGE_BYTES;
     auto dma = [&](auto s_c) {
       constexpr int S = decltype(s_c)::value;
-#ifdef FMSMO_ABLATE_NO_DMA
-      if (g.K < 0)
-#endif
       issue_part(fill, fill_k0, std::integral_constant<int, NLD * S / NKS>{},
                  std::integral_constant<int, NLD * (S + 1) / NKS>{});
     };
@@ -780,9 +770,6 @@ __global__ __launch_bounds__(WGM* WGN * 64, (Chk::enabled && (OP == MMA_I8 || Ch
     }
   }
 
-#ifdef FMSMO_CLK
-  if (blockIdx.x == 0 && tid == 0 && g.clk) { g.clk[2] = clock64(); g.clk[3] = wall_clock64(); }
-#endif
   // ---- epilogue: acc[i][j][v] is C(row, col) with
   //      row = 32 i + 8 (v / 4) + 4 (lane / 32) + v % 4,   col = 32 j + lane % 32
   const int m_base = row_lo + wm * TM + fg * 4;
@@ -820,9 +807,6 @@ __global__ __launch_bounds__(WGM* WGN * 64, (Chk::enabled && (OP == MMA_I8 || Ch
       }
     }
   }
-#ifdef FMSMO_CLK
-  if (blockIdx.x == 0 && tid == 0 && g.clk) { g.clk[4] = clock64(); g.clk[5] = wall_clock64(); }
-#endif
 #endif  // __HIP_DEVICE_COMPILE__
 }
 

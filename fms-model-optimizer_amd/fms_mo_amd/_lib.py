@@ -17,7 +17,7 @@ LIB_PATH = os.environ.get("FMSMO_LIB") or os.path.normpath(os.path.join(_HERE, "
 # dtype / enum codes of include/fmsmo_hip.h
 F16, BF16, F32 = 0, 1, 2
 OP_I8, OP_E4M3, OP_F16, OP_BF16, OP_F32 = 0, 1, 2, 3, 4
-EPI_REF_F16, EPI_F32, EPI_F32_MULADD = 0, 1, 2
+EPI_REF_F16, EPI_F32, EPI_F32_MULADD, EPI_SEQ_OUT = 0, 1, 2, 3
 SQ_RAW, SQ_FMO, SQ_U8_SHIFT, SQ_S8_NARROW = 0, 1, 2, 3
 DQ_PER_TENSOR, DQ_PER_COLUMN = 0, 1
 F8E_SAT, F8E_PER_TENSOR, F8E_PER_ROW = 0, 1, 2
@@ -38,6 +38,7 @@ SIGNATURES = {
     "fmsmo_fake_quant_fp8": [_P, _I, _L, _I, _P, _P, _L, _P, _L, _P, _P, _L, _L, _P],
     "fmsmo_quant_act_i8_mulscale": [_P, _I, _L, _P, _P, _I, _I, _I, _P, _L, _P, _L, _L, _P],
     "fmsmo_quant_act_fp8_pertoken": [_P, _I, _L, _I, _I, _P, _L, _P, _L, _L, _P],
+    "fmsmo_quant_act_fp8_dynamic": [_P, _I, _L, _I, _I, _P, _F, _I, _P, _L, _P, _L, _L, _P],
     "fmsmo_gemm_i8_i32": [_P, _L, _P, _L, _P, _L, _L, _L, _L, _P],
     "fmsmo_gemm_i8_i32_ws": [_P, _L, _P, _L, _P, _L, _L, _L, _L, _P, _L, _P],
     "fmsmo_gemm_i8_dq": [_P, _L, _P, _L, _P, _L, _P, _L, _P, _I, _I, _P, _I, _L, _L, _L, _L, _P],
@@ -51,6 +52,10 @@ SIGNATURES = {
     "fmsmo_decode_linear_fp8": [_P, _I, _L, _P, _L, _P, _L, _P, _I, _P, _I, _L, _P, _L, _L, _L, _P],
     "fmsmo_matmul_chunk_i8": [_P, _L, _P, _L, _P, _P, _L, _L, _L, _L, _I, _I, _I, _I, _P],
     "fmsmo_matmul_chunk_fp": [_P, _L, _P, _L, _I, _P, _P, _L, _L, _L, _L, _I, _I, _I, _I, _P],
+    "fmsmo_matmul_chunk_i8_dq": [_P, _L, _P, _L, _P, _L, _P, _L, _P, _I, _I, _P, _I, _L, _L, _L, _L,
+                                 _I, _I, _I, _I, _P],
+    "fmsmo_matmul_chunk_fp_dq": [_P, _L, _P, _L, _I, _P, _L, _P, _L, _P, _I, _I, _P, _I, _L, _L, _L, _L,
+                                 _I, _I, _I, _I, _P],
     "fmsmo_grouped_gemm_i8_dq": [_P, _L, _P, _L, _L, _P, _I, _L, _P, _P, _P, _I, _I, _P, _I, _L,
                                  _L, _L, _P],
     "fmsmo_quant_weight_i8": [_P, _I, _L, _P, _I, _P, _I, _L, _I, _P, _L, _P, _L, _L, _P],

@@ -185,6 +185,28 @@ def quant_act_fp8_pertoken(x, variant=L.FP8_LINEAR, static_scale=None):
     return q, scale
 
 
+def quant_act_fp8_dynamic(x, variant=L.FP8_LINEAR, per_tensor=False, scale_floor=1e-12,
+                          scale_in_x_dtype=False):
+    """(q e4m3 [M,K], scale fp32 [M] or [1]): the e4m3 quantizer with a dynamic scale
+    max(amax / 448, scale_floor) per token or for the whole tensor, the division in fp32 or in
+    x's dtype (see fmsmo_quant_act_fp8_dynamic).  Per tensor it is two passes over x (column
+    abs-max, quantizer) with nothing read back to the host."""
+    _need_gpu(x)
+    if x.dim() != 2:
+        raise ValueError("expected a 2-D tensor")
+    x = _rows(x)
+    M, K = x.shape
+    q = torch.empty((M, K), dtype=torch.float8_e4m3fn, device=x.device)
+    scale = torch.empty((1 if per_tensor else M,), dtype=torch.float32, device=x.device)
+    col_amax = absmax_cols(x) if per_tensor else None
+    with _dev(x):
+        L.call("fmsmo_quant_act_fp8_dynamic", x.data_ptr(), _dt(x), _ld(x), int(variant),
+               int(bool(per_tensor)), _ptr(col_amax), float(scale_floor),
+               _dt(x) if scale_in_x_dtype else L.F32, q.data_ptr(), K, scale.data_ptr(), M, K,
+               _stream(x))
+    return q, scale
+
+
 def quant_act_i8_static_t(x, mode, compute_dtype, scale, zp, sym=0, clip_lo=0.0, clip_hi=0.0):
     """int8 [M,K]: the static per-tensor formulas evaluated in ``compute_dtype`` (see
     fmsmo_quant_act_i8_static_t; mode is one of L.SQ_*).  All parameters are host numbers."""
@@ -199,11 +221,11 @@ def quant_act_i8_static_t(x, mode, compute_dtype, scale, zp, sym=0, clip_lo=0.0,
     return q
 
 
-def quant_act_i8_dynamic(x, per_column, levels, zp=0):
+def quant_act_i8_dynamic(x, per_column, levels, zp=0, want_amax=False):
     """(q int8 [M,K], scale fp32 [1] or [K]): dynamic symmetric quantizer with one scale for the
     whole tensor or one per column, abs-max / levels in x's dtype, codes shifted by zp (see
     fmsmo_quant_act_i8_dynamic).  Two passes over x: the column abs-max, then the quantizer; nothing
-    is read back to the host."""
+    is read back to the host.  want_amax: also return the fp32 [K] column abs-max."""
     _need_gpu(x)
     x = _rows(x)
     M, K = x.shape
@@ -214,7 +236,7 @@ def quant_act_i8_dynamic(x, per_column, levels, zp=0):
         L.call("fmsmo_quant_act_i8_dynamic", x.data_ptr(), _dt(x), _ld(x), col_amax.data_ptr(),
                L.DQ_PER_COLUMN if per_column else L.DQ_PER_TENSOR, int(levels), int(zp),
                q.data_ptr(), K, scale.data_ptr(), M, K, _stream(x))
-    return q, scale
+    return (q, scale, col_amax) if want_amax else (q, scale)
 
 
 def fake_quant_fp8(x, mode, want_values=True, want_codes=False):
@@ -440,6 +462,47 @@ def matmul_chunk(a, w, c=None, chunk_size=64, chunk_trun_bits=0, max_acc_bits=32
     return d
 
 
+def matmul_chunk_dq(a, w, a_scale, w_scale, bias=None, epilogue=L.EPI_SEQ_OUT, out_dtype=torch.float16,
+                    chunk_size=64, chunk_trun_bits=0, max_acc_bits=32, truncate_then_accumulate=True,
+                    clamp_acc_to_dl16=False):
+    """y [M,N] = epilogue(chunked accumulator of a [M,K] . w [N,K]^T): the chunk-truncate matmul and
+    its dequantization in one launch (see fmsmo_matmul_chunk_i8_dq / _fp_dq).  a_scale fp32 [M] or
+    [1], w_scale fp32 [N] or [1], bias [N] (fp16 / bf16 / fp32) or None, epilogue one of L.EPI_*."""
+    _need_gpu(a, w, a_scale, w_scale, bias)
+    if a.dtype != w.dtype or a.dtype not in _OPDT:
+        raise TypeError(f"unsupported operand dtypes {a.dtype}, {w.dtype}")
+    a, w = _rows(a), _rows(w)
+    M, K = a.shape
+    N = w.shape[0]
+    if w.shape[1] != K:
+        raise ValueError("K mismatch")
+    esz = a.element_size()
+    per16 = 16 // esz
+    if K % per16 or _ld(a) % per16 or _ld(w) % per16:  # zero-pad K: contributes nothing to any chunk
+        Kp = (K + 63) // 64 * 64
+        a = torch.nn.functional.pad(a.view(_BITS[esz]), (0, Kp - K)).view(a.dtype)
+        w = torch.nn.functional.pad(w.view(_BITS[esz]), (0, Kp - K)).view(w.dtype)
+        K = Kp
+    a_scale = _scale_vec(a_scale, M, a.device, "a_scale")
+    w_scale = _scale_vec(w_scale, N, a.device, "w_scale")
+    if bias is not None:
+        if bias.numel() != N or bias.dtype not in _DT:
+            raise ValueError("bias must hold N fp16 / bf16 / fp32 values")
+        bias = bias.reshape(-1).contiguous()
+    y = torch.empty((M, N), dtype=out_dtype, device=a.device)
+    common = (a_scale.data_ptr(), a_scale.numel(), w_scale.data_ptr(), w_scale.numel(), _ptr(bias),
+              _DT[bias.dtype] if bias is not None else L.F32, int(epilogue), y.data_ptr(), _DT[out_dtype],
+              N, M, N, K, int(chunk_size), int(chunk_trun_bits))
+    with _dev(a):
+        if a.dtype == torch.int8:
+            L.call("fmsmo_matmul_chunk_i8_dq", a.data_ptr(), _ld(a), w.data_ptr(), _ld(w), *common,
+                   int(max_acc_bits), int(bool(truncate_then_accumulate)), _stream(a))
+        else:
+            L.call("fmsmo_matmul_chunk_fp_dq", a.data_ptr(), _ld(a), w.data_ptr(), _ld(w), _OPDT[a.dtype],
+                   *common, int(bool(clamp_acc_to_dl16)), int(bool(truncate_then_accumulate)), _stream(a))
+    return y
+
+
 def quant_weight_i8(w, coef, smooth=None, mode="mul", want_row_sum=False):
     """Offline weight quantizer (see fmsmo_quant_weight_i8): w [N,K] fp16/bf16/fp32, coef [N] or [1]
     (``127 / clip_val`` for mode "mul", ``w_scale`` for mode "div"), smooth [K] or None.
@@ -577,6 +640,7 @@ _OPS = torch.library.Library("fms_mo_amd", "FRAGMENT")
 _quant_act_i8_pertoken_impl = quant_act_i8_pertoken
 _quant_act_i8_static_impl = quant_act_i8_static
 _quant_act_fp8_pertoken_impl = quant_act_fp8_pertoken
+_quant_act_fp8_dynamic_impl = quant_act_fp8_dynamic
 _gemm_i8_dq_impl = gemm_i8_dq
 _gemm_fp8_dq_impl = gemm_fp8_dq
 
@@ -613,6 +677,15 @@ _register(
         torch.empty(_rows_shape(x), dtype=torch.float8_e4m3fn, device=x.device),
         torch.empty((1 if static_scale is not None else x.shape[0],), dtype=torch.float32,
                     device=x.device)),
+)
+_register(
+    "quant_act_fp8_dynamic",
+    "(Tensor x, int variant, bool per_tensor, float scale_floor, bool scale_in_x_dtype) -> (Tensor, Tensor)",
+    lambda x, variant, per_tensor, scale_floor, scale_in_x_dtype: _quant_act_fp8_dynamic_impl(
+        x, variant, per_tensor, scale_floor, scale_in_x_dtype),
+    lambda x, variant, per_tensor, scale_floor, scale_in_x_dtype: (
+        torch.empty(_rows_shape(x), dtype=torch.float8_e4m3fn, device=x.device),
+        torch.empty((1 if per_tensor else x.shape[0],), dtype=torch.float32, device=x.device)),
 )
 _register(
     "gemm_i8_dq",
@@ -888,6 +961,19 @@ def quant_act_fp8_pertoken(x, variant=L.FP8_LINEAR, static_scale=None):  # noqa:
     if _eager(x, static_scale):
         return _quant_act_fp8_pertoken_impl(x, int(variant), static_scale)
     return torch.ops.fms_mo_amd.quant_act_fp8_pertoken(x, int(variant), static_scale)
+
+
+def quant_act_fp8_dynamic(x, variant=L.FP8_LINEAR, per_tensor=False, scale_floor=1e-12,  # noqa: F811
+                          scale_in_x_dtype=False):
+    """(q e4m3 [M,K], scale fp32 [M] or [1]), see fmsmo_quant_act_fp8_dynamic."""
+    _need_gpu(x)
+    if x.dim() != 2:
+        raise ValueError("expected a 2-D tensor")
+    if _eager(x):
+        return _quant_act_fp8_dynamic_impl(x, int(variant), bool(per_tensor), float(scale_floor),
+                                           bool(scale_in_x_dtype))
+    return torch.ops.fms_mo_amd.quant_act_fp8_dynamic(x, int(variant), bool(per_tensor),
+                                                      float(scale_floor), bool(scale_in_x_dtype))
 
 
 def gemm_i8_dq(a, w, a_scale, w_scale, bias=None, out_dtype=torch.float16, exact_ref=True,  # noqa: F811

@@ -12,8 +12,13 @@ Forward: activations are quantized with  q = e4m3(clamp(f32(x) / scale, +-448)) 
 per tensor, or dynamic = amax / 448 per token or per tensor), then one FP8 MFMA GEMM with fp32
 accumulation and the epilogue  y = out(acc * s_x[m] * s_w[n] + bias)  -- what the reference
 obtains from torch._scaled_mm through torchao's addmm_float8_unwrapped_inference (:275-283).
-The dynamic-scale rule inside torchao 0.11 is outside the reference tree; the rule used is the
-one of the reference's own test helper (tests/aiu_addons/test_fp8_addon.py:65-79).
+The dynamic-scale rule inside torchao 0.11 is outside the reference tree.  What the mathematics
+fixes is built in (the row maximum lands on the top code 448, the scale is fp32); the two
+properties only torchao's source fixes are module attributes: ``dynamic_scale_floor`` (lower
+clamp of the scale, default 1e-12 as in the reference's own test helper,
+tests/aiu_addons/test_fp8_addon.py:65-79) and ``dynamic_scale_in_input_dtype`` (False: the
+abs-max is widened to fp32 before the division by 448; True: the division runs in x's dtype and
+its result is widened).
 """
 from __future__ import annotations
 
@@ -25,6 +30,9 @@ from .. import kernels
 
 
 class FP8Linear(nn.Module):
+    dynamic_scale_floor = 1e-12
+    dynamic_scale_in_input_dtype = False
+
     def __init__(self, in_features: int, out_features: int, bias: bool, linear_config: dict):
         super().__init__()
         self.in_features = in_features
@@ -83,8 +91,12 @@ class FP8Linear(nn.Module):
                     raise NotImplementedError("static activation scales are per tensor")
                 q, s = kernels.quant_act_fp8_pertoken(x2, L.FP8_LINEAR, static_scale=self.input_scale.float())
             elif act["strategy"] == "tensor":
-                s_t = (x2.abs().amax().float() / 448.0).clamp(min=1e-12)
-                q, s = kernels.quant_act_fp8_pertoken(x2, L.FP8_LINEAR, static_scale=s_t)
+                # column abs-max and quantizer: two passes over x, the scale never leaves the device
+                q, s = kernels.quant_act_fp8_dynamic(x2, L.FP8_LINEAR, True, self.dynamic_scale_floor,
+                                                     self.dynamic_scale_in_input_dtype)
+            elif self.dynamic_scale_floor != 1e-12 or self.dynamic_scale_in_input_dtype:
+                q, s = kernels.quant_act_fp8_dynamic(x2, L.FP8_LINEAR, False, self.dynamic_scale_floor,
+                                                     self.dynamic_scale_in_input_dtype)
             elif kernels.decode_linear_ok(x2, None, x2.shape[1]):
                 # decode step of a few tokens: quantizer and weight-streaming matmul in one launch
                 y, _ = kernels.decode_linear_fp8(x2, self.weight, w_scale, bias, out_dtype=x.dtype)

@@ -170,7 +170,11 @@ class QLinear(nn.Linear):
         key = (a.data_ptr(), a._version, w.data_ptr(), w._version, x.dtype, x.device,
                (al.data_ptr(), al._version) if torch.is_tensor(al) else al)
         if self._sqcache is None or self._sqcache[0] != key:
-            scale = self.get_smoothq_scale(x)
+            # detached and built outside autograd: the cached tensor serves the kernel paths and
+            # no-grad evaluation only (forward() recomputes the scale inside the graph whenever a
+            # gradient can flow through it, as the reference does on every call)
+            with torch.no_grad():
+                scale = self.get_smoothq_scale(x).detach()
             self._sq_gen += 1  # names this scale in the keys of the weight caches
             self._sqcache = (key, scale if scale.numel() > 1 else None)
         return self._sqcache[1]
@@ -187,11 +191,18 @@ class QLinear(nn.Linear):
                 and self.quantize_feature.reduce_dim == -1
                 and isinstance(self.quantize_weight, Qmax))
 
+    @staticmethod
+    def _fp8_quantizer_ok(q):
+        # a q_mode with neither "_sat" nor "_scale" (and no per-channel / per-token flag) makes the
+        # reference's quantizer return None (quantizers.py:5423-5488): not a mode to accelerate
+        return (isinstance(q, to_fp8) and q.emulate
+                and bool(q.perCh or q.perToken or "_sat" in q.q_mode or "_scale" in q.q_mode))
+
     def _fp8_path_ok(self, x):
         return (self._eval_path_ok(x) and x.shape[-1] % 16 == 0
                 and x.dtype in (torch.float16, torch.bfloat16, torch.float32)
-                and isinstance(self.quantize_feature, to_fp8) and self.quantize_feature.emulate
-                and isinstance(self.quantize_weight, to_fp8) and self.quantize_weight.emulate)
+                and self._fp8_quantizer_ok(self.quantize_feature)
+                and self._fp8_quantizer_ok(self.quantize_weight))
 
     def _weights_key(self, scale):
         w = self.weight
@@ -274,7 +285,11 @@ class QLinear(nn.Linear):
             return y.reshape(tuple(x.shape[:-1]) + (self.out_features,))
         if not x.is_cuda:
             raise RuntimeError("fms_mo_amd.QLinear runs on an AMD GPU only; there is no CPU path")
-        if scale is None:
+        if self.smoothq and torch.is_grad_enabled() and (self.training or self.weight.requires_grad):
+            # a gradient can reach the weights through the scale: build it in this call's graph
+            # (a cached tensor would be backpropagated through twice under gradient accumulation)
+            scale = self.get_smoothq_scale(x)
+        elif scale is None:
             scale = torch.tensor([1.0]).to(x.dtype).to(x.device)
         # training / calibration / other quantizer modes: quantizer modules evaluated with torch ops
         if self.calib_counter > 0:
@@ -516,24 +531,32 @@ class QLinearINT8Deploy(nn.Linear):
         (dim -2); stores ``input_scale`` ([M,1] / [1,K]) and ``cvs[0:2]`` like the reference
         (linear.py:1085-1100)."""
         if self.useDynMaxQfunc == -2:
-            q, s = kernels.quant_act_i8_dynamic(x, True, 2 ** (self.nbits_a - 1) - 1)
+            q, s, col_amax = kernels.quant_act_i8_dynamic(x, True, 2 ** (self.nbits_a - 1) - 1,
+                                                          want_amax=True)
             s = s.reshape(1, -1).to(x.dtype)
+            amax = col_amax.reshape(1, -1).to(x.dtype)      # the abs-max itself, as the reference stores
         else:
             q, s = kernels.quant_act_i8_pertoken(x, None, compute_dtype=x.dtype)
             s = s.reshape(-1, 1)
+            # the per-token kernel hands over scales only: scale * 127 is the row maximum up to the
+            # scale's rounding (and 1e-5 where the clamp of a tiny row acted)
+            amax = s * 127
         self.input_scale = s
-        self.cvs[0], self.cvs[1] = s * 127, -(s * 127)
+        self.cvs[0], self.cvs[1] = amax, -amax
         return q
 
     def qa_dyn_max_fake_zero_shift(self, x):
         """One dynamic scale amax / (127 - zp) for the whole tensor, codes shifted by zp
         (linear.py:1102-1113).  The zero point is a construction-time constant."""
-        if getattr(self, "_fzs_zp", None) is None:
-            self._fzs_zp = int(self.input_zp)
+        zp = self.input_zp
+        key = (zp.data_ptr(), zp._version)
+        if getattr(self, "_fzs_key", None) != key:      # reading the buffer costs a host sync
+            self._fzs_key, self._fzs_zp = key, int(zp)
         levels = 2 ** (self.nbits_a - 1) - 1 - self._fzs_zp
-        q, s = kernels.quant_act_i8_dynamic(x, False, levels, self._fzs_zp)
+        q, s, col_amax = kernels.quant_act_i8_dynamic(x, False, levels, self._fzs_zp, want_amax=True)
         self.input_scale = s.reshape(()).to(x.dtype)
-        self.cvs[0], self.cvs[1] = self.input_scale * levels, -(self.input_scale * levels)
+        amax = col_amax.max().to(x.dtype)
+        self.cvs[0], self.cvs[1] = amax, -amax
         return q
 
     # -- matmul + dequant ----------------------------------------------------------------------
@@ -563,9 +586,24 @@ class QLinearINT8Deploy(nn.Linear):
         if K > self.chunk_size and self.use_int_kernel != "triton":
             cs = int(self.chunk_size)
             if cs >= 32 and not cs & (cs - 1):
+                # the accumulator is 2^t * (the reference's shifted one); (2^t a) * s == a * (2^t s) exactly
+                if (torch.result_type(self.input_scale, self.w_scale) == torch.float32
+                        and self.acc_dtype in (torch.float16, torch.bfloat16, torch.float32)):
+                    # fp32 scale product, multiply and add rounded separately, cast to acc_dtype: the
+                    # final expression of the reference's loop inside the kernel's epilogue (one launch)
+                    a_scale, w_scale = self.input_scale.float().reshape(-1), self._w_scale_f32()
+                    if self.useDynMaxQfunc == -2:      # [1,K] scales against [M,N] (K == N): a column scale
+                        if a_scale.numel() != w.shape[0]:
+                            raise RuntimeError("per-channel activation scales need in_features == out_features "
+                                               "(the reference's [1,K] scale broadcasts against [M,N])")
+                        w_scale = a_scale * w_scale
+                        a_scale = torch.ones(1, dtype=torch.float32, device=m1.device)
+                    return kernels.matmul_chunk_dq(m1, w, a_scale, w_scale, bias, L.EPI_F32_MULADD, self.acc_dtype,
+                                                   chunk_size=cs, chunk_trun_bits=int(self.truncate_lsb),
+                                                   max_acc_bits=self.max_acc_bits)
+                # 16-bit scale buffers on both sides: torch evaluates the chain in that dtype
                 acc = kernels.matmul_chunk(m1, w, None, chunk_size=cs, chunk_trun_bits=int(self.truncate_lsb),
                                            max_acc_bits=self.max_acc_bits)
-                # acc == 2^t * (the reference's shifted accumulator); (2^t a) * s == a * (2^t s) exactly
                 return (acc * (self.input_scale * self.w_scale) + bias).to(self.acc_dtype)
             # any other chunk size (ragged last chunk included): the reference's serial loop, one
             # exact int32 GEMM per chunk
@@ -587,6 +625,13 @@ class QLinearINT8Deploy(nn.Linear):
         if self.use_fake_zero_shift:
             updated_bias = bias - self.input_scale * self.corr_term
         if self.use_int_kernel == "triton" and self.truncate_lsb > 0:
+            cs = int(self.chunk_size)
+            cs = max(cs, 32) if cs & (cs - 1) == 0 else 32          # tl_matmul's chunk-size rule for int8
+            if self.useDynMaxQfunc != -2 and self.acc_dtype in (torch.float16, torch.float32) and cs >= 32:
+                # imatmul = the chunked kernel, then the fp16-scale epilogue: one launch
+                return kernels.matmul_chunk_dq(m1, w, self.input_scale.float().reshape(-1), self._w_scale_f32(),
+                                               updated_bias, L.EPI_REF_F16, self.acc_dtype, chunk_size=cs,
+                                               chunk_trun_bits=int(self.truncate_lsb))
             imm_out = tl_matmul(m1, m2, chunk_trun_bits=int(self.truncate_lsb), chunk_size=int(self.chunk_size))
             return (imm_out.float() * (self.input_scale * self.w_scale).to(torch.float16)
                     + updated_bias).to(self.acc_dtype)
@@ -609,8 +654,15 @@ class QLinearINT8Deploy(nn.Linear):
 
     def iaddmm_FP(self, bias, m1, m2):
         """The reference's non-integer emulation (torch.matmul on dequantized operands)."""
-        m1 = self._quantize(m1)
-        return torch.matmul(m1 * self.input_scale, m2 * self.w_scale) + bias
+        x_dtype = m1.dtype
+        if self.useDynMaxQfunc in [-1, -2]:
+            m1 = self.qa_dynamic_max_qfunc(m1)
+        elif self.usePTnativeQfunc:
+            m1 = self.qa_raw_qfunc(m1)
+        else:
+            m1 = self.qa_fmo_mo_qfunc(m1)
+        # the kernels hand the dynamic scale over as fp32 holding a value of x's dtype
+        return torch.matmul(m1 * self.input_scale.to(x_dtype), m2 * self.w_scale) + bias
 
     def set_matmul_op(self):
         from ..custom_ext_kernels.utils import imatmul_ops_reg
@@ -736,31 +788,39 @@ class LinearFPxAcc(torch.nn.Linear):
         out_shape = x.shape[:-1] + (self.weight.shape[0],)
         x = x.reshape(-1, x.shape[-1])
         weight = self.weight.detach()
+        # tl_matmul's chunk-size rule for the tensors the reference hands it: the FP8 codes travel as
+        # fp32 tensors there (minimum chunk 16, like 16-bit and fp32 operands)
+        cs = int(self.chunk_size)
+        # (a chunk of 8 sixteen-bit elements is emulated by the reference with interleaved zeros)
+        pad8 = cs == 8 and not self.fp8_dyn and x.dtype in (torch.float16, torch.bfloat16)
+        if not pad8:
+            cs = max(cs, 16) if cs & (cs - 1) == 0 else 16
         with torch.no_grad():
             if self.fp8_dyn:
                 variant = L.FP8_FPXACC_DL8 if self.clamp_acc_to_dl16 else L.FP8_FPXACC
-                if self.fp8_dyn == "per_tensor":
-                    # one scale per tensor, formed in the original dtype like the reference
-                    xs = (x.abs().amax() / 448.0).clamp(min=1e-5)
-                    wsc = (weight.abs().amax() / 448.0).clamp(min=1e-5)
-                    xq, _ = kernels.quant_act_fp8_pertoken(x, variant, static_scale=xs.float())
-                    wq, _ = kernels.quant_act_fp8_pertoken(weight, variant, static_scale=wsc.float())
-                    x_scale, w_scale = xs.reshape(1, 1), wsc.reshape(1, 1)
-                else:
-                    xq, xs = kernels.quant_act_fp8_pertoken(x, variant)
-                    wq, wsc = kernels.quant_act_fp8_pertoken(weight, variant)
-                    x_scale, w_scale = xs.reshape(-1, 1).to(org_dtype), wsc.reshape(-1, 1).to(weight.dtype)
-                acc = tl_matmul(xq, wq.t(), chunk_trun_bits=self.trun_bits, chunk_size=int(self.chunk_size),
-                                clamp_acc_to_dl16=self.clamp_acc_to_dl16)
+                per_tensor = self.fp8_dyn == "per_tensor"
+                # scales in the original dtype like the reference (the kernels hand them over as fp32
+                # holding those values); per tensor: column abs-max and quantizer, nothing read back
+                xq, xs = kernels.quant_act_fp8_dynamic(x, variant, per_tensor, 1e-5, True)
+                wq, wsc = kernels.quant_act_fp8_dynamic(weight, variant, per_tensor, 1e-5, True)
+                if cs < 32:
+                    # a chunk of 16 FP8-valued elements: every e4m3 value is an fp16 value, and the
+                    # fp16 matrix instructions take 16 elements per step
+                    xq, wq = xq.to(torch.float16), wq.to(torch.float16)
+                a_op, w_op = xq, wq
             else:
-                x_scale = torch.tensor(1.0, device=x.device, dtype=org_dtype)
-                w_scale = x_scale.clone().reshape(1, 1)
-                acc = tl_matmul(x.contiguous(), weight.to(x.dtype).t(), chunk_trun_bits=self.trun_bits,
-                                chunk_size=int(self.chunk_size), clamp_acc_to_dl16=self.clamp_acc_to_dl16)
-            out = (acc * x_scale * w_scale.t()).to(org_dtype).reshape(out_shape)
-            if self.bias is not None:
-                out = out + self.bias.to(org_dtype)
-        return out
+                xs = wsc = torch.ones(1, dtype=torch.float32, device=x.device)
+                a_op, w_op = x.contiguous(), weight.to(x.dtype)
+            if pad8:
+                out = tl_matmul(a_op, w_op.t(), chunk_trun_bits=self.trun_bits, chunk_size=8,
+                                clamp_acc_to_dl16=self.clamp_acc_to_dl16).to(org_dtype).reshape(out_shape)
+                if self.bias is not None:
+                    out = out + self.bias.to(org_dtype)
+                return out
+            # descale, cast to the original dtype, add the bias there: the kernel's epilogue
+            out = kernels.matmul_chunk_dq(a_op, w_op, xs, wsc, self.bias, L.EPI_SEQ_OUT, org_dtype, chunk_size=cs,
+                                          chunk_trun_bits=self.trun_bits, clamp_acc_to_dl16=self.clamp_acc_to_dl16)
+        return out.reshape(out_shape)
 
     def extra_repr(self) -> str:
         s = f"{self.in_features},{self.out_features}"
@@ -803,13 +863,19 @@ class QLinearINT8Train(torch.nn.Linear):
             x_i8, x_scale = kernels.quant_act_i8_pertoken(x, None, compute_dtype=x.dtype)
             w = self.weight.detach()
             w_i8, w_scale = kernels.quant_act_i8_pertoken(w, None, compute_dtype=w.dtype)
-            acc = tl_matmul(x_i8, w_i8.t(), chunk_trun_bits=self.lsb_trun_bits, chunk_size=self.chunk_size,
-                            max_acc_bits=self.max_acc_bits)
-            out = (acc.to(torch.float) * x_scale.reshape(-1, 1).to(org_dtype)
-                   * w_scale.reshape(1, -1).to(w.dtype)).reshape(out_shape).to(org_dtype)
-            if self.bias is not None:
-                out = out + self.bias.to(org_dtype)
-        return out
+            cs = int(self.chunk_size)
+            if cs == 8:     # emulated by the reference with interleaved zeros: its wrapper's business
+                acc = tl_matmul(x_i8, w_i8.t(), chunk_trun_bits=self.lsb_trun_bits, chunk_size=8,
+                                max_acc_bits=self.max_acc_bits)
+                out = (acc.to(torch.float) * x_scale.reshape(-1, 1).to(org_dtype)
+                       * w_scale.reshape(1, -1).to(w.dtype)).reshape(out_shape).to(org_dtype)
+                return out if self.bias is None else out + self.bias.to(org_dtype)
+            cs = max(cs, 32) if cs & (cs - 1) == 0 else 32      # tl_matmul's rule for int8
+            # (acc.float() * x_scale * w_scale.t()).to(org_dtype) + bias.to(org_dtype) in the epilogue
+            out = kernels.matmul_chunk_dq(x_i8, w_i8, x_scale, w_scale, self.bias, L.EPI_SEQ_OUT, org_dtype,
+                                          chunk_size=cs, chunk_trun_bits=self.lsb_trun_bits,
+                                          max_acc_bits=self.max_acc_bits)
+        return out.reshape(out_shape)
 
     def extra_repr(self) -> str:
         s = f"{self.in_features},{self.out_features},bias={self.bias is not None},chunk_size={self.chunk_size}"

@@ -98,8 +98,9 @@ def recompute_weight_with_sawb(weight_pre_quant, weight_int_as_fp, weight_per_ch
         weight_int_sawb = torch.where((cv_sawb < cv_max)[:, None], weight_int_sawb, weight_int_as_fp)
         cv_guarded = torch.where(cv_sawb < cv_max, cv_sawb, cv_max)
     else:
+        # per tensor the reference guards the clip value only: it builds the guarded integers
+        # (aiu_utils.py:196-199) and returns the SAWB integers regardless (:235)
         cv_max = weight_pre_quant.abs().max()
-        weight_int_sawb = weight_int_sawb if cv_sawb < cv_max else weight_int_as_fp
         cv_guarded = torch.min(cv_sawb, cv_max)
     new_sd[layer_name + ".quantize_weight.clip_val"] = cv_guarded
     new_sd[layer_name + ".quantize_weight.clip_valn"] = -cv_guarded

@@ -59,7 +59,13 @@ enum {
      multiply and add rounded separately -- `input_scale * w_scale * acc + bias` of
      QLinearCublasI8I32NT / QLinearCutlassI8I32NT.forward (fms_mo/modules/linear.py:1533-1535,
      1581-1583). */
-  FMSMO_EPI_F32_MULADD = 2
+  FMSMO_EPI_F32_MULADD = 2,
+  /* The chunked matmuls' fused forms only (fmsmo_matmul_chunk_*_dq): descale, cast, add the bias
+     in the output dtype T:  y = T( T( f32( f32(acc) * a_scale[m] ) * w_scale[n] ) + T(bias[n]) ),
+     no addition without a bias -- `(acc * x_scale * w_scale.t()).to(org_dtype) + bias.to(org_dtype)`
+     of LinearFuncFPxFwdBwd.forward and LinearFuncINT8FwdFP32Bwd.forward
+     (fms_mo/modules/linear.py:1955-1975, 2180-2189). */
+  FMSMO_EPI_SEQ_OUT = 3
 };
 
 int fmsmo_abi_version(void);
@@ -234,6 +240,30 @@ enum {
 int fmsmo_quant_act_fp8_pertoken(const void* x, int x_dtype, int64_t ldx, int variant,
                                  int static_scale, uint8_t* q, int64_t ldq, float* scale,
                                  int64_t M, int64_t K, fmsmo_stream_t stream);
+/*
+ * The same quantizer with the rule of its dynamic scale spelled out by the caller:
+ *   s = max( amax / 448, scale_floor )
+ * formed in fp32 from the widened abs-max (scale_dtype = FMSMO_F32) or with the quotient and the
+ * floor both rounded to x's dtype (scale_dtype = x_dtype: what torch computes when the division
+ * runs on the 16-bit tensor and the clamp bound is a python scalar).  The quotients, the clamp
+ * and the cast are the variant's.  per_tensor = 0: amax per row, scale [M] written.
+ * per_tensor = 1: amax over the whole tensor, taken from col_amax (fp32 [K] on the device, the
+ * per-column abs-max that fmsmo_absmax_cols left there), scale [1] written; nothing is read back
+ * to the host, so both launches can be captured in a HIP graph.
+ * FP8Linear's dynamic activation scale (fms_mo/aiu_addons/fp8/fp8_linear.py:163-194,236-251) is
+ * computed inside torchao (to_affine_quantized_floatx), which is not part of the reference tree:
+ * the floor and the dtype of the division are the two properties that code fixes and the
+ * reference's own files do not, hence parameters here; (1e-12, FMSMO_F32) is the rule of the
+ * reference's test helper (tests/aiu_addons/test_fp8_addon.py:65-79) and the default of
+ * fmsmo_quant_act_fp8_pertoken.  LinearFuncFPxFwdBwd's per-tensor scales
+ * (fms_mo/modules/linear.py:1939-1948) are (1e-5, x_dtype) with per_tensor = 1.
+ * scale_floor must be positive and below 2^60, and must not round to zero in scale_dtype
+ * (FMSMO_ERR_UNSUPPORTED otherwise: a zero row would be divided by a zero scale).
+ */
+int fmsmo_quant_act_fp8_dynamic(const void* x, int x_dtype, int64_t ldx, int variant,
+                                int per_tensor, const float* col_amax, float scale_floor,
+                                int scale_dtype, uint8_t* q, int64_t ldq, float* scale,
+                                int64_t M, int64_t K, fmsmo_stream_t stream);
 
 /* ------------------------------------------------------------------------------------------
  * 2. W8A8 GEMMs on MFMA.   C[M,N] = A[M,K] . B[N,K]^T
@@ -313,8 +343,9 @@ int64_t fmsmo_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
 
 /*
  * Which kernel the *_dq GEMMs run for a shape, without launching anything (host-only; for tests,
- * tuning and capacity planning).  with_workspace != 0 describes the *_dq_ws calls given a
- * sufficient workspace.  tile_m / tile_n are 0 for the decode and generic kernels; splits is the
+ * tuning and capacity planning).  with_workspace = 1 describes the *_dq_ws calls given a
+ * sufficient workspace, with_workspace = 2 what fmsmo_gemm_i8_dq_noalloc runs (the split that
+ * fits its static scratch; FMSMO_ERR_SCRATCH where that call returns it).  tile_m / tile_n are 0 for the decode and generic kernels; splits is the
  * number of K slices (1 = single pass).  The choice weighs the measured efficiency of each tile
  * shape against how full the last round of tiles leaves the 256 compute units, e.g.
  * 4096 x 6144 runs 512 tiles of 256 x 192 (two full rounds) rather than 384 of 256 x 256.
@@ -470,6 +501,34 @@ int fmsmo_matmul_chunk_fp(const void* a, int64_t lda, const void* b, int64_t ldb
                           const float* c_in, float* d, int64_t ldd, int64_t M, int64_t N,
                           int64_t K, int chunk_size, int chunk_trun_bits, int clamp_dl16,
                           int truncate_then_accumulate, fmsmo_stream_t stream);
+
+/*
+ * The two chunked matmuls with the dequantization fused into their epilogue (one launch instead of
+ * the matmul and three or four elementwise passes over [M,N]):
+ *   y[m,n] = epilogue( acc[m,n], a_scale[m or 0], w_scale[n or 0], bias[n] ),  epilogue one of
+ *   FMSMO_EPI_*; acc is the chunked accumulator of fmsmo_matmul_chunk_i8 / _fp with c_in = NULL
+ *   (for integers it still carries the factor 2^t of its cleared low bits; (2^t a) s = a (2^t s)
+ *   exactly, so the reference's `trun_scale * input_scale` needs no separate multiply).
+ * a_scale_n in {1, M}, w_scale_n in {1, N}; bias [N] of bias_dtype or NULL; y of y_dtype.
+ * With nothing to round or clamp (int8, t = 0, 32 accumulator bits) the call is fmsmo_gemm_i8_dq.
+ * Reference: the serial chunk loop of iaddmm_int and its final
+ * `accumulator * (trun_scale * input_scale * w_scale) + bias` = FMSMO_EPI_F32_MULADD
+ * (fms_mo/modules/linear.py:1142-1175); imatmul bound to tl_matmul_chunk_truncate followed by the
+ * fp16-scale epilogue = FMSMO_EPI_REF_F16 (:1213-1251, 1177-1188); LinearFuncFPxFwdBwd.forward and
+ * LinearFuncINT8FwdFP32Bwd.forward = FMSMO_EPI_SEQ_OUT (:1955-1975, 2180-2189).
+ */
+int fmsmo_matmul_chunk_i8_dq(const int8_t* a, int64_t lda, const int8_t* b, int64_t ldb,
+                             const float* a_scale, int64_t a_scale_n, const float* w_scale,
+                             int64_t w_scale_n, const void* bias, int bias_dtype, int epilogue,
+                             void* y, int y_dtype, int64_t ldy, int64_t M, int64_t N, int64_t K,
+                             int chunk_size, int chunk_trun_bits, int max_acc_bits,
+                             int truncate_then_accumulate, fmsmo_stream_t stream);
+int fmsmo_matmul_chunk_fp_dq(const void* a, int64_t lda, const void* b, int64_t ldb, int op_dtype,
+                             const float* a_scale, int64_t a_scale_n, const float* w_scale,
+                             int64_t w_scale_n, const void* bias, int bias_dtype, int epilogue,
+                             void* y, int y_dtype, int64_t ldy, int64_t M, int64_t N, int64_t K,
+                             int chunk_size, int chunk_trun_bits, int clamp_dl16,
+                             int truncate_then_accumulate, fmsmo_stream_t stream);
 
 /* ------------------------------------------------------------------------------------------
  * 5. Grouped int8 GEMM for mixture-of-experts FFNs (uneven rows per expert, one launch).

@@ -49,9 +49,16 @@ How each function is pinned (see tests/test_oracle_*.py):
                            (reciprocal-then-multiply, fp16 clamp), the cast against the enumerated
                            e4m3 grid with ties to even, every element of the scaled quantizers
                            re-derived the same way
-  * FP8Linear dynamic scale (computed inside torchao 0.11, not in the reference tree):
-                           PARITY UNPINNED -- the rule used is the one of the reference's test
-                           helper (tests/aiu_addons/test_fp8_addon.py:65-79).
+  * FP8Linear dynamic scale (computed inside torchao 0.11, not in the reference tree)
+                        -- what a symmetric e4m3 scale must satisfy whatever library forms it:
+                           quantizing a finite non-zero row with it puts the row maximum on the
+                           top code 448 and nothing beyond it, the top code dequantizes back to
+                           the row maximum within an fp32 rounding, the scale is fp32 for every
+                           input dtype, a zero row gives the floor and zero codes (each shown to
+                           fail for /240, /127, a 16-bit-rounded scale, a scale left in x's
+                           dtype).  The value of the floor and the dtype the division runs in are
+                           torchao's own choice and not derivable: both are arguments (defaults =
+                           the reference's test helper, tests/aiu_addons/test_fp8_addon.py:65-79).
 """
 from __future__ import annotations
 
@@ -443,6 +450,24 @@ def deploy_forward_general(x, st, chunk_size=100000, truncate_lsb=0, max_acc_bit
     return {"q_x": q_x, "input_scale": input_scale, "acc": acc, "y": y}
 
 
+def deploy_forward_triton(x, st, chunk_size=32, truncate_lsb=0):
+    """QLinearINT8Deploy.forward with use_int_kernel="triton" (linear.py:1213-1251 binds imatmul
+    to tl_matmul(chunk_trun_bits=truncate_lsb, chunk_size=chunk_size); iaddmm_int then skips its
+    PyTorch chunk loop, :1142, and takes the fp16-scale epilogue, :1177-1188).  max_acc_bits is
+    not forwarded to the kernel by the reference.  Dynamic per-token activations only."""
+    org_dtype = x.dtype
+    x2 = x.reshape(-1, x.shape[-1])
+    sq = st["smoothq_scale"]
+    if torch.all(sq != 1).item():
+        x2 = x2 / sq
+    q_x, input_scale = quant_act_dyn_max(x2, st["useDynMaxQfunc"])
+    cs = max(chunk_size, 32) if (chunk_size & (chunk_size - 1)) == 0 else 32
+    acc = chunk_matmul_i8(q_x, st["weight"], None, cs, truncate_lsb, 32)
+    y = (acc.float() * (input_scale * st["w_scale"]).to(torch.float16) + st["bias"]).to(st["acc_dtype"])
+    y = y.reshape(tuple(x.shape[:-1]) + (st["weight"].shape[0],)).to(org_dtype)
+    return {"q_x": q_x, "input_scale": input_scale, "acc": acc, "y": y}
+
+
 def i8i32nt_from_fms_mo(weight, bias, a_cv, a_cvn, w_cv):
     """QLinearCublasI8I32NT.from_fms_mo (linear.py:1429-1489): asymmetric (quint8) activations with
     the zero-point correction folded into the bias.  The weight integers are what the per-channel
@@ -650,16 +675,35 @@ def to_fp8_forward(x, q_mode="fp8_e4m3_sat", perCh=None, perToken=False):
     return None
 
 
+def qlinear_fp8_forward(x, weight, bias, qa_mode, qw_mode, smoothq_scale=None):
+    """QLinear.forward (fms_mo/modules/linear.py:248-305) with the FP8 emulation quantizers
+    (quantizers.py:5309-5488): F.linear on the fake-quantized tensors, each already rounded to its
+    own dtype, the products summed by torch's matmul in that dtype."""
+    s = torch.tensor([1.0], dtype=x.dtype) if smoothq_scale is None else smoothq_scale
+    xq = to_fp8_forward(x / s, qa_mode, perToken="perToken" in qa_mode).to(x.dtype)
+    wq = to_fp8_forward(weight * s, qw_mode, perCh=weight.shape[0] if "perCh" in qw_mode else None).to(weight.dtype)
+    return torch.nn.functional.linear(xq, wq, bias)
+
+
 def fp8_quant_static(x: torch.Tensor, scale: torch.Tensor):
     """_quantize_affine_float8_custom (fms_mo/aiu_addons/fp8/fp8_linear.py:54-72)."""
     t = x.to(torch.float32) / scale
     return t.clamp(min=-E4M3_MAX, max=E4M3_MAX).to(torch.float8_e4m3fn)
 
 
-def fp8_dynamic_scale(x: torch.Tensor):
-    """Per-row dynamic scale, rule of the reference's test helper
-    (tests/aiu_addons/test_fp8_addon.py:65-79).  PARITY UNPINNED w.r.t. torchao 0.11."""
-    return (x.abs().amax(dim=-1, keepdim=True).to(torch.float32) / E4M3_MAX).clamp(min=1e-12)
+def fp8_dynamic_scale(x: torch.Tensor, floor: float = 1e-12, in_x_dtype: bool = False,
+                      per_tensor: bool = False):
+    """Dynamic activation scale of FP8Linear (fms_mo/aiu_addons/fp8/fp8_linear.py:163-194 hands
+    the computation to torchao's to_affine_quantized_floatx with scale_dtype=torch.float32;
+    torchao 0.11 is not in the reference tree and not importable).  Fixed by the mathematics and
+    pinned by tests/test_oracle_pins.py: a symmetric e4m3 scale maps the abs-max onto the top
+    code 448, and the result is fp32.  Left open by them, hence arguments: the lower clamp
+    (default: the reference's own test helper, tests/aiu_addons/test_fp8_addon.py:65-79) and
+    whether the division by 448 runs on the fp32-widened abs-max or in x's dtype."""
+    amax = x.abs().amax().reshape(1, 1) if per_tensor else x.abs().amax(dim=-1, keepdim=True)
+    if in_x_dtype:
+        return (amax / E4M3_MAX).clamp(min=floor).to(torch.float32)
+    return (amax.to(torch.float32) / E4M3_MAX).clamp(min=floor)
 
 
 def scaled_mm_cpu(mat1, mat2, scale1, scale2, bias=None, out_dtype=torch.float32):
@@ -807,8 +851,8 @@ def aiu_convert_layer(weight, w_cv, sq_a_scale=None, sq_alpha=None, a_cv=None, a
 def aiu_recompute_narrow(weight_pre_quant, weight_int_as_fp, per_channel: bool):
     """recompute_weight_with_sawb (fms_mo/utils/aiu_utils.py:125-235) without SmoothQuant: when the
     integer weights are narrow (std below 20 levels, any row in per-channel mode) they are
-    re-quantized with a SAWB quantizer in training mode (clip from the statistics, :633-672) and
-    kept where that clip value is below the row (tensor) maximum.  Returns (integers or None,
+    re-quantized with a SAWB quantizer in training mode (clip from the statistics, :633-672) and,
+    per channel, kept where that clip value is below the row maximum.  Returns (integers or None,
     guarded clip value(s) in fp16 or None)."""
     if per_channel:
         recompute = any(w < 20 for w in weight_int_as_fp.std(dim=-1))
@@ -829,7 +873,9 @@ def aiu_recompute_narrow(weight_pre_quant, weight_int_as_fp, per_channel: bool):
     w_sawb = sawb_zero_forward(w32, clip, 8, dequantize=False)
     cv_sawb = clip.reshape(1).to(torch.float16)
     cv_max = weight_pre_quant.abs().max()
-    return (w_sawb if cv_sawb < cv_max else weight_int_as_fp), torch.min(cv_sawb, cv_max)
+    # per tensor the reference forms the guarded integers (:196-199) but returns the SAWB integers
+    # themselves (:235) beside the guarded clip value: kept as it is
+    return w_sawb, torch.min(cv_sawb, cv_max)
 
 
 def absmax_cols(x):

@@ -491,23 +491,46 @@ def test_lowered_model_compiles_fullgraph_and_replays_from_a_hip_graph(dev):
         assert torch.equal(bits(static_y.cpu()), bits(expect.cpu())), i
 
 
-def test_lower_qmodel_triton_swaps_both_kinds(dev):
+@pytest.mark.parametrize("trunc", [0, 6])
+def test_lower_qmodel_triton_swaps_both_kinds(dev, trunc):
+    """lower_qmodel_triton against the oracle, layer by layer on the oracle's own intermediate
+    activations: the two int8 layers bit-exact against deploy_forward_triton (codes, scales and
+    outputs), the plain layer's dynamic-FP8 chunked matmul within rtol / atol 1e-2 of
+    fpxacc_forward (the fp32 summation order inside a chunk is the matrix unit's)."""
+    import copy
+
     from fms_mo_amd.custom_ext_kernels.utils import lower_qmodel_triton
     from fms_mo_amd.modules.linear import LinearFPxAcc, QLinearINT8Deploy
 
-    net = _two_layer().to(dev)
-    x = torch.randn(16, 256, generator=gen(23)).half().to(dev)
-    with torch.no_grad():
-        y_fake = net(x)
-    low = lower_qmodel_triton(net, use_dyn_max_act=-1, max_acc_bits=32, num_lsb_to_truncate=0, chunk_size=64,
+    net = _two_layer()
+    ref_net = copy.deepcopy(net)
+    net.to(dev)
+    x = torch.randn(16, 256, generator=gen(23)).half()
+    low = lower_qmodel_triton(net, use_dyn_max_act=-1, max_acc_bits=32, num_lsb_to_truncate=trunc, chunk_size=64,
                               layer_to_exclude=None)
     assert isinstance(low.up, QLinearINT8Deploy) and low.up.use_int_kernel == "triton"
     assert isinstance(low.plain, LinearFPxAcc) and low.plain.fp8_dyn == "per_token"
+    h = x
+    for name in ("up", "down"):
+        lin = getattr(ref_net, name)
+        st = O.deploy_prepare_general(lin.weight.detach(), lin.bias.detach(), lin.quantize_weight.clip_val,
+                                      use_dynamic_max_act_Qfunc=-1)
+        ref = O.deploy_forward_triton(h, st, chunk_size=64, truncate_lsb=trunc)
+        mod = getattr(low, name)
+        with torch.no_grad():
+            y = mod(h.to(dev))
+        assert torch.equal(mod.weight.cpu(), st["weight"]), name
+        assert torch.equal(mod.input_scale.cpu().reshape(-1).float(), ref["input_scale"].float().reshape(-1)), name
+        assert torch.equal(bits(y.cpu()), bits(ref["y"])), name
+        h = ref["y"]
+        if name == "up":
+            h = torch.nn.functional.gelu(h.float()).half()
+    ref_plain = O.fpxacc_forward(h, ref_net.plain.weight.detach(), None, trunc, 64, "per_token", False)
     with torch.no_grad():
-        y = low(x)
-    # fp8 emulation of the plain layer costs a few percent; the int8 layers are tolerance-equal
-    assert torch.isfinite(y).all()
-    assert (y.float() - y_fake.float()).abs().mean() < 0.1 * y_fake.float().abs().mean() + 1e-3
+        y_plain = low.plain(h.to(dev))
+    torch.testing.assert_close(y_plain.cpu().float(), ref_plain.float(), rtol=1e-2, atol=1e-2)
+    with torch.no_grad():
+        assert torch.isfinite(low(x.to(dev))).all()
     net2 = _two_layer().to(dev)
     low2 = lower_qmodel_triton(net2, layer_to_exclude="plain")
     assert type(low2.plain) is torch.nn.Linear
@@ -563,6 +586,10 @@ def test_qlinear_fp8_modes_run_on_the_fp8_gemm(dev, modes, dtype):
     xq = O.to_fp8_forward(x, qa, perToken="perToken" in qa)
     wq = O.to_fp8_forward(m.weight.detach(), qw, perCh=N if "perCh" in qw else None)
     ref = torch.nn.functional.linear(xq.float(), wq.float(), m.bias.detach().float())
+    # the reference's own evaluation (F.linear in x's dtype on the same tensors) is that product
+    # rounded once more: the band below is stated against the exact product and covers both
+    ref_mod = O.qlinear_fp8_forward(x, m.weight.detach(), m.bias.detach(), qa, qw).float()
+    assert ((ref_mod - ref).abs() <= 1e-2 * ref.abs() + 1e-2 * max(1.0, float(ref.abs().mean()))).all()
     md = m.to(dev)
     with torch.no_grad():
         y = md(x.to(dev))
@@ -571,10 +598,15 @@ def test_qlinear_fp8_modes_run_on_the_fp8_gemm(dev, modes, dtype):
     assert torch.equal(bits(y.cpu()), bits(y_again.cpu()))
     tol = 1e-2 * ref.abs() + 1e-2 * max(1.0, float(ref.abs().mean()))
     assert ((y.cpu().float() - ref).abs() <= tol).all()
+    assert ((y.cpu().float() - ref_mod).abs() <= 2 * tol).all()
     md.train()
     with torch.no_grad():
         y_train = md(x.to(dev))                              # torch-op emulation path
     assert ((y_train.cpu().float() - ref).abs() <= 2 * tol).all()
+    # a q_mode the reference's quantizer answers with None is not sent to the kernels
+    md.eval()
+    md.quantize_feature.q_mode, md.quantize_feature.perToken = "fp8_e4m3", False
+    assert not md._fp8_path_ok(x.to(dev))
 
 
 # ----------------------------------------------------------------- QLinear SmoothQuant cache
@@ -609,3 +641,57 @@ def test_qlinear_set_act_scale_invalidates_the_cached_weights(dev):
     ref0 = O.qlinear_forward(x, w_cpu, b_cpu, None, 0.5, w_clip_val=cv)
     d0 = (y0.cpu().float() - ref0.float()).abs()
     assert (d0 > 1e-2 + 1e-2 * ref0.float().abs()).float().mean() < 2e-3
+
+
+def test_qlinear_smoothq_train_mode_backward_twice_without_optimizer_step(dev):
+    """Gradient accumulation: two forward / backward passes of a SmoothQuant QLinear in training
+    mode with no weight update in between.  The SmoothQuant scale depends on the weights, so it is
+    rebuilt inside every call's autograd graph (the reference recomputes it in every forward,
+    linear.py:345-368); the tensor cached for the kernel paths is detached and never enters one."""
+    from tests.test_gpu_modules import make_qlinear, outlier_x
+
+    K, N = 256, 128
+    m = make_qlinear(dev, K, N, smoothq=True, seed=31, dtype=torch.float32)
+    x = outlier_x(32, K, 32, dtype=torch.float32).to(dev)
+    m.set_act_scale(x.abs().amax(dim=0))
+    with torch.no_grad():
+        m.eval()
+        m(x)                                   # fills the cache on the no-grad kernel path first
+    assert m._sqcache is not None and not m._sqcache[1].requires_grad
+    m.train()
+    grads = []
+    for _ in range(2):
+        m.zero_grad()
+        y = m(x)
+        y.float().pow(2).mean().backward()     # a second backward through a freed graph would raise
+        assert m.weight.grad is not None and torch.isfinite(m.weight.grad).all()
+        grads.append(m.weight.grad.clone())
+    assert torch.equal(grads[0], grads[1])
+    assert grads[0].abs().sum() > 0
+
+
+def test_dynamic_quantizers_store_the_abs_max_as_clip_values(dev):
+    """qa_dynamic_max_qfunc (dim -2) and qa_dyn_max_fake_zero_shift leave +-amax in cvs[0:2] like
+    the reference (linear.py:1085-1113), not scale * levels; a changed input_zp buffer is seen by
+    the next forward."""
+    from fms_mo_amd.modules.linear import QLinearINT8Deploy
+    from tests.test_gpu_modules import make_qlinear
+
+    m = make_qlinear(None, 256, 256, seed=33)
+    x = static_x(40, 256, 34, torch.float16)
+    x[:, 7] *= 1e-7                              # a column whose scale is governed by the 1e-5 clamp
+
+    dep = QLinearINT8Deploy.from_fms_mo(m, use_dynamic_max_act_Qfunc=-2, recalc_clipvals=False, target_device=dev)
+    dep(x.to(dev))
+    amax = x.abs().amax(dim=0, keepdim=True)
+    assert torch.equal(dep.cvs[0].cpu(), amax) and torch.equal(dep.cvs[1].cpu(), -amax)
+    fz = QLinearINT8Deploy.from_fms_mo(m, use_dynamic_max_act_Qfunc=5, recalc_clipvals=False, target_device=dev)
+    assert fz.use_fake_zero_shift
+    fz(x.to(dev))
+    assert torch.equal(fz.cvs[0].cpu(), x.abs().max()) and torch.equal(fz.cvs[1].cpu(), -x.abs().max())
+    s5 = fz.input_scale.clone()
+    with torch.no_grad():
+        fz.input_zp.fill_(9)
+    fz(x.to(dev))
+    ref_q, ref_s = O.quant_act_fake_zero_shift(x, torch.tensor(9, dtype=torch.int))
+    assert torch.equal(fz.input_scale.cpu(), ref_s) and not torch.equal(fz.input_scale, s5)

@@ -296,6 +296,62 @@ def test_quant_act_fp8_linear(dev, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("per_tensor", [False, True])
+def test_quant_act_fp8_dynamic_scale_rules(dev, dtype, per_tensor):
+    """fmsmo_quant_act_fp8_dynamic: floor and division dtype of the dynamic scale as the caller
+    states them, per token and per tensor (column abs-max on the device, nothing read back);
+    scales and codes bit-exact against the oracle."""
+    from fms_mo_amd import _lib as L
+
+    for Kd, scale in ((4096, 2.0), (14336, 0.01), (64, 300.0), (20000, 1.0)):
+        x = _special_rows((torch.randn(37, Kd, generator=gen(61)) * scale).to(dtype))
+        x[5] = x[5] * 1e-4                                  # a row far below the tensor's maximum
+        for floor, in_xt in ((1e-12, False), (1e-5, False), (1e-5, True), (2e-3, True), (2e-3, False)):
+            if in_xt and dtype == torch.float16 and floor < 1e-7:
+                continue
+            s_ref = O.fp8_dynamic_scale(x, floor, in_xt, per_tensor)
+            q_ref = O.fp8_quant_static(x, s_ref)
+            q, s = K().quant_act_fp8_dynamic(x.to(dev), L.FP8_LINEAR, per_tensor, floor, in_xt)
+            assert s.dtype == torch.float32
+            assert torch.equal(s.cpu(), s_ref.reshape(-1)), (Kd, floor, in_xt)
+            assert torch.equal(q.cpu().view(torch.uint8), q_ref.view(torch.uint8)), (Kd, floor, in_xt)
+    # the defaults of the per-token entry point are (1e-12, fp32)
+    q0, s0 = K().quant_act_fp8_pertoken(x.to(dev), L.FP8_LINEAR)
+    q1, s1 = K().quant_act_fp8_dynamic(x.to(dev), L.FP8_LINEAR, False, 1e-12, False)
+    assert torch.equal(s0, s1) and torch.equal(q0.view(torch.uint8), q1.view(torch.uint8))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("dl8", [False, True])
+def test_quant_act_fp8_fpxacc_per_tensor(dev, dtype, dl8):
+    """The per-tensor scales of LinearFuncFPxFwdBwd.forward (amax / 448 in x's dtype, floor 1e-5)
+    from the device-side column abs-max."""
+    from fms_mo_amd import _lib as L
+
+    for Kd, scale in ((4096, 2.0), (12800, 0.05), (72, 100.0)):
+        x = _special_rows((torch.randn(29, Kd, generator=gen(62)) * scale).to(dtype))
+        q_ref, s_ref = O.fp8_quant_fpxacc(x, per_tensor=True, dl8=dl8)
+        q, s = K().quant_act_fp8_dynamic(x.to(dev), L.FP8_FPXACC_DL8 if dl8 else L.FP8_FPXACC,
+                                         True, 1e-5, True)
+        assert torch.equal(s.cpu(), s_ref.float().reshape(-1))
+        assert torch.equal(q.cpu().view(torch.uint8), q_ref.view(torch.uint8))
+    z = torch.zeros(8, 64, dtype=dtype)
+    q, s = K().quant_act_fp8_dynamic(z.to(dev), L.FP8_FPXACC, True, 1e-5, True)
+    assert s.item() == torch.tensor(1e-5).to(dtype).float().item() and not q.cpu().view(torch.uint8).any()
+
+
+def test_quant_act_fp8_dynamic_rejects_bad_options(dev):
+    from fms_mo_amd import _lib as L
+
+    x = torch.randn(4, 64, device=dev).half()
+    for floor in (0.0, -1.0, float("nan"), 2.0 ** 61):
+        with pytest.raises(L.FmsMoHipError):
+            K().quant_act_fp8_dynamic(x, L.FP8_LINEAR, False, floor, False)
+    with pytest.raises(L.FmsMoHipError):      # an fp16 floor that rounds to zero would divide by it
+        K().quant_act_fp8_dynamic(x, L.FP8_LINEAR, False, 1e-12, True)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("dl8", [False, True])
 def test_quant_act_fp8_fpxacc(dev, dtype, dl8):
     from fms_mo_amd import _lib as L
@@ -1524,3 +1580,99 @@ def test_fused_decode_linear_fp8_long_rows(dev, NK, dt, special):
         assert torch.equal(torch.isnan(y), torch.isnan(ref))
     else:
         torch.testing.assert_close(y, ref, rtol=1e-5, atol=1e-5)
+
+
+# ------------------------------------------------------------------ chunked matmuls, fused epilogue
+def _chunk_epilogue_ref(acc, a_s, w_s, bias, epi, out):
+    """The four epilogues restated with torch CPU ops in the reference's operation order."""
+    from fms_mo_amd import _lib as L
+
+    a_s, w_s = a_s.reshape(-1, 1), w_s.reshape(1, -1)
+    if epi == L.EPI_REF_F16:      # iaddmm_int's plain branch (linear.py:1185-1188)
+        return O.epilogue_ref(acc, a_s, w_s, bias, org_dtype=out,
+                              acc_dtype=torch.float32 if out == torch.float32 else torch.float16)
+    if epi == L.EPI_F32_MULADD:   # the last line of its chunk loop (linear.py:1166-1175)
+        y = acc.float() * (a_s * w_s)
+        return (y if bias is None else y + bias).to(out)
+    if epi == L.EPI_SEQ_OUT:      # LinearFuncFPxFwdBwd / LinearFuncINT8FwdFP32Bwd (linear.py:1955-1975, 2180-2189)
+        y = (acc.float() * a_s * w_s).to(out)
+        return y if bias is None else y + bias.to(out)
+    return O.epilogue_f32(acc, a_s, w_s, bias, out)
+
+
+@pytest.mark.parametrize("shape", [(70, 200, 4096), (33, 96, 80), (300, 130, 1024), (129, 257, 320)])
+def test_matmul_chunk_i8_fused_epilogues_bit_exact(dev, shape):
+    """fmsmo_matmul_chunk_i8_dq: the chunked accumulator is the oracle's, and every epilogue applied
+    to it inside the kernel gives the bits of the reference's torch expression."""
+    from fms_mo_amd import _lib as L
+
+    M, N, Kd = shape
+    g = gen(91)
+    a = torch.randint(-127, 128, (M, Kd), generator=g, dtype=torch.int8)
+    w = torch.randint(-127, 128, (N, Kd), generator=g, dtype=torch.int8)
+    a_s = (torch.rand(M, generator=g) * 1e-2 + 1e-3).half().float()
+    w_s = (torch.rand(N, generator=g) * 1e-3 + 1e-4)
+    bias16 = (torch.randn(N, generator=g) * 0.1).half()
+    cases = [(64, 5, 32, L.EPI_F32_MULADD, torch.float16, bias16, True),
+             (64, 7, 20, L.EPI_F32_MULADD, torch.float32, bias16.float(), True),
+             (32, 6, 32, L.EPI_REF_F16, torch.float16, bias16, True),
+             (128, 3, 32, L.EPI_REF_F16, torch.float32, None, True),
+             (64, 8, 24, L.EPI_SEQ_OUT, torch.bfloat16, bias16.bfloat16(), True),
+             (64, 8, 32, L.EPI_SEQ_OUT, torch.float16, bias16.float(), True),     # bias rounded to the output dtype
+             (32, 4, 32, L.EPI_SEQ_OUT, torch.float32, None, False),
+             (64, 0, 32, L.EPI_F32, torch.bfloat16, bias16, True),                # nothing to round: the plain GEMM
+             (64, 0, 32, L.EPI_SEQ_OUT, torch.float16, bias16, True),
+             (256, 9, 32, L.EPI_F32, torch.float16, bias16.float(), True)]
+    for cs, t, mab, epi, out, bias, per_row in cases:
+        tag = (shape, cs, t, mab, epi, out)
+        acc = O.chunk_matmul_i8(a, w, None, cs, t, mab)
+        sa = a_s if per_row else a_s[:1]
+        ref = _chunk_epilogue_ref(acc, sa if per_row else sa.expand(M), w_s, bias, epi, out)
+        y = K().matmul_chunk_dq(a.to(dev), w.to(dev), sa.to(dev), w_s.to(dev), None if bias is None else bias.to(dev),
+                                epi, out, chunk_size=cs, chunk_trun_bits=t, max_acc_bits=mab)
+        assert y.dtype == out and y.shape == (M, N), tag
+        assert torch.equal(y.cpu().view(torch.int32 if out == torch.float32 else torch.int16),
+                           ref.view(torch.int32 if out == torch.float32 else torch.int16)), tag
+    # one scale per tensor on the weight side too
+    acc = O.chunk_matmul_i8(a, w, None, 64, 5, 32)
+    ref = _chunk_epilogue_ref(acc, a_s, w_s[:1].expand(N), bias16, L.EPI_F32_MULADD, torch.float16)
+    y = K().matmul_chunk_dq(a.to(dev), w.to(dev), a_s.to(dev), w_s[:1].to(dev), bias16.to(dev), L.EPI_F32_MULADD,
+                            torch.float16, chunk_size=64, chunk_trun_bits=5)
+    assert torch.equal(y.cpu().view(torch.int16), ref.view(torch.int16))
+
+
+@pytest.mark.parametrize("dtype", [torch.float8_e4m3fn, torch.float16, torch.bfloat16, torch.float32])
+def test_matmul_chunk_fp_fused_epilogues_match_the_two_step_form(dev, dtype):
+    """fmsmo_matmul_chunk_fp_dq against fmsmo_matmul_chunk_fp followed by the reference's torch
+    expression on its fp32 accumulator: the same kernel accumulates, so the outputs are equal bit
+    for bit; on integer-valued operands (exact in any summation order) also against the oracle."""
+    from fms_mo_amd import _lib as L
+
+    g = gen(92)
+    for (M, N, Kd), cs, t, dl16 in (((70, 200, 1024), 64, 8, False), ((33, 96, 144), 32, 10, False),
+                                    ((150, 130, 512), 16 if dtype != torch.float8_e4m3fn else 32, 12, True)):
+        a = torch.randint(-6, 7, (M, Kd), generator=g).float().to(dtype)
+        w = torch.randint(-6, 7, (N, Kd), generator=g).float().to(dtype)
+        a_s = (torch.rand(M, generator=g) * 1e-1 + 1e-2).bfloat16().float()
+        w_s = (torch.rand(N, generator=g) * 1e-2 + 1e-3).bfloat16().float()
+        bias = (torch.randn(N, generator=g)).bfloat16()
+        acc_gpu = K().matmul_chunk(a.to(dev), w.to(dev), None, chunk_size=cs, chunk_trun_bits=t,
+                                   clamp_acc_to_dl16=dl16).cpu()
+        acc_ref = O.chunk_matmul_fp(a.float(), w.float(), None, cs, t, dl16)
+        assert torch.equal(acc_gpu, acc_ref)
+        for epi, out, b in ((L.EPI_SEQ_OUT, torch.bfloat16, bias), (L.EPI_SEQ_OUT, torch.float16, None),
+                            (L.EPI_SEQ_OUT, torch.float32, bias.float()), (L.EPI_F32_MULADD, torch.float16, bias),
+                            (L.EPI_F32, torch.float32, bias)):
+            ref = _chunk_epilogue_ref(acc_ref, a_s, w_s, b, epi, out)
+            y = K().matmul_chunk_dq(a.to(dev), w.to(dev), a_s.to(dev), w_s.to(dev), None if b is None else b.to(dev),
+                                    epi, out, chunk_size=cs, chunk_trun_bits=t, clamp_acc_to_dl16=dl16)
+            v = torch.int32 if out == torch.float32 else torch.int16
+            assert torch.equal(y.cpu().view(v), ref.view(v)), (dtype, M, N, Kd, epi, out)
+    # real-valued operands: equal to the unfused kernel's accumulator put through the same expression
+    a = torch.randn(96, 768, generator=g).to(dtype)
+    w = (torch.randn(160, 768, generator=g) * 0.5).to(dtype)
+    acc = K().matmul_chunk(a.to(dev), w.to(dev), None, chunk_size=64, chunk_trun_bits=9).cpu()
+    ref = _chunk_epilogue_ref(acc, a_s[:96], w_s[:1].expand(160), None, L.EPI_SEQ_OUT, torch.bfloat16)
+    y = K().matmul_chunk_dq(a.to(dev), w.to(dev), a_s[:96].to(dev), w_s[:1].to(dev), None, L.EPI_SEQ_OUT,
+                            torch.bfloat16, chunk_size=64, chunk_trun_bits=9)
+    assert torch.equal(y.cpu().view(torch.int16), ref.view(torch.int16))

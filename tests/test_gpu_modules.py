@@ -99,6 +99,41 @@ def test_deploy_module_random_layers_bit_exact_vs_oracle(dev):
         assert torch.equal(y.cpu().view(torch.int16), ref["y"].view(torch.int16)), tag
 
 
+@pytest.mark.parametrize("smoothq", [False, True])
+def test_deploy_module_iaddmm_FP_vs_oracle(dev, smoothq):
+    """use_int_kernel=False: the reference's emulation without an integer kernel
+    (iaddmm_FP, linear.py:1190-1211): torch.matmul on the dequantized operands, every buffer in
+    x's dtype.  The quantizer is still the device kernel: scales bit-exact, output within
+    rtol / atol 1e-2 of the oracle (an fp16 matmul's summation order is the library's)."""
+    from fms_mo_amd.modules.linear import QLinearINT8Deploy
+
+    B, S, K, N = 2, 37, 512, 384
+    m = make_qlinear(None, K, N, smoothq=smoothq)
+    x = outlier_x(B * S, K, 9).reshape(B, S, K)
+    act_scale = None
+    if smoothq:
+        act_scale = x.reshape(-1, K).float().abs().amax(dim=0)
+        m.set_act_scale(act_scale)
+    dep = QLinearINT8Deploy.from_fms_mo(m, use_int_kernel=False, use_dynamic_max_act_Qfunc=-1,
+                                        recalc_clipvals=False, target_device=dev).half()
+    assert dep.use_int_kernel is False and dep.iaddmm.__func__ is QLinearINT8Deploy.iaddmm_FP
+    for name in ("w_scale", "bias", "smoothq_scale"):
+        assert getattr(dep, name).dtype == torch.float16, name
+    y = dep(x.to(dev))
+    bufs = O.deploy_prepare(m.weight.detach(), m.bias.detach(), m.quantize_weight.clip_val, act_scale, 0.5)
+    bufs16 = {k: (v.half() if torch.is_tensor(v) and v.is_floating_point() else v) for k, v in bufs.items()}
+    ref = O.deploy_forward_fp(x, bufs16)
+    assert y.shape == (B, S, N) and y.dtype == torch.float16
+    x2 = x.reshape(-1, K)
+    _, s_ref, _ = O.quant_act_pertoken_i8(x2, bufs16["smoothq_scale"] if smoothq else None)
+    assert torch.equal(dep.input_scale.cpu().reshape(-1).float(), s_ref.float().reshape(-1))
+    torch.testing.assert_close(y.cpu().float(), ref.float(), rtol=1e-2, atol=1e-2)
+    # and it agrees with the integer-kernel module on the same layer at the same tolerance
+    dep_i = QLinearINT8Deploy.from_fms_mo(m, use_int_kernel="cutlass", use_dynamic_max_act_Qfunc=-1,
+                                          recalc_clipvals=False, target_device=dev)
+    torch.testing.assert_close(y.float(), dep_i(x.to(dev)).float(), rtol=1e-2, atol=1e-2)
+
+
 def test_deploy_module_converted_on_gpu_matches_within_tolerance(dev):
     """Converting on the GPU uses the GPU's pow / division roundings for the offline scales, so it
     is only tolerance-equal to the CPU-converted module."""
@@ -219,6 +254,29 @@ def test_linear_fpx_acc_dynamic_fp8_vs_oracle(dev, dl16):
     torch.testing.assert_close(y.float(), ref.float(), rtol=2e-2, atol=2e-2)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_linear_fpx_acc_per_tensor_fp8_vs_oracle(dev, dtype):
+    """dynamic_fp8="per_tensor": both scales come from the device-side abs-max (no torch
+    reductions, nothing read back); codes are the oracle's, so on a chunk of the whole reduction
+    without truncation the output is the oracle's up to the fp32 summation order."""
+    from fms_mo_amd import _lib as L
+    from fms_mo_amd import kernels as kn
+    from fms_mo_amd.modules.linear import LinearFPxAcc
+
+    lin = torch.nn.Linear(256, 192).to(dtype)
+    x = (torch.randn(40, 256, generator=gen(16)) * 2).to(dtype)
+    fpx = LinearFPxAcc.from_nn(lin.to(dev), trun_bits=8, chunk_size=64, dynamic_fp8="per_tensor")
+    y = fpx(x.to(dev)).cpu()
+    w = lin.weight.detach().cpu()
+    ref = O.fpxacc_forward(x, w, lin.bias.detach().cpu(), 8, 64, "per_tensor", False)
+    torch.testing.assert_close(y.float(), ref.float(), rtol=2e-2, atol=2e-2)
+    for t in (x, w):
+        q_ref, s_ref = O.fp8_quant_fpxacc(t, per_tensor=True)
+        q, s = kn.quant_act_fp8_dynamic(t.to(dev), L.FP8_FPXACC, True, 1e-5, True)
+        assert torch.equal(q.cpu().view(torch.uint8), q_ref.view(torch.uint8))
+        assert torch.equal(s.cpu().reshape(()), s_ref.float().reshape(()))
+
+
 def test_qlinear_int8_train_forward_vs_oracle(dev):
     from fms_mo_amd.modules.linear import QLinearINT8Train
 
@@ -257,6 +315,31 @@ def test_fp8_linear_vs_oracle(dev, cfg):
     exact = (qx.double() * s_x.double()) @ (m.weight.data.cpu().double() * m.weight_scale.data.cpu().double()).t() + b.double()
     torch.testing.assert_close(y.reshape(-1, 384).double(), exact, rtol=1e-2, atol=1e-2)
     torch.testing.assert_close(y.float(), ref.float(), rtol=3e-2, atol=3e-2)
+
+
+def test_fp8_linear_dynamic_scale_rule_attributes(dev):
+    """The floor and the division dtype of the dynamic activation scale are module attributes
+    (the two properties only torchao's source fixes); each setting matches the oracle with the
+    same arguments, per token and per tensor."""
+    from fms_mo_amd import kernels as kn
+    from fms_mo_amd.modules.fp8_linear import FP8Linear
+
+    g = gen(17)
+    W = 0.02 * torch.randn(256, 512, generator=g)
+    x = torch.randn(48, 512, generator=g).bfloat16()
+    x[3] = 0
+    for astrat in ("token", "tensor"):
+        m = FP8Linear.from_float(W, None, per_channel=False, act=astrat).to(dev)
+        for floor, in_xt in ((1e-12, False), (1e-5, True), (1e-3, False)):
+            m.dynamic_scale_floor, m.dynamic_scale_in_input_dtype = floor, in_xt
+            y = m(x.to(dev)).cpu()
+            s_x = O.fp8_dynamic_scale(x, floor, in_xt, astrat == "tensor")
+            ref, qx, _ = O.fp8_linear_forward(x, m.weight.data.cpu(), m.weight_scale.data.cpu(), None,
+                                              s_x if astrat == "token" else s_x.reshape(1))
+            q, s = kn.quant_act_fp8_dynamic(x.to(dev), 0, astrat == "tensor", floor, in_xt)
+            assert torch.equal(q.cpu().view(torch.uint8), qx.view(torch.uint8))
+            assert torch.equal(s.cpu(), s_x.reshape(-1))
+            torch.testing.assert_close(y.float(), ref.float(), rtol=3e-2, atol=3e-2)
 
 
 def test_swapped_mlp_replays_from_a_hip_graph(dev):

@@ -327,3 +327,28 @@ def test_bf16_quotient_from_reciprocal_rounds_like_ieee_division():
             t = (-q0.astype(np.float64) * s_.astype(np.float64) + e_.astype(np.float64)).astype(np.float32)
             q1 = (t.astype(np.float64) * r.astype(np.float64) + q0.astype(np.float64)).astype(np.float32)
             assert np.array_equal(to_bf16_bits(q1), exact), ulps
+
+
+def test_sawb_recompute_per_tensor_returns_the_sawb_integers_unguarded():
+    """recompute_weight_with_sawb, per tensor, when the statistics-aware clip is not below the
+    tensor maximum: the reference builds the guarded integers (fms_mo/utils/aiu_utils.py:196-199)
+    but returns the SAWB integers themselves (:235) beside the guarded clip value.  The writer and
+    the oracle reproduce that; per channel the guarded rows are what is returned."""
+    from fms_mo_amd.utils import aiu_utils as A
+
+    g = torch.Generator().manual_seed(5)
+    w = (0.01 * torch.randn(8, 8, generator=g)).half()
+    w[2, 3] = 1.0                          # one outlier among 64 weights: SAWB's clip exceeds it
+    w_int = torch.round(w.float() * 127).clamp(-127, 127)
+    assert w_int.std() < A.STD_THRESHOLD
+    new_sd = {}
+    got, recomputed = A.recompute_weight_with_sawb(w, w_int.to(w.dtype), False, None, "lin", new_sd)
+    ref_int, ref_cv = O.aiu_recompute_narrow(w, w_int.to(w.dtype), False)
+    clip = O.sawb_clip(w.float(), 8, perCh=False)
+    assert recomputed and clip > w.abs().max()                      # the case in question
+    assert torch.equal(new_sd["lin.quantize_weight.clip_val"], ref_cv)
+    assert ref_cv.item() == w.abs().max().item()                    # the clip value is guarded ...
+    assert torch.equal(got, ref_int)
+    assert torch.equal(got, O.sawb_zero_forward(w.float(), clip, 8, dequantize=False))   # ... the integers are not
+    assert not torch.equal(got, w_int)
+    assert got.abs().max() < 127                                    # quantized against the larger clip

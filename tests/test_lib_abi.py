@@ -19,6 +19,7 @@ def declared_symbols():
 def test_header_declares_the_expected_entry_points():
     syms = declared_symbols()
     for s in ["fmsmo_quant_act_i8_pertoken", "fmsmo_quant_act_i8_static", "fmsmo_quant_act_fp8_pertoken",
+              "fmsmo_quant_act_fp8_dynamic",
               "fmsmo_gemm_i8_i32", "fmsmo_gemm_i8_i32_ws", "fmsmo_gemm_i8_dq", "fmsmo_gemm_fp8_dq", "fmsmo_gemv_i8_dq",
               "fmsmo_gemv_fp8_dq", "fmsmo_matmul_chunk_i8", "fmsmo_matmul_chunk_fp",
               "fmsmo_grouped_gemm_i8_dq", "fmsmo_quant_weight_i8", "fmsmo_absmax_cols",
@@ -83,6 +84,14 @@ def test_argument_validation_without_a_gpu():
     assert lib.fmsmo_fake_quant_fp8(p, 0, 64, 7, None, p, 64, None, 0, None, None, 1, 64, None) == 4  # mode
     assert lib.fmsmo_gemm_i8_dq_noalloc(None, 64, p, 64, p, 1, p, 1, None, 0, 0, p, 0, 64, 1, 1, 64, None) == 1
     assert lib.fmsmo_gemm_i8_dq_noalloc(p, 64, p, 64, p, 1, p, 1, None, 0, 9, p, 0, 64, 1, 1, 64, None) == 4  # epilogue
+    # (the call above is rejected before the static scratch is looked up: no device is touched)
+    F32 = 2
+    assert lib.fmsmo_quant_act_fp8_dynamic(None, 0, 64, 0, 0, None, 1e-12, F32, p, 64, p, 1, 64, None) == 1
+    assert lib.fmsmo_quant_act_fp8_dynamic(p, 0, 64, 0, 1, None, 1e-12, F32, p, 64, p, 1, 64, None) == 1  # no col_amax
+    assert lib.fmsmo_quant_act_fp8_dynamic(p, 0, 64, 0, 0, None, 0.0, F32, p, 64, p, 1, 64, None) == 4    # floor <= 0
+    assert lib.fmsmo_quant_act_fp8_dynamic(p, 0, 64, 0, 0, None, 1e-12, 0, p, 64, p, 1, 64, None) == 4    # fp16 floor -> 0
+    assert lib.fmsmo_quant_act_fp8_dynamic(p, 0, 64, 0, 0, None, 1e-5, 1, p, 64, p, 1, 64, None) == 4     # not x's dtype
+    assert lib.fmsmo_quant_act_fp8_dynamic(p, 0, 64, 0, 0, None, 1e-5, 0, p, 64, p, 0, 64, None) == 0     # empty
 
 
 def test_python_wrapper_raises_on_cpu_tensors():
@@ -197,3 +206,23 @@ def test_gemm_plan_is_host_logic():
         K.gemm_plan(0, 4096, 4096)
     with pytest.raises(_lib.FmsMoHipError):
         K.gemm_plan(128, 128, 100)
+
+
+def test_plan_of_the_entry_point_that_allocates_nothing():
+    """with_workspace = 2 describes fmsmo_gemm_i8_dq_noalloc: the split that fits the 16 MiB static
+    scratch where the preferred one does not."""
+    from fms_mo_amd import _lib
+
+    lib = _lib.load()
+    k, tm, tn, sp = (ctypes.c_int() for _ in range(4))
+    # 512 x 4096 x 14336: four register-staged slices want 32 MiB; the scratch holds two 128 x 128 ones
+    assert lib.fmsmo_gemm_plan(512, 4096, 14336, 1, ctypes.byref(k), ctypes.byref(tm), ctypes.byref(tn), ctypes.byref(sp)) == 0
+    pref = (k.value, tm.value, tn.value, sp.value)
+    assert lib.fmsmo_gemm_plan(512, 4096, 14336, 2, ctypes.byref(k), ctypes.byref(tm), ctypes.byref(tn), ctypes.byref(sp)) == 0
+    fit = (k.value, tm.value, tn.value, sp.value)
+    assert pref[3] * 512 * 4096 * 4 > 16 * 2 ** 20 >= fit[3] * 512 * 4096 * 4 and fit[3] >= 2
+    assert fit != pref and fit[0] == _lib.PLAN_TILE_LDS_DMA
+    # a shape that needs no scratch reads the same in every mode
+    for mode in (0, 1, 2):
+        assert lib.fmsmo_gemm_plan(4, 4096, 4096, mode, ctypes.byref(k), ctypes.byref(tm), ctypes.byref(tn), ctypes.byref(sp)) == 0
+        assert k.value == _lib.PLAN_DECODE

@@ -283,10 +283,89 @@ def test_fp8_quantizers_closed_forms():
     qd, _ = O.fp8_quant_fpxacc(x * 1e-3 + 0, dl8=True)
     f = qd.float()
     assert torch.all((f == 0) | (f.abs() >= O.DL8_MIN))
+
+
+def _fp8_scale_properties(x, s, floor, exact):
+    """The properties a symmetric per-row e4m3 scale has whatever library computes it; returns the
+    list of those that fail.  ``exact``: the division ran on the fp32-widened abs-max."""
+    bad = []
+    xf = x.to(torch.float32)
+    amax = xf.abs().amax(dim=-1, keepdim=True)
+    live = (amax > 448 * floor * 1.01).reshape(-1)       # rows the floor does not govern
+    if s.dtype != torch.float32:
+        bad.append("dtype")
+    s32 = s.to(torch.float32).reshape(-1, 1)
+    q = O.fp8_quant_static(x, s32).to(torch.float32)
+    if not torch.all(q[live].abs().amax(dim=-1) == 448):
+        bad.append("row maximum on the top code")
+    # nothing beyond the top code before the clamp: quotients stay within one e4m3 rounding of 448
+    if not torch.all((xf / s32)[live].abs().amax(dim=-1) < 464):
+        bad.append("no quotient beyond the top code")
+    # the top code dequantizes to the row maximum: within an fp32 rounding when the division was
+    # exact, within half a unit in the last place of x's dtype when it ran there
+    err = (448 * s32.double() - amax.double()).abs()
+    if exact:
+        tol = amax.double() * 2.0 ** -23
+    else:
+        st = s32.to(x.dtype)                                  # spacing of x's dtype at the scale
+        ulp = ((st.view(torch.int16) + 1).view(x.dtype).double() - st.double()).abs()
+        tol = 448 * 0.5 * ulp * 1.001
+    if not torch.all((err <= tol)[live]):
+        bad.append("top code dequantizes to the row maximum")
+    zero = (amax == 0).reshape(-1)
+    if zero.any() and not (torch.all(s32[zero] == torch.tensor(floor, dtype=torch.float32))
+                           and torch.all(q[zero] == 0)):
+        bad.append("zero rows")
+    return bad
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+def test_fp8_dynamic_scale_pinned_by_invariants(dtype):
+    """FP8Linear's dynamic scale is formed inside torchao (absent).  The checks below are not the
+    oracle's formula retyped: they are what any correct symmetric e4m3 scale satisfies, and each
+    plausible wrong rule is shown to fail at least one.  Two properties stay torchao's own and are
+    arguments of the oracle and of the kernel (fmsmo_quant_act_fp8_dynamic): the floor's value and
+    the dtype the division runs in."""
+    g = gen(77)
+    x = (torch.randn(64, 256, generator=g) * torch.logspace(-3, 3, 64).reshape(-1, 1)).to(dtype)
+    x[5] = 0
+    x[9, 3] = x[9].abs().max() * -2          # the maximum is a negative element
+    for floor in (1e-12, 1e-5):
+        assert _fp8_scale_properties(x, O.fp8_dynamic_scale(x, floor), floor, True) == []
+    if dtype != torch.float32:
+        s_t = O.fp8_dynamic_scale(x, 1e-5, in_x_dtype=True)
+        assert _fp8_scale_properties(x, s_t, float(torch.tensor(1e-5).to(dtype)), False) == []
+        assert torch.equal(s_t, s_t.to(dtype).float())            # a value of x's dtype, widened
+    # wrong rules, each caught
+    amax = x.float().abs().amax(dim=-1, keepdim=True)
+    wrong = {
+        "e4m3fnuz maximum": (amax / 240).clamp(min=1e-12),
+        "int8 levels": (amax / 127).clamp(min=1e-12),
+        "e5m2 maximum": (amax / 57344).clamp(min=1e-12),
+        "reciprocal": (448 / amax.clamp(min=1e-12)),
+        "no floor": amax / 448,
+    }
+    if dtype != torch.float32:
+        wrong["left in x's dtype"] = (x.abs().amax(dim=-1, keepdim=True) / 448).clamp(min=1e-12)
+        wrong["rounded to x's dtype"] = (amax / 448).clamp(min=1e-12).to(dtype).float()
+    for name, s_bad in wrong.items():
+        if name == "rounded to x's dtype" and dtype == torch.float16:
+            # fp16 rounds the floor itself to zero; the live rows still show the rounding
+            s_bad = s_bad.clamp(min=1e-12)
+        assert _fp8_scale_properties(x, s_bad, 1e-12, True) != [], name
+    # per tensor: the same properties for the flattened tensor
+    s_pt = O.fp8_dynamic_scale(x, per_tensor=True)
+    assert s_pt.numel() == 1
+    assert _fp8_scale_properties(x.reshape(1, -1), s_pt.reshape(1, 1), 1e-12, True) == []
+
+
+def test_fp8_dynamic_scale_defaults():
+    x = (torch.randn(6, 128, generator=gen(30)) * 3).bfloat16()
     sd = O.fp8_dynamic_scale(x)
-    assert sd.dtype == torch.float32 and torch.allclose(sd, x.float().abs().amax(dim=1, keepdim=True) / 448)
+    assert sd.dtype == torch.float32 and sd.shape == (6, 1)
     z = torch.zeros(2, 16, dtype=torch.bfloat16)
     assert O.fp8_dynamic_scale(z).min().item() == pytest.approx(1e-12)
+    assert O.fp8_dynamic_scale(z, floor=1e-5).min().item() == pytest.approx(1e-5)
 
 
 def test_scaled_mm_cpu_is_plain_dequantized_matmul():

@@ -436,3 +436,26 @@ def test_deploy_prepare_with_sawb_weights_dequantized_product_identity():
     assert torch.equal(out["q_x"], q)
     exact = (q.double() * s.double()) @ deq.double().t() + b.double()
     torch.testing.assert_close(out["y"].double(), exact, rtol=2e-3, atol=2e-3)
+
+
+def test_triton_kernel_forward_reduces_to_the_plain_and_chunked_forms():
+    """deploy_forward_triton: without truncation it is the plain forward (chunks of an exact
+    integer sum add up to the sum); with truncation its accumulator is the chunked kernel's, whose
+    every chunk sum has its low t bits cleared, and the epilogue is the fp16-scale one."""
+    g = torch.Generator().manual_seed(71)
+    K, N = 256, 96
+    W = (0.05 * torch.randn(N, K, generator=g)).half()
+    b = (0.01 * torch.randn(N, generator=g)).half()
+    x = torch.randn(20, K, generator=g).half()
+    st = O.deploy_prepare_general(W, b, O.qmax_perch_clipval(W).float(), use_dynamic_max_act_Qfunc=-1)
+    plain = O.deploy_forward_general(x, st)
+    t0 = O.deploy_forward_triton(x, st, chunk_size=64, truncate_lsb=0)
+    assert torch.equal(t0["acc"], plain["acc"]) and torch.equal(t0["y"], plain["y"])
+    t8 = O.deploy_forward_triton(x, st, chunk_size=64, truncate_lsb=6)
+    assert torch.all(t8["acc"] % 64 == 0) and not torch.equal(t8["acc"], plain["acc"])
+    # every chunk contributes at most 2^(t-1) of rounding error
+    assert (t8["acc"] - plain["acc"]).abs().max() <= (K // 64) * 32
+    assert torch.equal(t8["y"], O.epilogue_ref(t8["acc"], t8["input_scale"], st["w_scale"], st["bias"]))
+    # a chunk size the kernel does not take falls back to its minimum of 32
+    t_odd = O.deploy_forward_triton(x, st, chunk_size=48, truncate_lsb=6)
+    assert torch.equal(t_odd["acc"], O.chunk_matmul_i8(t8["q_x"], st["weight"], None, 32, 6, 32))
