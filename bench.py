@@ -293,6 +293,102 @@ def vendor_int_mm(torch, K, layers):
     return res
 
 
+def power_account(torch, K, dev, layers, seconds=1.2):
+    """Evidence for how far the power limit, not the schedule, holds the GEMMs back: each loop below
+    runs for about `seconds` while a thread polls the amdgpu driver's hwmon sensors (power1_input:
+    socket power; freq1_input: the core clock the driver reports).  Loops: the four headline GEMMs through
+    fmsmo_gemm_i8_i32 and through torch._int_mm (hipBLASLt), each on the step's quantized operands
+    and on all-zero operands of the same shape; and the GEMM kernels' matrix instructions alone
+    (fmsmo_debug_mfma_loop: registers only, every SIMD busy) on Gaussian codes and on zeros -- the
+    ceiling of any schedule of those instructions on such operand bits."""
+    import glob
+    import threading
+
+    power_files = sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_input")
+                         + glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_average"))
+    freq_files = sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/freq1_input"))
+
+    def sample_while(fn):
+        samples, stop = [], [False]
+
+        def poll():
+            # the amdgpu driver's own sensors: socket power in microwatts, core clock in Hz
+            while not stop[0]:
+                try:
+                    w = float(open(power_files[0]).read()) / 1e6 if power_files else None
+                    mhz = float(open(freq_files[0]).read()) / 1e6 if freq_files else None
+                    samples.append((w, mhz))
+                except Exception as e:  # the sensors are evidence, not a dependency
+                    samples.append(("error: " + str(e)[:80], None))
+                    return
+                time.sleep(0.02)
+
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        th = threading.Thread(target=poll)
+        th.start()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0, n = time.perf_counter(), 0
+        e0.record()
+        while time.perf_counter() - t0 < seconds:
+            for _ in range(20):
+                fn()
+            n += 20
+            torch.cuda.synchronize()
+        e1.record()
+        torch.cuda.synchronize()
+        stop[0] = True
+        th.join()
+        ms = e0.elapsed_time(e1) / n
+        good = [s_ for s_ in samples[len(samples) // 4:] if isinstance(s_[0], float)]   # after the ramp
+        out = {"ms": round(ms, 4), "sensor_samples": len(good)}
+        if good:
+            out["socket_power_w"] = round(sum(s_[0] for s_ in good) / len(good), 1)
+            sc = [s_[1] for s_ in good if s_[1]]
+            if sc:
+                out["driver_sclk_mhz"] = round(sum(sc) / len(sc))
+        elif samples:
+            out["sensors"] = str(samples[0][0])
+        return out
+
+    res = {}
+    for (name, k, n), L_ in zip(LLAMA3_8B, layers):
+        ops = 2.0 * M_TOKENS * k * n
+        q, _ = K.quant_act_i8_pertoken(L_["x"], L_["smooth"])
+        zq, zw = torch.zeros_like(q), torch.zeros_like(L_["w"])
+        for label, a, w in (("step_operands", q, L_["w"]), ("zero_operands", zq, zw)):
+            wt = w.t()
+            for kname, fn in (("fmsmo_gemm_i8_i32", lambda: K.gemm_i8_i32(a, w)), ("torch_int_mm", lambda: torch._int_mm(a, wt))):
+                try:
+                    r = sample_while(fn)
+                    r["tops"] = round(ops / r["ms"] / 1e9, 1)
+                except Exception as e:
+                    r = {"error": str(e)[:160]}
+                res[f"{name}_{label}_{kname}"] = r
+        del zq, zw
+    g = torch.Generator(device=dev).manual_seed(11)
+    clk = torch.zeros(2, dtype=torch.int64, device=dev)
+    gauss = torch.randn(1 << 25, device=dev, generator=g)
+    datas = {"i8_gaussian_sigma29": (gauss * 29).clamp_(-127, 127).round_().to(torch.int8),
+             "i8_zeros": torch.zeros(1 << 25, dtype=torch.int8, device=dev),
+             "e4m3_gaussian_full_range": (gauss * (448.0 / 4.5)).clamp_(-448, 448).to(torch.float8_e4m3fn),
+             "e4m3_zeros": torch.zeros(1 << 25, dtype=torch.int8, device=dev).view(torch.float8_e4m3fn)}
+    for label, d in datas.items():
+        ops = [0.0]
+
+        def fn():
+            ops[0] = K.mfma_loop(d, 2000, clk)
+
+        r = sample_while(fn)
+        c = clk.cpu().tolist()
+        r["tops"] = round(ops[0] / r["ms"] / 1e9, 1)
+        r["frac_peak"] = round(ops[0] / r["ms"] / 1e9 / PEAK_INT8_TOPS, 4)
+        r["core_clock_mhz"] = round(c[0] / (c[1] / 100.0)) if c[1] else None
+        res["mfma_only_" + label] = r
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -466,6 +562,7 @@ def extras(torch, K, dev, layers):
     sample_ops = sum(2.0 * 2048 * k * n for _, k, n in LLAMA3_8B)
     res["cpu_baseline_sample_on_gpu_M2048"] = {"ms": round(ms, 4), "tops": round(sample_ops / ms / 1e9, 1)}
     res["vendor"] = vendor_int_mm(torch, K, layers)
+    res["power_account"] = power_account(torch, K, dev, layers)
     # batches of a few hundred rows (split-K territory) beside the vendor GEMM, launches replayed
     # from a HIP graph, weights rotated over > 300 MB: this library's fused-dequant GEMM, its raw
     # int32 GEMM and torch._int_mm (int32 out, no dequantization) on the same operands

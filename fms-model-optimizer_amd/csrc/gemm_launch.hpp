@@ -132,10 +132,6 @@ void launch_rs(const GemmArgs& g0, const Epi& epi, hipStream_t st) {
   if (!GROUPED) g.grid_m = div_up(g.M, 256);
   g.group_m = 4;
   dim3 grid((unsigned)(g.grid_m * g.grid_n)), block(256);
-  // three rounds or more over the 256 compute units: staggered start (FMSMO_SKEW=n sets the step
-  // in units of 256 cycles per phase, 0 switches it off; tuning aid)
-  static const int env_skew = getenv("FMSMO_SKEW") ? atoi(getenv("FMSMO_SKEW")) : -1;
-  g.skew = (long)g.grid_m * g.grid_n >= 3 * 256 ? (env_skew >= 0 ? env_skew : 0) : 0;
   hipLaunchKernelGGL((gemm_rs_kernel<OP, Epi, GROUPED, BN>), grid, block, 0, st, g, epi);
 }
 

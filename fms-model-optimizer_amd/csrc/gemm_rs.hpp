@@ -84,15 +84,6 @@ __global__ __launch_bounds__(256, 1) void gemm_rs_kernel(GemmArgs g, Epi epi) {
   }
   const int col_lo = tile_n * BN;
 
-  // Launches of several rounds: all compute units would finish their tiles together and store
-  // 128 KiB each at once, an HBM-bound burst of several microseconds per round during which no
-  // matrix unit works, while the memory idles during the K loops.  Starting the first round in
-  // eight phases a fraction of a microsecond apart keeps the units out of step for the whole
-  // launch (equal tiles, equal periods), so a unit's stores overlap the other units' K loops.
-  if (g.skew > 0 && blockIdx.x < 256) {
-    const int phase = (blockIdx.x >> 3) & 7;
-    for (int i = 0; i < phase * g.skew; ++i) __builtin_amdgcn_s_sleep(4);
-  }
   if (blockIdx.x == 0 && tid == 0 && g.clk) { g.clk[0] = clock64(); g.clk[1] = wall_clock64(); }
   // ---- global -> register staging: thread -> (row = tid / 8 + 32 j, 16-byte chunk = tid % 8)
   const int ld_row = tid >> 3, ld_chunk = tid & 7;

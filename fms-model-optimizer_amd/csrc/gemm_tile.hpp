@@ -40,8 +40,6 @@ struct GemmArgs {
   int64_t lda_e;       // uniform groups: bytes between groups in A (rows * lda for stacked batches,
                        // the K slice length when the groups are slices of one reduction)
   int k_rotate;  // register-staged kernel: block b starts its reduction at slab (b * k_rotate) % slabs
-  int skew;      // register-staged kernel: the blocks of the first round start (b / 8 % 8) * skew * 256
-                 // clock cycles late, so that the compute units do not all store their tiles at once
   // optional clock probe (register-staged kernel): block 0 stores {core clock counter, 100 MHz
   // wall clock} at its start, after its K loop and after its epilogue; null = off
   unsigned long long* clk;

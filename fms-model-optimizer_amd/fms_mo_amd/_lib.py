@@ -66,6 +66,7 @@ SIGNATURES = {
     "fmsmo_zero_shift_bias": [_P, _L, _P, _L, _P, _F, _P, _I, _P, _L, _L, _P],
     "fmsmo_debug_clock_probe": [_P],
     "fmsmo_debug_stream_read": [_P, _L, _P, _P],
+    "fmsmo_debug_mfma_loop": [_I, _P, _L, _I, _P, _P, _P],
     "fmsmo_gemm_plan": [_L, _L, _L, _I, _P, _P, _P, _P],
 }
 OTHER = {

@@ -309,6 +309,20 @@ def stream_read(t, sink):
     L.call("fmsmo_debug_stream_read", t.data_ptr(), t.numel() * t.element_size(), sink.data_ptr(), _stream(t))
 
 
+def mfma_loop(data, iters, clk=None):
+    """Diagnostic: the GEMM kernels' matrix instructions alone, fed from registers loaded once from
+    `data` (int8 or float8_e4m3fn, contiguous; see fmsmo_debug_mfma_loop).  Returns the operations
+    of one launch; `clk` (int64 [2] on the GPU) receives block 0's {core cycles, 100 MHz ticks}."""
+    _need_gpu(data, clk)
+    if data.dtype not in (torch.int8, torch.float8_e4m3fn) or not data.is_contiguous() or data.numel() % 4:
+        raise ValueError("data must be a contiguous int8 / float8_e4m3fn tensor of a multiple of 4 elements")
+    sink = torch.zeros(1, dtype=torch.float32, device=data.device)
+    with _dev(data):
+        L.call("fmsmo_debug_mfma_loop", _OPDT[data.dtype], data.data_ptr(), data.numel(), int(iters), _ptr(clk),
+               sink.data_ptr(), _stream(data))
+    return 1024.0 * iters * 2 * 16 * 2 * 32 * 32 * 64
+
+
 def core_clock_mhz(buf):
     """Average core clock (MHz) over the life of the probed block: core cycles per tick of the
     constant 100 MHz counter, start of the block to the end of its epilogue."""

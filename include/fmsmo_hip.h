@@ -97,6 +97,21 @@ int fmsmo_debug_clock_probe(uint64_t* dev6);
  */
 int fmsmo_debug_stream_read(const void* p, int64_t bytes, int32_t* sink, fmsmo_stream_t stream);
 
+/*
+ * Diagnostic with no counterpart in the reference: the matrix instructions of the GEMM kernels
+ * alone.  256 blocks of 4 waves, one wave per SIMD of every compute unit; each wave loads two
+ * sets of 4 + 4 operand fragments (64 bytes of K per fragment and lane, 512 bytes per lane in all)
+ * from `data` (device memory, `bytes` a multiple of 4; indices wrap) and then issues nothing but
+ * MFMAs from registers: per iteration 2 x 16 blocks of 32 x 32 x 64, as v_mfma_i32_32x32x32_i8
+ * pairs (op_dtype = FMSMO_OP_I8) or v_mfma_f32_32x32x64_f8f6f4 (FMSMO_OP_E4M3).  Operations per
+ * launch: 1024 waves x iters x 2 x 16 x 2 x 32 x 32 x 64.  clk2 (device, may be NULL) receives
+ * {core clock cycles, ticks of the 100 MHz counter} of block 0's loop.  What this loop reaches on
+ * given operand bits is the ceiling, under the part's power limit, of any kernel made of these
+ * instructions on such operands.  sink: 4 bytes of device memory, practically never written.
+ */
+int fmsmo_debug_mfma_loop(int op_dtype, const void* data, int64_t bytes, int iters, uint64_t* clk2,
+                          float* sink, fmsmo_stream_t stream);
+
 /* ------------------------------------------------------------------------------------------
  * 1. Activation quantizers (one pass over x: read 2-4 B, write 1 B per element).
  * ------------------------------------------------------------------------------------------ */

@@ -26,7 +26,7 @@ def test_header_declares_the_expected_entry_points():
               "fmsmo_quant_act_i8_mulscale", "fmsmo_zero_shift_bias", "fmsmo_quant_i8_affine",
               "fmsmo_bmm_i8_dq", "fmsmo_bmm_fp8_dq", "fmsmo_gemm_i8_dq_ws", "fmsmo_gemm_fp8_dq_ws", "fmsmo_gemm_i8_dq_noalloc",
               "fmsmo_gemm_tail_columns", "fmsmo_quant_act_i8_static_t", "fmsmo_quant_act_i8_dynamic", "fmsmo_fake_quant_fp8",
-              "fmsmo_gemm_workspace_bytes", "fmsmo_decode_linear_i8", "fmsmo_decode_linear_fp8", "fmsmo_decode_linear_ok", "fmsmo_decode_linear_f32s_ok", "fmsmo_debug_clock_probe", "fmsmo_debug_stream_read", "fmsmo_gemm_plan", "fmsmo_abi_version", "fmsmo_status_str", "fmsmo_last_error"]:
+              "fmsmo_gemm_workspace_bytes", "fmsmo_decode_linear_i8", "fmsmo_decode_linear_fp8", "fmsmo_decode_linear_ok", "fmsmo_decode_linear_f32s_ok", "fmsmo_debug_clock_probe", "fmsmo_debug_stream_read", "fmsmo_debug_mfma_loop", "fmsmo_matmul_chunk_i8_dq", "fmsmo_matmul_chunk_fp_dq", "fmsmo_gemm_plan", "fmsmo_abi_version", "fmsmo_status_str", "fmsmo_last_error"]:
         assert s in syms
 
 
@@ -75,6 +75,14 @@ def test_argument_validation_without_a_gpu():
     assert lib.fmsmo_debug_stream_read(None, 64, p, None) == 1
     assert lib.fmsmo_debug_stream_read(p, 24, p, None) == 2 and lib.fmsmo_debug_stream_read(p, 0, p, None) == 2
     assert lib.fmsmo_debug_stream_read(p + 1, 64, p, None) == 3
+    assert lib.fmsmo_debug_mfma_loop(0, None, 64, 1, None, p, None) == 1
+    assert lib.fmsmo_debug_mfma_loop(0, p, 64, 0, None, p, None) == 2 and lib.fmsmo_debug_mfma_loop(2, p, 64, 1, None, p, None) == 4
+    # the fused chunked matmuls validate like the plain ones, plus their epilogue arguments
+    assert lib.fmsmo_matmul_chunk_i8_dq(p, 64, p, 64, None, 1, p, 1, None, 0, 3, p, 0, 64, 1, 1, 64, 64, 0, 32, 1, None) == 1
+    assert lib.fmsmo_matmul_chunk_i8_dq(p, 64, p, 64, p, 1, p, 1, None, 0, 7, p, 0, 64, 1, 1, 64, 64, 0, 32, 1, None) == 4  # epilogue
+    assert lib.fmsmo_matmul_chunk_i8_dq(p, 64, p, 64, p, 3, p, 1, None, 0, 3, p, 0, 64, 1, 1, 64, 64, 0, 32, 1, None) == 2  # a_scale_n
+    assert lib.fmsmo_matmul_chunk_fp_dq(p, 64, p, 64, 0, p, 1, p, 1, None, 0, 3, p, 0, 64, 1, 1, 64, 64, 0, 0, 1, None) == 4  # op dtype
+    assert lib.fmsmo_matmul_chunk_fp_dq(p, 64, p, 64, 2, p, 1, p, 1, None, 0, 3, p, 0, 64, 1, 1, 64, 24, 0, 0, 1, None) == 4  # chunk
     assert lib.fmsmo_quant_act_i8_static_t(None, 0, 64, 0, 0, 1.0, 0.0, 0, 0.0, 0.0, p, 64, 1, 64, None) == 1
     assert lib.fmsmo_quant_act_i8_static_t(p, 0, 64, 9, 0, 1.0, 0.0, 0, 0.0, 0.0, p, 64, 1, 64, None) == 4  # mode
     assert lib.fmsmo_quant_act_i8_static_t(p, 0, 32, 0, 0, 1.0, 0.0, 0, 0.0, 0.0, p, 64, 1, 64, None) == 2  # ldx < K
