@@ -122,10 +122,22 @@ def gemm_sources_sha16():
 GRANITE_8B = [("qkv", 4096, 6144), ("o", 4096, 4096), ("gate_up", 4096, 25600), ("down", 12800, 4096)]
 
 
-def time_events(torch, fn, iters=30, warm=5):
-    """Average HIP-event time (ms) of fn over iters eager calls on the current stream."""
+def time_events(torch, fn, iters=30, warm=5, min_seconds=0.0):
+    """Average HIP-event time (ms) of fn over iters eager calls on the current stream; with
+    min_seconds the number of calls is raised so that the timed region lasts that long (the part
+    settles its clock over milliseconds: a burst of twenty launches is timed at whatever clock the
+    work before it left behind)."""
     for _ in range(warm):
         fn()
+    if min_seconds > 0:
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(5):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        iters = max(iters, int(min_seconds * 1e3 / max(e0.elapsed_time(e1) / 5, 1e-3)))
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     torch.cuda.synchronize()
     e0.record()
@@ -157,7 +169,8 @@ def fp8_rooflines(torch, K, dev):
             w8 = (w / (ws[:, None] if per_channel else ws)).clamp(-448, 448).to(torch.float8_e4m3fn)
             q, s = K.quant_act_fp8_pertoken(x, L.FP8_LINEAR)
             K.clock_probe(clk)
-            ms = time_events(torch, lambda: K.gemm_fp8_dq(q, w8, s, ws, None, out_dtype=torch.bfloat16), iters=20, warm=4)
+            ms = time_events(torch, lambda: K.gemm_fp8_dq(q, w8, s, ws, None, out_dtype=torch.bfloat16), iters=20, warm=4,
+                             min_seconds=0.15)
             K.clock_probe(None)
             ops = 2.0 * M * k * n
             tot_ms += ms
@@ -175,7 +188,8 @@ def fp8_rooflines(torch, K, dev):
             for vlabel, sa, sb in (("vendor_scaled_mm_rowwise", sa_row, sb_row), ("vendor_scaled_mm_tensorwise", one, one)):
                 try:
                     vms = time_events(torch, lambda: torch._scaled_mm(q, w8.t(), scale_a=sa, scale_b=sb,
-                                                                       out_dtype=torch.bfloat16), iters=20, warm=4)
+                                                                       out_dtype=torch.bfloat16), iters=20, warm=4,
+                                      min_seconds=0.15)
                     per[name][vlabel] = {"ms": round(vms, 4), "tflops": round(ops / (vms * 1e-3) / 1e12, 1)}
                     vend[vlabel] = vend.get(vlabel, 0.0) + vms
                 except Exception as e:  # the vendor path is evidence, not a dependency

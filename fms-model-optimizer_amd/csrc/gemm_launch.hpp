@@ -132,7 +132,18 @@ void launch_rs(const GemmArgs& g0, const Epi& epi, hipStream_t st) {
   if (!GROUPED) g.grid_m = div_up(g.M, 256);
   g.group_m = 4;
   dim3 grid((unsigned)(g.grid_m * g.grid_n)), block(256);
-  hipLaunchKernelGGL((gemm_rs_kernel<OP, Epi, GROUPED, BN>), grid, block, 0, st, g, epi);
+  if constexpr (OP == MMA_FP8) {
+    // e4m3: the 16 x 16 x 128 matrix instruction (more work per joule under the power limit: the
+    // four Llama-3-8B shapes at 4096 rows +1 ... +4 %) unless FMSMO_MFMA16=0 asks for 32 x 32 x 64
+    // (tuning aid).  int8 stays with 32 x 32 x 32: its 16 x 16 x 64 form issues four times as many
+    // instructions per slab and lost 3 ... 25 % in this kernel.
+    static const char* force16 = getenv("FMSMO_MFMA16");
+    if (!(force16 && force16[0] == '0')) {
+      hipLaunchKernelGGL((gemm_rs_kernel<OP, Epi, GROUPED, BN, true>), grid, block, 0, st, g, epi);
+      return;
+    }
+  }
+  hipLaunchKernelGGL((gemm_rs_kernel<OP, Epi, GROUPED, BN, false>), grid, block, 0, st, g, epi);
 }
 
 // Reduction of exactly 128 bytes (attention scores): persistent blocks over 128 x 256 tiles, two

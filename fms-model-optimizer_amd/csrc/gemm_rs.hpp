@@ -19,21 +19,44 @@
 
 namespace fmsmo {
 
+// The 16 x 16 x 128 form of the e4m3 matrix instruction: a lane holds row lane % 16 and the K group
+// lane / 16 (four groups of 32 bytes), so one instruction covers a whole 128-byte slab.  Under the
+// part's power limit it does more work per joule than 32 x 32 x 64 (the same loop of matrix
+// instructions alone on the same Gaussian codes: 4570 against 4000 TFLOP/s), and a GEMM of this
+// size runs against that limit, not against issue slots.  (int8 has 16 x 16 x 64, 3630 against
+// 3430 TOPS in that loop; in this kernel its four times as many instructions per slab lost
+// 3 ... 25 %, so int8 keeps the 32 x 32 x 32 form and there is no int8 specialization.)
+template <int OP>
+struct Mma16;
+template <>
+struct Mma16<MMA_FP8> {
+  typedef v8i Frag;
+  typedef v4f Acc;
+  typedef float Elem;
+  static constexpr int KSTEP = 128;
+  __device__ static __forceinline__ Acc mma(const Frag& a, const Frag& b, const Acc& c) {
+    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0);
+  }
+};
+
 // (A reduction of a single slab, K == 128, has its own kernel: gemm_k128.hpp.)
-template <int OP, class Epi, bool GROUPED = false, int BN_ = 256>
+template <int OP, class Epi, bool GROUPED = false, int BN_ = 256, bool B16 = false>
 __global__ __launch_bounds__(256, 1) void gemm_rs_kernel(GemmArgs g, Epi epi) {
 #if defined(__HIP_DEVICE_COMPILE__)
-  typedef Mma<OP> MM;
+  typedef typename std::conditional<B16, Mma16<OP>, Mma<OP>>::type MM;
   typedef typename MM::Frag Frag;
   typedef typename MM::Acc Acc;
   static_assert(BN_ == 256 || BN_ == 192 || BN_ == 128, "tile width");
   constexpr int BM = 256, BN = BN_, BK = 128, CPR = 8;
-  constexpr int TM = BM / 2, TN = BN / 2, FM = TM / 32, FN = TN / 32;
-  constexpr int NKS = BK / MM::KSTEP;   // MFMA k-steps per slab (int8 4, e4m3 2)
-  constexpr int CL = MM::KSTEP / 32;    // 16-byte chunks per lane per k-step
+  constexpr int RB = B16 ? 16 : 32;     // rows of a matrix-instruction block
+  constexpr int KG = 64 / RB;           // K groups of lanes
+  constexpr int NACC = RB * RB / 64;    // accumulator registers per block
+  constexpr int TM = BM / 2, TN = BN / 2, FM = TM / RB, FN = TN / RB;
+  constexpr int NKS = BK / MM::KSTEP;   // MFMA k-steps per slab (32 x 32: int8 4, e4m3 2; 16 x 16: 2, 1)
+  constexpr int CL = MM::KSTEP / KG / 16;  // 16-byte chunks per lane per k-step
   constexpr int SLAB = (BM + BN) * BK;  // 64 KiB (56 KiB for the 192-column tile)
   constexpr int NJ = BM / 32, NJB = BN / 32;  // row groups of 32 per thread: A, B
-  static_assert(NKS % 2 == 0, "fragment buffers alternate per k-step");
+  static_assert(NKS == 1 || NKS % 2 == 0, "fragment buffers alternate per k-step");
   __shared__ __attribute__((aligned(16))) uint8_t lds[2 * SLAB];
 
   const int tid = threadIdx.x;
@@ -105,17 +128,22 @@ __global__ __launch_bounds__(256, 1) void gemm_rs_kernel(GemmArgs g, Epi epi) {
     if (t >= nslab) t -= nslab;
     return t * BK;
   };
-  v4i sta[NJ], stb[NJB];
+  // Staging sets.  Two of them where the registers allow it (int8 with 32 x 32 blocks: 16-byte
+  // fragments): set t % 2 carries slab t, so a slab's loads are in flight for two slab times before
+  // they are needed instead of one -- the loop otherwise waits on them (the operand lines that miss
+  // the L2 come from the memory side and take longer than a slab lasts when the fabric is busy).
+  constexpr int NSET = (OP == MMA_I8 && !B16) ? 2 : 1;
+  v4i sta[NSET][NJ], stb[NSET][NJB];
   // The loads keep their program order (a scheduling barrier that only memory instructions may
   // not cross follows each one): the compiler's vmcnt bookkeeping is exact only if the order in
   // the prologue and in the loop is the same.
   constexpr int NOT_VMEM = 0x7ff & ~(0x010 | 0x020 | 0x040);
   auto load_a = [&](int j, int k0) {
-    sta[j] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, va, j * sa32 + k0, 0));
+    sta[0][j] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, va, j * sa32 + k0, 0));
     __builtin_amdgcn_sched_barrier(NOT_VMEM);
   };
   auto load_b = [&](int j, int k0) {
-    stb[j] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, vb, j * sb32 + k0, 0));
+    stb[0][j] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, vb, j * sb32 + k0, 0));
     __builtin_amdgcn_sched_barrier(NOT_VMEM);
   };
   auto load_slab = [&](int s) {
@@ -132,34 +160,36 @@ __global__ __launch_bounds__(256, 1) void gemm_rs_kernel(GemmArgs g, Epi epi) {
   auto store_slab = [&](uint8_t* buf) {
 #pragma unroll
     for (int j = 0; j < (NJ > NJB ? NJ : NJB); ++j) {
-      if (j < NJ) *(v4i*)(buf + wr + j * 32 * BK) = sta[j];
-      if (j < NJB) *(v4i*)(buf + BM * BK + wr + j * 32 * BK) = stb[j];
+      if (j < NJ) *(v4i*)(buf + wr + j * 32 * BK) = sta[0][j];
+      if (j < NJB) *(v4i*)(buf + BM * BK + wr + j * 32 * BK) = stb[0][j];
     }
   };
 
   // ---- LDS -> MFMA operand addressing
-  const int fr = lane & 31, fg = lane >> 5;
+  const int fr = lane % RB, fg = lane / RB;
   const int fsw = swz<CPR, 1>(fr);
   int a_rd[NKS][CL], b_rd[NKS][CL];
 #pragma unroll
   for (int s = 0; s < NKS; ++s)
 #pragma unroll
     for (int e = 0; e < CL; ++e) {
-      const int c = s * 2 * CL + fg * CL + e;
+      const int c = (s * KG + fg) * CL + e;
       a_rd[s][e] = (wm * TM + fr) * BK + ((c ^ fsw) * 16);
       b_rd[s][e] = BM * BK + (wn * TN + fr) * BK + ((c ^ fsw) * 16);
     }
   // operand fragments are kept as their 16-byte halves so that single reads can be placed
   // between MFMAs; index r enumerates the reads of one k-step: A (i, e) first, then B (j, e)
-  v4i ha[2][FM][CL], hb[2][FN][CL];
+  // (a slab of one k-step keeps a single set: a fragment is re-read right after its last use)
+  constexpr int NFB = NKS == 1 ? 1 : 2;
+  v4i ha[NFB][FM][CL], hb[NFB][FN][CL];
   constexpr int NRD = (FM + FN) * CL, NMMA = FM * FN;
   auto read_one = [&](const uint8_t* ls, int s, int buf, auto r_c) {
     constexpr int R = decltype(r_c)::value;
     if constexpr (R < FM * CL) {
-      ha[buf][R / CL][R % CL] = *(const v4i*)(ls + a_rd[s][R % CL] + (R / CL) * 32 * BK);
+      ha[buf][R / CL][R % CL] = *(const v4i*)(ls + a_rd[s][R % CL] + (R / CL) * RB * BK);
     } else {
       constexpr int Q = R - FM * CL;
-      hb[buf][Q / CL][Q % CL] = *(const v4i*)(ls + b_rd[s][Q % CL] + (Q / CL) * 32 * BK);
+      hb[buf][Q / CL][Q % CL] = *(const v4i*)(ls + b_rd[s][Q % CL] + (Q / CL) * RB * BK);
     }
   };
   auto read_all = [&](const uint8_t* ls, int s, int buf) {
@@ -184,7 +214,7 @@ __global__ __launch_bounds__(256, 1) void gemm_rs_kernel(GemmArgs g, Epi epi) {
 #pragma unroll
     for (int j = 0; j < FN; ++j)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
+      for (int v = 0; v < NACC; ++v) acc[i][j][v] = 0;
   auto mma_step = [&](int buf) {
 #pragma unroll
     for (int i = 0; i < FM; ++i)
@@ -197,18 +227,18 @@ __global__ __launch_bounds__(256, 1) void gemm_rs_kernel(GemmArgs g, Epi epi) {
   // and the staging pairs [P0, P1) spread evenly over the FM x FN MFMAs.  A pair = write one staged
   // 16-byte chunk into `wr_buf`, then re-load its registers from slab `k0`.  Pair p < NJ is
   // operand A row group p, pair p >= NJ operand B row group p - NJ.
-  auto pair = [&](uint8_t* wr_buf, int k0, auto p_c) {
-    constexpr int P = decltype(p_c)::value;
+  auto pair = [&](uint8_t* wr_buf, int k0, auto p_c, auto set_c) {
+    constexpr int P = decltype(p_c)::value, ST = decltype(set_c)::value;
     if constexpr (P < NJ) {
-      *(v4i*)(wr_buf + wr + P * 32 * BK) = sta[P];
-      sta[P] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, va, P * sa32 + k0, 0));
+      *(v4i*)(wr_buf + wr + P * 32 * BK) = sta[ST][P];
+      sta[ST][P] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, va, P * sa32 + k0, 0));
     } else {
-      *(v4i*)(wr_buf + BM * BK + wr + (P - NJ) * 32 * BK) = stb[P - NJ];
-      stb[P - NJ] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, vb, (P - NJ) * sb32 + k0, 0));
+      *(v4i*)(wr_buf + BM * BK + wr + (P - NJ) * 32 * BK) = stb[ST][P - NJ];
+      stb[ST][P - NJ] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, vb, (P - NJ) * sb32 + k0, 0));
     }
   };
   auto kstep = [&](auto mb_c, const uint8_t* rd_ls, auto rs_c, auto rb_c, uint8_t* wr_buf, int k0,
-                   auto p0_c, auto p1_c) {
+                   auto p0_c, auto p1_c, auto set_c) {
     constexpr int MB = decltype(mb_c)::value, RS = decltype(rs_c)::value, RB = decltype(rb_c)::value;
     constexpr int P0 = decltype(p0_c)::value, P1 = decltype(p1_c)::value, NP = P1 - P0;
     [&]<int... R>(std::integer_sequence<int, R...>) {
@@ -222,8 +252,8 @@ __global__ __launch_bounds__(256, 1) void gemm_rs_kernel(GemmArgs g, Epi epi) {
             if constexpr (2 * R + 1 < NRD) read_one(rd_ls, RS, RB, std::integral_constant<int, 2 * R + 1>{});
             if constexpr (NP > 0) {
               constexpr int PA = P0 + R * NP / NMMA, PB = P0 + (R + 1) * NP / NMMA;
-              if constexpr (PB > PA) pair(wr_buf, k0, std::integral_constant<int, PA>{});
-              if constexpr (PB > PA + 1) pair(wr_buf, k0, std::integral_constant<int, PA + 1>{});
+              if constexpr (PB > PA) pair(wr_buf, k0, std::integral_constant<int, PA>{}, set_c);
+              if constexpr (PB > PA + 1) pair(wr_buf, k0, std::integral_constant<int, PA + 1>{}, set_c);
             }
             __builtin_amdgcn_sched_barrier(0);
           }(),
@@ -237,7 +267,7 @@ __global__ __launch_bounds__(256, 1) void gemm_rs_kernel(GemmArgs g, Epi epi) {
   constexpr int NP0 = OP == MMA_I8 ? NPAIR / 2 : NPAIR;
   auto pairs_now = [&](uint8_t* wr_buf, int k0, auto p0_c, auto p1_c) {  // no MFMAs to hide behind
     [&]<int... P>(std::integer_sequence<int, P...>) {
-      (pair(wr_buf, k0, std::integral_constant<int, decltype(p0_c)::value + P>{}), ...);
+      (pair(wr_buf, k0, std::integral_constant<int, decltype(p0_c)::value + P>{}, std::integral_constant<int, 0>{}), ...);
     }(std::make_integer_sequence<int, decltype(p1_c)::value - decltype(p0_c)::value>{});
   };
   typedef std::integral_constant<int, 0> C0;
@@ -268,55 +298,163 @@ __global__ __launch_bounds__(256, 1) void gemm_rs_kernel(GemmArgs g, Epi epi) {
               if constexpr (P < NJ) *(v4i*)(lds + SLAB + wr + P * 32 * BK) = ta[P];
               else *(v4i*)(lds + SLAB + BM * BK + wr + (P - NJ) * 32 * BK) = tb[P - NJ];
             } else {
-              if constexpr (P < NJ) sta[P] = ta[P];
-              else stb[P - NJ] = tb[P - NJ];
+              // (slab 1 belongs to set 1 where there are two)
+              if constexpr (P < NJ) sta[NSET - 1][P] = ta[P];
+              else stb[NSET - 1][P - NJ] = tb[P - NJ];
             }
           }(),
           ...);
     }(std::make_integer_sequence<int, NPAIR>{});
-    const int k2 = slab_k0(2);
+    const int k2 = slab_k0(2), k3p = slab_k0(3);
+    // one set: its pairs [0, NP0) take slab 2.  Two sets: set 0 takes all of slab 2, the pairs
+    // [0, NP0) of set 1 take slab 3
     [&]<int... P>(std::integer_sequence<int, P...>) {
       (
           [&] {
-            if constexpr (P < NJ) sta[P] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, va, P * sa32 + k2, 0));
-            else stb[P - NJ] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, vb, (P - NJ) * sb32 + k2, 0));
+            if constexpr (P < NJ) sta[0][P] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, va, P * sa32 + k2, 0));
+            else stb[0][P - NJ] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, vb, (P - NJ) * sb32 + k2, 0));
             __builtin_amdgcn_sched_barrier(NOT_VMEM);
           }(),
           ...);
-    }(std::make_integer_sequence<int, NP0>{});
+    }(std::make_integer_sequence<int, NSET == 2 ? NPAIR : NP0>{});
+    if constexpr (NSET == 2) {
+      [&]<int... P>(std::integer_sequence<int, P...>) {
+        (
+            [&] {
+              if constexpr (P < NJ) sta[1][P] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, va, P * sa32 + k3p, 0));
+              else stb[1][P - NJ] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, vb, (P - NJ) * sb32 + k3p, 0));
+              __builtin_amdgcn_sched_barrier(NOT_VMEM);
+            }(),
+            ...);
+      }(std::make_integer_sequence<int, NP0>{});
+    }
   }
   __syncthreads();
   read_all(lds, 0, 0);
 
-  for (int s = 0; s < nslab; ++s) {
-    uint8_t* cur = lds + (s & 1) * SLAB;
-    uint8_t* nxt = lds + ((s + 1) & 1) * SLAB;
-    // first k-step: the rest of the staged slab s + 1 goes into `nxt`, re-loaded with slab s + 2
-    kstep(C0{}, cur, C1{}, C1{}, nxt, slab_k0(s + 2), CNP0{}, CNP{});
-    // middle k-steps
-    [&]<int... KS>(std::integer_sequence<int, KS...>) {
-      (kstep(std::integral_constant<int, (KS + 1) & 1>{}, cur, std::integral_constant<int, KS + 2>{},
-             std::integral_constant<int, KS & 1>{}, nxt, 0, C0{}, C0{}),
-       ...);
-    }(std::make_integer_sequence<int, NKS - 2>{});
-    // Last k-step.  Its fragments are in registers once the LDS counter drains; after the
-    // barrier nobody reads `cur` any more: the staged slab s + 2 starts to go into it, and the
-    // first fragments of slab s + 1 are read from `nxt`.
-    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-    __builtin_amdgcn_sched_barrier(0);
-    kstep(std::integral_constant<int, (NKS - 1) & 1>{}, nxt, C0{}, C0{}, cur, slab_k0(s + 3), C0{}, CNP0{});
+  if constexpr (NKS == 1) {
+    // One k-step per slab (16 x 16 x 128): FM x FN matrix instructions on a single set of
+    // fragments.  Entering slab s the fragments of slab s are in registers, buffer s % 2 is no
+    // longer read by anyone, buffer (s + 1) % 2 holds slab s + 1 and the staging registers hold
+    // slab s + 2.  Row 0 of the blocks is issued first; the barrier behind it tells every wave that
+    // all waves are done with slab s - 1 (their reads of buffer s % 2 and their writes of slab s + 1).
+    // Behind it, spread over the remaining rows: the staged slab goes into buffer s % 2 and the
+    // staging registers are re-loaded with slab s + 3; fragment A[i] is re-read from the other
+    // buffer (slab s + 1) once row i is issued, B[j] once the last row has used it -- each at least
+    // FN - 1 instructions ahead of its next use.
+    static_assert(FM >= 2 && NPAIR <= (FM - 2) * FN, "rows 1 .. FM - 2 carry the staging pairs");
+    for (int s = 0; s < nslab; ++s) {
+      uint8_t* cur = lds + (s & 1) * SLAB;
+      const uint8_t* nxt = lds + ((s + 1) & 1) * SLAB;
+      const int k3 = slab_k0(s + 3);
+      [&]<int... J>(std::integer_sequence<int, J...>) {
+        ((acc[0][J] = MM::mma(frag_a(0, 0), frag_b(0, J), acc[0][J]), __builtin_amdgcn_sched_barrier(0)), ...);
+      }(std::make_integer_sequence<int, FN>{});
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      __builtin_amdgcn_sched_barrier(0);
+      [&]<int... R>(std::integer_sequence<int, R...>) {
+        (
+            [&] {
+              constexpr int I = 1 + R / FN, J = R % FN;
+              acc[I][J] = MM::mma(frag_a(0, I), frag_b(0, J), acc[I][J]);
+              // fragment A[I - 1]: its CL reads behind the first CL instructions of row I
+              if constexpr (J < CL) read_one(nxt, 0, 0, std::integral_constant<int, (I - 1) * CL + J>{});
+              if constexpr (I == FM - 1) {
+                // last row: B[J] is free once (FM - 1, J) is issued; A[FM - 1] after the last one
+                read_one(nxt, 0, 0, std::integral_constant<int, FM * CL + J * CL>{});
+                if constexpr (CL > 1) read_one(nxt, 0, 0, std::integral_constant<int, FM * CL + J * CL + 1>{});
+                if constexpr (J == FN - 1) {
+                  read_one(nxt, 0, 0, std::integral_constant<int, (FM - 1) * CL>{});
+                  if constexpr (CL > 1) read_one(nxt, 0, 0, std::integral_constant<int, (FM - 1) * CL + 1>{});
+                }
+              } else {
+                // rows 1 .. FM - 2: the staging pairs, evenly spread
+                constexpr int RR = (I - 1) * FN + J, NR = (FM - 2) * FN;
+                constexpr int PA = RR * NPAIR / NR, PB = (RR + 1) * NPAIR / NR;
+                if constexpr (PB > PA) pair(cur, k3, std::integral_constant<int, PA>{}, C0{});
+                if constexpr (PB > PA + 1) pair(cur, k3, std::integral_constant<int, PA + 1>{}, C0{});
+              }
+              __builtin_amdgcn_sched_barrier(0);
+            }(),
+            ...);
+      }(std::make_integer_sequence<int, (FM - 1) * FN>{});
+    }
+  } else {
+    // One slab.  PAR = s % 2 as a constant (it names staging sets, i.e. registers).
+    auto slab = [&](int s, auto par_c) {
+      constexpr int PAR = decltype(par_c)::value;
+      // staging set and reload distance: one set carries every slab (written one slab after its
+      // reload); with two, set t % 2 carries slab t (written two slabs after its reload)
+      typedef std::integral_constant<int, NSET == 2 ? (PAR ^ 1) : 0> SetFirst;
+      typedef std::integral_constant<int, NSET == 2 ? PAR : 0> SetLast;
+      uint8_t* cur = lds + (s & 1) * SLAB;
+      uint8_t* nxt = lds + ((s + 1) & 1) * SLAB;
+      // first k-step: the rest of the staged slab s + 1 goes into `nxt`, its registers re-loaded
+      kstep(C0{}, cur, C1{}, C1{}, nxt, slab_k0(s + 1 + NSET), CNP0{}, CNP{}, SetFirst{});
+      // middle k-steps
+      [&]<int... KS>(std::integer_sequence<int, KS...>) {
+        (kstep(std::integral_constant<int, (KS + 1) & 1>{}, cur, std::integral_constant<int, KS + 2>{},
+               std::integral_constant<int, KS & 1>{}, nxt, 0, C0{}, C0{}, C0{}),
+         ...);
+      }(std::make_integer_sequence<int, NKS - 2>{});
+      // Last k-step.  Its fragments are in registers once the LDS counter drains; after the
+      // barrier nobody reads `cur` any more: the staged slab s + 2 starts to go into it, and the
+      // first fragments of slab s + 1 are read from `nxt`.
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      __builtin_amdgcn_sched_barrier(0);
+      kstep(std::integral_constant<int, (NKS - 1) & 1>{}, nxt, C0{}, C0{}, cur, slab_k0(s + 2 + NSET), C0{}, CNP0{},
+            SetLast{});
+    };
+    if constexpr (NSET == 2) {
+      int s = 0;
+      for (; s + 1 < nslab; s += 2) {
+        slab(s, C0{});
+        slab(s + 1, C1{});
+      }
+      if (s < nslab) slab(s, C0{});
+    } else {
+      for (int s = 0; s < nslab; ++s) slab(s, C0{});
+    }
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   if (blockIdx.x == 0 && tid == 0 && g.clk) { g.clk[2] = clock64(); g.clk[3] = wall_clock64(); }
 
   // ---- epilogue: acc[i][j][v] is C(row, col) with
-  //      row = 32 i + 8 (v / 4) + 4 (lane / 32) + v % 4,   col = 32 j + lane % 32
+  //      row = 32 i + 8 (v / 4) + 4 (lane / 32) + v % 4,   col = 32 j + lane % 32   (32 x 32 blocks)
+  //      row = 16 i + 4 (lane / 16) + v,                   col = 16 j + lane % 16   (16 x 16 blocks)
   const int m_base = row_lo + wm * TM + fg * 4;
   const int n_base = col_lo + wn * TN + fr;
   typename Epi::Col colctx[FN];
 #pragma unroll
-  for (int j = 0; j < FN; ++j) colctx[j] = epi.col(min(n_base + j * 32, g.N - 1), expert, g.N);
+  for (int j = 0; j < FN; ++j) colctx[j] = epi.col(min(n_base + j * RB, g.N - 1), expert, g.N);
   const bool interior = (row_lo + BM <= row_hi) && (col_lo + BN <= g.N);
+  if constexpr (B16) {
+#pragma unroll
+    for (int i = 0; i < FM; ++i) {
+      typename Epi::Row rowctx[4];
+#pragma unroll
+      for (int v = 0; v < 4; ++v) rowctx[v] = epi.row(min(m_base + i * 16 + v, row_hi - 1));
+      if (interior) {
+#pragma unroll
+        for (int v = 0; v < 4; ++v)
+#pragma unroll
+          for (int j = 0; j < FN; ++j)
+            epi.store(m_base + i * 16 + v, n_base + j * 16, acc[i][j][v], rowctx[v], colctx[j]);
+      } else {
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          const int m = m_base + i * 16 + v;
+          if (m < row_hi) {
+#pragma unroll
+            for (int j = 0; j < FN; ++j) {
+              const int n = n_base + j * 16;
+              if (n < g.N) epi.store(m, n, acc[i][j][v], rowctx[v], colctx[j]);
+            }
+          }
+        }
+      }
+    }
+  } else
 #pragma unroll
   for (int i = 0; i < FM; ++i) {
     typename Epi::Row rowctx[16];
