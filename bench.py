@@ -148,7 +148,7 @@ def time_events(torch, fn, iters=30, warm=5, min_seconds=0.0):
     return e0.elapsed_time(e1) / iters
 
 
-def fp8_rooflines(torch, K, dev):
+def fp8_rooflines(torch, K, dev, min_seconds=0.15):
     """The FP8 half of the metric: e4m3 x e4m3 GEMMs with fp32 accumulation and the dequantizing
     epilogue (per-token activation scale, bf16 out) against the 5.0 PFLOP/s dense FP8 peak, on the
     Llama-3-8B shapes at M = 4096 (per-channel weight scales) and the Granite-3-8B-like shapes at
@@ -170,7 +170,7 @@ def fp8_rooflines(torch, K, dev):
             q, s = K.quant_act_fp8_pertoken(x, L.FP8_LINEAR)
             K.clock_probe(clk)
             ms = time_events(torch, lambda: K.gemm_fp8_dq(q, w8, s, ws, None, out_dtype=torch.bfloat16), iters=20, warm=4,
-                             min_seconds=0.15)
+                             min_seconds=min_seconds)
             K.clock_probe(None)
             ops = 2.0 * M * k * n
             tot_ms += ms
@@ -189,7 +189,7 @@ def fp8_rooflines(torch, K, dev):
                 try:
                     vms = time_events(torch, lambda: torch._scaled_mm(q, w8.t(), scale_a=sa, scale_b=sb,
                                                                        out_dtype=torch.bfloat16), iters=20, warm=4,
-                                      min_seconds=0.15)
+                                      min_seconds=min_seconds)
                     per[name][vlabel] = {"ms": round(vms, 4), "tflops": round(ops / (vms * 1e-3) / 1e12, 1)}
                     vend[vlabel] = vend.get(vlabel, 0.0) + vms
                 except Exception as e:  # the vendor path is evidence, not a dependency
@@ -411,6 +411,11 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-fp8-decode", action="store_true",
                     help="skip the FP8 GEMM and decode rooflines (profiling runs of the INT8 step)")
+    ap.add_argument("--no-decode", action="store_true", help="skip the decode rooflines only (counter runs of the FP8 GEMMs)")
+    ap.add_argument("--burst", action="store_true",
+                    help="time the FP8 GEMMs over twenty launches instead of 0.15 s (counter runs: every launch is slow there)")
+    ap.add_argument("--no-power-account", action="store_true",
+                    help="--extras without its power account (counter runs: its loops make tens of thousands of launches)")
     ap.add_argument("--extras", action="store_true",
                     help="also time the vendor GEMM, mid-size batches, MoE, chunk-truncate, side kernels")
     args = ap.parse_args()
@@ -513,16 +518,17 @@ def main():
                      "frac_at_measured_clock": round(achieved / peak_at_clock, 4)},
     }
     if not args.no_fp8_decode:
-        out["roofline_fp8"] = fp8_rooflines(torch, K, dev)
-        out["roofline_decode"] = decode_rooflines(torch, K, dev)
+        out["roofline_fp8"] = fp8_rooflines(torch, K, dev, 0.0 if args.burst else 0.15)
+        if not args.no_decode:
+            out["roofline_decode"] = decode_rooflines(torch, K, dev)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(torch, layers)
     if args.extras:
-        out["extras"] = extras(torch, K, dev, layers)
+        out["extras"] = extras(torch, K, dev, layers, power=not args.no_power_account)
     print(json.dumps(out))
 
 
-def extras(torch, K, dev, layers):
+def extras(torch, K, dev, layers, power=True):
     """The vendor GEMM on the same operands, mid-size batches (M in 32 .. 128), the Mixtral-style
     grouped expert GEMMs, the chunk-truncate emulation and the side kernels; reported in addition
     to the headline value and the FP8 / decode rooflines of the default run."""
@@ -576,7 +582,8 @@ def extras(torch, K, dev, layers):
     sample_ops = sum(2.0 * 2048 * k * n for _, k, n in LLAMA3_8B)
     res["cpu_baseline_sample_on_gpu_M2048"] = {"ms": round(ms, 4), "tops": round(sample_ops / ms / 1e9, 1)}
     res["vendor"] = vendor_int_mm(torch, K, layers)
-    res["power_account"] = power_account(torch, K, dev, layers)
+    if power:
+        res["power_account"] = power_account(torch, K, dev, layers)
     # batches of a few hundred rows (split-K territory) beside the vendor GEMM, launches replayed
     # from a HIP graph, weights rotated over > 300 MB: this library's fused-dequant GEMM, its raw
     # int32 GEMM and torch._int_mm (int32 out, no dequantization) on the same operands
