@@ -3,6 +3,7 @@
 #pragma once
 #include "gemm_rs.hpp"
 #include "gemm_k128.hpp"
+#include <algorithm>
 #include <cmath>
 #include <cstdlib>
 
@@ -124,6 +125,20 @@ static bool use_register_staged(int op) {
   (void)op;
   return true;
 }
+// Compute units of the current device (the grid of the persistent blocks).
+inline int compute_units() {
+  static thread_local int cached_dev = -1, cached = 0;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) dev = 0;
+  if (dev != cached_dev) {
+    int cus = 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1) cus = 256;
+    cached_dev = dev;
+    cached = cus;
+  }
+  return cached;
+}
+
 template <int OP, bool GROUPED = false, int BN = 256, class Epi>
 void launch_rs(const GemmArgs& g0, const Epi& epi, hipStream_t st) {
   GemmArgs g = g0;
@@ -132,6 +147,9 @@ void launch_rs(const GemmArgs& g0, const Epi& epi, hipStream_t st) {
   if (!GROUPED) g.grid_m = div_up(g.M, 256);
   g.group_m = 4;
   dim3 grid((unsigned)(g.grid_m * g.grid_n)), block(256);
+  // mixture-of-experts mode: grid_m is only an upper bound on the row tiles (the row counts live
+  // on the device); the blocks are persistent, one per compute unit, and count the tiles themselves
+  if (GROUPED && g.rows_per_group == 0) grid.x = (unsigned)std::min<long>((long)grid.x, compute_units());
   if constexpr (OP == MMA_FP8) {
     // e4m3: the 16 x 16 x 128 matrix instruction (more work per joule under the power limit: the
     // four Llama-3-8B shapes at 4096 rows +1 ... +4 %) unless FMSMO_MFMA16=0 asks for 32 x 32 x 64

@@ -54,10 +54,15 @@ __global__ __launch_bounds__(256, 1) void gemm_rs_kernel(GemmArgs g, Epi epi) {
   constexpr int TM = BM / 2, TN = BN / 2, FM = TM / RB, FN = TN / RB;
   constexpr int NKS = BK / MM::KSTEP;   // MFMA k-steps per slab (32 x 32: int8 4, e4m3 2; 16 x 16: 2, 1)
   constexpr int CL = MM::KSTEP / KG / 16;  // 16-byte chunks per lane per k-step
-  constexpr int SLAB = (BM + BN) * BK;  // 64 KiB (56 KiB for the 192-column tile)
+  // LDS: [A of buffer 0][A of buffer 1][B of buffer 0][B of buffer 1], 32 KiB apart.  Both buffers
+  // of an operand lie within the 64 KiB that the 16-bit offset field of an LDS instruction spans,
+  // so one address register per operand fragment serves both (buffers 64 KiB apart needed a second
+  // set of address registers, which the persistent blocks' tile loop had no room for).
+  constexpr int SLAB = BM * BK;      // buffer 1 of an operand follows buffer 0
+  constexpr int BOFF = 2 * BM * BK;  // operand B follows both buffers of A
   constexpr int NJ = BM / 32, NJB = BN / 32;  // row groups of 32 per thread: A, B
   static_assert(NKS == 1 || NKS % 2 == 0, "fragment buffers alternate per k-step");
-  __shared__ __attribute__((aligned(16))) uint8_t lds[2 * SLAB];
+  __shared__ __attribute__((aligned(16))) uint8_t lds[BOFF + BM * BK + BN * BK];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -67,6 +72,15 @@ __global__ __launch_bounds__(256, 1) void gemm_rs_kernel(GemmArgs g, Epi epi) {
   int row_lo, row_hi = g.M, expert = 0;
   int64_t a_adj = 0;
   int a_rows = g.M;  // rows addressable through the A descriptor (numbered like row_lo)
+  // Mixture-of-experts mode: the blocks are persistent.  The host launches one block per compute
+  // unit (it does not know the row counts); the real tiles -- counted here from `offsets` -- are
+  // dealt to the 8 XCDs in contiguous spans of the tile sequence, and the blocks of an XCD take
+  // their span's tiles in turn (block slot, slot + slots, ...), so that the tiles resident on an
+  // XCD at one time are neighbours in the sequence and share A and B panels in its L2.  One tile
+  // per block left the order of the tiles to the dispatcher, which hands out work-groups in
+  // order, round-robin over the XCDs: with tiles of uneven cost (row tiles cut by an expert's
+  // end store less) compute units waited 5 us per tile for their turn.
+  [[maybe_unused]] int real_m = 0, p_next = 0, p_end = 0, p_step = 1;  // this block's positions in the tile sequence
   if constexpr (GROUPED) {
     if (g.rows_per_group > 0) {
       // batched matmul: every group has the same number of rows, the grid is exact
@@ -80,43 +94,30 @@ __global__ __launch_bounds__(256, 1) void gemm_rs_kernel(GemmArgs g, Epi epi) {
       a_adj = (int64_t)expert * (g.lda_e - (int64_t)g.rows_per_group * g.lda);
       a_rows = row_hi;
     } else {
-      // grouped (mixture-of-experts) mode, as in gemm_tile.hpp: the grid is an upper bound, only
-      // the first real_tiles block ids are mapped; a tile covers rows of one expert
-      int real_m = 0;
       for (int e = 0; e < g.num_experts; ++e) real_m += (g.offsets[e + 1] - g.offsets[e] + BM - 1) / BM;
       const int real_tiles = real_m * g.grid_n;
-      if ((int)blockIdx.x >= real_tiles) return;  // uniform for the whole block
-      tile_of_block(blockIdx.x, real_tiles, real_m, g.grid_n, g.group_m, tile_m, tile_n);
-      int t = tile_m;
-      row_lo = 0;
-      for (int e = 0; e < g.num_experts; ++e) {
-        const int lo = g.offsets[e], hi = g.offsets[e + 1];
-        const int nt = (hi - lo + BM - 1) / BM;
-        if (t < nt) {
-          row_lo = lo + t * BM;
-          row_hi = hi;
-          expert = e;
-          break;
-        }
-        t -= nt;
-      }
+      const int nx = min(8, (int)gridDim.x);
+      const int xcd = blockIdx.x % nx;
+      p_step = ((int)gridDim.x - xcd + nx - 1) / nx;  // blocks on this XCD
+      const int per = real_tiles / nx, rem = real_tiles % nx;
+      const int lo = xcd < rem ? xcd * (per + 1) : rem * (per + 1) + (xcd - rem) * per;
+      p_end = lo + per + (xcd < rem ? 1 : 0);
+      p_next = lo + blockIdx.x / nx;
+      if (p_next >= p_end) return;  // uniform for the whole block
     }
   } else {
     tile_of_block(blockIdx.x, gridDim.x, g.grid_m, g.grid_n, g.group_m, tile_m, tile_n);
     row_lo = tile_m * BM;
   }
-  const int col_lo = tile_n * BN;
 
-  if (blockIdx.x == 0 && tid == 0 && g.clk) { g.clk[0] = clock64(); g.clk[1] = wall_clock64(); }
   // ---- global -> register staging: thread -> (row = tid / 8 + 32 j, 16-byte chunk = tid % 8)
   const int ld_row = tid >> 3, ld_chunk = tid & 7;
   const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
       (void*)(g.a + a_adj), 0, (int)((int64_t)(a_rows - 1) * g.lda + g.K), 0x00020000);
-  const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(
-      (void*)(g.b + (GROUPED ? (int64_t)expert * g.ldb_e : 0)), 0,
-      (int)((int64_t)(g.N - 1) * g.ldb + g.K), 0x00020000);
-  const int va = (row_lo + ld_row) * (int)g.lda + ld_chunk * 16;
-  const int vb = (col_lo + ld_row) * (int)g.ldb + ld_chunk * 16;
+  // per tile (a persistent block re-assigns them): B descriptor of the tile's expert, first
+  // column, byte offsets of the thread's first A and B rows
+  __amdgpu_buffer_rsrc_t rsrc_b;
+  int col_lo, va, vb;
   const int sa32 = 32 * (int)g.lda, sb32 = 32 * (int)g.ldb;
   const int nslab = g.K / BK;
   // slabs past the end: never used.  With k_rotate the block walks the slabs from its own
@@ -157,11 +158,11 @@ __global__ __launch_bounds__(256, 1) void gemm_rs_kernel(GemmArgs g, Epi epi) {
   // LDS position of the thread's chunk: row-major [row][128 B], chunk c of row r at c ^ swz(r);
   // swz depends on r % 16 only, so it is the same for all 8 row groups
   const int wr = ld_row * BK + ((ld_chunk ^ swz<CPR, 1>(ld_row)) * 16);
-  auto store_slab = [&](uint8_t* buf) {
+  auto store_slab = [&](uint8_t* buf, int wr_t) {
 #pragma unroll
     for (int j = 0; j < (NJ > NJB ? NJ : NJB); ++j) {
-      if (j < NJ) *(v4i*)(buf + wr + j * 32 * BK) = sta[0][j];
-      if (j < NJB) *(v4i*)(buf + BM * BK + wr + j * 32 * BK) = stb[0][j];
+      if (j < NJ) *(v4i*)(buf + wr_t + j * 32 * BK) = sta[0][j];
+      if (j < NJB) *(v4i*)(buf + BOFF + wr_t + j * 32 * BK) = stb[0][j];
     }
   };
 
@@ -175,7 +176,7 @@ __global__ __launch_bounds__(256, 1) void gemm_rs_kernel(GemmArgs g, Epi epi) {
     for (int e = 0; e < CL; ++e) {
       const int c = (s * KG + fg) * CL + e;
       a_rd[s][e] = (wm * TM + fr) * BK + ((c ^ fsw) * 16);
-      b_rd[s][e] = BM * BK + (wn * TN + fr) * BK + ((c ^ fsw) * 16);
+      b_rd[s][e] = BOFF + (wn * TN + fr) * BK + ((c ^ fsw) * 16);
     }
   // operand fragments are kept as their 16-byte halves so that single reads can be placed
   // between MFMAs; index r enumerates the reads of one k-step: A (i, e) first, then B (j, e)
@@ -209,12 +210,6 @@ __global__ __launch_bounds__(256, 1) void gemm_rs_kernel(GemmArgs g, Epi epi) {
   };
 
   Acc acc[FM][FN];
-#pragma unroll
-  for (int i = 0; i < FM; ++i)
-#pragma unroll
-    for (int j = 0; j < FN; ++j)
-#pragma unroll
-      for (int v = 0; v < NACC; ++v) acc[i][j][v] = 0;
   auto mma_step = [&](int buf) {
 #pragma unroll
     for (int i = 0; i < FM; ++i)
@@ -233,7 +228,7 @@ __global__ __launch_bounds__(256, 1) void gemm_rs_kernel(GemmArgs g, Epi epi) {
       *(v4i*)(wr_buf + wr + P * 32 * BK) = sta[ST][P];
       sta[ST][P] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, va, P * sa32 + k0, 0));
     } else {
-      *(v4i*)(wr_buf + BM * BK + wr + (P - NJ) * 32 * BK) = stb[ST][P - NJ];
+      *(v4i*)(wr_buf + BOFF + wr + (P - NJ) * 32 * BK) = stb[ST][P - NJ];
       stb[ST][P - NJ] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, vb, (P - NJ) * sb32 + k0, 0));
     }
   };
@@ -275,6 +270,44 @@ __global__ __launch_bounds__(256, 1) void gemm_rs_kernel(GemmArgs g, Epi epi) {
   typedef std::integral_constant<int, NP0> CNP0;
   typedef std::integral_constant<int, NPAIR> CNP;
 
+  for (;;) {  // one pass per tile: a single one except for the persistent blocks
+  if constexpr (GROUPED) {
+    if (g.rows_per_group == 0) {
+      tile_of_pid(p_next, real_m, g.grid_n, g.group_m, tile_m, tile_n);
+      int t = tile_m;
+      row_lo = 0;
+      for (int e = 0; e < g.num_experts; ++e) {
+        const int lo = g.offsets[e], hi = g.offsets[e + 1];
+        const int nt = (hi - lo + BM - 1) / BM;
+        if (t < nt) {
+          row_lo = lo + t * BM;
+          row_hi = hi;
+          expert = e;
+          break;
+        }
+        t -= nt;
+      }
+    }
+  }
+  col_lo = tile_n * BN;
+  rsrc_b = __builtin_amdgcn_make_buffer_rsrc((void*)(g.b + (GROUPED ? (int64_t)expert * g.ldb_e : 0)), 0,
+                                             (int)((int64_t)(g.N - 1) * g.ldb + g.K), 0x00020000);
+  {
+    // (persistent blocks: derived from an opaque copy of the thread id, or the compiler hoists
+    // these products out of the tile loop and holds them in registers the K loop has no room for)
+    int t_id = tid;
+    if constexpr (GROUPED) asm volatile("" : "+v"(t_id));
+    va = (row_lo + (t_id >> 3)) * (int)g.lda + (t_id & 7) * 16;
+    vb = (col_lo + (t_id >> 3)) * (int)g.ldb + (t_id & 7) * 16;
+  }
+  if (blockIdx.x == 0 && tid == 0 && g.clk) { g.clk[0] = clock64(); g.clk[1] = wall_clock64(); }
+#pragma unroll
+  for (int i = 0; i < FM; ++i)
+#pragma unroll
+    for (int j = 0; j < FN; ++j)
+#pragma unroll
+      for (int v = 0; v < NACC; ++v) acc[i][j][v] = 0;
+
   // ---- prologue: slab 0 into LDS; slab 1: pairs [0, NP0) into LDS and their registers re-loaded
   // with slab 2, pairs [NP0, NPAIR) still staged (the first k-step of the loop writes them)
   // (slabs 0 and 1 are fetched together: the accumulators and fragments are not live yet, so
@@ -289,14 +322,16 @@ __global__ __launch_bounds__(256, 1) void gemm_rs_kernel(GemmArgs g, Epi epi) {
       if (j < NJB)
         tb[j] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, vb, j * sb32 + k1, 0));
     }
-    store_slab(lds);
+    int wr_t = wr;  // (persistent blocks: opaque, so that the addresses below are formed here)
+    if constexpr (GROUPED) asm volatile("" : "+v"(wr_t));
+    store_slab(lds, wr_t);
     // slab 1: pairs [0, NP0) go to LDS, the rest stay staged
     [&]<int... P>(std::integer_sequence<int, P...>) {
       (
           [&] {
             if constexpr (P < NP0) {
-              if constexpr (P < NJ) *(v4i*)(lds + SLAB + wr + P * 32 * BK) = ta[P];
-              else *(v4i*)(lds + SLAB + BM * BK + wr + (P - NJ) * 32 * BK) = tb[P - NJ];
+              if constexpr (P < NJ) *(v4i*)(lds + SLAB + wr_t + P * 32 * BK) = ta[P];
+              else *(v4i*)(lds + SLAB + BOFF + wr_t + (P - NJ) * 32 * BK) = tb[P - NJ];
             } else {
               // (slab 1 belongs to set 1 where there are two)
               if constexpr (P < NJ) sta[NSET - 1][P] = ta[P];
@@ -387,8 +422,9 @@ __global__ __launch_bounds__(256, 1) void gemm_rs_kernel(GemmArgs g, Epi epi) {
       // reload); with two, set t % 2 carries slab t (written two slabs after its reload)
       typedef std::integral_constant<int, NSET == 2 ? (PAR ^ 1) : 0> SetFirst;
       typedef std::integral_constant<int, NSET == 2 ? PAR : 0> SetLast;
-      uint8_t* cur = lds + (s & 1) * SLAB;
-      uint8_t* nxt = lds + ((s + 1) & 1) * SLAB;
+      // (two staging sets: the loop is unrolled by two and PAR == s % 2, a constant)
+      uint8_t* cur = lds + (NSET == 2 ? PAR : (s & 1)) * SLAB;
+      uint8_t* nxt = lds + (NSET == 2 ? PAR ^ 1 : ((s + 1) & 1)) * SLAB;
       // first k-step: the rest of the staged slab s + 1 goes into `nxt`, its registers re-loaded
       kstep(C0{}, cur, C1{}, C1{}, nxt, slab_k0(s + 1 + NSET), CNP0{}, CNP{}, SetFirst{});
       // middle k-steps
@@ -422,19 +458,59 @@ __global__ __launch_bounds__(256, 1) void gemm_rs_kernel(GemmArgs g, Epi epi) {
   // ---- epilogue: acc[i][j][v] is C(row, col) with
   //      row = 32 i + 8 (v / 4) + 4 (lane / 32) + v % 4,   col = 32 j + lane % 32   (32 x 32 blocks)
   //      row = 16 i + 4 (lane / 16) + v,                   col = 16 j + lane % 16   (16 x 16 blocks)
-  const int m_base = row_lo + wm * TM + fg * 4;
-  const int n_base = col_lo + wn * TN + fr;
+  int e_lane = lane;
+  if constexpr (GROUPED) asm volatile("" : "+v"(e_lane));  // as above
+  const int m_base = row_lo + wm * TM + (e_lane / RB) * 4;
+  const int n_base = col_lo + wn * TN + e_lane % RB;
   typename Epi::Col colctx[FN];
 #pragma unroll
   for (int j = 0; j < FN; ++j) colctx[j] = epi.col(min(n_base + j * RB, g.N - 1), expert, g.N);
-  const bool interior = (row_lo + BM <= row_hi) && (col_lo + BN <= g.N);
-  if constexpr (B16) {
+  // Rows are tested in groups that a wave's accumulator layout makes uniform (8 rows of a 32 x 32
+  // block, 16 of a 16 x 16 one): a group wholly below row_hi stores without any per-lane test, a
+  // group wholly past it is skipped by a scalar branch, and only the one group that row_hi cuts
+  // tests every lane.  (Per-lane tests around every store put each store into a basic block of its
+  // own: a row tile with 200 of its 256 rows valid then took twice as long to store as a full one.)
+  const bool cols_full = col_lo + BN <= g.N;
+  const int rows_left = row_hi - row_lo - wm * TM;  // valid rows from this wave's first row on; uniform
+  // whole tile: one straight run of stores (the row groups' branches cost the dense shapes 1 %; the
+  // persistent blocks have no registers for a third copy of the stores)
+  const bool interior = !GROUPED && cols_full && row_lo + BM <= row_hi;
+  if (interior) {
+    if constexpr (B16) {
+#pragma unroll
+      for (int i = 0; i < FM; ++i) {
+        typename Epi::Row rowctx[4];
+#pragma unroll
+        for (int v = 0; v < 4; ++v) rowctx[v] = epi.row(m_base + i * 16 + v);
+#pragma unroll
+        for (int v = 0; v < 4; ++v)
+#pragma unroll
+          for (int j = 0; j < FN; ++j)
+            epi.store(m_base + i * 16 + v, n_base + j * 16, acc[i][j][v], rowctx[v], colctx[j]);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < FM; ++i) {
+        typename Epi::Row rowctx[16];
+#pragma unroll
+        for (int v = 0; v < 16; ++v) rowctx[v] = epi.row(m_base + i * 32 + (v >> 2) * 8 + (v & 3));
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int m = m_base + i * 32 + (v >> 2) * 8 + (v & 3);
+#pragma unroll
+          for (int j = 0; j < FN; ++j) epi.store(m, n_base + j * 32, acc[i][j][v], rowctx[v], colctx[j]);
+        }
+      }
+    }
+  } else if constexpr (B16) {
 #pragma unroll
     for (int i = 0; i < FM; ++i) {
+      const int left = rows_left - i * 16;
+      if (left <= 0) break;
       typename Epi::Row rowctx[4];
 #pragma unroll
       for (int v = 0; v < 4; ++v) rowctx[v] = epi.row(min(m_base + i * 16 + v, row_hi - 1));
-      if (interior) {
+      if (left >= 16 && cols_full) {
 #pragma unroll
         for (int v = 0; v < 4; ++v)
 #pragma unroll
@@ -457,32 +533,46 @@ __global__ __launch_bounds__(256, 1) void gemm_rs_kernel(GemmArgs g, Epi epi) {
   } else
 #pragma unroll
   for (int i = 0; i < FM; ++i) {
+    if (rows_left - i * 32 <= 0) break;
     typename Epi::Row rowctx[16];
 #pragma unroll
     for (int v = 0; v < 16; ++v)
       rowctx[v] = epi.row(min(m_base + i * 32 + (v >> 2) * 8 + (v & 3), row_hi - 1));
-    if (interior) {
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int m = m_base + i * 32 + (v >> 2) * 8 + (v & 3);
+    for (int q = 0; q < 4; ++q) {
+      const int left = rows_left - i * 32 - q * 8;
+      if (left >= 8 && cols_full) {
 #pragma unroll
-        for (int j = 0; j < FN; ++j) epi.store(m, n_base + j * 32, acc[i][j][v], rowctx[v], colctx[j]);
-      }
-    } else {
+        for (int vv = 0; vv < 4; ++vv) {
+          const int v = q * 4 + vv, m = m_base + i * 32 + q * 8 + vv;
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int m = m_base + i * 32 + (v >> 2) * 8 + (v & 3);
-        if (m < row_hi) {
+          for (int j = 0; j < FN; ++j) epi.store(m, n_base + j * 32, acc[i][j][v], rowctx[v], colctx[j]);
+        }
+      } else if (left > 0) {
 #pragma unroll
-          for (int j = 0; j < FN; ++j) {
-            const int n = n_base + j * 32;
-            if (n < g.N) epi.store(m, n, acc[i][j][v], rowctx[v], colctx[j]);
+        for (int vv = 0; vv < 4; ++vv) {
+          const int v = q * 4 + vv, m = m_base + i * 32 + q * 8 + vv;
+          if (m < row_hi) {
+#pragma unroll
+            for (int j = 0; j < FN; ++j) {
+              const int n = n_base + j * 32;
+              if (n < g.N) epi.store(m, n, acc[i][j][v], rowctx[v], colctx[j]);
+            }
           }
         }
       }
     }
   }
   if (blockIdx.x == 0 && tid == 0 && g.clk) { g.clk[4] = clock64(); g.clk[5] = wall_clock64(); }
+  if constexpr (!GROUPED) {
+    break;
+  } else {
+    if (g.rows_per_group > 0) break;
+    p_next += p_step;
+    if (p_next >= p_end) break;
+    __syncthreads();  // every wave has read its last fragments: the slabs may be overwritten
+  }
+  }  // tiles
 #endif  // __HIP_DEVICE_COMPILE__
 }
 

@@ -186,6 +186,18 @@ __device__ __forceinline__ float trunc_f32(float p, unsigned round_bit, unsigned
   return x;
 }
 
+// Position `pid` of the tile sequence: column-major inside groups of `group_m` tile rows (the
+// second half of tile_of_block below, for blocks that walk the sequence themselves).
+__device__ __forceinline__ void tile_of_pid(int pid, int grid_m, int grid_n, int group_m, int& tm, int& tn) {
+  const int in_group = group_m * grid_n;
+  const int gid = pid / in_group;
+  const int first_m = gid * group_m;
+  const int gsz = min(grid_m - first_m, group_m);
+  const int r = pid - gid * in_group;
+  tm = first_m + r % gsz;
+  tn = r / gsz;
+}
+
 // Map the hardware block id to a tile.  Work-groups are dealt round-robin to the 8 XCDs (each
 // with a private L2), so block b runs on XCD b % 8; give every XCD one contiguous span of the
 // tile sequence, and order that sequence in column-major groups of `group_m` tile rows so the
@@ -206,7 +218,9 @@ __device__ __forceinline__ void tile_of_block(int bid, int nblk, int grid_m, int
 
 template <int BM, int BN, int BK, int NSTAGE, int WGM, int WGN, int OP, int SWZ, bool GROUPED,
           class Epi, class Chk = NoChunk>
-__global__ __launch_bounds__(WGM* WGN * 64, (Chk::enabled && (OP == MMA_I8 || Chk::fast)) ? 2 : 1) void gemm_tile_kernel(GemmArgs g, Epi epi, Chk chk) {
+// (two blocks per compute unit for the scheduled chunk hooks; the generic hook keeps a second
+// accumulator set and would spill at 256 registers)
+__global__ __launch_bounds__(WGM* WGN * 64, (Chk::enabled && Chk::fast) ? 2 : 1) void gemm_tile_kernel(GemmArgs g, Epi epi, Chk chk) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stub
   typedef Mma<OP> MM;
   typedef typename MM::Frag Frag;
