@@ -369,50 +369,69 @@ __global__ __launch_bounds__(256, 1) void gemm_rs_kernel(GemmArgs g, Epi epi) {
 
   if constexpr (NKS == 1) {
     // One k-step per slab (16 x 16 x 128): FM x FN matrix instructions on a single set of
-    // fragments.  Entering slab s the fragments of slab s are in registers, buffer s % 2 is no
-    // longer read by anyone, buffer (s + 1) % 2 holds slab s + 1 and the staging registers hold
-    // slab s + 2.  Row 0 of the blocks is issued first; the barrier behind it tells every wave that
-    // all waves are done with slab s - 1 (their reads of buffer s % 2 and their writes of slab s + 1).
-    // Behind it, spread over the remaining rows: the staged slab goes into buffer s % 2 and the
-    // staging registers are re-loaded with slab s + 3; fragment A[i] is re-read from the other
-    // buffer (slab s + 1) once row i is issued, B[j] once the last row has used it -- each at least
-    // FN - 1 instructions ahead of its next use.
-    static_assert(FM >= 2 && NPAIR <= (FM - 2) * FN, "rows 1 .. FM - 2 carry the staging pairs");
+    // fragments, re-read one by one as the instructions release them.  Entering slab s the
+    // fragments of slab s are in registers except A[HM ..] (below), buffer (s + 1) % 2 holds slab
+    // s + 1 and the staging registers hold slab s + 2.
+    //   row 0 of the blocks, and behind its instructions the reads of A[HM ..] of slab s;
+    //   barrier: every wave has all of slab s in registers and has written its part of slab s + 1;
+    //   rows 1 .. HM - 1 row by row, A[i - 1] re-read (slab s + 1) once row i is under way;
+    //   rows HM .. FM - 1 column by column, B[j] re-read once column j is done;
+    //   spread over everything behind the barrier: the staged slab goes into buffer s % 2 and the
+    //   staging registers are re-loaded with slab s + 3.
+    // Every re-read is at least FN - 1 instructions ahead of its use.  (All rows in row order left
+    // all FN fragments of B, and the last one of A, to be re-read behind the last row: 18 KiB per
+    // wave in the time of 8 instructions, more than twice what the LDS delivers.)
+    constexpr int HM = FM / 2, NCOL = FM - HM;
+    constexpr int NQ = (FM - 1) * FN;     // instructions behind the barrier
+    constexpr int NQP = NQ - NCOL;        // ... that carry staging pairs (not the last column)
+    constexpr int NDR = NCOL * CL;        // reads of A[HM ..] behind row 0
+    static_assert(FM >= 4 && FM % 2 == 0 && NPAIR <= NQP && CL <= NCOL, "schedule of a one-k-step slab");
     for (int s = 0; s < nslab; ++s) {
       uint8_t* cur = lds + (s & 1) * SLAB;
       const uint8_t* nxt = lds + ((s + 1) & 1) * SLAB;
       const int k3 = slab_k0(s + 3);
       [&]<int... J>(std::integer_sequence<int, J...>) {
-        ((acc[0][J] = MM::mma(frag_a(0, 0), frag_b(0, J), acc[0][J]), __builtin_amdgcn_sched_barrier(0)), ...);
+        (
+            [&] {
+              acc[0][J] = MM::mma(frag_a(0, 0), frag_b(0, J), acc[0][J]);
+              constexpr int R0 = J * NDR / FN, R1 = (J + 1) * NDR / FN;
+              if constexpr (R1 > R0) read_one(cur, 0, 0, std::integral_constant<int, HM * CL + R0>{});
+              if constexpr (R1 > R0 + 1) read_one(cur, 0, 0, std::integral_constant<int, HM * CL + R0 + 1>{});
+              static_assert(R1 <= R0 + 2, "at most two reads behind an instruction of row 0");
+              __builtin_amdgcn_sched_barrier(0);
+            }(),
+            ...);
       }(std::make_integer_sequence<int, FN>{});
       asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
       __builtin_amdgcn_sched_barrier(0);
-      [&]<int... R>(std::integer_sequence<int, R...>) {
+      [&]<int... Q>(std::integer_sequence<int, Q...>) {
         (
             [&] {
-              constexpr int I = 1 + R / FN, J = R % FN;
+              constexpr bool BYROW = Q < (HM - 1) * FN;
+              constexpr int Q2 = Q - (HM - 1) * FN;
+              constexpr int I = BYROW ? 1 + Q / FN : HM + Q2 % NCOL;
+              constexpr int J = BYROW ? Q % FN : Q2 / NCOL;
               acc[I][J] = MM::mma(frag_a(0, I), frag_b(0, J), acc[I][J]);
-              // fragment A[I - 1]: its CL reads behind the first CL instructions of row I
-              if constexpr (J < CL) read_one(nxt, 0, 0, std::integral_constant<int, (I - 1) * CL + J>{});
-              if constexpr (I == FM - 1) {
-                // last row: B[J] is free once (FM - 1, J) is issued; A[FM - 1] after the last one
-                read_one(nxt, 0, 0, std::integral_constant<int, FM * CL + J * CL>{});
-                if constexpr (CL > 1) read_one(nxt, 0, 0, std::integral_constant<int, FM * CL + J * CL + 1>{});
-                if constexpr (J == FN - 1) {
-                  read_one(nxt, 0, 0, std::integral_constant<int, (FM - 1) * CL>{});
-                  if constexpr (CL > 1) read_one(nxt, 0, 0, std::integral_constant<int, (FM - 1) * CL + 1>{});
-                }
+              if constexpr (BYROW) {
+                // fragment A[I - 1]: its CL reads behind the first CL instructions of row I
+                if constexpr (J < CL) read_one(nxt, 0, 0, std::integral_constant<int, (I - 1) * CL + J>{});
               } else {
-                // rows 1 .. FM - 2: the staging pairs, evenly spread
-                constexpr int RR = (I - 1) * FN + J, NR = (FM - 2) * FN;
-                constexpr int PA = RR * NPAIR / NR, PB = (RR + 1) * NPAIR / NR;
+                // A[HM - 1] behind the first instructions of the columns, B[J] behind column J
+                if constexpr (Q2 < CL) read_one(nxt, 0, 0, std::integral_constant<int, (HM - 1) * CL + Q2>{});
+                if constexpr (I == FM - 1) {
+                  read_one(nxt, 0, 0, std::integral_constant<int, FM * CL + J * CL>{});
+                  if constexpr (CL > 1) read_one(nxt, 0, 0, std::integral_constant<int, FM * CL + J * CL + 1>{});
+                }
+              }
+              if constexpr (Q < NQP) {
+                constexpr int PA = Q * NPAIR / NQP, PB = (Q + 1) * NPAIR / NQP;
                 if constexpr (PB > PA) pair(cur, k3, std::integral_constant<int, PA>{}, C0{});
                 if constexpr (PB > PA + 1) pair(cur, k3, std::integral_constant<int, PA + 1>{}, C0{});
               }
               __builtin_amdgcn_sched_barrier(0);
             }(),
             ...);
-      }(std::make_integer_sequence<int, (FM - 1) * FN>{});
+      }(std::make_integer_sequence<int, NQ>{});
     }
   } else {
     // One slab.  PAR = s % 2 as a constant (it names staging sets, i.e. registers).
