@@ -48,6 +48,7 @@ __global__ __launch_bounds__(256, 1) void gemm_rs_kernel(GemmArgs g, Epi epi) {
   typedef typename MM::Acc Acc;
   static_assert(BN_ == 256 || BN_ == 192 || BN_ == 128, "tile width");
   constexpr int BM = 256, BN = BN_, BK = 128, CPR = 8;
+  constexpr bool LOOPS = GROUPED;  // the block may walk several tiles
   constexpr int RB = B16 ? 16 : 32;     // rows of a matrix-instruction block
   constexpr int KG = 64 / RB;           // K groups of lanes
   constexpr int NACC = RB * RB / 64;    // accumulator registers per block
@@ -296,7 +297,7 @@ __global__ __launch_bounds__(256, 1) void gemm_rs_kernel(GemmArgs g, Epi epi) {
     // (persistent blocks: derived from an opaque copy of the thread id, or the compiler hoists
     // these products out of the tile loop and holds them in registers the K loop has no room for)
     int t_id = tid;
-    if constexpr (GROUPED) asm volatile("" : "+v"(t_id));
+    if constexpr (LOOPS) asm volatile("" : "+v"(t_id));
     va = (row_lo + (t_id >> 3)) * (int)g.lda + (t_id & 7) * 16;
     vb = (col_lo + (t_id >> 3)) * (int)g.ldb + (t_id & 7) * 16;
   }
@@ -323,7 +324,7 @@ __global__ __launch_bounds__(256, 1) void gemm_rs_kernel(GemmArgs g, Epi epi) {
         tb[j] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, vb, j * sb32 + k1, 0));
     }
     int wr_t = wr;  // (persistent blocks: opaque, so that the addresses below are formed here)
-    if constexpr (GROUPED) asm volatile("" : "+v"(wr_t));
+    if constexpr (LOOPS) asm volatile("" : "+v"(wr_t));
     store_slab(lds, wr_t);
     // slab 1: pairs [0, NP0) go to LDS, the rest stay staged
     [&]<int... P>(std::integer_sequence<int, P...>) {
@@ -478,7 +479,7 @@ __global__ __launch_bounds__(256, 1) void gemm_rs_kernel(GemmArgs g, Epi epi) {
   //      row = 32 i + 8 (v / 4) + 4 (lane / 32) + v % 4,   col = 32 j + lane % 32   (32 x 32 blocks)
   //      row = 16 i + 4 (lane / 16) + v,                   col = 16 j + lane % 16   (16 x 16 blocks)
   int e_lane = lane;
-  if constexpr (GROUPED) asm volatile("" : "+v"(e_lane));  // as above
+  if constexpr (LOOPS) asm volatile("" : "+v"(e_lane));  // as above
   const int m_base = row_lo + wm * TM + (e_lane / RB) * 4;
   const int n_base = col_lo + wn * TN + e_lane % RB;
   typename Epi::Col colctx[FN];

@@ -990,6 +990,43 @@ def test_grouped_gemm_row_remainders(dev, counts, NK, exact_ref, out_dtype):
             assert torch.equal(y[lo:hi][same].view(bits), want[same].view(bits))
 
 
+@pytest.mark.parametrize("counts", [
+    [700, 0, 13, 1300, 256, 511],        # 13 row tiles x 24 column tiles = 312 tiles
+    [300, 300, 300, 300, 300, 300, 300, 300, 300, 300, 300, 300]])   # 24 x 24 = 576: every block walks tiles of several experts
+def test_grouped_gemm_more_tiles_than_compute_units(dev, counts):
+    """The blocks of the grouped kernel are persistent (one per compute unit) and walk the tile
+    sequence themselves: with more tiles than compute units a block computes tiles of different
+    experts one after the other (accumulators, weight descriptor, scales re-made per tile).  Every
+    row must equal the per-expert product, bit for bit."""
+    N, Kd = 6144, 256
+    E = len(counts)
+    offsets = torch.zeros(E + 1, dtype=torch.int32)
+    offsets[1:] = torch.tensor(counts).cumsum(0)
+    T = int(offsets[-1])
+    a = _rand_i8((T, Kd), 176).to(dev)
+    w = _rand_i8((E, N, Kd), 177).to(dev)
+    s_a = (torch.rand(T, generator=gen(178)) * 0.05 + 1e-3).float().to(dev)
+    s_w = (torch.rand(E, N, generator=gen(179)) * 1e-3 + 1e-5).float().to(dev)
+    bias = (torch.randn(E, N, generator=gen(180)) * 0.01).half().to(dev)
+    y = K().grouped_gemm_i8_dq(a, w, offsets.to(dev), s_a, s_w, bias, out_dtype=torch.float16, exact_ref=True)
+    y2 = K().grouped_gemm_i8_dq(a, w, offsets.to(dev), s_a, s_w, bias, out_dtype=torch.float16, exact_ref=True)
+    assert torch.equal(y.view(torch.int16), y2.view(torch.int16))
+    for e in range(E):
+        lo, hi = int(offsets[e]), int(offsets[e + 1])
+        if hi == lo:
+            continue
+        ref = K().gemm_i8_dq(a[lo:hi], w[e], s_a[lo:hi], s_w[e], bias[e], out_dtype=torch.float16, exact_ref=True)
+        assert torch.equal(y[lo:hi].view(torch.int16), ref.view(torch.int16)), e
+    # one expert against the oracle's integers
+    e = 2
+    lo, hi = int(offsets[e]), int(offsets[e + 1])
+    acc = O.int_gemm(a[lo:hi].cpu(), w[e].cpu())
+    sa16 = s_a[lo:hi].cpu()
+    same = sa16.half().float() == sa16
+    want = O.epilogue_ref(acc, sa16[:, None].half(), s_w[e].cpu(), bias[e].cpu(), torch.float16)
+    assert torch.equal(y[lo:hi].cpu()[same].view(torch.int16), want[same].view(torch.int16))
+
+
 def test_grouped_gemm_random_expert_splits(dev):
     """Twelve seeded cases: 1 to 12 experts, a random split of the rows (empty experts included),
     any N, K in whole 128-byte slabs and not, per-expert bias or none: every expert's rows equal
