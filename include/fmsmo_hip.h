@@ -549,8 +549,10 @@ int fmsmo_matmul_chunk_fp_dq(const void* a, int64_t lda, const void* b, int64_t 
  * 5. Grouped int8 GEMM for mixture-of-experts FFNs (uneven rows per expert, one launch).
  *    Rows of A are sorted by expert; expert e owns rows [offsets[e], offsets[e+1]).
  *    B is [E][N][K] (expert stride ldb_e elements), w_scale [E][N], bias [E][N] or NULL.
- *    offsets is a DEVICE array of E+1 int32.  total_rows = offsets[E] must be given on the
- *    host (it sizes the grid).  Arithmetic per expert == fmsmo_gemm_i8_dq.
+ *    offsets is a DEVICE array of E+1 int32; the row counts are never read back.  total_rows =
+ *    offsets[E] must be given on the host (it sizes the output and bounds the grid; with whole
+ *    128-byte reductions the launch is one persistent block per compute unit and the blocks
+ *    count the tiles themselves).  Arithmetic per expert == fmsmo_gemm_i8_dq.
  *    The reference has no grouped type: every expert w1/w2/w3 is its own QLinearINT8Deploy
  *    (fms_mo/utils/dq_utils.py:86-106), so each expert's rows must equal that module's output.
  * ------------------------------------------------------------------------------------------ */
