@@ -290,19 +290,21 @@ def decode_rooflines(torch, K, dev, m_list=(1, 4, 16), ops=("i8", "fp8"), copies
 
 def vendor_int_mm(torch, K, layers):
     """The vendor library's int8 GEMM (torch._int_mm -> hipBLASLt, int32 out, no epilogue) on the
-    SAME quantized operands as the headline step, same event timing, beside this library's raw
-    int32 GEMM: how much of the distance to the published peak is the part's, not the kernel's."""
+    SAME quantized operands as the headline step, same event timing (each loop at least 0.15 s: a
+    burst of twenty launches runs on whatever clock the work before it left behind), beside this
+    library's raw int32 GEMM: how much of the distance to the published peak is the part's, not the
+    kernel's."""
     res = {}
     for (name, k, n), L in zip(LLAMA3_8B, layers):
         q, _ = K.quant_act_i8_pertoken(L["x"], L["smooth"])
         wt = L["w"].t()
         ops = 2.0 * M_TOKENS * k * n
         try:
-            ms_v = time_events(torch, lambda: torch._int_mm(q, wt), iters=20, warm=4)
+            ms_v = time_events(torch, lambda: torch._int_mm(q, wt), iters=20, warm=4, min_seconds=0.15)
             v = {"ms": round(ms_v, 4), "tops": round(ops / ms_v / 1e9, 1)}
         except Exception as e:  # the vendor path is evidence, not a dependency
             v = {"error": str(e)[:200]}
-        ms_o = time_events(torch, lambda: K.gemm_i8_i32(q, L["w"]), iters=20, warm=4)
+        ms_o = time_events(torch, lambda: K.gemm_i8_i32(q, L["w"]), iters=20, warm=4, min_seconds=0.15)
         res[name] = {"torch_int_mm": v, "fmsmo_gemm_i8_i32": {"ms": round(ms_o, 4), "tops": round(ops / ms_o / 1e9, 1)}}
     return res
 
