@@ -496,30 +496,42 @@ __global__ __launch_bounds__(256, 1) void gemm_rs_kernel(GemmArgs g, Epi epi) {
   // persistent blocks have no registers for a third copy of the stores)
   const bool interior = !GROUPED && cols_full && row_lo + BM <= row_hi;
   if (interior) {
+    // All row operands (the token scales) are requested before the first store: the compiler may
+    // not move a load across a store through an unrelated pointer, so fetched row block by row
+    // block their latency was paid FM times, between the blocks' stores.
     if constexpr (B16) {
+      typename Epi::Row rowctx[FM][4];
 #pragma unroll
-      for (int i = 0; i < FM; ++i) {
-        typename Epi::Row rowctx[4];
+      for (int i = 0; i < FM; ++i)
 #pragma unroll
-        for (int v = 0; v < 4; ++v) rowctx[v] = epi.row(m_base + i * 16 + v);
+        for (int v = 0; v < 4; ++v) rowctx[i][v] = epi.row(m_base + i * 16 + v);
+#pragma unroll
+      for (int i = 0; i < FM; ++i)
 #pragma unroll
         for (int v = 0; v < 4; ++v)
 #pragma unroll
           for (int j = 0; j < FN; ++j)
-            epi.store(m_base + i * 16 + v, n_base + j * 16, acc[i][j][v], rowctx[v], colctx[j]);
-      }
+            epi.store(m_base + i * 16 + v, n_base + j * 16, acc[i][j][v], rowctx[i][v], colctx[j]);
     } else {
+      // (two row blocks at a time: 64 operands at once left some instances without registers; the
+      // e4m3 instance with 32 x 32 blocks, kept for comparisons, has none for more than one block)
+      constexpr int RBB = OP == MMA_I8 ? 2 : 1;
+      static_assert(FM % RBB == 0, "row blocks in batches");
 #pragma unroll
-      for (int i = 0; i < FM; ++i) {
-        typename Epi::Row rowctx[16];
+      for (int i0 = 0; i0 < FM; i0 += RBB) {
+        typename Epi::Row rowctx[RBB][16];
 #pragma unroll
-        for (int v = 0; v < 16; ++v) rowctx[v] = epi.row(m_base + i * 32 + (v >> 2) * 8 + (v & 3));
+        for (int i = 0; i < RBB; ++i)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          const int m = m_base + i * 32 + (v >> 2) * 8 + (v & 3);
+          for (int v = 0; v < 16; ++v) rowctx[i][v] = epi.row(m_base + (i0 + i) * 32 + (v >> 2) * 8 + (v & 3));
 #pragma unroll
-          for (int j = 0; j < FN; ++j) epi.store(m, n_base + j * 32, acc[i][j][v], rowctx[v], colctx[j]);
-        }
+        for (int i = 0; i < RBB; ++i)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) {
+            const int m = m_base + (i0 + i) * 32 + (v >> 2) * 8 + (v & 3);
+#pragma unroll
+            for (int j = 0; j < FN; ++j) epi.store(m, n_base + j * 32, acc[i0 + i][j][v], rowctx[i][v], colctx[j]);
+          }
       }
     }
   } else if constexpr (B16) {
