@@ -789,34 +789,61 @@ __global__ __launch_bounds__(WGM* WGN * 64, (Chk::enabled && Chk::fast) ? 2 : 1)
   typename Epi::Col colctx[FN];
 #pragma unroll
   for (int j = 0; j < FN; ++j) colctx[j] = epi.col(min(n_base + j * 32, g.N - 1), expert, g.N);
-  // Interior tiles (the common case) take a branch-free path; per-row epilogue data is fetched
-  // 16 rows at a time with clamped indices so that the loads are issued back to back.
-  const bool interior = (row_lo + BM <= row_hi) && (col_lo + BN <= g.N);
+  // Whole tiles take a branch-free path.  The row operands (token scales) of up to two row blocks
+  // are requested before the blocks' first store: a load may not be moved across a store through an
+  // unrelated pointer, so requested block by block their latency is paid once per block.  Tiles cut
+  // by the last row test rows in the groups of 8 that the accumulator layout makes wave-uniform
+  // (whole groups store without per-lane tests, groups past the end are skipped by a scalar
+  // branch); per-lane tests around every store would put each store into a basic block of its own.
+  const bool cols_full = col_lo + BN <= g.N;
+  const bool interior = (row_lo + BM <= row_hi) && cols_full;
+  const int rows_left = row_hi - row_lo - wm * TM;  // valid rows from this wave's first row on; uniform
+  constexpr int RBB = FM % 2 == 0 ? 2 : 1;
 #pragma unroll
-  for (int i = 0; i < FM; ++i) {
-    typename Epi::Row rowctx[16];
+  for (int i0 = 0; i0 < FM; i0 += RBB) {
+    if (rows_left - i0 * 32 <= 0) break;
+    typename Epi::Row rowctx[RBB][16];
 #pragma unroll
-    for (int v = 0; v < 16; ++v)
-      rowctx[v] = epi.row(min(m_base + i * 32 + (v >> 2) * 8 + (v & 3), row_hi - 1));
+    for (int i = 0; i < RBB; ++i)
+#pragma unroll
+      for (int v = 0; v < 16; ++v)
+        rowctx[i][v] = epi.row(min(m_base + (i0 + i) * 32 + (v >> 2) * 8 + (v & 3), row_hi - 1));
     if (interior) {
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int m = m_base + i * 32 + (v >> 2) * 8 + (v & 3);
+      for (int i = 0; i < RBB; ++i)
 #pragma unroll
-        for (int j = 0; j < FN; ++j) epi.store(m, n_base + j * 32, acc[i][j][v], rowctx[v], colctx[j]);
-      }
+        for (int v = 0; v < 16; ++v) {
+          const int m = m_base + (i0 + i) * 32 + (v >> 2) * 8 + (v & 3);
+#pragma unroll
+          for (int j = 0; j < FN; ++j) epi.store(m, n_base + j * 32, acc[i0 + i][j][v], rowctx[i][v], colctx[j]);
+        }
     } else {
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int m = m_base + i * 32 + (v >> 2) * 8 + (v & 3);
-        if (m < row_hi) {
+      for (int i = 0; i < RBB; ++i)
 #pragma unroll
-          for (int j = 0; j < FN; ++j) {
-            const int n = n_base + j * 32;
-            if (n < g.N) epi.store(m, n, acc[i][j][v], rowctx[v], colctx[j]);
+        for (int q = 0; q < 4; ++q) {
+          const int left = rows_left - (i0 + i) * 32 - q * 8;
+          if (left >= 8 && cols_full) {
+#pragma unroll
+            for (int vv = 0; vv < 4; ++vv) {
+              const int v = q * 4 + vv, m = m_base + (i0 + i) * 32 + q * 8 + vv;
+#pragma unroll
+              for (int j = 0; j < FN; ++j) epi.store(m, n_base + j * 32, acc[i0 + i][j][v], rowctx[i][v], colctx[j]);
+            }
+          } else if (left > 0) {
+#pragma unroll
+            for (int vv = 0; vv < 4; ++vv) {
+              const int v = q * 4 + vv, m = m_base + (i0 + i) * 32 + q * 8 + vv;
+              if (m < row_hi) {
+#pragma unroll
+                for (int j = 0; j < FN; ++j) {
+                  const int n = n_base + j * 32;
+                  if (n < g.N) epi.store(m, n, acc[i0 + i][j][v], rowctx[i][v], colctx[j]);
+                }
+              }
+            }
           }
         }
-      }
     }
   }
 #endif  // __HIP_DEVICE_COMPILE__
