@@ -535,13 +535,16 @@ __global__ __launch_bounds__(256, 1) void gemm_rs_kernel(GemmArgs g, Epi epi) {
       }
     }
   } else if constexpr (B16) {
+    typename Epi::Row rowctx_all[FM][4];  // (all row operands first, as above; rows past the end take the last row's)
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) rowctx_all[i][v] = epi.row(min(m_base + i * 16 + v, row_hi - 1));
 #pragma unroll
     for (int i = 0; i < FM; ++i) {
       const int left = rows_left - i * 16;
       if (left <= 0) break;
-      typename Epi::Row rowctx[4];
-#pragma unroll
-      for (int v = 0; v < 4; ++v) rowctx[v] = epi.row(min(m_base + i * 16 + v, row_hi - 1));
+      typename Epi::Row(&rowctx)[4] = rowctx_all[i];
       if (left >= 16 && cols_full) {
 #pragma unroll
         for (int v = 0; v < 4; ++v)
