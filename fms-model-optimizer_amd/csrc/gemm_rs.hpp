@@ -72,7 +72,6 @@ __global__ __launch_bounds__(256, 1) void gemm_rs_kernel(GemmArgs g, Epi epi) {
   int tile_m, tile_n;
   int row_lo, row_hi = g.M, expert = 0;
   int64_t a_adj = 0;
-  int a_rows = g.M;  // rows addressable through the A descriptor (numbered like row_lo)
   // Mixture-of-experts mode: the blocks are persistent.  The host launches one block per compute
   // unit (it does not know the row counts); the real tiles -- counted here from `offsets` -- are
   // dealt to the 8 XCDs in contiguous spans of the tile sequence, and the blocks of an XCD take
@@ -93,7 +92,6 @@ __global__ __launch_bounds__(256, 1) void gemm_rs_kernel(GemmArgs g, Epi epi) {
       // rows are numbered as stacked groups (the layout of the output); A may be laid out
       // differently: shift its base so that stacked row numbers address the group's rows
       a_adj = (int64_t)expert * (g.lda_e - (int64_t)g.rows_per_group * g.lda);
-      a_rows = row_hi;
     } else {
       for (int e = 0; e < g.num_experts; ++e) real_m += (g.offsets[e + 1] - g.offsets[e] + BM - 1) / BM;
       const int real_tiles = real_m * g.grid_n;
@@ -113,8 +111,10 @@ __global__ __launch_bounds__(256, 1) void gemm_rs_kernel(GemmArgs g, Epi epi) {
 
   // ---- global -> register staging: thread -> (row = tid / 8 + 32 j, 16-byte chunk = tid % 8)
   const int ld_row = tid >> 3, ld_chunk = tid & 7;
-  const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
-      (void*)(g.a + a_adj), 0, (int)((int64_t)(a_rows - 1) * g.lda + g.K), 0x00020000);
+  // (mixture-of-experts mode re-makes it per tile so that it ends with the expert's last row: the
+  // rows of a cut tile past that row then load as zeros instead of the next expert's tokens, and
+  // matrix instructions on zeros draw far less power than on live codes)
+  __amdgpu_buffer_rsrc_t rsrc_a;
   // per tile (a persistent block re-assigns them): B descriptor of the tile's expert, first
   // column, byte offsets of the thread's first A and B rows
   __amdgpu_buffer_rsrc_t rsrc_b;
@@ -291,6 +291,7 @@ __global__ __launch_bounds__(256, 1) void gemm_rs_kernel(GemmArgs g, Epi epi) {
     }
   }
   col_lo = tile_n * BN;
+  rsrc_a = __builtin_amdgcn_make_buffer_rsrc((void*)(g.a + a_adj), 0, (int)((int64_t)(row_hi - 1) * g.lda + g.K), 0x00020000);
   rsrc_b = __builtin_amdgcn_make_buffer_rsrc((void*)(g.b + (GROUPED ? (int64_t)expert * g.ldb_e : 0)), 0,
                                              (int)((int64_t)(g.N - 1) * g.ldb + g.K), 0x00020000);
   {
