@@ -130,22 +130,37 @@ __global__ __launch_bounds__(TH) void quant_i8_pertoken16_kernel(
   v4i sm[SMOOTH ? NCH : 1];
   float sr[KEEP_RCP ? NCH : 1][8];
   bool ieee_block = false;
+  // bf16 divisors outside 2^-60 .. 2^60 (zero, subnormal, inf and NaN among them) are outside the
+  // fast quotient's proof: a thread that holds one reports NaN as its row maximum, which sends
+  // every row of the block down the IEEE path -- the rows' own reduction carries the flag, the
+  // set-up needs no barrier.  The test is on the packed exponent fields (biased 67 .. 186;
+  // 2^60 itself counts as outside, which only costs speed).
+  [[maybe_unused]] bool bad_divisor = false;
   if constexpr (SMOOTH) {
-    int bad = 0;
+    us2 worst = {0, 0};
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
       const int c = threadIdx.x + i * TH;
       if (c < nchunk) {
         sm[i] = *(const v4i*)(smooth + (size_t)c * AQ_VEC);
+        if constexpr (T == FMSMO_BF16) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const float d = cvt16<T>((u16)((uint32_t)sm[i][j >> 1] >> ((j & 1) * 16)));
-          if constexpr (T == FMSMO_BF16) bad |= !(fabsf(d) >= 8.6736174e-19f && fabsf(d) <= 1.1529215e18f);
-          if constexpr (KEEP_RCP) sr[i][j] = __builtin_amdgcn_rcpf(d);
+          for (int j = 0; j < 4; ++j) {
+            // (a borrow out of the low half only happens when that half is already out of range)
+            const uint32_t ex = (((uint32_t)sm[i][j] >> 7) & 0x00ff00ffu) - 0x00430043u;
+            us2 e2;
+            __builtin_memcpy(&e2, &ex, 4);
+            worst = __builtin_elementwise_max(worst, e2);
+          }
+        }
+        if constexpr (KEEP_RCP) {
+#pragma unroll
+          for (int j = 0; j < 8; ++j)
+            sr[i][j] = __builtin_amdgcn_rcpf(cvt16<T>((u16)((uint32_t)sm[i][j >> 1] >> ((j & 1) * 16))));
         }
       }
     }
-    if constexpr (T == FMSMO_BF16) ieee_block = __syncthreads_or(bad) != 0;
+    if constexpr (T == FMSMO_BF16) bad_divisor = worst[0] > 119 || worst[1] > 119;
   }
 
   const float nz = opaque_neg_zero();
@@ -203,6 +218,9 @@ __global__ __launch_bounds__(TH) void quant_i8_pertoken16_kernel(
           amax2 = __builtin_elementwise_max(amax2, m2);
         }
       }
+    }
+    if constexpr (SMOOTH && T == FMSMO_BF16) {
+      if (bad_divisor) amax2 = us2{0x7fff, 0x7fff};
     }
     uint32_t v = wave_max_u32((uint32_t)(amax2[0] > amax2[1] ? amax2[0] : amax2[1]));
     float* rb = red[parity];
@@ -664,22 +682,37 @@ __global__ __launch_bounds__(TH) void quant_i8_mulscale16_kernel(
   v4i sm[SMOOTH ? NCH : 1];
   float sr[KEEP_RCP ? NCH : 1][8];
   bool ieee_block = false;
+  // bf16 divisors outside 2^-60 .. 2^60 (zero, subnormal, inf and NaN among them) are outside the
+  // fast quotient's proof: a thread that holds one reports NaN as its row maximum, which sends
+  // every row of the block down the IEEE path -- the rows' own reduction carries the flag, the
+  // set-up needs no barrier.  The test is on the packed exponent fields (biased 67 .. 186;
+  // 2^60 itself counts as outside, which only costs speed).
+  [[maybe_unused]] bool bad_divisor = false;
   if constexpr (SMOOTH) {
-    int bad = 0;
+    us2 worst = {0, 0};
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
       const int c = threadIdx.x + i * TH;
       if (c < nchunk) {
         sm[i] = *(const v4i*)(smooth + (size_t)c * AQ_VEC);
+        if constexpr (T == FMSMO_BF16) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const float d = cvt16<T>((u16)((uint32_t)sm[i][j >> 1] >> ((j & 1) * 16)));
-          if constexpr (T == FMSMO_BF16) bad |= !(fabsf(d) >= 8.6736174e-19f && fabsf(d) <= 1.1529215e18f);
-          if constexpr (KEEP_RCP) sr[i][j] = __builtin_amdgcn_rcpf(d);
+          for (int j = 0; j < 4; ++j) {
+            // (a borrow out of the low half only happens when that half is already out of range)
+            const uint32_t ex = (((uint32_t)sm[i][j] >> 7) & 0x00ff00ffu) - 0x00430043u;
+            us2 e2;
+            __builtin_memcpy(&e2, &ex, 4);
+            worst = __builtin_elementwise_max(worst, e2);
+          }
+        }
+        if constexpr (KEEP_RCP) {
+#pragma unroll
+          for (int j = 0; j < 8; ++j)
+            sr[i][j] = __builtin_amdgcn_rcpf(cvt16<T>((u16)((uint32_t)sm[i][j >> 1] >> ((j & 1) * 16))));
         }
       }
     }
-    if constexpr (T == FMSMO_BF16) ieee_block = __syncthreads_or(bad) != 0;
+    if constexpr (T == FMSMO_BF16) bad_divisor = worst[0] > 119 || worst[1] > 119;
   }
 
   // per-tensor modes: one scale (and zero point) for all rows
@@ -747,6 +780,9 @@ __global__ __launch_bounds__(TH) void quant_i8_mulscale16_kernel(
           amax2 = __builtin_elementwise_max(amax2, m2);
         }
       }
+    }
+    if constexpr (SMOOTH && T == FMSMO_BF16) {
+      if (bad_divisor) amax2 = us2{0x7fff, 0x7fff};
     }
     uint32_t v = wave_max_u32((uint32_t)(amax2[0] > amax2[1] ? amax2[0] : amax2[1]));
     float* rb = red[parity];
@@ -1217,17 +1253,27 @@ extern "C" int fmsmo_quant_act_i8_pertoken(const void* x, int x_dtype, int64_t l
                        st, (const u16*)x, ldx, (const u16*)smooth, saturate, q, ldq, scale,      \
                        (int)M, (int)K);                                                          \
   }
+    // divisors with rows of up to 8192 elements: fp16 blocks run one row each and keep nothing;
+    // bf16 blocks (costlier reciprocals, checked divisors) keep theirs across rows once they walk
+    // several, i.e. beyond the resident grid
+#define SMOOTH16(T, NCH)                                                                         \
+  if (T == FMSMO_F16 ||                                                                          \
+      M <= resident_blocks((const void*)quant_i8_pertoken16_kernel<T, NCH, true, 256, false>, 256)) \
+    LAUNCH16(T, NCH, true, 256, false)                                                           \
+  else                                                                                           \
+    LAUNCH16(T, NCH, true, 256, true)
 #define PICK16(T)                                                                                        \
   switch (nch * 2 + (smooth ? 1 : 0)) {                                                                  \
-    case 2: LAUNCH16(T, 1, false, 256, true); break;  case 3: LAUNCH16(T, 1, true, 256, (T == FMSMO_BF16)); break;   \
-    case 4: LAUNCH16(T, 2, false, 256, true); break;  case 5: LAUNCH16(T, 2, true, 256, (T == FMSMO_BF16)); break;   \
-    case 8: LAUNCH16(T, 4, false, 256, true); break;  case 9: LAUNCH16(T, 4, true, 256, (T == FMSMO_BF16)); break;   \
+    case 2: LAUNCH16(T, 1, false, 256, true); break;  case 3: SMOOTH16(T, 1); break;   \
+    case 4: LAUNCH16(T, 2, false, 256, true); break;  case 5: SMOOTH16(T, 2); break;   \
+    case 8: LAUNCH16(T, 4, false, 256, true); break;  case 9: SMOOTH16(T, 4); break;   \
     case 16: LAUNCH16(T, 4, false, 512, true); break; case 17: LAUNCH16(T, 4, true, 512, false); break; \
     case 32: LAUNCH16(T, 8, false, 512, true); break;                                                   \
     default: LAUNCH16(T, 8, true, 512, false); break; /* 16384 < K <= 32768 */                          \
   }
     if (x_dtype == FMSMO_F16) { PICK16(FMSMO_F16) } else { PICK16(FMSMO_BF16) }
 #undef PICK16
+#undef SMOOTH16
 #undef LAUNCH16
     return fmsmo_check_launch();
   }
@@ -1341,17 +1387,26 @@ extern "C" int fmsmo_quant_act_i8_mulscale(const void* x, int x_dtype, int64_t l
   if (mode == 0) LAUNCH16M(T, 0, NCH, SM, TH, KEEP)       \
   else if (mode == 1) LAUNCH16M(T, 1, NCH, SM, TH, KEEP)  \
   else LAUNCH16M(T, 2, NCH, SM, TH, KEEP)
+    // (as in fmsmo_quant_act_i8_pertoken: fp16 blocks keep nothing, bf16 blocks keep their
+    // reciprocals once they walk several rows)
+#define SMOOTH16(T, NCH)                                                                         \
+  if (T == FMSMO_F16 ||                                                                          \
+      M <= resident_blocks((const void*)quant_i8_mulscale16_kernel<T, 0, NCH, true, 256, false>, 256)) \
+    LAUNCH16(T, NCH, true, 256, false)                                                           \
+  else                                                                                           \
+    LAUNCH16(T, NCH, true, 256, true)
 #define PICK16(T)                                                                                        \
   switch (nch * 2 + (smooth ? 1 : 0)) {                                                                  \
-    case 2: LAUNCH16(T, 1, false, 256, true); break;  case 3: LAUNCH16(T, 1, true, 256, (T == FMSMO_BF16)); break;   \
-    case 4: LAUNCH16(T, 2, false, 256, true); break;  case 5: LAUNCH16(T, 2, true, 256, (T == FMSMO_BF16)); break;   \
-    case 8: LAUNCH16(T, 4, false, 256, true); break;  case 9: LAUNCH16(T, 4, true, 256, (T == FMSMO_BF16)); break;   \
+    case 2: LAUNCH16(T, 1, false, 256, true); break;  case 3: SMOOTH16(T, 1); break;   \
+    case 4: LAUNCH16(T, 2, false, 256, true); break;  case 5: SMOOTH16(T, 2); break;   \
+    case 8: LAUNCH16(T, 4, false, 256, true); break;  case 9: SMOOTH16(T, 4); break;   \
     case 16: LAUNCH16(T, 4, false, 512, true); break; case 17: LAUNCH16(T, 4, true, 512, false); break; \
     case 32: LAUNCH16(T, 8, false, 512, true); break;                                                   \
     default: LAUNCH16(T, 8, true, 512, false); break; /* 16384 < K <= 32768 */                          \
   }
     if (x_dtype == FMSMO_F16) { PICK16(FMSMO_F16) } else { PICK16(FMSMO_BF16) }
 #undef PICK16
+#undef SMOOTH16
 #undef LAUNCH16
 #undef LAUNCH16M
     return fmsmo_check_launch();
