@@ -745,6 +745,14 @@ def extras(torch, K, dev, layers, power=True):
         ms = timeit(lambda: K.quant_act_i8_mulscale(xs[next(it) % 3], mode, clip=None if mode == L.MS_PER_TOKEN else clip, smooth=sm), iters=12, warm=3)
         gbs = M * k * 3 / (ms * 1e-3) / 1e9
         res[f"aiu_act_quant_{label}_smooth_M4096_K14336"] = {"us": round(ms * 1e3, 1), "GBps": round(gbs, 1), "frac_hbm": round(gbs / PEAK_HBM_GBS, 4)}
+    # the deploy module's static quantizers in the module's 16-bit dtype (clip values from
+    # calibration: qa_fmo_mo_qfunc, the default when the dynamic quantizer is not asked for,
+    # and qa_raw_qfunc)
+    step = float(torch.tensor(5.0 / 255).half())
+    for mode, label, args in ((L.SQ_FMO, "fmo_mo", (step, -102.0, 0, -2.0, 3.0)), (L.SQ_RAW, "raw", (step, 102.0, 0))):
+        ms = timeit(lambda: K.quant_act_i8_static_t(xs[next(it) % 3], mode, torch.float16, *args), iters=12, warm=3)
+        gbs = M * k * 3 / (ms * 1e-3) / 1e9
+        res[f"static_act_quant_{label}_fp16_M4096_K14336"] = {"us": round(ms * 1e3, 1), "GBps": round(gbs, 1), "frac_hbm": round(gbs / PEAK_HBM_GBS, 4)}
     from fms_mo_amd.aiu_addons.i8i8.i8i8_aiu_op import i8i8_aiu
     n = 4096
     w = torch.randint(-127, 128, (n, k), dtype=torch.int8, device=dev)

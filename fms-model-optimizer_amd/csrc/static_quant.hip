@@ -5,7 +5,8 @@
 // quantizers.  Every intermediate is rounded to the compute dtype T the way torch's elementwise
 // kernels do it: the operation is carried out in fp32 on operands widened from T and rounded back
 // (24 >= 2 * 11 + 2 significand bits make the double rounding of +, -, *, / harmless for fp16,
-// and all the more for bf16); divisions are IEEE divisions.
+// and all the more for bf16); divisions are IEEE divisions, or a shorter sequence that gives the
+// same rounded quotient (the 16-bit kernels).
 #include "quant_math.hpp"
 
 namespace fmsmo {
@@ -52,6 +53,76 @@ __global__ __launch_bounds__(256) void quant_i8_static_t_kernel(const void* __re
       b[i] = (uint8_t)(int)r;
     }
     store8((uint8_t*)q, (size_t)(m * ldq + k), b);
+  }
+}
+
+// The same formulas for a 16-bit compute dtype T on contiguous x of that dtype, at memory speed: the
+// kernel above spends ~30 vector instructions per element (an IEEE fp32 division, a 64-bit index
+// division per chunk, one conversion pair per rounding step), this one ~13.  The quotient of two
+// values of T is the three-operation sequence of the per-token quantizer (div16_mix: it rounds to
+// the same T as the IEEE quotient whenever no intermediate leaves the fp32 normal range, which the
+// launcher guarantees for the divisor and fp16 / bf16 x for the dividend; quotients of bf16 values
+// below 2^-118 may differ in their last bit, far below anything that survives the rounding to an
+// integer), passed through v_div_fixup so that zero, infinite and NaN operands give the IEEE
+// result.  Every other step is the operation of the generic kernel on the same fp32 values, with
+// the roundings to T done on pairs.  Integer codes come from the low mantissa bits of
+// t + 1.5 * 2^23 (round to nearest even for |t| < 2^22; the launcher checks the bound where the
+// formula itself does not clamp).
+template <int T, int MODE>
+__global__ __launch_bounds__(256) void quant_i8_static16_kernel(const u16* __restrict__ x, StaticArgs p,
+                                                                float rcp_scale, int8_t* __restrict__ q,
+                                                                int64_t nchunks) {
+  const float nz = opaque_neg_zero();
+  auto rnd2 = [](float& a, float& b) {
+    const uint32_t w = pack16<T>(a, b);
+    a = cvt16<T>((u16)(w & 0xffff));
+    b = cvt16<T>((u16)(w >> 16));
+  };
+  for (int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x; c < nchunks; c += (int64_t)gridDim.x * 256) {
+    const v4i raw = __builtin_nontemporal_load((const v4i*)(x + c * AQ_VEC));
+    uint32_t code[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const uint32_t w = (uint32_t)raw[j];
+      float e0 = cvt16<T>((u16)(w & 0xffff)), e1 = cvt16<T>((u16)(w >> 16));
+      if constexpr (MODE == FMSMO_SQ_FMO) {
+        e0 = fminf(fmaxf(e0, p.lo), p.hi);
+        e1 = fminf(fmaxf(e1, p.lo), p.hi);
+      }
+      float t0 = __builtin_amdgcn_div_fixupf(div16_mix<T>(e0, p.scale, rcp_scale, nz), p.scale, e0);
+      float t1 = __builtin_amdgcn_div_fixupf(div16_mix<T>(e1, p.scale, rcp_scale, nz), p.scale, e1);
+      rnd2(t0, t1);
+      if constexpr (MODE == FMSMO_SQ_FMO) {
+        t0 -= p.zp; t1 -= p.zp;
+        rnd2(t0, t1);
+      } else {
+        t0 += p.zp; t1 += p.zp;
+        rnd2(t0, t1);
+        if constexpr (MODE == FMSMO_SQ_RAW) {
+          t0 -= 128.0f; t1 -= 128.0f;
+          rnd2(t0, t1);
+          t0 += p.sym; t1 += p.sym;
+          rnd2(t0, t1);
+          t0 = fminf(fmaxf(t0, -128.0f), 127.0f);
+          t1 = fminf(fmaxf(t1, -128.0f), 127.0f);
+        } else if constexpr (MODE == FMSMO_SQ_U8_SHIFT) {
+          t0 = fminf(fmaxf(t0, 0.0f), 255.0f);
+          t1 = fminf(fmaxf(t1, 0.0f), 255.0f);
+        } else {
+          t0 = fminf(fmaxf(t0, -127.0f), 127.0f);
+          t1 = fminf(fmaxf(t1, -127.0f), 127.0f);
+        }
+      }
+      uint32_t c0 = __float_as_uint(t0 + 12582912.0f), c1 = __float_as_uint(t1 + 12582912.0f);
+      if constexpr (MODE == FMSMO_SQ_FMO) {
+        const uint32_t shift = (uint32_t)(128 - (int)p.sym);
+        c0 -= shift; c1 -= shift;
+      } else if constexpr (MODE == FMSMO_SQ_U8_SHIFT) {
+        c0 ^= 0x80u; c1 ^= 0x80u;
+      }
+      code[j] = (c0 & 0xffu) | ((c1 & 0xffu) << 8);
+    }
+    *(uint2*)(q + c * AQ_VEC) = make_uint2(code[0] | (code[1] << 16), code[2] | (code[3] << 16));
   }
 }
 
@@ -103,6 +174,44 @@ __global__ __launch_bounds__(256) void quant_i8_dynamic_kernel(const void* __res
       b[i] = (uint8_t)(int)r;
     }
     store8((uint8_t*)q, (size_t)(m * ldq + k), b);
+  }
+}
+
+// The per-tensor form on contiguous 16-bit x: the quotient of quant_i8_static16_kernel (the scale is
+// a finite value of T by construction; one outside 2^-60 .. 2^60, which only an absurd abs-max
+// gives, sends the whole launch through IEEE divisions), everything behind it as above.
+template <int T>
+__global__ __launch_bounds__(256) void quant_i8_dynamic16_kernel(const u16* __restrict__ x,
+                                                                 const float* __restrict__ scale, float zp,
+                                                                 int8_t* __restrict__ q, int64_t nchunks) {
+  const float s = scale[0];
+  const bool fast = fabsf(s) >= 8.6736174e-19f && fabsf(s) <= 1.1529215e18f;
+  const float r = __builtin_amdgcn_rcpf(s);
+  const float nz = opaque_neg_zero();
+  for (int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x; c < nchunks; c += (int64_t)gridDim.x * 256) {
+    const v4i raw = __builtin_nontemporal_load((const v4i*)(x + c * AQ_VEC));
+    uint32_t code[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const uint32_t w = (uint32_t)raw[j];
+      const float e0 = cvt16<T>((u16)(w & 0xffff)), e1 = cvt16<T>((u16)(w >> 16));
+      float t0, t1;
+      if (fast) {
+        t0 = __builtin_amdgcn_div_fixupf(div16_mix<T>(e0, s, r, nz), s, e0);
+        t1 = __builtin_amdgcn_div_fixupf(div16_mix<T>(e1, s, r, nz), s, e1);
+      } else {
+        t0 = e0 / s;
+        t1 = e1 / s;
+      }
+      uint32_t pk = pack16<T>(t0, t1);
+      t0 = __builtin_rintf(cvt16<T>((u16)(pk & 0xffff))) + zp;
+      t1 = __builtin_rintf(cvt16<T>((u16)(pk >> 16))) + zp;
+      pk = pack16<T>(t0, t1);
+      const uint32_t b0 = (uint32_t)(int)cvt16<T>((u16)(pk & 0xffff)) & 0xffu;
+      const uint32_t b1 = (uint32_t)(int)cvt16<T>((u16)(pk >> 16)) & 0xffu;
+      code[j] = b0 | (b1 << 8);
+    }
+    *(uint2*)(q + c * AQ_VEC) = make_uint2(code[0] | (code[1] << 16), code[2] | (code[3] << 16));
   }
 }
 
@@ -229,6 +338,31 @@ unsigned grid_for(int64_t M, int64_t K) {
   const int64_t blocks = (M * (K / AQ_VEC) + 255) / 256;
   return (unsigned)(blocks < 1 ? 1 : blocks > 8192 ? 8192 : blocks);
 }
+// Host-side rounding of a float to fp16 / bf16 (nearest even) and back.
+float host_round16(float f, int t) {
+  if (t == FMSMO_F16) return (float)(_Float16)f;
+  uint32_t u;
+  __builtin_memcpy(&u, &f, 4);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return f;  // NaN
+  u += 0x7fffu + ((u >> 16) & 1u);
+  u &= 0xffff0000u;
+  __builtin_memcpy(&f, &u, 4);
+  return f;
+}
+// Parameters the fast 16-bit static quantizer covers (see quant_i8_static16_kernel).
+bool static16_ok(const StaticArgs& p, int t) {
+  const float s = fabsf(p.scale);
+  if (!(s > 0.0f) || !(s < INFINITY) || host_round16(p.scale, t) != p.scale) return false;
+  if (t == FMSMO_BF16 && !(s >= 8.6736174e-19f && s <= 1.1529215e18f)) return false;
+  if (!(fabsf(p.zp) < 1.0e6f)) return false;
+  if (p.mode == FMSMO_SQ_FMO) {
+    // codes are not clamped: |clamp(x) / scale - zp| must stay far inside 2^22, and finite in T
+    // (an fp16 quotient that overflows to inf takes the generic kernel's conversion of inf)
+    const float m = fmaxf(fabsf(p.lo), fabsf(p.hi));
+    if (!(m < INFINITY) || !(m / s + fabsf(p.zp) < (t == FMSMO_F16 ? 6.0e4f : 1.0e6f))) return false;
+  }
+  return true;
+}
 int check_rows(const void* x, int x_dtype, int64_t ldx, int64_t M, int64_t K) {
   if (!x) return FMSMO_ERR_NULL;
   if (M < 0 || K <= 0 || ldx < K || M > 0x7fffffff || K > 0x7fffffff) return FMSMO_ERR_SHAPE;
@@ -255,6 +389,27 @@ extern "C" int fmsmo_quant_act_i8_static_t(const void* x, int x_dtype, int64_t l
   StaticArgs p{scale, zp, (float)(sym ? 1 : 0), clip_lo, clip_hi, mode};
   dim3 grid(grid_for(M, K)), block(256);
   hipStream_t st = (hipStream_t)stream;
+  // 16-bit compute dtype, contiguous rows, a divisor that is a finite non-zero value of that dtype
+  // (inside 2^-60 .. 2^60 for bf16) and, for the formula that does not clamp its codes, clip values
+  // whose quotients stay small: the fast kernel.  Anything else takes the generic one below.
+  if (compute_dtype != FMSMO_F32 && ldx == K && ldq == K && static16_ok(p, compute_dtype)) {
+    const int64_t nchunks = M * (K / AQ_VEC);
+    const float rcp = 1.0f / scale;  // correctly rounded: at least as good as the device's rcp
+#define FAST(T, MD)                                                                            \
+  hipLaunchKernelGGL((quant_i8_static16_kernel<T, MD>), grid, block, 0, st, (const u16*)x, p, rcp, \
+                     q, nchunks)
+#define FAST_T(T)                                        \
+  switch (mode) {                                        \
+    case FMSMO_SQ_RAW: FAST(T, FMSMO_SQ_RAW); break;     \
+    case FMSMO_SQ_FMO: FAST(T, FMSMO_SQ_FMO); break;     \
+    case FMSMO_SQ_U8_SHIFT: FAST(T, FMSMO_SQ_U8_SHIFT); break; \
+    default: FAST(T, FMSMO_SQ_S8_NARROW); break;         \
+  }
+    if (x_dtype == FMSMO_F16) { FAST_T(FMSMO_F16) } else { FAST_T(FMSMO_BF16) }
+#undef FAST_T
+#undef FAST
+    return fmsmo_check_launch();
+  }
 #define LAUNCH(XT, T) \
   hipLaunchKernelGGL((quant_i8_static_t_kernel<XT, T>), grid, block, 0, st, x, ldx, p, q, ldq, (int)M, (int)K)
   if (compute_dtype == FMSMO_F32) {
@@ -289,9 +444,14 @@ extern "C" int fmsmo_quant_act_i8_dynamic(const void* x, int x_dtype, int64_t ld
   {                                                                                             \
     hipLaunchKernelGGL((dyn_scale_kernel<T>), sgrid, block, 0, st, col_amax, (int)K, pc,        \
                        (float)levels, scale);                                                   \
-    if (M > 0)                                                                                  \
-      hipLaunchKernelGGL((quant_i8_dynamic_kernel<T>), grid, block, 0, st, x, ldx,              \
-                         (const float*)scale, pc, (float)zp, q, ldq, (int)M, (int)K);           \
+    if (M > 0) {                                                                                \
+      if (T != FMSMO_F32 && !pc && ldx == K && ldq == K)                                        \
+        hipLaunchKernelGGL((quant_i8_dynamic16_kernel<T == FMSMO_F32 ? FMSMO_F16 : T>), grid, block, 0, st, \
+                           (const u16*)x, (const float*)scale, (float)zp, q, M * (K / AQ_VEC)); \
+      else                                                                                      \
+        hipLaunchKernelGGL((quant_i8_dynamic_kernel<T>), grid, block, 0, st, x, ldx,            \
+                           (const float*)scale, pc, (float)zp, q, ldq, (int)M, (int)K);         \
+    }                                                                                           \
   }
   switch (x_dtype) {
     case FMSMO_F16: LAUNCH(FMSMO_F16) break;

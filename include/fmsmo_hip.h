@@ -155,7 +155,8 @@ int fmsmo_quant_act_i8_static(const void* x, int x_dtype, int64_t ldx, float sca
  * Static per-tensor int8 quantizers evaluated in the compute dtype T = compute_dtype (torch's
  * promotion of x's dtype with the dtype of the module's scale buffer: x's own dtype for a module
  * cast to the model dtype, fp32 for fp32 quantizer buffers); every intermediate is rounded to T,
- * divisions are IEEE divisions, rint is half-to-even:
+ * quotients are the IEEE quotients (contiguous rows with a 16-bit T, ldx == ldq == K, run at memory
+ * speed on a shorter division sequence with the same results), rint is half-to-even:
  *   FMSMO_SQ_RAW        q = clamp( rint( (((x / scale) + zp) - 128) + sym ), -128, 127 )
  *                       QLinearINT8Deploy.qa_raw_qfunc (fms_mo/modules/linear.py:1061-1071)
  *   FMSMO_SQ_FMO        q = int8( rint( clamp(x, clip_lo, clip_hi) / scale - zp ) - (128 - sym) )

@@ -106,6 +106,86 @@ def test_static_quantizer_fp16_exact_ties(dev):
     assert torch.equal(q.cpu(), ref)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_static_quantizer_16bit_kernel_on_every_pattern(dev, dtype):
+    """Contiguous rows in a 16-bit compute dtype take a kernel with a three-operation quotient instead
+    of the IEEE division.  Every 16-bit pattern of x: bit-identical to the generic kernel (which a
+    padded output selects) for all four formulas, NaN and infinities included, and to the oracle on
+    the finite patterns.  Parameters outside the fast kernel's domain (a scale that is not a value
+    of the dtype, fp16 quotients that overflow) must give the generic kernel's codes as well."""
+    from fms_mo_amd import _lib as L
+
+    code = L.F16 if dtype == torch.float16 else L.BF16
+    pats = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(dtype).reshape(8, 8192).contiguous()
+    xd = pats.to(dev)
+    M, K = pats.shape
+    lib, st = L.load(), torch.cuda.current_stream().cuda_stream
+    finite = torch.isfinite(pats.float())
+
+    def both(mode, scale, zp, sym, lo, hi):
+        qf = torch.empty(M, K, dtype=torch.int8, device=dev)
+        qg = torch.empty(M, K + 8, dtype=torch.int8, device=dev)
+        for q, ld in ((qf, K), (qg, K + 8)):
+            assert lib.fmsmo_quant_act_i8_static_t(xd.data_ptr(), code, K, mode, code, scale, zp, sym, lo, hi,
+                                                   q.data_ptr(), ld, M, K, st) == 0
+        torch.cuda.synchronize()
+        assert torch.equal(qf, qg[:, :K]), (mode, scale, zp, sym, lo, hi)
+        return qf.cpu()
+
+    t = lambda v: float(torch.tensor(v, dtype=dtype))
+    for scale, zp, sym in ((t(0.0343), 95.0, 0), (t(0.0343), 95.0, 1), (t(1.0), 0.0, 0), (t(250.0), -5.0, 1),
+                           (t(6.1e-5), 128.0, 0), (0.0343, 3.0, 0)):          # the last: not a value of the dtype
+        q = both(L.SQ_RAW, scale, zp, sym, 0.0, 0.0)
+        if t(scale) == scale:
+            ref = O.quant_act_static_raw(pats, torch.tensor([scale], dtype=dtype), torch.tensor([int(zp)], dtype=torch.int), sym)
+            assert torch.equal(q[finite], ref[finite]), ("raw", scale, zp, sym)
+        both(L.SQ_U8_SHIFT, scale, zp, 0, 0.0, 0.0)
+        both(L.SQ_S8_NARROW, scale, zp, 0, 0.0, 0.0)
+    for (cvn, cv), sym in (((-3.25, 5.5), 0), ((-3.25, 5.5), 1), ((-0.01, 0.0), 0), ((-1e4, 1e4), 0)):
+        cvn_t, cv_t = torch.tensor([cvn], dtype=dtype), torch.tensor([cv], dtype=dtype)
+        qs = 255 / (cv_t - cvn_t)
+        step, qzp = 1.0 / qs, torch.round(cvn_t * qs)
+        q = both(L.SQ_FMO, float(step), float(qzp), sym, float(cvn_t), float(cv_t))
+        ref = O.quant_act_fmo_mo(pats, cvn_t, cv_t, step, qzp, sym)
+        assert torch.equal(q[finite], ref[finite]), ("fmo", cvn, cv, sym)
+    # fp16 quotients that overflow to inf: the generic kernel's conversion, whichever kernel runs
+    both(L.SQ_FMO, t(3.0e-5), 3.0, 1, -2.5, 3.0)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_dynamic_per_tensor_quantizer_16bit_kernel_on_every_pattern(dev, dtype):
+    """The per-tensor dynamic quantizer on contiguous 16-bit rows (fast quotient) against the generic
+    kernel (padded output) on every 16-bit pattern of x, for abs-max values from under the 1e-5
+    floor to infinity and NaN; and against the oracle's formula where the abs-max is the data's."""
+    from fms_mo_amd import _lib as L
+
+    code = L.F16 if dtype == torch.float16 else L.BF16
+    pats = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(dtype).reshape(8, 8192).contiguous()
+    xd = pats.to(dev)
+    M, K = pats.shape
+    lib, st = L.load(), torch.cuda.current_stream().cuda_stream
+    for amax in (1.0, 6.0, 65504.0, 1e-7, 3.0e-3, 1.0e21, 3.0e38, float("inf"), float("nan")):
+        for levels, zp in ((127, 0), (126, 1), (110, 17), (63, 64)):
+            col = torch.zeros(K, device=dev)
+            col[K // 3] = amax
+            out = []
+            for ld in (K, K + 8):
+                q = torch.empty(M, ld, dtype=torch.int8, device=dev)
+                sc = torch.empty(1, dtype=torch.float32, device=dev)
+                assert lib.fmsmo_quant_act_i8_dynamic(xd.data_ptr(), code, K, col.data_ptr(), 0, levels, zp,
+                                                      q.data_ptr(), ld, sc.data_ptr(), M, K, st) == 0
+                out.append((q[:, :K].clone(), sc.clone()))
+            torch.cuda.synchronize()
+            assert torch.equal(out[0][0], out[1][0]) and torch.equal(out[0][1], out[1][1]), (amax, levels, zp)
+    # the data's own abs-max, finite values only: the oracle
+    x = pats.clone()
+    x[~torch.isfinite(x.float())] = 0
+    for zp in (1, 64):
+        ref_q, ref_s = O.quant_act_fake_zero_shift(x, torch.tensor(zp, dtype=torch.int))
+        q, sc = Kn().quant_act_i8_dynamic(x.to(dev), False, 127 - zp, zp)
+        assert torch.equal(sc.cpu().reshape(()), ref_s.float()) and torch.equal(q.cpu(), ref_q), zp
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
 def test_dynamic_per_tensor_and_per_column_quantizers(dev, dtype):
     x = (torch.randn(70, 384, generator=gen(2)) * torch.linspace(0.01, 4, 384)).to(dtype)
