@@ -1071,11 +1071,14 @@ __global__ __launch_bounds__(AQ_THREADS) void quant_fp8_pertoken_kernel(
 // hardware OCP e4m3 conversion on values clamped to +-448 (torch maps (448, 464] to 448 and
 // finite rows cannot exceed that).  Rows whose maximum is inf / NaN take the IEEE + software
 // encoder route of the generic kernel.
-template <int XT, int NCH>
+// LIN: the FP8Linear recipe as a compile-time fact (the serving path: no per-element variant
+// tests, the fp16 -> fp32 widening folded into the quotient's fmas, the clamp a single median).
+template <int XT, int NCH, bool LIN = false>
 __global__ __launch_bounds__(AQ_THREADS) void quant_fp8_pertoken16_kernel(
-    const u16* __restrict__ x, int64_t ldx, int variant, uint8_t* __restrict__ q, int64_t ldq,
+    const u16* __restrict__ x, int64_t ldx, int variant_rt, uint8_t* __restrict__ q, int64_t ldq,
     float* __restrict__ scale, int M, int K, float scale_floor, int scale_in_xt,
     int fixed_scale) {
+  const int variant = LIN ? (int)FMSMO_FP8_LINEAR : variant_rt;
   __shared__ float red[2][AQ_THREADS / 64];
   const int nchunk = K / AQ_VEC;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -1136,6 +1139,7 @@ __global__ __launch_bounds__(AQ_THREADS) void quant_fp8_pertoken16_kernel(
     if (fast) {
       const float r1 = rcp_refined(s);
       const bool dl8 = variant == FMSMO_FP8_FPXACC_DL8;
+      [[maybe_unused]] const float nz = opaque_neg_zero();
 #pragma unroll
       for (int i = 0; i < NCH; ++i) {
         const int c = threadIdx.x + i * AQ_THREADS;
@@ -1144,12 +1148,19 @@ __global__ __launch_bounds__(AQ_THREADS) void quant_fp8_pertoken16_kernel(
 #pragma unroll
           for (int j = 0; j < 8; ++j) {
             const float xv = cvt16<XT>((u16)((uint32_t)cur[i][j >> 1] >> ((j & 1) * 16)));
-            if (variant == FMSMO_FP8_LINEAR) t[j] = div32_fast(xv, s, r1);
-            else t[j] = cvt16<XT>(to16<XT>(div16<XT, false>(xv, s, r1)));
-            // the residual corrections lose the sign of a zero quotient; s > 0
-            t[j] = __builtin_copysignf(fminf(fmaxf(t[j], -448.0f), 448.0f), xv);
-            // DL8: the codes 1..4 (|t| up to the tie 4.5 * 2^-9, which rounds to code 4) flush to +0
-            if (dl8) t[j] = fabsf(t[j]) <= 0.0087890625f ? 0.0f : t[j];
+            if constexpr (LIN) {
+              // (the row is finite here, so the median of three is the clamp)
+              if constexpr (XT == FMSMO_F16) t[j] = div32_fast_mix(xv, s, r1, nz);
+              else t[j] = div32_fast(xv, s, r1);
+              t[j] = __builtin_copysignf(__builtin_amdgcn_fmed3f(t[j], -448.0f, 448.0f), xv);
+            } else {
+              if (variant == FMSMO_FP8_LINEAR) t[j] = div32_fast(xv, s, r1);
+              else t[j] = cvt16<XT>(to16<XT>(div16<XT, false>(xv, s, r1)));
+              // the residual corrections lose the sign of a zero quotient; s > 0
+              t[j] = __builtin_copysignf(fminf(fmaxf(t[j], -448.0f), 448.0f), xv);
+              // DL8: the codes 1..4 (|t| up to the tie 4.5 * 2^-9, which rounds to code 4) flush to +0
+              if (dl8) t[j] = fabsf(t[j]) <= 0.0087890625f ? 0.0f : t[j];
+            }
           }
           int o0 = 0, o1 = 0;
           o0 = __builtin_amdgcn_cvt_pk_fp8_f32(t[0], t[1], o0, false);
@@ -1491,11 +1502,15 @@ static int launch_quant_fp8(const void* x, int x_dtype, int64_t ldx, int variant
     dim3 block16(AQ_THREADS);
 #define LAUNCH8(XT, NCH)                                                                          \
   {                                                                                               \
-    const int64_t resident = resident_blocks((const void*)quant_fp8_pertoken16_kernel<XT, NCH>);  \
-    dim3 grid16((unsigned)row_walk_grid(M, resident, true));                                      \
-    hipLaunchKernelGGL((quant_fp8_pertoken16_kernel<XT, NCH>), grid16, block16, 0, st,            \
-                       (const u16*)x, ldx, variant, q, ldq, scale, (int)M, (int)K, scale_floor,   \
-                       scale_in_xt, scale_mode != 0);                                             \
+    dim3 grid16((unsigned)M); /* one row per block: see row_walk_grid */                          \
+    if (variant == FMSMO_FP8_LINEAR)                                                              \
+      hipLaunchKernelGGL((quant_fp8_pertoken16_kernel<XT, NCH, true>), grid16, block16, 0, st,    \
+                         (const u16*)x, ldx, variant, q, ldq, scale, (int)M, (int)K, scale_floor, \
+                         scale_in_xt, scale_mode != 0);                                           \
+    else                                                                                          \
+      hipLaunchKernelGGL((quant_fp8_pertoken16_kernel<XT, NCH, false>), grid16, block16, 0, st,   \
+                         (const u16*)x, ldx, variant, q, ldq, scale, (int)M, (int)K, scale_floor, \
+                         scale_in_xt, scale_mode != 0);                                           \
   }
 #define PICK8(XT)                                  \
   if (per_thread <= 1) LAUNCH8(XT, 1)              \
