@@ -316,6 +316,9 @@ __global__ __launch_bounds__(TH) void quant_i8_pertoken_f16x_f32s_kernel(
 
   // divisors (and refined reciprocals) of this thread's columns; kept across rows for short rows,
   // re-read from L2 per row otherwise
+  // A thread that holds a divisor outside 2^-60 .. 2^60 (or NaN) reports NaN as its row maximum:
+  // the row's own reduction then sends the whole row down the IEEE path, and the set-up needs no
+  // barrier.
   float sv[KEEP ? NCH : 1][8], sr[KEEP ? NCH : 1][8];
   int bad = 0;
 #pragma unroll
@@ -328,7 +331,7 @@ __global__ __launch_bounds__(TH) void quant_i8_pertoken_f16x_f32s_kernel(
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         const float m = fabsf(d[j]);
-        bad |= !(m >= 8.6736174e-19f && m <= 1.1529215e18f);  // outside 2^-60 .. 2^60, or NaN
+        bad |= !(m >= 8.6736174e-19f && m <= 1.1529215e18f);
         if constexpr (KEEP) {
           sv[i][j] = d[j];
           sr[i][j] = rcp_refined(d[j]);
@@ -336,7 +339,7 @@ __global__ __launch_bounds__(TH) void quant_i8_pertoken_f16x_f32s_kernel(
       }
     }
   }
-  const bool ieee_block = __syncthreads_or(bad) != 0;
+  constexpr bool ieee_block = false;
 
   const float nz = opaque_neg_zero();
   v4i cur[NCH], nxt[NCH];
@@ -372,6 +375,9 @@ __global__ __launch_bounds__(TH) void quant_i8_pertoken_f16x_f32s_kernel(
           amax = fmaxf(amax, fabsf(e[i][j]));
         }
       }
+    }
+    if constexpr (!IEEE) {
+      if (bad) amax = __builtin_nanf("");
     }
     return amax;
   };
@@ -412,6 +418,10 @@ __global__ __launch_bounds__(TH) void quant_i8_pertoken_f16x_f32s_kernel(
     const float rs = rcp_refined(s);
     if (threadIdx.x == 0) scale[row] = s;
     int8_t* qr = q + (size_t)row * ldq;
+    // (the two block-uniform choices are made outside the element loops: tested per element they
+    // cut the unrolled code into one basic block per element, which serializes the quotients)
+    auto emit_row = [&](auto ieee_tag, auto sat_tag) {
+      constexpr bool IEEE = decltype(ieee_tag)::value, SAT = decltype(sat_tag)::value;
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
       const int c = threadIdx.x + i * TH;
@@ -419,8 +429,8 @@ __global__ __launch_bounds__(TH) void quant_i8_pertoken_f16x_f32s_kernel(
         uint32_t code[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-          float r = ieee ? e[i][j] / s : div32_fast(e[i][j], s, rs);
-          if (saturate) r = fminf(fmaxf(r, -127.0f), 127.0f);  // the bounds are integers
+          float r = IEEE ? e[i][j] / s : div32_fast(e[i][j], s, rs);
+          if constexpr (SAT) r = fminf(fmaxf(r, -127.0f), 127.0f);  // the bounds are integers
           // |r| <= 128.5 in every finite row: the addition of 1.5 * 2^23 itself rounds r to the
           // nearest integer, ties to even, and leaves it in two's complement in the low mantissa
           // bits
@@ -436,6 +446,14 @@ __global__ __launch_bounds__(TH) void quant_i8_pertoken_f16x_f32s_kernel(
         }
         *(uint2*)(qr + (size_t)c * AQ_VEC) = make_uint2(o[0], o[1]);
       }
+    }
+    };
+    if (ieee) {
+      if (saturate) emit_row(std::true_type{}, std::true_type{});
+      else emit_row(std::true_type{}, std::false_type{});
+    } else {
+      if (saturate) emit_row(std::false_type{}, std::true_type{});
+      else emit_row(std::false_type{}, std::false_type{});
     }
 #pragma unroll
     for (int i = 0; i < NCH; ++i) cur[i] = nxt[i];
