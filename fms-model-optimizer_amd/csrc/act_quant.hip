@@ -1089,14 +1089,16 @@ __global__ __launch_bounds__(AQ_THREADS) void quant_fp8_pertoken_kernel(
 // hardware OCP e4m3 conversion on values clamped to +-448 (torch maps (448, 464] to 448 and
 // finite rows cannot exceed that).  Rows whose maximum is inf / NaN take the IEEE + software
 // encoder route of the generic kernel.
-// LIN: the FP8Linear recipe as a compile-time fact (the serving path: no per-element variant
-// tests, the fp16 -> fp32 widening folded into the quotient's fmas, the clamp a single median).
-template <int XT, int NCH, bool LIN = false>
+// The recipe (VAR: FMSMO_FP8_LINEAR / _FPXACC / _FPXACC_DL8) is a compile-time fact: no
+// per-element variant tests, the fp16 -> fp32 widening of the FP8Linear quotient folded into its
+// fmas, the clamp a single median.
+template <int XT, int NCH, int VAR>
 __global__ __launch_bounds__(AQ_THREADS) void quant_fp8_pertoken16_kernel(
-    const u16* __restrict__ x, int64_t ldx, int variant_rt, uint8_t* __restrict__ q, int64_t ldq,
+    const u16* __restrict__ x, int64_t ldx, uint8_t* __restrict__ q, int64_t ldq,
     float* __restrict__ scale, int M, int K, float scale_floor, int scale_in_xt,
     int fixed_scale) {
-  const int variant = LIN ? (int)FMSMO_FP8_LINEAR : variant_rt;
+  constexpr int variant = VAR;
+  constexpr bool LIN = VAR == FMSMO_FP8_LINEAR;
   __shared__ float red[2][AQ_THREADS / 64];
   const int nchunk = K / AQ_VEC;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -1156,7 +1158,6 @@ __global__ __launch_bounds__(AQ_THREADS) void quant_fp8_pertoken16_kernel(
                       (!fixed_scale || (s >= 0x1p-60f && s <= 0x1p60f && amax <= s * 0x1p100f));
     if (fast) {
       const float r1 = rcp_refined(s);
-      const bool dl8 = variant == FMSMO_FP8_FPXACC_DL8;
       [[maybe_unused]] const float nz = opaque_neg_zero();
 #pragma unroll
       for (int i = 0; i < NCH; ++i) {
@@ -1172,12 +1173,11 @@ __global__ __launch_bounds__(AQ_THREADS) void quant_fp8_pertoken16_kernel(
               else t[j] = div32_fast(xv, s, r1);
               t[j] = __builtin_copysignf(__builtin_amdgcn_fmed3f(t[j], -448.0f, 448.0f), xv);
             } else {
-              if (variant == FMSMO_FP8_LINEAR) t[j] = div32_fast(xv, s, r1);
-              else t[j] = cvt16<XT>(to16<XT>(div16<XT, false>(xv, s, r1)));
+              t[j] = cvt16<XT>(to16<XT>(div16<XT, false>(xv, s, r1)));
               // the residual corrections lose the sign of a zero quotient; s > 0
-              t[j] = __builtin_copysignf(fminf(fmaxf(t[j], -448.0f), 448.0f), xv);
+              t[j] = __builtin_copysignf(__builtin_amdgcn_fmed3f(t[j], -448.0f, 448.0f), xv);
               // DL8: the codes 1..4 (|t| up to the tie 4.5 * 2^-9, which rounds to code 4) flush to +0
-              if (dl8) t[j] = fabsf(t[j]) <= 0.0087890625f ? 0.0f : t[j];
+              if constexpr (VAR == FMSMO_FP8_FPXACC_DL8) t[j] = fabsf(t[j]) <= 0.0087890625f ? 0.0f : t[j];
             }
           }
           int o0 = 0, o1 = 0;
@@ -1518,17 +1518,16 @@ static int launch_quant_fp8(const void* x, int x_dtype, int64_t ldx, int variant
   if (x_dtype != FMSMO_F32 && walk_ok && K <= AQ_MAXCHUNK * AQ_THREADS * AQ_VEC) {
     const int64_t per_thread = div_up(K, AQ_THREADS * AQ_VEC);
     dim3 block16(AQ_THREADS);
+#define LAUNCH8V(XT, NCH, VAR)                                                                    \
+  hipLaunchKernelGGL((quant_fp8_pertoken16_kernel<XT, NCH, VAR>), grid16, block16, 0, st,         \
+                     (const u16*)x, ldx, q, ldq, scale, (int)M, (int)K, scale_floor, scale_in_xt, \
+                     scale_mode != 0);
 #define LAUNCH8(XT, NCH)                                                                          \
   {                                                                                               \
     dim3 grid16((unsigned)M); /* one row per block: see row_walk_grid */                          \
-    if (variant == FMSMO_FP8_LINEAR)                                                              \
-      hipLaunchKernelGGL((quant_fp8_pertoken16_kernel<XT, NCH, true>), grid16, block16, 0, st,    \
-                         (const u16*)x, ldx, variant, q, ldq, scale, (int)M, (int)K, scale_floor, \
-                         scale_in_xt, scale_mode != 0);                                           \
-    else                                                                                          \
-      hipLaunchKernelGGL((quant_fp8_pertoken16_kernel<XT, NCH, false>), grid16, block16, 0, st,   \
-                         (const u16*)x, ldx, variant, q, ldq, scale, (int)M, (int)K, scale_floor, \
-                         scale_in_xt, scale_mode != 0);                                           \
+    if (variant == FMSMO_FP8_LINEAR) LAUNCH8V(XT, NCH, FMSMO_FP8_LINEAR)                          \
+    else if (variant == FMSMO_FP8_FPXACC) LAUNCH8V(XT, NCH, FMSMO_FP8_FPXACC)                     \
+    else LAUNCH8V(XT, NCH, FMSMO_FP8_FPXACC_DL8)                                                  \
   }
 #define PICK8(XT)                                  \
   if (per_thread <= 1) LAUNCH8(XT, 1)              \
@@ -1538,6 +1537,7 @@ static int launch_quant_fp8(const void* x, int x_dtype, int64_t ldx, int variant
     if (x_dtype == FMSMO_F16) { PICK8(FMSMO_F16) } else { PICK8(FMSMO_BF16) }
 #undef PICK8
 #undef LAUNCH8
+#undef LAUNCH8V
     return fmsmo_check_launch();
   }
   dim3 grid((unsigned)M), block(AQ_THREADS);
