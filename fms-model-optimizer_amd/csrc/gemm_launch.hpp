@@ -284,7 +284,7 @@ int launch_dq(const GemmArgs& g, const float* a_scale, int a_stride, const float
   }
 #define GO(OUT, BIAS)                                                                         \
   {                                                                                           \
-    EpiDequant<OUT, BIAS, REF, AccT> epi{y, ldy, a_scale, w_scale, bias, a_stride, w_stride, muladd}; \
+    EpiDequant<OUT, BIAS, REF, AccT, OP == MMA_I8 || OUT == FMSMO_F32> epi{y, ldy, a_scale, w_scale, bias, a_stride, w_stride, muladd}; \
     if constexpr (GROUPED) {                                                                  \
       if (g.K % 128 == 0 && use_register_staged(OP)) launch_rs<OP, true>(g, epi, st);         \
       else launch_tile<TileBig, OP, true>(g, epi, st);                                        \
@@ -457,7 +457,7 @@ int launch_split_k(const SplitPlan& p, const GemmArgs& g0, void* workspace, cons
   dim3 grid(div_up(g0.N, 256), (unsigned)g0.M), block(256);
 #define GO(OUT, BIAS)                                                                         \
   {                                                                                           \
-    EpiDequant<OUT, BIAS, REF, AccT> epi{y, ldy, a_scale, w_scale, bias, a_stride, w_stride, muladd}; \
+    EpiDequant<OUT, BIAS, REF, AccT, OP == MMA_I8 || OUT == FMSMO_F32> epi{y, ldy, a_scale, w_scale, bias, a_stride, w_stride, muladd}; \
     hipLaunchKernelGGL((splitk_reduce_kernel<AccT, decltype(epi)>), grid, block, 0, st,       \
                        (const AccT*)workspace, p.splits, g0.M, g0.N, epi);                    \
   }

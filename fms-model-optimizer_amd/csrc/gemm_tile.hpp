@@ -875,7 +875,12 @@ struct EpiStoreF32 {
 };
 
 // y = acc * (a_scale[m] x w_scale[n]) + bias[n], see FMSMO_EPI_* in fmsmo_hip.h.
-template <int OUT, int BIAS, bool REF_F16, class AccT>
+// MULADD_SWITCH: whether the fp32-scale form looks at `muladd` at all.  The e4m3 GEMMs never ask
+// for the separate multiply and add; without the test their 256 stores per lane are one straight
+// run (the block-uniform test per element cost them 0.5 ... 1.5 % of the whole launch).  Their
+// fp32-output instances keep the switch: without it the register allocation of the 256 x 256
+// tile came out four registers short.
+template <int OUT, int BIAS, bool REF_F16, class AccT, bool MULADD_SWITCH = true>
 struct EpiDequant {
   static constexpr bool UNIFORM_ROWS = false;
   void* y;
@@ -912,7 +917,7 @@ struct EpiDequant {
       else store_from_f32<OUT>(y, idx, f16_to_f32(f32_to_f16(t)));
     } else {
       const float sc = __fmul_rn(r.as, c.ws);
-      const float t = muladd ? __fadd_rn(__fmul_rn((float)v, sc), c.b) : __fmaf_rn((float)v, sc, c.b);
+      const float t = (MULADD_SWITCH && muladd) ? __fadd_rn(__fmul_rn((float)v, sc), c.b) : __fmaf_rn((float)v, sc, c.b);
       store_from_f32<OUT>(y, idx, t);
     }
   }
